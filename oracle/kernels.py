@@ -1,0 +1,175 @@
+"""ctypes front end of the CPU oracle kernels (``oracle/kv_kernels.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py``; the shipped package never imports it.
+
+Every wrapper takes numpy arrays (fp16 as ``np.float16``, indices as ``np.int32``) in the
+argument order of the reference kernel it restates and writes its outputs in place, like
+the destination-passing kernels of the reference.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liborc_kernels.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile the C oracle with the committed Makefile."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-C", _HERE, "liborc_kernels.so"], stdout=subprocess.DEVNULL)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+    return _lib
+
+
+def _p(a):
+    assert a.flags["C_CONTIGUOUS"], "oracle kernels need contiguous arrays"
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def _i32(a):
+    a = np.ascontiguousarray(a, dtype=np.int32)
+    return a
+
+
+_c_int, _c_i64, _c_f = ctypes.c_int, ctypes.c_int64, ctypes.c_float
+
+
+def fused_rope(qkv, position_map, q, k, v, apply_rope, *, theta=1e4, scale=1.0, rotary_dim=None):
+    n, fused, d = qkv.shape
+    hq, hkv = q.shape[1], k.shape[1]
+    assert fused == hq + 2 * hkv
+    pm = _i32(position_map)
+    lib().orc_fused_rope(_p(qkv), _p(pm), _p(q), _p(k), _p(v), _c_i64(n), _c_int(hq), _c_int(hkv),
+                         _c_int(d), _c_int(rotary_dim or d), _c_i64(int(apply_rope)), _c_f(theta),
+                         _c_f(scale))
+
+
+def transpose_append(pages, k_data, v_data, position_map):
+    _, two, hkv, ps, d = pages.shape
+    assert two == 2
+    pm = _i32(position_map)
+    lib().orc_transpose_append(_p(pages), _p(k_data), _p(v_data), _p(pm), _c_i64(len(pm)),
+                               _c_int(hkv), _c_int(ps), _c_int(d))
+
+
+def transpose_append_mla(pages, kv_data, position_map):
+    _, ps, d = pages.shape
+    pm = _i32(position_map)
+    lib().orc_transpose_append_mla(_p(pages), _p(kv_data), _p(pm), _c_i64(len(pm)), _c_int(ps),
+                                   _c_int(d))
+
+
+def debug_get_kv(pages, position_map, k_data, v_data, layer_id):
+    _, _, hkv, ps, d = pages.shape
+    pm = _i32(position_map)
+    lib().orc_debug_get_kv(_p(pages), _p(pm), _p(k_data), _p(v_data), _c_i64(layer_id),
+                           _c_i64(len(pm)), _c_int(hkv), _c_int(ps), _c_int(d))
+
+
+def debug_get_kv_mla(pages, position_map, kv_data, layer_id):
+    _, ps, d = pages.shape
+    pm = _i32(position_map)
+    lib().orc_debug_get_kv_mla(_p(pages), _p(pm), _p(kv_data), _c_i64(layer_id), _c_i64(len(pm)),
+                               _c_int(ps), _c_int(d))
+
+
+def copy_single_page(pages, src_page_id, tgt_page_id, copy_length):
+    _, _, hkv, ps, d = pages.shape
+    lib().orc_copy_single_page(_p(pages), _c_i64(src_page_id), _c_i64(tgt_page_id),
+                               _c_i64(copy_length), _c_int(hkv), _c_int(ps), _c_int(d))
+
+
+def copy_single_page_mla(pages, src_page_id, tgt_page_id, copy_length):
+    _, ps, d = pages.shape
+    lib().orc_copy_single_page_mla(_p(pages), _c_i64(src_page_id), _c_i64(tgt_page_id),
+                                   _c_i64(copy_length), _c_int(ps), _c_int(d))
+
+
+def compact_kv_copy(pages, copy_length_indptr, copy_src_dst_pos, batch_size):
+    _, _, hkv, ps, d = pages.shape
+    ip = _i32(copy_length_indptr)
+    sd = _i32(copy_src_dst_pos)
+    lib().orc_compact_kv_copy(_p(pages), _p(ip), _p(sd), _c_int(batch_size), _c_int(sd.shape[1]),
+                              _c_int(hkv), _c_int(ps), _c_int(d))
+
+
+def decode(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position,
+           output, lse, rotary_mode, rope_scale, rope_theta, sm_scale):
+    b, hq, d = q.shape
+    _, _, hkv, ps, _ = pages.shape
+    li = _i32(length_info)
+    args = [_i32(page_indptr), _i32(page_values), li, _i32(k_rope_pos_offset), _i32(q_rope_position)]
+    lib().orc_decode(_p(q), _p(pages), *[_p(a) for a in args], _p(output), _p(lse), _c_int(b),
+                     _c_int(hq), _c_int(hkv), _c_int(d), _c_int(ps), _c_int(int(li.ndim == 2)),
+                     _c_int(rotary_mode), _c_f(rope_scale), _c_f(rope_theta), _c_f(sm_scale))
+
+
+def decode_range(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset,
+                 q_rope_position, output, lse, b_begin, b_end, sm_scale):
+    b, hq, d = q.shape
+    _, _, hkv, ps, _ = pages.shape
+    args = [_i32(page_indptr), _i32(page_values), _i32(length_info), _i32(k_rope_pos_offset),
+            _i32(q_rope_position)]
+    lib().orc_decode_range(_p(q), _p(pages), *[_p(a) for a in args], _p(output), _p(lse),
+                           _c_int(b_begin), _c_int(b_end), _c_int(b), _c_int(hq), _c_int(hkv),
+                           _c_int(d), _c_int(ps), _c_f(sm_scale))
+
+
+def merge_state_inplace(v, s, v_other, s_other):
+    n, h, d = v.shape
+    lib().orc_merge_state_inplace(_p(v), _p(s), _p(v_other), _p(s_other), _c_i64(n), _c_int(h),
+                                  _c_int(d))
+
+
+def prefill_paged(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset,
+                  q_rope_position, output, lse, causal, rotary_mode, rope_scale, rope_theta,
+                  sm_scale, sliding_window_size=1024):
+    _, hq, d = q.shape
+    _, _, hkv, ps, _ = pages.shape
+    qi = _i32(q_indptr)
+    li = _i32(length_info)
+    args = [_i32(page_indptr), _i32(page_values), li, _i32(k_rope_pos_offset), _i32(q_rope_position)]
+    lib().orc_prefill_paged(_p(q), _p(qi), _p(pages), *[_p(a) for a in args], _p(output), _p(lse),
+                            _c_int(len(qi) - 1), _c_int(hq), _c_int(hkv), _c_int(d), _c_int(ps),
+                            _c_int(int(li.ndim == 2)), _c_int(sliding_window_size),
+                            _c_int(int(causal)), _c_int(rotary_mode), _c_f(rope_scale),
+                            _c_f(rope_theta), _c_f(sm_scale))
+
+
+def prefill_ragged(q, q_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_offset, output, lse,
+                   causal, rotary_mode, rope_scale, rope_theta, sm_scale):
+    _, hq, dqk = q.shape
+    _, hkv, dv = v.shape
+    qi, ki = _i32(q_indptr), _i32(kv_indptr)
+    qp, ko = _i32(q_rope_position), _i32(k_rope_pos_offset)
+    lib().orc_prefill_ragged(_p(q), _p(qi), _p(k), _p(v), _p(ki), _p(qp), _p(ko), _p(output),
+                             _p(lse), _c_int(len(qi) - 1), _c_int(hq), _c_int(hkv), _c_int(dqk),
+                             _c_int(dv), _c_int(int(causal)), _c_int(rotary_mode),
+                             _c_f(rope_scale), _c_f(rope_theta), _c_f(sm_scale))
+
+
+def prefill_paged_mla(q, q_indptr, pages, page_indptr, page_values, length_info, output, lse,
+                      causal, sm_scale, d_latent=512):
+    _, hq, dqk = q.shape
+    _, ps, _ = pages.shape
+    qi = _i32(q_indptr)
+    li = _i32(length_info)
+    pi, pv = _i32(page_indptr), _i32(page_values)  # keep the converted arrays alive
+    lib().orc_prefill_paged_mla(_p(q), _p(qi), _p(pages), _p(pi), _p(pv), _p(li), _p(output),
+                                _p(lse),
+                                _c_int(len(qi) - 1), _c_int(hq), _c_int(d_latent),
+                                _c_int(dqk - d_latent), _c_int(ps), _c_int(int(li.ndim == 2)),
+                                _c_int(int(causal)), _c_f(sm_scale))

@@ -1,0 +1,510 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- CPU restatement of the reference's llvm-target
+ * KV-cache kernels.  Nothing in the shipped package may link or call this
+ * file; it is the checker for the HIP kernels and the CPU baseline of the
+ * benchmark.
+ *
+ * Every function follows one TVMScript kernel of the reference, statement by
+ * statement (serial loops, fp16 storage, fp32 arithmetic, base-2 softmax,
+ * online-softmax state initialised to m = -5e4, d = 1).  Citations are
+ * file:line into the reference tree:
+ *
+ *   orc_fused_rope              python/tvm/relax/frontend/nn/llm/position_embedding.py:525-565
+ *                               (frequency: :32-67, rotate-half term: :493-523)
+ *   orc_transpose_append        python/tvm/relax/frontend/nn/llm/_page_kernels.py:40-74
+ *   orc_transpose_append_mla    _page_kernels.py:77-103
+ *   orc_debug_get_kv(_mla)      _page_kernels.py:106-166
+ *   orc_copy_single_page(_mla)  _page_kernels.py:169-232
+ *   orc_compact_kv_copy         _page_kernels.py:266-293
+ *   orc_decode                  python/tvm/relax/frontend/nn/llm/_decode_kernels.py:49-178
+ *   orc_merge_state_inplace     _decode_kernels.py:414-452
+ *   orc_prefill_paged           python/tvm/relax/frontend/nn/llm/_prefill_kernels.py:54-214
+ *   orc_prefill_ragged          _prefill_kernels.py:677-791
+ *   orc_prefill_paged_mla       _prefill_kernels.py:927-1071 (GPU-only kernel in the
+ *                               reference; restated here row by row, see below)
+ *   helpers                     python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-170
+ *
+ * Parity pins (tests/test_oracle_*.py): RoPE against the numpy closed form of
+ * the reference's own test (tests/python/relax/
+ * test_runtime_builtin_paged_attention_kv_cache_cpu.py:305-324), attention
+ * against softmax(QK^T*scale + causal mask)V with GQA head repeat (:499-535),
+ * merge against the two-way log-sum-exp identity, append/gather by round trip.
+ *
+ * PARITY UNPINNED relative to "the reference's llvm kernels":
+ *   orc_prefill_paged_mla -- the reference has no llvm MLA kernel
+ *   (python/tvm/relax/frontend/nn/llm/kv_cache.py:676-677); this function is
+ *   pinned to the mathematical definition (torch closed form of
+ *   tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_mla_tir.py:351-398)
+ *   only.
+ *
+ * Deliberate deviations from the reference text, none of which changes a
+ * result for valid inputs:
+ *   - _prefill_kernels.py:162 loops row_idx over max_num_pages*page_size and
+ *     guards with row_idx < kv_len; here the loop bound is kv_len.
+ *   - _prefill_kernels.py:204 reads scale_O[d_idx] from a 1-element buffer;
+ *     restated as scale_O[0].
+ *   - new_m (:132) is an uninitialised allocation in the reference; it starts
+ *     at m_val here (it only matters when the very first column of a row is
+ *     masked out).
+ */
+#include <immintrin.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+typedef uint16_t f16;
+
+static inline float h2f(f16 h) { return _cvtsh_ss(h); }
+static inline f16 f2h(float f) { return _cvtss_sh(f, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC); }
+
+#define LOG2E_F ((float)1.4426950408889634) /* math.log2(math.exp(1)) */
+
+/* ---- _kernel_common.py:155-170 ------------------------------------------------ */
+static inline int kv_chunk_len(int num_pages, int page_size, int seq_id, const int32_t* length_info,
+                               int B, int sliding_window) {
+  if (num_pages == 0) return 0;
+  if (!sliding_window) return (num_pages - 1) * page_size + length_info[seq_id];
+  return (num_pages - 1) * page_size + length_info[seq_id] - length_info[B + seq_id] +
+         length_info[2 * B + seq_id];
+}
+
+static inline int seq_offset(int pos, int seq_id, const int32_t* length_info, int B,
+                             int sliding_window) {
+  if (!sliding_window) return pos;
+  int sink = length_info[2 * B + seq_id];
+  return pos < sink ? pos : pos - sink + length_info[B + seq_id];
+}
+
+/* _kernel_common.py:130-144 */
+static inline int causal_mask(int causal, int row, int col, int kv_len, int qo_len) {
+  return causal > 0 ? (col < kv_len - qo_len + row + 1) : (col < kv_len);
+}
+
+static inline int causal_or_sliding_cross_mask(int causal, int row, int col, int kv_len, int qo_len,
+                                               int sliding_window_size) {
+  int visible_past = sliding_window_size - row - 1;
+  if (visible_past < 0) visible_past = 0;
+  if (causal > 0 && sliding_window_size > 0) {
+    int lo = kv_len - visible_past;
+    if (lo < 0) lo = 0;
+    return col < kv_len && col >= lo;
+  }
+  return causal_mask(causal, row, col, kv_len, qo_len);
+}
+
+/* ---- RoPE (position_embedding.py:32-67 + _kernel_common.py:115-127) ----------- */
+/* x points at element 0 of the head vector; returns the rotated element d,
+ * rounded to fp16 exactly where the reference casts. */
+static inline f16 rope_elem(const f16* x, int d, int rotary_dim, float pos_times_scale, float theta) {
+  float freq = pos_times_scale / powf(theta, (float)((d * 2) % rotary_dim) / (float)rotary_dim);
+  float c = cosf(freq) * h2f(x[d]);
+  f16 other = d < rotary_dim / 2 ? (f16)(x[d + rotary_dim / 2] ^ 0x8000u) : x[d - rotary_dim / 2];
+  float s = sinf(freq) * h2f(other);
+  return f2h(c + s);
+}
+
+void orc_fused_rope(const f16* qkv, const int32_t* position_map, f16* q, f16* k, f16* v,
+                    int64_t seq_len, int num_q_heads, int num_kv_heads, int head_dim,
+                    int rotary_dim, int64_t apply_rope, float theta, float scale) {
+  int fused_heads = num_q_heads + 2 * num_kv_heads;
+  for (int64_t s = 0; s < seq_len; ++s) {
+    for (int h = 0; h < fused_heads; ++h) {
+      const f16* x = qkv + (s * fused_heads + h) * head_dim;
+      for (int d = 0; d < head_dim; ++d) {
+        if (h < num_q_heads) {
+          q[(s * num_q_heads + h) * head_dim + d] =
+              (apply_rope > 0 && d < rotary_dim)
+                  ? rope_elem(x, d, rotary_dim, (float)position_map[s] * scale, theta)
+                  : x[d];
+        } else if (h < num_q_heads + num_kv_heads) {
+          k[(s * num_kv_heads + (h - num_q_heads)) * head_dim + d] =
+              (apply_rope > 0 && d < rotary_dim)
+                  ? rope_elem(x, d, rotary_dim, (float)position_map[s] * scale, theta)
+                  : x[d];
+        } else {
+          v[(s * num_kv_heads + (h - num_q_heads - num_kv_heads)) * head_dim + d] = x[d];
+        }
+      }
+    }
+  }
+}
+
+/* ---- page kernels ------------------------------------------------------------ */
+#define PAGE_AT(pages, Hkv, ps, D, page, kv, h, slot) \
+  ((pages) + ((((int64_t)(page) * 2 + (kv)) * (Hkv) + (h)) * (ps) + (slot)) * (int64_t)(D))
+
+void orc_transpose_append(f16* pages, const f16* k_data, const f16* v_data,
+                          const int32_t* position_map, int64_t ntoken, int Hkv, int page_size,
+                          int D) {
+  for (int64_t g = 0; g < ntoken; ++g) {
+    int32_t position = position_map[g];
+    if (position == -1) continue;
+    for (int h = 0; h < Hkv; ++h) {
+      f16* kd = PAGE_AT(pages, Hkv, page_size, D, position / page_size, 0, h, position % page_size);
+      f16* vd = PAGE_AT(pages, Hkv, page_size, D, position / page_size, 1, h, position % page_size);
+      for (int f = 0; f < D; ++f) {
+        kd[f] = k_data[(g * Hkv + h) * D + f];
+        vd[f] = v_data[(g * Hkv + h) * D + f];
+      }
+    }
+  }
+}
+
+void orc_transpose_append_mla(f16* pages, const f16* kv_data, const int32_t* position_map,
+                              int64_t ntoken, int page_size, int d_qk) {
+  for (int64_t g = 0; g < ntoken; ++g) {
+    int32_t position = position_map[g];
+    if (position == -1) continue;
+    f16* dst = pages + ((int64_t)(position / page_size) * page_size + position % page_size) * d_qk;
+    for (int f = 0; f < d_qk; ++f) dst[f] = kv_data[g * d_qk + f];
+  }
+}
+
+void orc_debug_get_kv(const f16* pages, const int32_t* position_map, f16* k_data, f16* v_data,
+                      int64_t layer_id, int64_t seqlen, int Hkv, int page_size, int D) {
+  for (int64_t p = 0; p < seqlen; ++p) {
+    int32_t position = position_map[p];
+    for (int h = 0; h < Hkv; ++h) {
+      const f16* ks = PAGE_AT(pages, Hkv, page_size, D, position / page_size, 0, h, position % page_size);
+      const f16* vs = PAGE_AT(pages, Hkv, page_size, D, position / page_size, 1, h, position % page_size);
+      int64_t o = ((layer_id * seqlen + p) * Hkv + h) * D;
+      for (int d = 0; d < D; ++d) {
+        k_data[o + d] = ks[d];
+        v_data[o + d] = vs[d];
+      }
+    }
+  }
+}
+
+void orc_debug_get_kv_mla(const f16* pages, const int32_t* position_map, f16* kv_data,
+                          int64_t layer_id, int64_t seqlen, int page_size, int d_qk) {
+  for (int64_t p = 0; p < seqlen; ++p) {
+    int32_t position = position_map[p];
+    const f16* src = pages + ((int64_t)(position / page_size) * page_size + position % page_size) * d_qk;
+    for (int d = 0; d < d_qk; ++d) kv_data[(layer_id * seqlen + p) * d_qk + d] = src[d];
+  }
+}
+
+void orc_copy_single_page(f16* pages, int64_t src_page_id, int64_t tgt_page_id, int64_t copy_length,
+                          int Hkv, int page_size, int D) {
+  int64_t total = copy_length * Hkv * D;
+  for (int64_t i = 0; i < total; ++i) {
+    int vh = (int)(i / (copy_length * D));
+    int vp = (int)(i % (copy_length * D) / D);
+    int vd = (int)(i % D);
+    PAGE_AT(pages, Hkv, page_size, D, tgt_page_id, 0, vh, vp)[vd] =
+        PAGE_AT(pages, Hkv, page_size, D, src_page_id, 0, vh, vp)[vd];
+    PAGE_AT(pages, Hkv, page_size, D, tgt_page_id, 1, vh, vp)[vd] =
+        PAGE_AT(pages, Hkv, page_size, D, src_page_id, 1, vh, vp)[vd];
+  }
+}
+
+void orc_copy_single_page_mla(f16* pages, int64_t src_page_id, int64_t tgt_page_id,
+                              int64_t copy_length, int page_size, int d_qk) {
+  for (int64_t i = 0; i < copy_length * d_qk; ++i) {
+    int64_t vp = i / d_qk, vd = i % d_qk;
+    pages[(tgt_page_id * page_size + vp) * d_qk + vd] = pages[(src_page_id * page_size + vp) * d_qk + vd];
+  }
+}
+
+void orc_compact_kv_copy(f16* pages, const int32_t* copy_length_indptr, const int32_t* copy_src_dst_pos,
+                         int32_t batch_size, int32_t total_copy_length, int Hkv, int page_size, int D) {
+  for (int b = 0; b < batch_size; ++b)
+    for (int h = 0; h < Hkv; ++h)
+      for (int d = 0; d < D; ++d)
+        for (int i = 0; i < copy_length_indptr[b + 1] - copy_length_indptr[b]; ++i) {
+          int32_t src_pos = copy_src_dst_pos[copy_length_indptr[b] + i];
+          int32_t dst_pos = copy_src_dst_pos[total_copy_length + copy_length_indptr[b] + i];
+          PAGE_AT(pages, Hkv, page_size, D, dst_pos / page_size, 0, h, dst_pos % page_size)[d] =
+              PAGE_AT(pages, Hkv, page_size, D, src_pos / page_size, 0, h, src_pos % page_size)[d];
+          PAGE_AT(pages, Hkv, page_size, D, dst_pos / page_size, 1, h, dst_pos % page_size)[d] =
+              PAGE_AT(pages, Hkv, page_size, D, src_pos / page_size, 1, h, src_pos % page_size)[d];
+        }
+}
+
+/* ---- batch_decode_paged_kv_cpu (_decode_kernels.py:103-176) -------------------- */
+void orc_decode(const f16* Q, const f16* pages, const int32_t* page_table_indptr,
+                const int32_t* page_table_values, const int32_t* length_info,
+                const int32_t* k_rope_pos_offset, const int32_t* q_rope_position, f16* output,
+                float* lse, int B, int H_qo, int H_kv, int D, int page_size, int sliding_window,
+                int rotary_mode, float rope_scale, float rope_theta, float sm_scale) {
+  int group_size = H_qo / H_kv;
+  float* O_local = (float*)malloc(sizeof(float) * D * 4);
+  float *Q_local = O_local + D, *K_local = Q_local + D, *V_local = K_local + D;
+  for (int b = 0; b < B; ++b) {
+    int begin = page_table_indptr[b], end = page_table_indptr[b + 1];
+    int kv_len = kv_chunk_len(end - begin, page_size, b, length_info, B, sliding_window);
+    for (int h_qo = 0; h_qo < H_qo; ++h_qo) {
+      float m_val = -5e4f, d_val = 1.0f;
+      const f16* qrow = Q + ((int64_t)b * H_qo + h_qo) * D;
+      for (int d = 0; d < D; ++d) O_local[d] = 0.0f;
+      for (int d = 0; d < D; ++d)
+        Q_local[d] = rotary_mode == 1
+                         ? h2f(rope_elem(qrow, d, D, (float)q_rope_position[b] * rope_scale, rope_theta))
+                         : h2f(qrow[d]);
+      for (int row_idx = 0; row_idx < kv_len; ++row_idx) {
+        int so = seq_offset(row_idx, b, length_info, B, sliding_window);
+        int page_no = page_table_values[begin + so / page_size];
+        int page_offset = so % page_size;
+        const f16* krow = PAGE_AT(pages, H_kv, page_size, D, page_no, 0, h_qo / group_size, page_offset);
+        const f16* vrow = PAGE_AT(pages, H_kv, page_size, D, page_no, 1, h_qo / group_size, page_offset);
+        for (int d = 0; d < D; ++d)
+          K_local[d] = rotary_mode == 1
+                           ? h2f(rope_elem(krow, d, D, (float)(k_rope_pos_offset[b] + row_idx) * rope_scale, rope_theta))
+                           : h2f(krow[d]);
+        float S_val = 0.0f;
+        for (int d = 0; d < D; ++d) S_val += Q_local[d] * K_local[d];
+        S_val *= sm_scale * LOG2E_F;
+        float new_m = fmaxf(m_val, S_val);
+        d_val = d_val * exp2f(m_val - new_m) + exp2f(S_val - new_m);
+        float scale_O = exp2f(m_val - new_m);
+        for (int d = 0; d < D; ++d) O_local[d] = O_local[d] * scale_O;
+        m_val = new_m;
+        for (int d = 0; d < D; ++d) V_local[d] = h2f(vrow[d]);
+        float factor = exp2f(S_val - m_val);
+        for (int d = 0; d < D; ++d) O_local[d] = O_local[d] + V_local[d] * factor;
+      }
+      for (int d = 0; d < D; ++d) {
+        O_local[d] = O_local[d] / d_val;
+        output[((int64_t)b * H_qo + h_qo) * D + d] = f2h(O_local[d]);
+      }
+      lse[(int64_t)b * H_qo + h_qo] = m_val + log2f(d_val);
+    }
+  }
+  free(O_local);
+}
+
+/* ---- merge_state_inplace_cpu (_decode_kernels.py:432-450) ---------------------- */
+void orc_merge_state_inplace(f16* V, float* S, const f16* V_other, const float* S_other, int64_t N,
+                             int H, int D) {
+  for (int64_t n = 0; n < N; ++n)
+    for (int h = 0; h < H; ++h) {
+      float s_val = S[n * H + h], s_other_val = S_other[n * H + h];
+      float s_max = fmaxf(s_val, s_other_val);
+      s_val = exp2f(s_val - s_max);
+      s_other_val = exp2f(s_other_val - s_max);
+      float scale = s_val / (s_val + s_other_val);
+      float other_scale = s_other_val / (s_val + s_other_val);
+      for (int d = 0; d < D; ++d) {
+        int64_t i = (n * H + h) * D + d;
+        V[i] = f2h(h2f(V[i]) * scale + h2f(V_other[i]) * other_scale);
+      }
+      S[n * H + h] = log2f(s_val + s_other_val) + s_max;
+    }
+}
+
+/* ---- batch_prefill_paged_kv_cpu (_prefill_kernels.py:121-213) ------------------ */
+void orc_prefill_paged(const f16* q, const int32_t* q_indptr, const f16* pages,
+                       const int32_t* page_indptr, const int32_t* page_values,
+                       const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                       const int32_t* q_rope_position, f16* output, float* lse, int batch_size,
+                       int h_q, int h_kv, int d, int page_size, int sliding_window,
+                       int sliding_window_size, int causal, int rotary_mode, float rope_scale,
+                       float rope_theta, float sm_scale) {
+  int group_size = h_q / h_kv;
+  float* O_local = (float*)malloc(sizeof(float) * d * 4);
+  float *Q_local = O_local + d, *K_local = Q_local + d, *V_local = K_local + d;
+  for (int h_qo = 0; h_qo < h_q; ++h_qo) {
+    for (int b_idx = 0; b_idx < batch_size; ++b_idx) {
+      int begin = page_indptr[b_idx], end = page_indptr[b_idx + 1];
+      int kv_len = kv_chunk_len(end - begin, page_size, b_idx, length_info, batch_size, sliding_window);
+      int qo_len = q_indptr[b_idx + 1] - q_indptr[b_idx];
+      float new_m = -5e4f;
+      for (int q_idx = 0; q_idx < qo_len; ++q_idx) {
+        float m_val = -5e4f, d_val = 1.0f;
+        if (q_idx == 0) new_m = m_val;
+        for (int i = 0; i < d; ++i) O_local[i] = 0.0f;
+        int curl_q = q_indptr[b_idx] + q_idx;
+        const f16* qrow = q + ((int64_t)curl_q * h_q + h_qo) * d;
+        for (int i = 0; i < d; ++i)
+          Q_local[i] = rotary_mode == 1
+                           ? h2f(rope_elem(qrow, i, d, (float)q_rope_position[curl_q] * rope_scale, rope_theta))
+                           : h2f(qrow[i]);
+        for (int row_idx = 0; row_idx < kv_len; ++row_idx) {
+          int so = seq_offset(row_idx, b_idx, length_info, batch_size, sliding_window);
+          int page_no = page_values[begin + so / page_size];
+          int page_offset = so % page_size;
+          const f16* krow = PAGE_AT(pages, h_kv, page_size, d, page_no, 0, h_qo / group_size, page_offset);
+          const f16* vrow = PAGE_AT(pages, h_kv, page_size, d, page_no, 1, h_qo / group_size, page_offset);
+          for (int i = 0; i < d; ++i) {
+            K_local[i] = rotary_mode == 1
+                             ? h2f(rope_elem(krow, i, d, (float)(k_rope_pos_offset[b_idx] + row_idx) * rope_scale, rope_theta))
+                             : h2f(krow[i]);
+            V_local[i] = h2f(vrow[i]);
+          }
+          float S_val = 0.0f;
+          for (int i = 0; i < d; ++i) S_val += Q_local[i] * K_local[i];
+          S_val *= sm_scale * LOG2E_F;
+          if (causal_or_sliding_cross_mask(causal, q_idx, row_idx, kv_len, qo_len,
+                                           sliding_window ? sliding_window_size : 0)) {
+            new_m = fmaxf(m_val, S_val);
+          } else {
+            S_val = -5e4f;
+          }
+          d_val *= exp2f(m_val - new_m);
+          d_val += exp2f(S_val - new_m);
+          float scale_O = exp2f(m_val - new_m);
+          m_val = new_m;
+          float factor = exp2f(S_val - m_val);
+          for (int i = 0; i < d; ++i) O_local[i] = O_local[i] * scale_O;
+          for (int i = 0; i < d; ++i) O_local[i] += V_local[i] * factor;
+        }
+        for (int i = 0; i < d; ++i) {
+          O_local[i] = O_local[i] / d_val;
+          output[((int64_t)curl_q * h_q + h_qo) * d + i] = f2h(O_local[i]);
+        }
+        lse[(int64_t)curl_q * h_q + h_qo] = m_val + log2f(d_val);
+      }
+    }
+  }
+  free(O_local);
+}
+
+/* ---- batch_prefill_ragged_kv (cpu) (_prefill_kernels.py:715-790) ---------------- */
+void orc_prefill_ragged(const f16* q, const int32_t* q_indptr, const f16* k, const f16* v,
+                        const int32_t* kv_indptr, const int32_t* q_rope_position,
+                        const int32_t* k_rope_pos_offset, f16* output, float* lse, int batch_size,
+                        int h_q, int h_kv, int d_qk, int d_v, int causal, int rotary_mode,
+                        float rope_scale, float rope_theta, float sm_scale) {
+  int group_size = h_q / h_kv;
+  int max_kv = 1;
+  for (int b = 0; b < batch_size; ++b)
+    if (kv_indptr[b + 1] - kv_indptr[b] > max_kv) max_kv = kv_indptr[b + 1] - kv_indptr[b];
+  float* attention_scores = (float*)malloc(sizeof(float) * (size_t)max_kv * h_q * 2);
+  float* exp_scores = attention_scores + (size_t)max_kv * h_q;
+  float* hbuf = (float*)malloc(sizeof(float) * (h_q * 6 + d_v + d_qk));
+  float *softmax_sum = hbuf, *m_prev = hbuf + h_q, *m_new = hbuf + 2 * h_q, *d_prev = hbuf + 3 * h_q,
+        *d_new = hbuf + 4 * h_q, *max_score = hbuf + 5 * h_q, *p_sum = hbuf + 6 * h_q,
+        *qbuf = hbuf + 6 * h_q + d_v;
+  for (int b = 0; b < batch_size; ++b) {
+    int qo_len = q_indptr[b + 1] - q_indptr[b];
+    int kv_len = kv_indptr[b + 1] - kv_indptr[b];
+    for (int q_idx = 0; q_idx < qo_len; ++q_idx) {
+      for (int i = 0; i < h_q; ++i) {
+        max_score[i] = -5e4f;
+        m_prev[i] = -5e4f;
+        d_prev[i] = 1.0f;
+        m_new[i] = -5e4f; /* never read before the k loop assigns it when kv_len > 0 */
+      }
+      for (int h = 0; h < h_q; ++h) {
+        int h_kv_idx = h / group_size;
+        const f16* qrow = q + ((int64_t)(q_indptr[b] + q_idx) * h_q + h) * d_qk;
+        for (int i = 0; i < d_qk; ++i)
+          qbuf[i] = rotary_mode == 1
+                        ? h2f(rope_elem(qrow, i, d_qk, (float)q_rope_position[q_indptr[b] + q_idx] * rope_scale, rope_theta))
+                        : h2f(qrow[i]);
+        for (int k_idx = 0; k_idx < kv_len; ++k_idx) {
+          float attention_score;
+          if (causal_mask(causal, q_idx, k_idx, kv_len, qo_len)) {
+            const f16* krow = k + ((int64_t)(kv_indptr[b] + k_idx) * h_kv + h_kv_idx) * d_qk;
+            float result = 0.0f;
+            for (int i = 0; i < d_qk; ++i) {
+              float key_val = rotary_mode == 1
+                                  ? h2f(rope_elem(krow, i, d_qk, (float)(k_rope_pos_offset[b] + k_idx) * rope_scale, rope_theta))
+                                  : h2f(krow[i]);
+              result += qbuf[i] * key_val;
+            }
+            attention_score = result * LOG2E_F * sm_scale;
+          } else {
+            attention_score = -5e4f * LOG2E_F * sm_scale;
+          }
+          attention_scores[(size_t)k_idx * h_q + h] = attention_score;
+          max_score[h] = fmaxf(max_score[h], attention_score);
+          m_new[h] = fmaxf(m_prev[h], max_score[h]);
+        }
+      }
+      for (int h = 0; h < h_q; ++h) d_new[h] = d_prev[h] * exp2f(m_prev[h] - m_new[h]);
+      for (int h = 0; h < h_q; ++h) {
+        softmax_sum[h] = 0.0f;
+        for (int k_idx = 0; k_idx < kv_len; ++k_idx) {
+          exp_scores[(size_t)k_idx * h_q + h] = exp2f(attention_scores[(size_t)k_idx * h_q + h] - m_new[h]);
+          softmax_sum[h] += exp_scores[(size_t)k_idx * h_q + h];
+        }
+        d_new[h] += softmax_sum[h];
+      }
+      for (int h = 0; h < h_q; ++h) {
+        int h_kv_idx = h / group_size;
+        for (int i = 0; i < d_v; ++i) p_sum[i] = 0.0f;
+        for (int v_idx = 0; v_idx < kv_len; ++v_idx) {
+          float weight = exp_scores[(size_t)v_idx * h_q + h] / d_new[h];
+          const f16* vrow = v + ((int64_t)(kv_indptr[b] + v_idx) * h_kv + h_kv_idx) * d_v;
+          for (int i = 0; i < d_v; ++i) p_sum[i] += h2f(vrow[i]) * weight;
+        }
+        for (int i = 0; i < d_v; ++i)
+          output[((int64_t)(q_indptr[b] + q_idx) * h_q + h) * d_v + i] = f2h(p_sum[i]);
+        lse[(int64_t)(q_indptr[b] + q_idx) * h_q + h] = m_new[h] + log2f(d_new[h]);
+      }
+    }
+  }
+  free(attention_scores);
+  free(hbuf);
+}
+
+/* ---- batch_prefill_paged_kv_mla (_prefill_kernels.py:979-1064) ------------------
+ * The reference only has the tiled GPU form.  Per output row its arithmetic is:
+ * S = sum_j q[j]*kv[j] over all d_qk features, scaled by sm_scale*log2(e); online
+ * softmax per tile with masked entries contributing exp2(-5e4 - m); O accumulates
+ * p * kv[:d_latent]; out = O/d, lse = m + log2 d.  Restated here one key row at a
+ * time (tile size 1), which is the same recurrence the llvm decode kernel uses. */
+void orc_prefill_paged_mla(const f16* q, const int32_t* q_indptr, const f16* pages,
+                           const int32_t* page_indptr, const int32_t* page_values,
+                           const int32_t* length_info, f16* output, float* lse, int batch_size,
+                           int h_q, int d_latent, int d_rope, int page_size, int sliding_window,
+                           int causal, float sm_scale) {
+  int d_qk = d_latent + d_rope;
+  float* O_local = (float*)malloc(sizeof(float) * (d_latent + d_qk));
+  float* Q_local = O_local + d_latent;
+  for (int b_idx = 0; b_idx < batch_size; ++b_idx) {
+    int begin = page_indptr[b_idx], end = page_indptr[b_idx + 1];
+    int kv_len = kv_chunk_len(end - begin, page_size, b_idx, length_info, batch_size, sliding_window);
+    int qo_len = q_indptr[b_idx + 1] - q_indptr[b_idx];
+    for (int q_idx = 0; q_idx < qo_len; ++q_idx) {
+      int cur_L = q_indptr[b_idx] + q_idx;
+      for (int h = 0; h < h_q; ++h) {
+        float m_val = -5e4f, d_val = 1.0f;
+        for (int i = 0; i < d_latent; ++i) O_local[i] = 0.0f;
+        for (int i = 0; i < d_qk; ++i) Q_local[i] = h2f(q[((int64_t)cur_L * h_q + h) * d_qk + i]);
+        for (int row_idx = 0; row_idx < kv_len; ++row_idx) {
+          int so = seq_offset(row_idx, b_idx, length_info, batch_size, sliding_window);
+          int page_no = page_values[begin + so / page_size];
+          const f16* kvrow = pages + ((int64_t)page_no * page_size + so % page_size) * d_qk;
+          float S_val = 0.0f;
+          for (int i = 0; i < d_qk; ++i) S_val += Q_local[i] * h2f(kvrow[i]);
+          S_val *= sm_scale * LOG2E_F;
+          float m_prev = m_val;
+          if (causal_mask(causal, q_idx, row_idx, kv_len, qo_len)) {
+            m_val = fmaxf(m_val, S_val);
+          } else {
+            S_val = -5e4f;
+          }
+          float p = exp2f(S_val - m_val);
+          float o_scale = exp2f(m_prev - m_val);
+          d_val = d_val * o_scale + p;
+          for (int i = 0; i < d_latent; ++i) O_local[i] = O_local[i] * o_scale + p * h2f(kvrow[i]);
+        }
+        for (int i = 0; i < d_latent; ++i)
+          output[((int64_t)cur_L * h_q + h) * d_latent + i] = f2h(O_local[i] / d_val);
+        lse[(int64_t)cur_L * h_q + h] = m_val + log2f(d_val);
+      }
+    }
+  }
+  free(O_local);
+}
+
+/* ---- OpenMP-free helper for the benchmark: run orc_decode on a sub-range of the
+ * batch so that several host threads can be timed side by side. ------------------ */
+void orc_decode_range(const f16* Q, const f16* pages, const int32_t* page_table_indptr,
+                      const int32_t* page_table_values, const int32_t* length_info,
+                      const int32_t* k_rope_pos_offset, const int32_t* q_rope_position, f16* output,
+                      float* lse, int b_begin, int b_end, int B, int H_qo, int H_kv, int D,
+                      int page_size, float sm_scale) {
+  /* Non-sliding, rotary_mode 0 only: each batch row is independent, so calling the
+   * literal kernel on a one-row view gives the same numbers as the full call. */
+  for (int b = b_begin; b < b_end; ++b) {
+    int32_t indptr[2] = {page_table_indptr[b], page_table_indptr[b + 1]};
+    orc_decode(Q + (int64_t)b * H_qo * D, pages, indptr, page_table_values, length_info + b,
+               k_rope_pos_offset + b, q_rope_position + b, output + (int64_t)b * H_qo * D,
+               lse + (int64_t)b * H_qo, 1, H_qo, H_kv, D, page_size, 0, 0, 1.0f, 1e4f, sm_scale);
+  }
+}

@@ -1,0 +1,325 @@
+"""Pins the C oracle (oracle/kv_kernels.c) to closed forms, invariants and brute force.
+
+No formula of the oracle is retyped here: the expected values come from oracle/closed_form.py
+(the numpy definitions that the reference's own tests use) and from special cases whose answer
+is known a priori.
+"""
+import numpy as np
+import pytest
+
+from oracle import closed_form as cf
+from oracle import kernels as ok
+from tests.util import assert_close, build_paged_kv
+
+F16 = np.float16
+
+
+# ----------------------------------------------------------------------------- RoPE
+@pytest.mark.parametrize("d", [64, 128])
+def test_rope_matches_closed_form(d):
+    rng = np.random.default_rng(0)
+    hq, hkv = 8, 2
+    positions = np.array([0, 1, 2, 17, 2047, 131071], np.int32)
+    n = len(positions)
+    qkv = rng.standard_normal((n, hq + 2 * hkv, d)).astype(F16)
+    q = np.zeros((n, hq, d), F16)
+    k = np.zeros((n, hkv, d), F16)
+    v = np.zeros((n, hkv, d), F16)
+    ok.fused_rope(qkv, positions, q, k, v, 1)
+    exp_q = cf.apply_rotary(qkv[:, :hq], positions)
+    exp_k = cf.apply_rotary(qkv[:, hq:hq + hkv], positions)
+    # fp16 rounding of the result (2^-11 relative) plus fp32 angle error at pos 131071
+    # (ulp(131071) ~ 0.0078 rad times |x| <~ 4)
+    small = positions < 4096
+    assert_close(q[small], exp_q[small], atol=2e-3, rtol=2e-3, what="q rope")
+    assert_close(k[small], exp_k[small], atol=2e-3, rtol=2e-3, what="k rope")
+    assert_close(q, exp_q, atol=6e-2, rtol=2e-3, what="q rope long")
+    assert np.array_equal(v, qkv[:, hq + hkv:]), "v must be a plain split"
+
+
+def test_rope_invariants():
+    rng = np.random.default_rng(1)
+    d, hq, hkv, n = 128, 4, 4, 5
+    qkv = rng.standard_normal((n, hq + 2 * hkv, d)).astype(F16)
+    q = np.zeros((n, hq, d), F16)
+    k = np.zeros((n, hkv, d), F16)
+    v = np.zeros((n, hkv, d), F16)
+    # position 0 is the identity
+    ok.fused_rope(qkv, np.zeros(n, np.int32), q, k, v, 1)
+    assert np.array_equal(q, qkv[:, :hq]) and np.array_equal(k, qkv[:, hq:hq + hkv])
+    # apply_rope = 0 is a plain split at any position
+    ok.fused_rope(qkv, np.arange(n, dtype=np.int32) * 1000, q, k, v, 0)
+    assert np.array_equal(q, qkv[:, :hq]) and np.array_equal(k, qkv[:, hq:hq + hkv])
+    # rotation preserves the norm of every (d, d + D/2) pair
+    pos = np.array([3, 50, 700, 9000, 65000], np.int32)
+    ok.fused_rope(qkv, pos, q, k, v, 1)
+    x = qkv[:, :hq].astype(np.float64)
+    y = q.astype(np.float64)
+    n_in = x[..., :d // 2] ** 2 + x[..., d // 2:] ** 2
+    n_out = y[..., :d // 2] ** 2 + y[..., d // 2:] ** 2
+    assert_close(n_out, n_in, atol=2e-2, rtol=5e-3, what="pair norm")
+    # the relative-position property: <rope(q,p), rope(k,p)> depends on p only through p-p = 0
+    dot_in = (qkv[:, :hq].astype(np.float64) * np.repeat(qkv[:, hq:hq + hkv], 1, axis=1).astype(np.float64)).sum(-1)
+    dot_out = (q.astype(np.float64) * k.astype(np.float64)).sum(-1)
+    assert_close(dot_out, dot_in, atol=5e-2, rtol=1e-2, what="relative position")
+
+
+# ----------------------------------------------------------------------------- append / gather
+def test_append_gather_round_trip_and_skip():
+    rng = np.random.default_rng(2)
+    hkv, ps, d, npages = 3, 16, 64, 9
+    pages = np.zeros((npages, 2, hkv, ps, d), F16)
+    n = 40
+    slots = rng.permutation(npages * ps)[:n].astype(np.int32)
+    slots[5] = -1
+    k = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    ok.transpose_append(pages, k, v, slots)
+    # brute force: the documented layout pages[p // ps, 0|1, h, p % ps, :]
+    expect = np.zeros_like(pages)
+    for i, p in enumerate(slots):
+        if p >= 0:
+            expect[p // ps, 0, :, p % ps] = k[i]
+            expect[p // ps, 1, :, p % ps] = v[i]
+    assert np.array_equal(pages, expect)
+    keep = slots >= 0
+    kd = np.zeros((2, keep.sum(), hkv, d), F16)
+    vd = np.zeros_like(kd)
+    ok.debug_get_kv(pages, slots[keep], kd, vd, 1)
+    assert np.array_equal(kd[1], k[keep]) and np.array_equal(vd[1], v[keep])
+    assert not kd[0].any()
+
+
+def test_append_gather_mla_round_trip():
+    rng = np.random.default_rng(3)
+    ps, d, npages, n = 64, 576, 4, 70
+    pages = np.zeros((npages, ps, d), F16)
+    slots = rng.permutation(npages * ps)[:n].astype(np.int32)
+    slots[0] = -1
+    kv = rng.standard_normal((n, d)).astype(F16)
+    ok.transpose_append_mla(pages, kv, slots)
+    flat = pages.reshape(npages * ps, d)
+    assert np.array_equal(flat[slots[1:]], kv[1:])
+    assert np.count_nonzero(flat.any(axis=1)) == n - 1
+    out = np.zeros((1, n - 1, d), F16)
+    ok.debug_get_kv_mla(pages, slots[1:], out, 0)
+    assert np.array_equal(out[0], kv[1:])
+
+
+def test_copy_single_page_and_compact_copy():
+    rng = np.random.default_rng(4)
+    hkv, ps, d, npages = 2, 16, 32, 5
+    pages = rng.standard_normal((npages, 2, hkv, ps, d)).astype(F16)
+    before = pages.copy()
+    ok.copy_single_page(pages, 1, 3, 7)
+    assert np.array_equal(pages[3, :, :, :7], before[1, :, :, :7])
+    assert np.array_equal(pages[3, :, :, 7:], before[3, :, :, 7:])
+    assert np.array_equal(np.delete(pages, 3, axis=0), np.delete(before, 3, axis=0))
+    # compact copy: batch of 2, copies src->dst slot by slot
+    before = pages.copy()
+    indptr = np.array([0, 2, 3], np.int32)
+    src_dst = np.array([[20, 21, 70], [17, 18, 65]], np.int32)
+    ok.compact_kv_copy(pages, indptr, src_dst, 2)
+    flat_b = before.transpose(0, 3, 1, 2, 4).reshape(npages * ps, 2, hkv, d)
+    flat_a = pages.transpose(0, 3, 1, 2, 4).reshape(npages * ps, 2, hkv, d)
+    for s, t in src_dst.T:
+        assert np.array_equal(flat_a[t], flat_b[s])
+    mla = rng.standard_normal((4, 64, 576)).astype(F16)
+    mb = mla.copy()
+    ok.copy_single_page_mla(mla, 0, 2, 33)
+    assert np.array_equal(mla[2, :33], mb[0, :33]) and np.array_equal(mla[2, 33:], mb[2, 33:])
+
+
+# ----------------------------------------------------------------------------- attention
+def _decode_case(rng, kv_lens, hq, hkv, d, ps=16, npages=64):
+    pages, indptr, values, last, ks, vs = build_paged_kv(rng, kv_lens, npages, hkv, ps, d)
+    b = len(kv_lens)
+    q = rng.standard_normal((b, hq, d)).astype(F16)
+    out = np.zeros((b, hq, d), F16)
+    lse = np.zeros((b, hq), np.float32)
+    zeros = np.zeros(b, np.int32)
+    ok.decode(q, pages, indptr, values, last, zeros, zeros, out, lse, 0, 1.0, 1e4, d ** -0.5)
+    return q, ks, vs, out, lse
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (4, 4, 64), (8, 1, 128)])
+def test_decode_matches_softmax_closed_form(hq, hkv, d):
+    rng = np.random.default_rng(5)
+    kv_lens = [1, 15, 16, 17, 100, 0]
+    q, ks, vs, out, lse = _decode_case(rng, kv_lens, hq, hkv, d)
+    for i, n in enumerate(kv_lens):
+        if n == 0:
+            assert not out[i].any() and np.all(lse[i] == np.float32(-5e4))
+            continue
+        eo, el = cf.attention(q[i:i + 1], ks[i], vs[i], d ** -0.5, causal=False)
+        assert_close(out[i], eo[0], atol=2e-3, rtol=2e-3, what=f"decode out seq {i}")
+        assert_close(lse[i], el[0], atol=1e-3, rtol=1e-4, what=f"decode lse seq {i}")
+
+
+def test_decode_single_key_returns_its_value():
+    rng = np.random.default_rng(6)
+    q, ks, vs, out, lse = _decode_case(rng, [1], 4, 2, 64)
+    assert np.array_equal(out[0], np.repeat(vs[0][0], 2, axis=0))
+
+
+def _ragged_case(rng, lens, hq, hkv, dqk, dv, causal):
+    n = sum(lens)
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, dqk)).astype(F16)
+    k = rng.standard_normal((n, hkv, dqk)).astype(F16)
+    v = rng.standard_normal((n, hkv, dv)).astype(F16)
+    out = np.zeros((n, hq, dv), F16)
+    lse = np.zeros((n, hq), np.float32)
+    ok.prefill_ragged(q, indptr, k, v, indptr, np.zeros(n, np.int32), np.zeros(len(lens), np.int32),
+                      out, lse, causal, 0, 1.0, 1e4, dqk ** -0.5)
+    return indptr, q, k, v, out, lse
+
+
+@pytest.mark.parametrize("hq,hkv,dqk,dv,causal", [(8, 2, 128, 128, 1), (4, 4, 192, 128, 1), (4, 2, 64, 64, 0)])
+def test_ragged_prefill_matches_closed_form(hq, hkv, dqk, dv, causal):
+    rng = np.random.default_rng(7)
+    lens = [1, 5, 33, 16]
+    indptr, q, k, v, out, lse = _ragged_case(rng, lens, hq, hkv, dqk, dv, causal)
+    for i in range(len(lens)):
+        s, e = indptr[i], indptr[i + 1]
+        eo, el = cf.attention(q[s:e], k[s:e], v[s:e], dqk ** -0.5, causal=bool(causal))
+        assert_close(out[s:e], eo, atol=2e-3, rtol=2e-3, what=f"ragged out seq {i}")
+        assert_close(lse[s:e], el, atol=1e-3, rtol=1e-4, what=f"ragged lse seq {i}")
+
+
+def test_ragged_first_row_sees_only_itself():
+    rng = np.random.default_rng(8)
+    indptr, q, k, v, out, lse = _ragged_case(rng, [9], 4, 2, 64, 64, 1)
+    assert np.array_equal(out[0], np.repeat(v[0], 2, axis=0))
+
+
+@pytest.mark.parametrize("causal", [0, 1])
+def test_paged_prefill_matches_closed_form(causal):
+    rng = np.random.default_rng(9)
+    hq, hkv, d = 8, 2, 128
+    kv_lens = [40, 16, 0, 75]
+    q_lens = [7, 16, 3, 30]
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, kv_lens, 32, hkv, 16, d)
+    n = sum(q_lens)
+    qindptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    out = np.zeros((n, hq, d), F16)
+    lse = np.zeros((n, hq), np.float32)
+    zb = np.zeros(len(kv_lens), np.int32)
+    ok.prefill_paged(q, qindptr, pages, pindptr, pvalues, last, zb, np.zeros(n, np.int32), out, lse,
+                     causal, 0, 1.0, 1e4, d ** -0.5)
+    for i, (nk, nq) in enumerate(zip(kv_lens, q_lens)):
+        s, e = qindptr[i], qindptr[i + 1]
+        if nk == 0:
+            assert not out[s:e].any() and np.all(lse[s:e] == np.float32(-5e4))
+            continue
+        eo, el = cf.attention(q[s:e], ks[i], vs[i], d ** -0.5, causal=bool(causal))
+        assert_close(out[s:e], eo, atol=2e-3, rtol=2e-3, what=f"paged out seq {i}")
+        assert_close(lse[s:e], el, atol=1e-3, rtol=1e-4, what=f"paged lse seq {i}")
+
+
+def test_decode_equals_paged_prefill_with_one_query():
+    rng = np.random.default_rng(10)
+    hq, hkv, d = 8, 4, 64
+    kv_lens = [33, 7]
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, kv_lens, 8, hkv, 16, d)
+    q = rng.standard_normal((2, hq, d)).astype(F16)
+    o1, o2 = np.zeros((2, hq, d), F16), np.zeros((2, hq, d), F16)
+    l1, l2 = np.zeros((2, hq), np.float32), np.zeros((2, hq), np.float32)
+    z = np.zeros(2, np.int32)
+    ok.decode(q, pages, pindptr, pvalues, last, z, z, o1, l1, 0, 1.0, 1e4, 0.125)
+    ok.prefill_paged(q, np.array([0, 1, 2], np.int32), pages, pindptr, pvalues, last, z, z, o2, l2,
+                     0, 0, 1.0, 1e4, 0.125)
+    assert np.array_equal(o1, o2) and np.array_equal(l1, l2)
+
+
+def test_inline_rope_equals_rope_then_attend():
+    """rotary_mode=1 inside the kernels must equal RoPE applied up front (NORMAL mode)."""
+    rng = np.random.default_rng(11)
+    hq, hkv, d, n = 4, 2, 64, 21
+    k_raw = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    q_raw = rng.standard_normal((1, hq, d)).astype(F16)
+    pages = np.zeros((4, 2, hkv, 16, d), F16)
+    slots = np.arange(n, dtype=np.int32) + 16
+    ok.transpose_append(pages, k_raw, v, slots)
+    pindptr, pvalues, last = np.array([0, 2], np.int32), np.array([1, 2], np.int32), np.array([5], np.int32)
+    out_inline = np.zeros((1, hq, d), F16)
+    lse_inline = np.zeros((1, hq), np.float32)
+    ok.decode(q_raw, pages, pindptr, pvalues, last, np.array([100], np.int32), np.array([100 + n - 1], np.int32),
+              out_inline, lse_inline, 1, 1.0, 1e4, d ** -0.5)
+    k_rot = cf.apply_rotary(k_raw, 100 + np.arange(n)).astype(F16)
+    q_rot = cf.apply_rotary(q_raw, [100 + n - 1]).astype(F16)
+    eo, el = cf.attention(q_rot, k_rot, v, d ** -0.5, causal=False)
+    assert_close(out_inline[0], eo[0], atol=3e-3, rtol=3e-3, what="inline rope out")
+
+
+# ----------------------------------------------------------------------------- merge
+def test_merge_closed_form_and_special_cases():
+    rng = np.random.default_rng(12)
+    n, h, d = 6, 4, 64
+    v1 = rng.standard_normal((n, h, d)).astype(F16)
+    v2 = rng.standard_normal((n, h, d)).astype(F16)
+    s1 = (rng.standard_normal((n, h)) * 3).astype(np.float32)
+    s2 = (rng.standard_normal((n, h)) * 3).astype(np.float32)
+    s2[0] = -5e4  # empty other side -> unchanged
+    s2[1] = s1[1]  # equal weights -> mean
+    ev, es = cf.merge(v1, s1, v2, s2)
+    mv, ms = v1.copy(), s1.copy()
+    ok.merge_state_inplace(mv, ms, v2, s2)
+    assert_close(mv, ev, atol=1e-3, rtol=1e-3, what="merge v")
+    assert_close(ms, es, atol=1e-5, rtol=1e-6, what="merge s")
+    assert np.array_equal(mv[0], v1[0]) and np.array_equal(ms[0], s1[0])
+    assert_close(mv[1], (v1[1].astype(np.float64) + v2[1].astype(np.float64)) / 2, atol=1e-3, rtol=1e-3)
+
+
+def test_self_plus_cross_merge_equals_full_attention():
+    """merge(ragged causal over the chunk, paged non-causal over the prefix) = attention over
+    prefix+chunk: the identity the chunked-prefill composition of the cache relies on."""
+    rng = np.random.default_rng(13)
+    hq, hkv, d = 8, 2, 128
+    prefix, chunk = 45, 19
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, [prefix], 8, hkv, 16, d)
+    q = rng.standard_normal((chunk, hq, d)).astype(F16)
+    k = rng.standard_normal((chunk, hkv, d)).astype(F16)
+    v = rng.standard_normal((chunk, hkv, d)).astype(F16)
+    ind = np.array([0, chunk], np.int32)
+    o_self, l_self = np.zeros((chunk, hq, d), F16), np.zeros((chunk, hq), np.float32)
+    o_cross, l_cross = np.zeros((chunk, hq, d), F16), np.zeros((chunk, hq), np.float32)
+    z1 = np.zeros(1, np.int32)
+    zc = np.zeros(chunk, np.int32)
+    ok.prefill_ragged(q, ind, k, v, ind, zc, z1, o_self, l_self, 1, 0, 1.0, 1e4, d ** -0.5)
+    ok.prefill_paged(q, ind, pages, pindptr, pvalues, last, z1, zc, o_cross, l_cross, 0, 0, 1.0, 1e4, d ** -0.5)
+    ok.merge_state_inplace(o_self, l_self, o_cross, l_cross)
+    eo, el = cf.attention(q, np.concatenate([ks[0], k]), np.concatenate([vs[0], v]), d ** -0.5, causal=True)
+    assert_close(o_self, eo, atol=3e-3, rtol=3e-3, what="merged out")
+    assert_close(l_self, el, atol=1e-3, rtol=1e-4, what="merged lse")
+
+
+# ----------------------------------------------------------------------------- MLA
+def test_mla_absorbed_equals_expanded_definition():
+    """Absorbed latent attention (what the paged MLA kernel computes) against the definition:
+    expand the latent with w_kv and run plain multi-head attention."""
+    rng = np.random.default_rng(14)
+    h, d_lat, d_rope, d_nope, d_v, ps = 4, 32, 8, 16, 12, 8
+    prefix, nq = 21, 3
+    latent = (rng.standard_normal((prefix, d_lat + d_rope)) * 0.5).astype(F16)
+    w_kv = (rng.standard_normal((d_lat, h * (d_nope + d_v))) * 0.3).astype(np.float64)
+    pages = np.zeros((5, ps, d_lat + d_rope), F16)
+    page_ids = np.array([3, 0, 4], np.int32)
+    slots = np.array([page_ids[t // ps] * ps + t % ps for t in range(prefix)], np.int32)
+    ok.transpose_append_mla(pages, latent, slots)
+    q = (rng.standard_normal((nq, h, d_nope + d_rope)) * 0.5).astype(np.float64)
+    w = w_kv.reshape(d_lat, h, d_nope + d_v)
+    w_uk, w_uv = w[..., :d_nope], w[..., d_nope:]
+    q_abs = np.concatenate([np.einsum("qhn,lhn->qhl", q[..., :d_nope], w_uk), q[..., d_nope:]], axis=-1).astype(F16)
+    out = np.zeros((nq, h, d_lat), F16)
+    lse = np.zeros((nq, h), np.float32)
+    sm = (d_nope + d_rope) ** -0.5
+    ok.prefill_paged_mla(q_abs, np.array([0, nq], np.int32), pages, np.array([0, 3], np.int32), page_ids,
+                         np.array([prefix - 2 * ps], np.int32), out, lse, 0, sm, d_latent=d_lat)
+    k_full, v_full = cf.mla_expand(latent, w_kv, h, d_nope, d_v)
+    eo, el = cf.attention(q, k_full, v_full, sm, causal=False)
+    got = np.einsum("qhl,lhv->qhv", out.astype(np.float64), w_uv)
+    assert_close(got, eo, atol=1e-2, rtol=1e-2, what="mla out")
+    assert_close(lse, el, atol=2e-2, rtol=1e-3, what="mla lse")
