@@ -1,0 +1,300 @@
+/*
+ * tvmkv -- MI355X (gfx950) paged KV-cache attention behind the interface of apache/tvm's
+ * PagedAttentionKVCache.  C ABI: plain pointers and sizes, no C++ or framework types.
+ *
+ * Two layers, both exported from libtvmkv.so:
+ *
+ *  (1) KERNEL LAUNCHERS.  One per kernel slot that the reference's
+ *      `vm.builtin.paged_attention_kv_cache_create` takes as an ffi::Function
+ *      (src/runtime/vm/paged_kv_cache.cc:2562-2585).  Tensor arguments appear in the order
+ *      of the reference's "tirx" calling convention (src/runtime/vm/attn_backend.h); what a
+ *      DLTensor would carry implicitly (shapes, byte_offset-adjusted data pointers, the
+ *      stream) is passed explicitly after them.  All data pointers are DEVICE pointers, fp16
+ *      for K/V/Q/O data, int32 for index arrays, fp32 for log-sum-exp.  Index arrays that the
+ *      reference passes as views with a non-zero byte_offset (src/runtime/vm/attn_utils.h:
+ *      1027-1035) must already have that offset added.  `stream` is a hipStream_t (NULL = the
+ *      null stream).  Launchers are asynchronous and never synchronise the device.
+ *
+ *  (2) CACHE OBJECT.  `tvmkv_cache_*` / `tvmkv_kv_state_*` / `tvmkv_attention_kv_cache_*`:
+ *      the host-side page pool, block tree and per-step auxiliary arrays, with the verbs and
+ *      error behaviour of the reference's global functions `vm.builtin.kv_state_*` and
+ *      `vm.builtin.attention_kv_cache_*` (src/runtime/vm/kv_state.cc:33-116), calling (1).
+ *
+ * Error convention: every function returning int returns 0 on success and a negative
+ * TVMKV_E* code on failure; tvmkv_last_error() then returns a thread-local message (the
+ * text of the reference's failed check where one exists).  Nothing throws across the ABI.
+ *
+ * Threading: a cache object is not thread-safe (neither is the reference's).  The split-KV
+ * decode launcher uses one lazily grown workspace per device: calls on the same device must
+ * be ordered on one stream.
+ */
+#ifndef TVMKV_H_
+#define TVMKV_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TVMKV_OK 0
+#define TVMKV_EINVAL (-1)      /* a check of the reference failed (bad argument / state)   */
+#define TVMKV_EUNSUPPORTED (-2) /* valid in the reference, not built here (clear message)   */
+#define TVMKV_EDEVICE (-3)     /* a HIP runtime call failed                                */
+#define TVMKV_ENODEVICE (-4)   /* device work requested from a host-only cache             */
+
+/* Thread-local message of the last failed call on this thread ("" if none). */
+const char* tvmkv_last_error(void);
+/* Library version string. */
+const char* tvmkv_version(void);
+
+/* ======================================================================================
+ * (1) Kernel launchers
+ * ====================================================================================== */
+
+/* Slot 24 `f_split_rotary` -- replaces `fused_rope`
+ * (python/tvm/relax/frontend/nn/llm/position_embedding.py:525-565), called at
+ * src/runtime/vm/paged_kv_cache.cc:1360-1366 as (qkv, q_rope_position_map, q, k, v, apply_rope).
+ * qkv (seq_len, num_q_heads + 2*num_kv_heads, head_dim) -> q (seq_len, num_q_heads, head_dim),
+ * k, v (seq_len, num_kv_heads, head_dim); rotate-half RoPE on q and k in fp32 when apply_rope>0.
+ * theta/scale are baked into the reference kernel at build time; here they are arguments. */
+int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
+                     int64_t apply_rope, int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
+                     int32_t head_dim, double rope_scale, double rope_theta, void* stream);
+
+/* Slot 13 `f_transpose_append_mha` -- replaces `tir_kv_cache_transpose_append`
+ * (python/tvm/relax/frontend/nn/llm/_page_kernels.py:40-74), called at paged_kv_cache.cc:1371
+ * as (pages, k_data, v_data, position_map).  pages (num_pages, 2, num_kv_heads, page_size,
+ * head_dim); row i goes to slot position_map[i] (= page*page_size + offset), -1 = skip. */
+int tvmkv_kv_cache_transpose_append(void* pages, const void* k_data, const void* v_data,
+                                    const int32_t* position_map, int64_t ntoken, int64_t num_pages,
+                                    int32_t num_kv_heads, int32_t page_size, int32_t head_dim,
+                                    void* stream);
+
+/* Slot 14 `f_transpose_append_mla` -- replaces `tir_kv_cache_transpose_append_mla`
+ * (_page_kernels.py:77-103), called at paged_kv_cache.cc:1550 as (pages, kv_data, position_map).
+ * pages (num_pages, page_size, d_qk). */
+int tvmkv_kv_cache_transpose_append_mla(void* pages, const void* kv_data, const int32_t* position_map,
+                                        int64_t ntoken, int64_t num_pages, int32_t page_size,
+                                        int32_t d_qk, void* stream);
+
+/* Slot 15 ragged prefill -- replaces `batch_prefill_ragged_kv`
+ * (python/tvm/relax/frontend/nn/llm/_prefill_kernels.py:795-923; llvm form :677-791), calling
+ * convention src/runtime/vm/attn_backend.h:392-395:
+ * (q, qo_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_offset, out, lse, causal,
+ *  rotary_mode, rope_scale, rope_theta, sm_scale).
+ * q (total_q, h_q, d_qk), k (total_kv, h_kv, d_qk), v (total_kv, h_kv, d_v),
+ * out (total_q, h_q, d_v) fp16, lse (total_q, h_q) fp32 base-2.  rotary_mode must be 0 (RoPE
+ * applied up front); 1 (inline RoPE) returns TVMKV_EUNSUPPORTED. */
+int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                                  const int32_t* kv_indptr, const int32_t* q_rope_position,
+                                  const int32_t* k_rope_pos_offset, void* output, float* lse,
+                                  int64_t causal, int64_t rotary_mode, double rope_scale,
+                                  double rope_theta, double sm_scale, int32_t batch_size,
+                                  int64_t total_q, int32_t h_q, int32_t h_kv, int32_t d_qk,
+                                  int32_t d_v, void* stream);
+
+/* Slots 16/18 paged prefill -- replaces `batch_prefill_paged_kv`
+ * (_prefill_kernels.py:217-391; llvm form :54-214), calling convention attn_backend.h:239-242:
+ * (q, qo_indptr, pages, page_indptr, page_indices, length_info, k_rope_pos_offset,
+ *  q_rope_position, out, lse, causal, rotary_mode, rope_scale, rope_theta, sm_scale).
+ * length_info is (batch,) = last_page_len, or (3, batch) = [last_page_len; sliding_window_offset;
+ * sink_size] when sliding_window != 0 (python/tvm/relax/frontend/nn/llm/_kernel_common.py:147-170).
+ * kv_len = (npages-1)*page_size + last_page_len, 0 without pages. */
+int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const void* pages,
+                                 const int32_t* page_indptr, const int32_t* page_values,
+                                 const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                                 const int32_t* q_rope_position, void* output, float* lse,
+                                 int64_t causal, int64_t rotary_mode, double rope_scale,
+                                 double rope_theta, double sm_scale, int32_t batch_size,
+                                 int64_t total_q, int64_t nnz_pages, int64_t num_pages, int32_t h_q,
+                                 int32_t h_kv, int32_t d, int32_t page_size, int32_t sliding_window,
+                                 int32_t sliding_window_size, void* stream);
+
+/* Slots 17/19 paged decode -- replaces `batch_decode_paged_kv`
+ * (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:181-411; llvm form :49-178), calling
+ * convention attn_backend.h:511-514:
+ * (q, pages, page_indptr, page_indices, length_info, k_rope_pos_offset, q_rope_position, out,
+ *  lse, rotary_mode, rope_scale, rope_theta, sm_scale).
+ * q/out (B, h_q, d) fp16, lse (B, h_q) fp32.  Split-KV across workgroups with a merge pass;
+ * the partition count is derived from B and nnz_pages only (no host read of the page table). */
+int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t* page_indptr,
+                                const int32_t* page_values, const int32_t* length_info,
+                                const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,
+                                void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                                double rope_theta, double sm_scale, int32_t batch_size,
+                                int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                                int32_t d, int32_t page_size, int32_t sliding_window, void* stream);
+
+/* Slot 22 MLA paged prefill (also used for MLA decode, paged_kv_cache.cc:954-956) -- replaces
+ * `batch_prefill_paged_kv_mla` (_prefill_kernels.py:927-1071), calling convention
+ * attn_backend.h:248-249: (q, qo_indptr, pages, page_indptr, page_indices, length_info, out, lse,
+ * causal, sm_scale).  q (total_q, h_q, d_latent + d_rope), pages (num_pages, page_size,
+ * d_latent + d_rope), out (total_q, h_q, d_latent). */
+int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_indptr, const void* pages,
+                                     const int32_t* page_indptr, const int32_t* page_values,
+                                     const int32_t* length_info, void* output, float* lse,
+                                     int64_t causal, double sm_scale, int32_t batch_size,
+                                     int64_t total_q, int64_t nnz_pages, int64_t num_pages,
+                                     int32_t h_q, int32_t d_latent, int32_t d_rope,
+                                     int32_t page_size, void* stream);
+
+/* Slot 23 `f_merge_inplace` -- replaces `merge_state_inplace` (_decode_kernels.py:455-526),
+ * called at paged_kv_cache.cc:2292, :2329, :1557 as (v, s, v_other, s_other).
+ * v (N, H, D) fp16 and s (N, H) fp32 are updated in place. */
+int tvmkv_merge_state_inplace(void* v, float* s, const void* v_other, const float* s_other,
+                              int64_t n, int32_t h, int32_t d, void* stream);
+
+/* Slot 25 `f_copy_single_page` -- replaces `copy_single_page` / `copy_single_page_mla`
+ * (_page_kernels.py:169-210), called at paged_kv_cache.cc:728 as
+ * (pages, src_page_id, tgt_page_id, copy_length). */
+int tvmkv_copy_single_page(void* pages, int64_t src_page_id, int64_t tgt_page_id, int64_t copy_length,
+                           int64_t num_pages, int32_t num_kv_heads, int32_t page_size,
+                           int32_t head_dim, void* stream);
+int tvmkv_copy_single_page_mla(void* pages, int64_t src_page_id, int64_t tgt_page_id,
+                               int64_t copy_length, int64_t num_pages, int32_t page_size,
+                               int32_t d_qk, void* stream);
+
+/* Slot 26 `f_debug_get_kv` -- replaces `tir_kv_cache_debug_get_kv(_mla)`
+ * (_page_kernels.py:106-166), called at paged_kv_cache.cc:1718 / :1764 as
+ * (pages, position_map, k_data, v_data, layer_id) / (pages, position_map, kv_data, layer_id).
+ * k_data/v_data (num_layers, seqlen, num_kv_heads, head_dim); writes layer `layer_id`. */
+int tvmkv_kv_cache_debug_get_kv(const void* pages, const int32_t* position_map, void* k_data,
+                                void* v_data, int64_t layer_id, int64_t seqlen, int64_t num_pages,
+                                int32_t num_kv_heads, int32_t page_size, int32_t head_dim,
+                                void* stream);
+int tvmkv_kv_cache_debug_get_kv_mla(const void* pages, const int32_t* position_map, void* kv_data,
+                                    int64_t layer_id, int64_t seqlen, int64_t num_pages,
+                                    int32_t page_size, int32_t d_qk, void* stream);
+
+/* Slot 27 `f_compact_copy` -- replaces `compact_kv_copy` (_page_kernels.py:235-263), called at
+ * paged_kv_cache.cc:759-760 as (pages, copy_length_indptr, copy_src_dst_pos, batch_size).
+ * copy_src_dst_pos is (2, total_copy_length): row 0 = source slots, row 1 = destination slots. */
+int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr,
+                          const int32_t* copy_src_dst_pos, int32_t batch_size,
+                          int32_t total_copy_length, int64_t num_pages, int32_t num_kv_heads,
+                          int32_t page_size, int32_t head_dim, void* stream);
+
+/* ======================================================================================
+ * (2) Cache object
+ * ====================================================================================== */
+
+typedef struct tvmkv_cache tvmkv_cache;
+
+/* attn_kinds values (src/runtime/vm/attn_utils.h:66-71) and rope modes (:341-345). */
+#define TVMKV_ATTN_MHA 0
+#define TVMKV_ATTN_MLA 1
+#define TVMKV_ATTN_MHA_SLIDING 3
+#define TVMKV_ROPE_NONE 0
+#define TVMKV_ROPE_NORMAL 1
+#define TVMKV_ROPE_INLINE 2
+
+/* `vm.builtin.paged_attention_kv_cache_create` (paged_kv_cache.cc:2532-2640) without the
+ * kernel-function arguments (the kernels are this library's own).
+ *   cache_config  [reserved_num_seqs, total_token_capacity, prefill_chunk_size, page_size,
+ *                  support_sliding_window(, layer_sliding_window_size)]   (n_config 5 or 6)
+ *   layer_indptr  [begin, end] layer range owned by this cache (one group: {0, num_layers})
+ *   attn_kinds    one TVMKV_ATTN_* per global layer id
+ *   dtype_bits    16 (fp16 storage; the only one built)
+ *   device_id     HIP device ordinal, or -1 for a HOST-ONLY cache: page-pool bookkeeping and
+ *                 auxiliary arrays work, anything that touches device memory returns
+ *                 TVMKV_ENODEVICE. */
+int tvmkv_cache_create(const int64_t* cache_config, int32_t n_config, const int64_t* layer_indptr,
+                       int32_t n_layer_indptr, int64_t num_qo_heads, int64_t num_kv_heads,
+                       int64_t qk_head_dim, int64_t v_head_dim, const int64_t* attn_kinds,
+                       int32_t n_attn_kinds, int32_t enable_kv_transfer, int32_t rope_mode,
+                       double rope_scale, double rope_theta, int32_t dtype_bits, int32_t device_id,
+                       tvmkv_cache** out);
+void tvmkv_cache_destroy(tvmkv_cache* cache);
+/* Stream on which the cache enqueues kernels (the reference uses the device's current stream,
+ * paged_kv_cache.cc:524).  Default: the null stream. */
+int tvmkv_cache_set_stream(tvmkv_cache* cache, void* stream);
+
+/* vm.builtin.kv_state_* (src/runtime/vm/kv_state.cc:33-55). */
+int tvmkv_kv_state_clear(tvmkv_cache* cache);
+int tvmkv_kv_state_add_sequence(tvmkv_cache* cache, int64_t seq_id);
+int tvmkv_kv_state_remove_sequence(tvmkv_cache* cache, int64_t seq_id);
+int tvmkv_kv_state_fork_sequence(tvmkv_cache* cache, int64_t parent_seq_id, int64_t child_seq_id,
+                                 int64_t fork_pos);
+int tvmkv_kv_state_popn(tvmkv_cache* cache, int64_t seq_id, int32_t n);
+/* token_tree_parent_ptr may be NULL (n_tree ignored). */
+int tvmkv_kv_state_begin_forward(tvmkv_cache* cache, const int64_t* seq_ids,
+                                 const int64_t* append_lengths, int32_t batch_size,
+                                 const int64_t* token_tree_parent_ptr, int32_t n_tree);
+int tvmkv_kv_state_end_forward(tvmkv_cache* cache);
+
+/* vm.builtin.attention_kv_cache_* (src/runtime/vm/kv_state.cc:58-116).  Tensors are device
+ * pointers to contiguous arrays; the row counts are shape[0] of the reference's tensors. */
+int tvmkv_attention_kv_cache_enable_sliding_window_for_seq(tvmkv_cache* cache, int64_t seq_id,
+                                                           int32_t sliding_window_size,
+                                                           int32_t attn_sink_size);
+int tvmkv_attention_kv_cache_commit_accepted_token_tree_nodes(tvmkv_cache* cache,
+                                                              const int64_t* seq_ids,
+                                                              const int64_t* leaf_indices,
+                                                              int32_t n);
+int tvmkv_attention_kv_cache_empty(tvmkv_cache* cache, int32_t* out);
+int tvmkv_attention_kv_cache_get_num_available_pages(tvmkv_cache* cache, int32_t* out);
+int tvmkv_attention_kv_cache_get_total_sequence_length(tvmkv_cache* cache, int32_t* out);
+/* Returns a device pointer to q_rope_position_map (int32) and its length. */
+int tvmkv_attention_kv_cache_get_query_positions(tvmkv_cache* cache, const int32_t** device_ptr,
+                                                 int64_t* length);
+/* (cache, layer_id, sm_scale, qkv, out): qkv (qkv_rows, Hq+2Hkv, D), out (out_rows, Hq, D). */
+int tvmkv_attention_kv_cache_attention_with_fused_qkv(tvmkv_cache* cache, int64_t layer_id,
+                                                      double sm_scale, const void* qkv,
+                                                      int64_t qkv_rows, void* out, int64_t out_rows);
+/* (cache, layer_id, sm_scale, q, k, v, o, lse): rows must equal the batch's total append length. */
+int tvmkv_attention_kv_cache_self_attention(tvmkv_cache* cache, int64_t layer_id, double sm_scale,
+                                            const void* q, const void* k, const void* v, void* o,
+                                            float* lse, int64_t rows, int32_t k_heads,
+                                            int32_t qk_dim, int32_t v_dim);
+/* (cache, layer_id, sm_scale, q, o, lse). */
+int tvmkv_attention_kv_cache_cross_attention(tvmkv_cache* cache, int64_t layer_id, double sm_scale,
+                                             const void* q, void* o, float* lse, int64_t rows);
+/* (cache, layer_id, kv): kv (rows, qk_head_dim). */
+int tvmkv_attention_kv_cache_append_mla_kv(tvmkv_cache* cache, int64_t layer_id, const void* kv,
+                                           int64_t rows);
+/* (cache, o_self, lse_self, o_cross, lse_cross): merges into o_self / lse_self. */
+int tvmkv_attention_kv_cache_merge_attn_output_inplace(tvmkv_cache* cache, void* o_self,
+                                                       float* lse_self, const void* o_cross,
+                                                       const float* lse_cross, int64_t rows,
+                                                       int32_t heads, int32_t dim);
+/* (cache, seq_id, start_pos, end_pos, k_data, v_data): (num_layers, end-start, Hkv, D) each.
+ * Synchronises the stream before returning (debug path). */
+int tvmkv_attention_kv_cache_debug_get_kv(tvmkv_cache* cache, int64_t seq_id, int64_t start_pos,
+                                          int64_t end_pos, void* k_data, void* v_data);
+int tvmkv_attention_kv_cache_debug_get_kv_mla(tvmkv_cache* cache, int64_t seq_id, int64_t start_pos,
+                                              int64_t end_pos, void* kv_data);
+
+/* ---- introspection (no counterpart in the reference's public functions; used by the parity
+ * tests to compare page tables, append indices and pool state bit for bit) --------------- */
+
+/* Host copy of one auxiliary array built by begin_forward.  `name` is the reference's member
+ * name without the `_on_depths_host_` / `_host_` suffix: "qo_indptr", "page_indptr",
+ * "page_indices", "last_page_len", "sliding_window_offset", "sink_size", "k_rope_pos_offset",
+ * "page_indptr_sliding_window", "page_indices_sliding_window",
+ * "k_rope_pos_offset_sliding_window", "tree_attn_mask", "tree_attn_mn_indptr" (per depth) and
+ * "q_rope_position_map", "append_position_map", "cur_append_lengths_indptr",
+ * "k_ragged_rope_pos_offset", "commit_copy_length_indptr", "commit_copy_src_pos",
+ * "commit_copy_dst_pos" (depth ignored).  The pointer stays valid until the next call on the cache. */
+int tvmkv_cache_get_aux(tvmkv_cache* cache, const char* name, int32_t depth, const int32_t** data,
+                        int64_t* size);
+/* flags[0]=num_depths, [1]=append_before_attn, [2]=is_decode_request,
+ * [3..4]=use_decode_kernel per depth, [5..6]=is_chain per depth, [7]=num_total_pages,
+ * [8]=rope_mode in effect. */
+int tvmkv_cache_get_flags(tvmkv_cache* cache, int64_t* flags, int32_t n_flags);
+/* Serialises the pool into `buf` (int64): [n_free_pages, pages..., n_free_blocks, blocks...,
+ * n_blocks, {n_pages, pages..., seq_length, start_pos, sink_length, sliding_window_offset,
+ * parent_idx, external_ref_cnt}..., n_seqs, {seq_id, last_block_idx, seq_length,
+ * sliding_window_size, last_block_attn_sink_size}... (ascending seq_id)].  *needed receives the
+ * element count; returns TVMKV_EINVAL if cap is too small (call again with a bigger buffer). */
+int tvmkv_cache_dump_state(tvmkv_cache* cache, int64_t* buf, int64_t cap, int64_t* needed);
+/* Log of the page copies issued by fork (src, tgt, length) triples since the last clear. */
+int tvmkv_cache_get_copy_log(tvmkv_cache* cache, const int64_t** triples, int64_t* n_triples);
+/* Device pointer of one layer's page pool (local layer index). */
+int tvmkv_cache_get_pages(tvmkv_cache* cache, int64_t local_layer, void** device_ptr,
+                          int64_t* num_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TVMKV_H_ */

@@ -1,0 +1,98 @@
+"""Loader of libtvmkv.so.  There is no fallback: if the library is missing or does not export
+a symbol declared in include/tvmkv.h, importing this module raises."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libtvmkv.so")
+
+c_i32, c_i64, c_f64, c_vp = ctypes.c_int32, ctypes.c_int64, ctypes.c_double, ctypes.c_void_p
+p_i32, p_i64 = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64)
+
+
+class KVError(RuntimeError):
+    """A failed call into libtvmkv; carries the library's error code and message (the text of
+    the reference's failed check where one exists)."""
+
+    def __init__(self, code, message):
+        super().__init__(message)
+        self.code = code
+
+
+# name -> argument ctypes, in the order of include/tvmkv.h
+SIGNATURES = {
+    "tvmkv_fused_rope": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_i32, c_f64, c_f64, c_vp],
+    "tvmkv_kv_cache_transpose_append": [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_kv_cache_transpose_append_mla": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_vp],
+    "tvmkv_batch_prefill_ragged_kv": [c_vp] * 9 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i32, c_i32,
+                                                   c_i32, c_i32, c_vp],
+    "tvmkv_batch_prefill_paged_kv": [c_vp] * 10 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i64,
+                                                   c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_batch_decode_paged_kv": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32, c_i32,
+                                                 c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_batch_prefill_paged_kv_mla": [c_vp] * 8 + [c_i64, c_f64, c_i32, c_i64, c_i64, c_i64, c_i32, c_i32,
+                                                      c_i32, c_i32, c_vp],
+    "tvmkv_merge_state_inplace": [c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_i32, c_vp],
+    "tvmkv_copy_single_page": [c_vp, c_i64, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_copy_single_page_mla": [c_vp, c_i64, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
+    "tvmkv_kv_cache_debug_get_kv": [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_kv_cache_debug_get_kv_mla": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
+    "tvmkv_compact_kv_copy": [c_vp, c_vp, c_vp, c_i32, c_i32, c_i64, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_cache_create": [p_i64, c_i32, p_i64, c_i32, c_i64, c_i64, c_i64, c_i64, p_i64, c_i32, c_i32, c_i32,
+                           c_f64, c_f64, c_i32, c_i32, ctypes.POINTER(c_vp)],
+    "tvmkv_cache_set_stream": [c_vp, c_vp],
+    "tvmkv_kv_state_clear": [c_vp],
+    "tvmkv_kv_state_add_sequence": [c_vp, c_i64],
+    "tvmkv_kv_state_remove_sequence": [c_vp, c_i64],
+    "tvmkv_kv_state_fork_sequence": [c_vp, c_i64, c_i64, c_i64],
+    "tvmkv_kv_state_popn": [c_vp, c_i64, c_i32],
+    "tvmkv_kv_state_begin_forward": [c_vp, p_i64, p_i64, c_i32, p_i64, c_i32],
+    "tvmkv_kv_state_end_forward": [c_vp],
+    "tvmkv_attention_kv_cache_enable_sliding_window_for_seq": [c_vp, c_i64, c_i32, c_i32],
+    "tvmkv_attention_kv_cache_commit_accepted_token_tree_nodes": [c_vp, p_i64, p_i64, c_i32],
+    "tvmkv_attention_kv_cache_empty": [c_vp, p_i32],
+    "tvmkv_attention_kv_cache_get_num_available_pages": [c_vp, p_i32],
+    "tvmkv_attention_kv_cache_get_total_sequence_length": [c_vp, p_i32],
+    "tvmkv_attention_kv_cache_get_query_positions": [c_vp, ctypes.POINTER(c_vp), p_i64],
+    "tvmkv_attention_kv_cache_attention_with_fused_qkv": [c_vp, c_i64, c_f64, c_vp, c_i64, c_vp, c_i64],
+    "tvmkv_attention_kv_cache_self_attention": [c_vp, c_i64, c_f64, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i32,
+                                                c_i32, c_i32],
+    "tvmkv_attention_kv_cache_cross_attention": [c_vp, c_i64, c_f64, c_vp, c_vp, c_vp, c_i64],
+    "tvmkv_attention_kv_cache_append_mla_kv": [c_vp, c_i64, c_vp, c_i64],
+    "tvmkv_attention_kv_cache_merge_attn_output_inplace": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_i32],
+    "tvmkv_attention_kv_cache_debug_get_kv": [c_vp, c_i64, c_i64, c_i64, c_vp, c_vp],
+    "tvmkv_attention_kv_cache_debug_get_kv_mla": [c_vp, c_i64, c_i64, c_i64, c_vp],
+    "tvmkv_cache_get_aux": [c_vp, ctypes.c_char_p, c_i32, ctypes.POINTER(p_i32), p_i64],
+    "tvmkv_cache_get_flags": [c_vp, p_i64, c_i32],
+    "tvmkv_cache_dump_state": [c_vp, p_i64, c_i64, p_i64],
+    "tvmkv_cache_get_copy_log": [c_vp, ctypes.POINTER(p_i64), p_i64],
+    "tvmkv_cache_get_pages": [c_vp, c_i64, ctypes.POINTER(c_vp), p_i64],
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library with argtypes set.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "or `make -C tvm_amd/csrc`. There is no CPU fallback.")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, argtypes in SIGNATURES.items():
+            fn = getattr(handle, name)  # AttributeError if the symbol is not exported
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+        handle.tvmkv_cache_destroy.argtypes = [c_vp]
+        handle.tvmkv_cache_destroy.restype = None
+        handle.tvmkv_last_error.restype = ctypes.c_char_p
+        handle.tvmkv_version.restype = ctypes.c_char_p
+        _lib = handle
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise KVError(rc, lib().tvmkv_last_error().decode())

@@ -1,0 +1,381 @@
+// Batched paged decode attention for gfx950, written as an HBM-bound streaming kernel.
+//
+// Replaces batch_decode_paged_kv (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:181-411),
+// which walks the whole KV of one (sequence, kv head) in a single block.  Here the KV of a
+// sequence is cut into chunks of `chunk_pages` pages; every (chunk, kv head) is one workgroup,
+// so a handful of very long sequences still fill 256 CUs, and a second kernel merges the
+// per-chunk partial states.  Arithmetic follows the reference: scores scaled by
+// sm_scale*log2(e), base-2 online softmax with m = -5e4, d = 1 as the initial state, fp32
+// accumulation, output O/d rounded once to fp16, lse = m + log2(d).
+//
+// Data path of one workgroup (4 wavefronts, one kv head, all `GROUP` query heads of it):
+//   * wave w takes pages w, w+4, ... of the chunk; a page of one kv head is 4 KiB of K and
+//     4 KiB of V, each contiguous, read with 16-byte loads: 16 lanes cover one 256-byte row,
+//     one wave-wide load covers 4 rows = 1 KiB, fully coalesced; the next page's loads are
+//     issued before the current page is consumed;
+//   * q.k: packed fp16 dot products accumulate in fp32 per lane, then a 4-step DPP reduction
+//     inside the 16-lane row; every 16-lane group keeps its own online-softmax state, so the
+//     inner loop has no cross-group traffic;
+//   * at the end the four lane groups are merged with wavefront shuffles, the four waves
+//     through LDS, and the chunk result goes either straight to the output (single-chunk
+//     sequence) or to the fp32 partial buffer.
+//
+// Chunk slots without a prologue kernel: sequence b owns slots
+//   [floor(page_indptr[b]/CP) + b, floor(page_indptr[b+1]/CP) + b + 1)
+// which always holds ceil(npages_b/CP) chunks; a workgroup finds its sequence by binary search
+// on page_indptr, so the grid size depends on shapes only (floor(nnz_pages/CP) + B slots).
+#include "kernels_common.cuh"
+
+namespace tvmkv {
+
+struct DecodeParams {
+  const half_t* q;
+  const half_t* pages;
+  const int32_t* page_indptr;
+  const int32_t* page_values;
+  const int32_t* last_page_len;
+  half_t* output;
+  float* lse;
+  float* part_o;   // (slots, h_q, D) fp32, unnormalised, relative to part_ml[..][0]
+  float* part_ml;  // (slots, h_q, 2) fp32: running max m, running sum l
+  int batch_size;
+  int h_q;
+  int h_kv;
+  int chunk_pages;
+  float scale_log2;  // sm_scale * log2(e)
+};
+
+__device__ __forceinline__ int slot_begin(const int32_t* page_indptr, int b, int cp) {
+  return page_indptr[b] / cp + b;
+}
+
+// Largest b in [0, batch) with slot_begin(b) <= slot.
+__device__ __forceinline__ int find_sequence(const int32_t* page_indptr, int batch, int cp, int slot) {
+  int lo = 0, hi = batch - 1;
+  while (lo < hi) {
+    int mid = (lo + hi + 1) >> 1;
+    if (slot_begin(page_indptr, mid, cp) <= slot) {
+      lo = mid;
+    } else {
+      hi = mid - 1;
+    }
+  }
+  return lo;
+}
+
+template <int D, int GROUP, int PS>
+__global__ __launch_bounds__(256) void decode_splitkv_kernel(DecodeParams p) {
+  constexpr int LPR = D / 8;         // lanes per K/V row
+  constexpr int TPL = 64 / LPR;      // rows (tokens) covered by one wave-wide 16-byte load
+  constexpr int LOADS = PS / TPL;    // loads per page for K (and as many for V)
+  constexpr int NGRP = TPL;          // independent lane groups per wave
+  static_assert(PS % TPL == 0, "page must be a whole number of wave-wide loads");
+
+  const int slot = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int grp = lane / LPR;   // which row of a wave-wide load this lane reads
+  const int sub = lane % LPR;   // which 16-byte piece of the row
+
+  const int cp = p.chunk_pages;
+  const int b = find_sequence(p.page_indptr, p.batch_size, cp, slot);
+  const int pbeg = p.page_indptr[b];
+  const int pend = p.page_indptr[b + 1];
+  const int npages = pend - pbeg;
+  const int chunk = slot - slot_begin(p.page_indptr, b, cp);
+  const int nchunks = (npages + cp - 1) / cp;
+  if (chunk >= nchunks) return;  // spare slot
+  const int kv_len = (npages - 1) * PS + p.last_page_len[b];
+  const int page_lo = chunk * cp;
+  const int page_hi = min(page_lo + cp, npages);
+
+  // q of the GROUP heads sharing this kv head: the 8 features this lane owns, packed fp16.
+  Vec16 qv[GROUP];
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g) {
+    qv[g] = ld16(p.q + (static_cast<int64_t>(b) * p.h_q + kvh * GROUP + g) * D + sub * 8);
+  }
+
+  float m[GROUP], l[GROUP], o[GROUP][8];
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g) {
+    m[g] = kNegInit;
+    l[g] = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[g][e] = 0.f;
+  }
+
+  const int64_t head_stride = static_cast<int64_t>(PS) * D;  // elements of one (page, k|v, head)
+  auto issue = [&](int page_idx, Vec16* kreg, Vec16* vreg) {
+    const int page = __builtin_amdgcn_readfirstlane(p.page_values[pbeg + page_idx]);
+    const half_t* kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * head_stride + lane * 8;
+    const half_t* vbase = kbase + static_cast<int64_t>(p.h_kv) * head_stride;
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) {
+      kreg[j] = ld16(kbase + j * TPL * D);
+      vreg[j] = ld16(vbase + j * TPL * D);
+    }
+  };
+
+  auto consume = [&](int page_idx, const Vec16* kreg, Vec16* vreg) {
+    const int tok0 = page_idx * PS + grp;  // token of load j is tok0 + j*TPL
+    const bool partial = (page_idx + 1) * PS > kv_len;  // wave-uniform: only the last page
+    bool valid[LOADS];
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) {
+      valid[j] = !partial || (tok0 + j * TPL < kv_len);
+      if (partial && !valid[j]) vreg[j] = zero16();  // slots beyond kv_len hold arbitrary bits
+    }
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g) {
+      float s[LOADS];
+      float mx = m[g];
+#pragma unroll
+      for (int j = 0; j < LOADS; ++j) {
+        float acc = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2(qv[g].h2[e], kreg[j].h2[e], acc, false);
+        acc = group_sum<LPR>(acc) * p.scale_log2;
+        s[j] = valid[j] ? acc : kNegInit;
+        mx = fmaxf(mx, s[j]);
+      }
+      const float alpha = fast_exp2(m[g] - mx);
+      m[g] = mx;
+      l[g] *= alpha;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[g][e] *= alpha;
+#pragma unroll
+      for (int j = 0; j < LOADS; ++j) {
+        const float pj = valid[j] ? fast_exp2(s[j] - mx) : 0.f;
+        l[g] += pj;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[g][e] = fmaf(pj, static_cast<float>(vreg[j].h[e]), o[g][e]);
+      }
+    }
+  };
+
+  // Two register buffers: the loads of the next page are in flight while this one is consumed.
+  Vec16 k0[LOADS], v0[LOADS], k1[LOADS], v1[LOADS];
+  int pi = page_lo + wave;
+  if (pi < page_hi) issue(pi, k0, v0);
+  while (pi < page_hi) {
+    const int pn = pi + 4;
+    if (pn < page_hi) issue(pn, k1, v1);
+    consume(pi, k0, v0);
+    pi = pn;
+    if (pi >= page_hi) break;
+    const int pn2 = pi + 4;
+    if (pn2 < page_hi) issue(pn2, k0, v0);
+    consume(pi, k1, v1);
+    pi = pn2;
+  }
+
+  // ---- merge the NGRP lane groups of this wave (butterfly over the group index) -------------
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g) {
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) {
+      const float m_o = __shfl_xor(m[g], off, 64);
+      const float l_o = __shfl_xor(l[g], off, 64);
+      const float mx = fmaxf(m[g], m_o);
+      const float a = fast_exp2(m[g] - mx);
+      const float bsc = fast_exp2(m_o - mx);
+      l[g] = l[g] * a + l_o * bsc;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float o_o = __shfl_xor(o[g][e], off, 64);
+        o[g][e] = o[g][e] * a + o_o * bsc;
+      }
+      m[g] = mx;
+    }
+  }
+  (void)NGRP;
+
+  // ---- merge the 4 waves through LDS --------------------------------------------------------
+  __shared__ float sm_o[4][GROUP][D];
+  __shared__ float sm_m[4][GROUP];
+  __shared__ float sm_l[4][GROUP];
+  if (grp == 0) {
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sm_o[wave][g][sub * 8 + e] = o[g][e];
+      if (sub == 0) {
+        sm_m[wave][g] = m[g];
+        sm_l[wave][g] = l[g];
+      }
+    }
+  }
+  __syncthreads();
+
+  const bool single_chunk = nchunks == 1;
+  for (int idx = tid; idx < GROUP * D; idx += 256) {
+    const int g = idx / D;
+    const int d = idx % D;
+    float mx = sm_m[0][g];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, sm_m[w][g]);
+    float lsum = 0.f, acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float sc = fast_exp2(sm_m[w][g] - mx);
+      lsum += sm_l[w][g] * sc;
+      acc += sm_o[w][g][d] * sc;
+    }
+    const int hq = kvh * GROUP + g;
+    if (single_chunk) {
+      // the reference's initial state (m=-5e4, d=1) leaves a term exp2(-5e4 - m) in the sum
+      const float denom = lsum + fast_exp2(kNegInit - mx);
+      p.output[(static_cast<int64_t>(b) * p.h_q + hq) * D + d] = static_cast<half_t>(acc / denom);
+      if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = mx + fast_log2(denom);
+    } else {
+      p.part_o[(static_cast<int64_t>(slot) * p.h_q + hq) * D + d] = acc;
+      if (d == 0) {
+        p.part_ml[(static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 0] = mx;
+        p.part_ml[(static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 1] = lsum;
+      }
+    }
+  }
+}
+
+// One block per (sequence, query head); D threads.  Sequences with one chunk were finished by
+// the main kernel; sequences without pages get the empty-KV answer out = 0, lse = -5e4
+// (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:129-130,173-176).
+template <int D>
+__global__ __launch_bounds__(D) void decode_merge_kernel(DecodeParams p, int page_size) {
+  const int b = blockIdx.x;
+  const int hq = blockIdx.y;
+  const int d = threadIdx.x;
+  const int cp = p.chunk_pages;
+  const int npages = p.page_indptr[b + 1] - p.page_indptr[b];
+  const int nchunks = (npages + cp - 1) / cp;
+  const int64_t out_idx = (static_cast<int64_t>(b) * p.h_q + hq) * D + d;
+  if (nchunks == 1) return;
+  if (nchunks == 0) {
+    p.output[out_idx] = static_cast<half_t>(0.f);
+    if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = kNegInit;
+    return;
+  }
+  const int s0 = slot_begin(p.page_indptr, b, cp);
+  float mx = kNegInit;
+  for (int c = 0; c < nchunks; ++c) mx = fmaxf(mx, p.part_ml[(static_cast<int64_t>(s0 + c) * p.h_q + hq) * 2]);
+  float lsum = 0.f, acc = 0.f;
+  for (int c = 0; c < nchunks; ++c) {
+    const int64_t base = static_cast<int64_t>(s0 + c) * p.h_q + hq;
+    const float sc = fast_exp2(p.part_ml[base * 2] - mx);
+    lsum += p.part_ml[base * 2 + 1] * sc;
+    acc += p.part_o[base * D + d] * sc;
+  }
+  const float denom = lsum + fast_exp2(kNegInit - mx);
+  p.output[out_idx] = static_cast<half_t>(acc / denom);
+  if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = mx + fast_log2(denom);
+}
+
+// ---- per-device workspace for the partial states, grown on demand --------------------------
+struct Workspace {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
+static Workspace g_workspace[64];
+
+static void* get_workspace(size_t bytes) {
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  KV_CHECK(dev >= 0 && dev < 64) << "device ordinal " << dev << " out of range";
+  Workspace& ws = g_workspace[dev];
+  if (ws.bytes < bytes) {
+    if (ws.ptr) {
+      HIP_CHECK(hipDeviceSynchronize());  // kernels of earlier calls may still read the old buffer
+      HIP_CHECK(hipFree(ws.ptr));
+      ws.ptr = nullptr;
+      ws.bytes = 0;
+    }
+    size_t want = bytes + bytes / 2;
+    HIP_CHECK(hipMalloc(&ws.ptr, want));
+    ws.bytes = want;
+  }
+  return ws.ptr;
+}
+
+// Pages per chunk from shapes only: aim at ~8K workgroups, keep a chunk between 4 and 64 pages.
+static int pick_chunk_pages(int64_t nnz_pages, int h_kv) {
+  int64_t cp = nnz_pages * h_kv / 8192;
+  int pow2 = 4;
+  while (pow2 * 2 <= cp && pow2 < 64) pow2 *= 2;
+  return pow2;
+}
+
+template <int D, int PS>
+static void launch_decode(const DecodeParams& p, int group, dim3 grid, hipStream_t stream) {
+  switch (group) {
+    case 1: hipLaunchKernelGGL((decode_splitkv_kernel<D, 1, PS>), grid, dim3(256), 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((decode_splitkv_kernel<D, 2, PS>), grid, dim3(256), 0, stream, p); break;
+    case 4: hipLaunchKernelGGL((decode_splitkv_kernel<D, 4, PS>), grid, dim3(256), 0, stream, p); break;
+    case 8: hipLaunchKernelGGL((decode_splitkv_kernel<D, 8, PS>), grid, dim3(256), 0, stream, p); break;
+    default:
+      throw Error(TVMKV_EUNSUPPORTED, "batch_decode_paged_kv: GQA group size " + std::to_string(group) +
+                                          " is not built (1, 2, 4, 8)");
+  }
+}
+
+}  // namespace tvmkv
+
+using namespace tvmkv;
+
+extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t* page_indptr,
+                                           const int32_t* page_values, const int32_t* length_info,
+                                           const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,
+                                           void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                                           double rope_theta, double sm_scale, int32_t batch_size,
+                                           int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                                           int32_t d, int32_t page_size, int32_t sliding_window, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(batch_size >= 0 && nnz_pages >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
+      << "batch_decode_paged_kv: bad shape";
+  KV_UNSUPPORTED(rotary_mode != 0) << "batch_decode_paged_kv: inline RoPE (rotary_mode=1) is not built; the "
+                                      "cache applies RoPE before the append (RoPE mode NORMAL) or not at all";
+  KV_UNSUPPORTED(sliding_window != 0) << "batch_decode_paged_kv: sliding-window length_info (3, B) is not built";
+  KV_UNSUPPORTED(page_size != 16) << "batch_decode_paged_kv: page_size " << page_size << " is not built (16)";
+  KV_UNSUPPORTED(d != 64 && d != 128) << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 128)";
+  if (batch_size == 0) return TVMKV_OK;
+  KV_CHECK(q && pages && page_indptr && length_info && output && lse) << "batch_decode_paged_kv: NULL tensor";
+  KV_CHECK(nnz_pages == 0 || page_values) << "batch_decode_paged_kv: NULL page table";
+
+  DecodeParams p;
+  p.q = static_cast<const half_t*>(q);
+  p.pages = static_cast<const half_t*>(pages);
+  p.page_indptr = page_indptr;
+  p.page_values = page_values;
+  p.last_page_len = length_info;
+  p.output = static_cast<half_t*>(output);
+  p.lse = lse;
+  p.batch_size = batch_size;
+  p.h_q = h_q;
+  p.h_kv = h_kv;
+  p.chunk_pages = pick_chunk_pages(nnz_pages, h_kv);
+  p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
+  const int64_t slots = nnz_pages / p.chunk_pages + batch_size;
+  KV_CHECK(slots < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many chunks";
+  const size_t part_o_bytes = static_cast<size_t>(slots) * h_q * d * sizeof(float);
+  const size_t part_ml_bytes = static_cast<size_t>(slots) * h_q * 2 * sizeof(float);
+  char* ws = static_cast<char*>(get_workspace(part_o_bytes + part_ml_bytes));
+  p.part_o = reinterpret_cast<float*>(ws);
+  p.part_ml = reinterpret_cast<float*>(ws + part_o_bytes);
+
+  const dim3 grid(static_cast<unsigned>(slots), h_kv);
+  const int group = h_q / h_kv;
+  hipStream_t s = as_stream(stream);
+  if (d == 128) {
+    launch_decode<128, 16>(p, group, grid, s);
+    KV_LAUNCH_CHECK();
+    hipLaunchKernelGGL(decode_merge_kernel<128>, dim3(batch_size, h_q), dim3(128), 0, s, p, page_size);
+  } else {
+    launch_decode<64, 16>(p, group, grid, s);
+    KV_LAUNCH_CHECK();
+    hipLaunchKernelGGL(decode_merge_kernel<64>, dim3(batch_size, h_q), dim3(64), 0, s, p, page_size);
+  }
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}

@@ -1,0 +1,414 @@
+// Page-granular data movement kernels of the paged KV cache and the two-way state merge:
+// fused qkv split + RoPE, K/V append scatter (MHA and MLA), single-page copy for fork,
+// gather for debug reads, compaction copy, and merge_state_inplace.
+//
+// All of them are HBM-bound byte movers: one thread owns 16 bytes (8 fp16), consecutive
+// lanes own consecutive 16-byte pieces of one head vector, so every wavefront access is a
+// run of full 128-byte lines.
+#include <cmath>
+
+#include "kernels_common.cuh"
+
+namespace tvmkv {
+
+// ------------------------------------------------------------------------------------------
+// fused_rope: split qkv and rotate q,k.
+// Reference arithmetic (python/tvm/relax/frontend/nn/llm/position_embedding.py:32-67,493-523):
+//   freq = (pos * scale) / pow(theta, (2d mod D) / D);  out[d] = cos(freq)*x[d] + sin(freq)*y[d]
+//   y[d] = -x[d + D/2] for d < D/2, x[d - D/2] otherwise; fp32 math, one rounding to fp16.
+// The D/2 divisors pow(theta, 2i/D) are computed on the host with the same libm call the CPU
+// kernels use and travel as a kernel argument, so the angle is formed by one IEEE division.
+// ------------------------------------------------------------------------------------------
+constexpr int kMaxHalfDim = 128;
+struct RopeDivisors {
+  float v[kMaxHalfDim];
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restrict__ qkv,
+                                                         const int32_t* __restrict__ position_map,
+                                                         half_t* __restrict__ q, half_t* __restrict__ k,
+                                                         half_t* __restrict__ v, int64_t seq_len, int num_q_heads,
+                                                         int num_kv_heads, int apply_rope, float scale,
+                                                         RopeDivisors div) {
+  constexpr int kThreadsPerHead = D / 16;  // a thread owns d-range [8c, 8c+8) and its partner +D/2
+  const int fused_heads = num_q_heads + 2 * num_kv_heads;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int c = gid % kThreadsPerHead;
+  const int64_t row = gid / kThreadsPerHead;  // (token, fused head)
+  if (row >= seq_len * fused_heads) return;
+  const int64_t s = row / fused_heads;
+  const int h = row % fused_heads;
+  const half_t* src = qkv + row * D + c * 8;
+  Vec16 lo = ld16(src);
+  Vec16 hi = ld16(src + D / 2);
+  half_t* dst;
+  if (h < num_q_heads) {
+    dst = q + (s * num_q_heads + h) * D;
+  } else if (h < num_q_heads + num_kv_heads) {
+    dst = k + (s * num_kv_heads + (h - num_q_heads)) * D;
+  } else {
+    dst = v + (s * num_kv_heads + (h - num_q_heads - num_kv_heads)) * D;
+  }
+  if (apply_rope > 0 && h < num_q_heads + num_kv_heads) {
+    const float pos_scaled = static_cast<float>(position_map[s]) * scale;
+    Vec16 out_lo, out_hi;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float freq = pos_scaled / div.v[c * 8 + e];
+      const float cs = cosf(freq);
+      const float sn = sinf(freq);
+      const float xl = static_cast<float>(lo.h[e]);
+      const float xh = static_cast<float>(hi.h[e]);
+      out_lo.h[e] = static_cast<half_t>(cs * xl + sn * (-xh));
+      out_hi.h[e] = static_cast<half_t>(cs * xh + sn * xl);
+    }
+    lo = out_lo;
+    hi = out_hi;
+  }
+  st16(dst + c * 8, lo);
+  st16(dst + D / 2 + c * 8, hi);
+}
+
+// ------------------------------------------------------------------------------------------
+// transpose_append: k|v[i, h, :] -> pages[p / ps, 0|1, h, p % ps, :], p = position_map[i] != -1
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void transpose_append_kernel(half_t* __restrict__ pages,
+                                                               const half_t* __restrict__ k_data,
+                                                               const half_t* __restrict__ v_data,
+                                                               const int32_t* __restrict__ position_map,
+                                                               int64_t ntoken, int num_kv_heads, int page_size,
+                                                               int head_dim) {
+  const int chunks = head_dim / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int c = gid % chunks;
+  const int64_t row = gid / chunks;  // (token, kv head)
+  if (row >= ntoken * num_kv_heads) return;
+  const int64_t i = row / num_kv_heads;
+  const int h = row % num_kv_heads;
+  const int32_t position = position_map[i];
+  if (position == -1) return;
+  const int64_t page = position / page_size;
+  const int slot = position % page_size;
+  const int64_t head_stride = static_cast<int64_t>(page_size) * head_dim;
+  half_t* kdst = pages + ((page * 2 + 0) * num_kv_heads + h) * head_stride + slot * head_dim + c * 8;
+  half_t* vdst = kdst + num_kv_heads * head_stride;
+  st16(kdst, ld16(k_data + row * head_dim + c * 8));
+  st16(vdst, ld16(v_data + row * head_dim + c * 8));
+}
+
+__global__ __launch_bounds__(256) void transpose_append_mla_kernel(half_t* __restrict__ pages,
+                                                                   const half_t* __restrict__ kv_data,
+                                                                   const int32_t* __restrict__ position_map,
+                                                                   int64_t ntoken, int d_qk) {
+  const int chunks = d_qk / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int c = gid % chunks;
+  const int64_t i = gid / chunks;
+  if (i >= ntoken) return;
+  const int32_t position = position_map[i];
+  if (position == -1) return;
+  // pages (num_pages, page_size, d_qk): slot p lives at row p of the flattened (slots, d_qk) view.
+  st16(pages + static_cast<int64_t>(position) * d_qk + c * 8, ld16(kv_data + i * d_qk + c * 8));
+}
+
+// ------------------------------------------------------------------------------------------
+// copy_single_page: first copy_length slots of every head, K and V.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void copy_single_page_kernel(half_t* __restrict__ pages, int64_t src_page,
+                                                               int64_t tgt_page, int copy_length, int num_heads,
+                                                               int page_size, int head_dim) {
+  const int chunks = head_dim / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t total = static_cast<int64_t>(2) * num_heads * copy_length * chunks;
+  if (gid >= total) return;
+  const int c = gid % chunks;
+  const int slot = (gid / chunks) % copy_length;
+  const int kvh = gid / (static_cast<int64_t>(chunks) * copy_length);  // (k|v, head) flattened
+  const int64_t page_stride = static_cast<int64_t>(2) * num_heads * page_size * head_dim;
+  const int64_t off = (static_cast<int64_t>(kvh) * page_size + slot) * head_dim + c * 8;
+  st16(pages + tgt_page * page_stride + off, ld16(pages + src_page * page_stride + off));
+}
+
+__global__ __launch_bounds__(256) void copy_single_page_mla_kernel(half_t* __restrict__ pages, int64_t src_page,
+                                                                   int64_t tgt_page, int copy_length,
+                                                                   int page_size, int d_qk) {
+  const int chunks = d_qk / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (gid >= static_cast<int64_t>(copy_length) * chunks) return;
+  const int64_t page_stride = static_cast<int64_t>(page_size) * d_qk;
+  st16(pages + tgt_page * page_stride + gid * 8, ld16(pages + src_page * page_stride + gid * 8));
+}
+
+// ------------------------------------------------------------------------------------------
+// debug_get_kv: gather rows by slot id into (num_layers, seqlen, H, D)[layer_id].
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void debug_get_kv_kernel(const half_t* __restrict__ pages,
+                                                           const int32_t* __restrict__ position_map,
+                                                           half_t* __restrict__ k_data, half_t* __restrict__ v_data,
+                                                           int64_t layer_id, int64_t seqlen, int num_kv_heads,
+                                                           int page_size, int head_dim) {
+  const int chunks = head_dim / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int c = gid % chunks;
+  const int64_t row = gid / chunks;  // (p, h)
+  if (row >= seqlen * num_kv_heads) return;
+  const int64_t p = row / num_kv_heads;
+  const int h = row % num_kv_heads;
+  const int32_t position = position_map[p];
+  const int64_t page = position / page_size;
+  const int slot = position % page_size;
+  const int64_t head_stride = static_cast<int64_t>(page_size) * head_dim;
+  const half_t* ksrc = pages + ((page * 2 + 0) * num_kv_heads + h) * head_stride + slot * head_dim + c * 8;
+  const half_t* vsrc = ksrc + num_kv_heads * head_stride;
+  const int64_t dst = ((layer_id * seqlen + p) * num_kv_heads + h) * head_dim + c * 8;
+  st16(k_data + dst, ld16(ksrc));
+  st16(v_data + dst, ld16(vsrc));
+}
+
+__global__ __launch_bounds__(256) void debug_get_kv_mla_kernel(const half_t* __restrict__ pages,
+                                                               const int32_t* __restrict__ position_map,
+                                                               half_t* __restrict__ kv_data, int64_t layer_id,
+                                                               int64_t seqlen, int d_qk) {
+  const int chunks = d_qk / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int c = gid % chunks;
+  const int64_t p = gid / chunks;
+  if (p >= seqlen) return;
+  st16(kv_data + (layer_id * seqlen + p) * d_qk + c * 8,
+       ld16(pages + static_cast<int64_t>(position_map[p]) * d_qk + c * 8));
+}
+
+// ------------------------------------------------------------------------------------------
+// compact_kv_copy: per batch row, copies run in order (a later destination may be an earlier
+// source), so one thread walks the whole list for its (b, k|v, head, 16-byte piece).
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void compact_kv_copy_kernel(half_t* __restrict__ pages,
+                                                              const int32_t* __restrict__ copy_length_indptr,
+                                                              const int32_t* __restrict__ copy_src_dst_pos,
+                                                              int batch_size, int total_copy_length, int num_heads,
+                                                              int page_size, int head_dim) {
+  const int chunks = head_dim / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t per_batch = static_cast<int64_t>(2) * num_heads * chunks;
+  if (gid >= batch_size * per_batch) return;
+  const int b = gid / per_batch;
+  const int rem = gid % per_batch;
+  const int c = rem % chunks;
+  const int kvh = rem / chunks;  // (k|v, head) flattened: kv = kvh / num_heads, h = kvh % num_heads
+  const int kv = kvh / num_heads;
+  const int h = kvh % num_heads;
+  const int64_t head_stride = static_cast<int64_t>(page_size) * head_dim;
+  for (int i = copy_length_indptr[b]; i < copy_length_indptr[b + 1]; ++i) {
+    const int32_t src_pos = copy_src_dst_pos[i];
+    const int32_t dst_pos = copy_src_dst_pos[total_copy_length + i];
+    const half_t* src = pages + ((static_cast<int64_t>(src_pos / page_size) * 2 + kv) * num_heads + h) * head_stride +
+                        (src_pos % page_size) * head_dim + c * 8;
+    half_t* dst = pages + ((static_cast<int64_t>(dst_pos / page_size) * 2 + kv) * num_heads + h) * head_stride +
+                  (dst_pos % page_size) * head_dim + c * 8;
+    st16(dst, ld16(src));
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// merge_state_inplace (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:497-521):
+//   smax = max(s, s'); w = 2^(s-smax), w' = 2^(s'-smax)
+//   V = V*w/(w+w') + V'*w'/(w+w') (rounded to fp16);  S = log2(w+w') + smax
+// A row (n, h) is owned by D/8 consecutive lanes of ONE wavefront: every lane reads S before
+// lane 0 of the group overwrites it (lock-step execution inside the wavefront).
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void merge_state_inplace_kernel(half_t* __restrict__ v, float* __restrict__ s,
+                                                                  const half_t* __restrict__ v_other,
+                                                                  const float* __restrict__ s_other, int64_t rows,
+                                                                  int d) {
+  const int chunks = d / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int c = gid % chunks;
+  const int64_t row = gid / chunks;
+  if (row >= rows) return;
+  float s_val = s[row];
+  float s_other_val = s_other[row];
+  const float s_max = fmaxf(s_val, s_other_val);
+  s_val = exp2f(s_val - s_max);
+  s_other_val = exp2f(s_other_val - s_max);
+  const float scale = s_val / (s_val + s_other_val);
+  const float other_scale = s_other_val / (s_val + s_other_val);
+  Vec16 a = ld16(v + row * d + c * 8);
+  const Vec16 b = ld16(v_other + row * d + c * 8);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    a.h[e] = static_cast<half_t>(static_cast<float>(a.h[e]) * scale + static_cast<float>(b.h[e]) * other_scale);
+  }
+  st16(v + row * d + c * 8, a);
+  if (c == 0) s[row] = log2f(s_val + s_other_val) + s_max;
+}
+
+inline dim3 grid_for(int64_t threads, int block = 256) { return dim3(static_cast<unsigned>((threads + block - 1) / block)); }
+
+}  // namespace tvmkv
+
+using namespace tvmkv;
+
+extern "C" {
+
+int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void* k, void* v, int64_t apply_rope,
+                     int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                     double rope_scale, double rope_theta, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(seq_len >= 0 && num_q_heads > 0 && num_kv_heads > 0) << "fused_rope: bad shape";
+  KV_UNSUPPORTED(head_dim != 64 && head_dim != 128 && head_dim != 256)
+      << "fused_rope: head_dim " << head_dim << " is not built (64, 128, 256)";
+  if (seq_len == 0) return TVMKV_OK;
+  KV_CHECK(qkv && position_map && q && k && v) << "fused_rope: NULL tensor";
+  RopeDivisors div;
+  const float theta = static_cast<float>(rope_theta);
+  for (int i = 0; i < head_dim / 2; ++i) {
+    div.v[i] = powf(theta, static_cast<float>((i * 2) % head_dim) / static_cast<float>(head_dim));
+  }
+  const int64_t threads = seq_len * (num_q_heads + 2 * num_kv_heads) * (head_dim / 16);
+  const float scale = static_cast<float>(rope_scale);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid_for(threads), dim3(256), 0, as_stream(stream), static_cast<const half_t*>(qkv),
+                       position_map, static_cast<half_t*>(q), static_cast<half_t*>(k), static_cast<half_t*>(v),
+                       seq_len, num_q_heads, num_kv_heads, static_cast<int>(apply_rope > 0), scale, div);
+  };
+  if (head_dim == 64) {
+    launch(fused_rope_kernel<64>);
+  } else if (head_dim == 128) {
+    launch(fused_rope_kernel<128>);
+  } else {
+    launch(fused_rope_kernel<256>);
+  }
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+static void check_slot_layout(const char* what, int32_t page_size, int32_t head_dim) {
+  KV_CHECK(page_size > 0) << what << ": page_size must be positive";
+  KV_CHECK(head_dim > 0 && head_dim % 8 == 0) << what << ": feature dim " << head_dim << " must be a multiple of 8";
+}
+
+int tvmkv_kv_cache_transpose_append(void* pages, const void* k_data, const void* v_data,
+                                    const int32_t* position_map, int64_t ntoken, int64_t num_pages,
+                                    int32_t num_kv_heads, int32_t page_size, int32_t head_dim, void* stream) {
+  KV_API_BEGIN();
+  check_slot_layout("transpose_append", page_size, head_dim);
+  KV_CHECK(ntoken >= 0 && num_kv_heads > 0) << "transpose_append: bad shape";
+  KV_CHECK(num_pages * page_size <= INT32_MAX) << "transpose_append: slot ids do not fit int32";
+  if (ntoken == 0) return TVMKV_OK;
+  KV_CHECK(pages && k_data && v_data && position_map) << "transpose_append: NULL tensor";
+  const int64_t threads = ntoken * num_kv_heads * (head_dim / 8);
+  hipLaunchKernelGGL(transpose_append_kernel, grid_for(threads), dim3(256), 0, as_stream(stream),
+                     static_cast<half_t*>(pages), static_cast<const half_t*>(k_data),
+                     static_cast<const half_t*>(v_data), position_map, ntoken, num_kv_heads, page_size, head_dim);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_kv_cache_transpose_append_mla(void* pages, const void* kv_data, const int32_t* position_map,
+                                        int64_t ntoken, int64_t num_pages, int32_t page_size, int32_t d_qk,
+                                        void* stream) {
+  KV_API_BEGIN();
+  check_slot_layout("transpose_append_mla", page_size, d_qk);
+  KV_CHECK(ntoken >= 0) << "transpose_append_mla: bad shape";
+  if (ntoken == 0) return TVMKV_OK;
+  KV_CHECK(pages && kv_data && position_map) << "transpose_append_mla: NULL tensor";
+  hipLaunchKernelGGL(transpose_append_mla_kernel, grid_for(ntoken * (d_qk / 8)), dim3(256), 0, as_stream(stream),
+                     static_cast<half_t*>(pages), static_cast<const half_t*>(kv_data), position_map, ntoken, d_qk);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_copy_single_page(void* pages, int64_t src_page_id, int64_t tgt_page_id, int64_t copy_length,
+                           int64_t num_pages, int32_t num_kv_heads, int32_t page_size, int32_t head_dim,
+                           void* stream) {
+  KV_API_BEGIN();
+  check_slot_layout("copy_single_page", page_size, head_dim);
+  KV_CHECK(src_page_id >= 0 && src_page_id < num_pages && tgt_page_id >= 0 && tgt_page_id < num_pages)
+      << "copy_single_page: page id out of range";
+  KV_CHECK(copy_length >= 0 && copy_length <= page_size) << "copy_single_page: copy_length out of range";
+  if (copy_length == 0) return TVMKV_OK;
+  const int64_t threads = 2 * num_kv_heads * copy_length * (head_dim / 8);
+  hipLaunchKernelGGL(copy_single_page_kernel, grid_for(threads), dim3(256), 0, as_stream(stream),
+                     static_cast<half_t*>(pages), src_page_id, tgt_page_id, static_cast<int>(copy_length),
+                     num_kv_heads, page_size, head_dim);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_copy_single_page_mla(void* pages, int64_t src_page_id, int64_t tgt_page_id, int64_t copy_length,
+                               int64_t num_pages, int32_t page_size, int32_t d_qk, void* stream) {
+  KV_API_BEGIN();
+  check_slot_layout("copy_single_page_mla", page_size, d_qk);
+  KV_CHECK(src_page_id >= 0 && src_page_id < num_pages && tgt_page_id >= 0 && tgt_page_id < num_pages)
+      << "copy_single_page_mla: page id out of range";
+  KV_CHECK(copy_length >= 0 && copy_length <= page_size) << "copy_single_page_mla: copy_length out of range";
+  if (copy_length == 0) return TVMKV_OK;
+  hipLaunchKernelGGL(copy_single_page_mla_kernel, grid_for(copy_length * (d_qk / 8)), dim3(256), 0,
+                     as_stream(stream), static_cast<half_t*>(pages), src_page_id, tgt_page_id,
+                     static_cast<int>(copy_length), page_size, d_qk);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_kv_cache_debug_get_kv(const void* pages, const int32_t* position_map, void* k_data, void* v_data,
+                                int64_t layer_id, int64_t seqlen, int64_t num_pages, int32_t num_kv_heads,
+                                int32_t page_size, int32_t head_dim, void* stream) {
+  KV_API_BEGIN();
+  check_slot_layout("debug_get_kv", page_size, head_dim);
+  if (seqlen == 0) return TVMKV_OK;
+  KV_CHECK(pages && position_map && k_data && v_data) << "debug_get_kv: NULL tensor";
+  hipLaunchKernelGGL(debug_get_kv_kernel, grid_for(seqlen * num_kv_heads * (head_dim / 8)), dim3(256), 0,
+                     as_stream(stream), static_cast<const half_t*>(pages), position_map,
+                     static_cast<half_t*>(k_data), static_cast<half_t*>(v_data), layer_id, seqlen, num_kv_heads,
+                     page_size, head_dim);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_kv_cache_debug_get_kv_mla(const void* pages, const int32_t* position_map, void* kv_data, int64_t layer_id,
+                                    int64_t seqlen, int64_t num_pages, int32_t page_size, int32_t d_qk,
+                                    void* stream) {
+  KV_API_BEGIN();
+  check_slot_layout("debug_get_kv_mla", page_size, d_qk);
+  if (seqlen == 0) return TVMKV_OK;
+  KV_CHECK(pages && position_map && kv_data) << "debug_get_kv_mla: NULL tensor";
+  hipLaunchKernelGGL(debug_get_kv_mla_kernel, grid_for(seqlen * (d_qk / 8)), dim3(256), 0, as_stream(stream),
+                     static_cast<const half_t*>(pages), position_map, static_cast<half_t*>(kv_data), layer_id,
+                     seqlen, d_qk);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr, const int32_t* copy_src_dst_pos,
+                          int32_t batch_size, int32_t total_copy_length, int64_t num_pages, int32_t num_kv_heads,
+                          int32_t page_size, int32_t head_dim, void* stream) {
+  KV_API_BEGIN();
+  check_slot_layout("compact_kv_copy", page_size, head_dim);
+  if (batch_size == 0 || total_copy_length == 0) return TVMKV_OK;
+  KV_CHECK(pages && copy_length_indptr && copy_src_dst_pos) << "compact_kv_copy: NULL tensor";
+  const int64_t threads = static_cast<int64_t>(batch_size) * 2 * num_kv_heads * (head_dim / 8);
+  hipLaunchKernelGGL(compact_kv_copy_kernel, grid_for(threads), dim3(256), 0, as_stream(stream),
+                     static_cast<half_t*>(pages), copy_length_indptr, copy_src_dst_pos, batch_size,
+                     total_copy_length, num_kv_heads, page_size, head_dim);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_merge_state_inplace(void* v, float* s, const void* v_other, const float* s_other, int64_t n, int32_t h,
+                              int32_t d, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(n >= 0 && h > 0) << "merge_state_inplace: bad shape";
+  // D/8 lanes of one wavefront own a row: D/8 must divide 64.
+  KV_UNSUPPORTED(d <= 0 || d % 8 != 0 || d > 512 || 64 % (d / 8) != 0)
+      << "merge_state_inplace: head dim " << d << " is not built (8..512, D/8 a divisor of 64)";
+  if (n == 0) return TVMKV_OK;
+  KV_CHECK(v && s && v_other && s_other) << "merge_state_inplace: NULL tensor";
+  const int64_t rows = n * h;
+  hipLaunchKernelGGL(merge_state_inplace_kernel, grid_for(rows * (d / 8)), dim3(256), 0, as_stream(stream),
+                     static_cast<half_t*>(v), s, static_cast<const half_t*>(v_other), s_other, rows, d);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+}  // extern "C"
