@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged KV-cache attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one decode step of one layer over the synthetic batch of BASELINE.json
+configs[1]: 64 sequences, contexts uniform in [1024, 8192], 32 query / 8 kv heads, head_dim
+128, page 16, pages drawn from a seeded permutation of a 65536-page pool; every step appends
+one token per sequence (split + RoPE, append scatter) and runs split-KV decode attention.
+All inputs, page tables of every step included, are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` is the algorithmic GB/s of the whole step; `roofline` is the
+decode-attention entry point alone against the 8 TB/s HBM peak; `cpu_baseline` is the CPU
+oracle (restatement of the reference's llvm decode kernel) on this host.  A chunked-prefill
+figure (configs[2]) is reported under `prefill`.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
+
+HQ, HKV, D, PS = 32, 8, 128, 16
+TOKEN_BYTES = 2 * HKV * D * 2  # K and V rows of every kv head, fp16
+
+
+# --------------------------------------------------------------------------------------------
+# workload builders (also imported by tests/)
+# --------------------------------------------------------------------------------------------
+def decode_workload(batch=64, ctx_lo=1024, ctx_hi=8192, pool_pages=65536, steps=16, seed=1):
+    """Page tables of `steps` consecutive decode steps.  Step s sees contexts ctx + s + 1 (the
+    appended token included, as the cache builds them when it appends before attention)."""
+    rng = np.random.default_rng(seed)
+    ctx = rng.integers(ctx_lo, ctx_hi, size=batch, endpoint=True)
+    perm = rng.permutation(pool_pages).astype(np.int32)
+    max_pages = [(int(c) + steps + PS - 1) // PS for c in ctx]
+    starts = np.concatenate([[0], np.cumsum(max_pages)])
+    assert starts[-1] <= pool_pages, "pool too small for the batch"
+    owned = [perm[starts[i]:starts[i + 1]] for i in range(batch)]
+    tables = []
+    for s in range(steps):
+        kv_len = ctx + s + 1
+        npages = (kv_len + PS - 1) // PS
+        indptr = np.concatenate([[0], np.cumsum(npages)]).astype(np.int32)
+        values = np.concatenate([owned[i][:npages[i]] for i in range(batch)]).astype(np.int32)
+        last = ((kv_len - 1) % PS + 1).astype(np.int32)
+        pos = (kv_len - 1).astype(np.int32)
+        slots = np.array([owned[i][(kv_len[i] - 1) // PS] * PS + (kv_len[i] - 1) % PS for i in range(batch)], np.int32)
+        tables.append(dict(kv_len=kv_len.astype(np.int64), page_indptr=indptr, page_values=values,
+                           last_page_len=last, q_rope_position=pos, append_position_map=slots))
+    return dict(ctx=ctx, owned=owned, tables=tables, pool_pages=pool_pages, batch=batch)
+
+
+def prefill_workload(batch=8, prefix_hi=4096, chunk_lo=128, chunk_hi=2048, seed=2):
+    rng = np.random.default_rng(seed)
+    prefix = rng.integers(0, prefix_hi, size=batch, endpoint=True)
+    chunk = rng.integers(chunk_lo, chunk_hi, size=batch, endpoint=True)
+    npages = (prefix + PS - 1) // PS              # pages the attention reads (the cached prefix)
+    npages_after = (prefix + chunk + PS - 1) // PS  # pages owned once the chunk is appended
+    pool_pages = int(npages_after.sum()) + 8
+    perm = rng.permutation(pool_pages).astype(np.int32)
+    starts = np.concatenate([[0], np.cumsum(npages_after)])
+    owned = [perm[starts[i]:starts[i + 1]] for i in range(batch)]
+    page_values = np.concatenate([owned[i][:npages[i]] for i in range(batch)])
+    append_map = np.concatenate([[owned[i][t // PS] * PS + t % PS for t in range(prefix[i], prefix[i] + chunk[i])]
+                                 for i in range(batch)]).astype(np.int32)
+    flops = 4.0 * HQ * D * float(np.sum(chunk * (chunk + 1) / 2 + chunk * prefix))
+    return dict(prefix=prefix, chunk=chunk, pool_pages=pool_pages,
+                q_indptr=np.concatenate([[0], np.cumsum(chunk)]).astype(np.int32),
+                page_indptr=np.concatenate([[0], np.cumsum(npages)]).astype(np.int32),
+                page_values=page_values.astype(np.int32), append_position_map=append_map,
+                last_page_len=np.where(prefix == 0, 0, (prefix - 1) % PS + 1).astype(np.int32), flops=flops)
+
+
+# --------------------------------------------------------------------------------------------
+def time_region(torch, fn, iters):
+    """Milliseconds per call of fn, by HIP events on the stream the kernels run on."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(iters):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=16)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (profiling runs)")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the chunked-prefill leg (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; the path shards per kv head without any exchange "
+                 "(see DESIGN.md), and no multi-GPU figure is produced. Use --gpus 1.")
+
+    import torch
+
+    from tvm_amd import kernels as K  # raises if libtvmkv.so is missing: there is no fallback
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    K_steps, W = args.steps, args.warmup
+    total_steps = K_steps + W
+
+    # ---- decode workload, resident in HBM ---------------------------------------------------
+    wl = decode_workload(steps=total_steps)
+    B = wl["batch"]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    pages = torch.empty((wl["pool_pages"], 2, HKV, PS, D), dtype=torch.float16, device=dev)
+    for lo in range(0, wl["pool_pages"], 8192):  # fill in slices: randn makes an fp32 temporary
+        pages[lo:lo + 8192].copy_(torch.randn(pages[lo:lo + 8192].shape, generator=gen, device=dev))
+    qkv = torch.randn((total_steps, B, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16)
+    q = torch.empty((B, HQ, D), dtype=torch.float16, device=dev)
+    k = torch.empty((B, HKV, D), dtype=torch.float16, device=dev)
+    v = torch.empty((B, HKV, D), dtype=torch.float16, device=dev)
+    out = torch.empty((B, HQ, D), dtype=torch.float16, device=dev)
+    lse = torch.empty((B, HQ), dtype=torch.float32, device=dev)
+    zeros_b = torch.zeros(B, dtype=torch.int32, device=dev)
+
+    def i32(a):
+        return torch.tensor(a, dtype=torch.int32, device=dev)
+
+    tabs = [{key: i32(t[key]) for key in ("page_indptr", "page_values", "last_page_len", "q_rope_position",
+                                          "append_position_map")} for t in wl["tables"]]
+    sm_scale = D ** -0.5
+
+    def rope_append(s):
+        t = tabs[s]
+        K.fused_rope(qkv[s], t["q_rope_position"], q, k, v, 1, 1.0, 1e4)
+        K.tir_kv_cache_transpose_append(pages, k, v, t["append_position_map"])
+
+    def decode_only(s):
+        t = tabs[s]
+        K.batch_decode_paged_kv(q, pages, t["page_indptr"], t["page_values"], t["last_page_len"], zeros_b,
+                                t["q_rope_position"], out, lse, 0, 1.0, 1e4, sm_scale)
+
+    def step(s):
+        rope_append(s)
+        decode_only(s)
+
+    for s in range(W):
+        step(s)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms_step = time_region(torch, lambda i: step(W + i), K_steps)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / K_steps
+    # the decode entry point alone (split-KV kernel + merge kernel), same page tables
+    ms_decode = time_region(torch, lambda i: decode_only(W + i), K_steps)
+
+    kv_tokens = np.array([t["kv_len"].sum() for t in wl["tables"][W:]], dtype=np.float64)
+    qo_bytes = B * HQ * D * 2 * 2
+    step_bytes = kv_tokens.mean() * TOKEN_BYTES + qo_bytes + B * (HQ + 2 * HKV) * D * 2 + B * TOKEN_BYTES
+    decode_bytes = kv_tokens.mean() * TOKEN_BYTES + qo_bytes
+    gbps_step = step_bytes / (ms_step * 1e-3) / 1e9
+    gbps_decode = decode_bytes / (ms_decode * 1e-3) / 1e9
+
+    result = {
+        "metric": "paged decode attn GB/s",
+        "value": round(gbps_step, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K_steps,
+        "warmup": W,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: batched paged decode, 1 layer, B=64, ctx U[1024,8192] seed 1, "
+                               "Hq32/Hkv8/D128 fp16, page 16, permuted 65536-page pool, append 1 token/seq/step "
+                               "(split+RoPE, append, split-KV decode + merge)",
+                   "kv_tokens_per_step": int(kv_tokens.mean()), "bytes_per_step": int(step_bytes)},
+        "tokens_per_s": round(B / (ms_step * 1e-3), 1),
+        "host_wall_ms_per_step": round(wall_ms, 4),
+        "roofline": {"bound": "hbm", "achieved": round(gbps_decode, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps_decode / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "tvmkv_batch_decode_paged_kv (decode_splitkv_kernel + decode_merge_kernel)",
+                     "ms": round(ms_decode, 4), "algorithmic_bytes": int(decode_bytes)},
+    }
+
+    # ---- chunked prefill (configs[2]): ragged causal + paged non-causal + merge + append -------
+    if not args.no_prefill:
+        pw = prefill_workload()
+        n = int(pw["q_indptr"][-1])
+        nb = len(pw["chunk"])
+        ppages = torch.randn((pw["pool_pages"], 2, HKV, PS, D), generator=gen, device=dev).to(torch.float16)
+        pq = torch.randn((n, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16)
+        q2 = torch.empty((n, HQ, D), dtype=torch.float16, device=dev)
+        k2 = torch.empty((n, HKV, D), dtype=torch.float16, device=dev)
+        v2 = torch.empty((n, HKV, D), dtype=torch.float16, device=dev)
+        o1 = torch.empty((n, HQ, D), dtype=torch.float16, device=dev)
+        o2 = torch.empty_like(o1)
+        l1 = torch.empty((n, HQ), dtype=torch.float32, device=dev)
+        l2 = torch.empty_like(l1)
+        q_indptr, page_indptr = i32(pw["q_indptr"]), i32(pw["page_indptr"])
+        page_values, last = i32(pw["page_values"]), i32(pw["last_page_len"])
+        qpos = i32(np.concatenate([p + np.arange(c) for p, c in zip(pw["prefix"], pw["chunk"])]))
+        kofs = i32(pw["prefix"])
+        zb = torch.zeros(nb, dtype=torch.int32, device=dev)
+        amap = i32(pw["append_position_map"])
+
+        def prefill_step(_):
+            K.fused_rope(pq, qpos, q2, k2, v2, 1, 1.0, 1e4)
+            K.batch_prefill_ragged_kv(q2, q_indptr, k2, v2, q_indptr, qpos, kofs, o1, l1, 1, 0, 1.0, 1e4, sm_scale)
+            K.batch_prefill_paged_kv(q2, q_indptr, ppages, page_indptr, page_values, last, zb, qpos, o2, l2, 0, 0,
+                                     1.0, 1e4, sm_scale)
+            K.merge_state_inplace(o1, l1, o2, l2)
+            K.tir_kv_cache_transpose_append(ppages, k2, v2, amap)
+
+        prefill_step(0)
+        ms_prefill = time_region(torch, prefill_step, 5)
+        tflops = pw["flops"] / (ms_prefill * 1e-3) / 1e12
+        result["prefill"] = {"workload": "configs[2]: chunked causal prefill, 8 seqs, prefix U[0,4096], chunk "
+                                         "U[128,2048] seed 2 (split+RoPE, ragged causal, paged non-causal, merge, append)",
+                             "tflops": round(tflops, 2), "ms": round(ms_prefill, 4),
+                             "algorithmic_flops": pw["flops"],
+                             "frac_of_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
+
+    # ---- CPU baseline: the oracle's restatement of the reference's llvm decode kernel ---------
+    if not args.no_cpu_baseline:
+        from oracle import kernels as ok
+
+        s = W + K_steps - 1
+        t = wl["tables"][s]
+        # compact host copy of the pages this step reads (same bytes, renumbered page ids)
+        used = t["page_values"]
+        host_pages = pages[torch.tensor(used, dtype=torch.int64, device=dev)].cpu().numpy()
+        new_values = np.arange(len(used), dtype=np.int32)
+        qh = q.cpu().numpy()  # q of the last timed step
+        eo = np.zeros((B, HQ, D), np.float16)
+        el = np.zeros((B, HQ), np.float32)
+        z = np.zeros(B, np.int32)
+        c0 = time.perf_counter()
+        ok.decode(qh, host_pages, t["page_indptr"], new_values, t["last_page_len"], z, z, eo, el, 0, 1.0, 1e4,
+                  sm_scale)
+        cpu_s = time.perf_counter() - c0
+        cpu_bytes = float(t["kv_len"].sum()) * TOKEN_BYTES + qo_bytes
+        err = float(np.max(np.abs(out.cpu().numpy().astype(np.float32) - eo.astype(np.float32))))
+        result["cpu_baseline"] = {"value": round(cpu_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1,
+                                  "kind": "port",
+                                  "sample": "one full decode step of the same workload (64 sequences, "
+                                            f"{int(t['kv_len'].sum())} kv tokens), 1 thread, "
+                                            f"{cpu_s:.1f} s; the reference kernel is T.serial",
+                                  "tokens_per_s": round(B / cpu_s, 2), "host_cpus": os.cpu_count(),
+                                  "gpu_vs_cpu_max_abs_err": err}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,41 @@
+"""The C-ABI library loads without a GPU and exports every function include/tvmkv.h declares."""
+import ctypes
+import os
+import re
+
+import tvm_amd
+from tvm_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "tvmkv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tvmkv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert len(names) >= 40
+    handle = ctypes.CDLL(tvm_amd.LIB_PATH)
+    missing = [n for n in names if not hasattr(handle, n)]
+    assert not missing, f"declared in include/tvmkv.h but not exported: {missing}"
+
+
+def test_python_signatures_cover_the_header():
+    names = set(declared_functions()) - {"tvmkv_last_error", "tvmkv_version", "tvmkv_cache_destroy"}
+    assert names == set(_lib.SIGNATURES), names ^ set(_lib.SIGNATURES)
+
+
+def test_version_and_error_channel():
+    lib = tvm_amd.lib()
+    assert b"gfx950" in lib.tvmkv_version()
+    # argument validation happens before any device work, so it can be exercised without a GPU
+    rc = lib.tvmkv_batch_decode_paged_kv(None, None, None, None, None, None, None, None, None, 1, 1.0, 1e4, 1.0,
+                                         1, 1, 1, 8, 2, 128, 16, 0, None)
+    assert rc == -2 and b"inline RoPE" in lib.tvmkv_last_error()
+    rc = lib.tvmkv_merge_state_inplace(None, None, None, None, 1, 1, 100, None)
+    assert rc == -2 and b"head dim 100" in lib.tvmkv_last_error()
+    rc = lib.tvmkv_fused_rope(None, None, None, None, None, 1, 0, 8, 2, 128, 1.0, 1e4, None)
+    assert rc == 0  # empty input is a no-op

@@ -1,0 +1,167 @@
+"""GPU parity of the whole cache object: the reference's scenario batches through the
+HIP-backed cache, checked (a) against the numpy closed form the reference's own test uses,
+(b) against the CPU oracle cache on identical seeded inputs, with page tables / append
+indices / pool state compared bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+import tvm_amd
+from oracle.paged_kv_cache import OraclePagedKVCache
+from tests import scenario as S
+from tests.gpu_util import DEV, GpuCache, dev, host
+from tests.test_host_cache_parity import GLOBAL, PER_DEPTH
+from tests.util import assert_close
+from tvm_amd import get_global_func as gf
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("d,rope_mode", [(128, S.ROPE_NORMAL), (64, S.ROPE_NORMAL), (128, S.ROPE_NONE)])
+@pytest.mark.parametrize("runner", [S.run_prefill_and_decode, S.run_remove_sequence, S.run_fork_sequence,
+                                    S.run_unlimited_depth, S.run_popn])
+def test_reference_scenarios_on_the_gpu(runner, d, rope_mode):
+    """tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_cpu.py:706-909 of the
+    reference with its geometry (32 query / 4 kv heads, page 16, capacity 2048)."""
+    layers, hq, hkv = 2, 32, 4
+    cache = GpuCache([32, 2048, 512, 16, 0], layers, hq, hkv, d, d, rope_mode=rope_mode)
+    sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=rope_mode, seed=5, tol=4e-3)
+    runner(sc)
+
+
+class Mirror:
+    """Feeds the oracle cache and the GPU cache the same calls and the same tensors."""
+
+    def __init__(self, cache_config, layers, hq, hkv, d, rope_mode=1):
+        self.o = OraclePagedKVCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode)
+        self.g = GpuCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode)
+        self.layers, self.hq, self.hkv, self.d = layers, hq, hkv, d
+        self.rng = np.random.default_rng(21)
+        self.lengths = {}
+
+    def compare_bookkeeping(self):
+        aux = self.o.host.aux
+        c = self.g.cache
+        flags = c.flags()
+        assert flags["num_depths"] == aux["num_depths"]
+        assert bool(flags["append_before_attn"]) == aux["append_before_attn"]
+        for dd in range(aux["num_depths"]):
+            for name in PER_DEPTH:
+                assert c.aux(name, dd) == aux[name][dd], f"{name}[{dd}]"
+        for name in GLOBAL:
+            assert c.aux(name) == aux[name], name
+        so, sg = self.o.host.state(), c.state()
+        assert sg["free_page_ids"] == so["free_page_ids"] and sg["free_block_idx"] == so["free_block_idx"]
+        assert [tuple(b) for b in sg["blocks"]] == [tuple(b) for b in so["blocks"]] and sg["seqs"] == so["seqs"]
+        assert c.copy_log() == self.o.host.copies
+
+    def step(self, batch):
+        ids, lens = [], []
+        for item, n in batch:
+            if isinstance(item, tuple):
+                sid, parent, pos = item
+                self.o.fork_sequence(parent, sid, pos)
+                self.g.fork_sequence(parent, sid, pos)
+                self.lengths[sid] = self.lengths[parent] if pos == -1 else pos
+            else:
+                sid = item
+                if sid not in self.lengths:
+                    self.o.add_sequence(sid)
+                    self.g.add_sequence(sid)
+                    self.lengths[sid] = 0
+            ids.append(sid)
+            lens.append(n)
+        self.o.begin_forward(ids, lens)
+        self.g.begin_forward(ids, lens)
+        self.compare_bookkeeping()
+        total = sum(lens)
+        for layer in range(self.layers):
+            qkv = self.rng.standard_normal((total, self.hq + 2 * self.hkv, self.d)).astype(np.float16)
+            eo = np.zeros((total, self.hq, self.d), np.float16)
+            go = np.zeros_like(eo)
+            self.o.attention_with_fused_qkv(layer, self.d ** -0.5, qkv, eo)
+            self.g.attention_with_fused_qkv(layer, self.d ** -0.5, qkv, go)
+            assert_close(go, eo, what=f"layer {layer} output vs oracle cache")
+        self.o.end_forward()
+        self.g.end_forward()
+        for sid, n in zip(ids, lens):
+            self.lengths[sid] += n
+            L = self.lengths[sid]
+            ek = np.zeros((self.layers, L, self.hkv, self.d), np.float16)
+            ev, gk, gv = np.zeros_like(ek), np.zeros_like(ek), np.zeros_like(ek)
+            self.o.debug_get_kv(sid, 0, L, ek, ev)
+            self.g.debug_get_kv(sid, 0, L, gk, gv)
+            assert np.array_equal(gv, ev), f"cached V of seq {sid}"
+            assert_close(gk, ek, atol=1e-3, rtol=2e-3, what=f"cached K of seq {sid}")
+
+
+def test_identical_inputs_through_oracle_and_gpu_caches():
+    m = Mirror([16, 4096, 1024, 16, 0], 2, 32, 8, 128)
+    m.step([(0, 60), (1, 88), (2, 17), (3, 4)])
+    m.step([((4, 3, -1), 35)])
+    m.step([((5, 0, 33), 20)])            # fork inside a page -> page copy on the device
+    m.step([(0, 1), (1, 1), (2, 1), (4, 1), (5, 1)])
+    m.step([((6, 5, -1), 40), (2, 3)])
+    m.step([(6, 1), (5, 1), (0, 1)])      # two block depths + merge_state
+    m.o.popn(6, 30)
+    m.g.popn(6, 30)
+    m.lengths[6] -= 30
+    m.step([(6, 1), (1, 200)])
+    m.step([(i, 1) for i in (0, 1, 2, 4, 5, 6)])
+
+
+def test_cfg1_decode_through_the_cache_verbs():
+    """BASELINE configs[0] end to end: 1024-page pool, contexts 512/1024/1500/2048 prefilled through
+    the real verbs, then one decode step; page table as derived by hand from the reference."""
+    m = Mirror([32, 16368, 8192, 16, 0], 1, 32, 8, 128)
+    m.step([(0, 512), (1, 1024), (2, 1500), (3, 2048)])
+    m.step([(0, 1), (1, 1), (2, 1), (3, 1)])
+    c = m.g.cache
+    assert c.aux("page_indptr") == [0, 33, 98, 192, 321]
+    assert c.aux("append_position_map") == [5088, 5104, 3036, 5120]
+    assert c.aux("last_page_len") == [1, 1, 13, 1]
+    assert c.aux("q_rope_position_map") == [512, 1024, 1500, 2048]
+    assert gf("vm.builtin.attention_kv_cache_get_num_available_pages")(c) == 703
+
+
+def test_error_paths_on_the_device_cache():
+    cache = GpuCache([4, 64, 32, 16, 0], 1, 8, 2, 128, 128)
+    c = cache.cache
+    cache.add_sequence(0)
+    qkv = torch.zeros((4, 12, 128), dtype=torch.float16, device=DEV)
+    out = torch.zeros((4, 8, 128), dtype=torch.float16, device=DEV)
+    attn = gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")
+    with pytest.raises(tvm_amd.KVError, match="begin_forward has not been called"):
+        attn(c, 0, 1.0, qkv, out)
+    cache.begin_forward([0], [8])
+    with pytest.raises(tvm_amd.KVError, match="fewer than the batch appends"):
+        attn(c, 0, 1.0, qkv, out)
+    with pytest.raises(tvm_amd.KVError, match="out of range"):
+        attn(c, 3, 1.0, torch.zeros((8, 12, 128), dtype=torch.float16, device=DEV),
+             torch.zeros((8, 8, 128), dtype=torch.float16, device=DEV))
+    cache.add_sequence(1)
+    with pytest.raises(tvm_amd.KVError, match="The KV cache is full"):
+        cache.begin_forward([1], [80])
+    with pytest.raises(tvm_amd.KVError, match="not built"):  # sliding window forces inline RoPE
+        c2 = GpuCache([4, 64, 32, 16, 1], 1, 8, 2, 128, 128, rope_mode=1)
+        c2.add_sequence(0)
+        c2.begin_forward([0], [4])
+        attn(c2.cache, 0, 1.0, qkv, out)
+
+
+def test_padded_qkv_rows_are_ignored():
+    """qkv / out may carry more rows than the batch appends (src/runtime/vm/paged_kv_cache.cc:1330-1354)."""
+    layers, hq, hkv, d = 1, 8, 2, 128
+    a = GpuCache([4, 256, 64, 16, 0], layers, hq, hkv, d, d)
+    b = GpuCache([4, 256, 64, 16, 0], layers, hq, hkv, d, d)
+    rng = np.random.default_rng(3)
+    qkv = rng.standard_normal((10, hq + 2 * hkv, d)).astype(np.float16)
+    for cache in (a, b):
+        cache.add_sequence(0)
+        cache.begin_forward([0], [10])
+    o_exact = np.zeros((10, hq, d), np.float16)
+    a.attention_with_fused_qkv(0, d ** -0.5, qkv, o_exact)
+    padded = np.concatenate([qkv, np.full((6, hq + 2 * hkv, d), np.nan, np.float16)])
+    o_pad = np.full((16, hq, d), 3.0, np.float16)
+    b.attention_with_fused_qkv(0, d ** -0.5, padded, o_pad)
+    assert np.array_equal(o_pad[:10], o_exact)

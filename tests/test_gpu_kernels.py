@@ -1,0 +1,292 @@
+"""GPU parity of every HIP kernel launcher against the CPU oracle on identical seeded inputs.
+
+Integer/byte work (append scatter, gathers, page copies) must be bit-exact; attention outputs
+are fp16 with fp32 accumulation and must agree within atol = rtol = 1e-2 (the tolerance the
+path is specified to); RoPE outputs are compared at one fp16 ulp."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import kernels as ok
+from tests.gpu_util import DEV, dev, host, i32
+from tests.util import ATOL, RTOL, assert_close, build_paged_kv
+from tvm_amd import KVError
+from tvm_amd import kernels as K
+
+pytestmark = pytest.mark.gpu
+F16 = np.float16
+
+
+# ------------------------------------------------------------------------------ RoPE / append
+@pytest.mark.parametrize("d,hq,hkv", [(128, 32, 8), (64, 8, 2), (256, 4, 4)])
+@pytest.mark.parametrize("apply_rope", [1, 0])
+def test_fused_rope(d, hq, hkv, apply_rope):
+    rng = np.random.default_rng(0)
+    pos = np.array([0, 1, 2, 3, 100, 511, 2047, 4096, 65535, 131071, 7, 9, 33], np.int32)
+    n = len(pos)
+    qkv = rng.standard_normal((n, hq + 2 * hkv, d)).astype(F16)
+    eq, ek, ev = np.zeros((n, hq, d), F16), np.zeros((n, hkv, d), F16), np.zeros((n, hkv, d), F16)
+    ok.fused_rope(qkv, pos, eq, ek, ev, apply_rope)
+    q, k, v = (torch.zeros(a.shape, dtype=torch.float16, device=DEV) for a in (eq, ek, ev))
+    K.fused_rope(dev(qkv), i32(pos), q, k, v, apply_rope, 1.0, 1e4)
+    assert np.array_equal(host(v), ev)
+    if not apply_rope:
+        assert np.array_equal(host(q), eq) and np.array_equal(host(k), ek)
+        return
+    # same fp32 formula on both sides; device cos/sin may differ from libm in the last ulp, which
+    # can flip the fp16 rounding: allow one fp16 ulp (2^-10 relative) plus fp16 denormal spacing
+    assert_close(host(q), eq, atol=1e-3, rtol=2e-3, what="rope q")
+    assert_close(host(k), ek, atol=1e-3, rtol=2e-3, what="rope k")
+    exact = np.mean(host(q) == eq)
+    assert exact > 0.99, f"only {exact:.4f} of the rotated q elements are bit-identical to the oracle"
+
+
+def test_transpose_append_bit_exact_with_skips():
+    rng = np.random.default_rng(1)
+    hkv, ps, d, npages, n = 8, 16, 128, 64, 300
+    pages0 = rng.standard_normal((npages, 2, hkv, ps, d)).astype(F16)
+    slots = rng.permutation(npages * ps)[:n].astype(np.int32)
+    slots[[3, 77, 299]] = -1
+    k = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    expect = pages0.copy()
+    ok.transpose_append(expect, k, v, slots)
+    pages = dev(pages0)
+    K.tir_kv_cache_transpose_append(pages, dev(k), dev(v), i32(slots))
+    assert np.array_equal(host(pages), expect)
+    # gather back
+    keep = slots[slots >= 0]
+    kd = torch.zeros((3, len(keep), hkv, d), dtype=torch.float16, device=DEV)
+    vd = torch.zeros_like(kd)
+    K.tir_kv_cache_debug_get_kv(pages, i32(keep), kd, vd, 2)
+    assert np.array_equal(host(kd)[2], k[slots >= 0]) and np.array_equal(host(vd)[2], v[slots >= 0])
+    assert not host(kd)[:2].any()
+    K.tir_kv_cache_transpose_append(pages, dev(k[:0]), dev(v[:0]), i32(slots[:0]))  # empty append is a no-op
+    assert np.array_equal(host(pages), expect)
+
+
+def test_transpose_append_mla_and_gather_bit_exact():
+    rng = np.random.default_rng(2)
+    ps, d, npages, n = 64, 576, 6, 200
+    pages0 = rng.standard_normal((npages, ps, d)).astype(F16)
+    slots = rng.permutation(npages * ps)[:n].astype(np.int32)
+    slots[0] = -1
+    kv = rng.standard_normal((n, d)).astype(F16)
+    expect = pages0.copy()
+    ok.transpose_append_mla(expect, kv, slots)
+    pages = dev(pages0)
+    K.tir_kv_cache_transpose_append_mla(pages, dev(kv), i32(slots))
+    assert np.array_equal(host(pages), expect)
+    out = torch.zeros((2, n - 1, d), dtype=torch.float16, device=DEV)
+    K.tir_kv_cache_debug_get_kv_mla(pages, i32(slots[1:]), out, 1)
+    assert np.array_equal(host(out)[1], kv[1:])
+
+
+def test_copy_single_page_and_compact_copy_bit_exact():
+    rng = np.random.default_rng(3)
+    hkv, ps, d, npages = 8, 16, 128, 12
+    pages0 = rng.standard_normal((npages, 2, hkv, ps, d)).astype(F16)
+    expect = pages0.copy()
+    pages = dev(pages0)
+    for src, tgt, n in [(1, 3, 7), (0, 11, 16), (5, 6, 1), (2, 4, 0)]:
+        ok.copy_single_page(expect, src, tgt, n)
+        K.copy_single_page(pages, src, tgt, n)
+    assert np.array_equal(host(pages), expect)
+    indptr = np.array([0, 2, 2, 5], np.int32)
+    src_dst = np.array([[20, 21, 70, 71, 72], [17, 20, 65, 70, 71]], np.int32)  # later dst = earlier src
+    ok.compact_kv_copy(expect, indptr, src_dst, 3)
+    K.compact_kv_copy(pages, i32(indptr), i32(src_dst), 3)
+    assert np.array_equal(host(pages), expect)
+    mla0 = rng.standard_normal((5, 64, 576)).astype(F16)
+    em = mla0.copy()
+    ok.copy_single_page_mla(em, 4, 1, 33)
+    mp = dev(mla0)
+    K.copy_single_page_mla(mp, 4, 1, 33)
+    assert np.array_equal(host(mp), em)
+    with pytest.raises(KVError, match="out of range"):
+        K.copy_single_page(pages, 0, npages, 3)
+
+
+# ------------------------------------------------------------------------------ merge
+@pytest.mark.parametrize("h,d", [(32, 128), (8, 64), (128, 512)])
+def test_merge_state_inplace(h, d):
+    rng = np.random.default_rng(4)
+    n = 37
+    v1 = rng.standard_normal((n, h, d)).astype(F16)
+    v2 = rng.standard_normal((n, h, d)).astype(F16)
+    s1 = (rng.standard_normal((n, h)) * 4).astype(np.float32)
+    s2 = (rng.standard_normal((n, h)) * 4).astype(np.float32)
+    s2[0] = -5e4
+    s1[1] = -5e4
+    ev, es = v1.copy(), s1.copy()
+    ok.merge_state_inplace(ev, es, v2, s2)
+    gv, gs = dev(v1), dev(s1)
+    K.merge_state_inplace(gv, gs, dev(v2), dev(s2))
+    assert_close(host(gv), ev, atol=1e-3, rtol=1e-3, what="merge v")
+    assert_close(host(gs), es, atol=1e-4, rtol=1e-6, what="merge s")
+    assert np.array_equal(host(gv)[0], v1[0])  # empty other side leaves the row untouched
+
+
+# ------------------------------------------------------------------------------ decode
+def _decode_both(rng, kv_lens, hq, hkv, d, npages, scale=1.0):
+    pages, indptr, values, last, ks, vs = build_paged_kv(rng, kv_lens, npages, hkv, 16, d, scale=scale)
+    b = len(kv_lens)
+    q = rng.standard_normal((b, hq, d)).astype(F16)
+    eo, el = np.zeros((b, hq, d), F16), np.zeros((b, hq), np.float32)
+    z = np.zeros(b, np.int32)
+    ok.decode(q, pages, indptr, values, last, z, z, eo, el, 0, 1.0, 1e4, d ** -0.5)
+    go = torch.full((b, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((b, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_decode_paged_kv(dev(q), dev(pages), i32(indptr), i32(values), i32(last), i32(z), i32(z), go, gl, 0,
+                            1.0, 1e4, d ** -0.5)
+    return host(go), host(gl), eo, el
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (64, 8, 128), (8, 8, 128), (8, 4, 64), (16, 2, 64)])
+def test_decode_ragged_lengths_against_oracle(hq, hkv, d):
+    rng = np.random.default_rng(5)
+    # empty, single token, page boundaries, several chunks, spare slots
+    kv_lens = [0, 1, 15, 16, 17, 63, 64, 65, 100, 257, 0, 700, 33]
+    go, gl, eo, el = _decode_both(rng, kv_lens, hq, hkv, d, npages=160)
+    assert_close(go, eo, what="decode out")
+    assert_close(gl, el, atol=1e-3, rtol=1e-4, what="decode lse")
+    for i, n in enumerate(kv_lens):
+        if n == 0:
+            assert not go[i].any() and np.all(gl[i] == np.float32(-5e4))
+
+
+def test_decode_cfg1_shapes_against_oracle():
+    """BASELINE configs[0]: 4 sequences, contexts 512/1024/1500/2048 (+1 appended), 32/8 heads."""
+    rng = np.random.default_rng(6)
+    go, gl, eo, el = _decode_both(rng, [513, 1025, 1501, 2049], 32, 8, 128, npages=1024)
+    assert_close(go, eo, what="cfg1 decode out")
+    assert_close(gl, el, atol=1e-3, rtol=1e-4, what="cfg1 decode lse")
+
+
+def test_decode_long_sequence_many_chunks():
+    rng = np.random.default_rng(7)
+    go, gl, eo, el = _decode_both(rng, [9000, 5], 32, 8, 128, npages=600)
+    assert_close(go, eo, what="long decode out")
+    assert_close(gl, el, atol=1e-3, rtol=1e-4, what="long decode lse")
+
+
+def test_decode_ignores_garbage_beyond_last_page_len():
+    """Slots of the last page beyond last_page_len may hold NaN/Inf bit patterns."""
+    rng = np.random.default_rng(8)
+    hq, hkv, d = 8, 2, 128
+    pages, indptr, values, last, ks, vs = build_paged_kv(rng, [21], 4, hkv, 16, d)
+    pages[values[1], :, :, 5:, :] = np.float16(np.nan)
+    q = rng.standard_normal((1, hq, d)).astype(F16)
+    eo, el = np.zeros((1, hq, d), F16), np.zeros((1, hq), np.float32)
+    z = np.zeros(1, np.int32)
+    clean = pages.copy()
+    clean[values[1], :, :, 5:, :] = 0
+    ok.decode(q, clean, indptr, values, last, z, z, eo, el, 0, 1.0, 1e4, d ** -0.5)
+    go = torch.zeros((1, hq, d), dtype=torch.float16, device=DEV)
+    gl = torch.zeros((1, hq), dtype=torch.float32, device=DEV)
+    K.batch_decode_paged_kv(dev(q), dev(pages), i32(indptr), i32(values), i32(last), i32(z), i32(z), go, gl, 0, 1.0,
+                            1e4, d ** -0.5)
+    assert np.isfinite(host(go)).all()
+    assert_close(host(go), eo, what="decode with NaN padding")
+
+
+def test_decode_rejects_what_is_not_built():
+    t = torch.zeros((1, 8, 128), dtype=torch.float16, device=DEV)
+    pages = torch.zeros((2, 2, 2, 16, 128), dtype=torch.float16, device=DEV)
+    lse = torch.zeros((1, 8), dtype=torch.float32, device=DEV)
+    one = i32([0, 1])
+    with pytest.raises(KVError, match="inline RoPE") as info:
+        K.batch_decode_paged_kv(t, pages, one, i32([0]), i32([1]), i32([0]), i32([0]), t, lse, 1, 1.0, 1e4, 1.0)
+    assert info.value.code == -2
+
+
+# ------------------------------------------------------------------------------ prefill
+def _ragged_both(rng, lens, hq, hkv, dqk, dv, causal, scale=1.0):
+    n = sum(lens)
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    q = (rng.standard_normal((n, hq, dqk)) * scale).astype(F16)
+    k = (rng.standard_normal((n, hkv, dqk)) * scale).astype(F16)
+    v = (rng.standard_normal((n, hkv, dv)) * scale).astype(F16)
+    eo, el = np.zeros((n, hq, dv), F16), np.zeros((n, hq), np.float32)
+    zq, zb = np.zeros(n, np.int32), np.zeros(len(lens), np.int32)
+    ok.prefill_ragged(q, indptr, k, v, indptr, zq, zb, eo, el, causal, 0, 1.0, 1e4, dqk ** -0.5)
+    go = torch.full((n, hq, dv), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_ragged_kv(dev(q), i32(indptr), dev(k), dev(v), i32(indptr), i32(zq), i32(zb), go, gl, causal, 0,
+                              1.0, 1e4, dqk ** -0.5)
+    return host(go), host(gl), eo, el
+
+
+@pytest.mark.parametrize("hq,hkv,dqk,dv", [(32, 8, 128, 128), (8, 8, 128, 128), (8, 2, 64, 64), (16, 16, 192, 128)])
+@pytest.mark.parametrize("causal", [1, 0])
+def test_ragged_prefill_against_oracle(hq, hkv, dqk, dv, causal):
+    rng = np.random.default_rng(9)
+    lens = [1, 2, 31, 32, 33, 63, 64, 65, 130, 7]
+    go, gl, eo, el = _ragged_both(rng, lens, hq, hkv, dqk, dv, causal)
+    assert_close(go, eo, what="ragged out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="ragged lse")
+
+
+def test_ragged_prefill_longer_chunk():
+    rng = np.random.default_rng(10)
+    go, gl, eo, el = _ragged_both(rng, [300, 5, 200], 32, 8, 128, 128, 1)
+    assert_close(go, eo, what="ragged out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="ragged lse")
+
+
+def _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages):
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, kv_lens, npages, hkv, 16, d)
+    n = sum(q_lens)
+    qindptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    zb, zq = np.zeros(len(kv_lens), np.int32), np.zeros(n, np.int32)
+    ok.prefill_paged(q, qindptr, pages, pindptr, pvalues, last, zb, zq, eo, el, causal, 0, 1.0, 1e4, d ** -0.5)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_paged_kv(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(zb),
+                             i32(zq), go, gl, causal, 0, 1.0, 1e4, d ** -0.5)
+    return host(go), host(gl), eo, el
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("causal", [0, 1])
+def test_paged_prefill_against_oracle(hq, hkv, d, causal):
+    rng = np.random.default_rng(11)
+    kv_lens = [40, 16, 0, 75, 200, 64, 1]
+    q_lens = [7, 16, 3, 30, 64, 1, 1]
+    if causal:  # causal paged calls see a KV that already holds the queries' own tokens
+        kv_lens = [max(k, q) for k, q in zip(kv_lens, q_lens)]
+    go, gl, eo, el = _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages=64)
+    assert_close(go, eo, what="paged out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="paged lse")
+
+
+def test_chunked_prefill_composition_matches_oracle():
+    """ragged(causal) + paged(non-causal) + merge_state: the chunked-prefill path of the cache."""
+    rng = np.random.default_rng(12)
+    hq, hkv, d = 32, 8, 128
+    prefix, chunk = [100, 0, 333], [50, 20, 129]
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, prefix, 64, hkv, 16, d)
+    n = sum(chunk)
+    ind = np.concatenate([[0], np.cumsum(chunk)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    zq, zb = np.zeros(n, np.int32), np.zeros(3, np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    to, tl = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    ok.prefill_ragged(q, ind, k, v, ind, zq, zb, eo, el, 1, 0, 1.0, 1e4, d ** -0.5)
+    ok.prefill_paged(q, ind, pages, pindptr, pvalues, last, zb, zq, to, tl, 0, 0, 1.0, 1e4, d ** -0.5)
+    ok.merge_state_inplace(eo, el, to, tl)
+    go = torch.zeros((n, hq, d), dtype=torch.float16, device=DEV)
+    gl = torch.zeros((n, hq), dtype=torch.float32, device=DEV)
+    ho = torch.zeros((n, hq, d), dtype=torch.float16, device=DEV)
+    hl = torch.zeros((n, hq), dtype=torch.float32, device=DEV)
+    qd = dev(q)
+    K.batch_prefill_ragged_kv(qd, i32(ind), dev(k), dev(v), i32(ind), i32(zq), i32(zb), go, gl, 1, 0, 1.0, 1e4, d ** -0.5)
+    K.batch_prefill_paged_kv(qd, i32(ind), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(zb), i32(zq), ho, hl,
+                             0, 0, 1.0, 1e4, d ** -0.5)
+    K.merge_state_inplace(go, gl, ho, hl)
+    assert_close(host(go), eo, what="chunked prefill out")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="chunked prefill lse")
