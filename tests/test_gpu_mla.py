@@ -1,0 +1,130 @@
+"""GPU parity of the MLA latent-cache path: the paged MLA kernel against the CPU oracle on
+identical inputs (decode-shaped calls take the split-KV route, prefill-shaped calls do not), and
+the cache-level flow of the reference's MLA test (append_mla_kv, self_attention on expanded
+192/128-dim heads, cross_attention on the absorbed query, merge) against the definition of MLA:
+expand the latent with w_kv and run plain multi-head attention
+(tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_mla_tir.py:293-398).
+
+Relative to "the reference's llvm kernels" MLA parity is unpinned by construction: the reference
+has no llvm MLA kernel; the oracle function is pinned to the closed form in
+tests/test_oracle_kernels.py."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import closed_form as cf
+from oracle import kernels as ok
+from tests.gpu_util import DEV, GpuCache, dev, host, i32
+from tests.util import assert_close
+from tvm_amd import kernels as K
+
+pytestmark = pytest.mark.gpu
+F16 = np.float16
+H, D_LAT, D_ROPE, D_NOPE, D_V = 128, 512, 64, 128, 128
+D_QK = D_LAT + D_ROPE
+
+
+def _latent_pool(rng, kv_lens, ps, npages):
+    pages = np.zeros((npages, ps, D_QK), F16)
+    order = rng.permutation(npages)
+    indptr, values, last, rows = [0], [], [], []
+    cursor = 0
+    for n in kv_lens:
+        npg = (n + ps - 1) // ps
+        ids = order[cursor:cursor + npg]
+        cursor += npg
+        lat = (rng.standard_normal((n, D_QK)) * 0.5).astype(F16)
+        for t in range(n):
+            pages[ids[t // ps], t % ps] = lat[t]
+        values.extend(int(x) for x in ids)
+        indptr.append(len(values))
+        last.append(0 if n == 0 else (n - 1) % ps + 1)
+        rows.append(lat)
+    return pages, np.array(indptr, np.int32), np.array(values, np.int32), np.array(last, np.int32), rows
+
+
+def _mla_both(rng, kv_lens, q_lens, ps, npages, causal=0, heads=H):
+    pages, pindptr, pvalues, last, _ = _latent_pool(rng, kv_lens, ps, npages)
+    n = sum(q_lens)
+    qindptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    q = (rng.standard_normal((n, heads, D_QK)) * 0.5).astype(F16)
+    eo, el = np.zeros((n, heads, D_LAT), F16), np.zeros((n, heads), np.float32)
+    sm = (D_NOPE + D_ROPE) ** -0.5
+    ok.prefill_paged_mla(q, qindptr, pages, pindptr, pvalues, last, eo, el, causal, sm, d_latent=D_LAT)
+    go = torch.full((n, heads, D_LAT), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, heads), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_paged_kv_mla(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(last), go, gl,
+                                 causal, sm)
+    return host(go), host(gl), eo, el
+
+
+@pytest.mark.parametrize("ps", [64, 16])
+def test_mla_decode_shaped_split_kv(ps):
+    rng = np.random.default_rng(30)
+    kv_lens = [1, 63, 64, 65, 200, 1000, 0, 129]
+    go, gl, eo, el = _mla_both(rng, kv_lens, [1] * len(kv_lens), ps, npages=(40 if ps == 64 else 130))
+    assert_close(go, eo, what="mla decode out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla decode lse")
+    assert not go[6].any() and np.all(gl[6] == np.float32(-5e4))
+
+
+@pytest.mark.parametrize("causal", [0, 1])
+def test_mla_prefill_shaped(causal):
+    rng = np.random.default_rng(31)
+    kv_lens, q_lens = [300, 40, 0, 77], [33, 5, 2, 77]
+    if causal:
+        kv_lens = [max(k, q) for k, q in zip(kv_lens, q_lens)]
+    go, gl, eo, el = _mla_both(rng, kv_lens, q_lens, 64, npages=16, causal=causal, heads=16)
+    assert_close(go, eo, what="mla prefill out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla prefill lse")
+
+
+def test_mla_cache_flow_matches_the_definition():
+    """Prefill a chunk on a cached prefix, then decode one token, through the cache verbs."""
+    rng = np.random.default_rng(32)
+    heads, layers, ps = 16, 1, 64
+    sm = (D_NOPE + D_ROPE) ** -0.5
+    w_kv = (rng.standard_normal((D_LAT, heads * (D_NOPE + D_V))) * 0.04).astype(np.float64)
+    w = w_kv.reshape(D_LAT, heads, D_NOPE + D_V)
+    w_uk, w_uv = w[..., :D_NOPE], w[..., D_NOPE:]
+    cache = GpuCache([4, 1024, 256, ps, 0], layers, heads, 1, D_QK, D_LAT, attn_kinds=[1], rope_mode=0)
+    cached = {0: np.zeros((0, D_QK), F16), 1: np.zeros((0, D_QK), F16)}
+    cache.add_sequence(0)
+    cache.add_sequence(1)
+    for lens in ([70, 3], [37, 90], [1, 1]):
+        ids = [0, 1]
+        cache.begin_forward(ids, lens)
+        total = sum(lens)
+        q = (rng.standard_normal((total, heads, D_NOPE + D_ROPE)) * 0.5).astype(F16)
+        kv = (rng.standard_normal((total, D_QK)) * 0.5).astype(F16)
+        is_decode = all(n == 1 for n in lens)
+        all_new = all(cached[s].shape[0] == 0 for s in ids)
+        cache.append_mla_kv(0, kv)
+        o1 = np.zeros((total, heads, D_V), F16)
+        l1 = np.zeros((total, heads), np.float32)
+        if not is_decode:
+            k_full, v_full = cf.mla_expand(kv, w_kv, heads, D_NOPE, D_V)
+            cache.self_attention(0, sm, q, k_full.astype(F16), v_full.astype(F16), o1, l1)
+        if not all_new or is_decode:
+            q_abs = np.concatenate([np.einsum("qhn,lhn->qhl", q[..., :D_NOPE].astype(np.float64), w_uk),
+                                    q[..., D_NOPE:].astype(np.float64)], axis=-1).astype(F16)
+            o2 = np.zeros((total, heads, D_LAT), F16)
+            l2 = np.zeros((total, heads), np.float32)
+            cache.cross_attention(0, sm, q_abs, o2, l2)
+            cross = np.einsum("qhl,lhv->qhv", o2.astype(np.float64), w_uv).astype(F16)
+            if is_decode:
+                o1 = cross
+            else:
+                cache.merge_attn_output_inplace(o1, l1, cross, l2)
+        cache.end_forward()
+        cursor = 0
+        for sid, n in zip(ids, lens):
+            cached[sid] = np.concatenate([cached[sid], kv[cursor:cursor + n]])
+            k_seq, v_seq = cf.mla_expand(cached[sid], w_kv, heads, D_NOPE, D_V)
+            k_seq = k_seq.astype(F16) if not is_decode else k_seq
+            expected, _ = cf.attention(q[cursor:cursor + n], k_seq, v_seq, sm, causal=True)
+            assert_close(o1[cursor:cursor + n], expected, atol=1e-2, rtol=2e-2, what=f"mla flow seq {sid} lens {lens}")
+            back = np.zeros((layers, cached[sid].shape[0], D_QK), F16)
+            cache.debug_get_kv_mla(sid, 0, cached[sid].shape[0], back)
+            assert np.array_equal(back[0], cached[sid])
+            cursor += n
