@@ -94,6 +94,28 @@ def time_region(torch, fn, iters):
     return start.elapsed_time(stop) / iters
 
 
+def calibrate(num_bytes=2 << 30, iters=10):
+    """Plain streaming read and copy of `num_bytes`: what the memory system of this box delivers
+    to the simplest possible kernel.  Prints one JSON line."""
+    import torch
+
+    from tvm_amd import kernels as K
+
+    dev = "cuda:0"
+    src = torch.empty(num_bytes // 2, dtype=torch.float16, device=dev).normal_()
+    dst = torch.empty_like(src)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    K.stream_read(src, sink)
+    K.stream_copy(src, dst)
+    ms_read = time_region(torch, lambda i: K.stream_read(src, sink), iters)
+    ms_copy = time_region(torch, lambda i: K.stream_copy(src, dst), iters)
+    out = {"calibration": "plain streaming kernels", "bytes": num_bytes,
+           "read_GBps": round(num_bytes / ms_read / 1e6, 1), "read_ms": round(ms_read, 4),
+           "copy_GBps_read_plus_write": round(2 * num_bytes / ms_copy / 1e6, 1), "copy_ms": round(ms_copy, 4)}
+    print(json.dumps(out))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -101,7 +123,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (profiling runs)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the chunked-prefill leg (profiling runs)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="only run the plain 2 GiB streaming read and copy kernels (bandwidth calibration; "
+                         "known-size dispatches for scaling rocprofv3 traffic counters)")
     args = ap.parse_args()
+    if args.calibrate:
+        return calibrate()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; the path shards per kv head without any exchange "
                  "(see DESIGN.md), and no multi-GPU figure is produced. Use --gpus 1.")

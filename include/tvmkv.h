@@ -175,6 +175,13 @@ int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr,
                           int32_t total_copy_length, int64_t num_pages, int32_t num_kv_heads,
                           int32_t page_size, int32_t head_dim, void* stream);
 
+/* Measurement utilities (no counterpart in the reference): a plain streaming read (XOR-folded,
+ * the result is discarded) and a plain copy of `num_bytes` (a multiple of 16) bytes.  The
+ * benchmark uses them to calibrate the achievable HBM bandwidth of the box, and the profiling
+ * notes use the copy to scale the FETCH_SIZE / WRITE_SIZE counters. `sink` is 4 writable bytes. */
+int tvmkv_stream_read(const void* src, int64_t num_bytes, void* sink, void* stream);
+int tvmkv_stream_copy(const void* src, void* dst, int64_t num_bytes, void* stream);
+
 /* ======================================================================================
  * (2) Cache object
  * ====================================================================================== */

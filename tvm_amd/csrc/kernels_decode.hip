@@ -24,6 +24,9 @@
 //   [floor(page_indptr[b]/CP) + b, floor(page_indptr[b+1]/CP) + b + 1)
 // which always holds ceil(npages_b/CP) chunks; a workgroup finds its sequence by binary search
 // on page_indptr, so the grid size depends on shapes only (floor(nnz_pages/CP) + B slots).
+#include <algorithm>
+#include <cstdlib>
+
 #include "kernels_common.cuh"
 
 namespace tvmkv {
@@ -61,6 +64,22 @@ __device__ __forceinline__ int find_sequence(const int32_t* page_indptr, int bat
     }
   }
   return lo;
+}
+
+// Same answer as find_sequence, computed by one wavefront with one round trip per 64 sequences:
+// lane i evaluates slot_begin(base + i) <= slot, and because slot_begin is increasing the number
+// of set lanes is the position of the last sequence that qualifies.
+__device__ __forceinline__ int find_sequence_wave(const int32_t* page_indptr, int batch, int cp, int slot,
+                                                  int lane) {
+  int b = 0;
+  for (int base = 0; base < batch; base += 64) {
+    const int idx = base + lane;
+    const bool le = idx < batch && slot_begin(page_indptr, idx, cp) <= slot;
+    const int count = __popcll(__ballot(le));
+    if (count > 0) b = base + count - 1;
+    if (count < 64) break;
+  }
+  return b;
 }
 
 template <int D, int GROUP, int PS>
@@ -240,37 +259,304 @@ __global__ __launch_bounds__(256) void decode_splitkv_kernel(DecodeParams p) {
   }
 }
 
-// One block per (sequence, query head); D threads.  Sequences with one chunk were finished by
-// the main kernel; sequences without pages get the empty-KV answer out = 0, lse = -5e4
+// ------------------------------------------------------------------------------------------
+// MFMA variant for head_dim 128 (any GQA group up to 16).
+//
+// The VALU kernel above spends ~90*GROUP vector instructions per 8 KiB page, which for groups of
+// 4-8 query heads is about as much issue time as the page's HBM time.  Here the two contractions
+// run on v_mfma_f32_16x16x32_f16 with the query heads of the group padded to the 16-wide N axis:
+//   S^T[token, head] = K Q^T   -- K fragments come straight from global memory in the MFMA
+//                                 A-layout (lane = token row, 16 bytes of features), no staging;
+//   O^T[d, head]     = V^T P^T -- V is loaded coalesced (16 lanes per 256-byte row), transposed
+//                                 through a wave-private LDS tile so that tokens run along the
+//                                 contraction axis; P stays in registers (the S^T accumulator
+//                                 layout is the B-operand layout).
+// A wave consumes two pages (32 tokens) per step: 16 KiB of K/V, 16 MFMAs, a handful of vector
+// instructions for the softmax.  Per-head state (m, l) is lane-local; the running maximum is
+// shared across the four lane groups with two shuffles per step.
+// ------------------------------------------------------------------------------------------
+constexpr int DM_D = 128;
+constexpr int DM_PS = 16;
+constexpr int DM_VROW = 36;  // halfs per row of the transposed V tile (32 tokens + padding)
+
+__global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int group, int num_items) {
+  constexpr int D = DM_D, PS = DM_PS, VROW = DM_VROW;
+  static_assert(D * VROW * sizeof(half_t) >= 16 * D * sizeof(float), "the merge buffer aliases the V tile");
+  __shared__ __attribute__((aligned(16))) half_t Vt_all[4][D * VROW];
+  __shared__ float sm_m[4][16];
+  __shared__ float sm_l[4][16];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int c16 = lane & 15;   // MFMA column (query head in group) / A-row (token) / V feature piece
+  const int g4 = lane >> 4;    // lane group 0..3
+  const int cp = p.chunk_pages;
+  half_t* Vt = Vt_all[wave];
+  const int64_t head_stride = static_cast<int64_t>(PS) * D;
+
+  // Persistent workgroups: item = (chunk slot, kv head), strided over the grid.  Neighbouring
+  // workgroups take the kv heads of one slot, i.e. the same pages.
+  for (int item = blockIdx.x; item < num_items; item += gridDim.x) {
+  const int slot = item / p.h_kv;
+  const int kvh = item - slot * p.h_kv;
+  const int b = find_sequence_wave(p.page_indptr, p.batch_size, cp, slot, lane);
+  const int pbeg = p.page_indptr[b];
+  const int npages = p.page_indptr[b + 1] - pbeg;
+  const int chunk = slot - slot_begin(p.page_indptr, b, cp);
+  const int nchunks = (npages + cp - 1) / cp;
+  if (chunk >= nchunks) continue;  // spare slot (uniform over the workgroup)
+  const int kv_len = (npages - 1) * PS + p.last_page_len[b];
+  const int page_lo = chunk * cp;
+  const int page_hi = min(page_lo + cp, npages);
+
+  // Q^T fragments (B operand): column = head c16 of the group, contraction slots = 8 features.
+  half8_t qf[4];
+  {
+    const half_t* qrow = p.q + (static_cast<int64_t>(b) * p.h_q + kvh * group + c16) * D + g4 * 8;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) qf[ks] = c16 < group ? ld16(qrow + ks * 32).h8 : zero16().h8;
+  }
+  float4_t o[8];
+#pragma unroll
+  for (int db = 0; db < 8; ++db) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
+  float m = kNegInit, lsum = 0.f;
+
+  // One step = pages (pi, pi+1).  K: lane reads row c16 of the page, features ks*32 + g4*8.
+  // V: lane reads rows 4*g4 + j of the page, features c16*8 (coalesced 256-byte rows).
+  struct Regs {
+    Vec16 k[2][4];
+    Vec16 v[2][4];
+  };
+  auto issue = [&](int pi, Regs& r) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (pi + h < page_hi) {
+        const int page = __builtin_amdgcn_readfirstlane(p.page_values[pbeg + pi + h]);
+        const half_t* kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * head_stride;
+        const half_t* vbase = kbase + static_cast<int64_t>(p.h_kv) * head_stride;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r.v[h][j] = ld16(vbase + (4 * g4 + j) * D + c16 * 8);
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = zero16();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r.v[h][j] = zero16();
+      }
+    }
+  };
+
+  auto consume = [&](int pi, Regs& r) {
+    const bool partial = (pi + 2) * PS > kv_len;  // wave-uniform
+    // ---- V: zero the rows beyond kv_len, transpose into the wave's LDS tile ----------------
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (partial) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if ((pi + h) * PS + 4 * g4 + j >= kv_len) r.v[h][j] = zero16();
+        }
+      }
+#pragma unroll
+      for (int e2 = 0; e2 < 4; ++e2) {
+        const uint32_t w0 = r.v[h][0].w[e2], w1 = r.v[h][1].w[e2], w2 = r.v[h][2].w[e2], w3 = r.v[h][3].w[e2];
+        uint2 even, odd;
+        even.x = (w0 & 0xffffu) | (w1 << 16);
+        even.y = (w2 & 0xffffu) | (w3 << 16);
+        odd.x = (w0 >> 16) | (w1 & 0xffff0000u);
+        odd.y = (w2 >> 16) | (w3 & 0xffff0000u);
+        *reinterpret_cast<uint2*>(Vt + (c16 * 8 + 2 * e2) * VROW + h * 16 + 4 * g4) = even;
+        *reinterpret_cast<uint2*>(Vt + (c16 * 8 + 2 * e2 + 1) * VROW + h * 16 + 4 * g4) = odd;
+      }
+    }
+    // ---- S^T = K Q^T for both pages ---------------------------------------------------------
+    float4_t s[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      s[h] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) s[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][ks].h8, qf[ks], s[h], 0, 0, 0);
+    }
+    // s[h][j]: token (pi+h)*PS + 4*g4 + j, head c16
+    float mx = kNegInit;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float v = s[h][j] * p.scale_log2;
+        if (partial) v = ((pi + h) * PS + 4 * g4 + j < kv_len) ? v : kNegInit;
+        s[h][j] = v;
+        mx = fmaxf(mx, v);
+      }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = fast_exp2(m - m_new);
+    m = m_new;
+    lsum *= alpha;
+    if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {
+#pragma unroll
+      for (int db = 0; db < 8; ++db) o[db] *= alpha;
+    }
+    half8_t pf;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float pj = fast_exp2(s[h][j] - m_new);
+        if (partial) pj = ((pi + h) * PS + 4 * g4 + j < kv_len) ? pj : 0.f;
+        lsum += pj;
+        pf[h * 4 + j] = static_cast<half_t>(pj);
+      }
+    }
+    // the LDS tile is written and read by this wave only: order the two without a block barrier
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // ---- O^T += V^T P^T: contraction slot g4*8 + i <-> page i/4, token 4*g4 + i%4 ------------
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      const half_t* vrow = Vt + (db * 16 + c16) * VROW + 4 * g4;
+      const half4_t lo = *reinterpret_cast<const half4_t*>(vrow);
+      const half4_t hi = *reinterpret_cast<const half4_t*>(vrow + 16);
+      half8_t a;
+      a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
+      a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pf, o[db], 0, 0, 0);
+    }
+    // next step's LDS writes must not overtake these reads
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  // No software pipelining: three waves per SIMD (twelve per CU, each with 16 KiB of loads in
+  // flight while it waits) hide the load latency; a second register buffer costs occupancy and
+  // measured slower.
+  Regs ra;
+  for (int pi = page_lo + 2 * wave; pi < page_hi; pi += 8) {
+    issue(pi, ra);
+    consume(pi, ra);
+  }
+
+  // ---- the row sums are per lane group: add them up; m is already common -----------------------
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+
+  // ---- merge the 4 waves through LDS: o[db][j] is feature db*16 + 4*g4 + j of head c16 ---------
+  // (the wave's V tile is dead now and becomes its [16][D] fp32 output buffer)
+  float* sm_o_w = reinterpret_cast<float*>(Vt_all[wave]);
+#pragma unroll
+  for (int db = 0; db < 8; ++db) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sm_o_w[c16 * D + db * 16 + 4 * g4 + j] = o[db][j];
+  }
+  if (g4 == 0) {
+    sm_m[wave][c16] = m;
+    sm_l[wave][c16] = lsum;
+  }
+  __syncthreads();
+
+  const bool single_chunk = nchunks == 1;
+  for (int idx = tid; idx < group * D; idx += 256) {
+    const int g = idx / D;
+    const int d = idx % D;
+    float mx = sm_m[0][g];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, sm_m[w][g]);
+    float lt = 0.f, acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float sc = fast_exp2(sm_m[w][g] - mx);
+      lt += sm_l[w][g] * sc;
+      acc += reinterpret_cast<const float*>(Vt_all[w])[g * D + d] * sc;
+    }
+    const int hq = kvh * group + g;
+    if (single_chunk) {
+      const float denom = lt + fast_exp2(kNegInit - mx);
+      p.output[(static_cast<int64_t>(b) * p.h_q + hq) * D + d] = static_cast<half_t>(acc / denom);
+      if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = mx + fast_log2(denom);
+    } else {
+      p.part_o[(static_cast<int64_t>(slot) * p.h_q + hq) * D + d] = acc;
+      if (d == 0) {
+        p.part_ml[(static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 0] = mx;
+        p.part_ml[(static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 1] = lt;
+      }
+    }
+  }
+  __syncthreads();  // the merge buffers are the next item's V tiles
+  }  // items
+}
+
+// Merge of the per-chunk partial states.  One wavefront per (sequence, query head), four per
+// block.  Lane c first fetches (m, l) of chunk c, a wave reduction gives the common maximum and
+// the total sum, and every lane keeps the rescale factor of "its" chunk; the second pass streams
+// the partial outputs (each lane owns D/64 features) with the factor broadcast by shuffle, loads
+// of several chunks in flight at once.  Sequences with one chunk were finished by the main
+// kernel; sequences without pages get the empty-KV answer out = 0, lse = -5e4
 // (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:129-130,173-176).
 template <int D>
-__global__ __launch_bounds__(D) void decode_merge_kernel(DecodeParams p, int page_size) {
-  const int b = blockIdx.x;
-  const int hq = blockIdx.y;
-  const int d = threadIdx.x;
+__global__ __launch_bounds__(256) void decode_merge_kernel(DecodeParams p, int total_rows) {
+  constexpr int EPL = D / 64;  // features per lane
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // (b, hq) flattened
+  if (row >= total_rows) return;
+  const int b = row / p.h_q;
+  const int hq = row % p.h_q;
   const int cp = p.chunk_pages;
   const int npages = p.page_indptr[b + 1] - p.page_indptr[b];
   const int nchunks = (npages + cp - 1) / cp;
-  const int64_t out_idx = (static_cast<int64_t>(b) * p.h_q + hq) * D + d;
   if (nchunks == 1) return;
+  half_t* out = p.output + static_cast<int64_t>(row) * D + lane * EPL;
   if (nchunks == 0) {
-    p.output[out_idx] = static_cast<half_t>(0.f);
-    if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = kNegInit;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) out[e] = static_cast<half_t>(0.f);
+    if (lane == 0) p.lse[row] = kNegInit;
     return;
   }
   const int s0 = slot_begin(p.page_indptr, b, cp);
-  float mx = kNegInit;
-  for (int c = 0; c < nchunks; ++c) mx = fmaxf(mx, p.part_ml[(static_cast<int64_t>(s0 + c) * p.h_q + hq) * 2]);
-  float lsum = 0.f, acc = 0.f;
-  for (int c = 0; c < nchunks; ++c) {
-    const int64_t base = static_cast<int64_t>(s0 + c) * p.h_q + hq;
-    const float sc = fast_exp2(p.part_ml[base * 2] - mx);
-    lsum += p.part_ml[base * 2 + 1] * sc;
-    acc += p.part_o[base * D + d] * sc;
+  float mx = kNegInit, lsum = 0.f;
+  float acc[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
+  for (int c0 = 0; c0 < nchunks; c0 += 64) {
+    const int c = c0 + lane;
+    float m_c = kNegInit, l_c = 0.f;
+    if (c < nchunks) {
+      const float2 ml = *reinterpret_cast<const float2*>(p.part_ml + (static_cast<int64_t>(s0 + c) * p.h_q + hq) * 2);
+      m_c = ml.x;
+      l_c = ml.y;
+    }
+    float mx_new = m_c;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx_new = fmaxf(mx_new, __shfl_xor(mx_new, off, 64));
+    mx_new = fmaxf(mx_new, mx);
+    const float rescale_old = fast_exp2(mx - mx_new);
+    const float sc = fast_exp2(m_c - mx_new);
+    float lpart = l_c * sc;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) lpart += __shfl_xor(lpart, off, 64);
+    lsum = lsum * rescale_old + lpart;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[e] *= rescale_old;
+    mx = mx_new;
+    const int n_here = min(64, nchunks - c0);
+    const float* po = p.part_o + (static_cast<int64_t>(s0 + c0) * p.h_q + hq) * D + lane * EPL;
+    const int64_t stride = static_cast<int64_t>(p.h_q) * D;
+#pragma unroll 8
+    for (int k = 0; k < n_here; ++k) {
+      const float w = __shfl(sc, k, 64);
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) acc[e] = fmaf(po[k * stride + e], w, acc[e]);
+    }
   }
   const float denom = lsum + fast_exp2(kNegInit - mx);
-  p.output[out_idx] = static_cast<half_t>(acc / denom);
-  if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = mx + fast_log2(denom);
+  const float inv = 1.0f / denom;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) out[e] = static_cast<half_t>(acc[e] * inv);
+  if (lane == 0) p.lse[row] = mx + fast_log2(denom);
 }
 
 // ---- per-device workspace for the partial states, grown on demand --------------------------
@@ -299,11 +585,29 @@ static void* get_workspace(size_t bytes) {
   return ws.ptr;
 }
 
+static int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    HIP_CHECK(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+    cached[dev] = n > 0 ? n : 256;
+  }
+  return cached[dev];
+}
+
 // Pages per chunk from shapes only: aim at ~8K workgroups, keep a chunk between 4 and 64 pages.
 static int pick_chunk_pages(int64_t nnz_pages, int h_kv) {
-  int64_t cp = nnz_pages * h_kv / 8192;
-  int pow2 = 4;
-  while (pow2 * 2 <= cp && pow2 < 64) pow2 *= 2;
+  static const char* forced = getenv("TVMKV_DECODE_CHUNK_PAGES");  // tuning aid
+  if (forced != nullptr && atoi(forced) >= 8 && atoi(forced) % 8 == 0) return atoi(forced);
+  // ~2300 work items = three rounds of 3 workgroups x 256 CUs; every item pays ~2 us of fixed
+  // cost (locating its sequence, q, the cross-wave merge), so chunks should not be smaller than
+  // that buys.  One step of the MFMA kernel is 2 pages per wave, 8 per workgroup.
+  const int64_t cp = nnz_pages * h_kv / 2304;
+  int pow2 = 8;
+  while (pow2 < 128 && pow2 * 3 / 2 <= cp) pow2 *= 2;  // nearest power of two
   return pow2;
 }
 
@@ -367,14 +671,28 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
   const dim3 grid(static_cast<unsigned>(slots), h_kv);
   const int group = h_q / h_kv;
   hipStream_t s = as_stream(stream);
-  if (d == 128) {
+  if (d == 128 && group <= 16) {
+    const int64_t num_items = slots * h_kv;
+    KV_CHECK(num_items < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many work items";
+    // One item per workgroup by default (measured a little faster than a resident-size grid
+    // striding over the items); TVMKV_DECODE_WGS_PER_CU=n caps the grid at n workgroups per CU.
+    static const char* wgs_env = getenv("TVMKV_DECODE_WGS_PER_CU");
+    int64_t grid_x = num_items;
+    if (wgs_env != nullptr && atoi(wgs_env) > 0) {
+      grid_x = std::min<int64_t>(num_items, static_cast<int64_t>(compute_units()) * atoi(wgs_env));
+    }
+    hipLaunchKernelGGL(decode_mfma_kernel, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group,
+                       static_cast<int>(num_items));
+    KV_LAUNCH_CHECK();
+    hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
+  } else if (d == 128) {
     launch_decode<128, 16>(p, group, grid, s);
     KV_LAUNCH_CHECK();
-    hipLaunchKernelGGL(decode_merge_kernel<128>, dim3(batch_size, h_q), dim3(128), 0, s, p, page_size);
+    hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
   } else {
     launch_decode<64, 16>(p, group, grid, s);
     KV_LAUNCH_CHECK();
-    hipLaunchKernelGGL(decode_merge_kernel<64>, dim3(batch_size, h_q), dim3(64), 0, s, p, page_size);
+    hipLaunchKernelGGL(decode_merge_kernel<64>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
   }
   KV_LAUNCH_CHECK();
   KV_API_END();

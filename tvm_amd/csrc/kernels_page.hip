@@ -243,6 +243,27 @@ __global__ __launch_bounds__(256) void merge_state_inplace_kernel(half_t* __rest
   if (c == 0) s[row] = log2f(s_val + s_other_val) + s_max;
 }
 
+// ------------------------------------------------------------------------------------------
+// Measurement utilities: a plain streaming read and a plain copy of known size, used to
+// calibrate what the memory system delivers and to scale hardware traffic counters.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ src, int64_t n16,
+                                                          uint32_t* __restrict__ sink) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  uint32_t acc = 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride) {
+    const uint4 v = src[i];
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  if (acc == 0x9e3779b9u) sink[0] = acc;  // keeps the loads alive; practically never taken
+}
+
+__global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                          int64_t n16) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
 inline dim3 grid_for(int64_t threads, int block = 256) { return dim3(static_cast<unsigned>((threads + block - 1) / block)); }
 
 }  // namespace tvmkv
@@ -391,6 +412,26 @@ int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr, const 
   hipLaunchKernelGGL(compact_kv_copy_kernel, grid_for(threads), dim3(256), 0, as_stream(stream),
                      static_cast<half_t*>(pages), copy_length_indptr, copy_src_dst_pos, batch_size,
                      total_copy_length, num_kv_heads, page_size, head_dim);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_stream_read(const void* src, int64_t num_bytes, void* sink, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(src && sink && num_bytes >= 0 && num_bytes % 16 == 0) << "stream_read: bad arguments";
+  if (num_bytes == 0) return TVMKV_OK;
+  hipLaunchKernelGGL(stream_read_kernel, dim3(256 * 16), dim3(256), 0, as_stream(stream),
+                     static_cast<const uint4*>(src), num_bytes / 16, static_cast<uint32_t*>(sink));
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_stream_copy(const void* src, void* dst, int64_t num_bytes, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(src && dst && num_bytes >= 0 && num_bytes % 16 == 0) << "stream_copy: bad arguments";
+  if (num_bytes == 0) return TVMKV_OK;
+  hipLaunchKernelGGL(stream_copy_kernel, dim3(256 * 16), dim3(256), 0, as_stream(stream),
+                     static_cast<const uint4*>(src), static_cast<uint4*>(dst), num_bytes / 16);
   KV_LAUNCH_CHECK();
   KV_API_END();
 }

@@ -153,3 +153,13 @@ def compact_kv_copy(pages, copy_length_indptr, copy_src_dst_pos, batch_size):
     num_pages, _, hkv, ps, d = pages.shape
     check(lib().tvmkv_compact_kv_copy(_p(pages), _p(copy_length_indptr), _p(copy_src_dst_pos), batch_size,
                                       copy_src_dst_pos.shape[1], num_pages, hkv, ps, d, _stream()))
+
+
+def stream_read(src, sink):
+    """Plain streaming read of the whole tensor (bandwidth calibration)."""
+    check(lib().tvmkv_stream_read(_p(src), src.numel() * src.element_size(), _p(sink), _stream()))
+
+
+def stream_copy(src, dst):
+    """Plain copy of the whole tensor (bandwidth calibration, counter scaling)."""
+    check(lib().tvmkv_stream_copy(_p(src), _p(dst), src.numel() * src.element_size(), _stream()))
