@@ -55,7 +55,7 @@ __device__ __forceinline__ int tile_slot_begin(const int32_t* q_indptr, int b, i
 }
 
 template <int DQK, int DV, bool PAGED, int PS>
-__global__ __launch_bounds__(256) void prefill_kernel(PrefillParams p) {
+__global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   static_assert(DQK % 16 == 0 && DV % 32 == 0, "feature dims must fit the MFMA tiles");
   constexpr int KS = DQK / 16;                  // k-steps of the QK^T product
   constexpr int DB = DV / 32;                   // 32-wide output feature blocks
@@ -70,19 +70,22 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillParams p) {
   static_assert(BN * KCH % 256 == 0, "K tile must divide evenly over the workgroup");
   static_assert(!PAGED || PS % 4 == 0, "page size must be a multiple of 4");
 
-  __shared__ __attribute__((aligned(16))) half_t Ks[BN * KROW];
-  __shared__ __attribute__((aligned(16))) half_t Vt[DV * VROW];
+  // two LDS buffers: tile t+1 is stored while the other waves still read tile t, one barrier per tile
+  __shared__ __attribute__((aligned(16))) half_t Ks_buf[2][BN * KROW];
+  __shared__ __attribute__((aligned(16))) half_t Vt_buf[2][DV * VROW];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
   const int col = lane & 31;
   const int half = lane >> 5;
-  const int kvh = blockIdx.y;
+  // grid = (h_kv, slots): the kv head is the fastest-varying workgroup index, so with 8 kv heads
+  // and 8 XCDs (workgroups are dealt round-robin to XCDs) all row tiles of one head share one L2
+  const int kvh = blockIdx.x;
   const int group = p.group;
 
   // ---- which (sequence, row tile) ---------------------------------------------------------
-  const int slot = blockIdx.x;
+  const int slot = blockIdx.y;
   int b;
   {
     int lo = 0, hi = p.batch_size - 1;
@@ -99,8 +102,12 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillParams p) {
   const int q_start = p.q_indptr[b];
   const int qo_len = p.q_indptr[b + 1] - q_start;
   const int rows = qo_len * group;
-  const int r0 = (slot - tile_slot_begin(p.q_indptr, b, group)) * BM;
-  if (r0 >= rows) return;
+  // tiles of a sequence are handed out last-first: under the causal mask the last rows see the
+  // most keys, and the longest workgroups should start first
+  const int local_slot = slot - tile_slot_begin(p.q_indptr, b, group);
+  const int n_row_tiles = (rows + BM - 1) / BM;
+  if (local_slot >= n_row_tiles) return;
+  const int r0 = (n_row_tiles - 1 - local_slot) * BM;
 
   int kv_len, kv_start = 0, pbeg = 0;
   if (PAGED) {
@@ -192,7 +199,7 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillParams p) {
       }
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](half_t* Ks, half_t* Vt) {
 #pragma unroll
     for (int r = 0; r < KLOADS; ++r) {
       const int c = r * 256 + tid;
@@ -224,81 +231,85 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillParams p) {
   if (n_tiles > 0) load_tile(0);
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int kv0 = tile * BN;
-    __syncthreads();  // everyone is done reading the previous tile
-    store_tile();
+    half_t* Ks = Ks_buf[tile & 1];
+    half_t* Vt = Vt_buf[tile & 1];
+    // buffer (tile & 1) was last read during tile-2; every wave passed the barrier of tile-1 since
+    store_tile(Ks, Vt);
     __syncthreads();
     if (tile + 1 < n_tiles) load_tile(kv0 + BN);
 
     if (kv0 < wave_limit_max) {  // wave-uniform: otherwise every row of this wave is masked out
-      // ---- S^T = K Q^T ----------------------------------------------------------------------
-      float16_t acc[TB];
+      // The 64-token tile is consumed as TB sub-tiles of 32 tokens.  Per sub-tile the LDS reads are
+      // issued in two batches well ahead of their MFMAs (the compiler otherwise serialises one
+      // read per MFMA and exposes the LDS latency 32 times per tile): K fragments first, then the
+      // V^T fragments, whose latency hides behind the softmax arithmetic.
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb) {
+        const int t0 = kv0 + tb * 32;
+        if (t0 >= wave_limit_max) break;  // wave-uniform
+        half8_t kf[KS];
+        {
+          const half_t* krow = Ks + (tb * 32 + col) * KROW + half * 8;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) acc[tb][j] = 0.f;
-        const half_t* krow = Ks + (tb * 32 + col) * KROW + half * 8;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const half8_t a = ld16(krow + ks * 16).h8;
-          acc[tb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], acc[tb], 0, 0, 0);
+          for (int ks = 0; ks < KS; ++ks) kf[ks] = ld16(krow + ks * 16).h8;
         }
-      }
-      // ---- scale, mask, online softmax (lane-local per query) -------------------------------
-      const bool need_mask = kv0 + BN > wave_limit_min;
-      float mx = kNegInit;
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- S^T = K Q^T --------------------------------------------------------------------
+        float16_t acc;
 #pragma unroll
-      for (int tb = 0; tb < TB; ++tb) {
+        for (int j = 0; j < 16; ++j) acc[j] = 0.f;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          float s = acc[tb][j] * p.scale_log2;
-          if (need_mask) {
-            const int t = kv0 + tb * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
-            s = t < my_limit ? s : kNegInit;
-          }
-          acc[tb][j] = s;
-          mx = fmaxf(mx, s);
-        }
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m, mx);
-      const float alpha = fast_exp2(m - m_new);
-      m = m_new;
-      lsum *= alpha;
+        for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], acc, 0, 0, 0);
+        // ---- V^T fragments: contraction slot half*8+i holds token kk*16 + (i/4)*8 + half*4 + i%4
+        half8_t vf[DB][2];
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-#pragma unroll
-        for (int j = 0; j < 16; ++j) o[db][j] *= alpha;
-      }
-      half8_t pf[TB][2];
-#pragma unroll
-      for (int tb = 0; tb < TB; ++tb) {
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          float pj = fast_exp2(acc[tb][j] - m_new);
-          if (need_mask) {
-            const int t = kv0 + tb * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
-            pj = t < my_limit ? pj : 0.f;
-          }
-          lsum += pj;
-          pf[tb][j >> 3][j & 7] = static_cast<half_t>(pj);
-        }
-      }
-      // ---- O^T += V^T P^T -------------------------------------------------------------------
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const half_t* vrow = Vt + (db * 32 + col) * VROW + half * 4;
-#pragma unroll
-        for (int tb = 0; tb < TB; ++tb) {
+        for (int db = 0; db < DB; ++db) {
+          const half_t* vrow = Vt + (db * 32 + col) * VROW + half * 4 + tb * 32;
 #pragma unroll
           for (int kk = 0; kk < 2; ++kk) {
-            // contraction slot half*8+i holds token tb*32 + kk*16 + (i/4)*8 + half*4 + i%4
-            const half4_t lo = *reinterpret_cast<const half4_t*>(vrow + tb * 32 + kk * 16);
-            const half4_t hi = *reinterpret_cast<const half4_t*>(vrow + tb * 32 + kk * 16 + 8);
-            half8_t a;
-            a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
-            a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
-            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[tb][kk], o[db], 0, 0, 0);
+            const half4_t lo = *reinterpret_cast<const half4_t*>(vrow + kk * 16);
+            const half4_t hi = *reinterpret_cast<const half4_t*>(vrow + kk * 16 + 8);
+            vf[db][kk][0] = lo[0]; vf[db][kk][1] = lo[1]; vf[db][kk][2] = lo[2]; vf[db][kk][3] = lo[3];
+            vf[db][kk][4] = hi[0]; vf[db][kk][5] = hi[1]; vf[db][kk][6] = hi[2]; vf[db][kk][7] = hi[3];
           }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- mask, online softmax (lane-local per query); the scale is folded into the exponent:
+        // p = exp2(acc*scale - m)
+        if (t0 + 32 > wave_limit_min) {  // wave-uniform; only tiles on the diagonal or at the tail
+          asm volatile("" ::: "memory");  // keep this a branch: if-converted it costs 5 ops per element everywhere
+          const int rel = my_limit - t0 - half * 4;  // element j is token t0 + half*4 + (j/4)*8 + j%4
+#pragma unroll
+          for (int j = 0; j < 16; ++j) acc[j] = ((j >> 2) * 8 + (j & 3)) < rel ? acc[j] : -3.0e38f;
+        }
+        float mx_raw = -3.0e38f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) mx_raw = fmaxf(mx_raw, acc[j]);
+        mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 32, 64));
+        // a fully masked row keeps its old maximum (the scaled sentinel is far below -5e4)
+        const float m_new = fmaxf(m, fmaxf(mx_raw * p.scale_log2, -1.0e30f));
+        const float alpha = fast_exp2(m - m_new);
+        m = m_new;
+        lsum *= alpha;
+        if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {  // wave-uniform: skip when no maximum moved
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) o[db][j] *= alpha;
+          }
+        }
+        half8_t pf[2];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const float pj = fast_exp2(fmaf(acc[j], p.scale_log2, -m_new));  // masked: exp2(-3e38*scale - m) = 0
+          lsum += pj;
+          pf[j >> 3][j & 7] = static_cast<half_t>(pj);
+        }
+        // ---- O^T += V^T P^T -----------------------------------------------------------------
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[db][kk], pf[kk], o[db], 0, 0, 0);
         }
       }
     }
@@ -327,8 +338,8 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillParams p) {
 template <int DQK, int DV, bool PAGED, int PS>
 static void launch_prefill(const PrefillParams& p, int64_t total_q, hipStream_t stream) {
   const int64_t slots = total_q * p.group / BM + p.batch_size;
-  if (slots >= (int64_t{1} << 31)) throw Error(TVMKV_EINVAL, "prefill: too many row tiles");
-  hipLaunchKernelGGL((prefill_kernel<DQK, DV, PAGED, PS>), dim3(static_cast<unsigned>(slots), p.h_kv), dim3(256), 0,
+  if (slots >= 65536) throw Error(TVMKV_EINVAL, "prefill: too many row tiles for one launch (65535 x 128 rows)");
+  hipLaunchKernelGGL((prefill_kernel<DQK, DV, PAGED, PS>), dim3(p.h_kv, static_cast<unsigned>(slots)), dim3(256), 0,
                      stream, p);
 }
 
