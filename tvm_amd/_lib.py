@@ -4,7 +4,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libtvmkv.so")
+# TVMKV_LIB_PATH points the loader at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("TVMKV_LIB_PATH") or os.path.join(_HERE, "lib", "libtvmkv.so")
 
 c_i32, c_i64, c_f64, c_vp = ctypes.c_int32, ctypes.c_int64, ctypes.c_double, ctypes.c_void_p
 p_i32, p_i64 = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64)

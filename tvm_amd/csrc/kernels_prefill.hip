@@ -11,12 +11,17 @@
 // (_kernel_common.py:130-135).
 //
 // Tiling: a workgroup of 4 wavefronts owns 128 rows x one kv head; each wave owns 32 rows, one
-// row per lane%32, and keeps Q as MFMA B-fragments in registers.  K/V tiles of 64 tokens go
-// through LDS (K row-major, V transposed so that the token axis is contiguous); the next tile's
-// global loads are issued before the current tile's math.  S^T = K Q^T and O^T = V^T P^T use
-// v_mfma_f32_32x32x16_f16 with the query on the N axis: all per-query softmax state (m, l, the
-// O rescale factor) is lane-local, and the S^T accumulator registers are exactly the B-operand
-// of the PV product, so P never leaves registers.
+// row per lane%32, and keeps Q as MFMA B-fragments in registers.  K/V tiles of 64 tokens are
+// copied from global memory straight into LDS (global_load_lds_dwordx4: no staging registers, no
+// ds_write), row-major and unpadded, two stages deep, so that tile t+1 lands while tile t is
+// multiplied.  Bank conflicts are avoided by an XOR swizzle of the 16-byte pieces of a row; the
+// copy applies it on the source side (lane L always fills LDS piece L of the 1 KiB an
+// instruction writes, and fetches the global piece that belongs there).  S^T = K Q^T and
+// O^T = V^T P^T use v_mfma_f32_32x32x16_f16 with the query on the N axis: all per-query softmax
+// state (m, l, the O rescale factor) is lane-local, and the S^T accumulator registers are exactly
+// the B-operand of the PV product, so P never leaves registers.  The V^T A-fragments come from
+// the row-major V tile through ds_read_b64_tr_b16, which hands each lane four consecutive tokens
+// of one feature.
 //
 // Workgroup -> (sequence, row tile) without a prologue kernel: sequence b owns tile slots
 //   [floor(q_indptr[b]*group/128) + b, floor(q_indptr[b+1]*group/128) + b + 1)
@@ -27,8 +32,38 @@ namespace tvmkv {
 
 constexpr int BM = 128;  // rows per workgroup
 constexpr int BN = 64;   // kv tokens per tile
-constexpr int KPAD = 8;  // halfs of padding per K row in LDS
-constexpr int VPAD = 4;  // halfs of padding per V^T row in LDS
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// One global_load_lds_dwordx4: lane L copies the 16 bytes at its own global address to LDS address
+// lds_addr + 16*L (lds_addr must be the same in every lane).  The copy is asynchronous and counted
+// by vmcnt.  It is issued from inline assembly on purpose: when the compiler knows of a copy in
+// flight it puts s_waitcnt vmcnt(0) in front of the next LDS read it cannot tell apart from the
+// copy's destination, which would serialise the two-stage pipeline; here the one wait per tile is
+// written by hand in front of the workgroup barrier.  The compiler sets M0 itself right before
+// each of its own uses, so the asm does not have to restore it.
+// src_base (the same in every lane) + byte_off (per lane, unsigned 32 bit) is the global address.
+__device__ __forceinline__ void copy16_to_lds(const void* src_base, uint32_t byte_off, uint32_t lds_addr) {
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               ::"v"(byte_off), "s"(src_base), "s"(lds_addr) : "memory");
+}
+
+// Tells the compiler that a pointer holds the same value in every lane.
+__device__ __forceinline__ const half_t* uniform_ptr(const half_t* p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+  return reinterpret_cast<const half_t*>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) short4_t* lds_short4_ptr_t;
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane l receives element l%4 of the four
+// 8-byte rows addressed by lanes l/4, 4 + l/4, 8 + l/4 and 12 + l/4 of the group.
+__device__ __forceinline__ half4_t lds_read_tr16(const half_t* p) {
+  return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr_t)p));
+}
 
 struct PrefillParams {
   const half_t* q;
@@ -54,25 +89,48 @@ __device__ __forceinline__ int tile_slot_begin(const int32_t* q_indptr, int b, i
   return static_cast<int>((static_cast<int64_t>(q_indptr[b]) * group) / BM) + b;
 }
 
+// LDS image of a tile of BN token rows x W features (W = 64 or 128), pieces of 8 features.
+// Piece c of row r is kept at piece position c ^ swz(r).
+//  * K is read as MFMA A-fragments with ds_read_b128, 16 lanes = 16 consecutive rows at the same
+//    piece: swz spreads 16 consecutive rows over the 16 piece positions of a 256-byte bank line.
+//  * V is read with ds_read_b64_tr_b16, 32 lanes = 4 consecutive rows x 64 bytes: swz moves the 4
+//    rows to the 4 different 64-byte quarters of the bank line.
+template <int W>
+__device__ __forceinline__ int k_swizzle(int row) {
+  return W == 128 ? (row & 15) : ((row >> 1) & 7);
+}
+template <int W>
+__device__ __forceinline__ int v_swizzle(int row) {
+  return W == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
+}
+
+// Scheduling hint for the region it is placed in: N groups of (1 MFMA, then a few vector ALU ops).
+template <int N>
+__device__ __forceinline__ void interleave_mfma_valu() {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+    __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);  // VALU
+  }
+}
+
 template <int DQK, int DV, bool PAGED, int PS>
 __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
-  static_assert(DQK % 16 == 0 && DV % 32 == 0, "feature dims must fit the MFMA tiles");
+  static_assert(DQK % 64 == 0 && DV % 64 == 0, "feature dims must be multiples of 64");
   constexpr int KS = DQK / 16;                  // k-steps of the QK^T product
   constexpr int DB = DV / 32;                   // 32-wide output feature blocks
   constexpr int TB = BN / 32;                   // 32-token blocks per tile
-  constexpr int KROW = DQK + KPAD;              // LDS row stride of K (halfs)
-  constexpr int VROW = BN + VPAD;               // LDS row stride of V^T (halfs)
-  constexpr int KCH = DQK / 8;                  // 16-byte pieces per K row
-  constexpr int KLOADS = BN * KCH / 256;        // K pieces per thread per tile
-  constexpr int VCH = DV / 8;                   // 16-byte pieces per V row
-  constexpr int VUNITS = (BN / 4) * VCH;        // (4 tokens x 8 features) units per tile
-  constexpr int VT = (VUNITS + 255) / 256;      // units per thread
-  static_assert(BN * KCH % 256 == 0, "K tile must divide evenly over the workgroup");
-  static_assert(!PAGED || PS % 4 == 0, "page size must be a multiple of 4");
+  constexpr int KW = DQK % 128 == 0 ? 128 : 64; // K is kept as DQK/KW column blocks of width KW
+  constexpr int KBLK = DQK / KW;
+  constexpr int KCH = KW / 8;                   // 16-byte pieces per row of a K block
+  constexpr int VW = DV % 128 == 0 ? 128 : 64;
+  constexpr int VBLK = DV / VW;
+  constexpr int VCH = VW / 8;
+  constexpr int STAGE = BN * (DQK + DV);        // halfs per pipeline stage
+  static_assert(!PAGED || PS % 16 == 0, "page size must be a multiple of 16");
 
-  // two LDS buffers: tile t+1 is stored while the other waves still read tile t, one barrier per tile
-  __shared__ __attribute__((aligned(16))) half_t Ks_buf[2][BN * KROW];
-  __shared__ __attribute__((aligned(16))) half_t Vt_buf[2][DV * VROW];
+  // two stages; the workgroup's 4 waves each copy 16 of the 64 token rows of a tile
+  extern __shared__ __attribute__((aligned(16))) half_t lds_tiles[];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -151,167 +209,226 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   }
   float m = kNegInit, lsum = 0.f;
 
-  // ---- tile loaders ----------------------------------------------------------------------
-  Vec16 kreg[KLOADS];
-  Vec16 vreg[VT][4];
-  auto load_tile = [&](int kv0) {
+  // ---- tile copy: global -> LDS ---------------------------------------------------------------
+  // Rows past the end of the sequence repeat its last token: their scores are masked, and P = 0
+  // times a finite V is 0 (unwritten page memory could hold NaN patterns).
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds_tiles));
+  const int last_tok = kv_len - 1;
+  // Page holding this wave's 16 rows of the tile at kv0.  The value is the same in every lane but
+  // is deliberately computed per lane: a wave-uniform load would be moved to a scalar register
+  // right away, and that wait would also wait for the tile copy issued just before it.
+  auto page_of = [&](int kv0) -> int {
+    if (!PAGED) return 0;
+    const int pslot = min(kv0 + wave * 16, last_tok) / PS;
+    return p.page_values[pbeg + pslot];
+  };
+  // Global addresses are a wave-uniform base (scalar registers) plus a 32-bit byte offset per lane.
+  // Ragged: the base is the sequence's first K/V row of this head, the offset token * row stride,
+  // so one sequence's K (or V) must stay below 4 GiB.  Paged: the base is the page, the offset the
+  // row inside it.
+  const half_t* k_seq = PAGED ? nullptr : uniform_ptr(p.k + (static_cast<int64_t>(kv_start) * p.h_kv + kvh) * DQK);
+  const half_t* v_seq = PAGED ? nullptr : uniform_ptr(p.v + (static_cast<int64_t>(kv_start) * p.h_kv + kvh) * DV);
+  const uint32_t k_stride_bytes = static_cast<uint32_t>(p.h_kv) * DQK * 2;
+  const uint32_t v_stride_bytes = static_cast<uint32_t>(p.h_kv) * DV * 2;
+  auto issue_tile = [&](int kv0, int page_v, int stage_index) {
+    const uint32_t stage = lds_base + stage_index * (STAGE * 2);  // LDS byte address
+    const half_t* kbase = k_seq;
+    const half_t* vbase = v_seq;
+    if (PAGED) {
+      const int page = __builtin_amdgcn_readfirstlane(page_v);
+      kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * (PS * DQK);
+      vbase = kbase + static_cast<int64_t>(p.h_kv) * (PS * DQK);
+    }
 #pragma unroll
-    for (int r = 0; r < KLOADS; ++r) {
-      const int c = r * 256 + tid;
-      const int row = c / KCH;
-      const int piece = c % KCH;
-      const int t = kv0 + row;
-      if (t < kv_len) {
-        const half_t* src;
-        if (PAGED) {
-          const int page = p.page_values[pbeg + t / PS];
-          src = p.pages + ((static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * PS + t % PS) * DQK + piece * 8;
-        } else {
-          src = p.k + (static_cast<int64_t>(kv_start + t) * p.h_kv + kvh) * DQK + piece * 8;
-        }
-        kreg[r] = ld16(src);
-      } else {
-        kreg[r] = zero16();
+    for (int blk = 0; blk < KBLK; ++blk) {
+      constexpr int RPI = 64 / KCH;  // rows per instruction
+#pragma unroll
+      for (int i = 0; i < 16 / RPI; ++i) {
+        const int row = wave_u * 16 + i * RPI + lane / KCH;
+        const int piece = (lane % KCH) ^ k_swizzle<KW>(row);
+        const uint32_t t = min(kv0 + row, last_tok);
+        const uint32_t off = (PAGED ? (t % PS) * (DQK * 2) : __umul24(t, k_stride_bytes)) + (blk * KW + piece * 8) * 2;
+        copy16_to_lds(kbase, off, stage + (blk * (BN * KW) + (wave_u * 16 + i * RPI) * KW) * 2);
       }
     }
 #pragma unroll
-    for (int u = 0; u < VT; ++u) {
-      const int idx = u * 256 + tid;
-      const int dchunk = idx % VCH;
-      const int tgroup = idx / VCH;
-      const int t0 = kv0 + tgroup * 4;
-      const half_t* src = nullptr;
-      int64_t tok_stride = 0;
-      if (idx < VUNITS && t0 < kv_len) {
-        if (PAGED) {
-          const int page = p.page_values[pbeg + t0 / PS];
-          src = p.pages + ((static_cast<int64_t>(page) * 2 + 1) * p.h_kv + kvh) * (static_cast<int64_t>(PS) * DV) +
-                (t0 % PS) * DV + dchunk * 8;
-          tok_stride = DV;
-        } else {
-          src = p.v + (static_cast<int64_t>(kv_start + t0) * p.h_kv + kvh) * DV + dchunk * 8;
-          tok_stride = static_cast<int64_t>(p.h_kv) * DV;
-        }
-      }
+    for (int blk = 0; blk < VBLK; ++blk) {
+      constexpr int RPI = 64 / VCH;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        vreg[u][r] = (src != nullptr && t0 + r < kv_len) ? ld16(src + r * tok_stride) : zero16();
+      for (int i = 0; i < 16 / RPI; ++i) {
+        const int row = wave_u * 16 + i * RPI + lane / VCH;
+        const int piece = (lane % VCH) ^ v_swizzle<VW>(row);
+        const uint32_t t = min(kv0 + row, last_tok);
+        const uint32_t off = (PAGED ? (t % PS) * (DV * 2) : __umul24(t, v_stride_bytes)) + (blk * VW + piece * 8) * 2;
+        copy16_to_lds(vbase, off, stage + (BN * DQK + blk * (BN * VW) + (wave_u * 16 + i * RPI) * VW) * 2);
       }
     }
   };
-  auto store_tile = [&](half_t* Ks, half_t* Vt) {
+
+  // ---- per-lane fragment addressing (halfs, relative to the K / V part of a stage) -----------
+  // K A-fragment of k-step ks, token block tb: row tb*32 + col, features ks*16 + half*8 .. +7
+  const int k_swz = k_swizzle<KW>(col);  // same for col + 32
+  // V^T A-fragment via the transposing read: lane li of a 16-lane group points at 4 features of
+  // token (li >> 2) of the group's 4 tokens; the group as a whole covers 16 features, and lane li
+  // receives feature li of them for the 4 tokens.
+  const int li = lane & 15;
+  const int gg = (lane >> 4) & 1;
+  const int v_row = half * 4 + (li >> 2);           // + tb*32 + kk*16 + {0, 8}
+  const int v_swz = v_swizzle<VW>(v_row);           // the added terms are multiples of 8
+  const int v_lane_off = v_row * VW + (li & 1) * 4; // halfs
+
+  auto read_k = [&](const half_t* Ks, int tb, half8_t (&kf)[KS]) {
 #pragma unroll
-    for (int r = 0; r < KLOADS; ++r) {
-      const int c = r * 256 + tid;
-      st16(Ks + (c / KCH) * KROW + (c % KCH) * 8, kreg[r]);
+    for (int ks = 0; ks < KS; ++ks) {
+      constexpr int SPB = KW / 16;  // k-steps per column block
+      const int piece = ((ks % SPB) * 2 + half) ^ k_swz;
+      kf[ks] = *reinterpret_cast<const half8_t*>(Ks + (ks / SPB) * (BN * KW) + (tb * 32 + col) * KW + piece * 8);
     }
+  };
+  // contraction slot half*8+i of fragment kk holds token kk*16 + (i/4)*8 + half*4 + i%4 of the block,
+  // the order in which the S^T accumulator registers hold the tokens
+  auto read_v = [&](const half_t* Vs, int tb, half8_t (&vf)[DB][2]) {
 #pragma unroll
-    for (int u = 0; u < VT; ++u) {
-      const int idx = u * 256 + tid;
-      if (idx < VUNITS) {
-        const int dchunk = idx % VCH;
-        const int tgroup = idx / VCH;
+    for (int db = 0; db < DB; ++db) {
+      constexpr int BPB = VW / 32;  // feature blocks per column block
+      const int piece = (((db % BPB) * 4 + gg * 2 + ((li & 3) >> 1)) ^ v_swz);
+      const half_t* vp = Vs + (db / BPB) * (BN * VW) + v_lane_off + piece * 8 + tb * 32 * VW;
 #pragma unroll
-        for (int e2 = 0; e2 < 4; ++e2) {
-          // words e2 of the four token rows hold features (2*e2, 2*e2+1)
-          const uint32_t w0 = vreg[u][0].w[e2], w1 = vreg[u][1].w[e2], w2 = vreg[u][2].w[e2], w3 = vreg[u][3].w[e2];
-          uint2 even, odd;  // 4 tokens of feature 2*e2 / 2*e2+1
-          even.x = (w0 & 0xffffu) | (w1 << 16);
-          even.y = (w2 & 0xffffu) | (w3 << 16);
-          odd.x = (w0 >> 16) | (w1 & 0xffff0000u);
-          odd.y = (w2 >> 16) | (w3 & 0xffff0000u);
-          *reinterpret_cast<uint2*>(Vt + (dchunk * 8 + 2 * e2) * VROW + tgroup * 4) = even;
-          *reinterpret_cast<uint2*>(Vt + (dchunk * 8 + 2 * e2 + 1) * VROW + tgroup * 4) = odd;
-        }
+      for (int kk = 0; kk < 2; ++kk) {
+        const half4_t lo = lds_read_tr16(vp + (kk * 16) * VW);
+        const half4_t hi = lds_read_tr16(vp + (kk * 16 + 8) * VW);
+        vf[db][kk][0] = lo[0]; vf[db][kk][1] = lo[1]; vf[db][kk][2] = lo[2]; vf[db][kk][3] = lo[3];
+        vf[db][kk][4] = hi[0]; vf[db][kk][5] = hi[1]; vf[db][kk][6] = hi[2]; vf[db][kk][7] = hi[3];
       }
+    }
+  };
+  // S^T = K Q^T for one 32-token block
+  auto qk = [&](const half8_t (&kf)[KS]) -> float16_t {
+    float16_t acc;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], acc, 0, 0, 0);
+    return acc;
+  };
+  // online softmax, lane-local per query; the scale is folded into the exponent: p = exp2(s*scale - m)
+  auto row_max = [&](const float16_t& acc) -> float {
+    float mx = -3.0e38f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) mx = fmaxf(mx, acc[j]);
+    return fmaxf(mx, __shfl_xor(mx, 32, 64));
+  };
+  auto advance_max = [&](float mx_raw) -> float {  // returns the factor that rescales the old state
+    // a fully masked row keeps its old maximum (the scaled sentinel is far below -5e4)
+    const float m_new = fmaxf(m, fmaxf(mx_raw * p.scale_log2, -1.0e30f));
+    const float alpha = fast_exp2(m - m_new);
+    m = m_new;
+    lsum *= alpha;
+    return alpha;
+  };
+  auto rescale = [&](float alpha) {
+    if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {  // wave-uniform: skip when no maximum moved
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) o[db][j] *= alpha;
+      }
+    }
+  };
+  auto probs = [&](const float16_t& acc, half8_t (&pf)[2]) {  // uses the current m
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float pj = fast_exp2(fmaf(acc[j], p.scale_log2, -m));  // masked: exp2(-3e38*scale - m) = 0
+      lsum += pj;
+      pf[j >> 3][j & 7] = static_cast<half_t>(pj);
+    }
+  };
+  // O^T += V^T P^T for one 32-token block
+  auto pv = [&](const half8_t (&vf)[DB][2], const half8_t (&pf)[2]) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[db][kk], pf[kk], o[db], 0, 0, 0);
     }
   };
 
   const int n_tiles = (kv_end + BN - 1) / BN;
-  if (n_tiles > 0) load_tile(0);
+  int page_next = 0;
+  if (n_tiles > 0) {
+    issue_tile(0, page_of(0), 0);
+    if (n_tiles > 1) page_next = page_of(BN);
+  }
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int kv0 = tile * BN;
-    half_t* Ks = Ks_buf[tile & 1];
-    half_t* Vt = Vt_buf[tile & 1];
-    // buffer (tile & 1) was last read during tile-2; every wave passed the barrier of tile-1 since
-    store_tile(Ks, Vt);
+    const half_t* Ks = lds_tiles + (tile & 1) * STAGE;
+    const half_t* Vs = Ks + BN * DQK;
+    // this wave's part of the tile has landed; after the barrier everyone's has, and every wave
+    // is done reading the other stage (tile-1), which the next copy overwrites
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
-    if (tile + 1 < n_tiles) load_tile(kv0 + BN);
+    if (tile + 1 < n_tiles) {
+      issue_tile(kv0 + BN, page_next, (tile + 1) & 1);
+      if (tile + 2 < n_tiles) page_next = page_of(kv0 + 2 * BN);
+    }
 
-    if (kv0 < wave_limit_max) {  // wave-uniform: otherwise every row of this wave is masked out
-      // The 64-token tile is consumed as TB sub-tiles of 32 tokens.  Per sub-tile the LDS reads are
-      // issued in two batches well ahead of their MFMAs (the compiler otherwise serialises one
-      // read per MFMA and exposes the LDS latency 32 times per tile): K fragments first, then the
-      // V^T fragments, whose latency hides behind the softmax arithmetic.
+    if (kv0 >= wave_limit_max) continue;  // wave-uniform: every row of this wave is masked out
+
+    if (TB == 2 && kv0 + BN <= wave_limit_min) {
+      // Every row of the wave sees the whole tile (all tiles left of the causal diagonal): no
+      // masking, and the two 32-token halves are software-pipelined so that the wave's own matrix
+      // and vector work overlap: S1 = K1 Q^T runs under the softmax of S0, and O += V0 P0 under the
+      // softmax of S1.
+      half8_t kf[KS];
+      half8_t vf[DB][2];
+      half8_t pf[2];
+      read_k(Ks, 0, kf);
+      __builtin_amdgcn_sched_barrier(0);
+      float16_t s0 = qk(kf);
+      read_k(Ks, 1, kf);
+      read_v(Vs, 0, vf);
+      const float a0 = advance_max(row_max(s0));
+      rescale(a0);
+      __builtin_amdgcn_sched_barrier(0);
+      float16_t s1 = qk(kf);
+      probs(s0, pf);
+      interleave_mfma_valu<KS>();
+      __builtin_amdgcn_sched_barrier(0);
+      const float a1 = advance_max(row_max(s1));
+      pv(vf, pf);
+      probs(s1, pf);
+      interleave_mfma_valu<2 * DB>();
+      __builtin_amdgcn_sched_barrier(0);
+      read_v(Vs, 1, vf);
+      rescale(a1);
+      pv(vf, pf);
+      continue;
+    }
+
+    // Tiles on the causal diagonal or at the end of the sequence: one 32-token block at a time,
+    // masked.  The LDS reads of a block are issued in two batches ahead of their MFMAs (K
+    // fragments, then the V^T fragments, whose latency hides behind the softmax arithmetic).
 #pragma unroll
-      for (int tb = 0; tb < TB; ++tb) {
-        const int t0 = kv0 + tb * 32;
-        if (t0 >= wave_limit_max) break;  // wave-uniform
-        half8_t kf[KS];
-        {
-          const half_t* krow = Ks + (tb * 32 + col) * KROW + half * 8;
+    for (int tb = 0; tb < TB; ++tb) {
+      const int t0 = kv0 + tb * 32;
+      if (t0 >= wave_limit_max) break;  // wave-uniform
+      half8_t kf[KS];
+      half8_t vf[DB][2];
+      half8_t pf[2];
+      read_k(Ks, tb, kf);
+      __builtin_amdgcn_sched_barrier(0);
+      float16_t acc = qk(kf);
+      read_v(Vs, tb, vf);
+      __builtin_amdgcn_sched_barrier(0);
+      if (t0 + 32 > wave_limit_min) {  // wave-uniform
+        asm volatile("" ::: "memory");  // keep this a branch: if-converted it costs 5 ops per element everywhere
+        const int rel = my_limit - t0 - half * 4;  // element j is token t0 + half*4 + (j/4)*8 + j%4
 #pragma unroll
-          for (int ks = 0; ks < KS; ++ks) kf[ks] = ld16(krow + ks * 16).h8;
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- S^T = K Q^T --------------------------------------------------------------------
-        float16_t acc;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) acc[j] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], acc, 0, 0, 0);
-        // ---- V^T fragments: contraction slot half*8+i holds token kk*16 + (i/4)*8 + half*4 + i%4
-        half8_t vf[DB][2];
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const half_t* vrow = Vt + (db * 32 + col) * VROW + half * 4 + tb * 32;
-#pragma unroll
-          for (int kk = 0; kk < 2; ++kk) {
-            const half4_t lo = *reinterpret_cast<const half4_t*>(vrow + kk * 16);
-            const half4_t hi = *reinterpret_cast<const half4_t*>(vrow + kk * 16 + 8);
-            vf[db][kk][0] = lo[0]; vf[db][kk][1] = lo[1]; vf[db][kk][2] = lo[2]; vf[db][kk][3] = lo[3];
-            vf[db][kk][4] = hi[0]; vf[db][kk][5] = hi[1]; vf[db][kk][6] = hi[2]; vf[db][kk][7] = hi[3];
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- mask, online softmax (lane-local per query); the scale is folded into the exponent:
-        // p = exp2(acc*scale - m)
-        if (t0 + 32 > wave_limit_min) {  // wave-uniform; only tiles on the diagonal or at the tail
-          asm volatile("" ::: "memory");  // keep this a branch: if-converted it costs 5 ops per element everywhere
-          const int rel = my_limit - t0 - half * 4;  // element j is token t0 + half*4 + (j/4)*8 + j%4
-#pragma unroll
-          for (int j = 0; j < 16; ++j) acc[j] = ((j >> 2) * 8 + (j & 3)) < rel ? acc[j] : -3.0e38f;
-        }
-        float mx_raw = -3.0e38f;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) mx_raw = fmaxf(mx_raw, acc[j]);
-        mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 32, 64));
-        // a fully masked row keeps its old maximum (the scaled sentinel is far below -5e4)
-        const float m_new = fmaxf(m, fmaxf(mx_raw * p.scale_log2, -1.0e30f));
-        const float alpha = fast_exp2(m - m_new);
-        m = m_new;
-        lsum *= alpha;
-        if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {  // wave-uniform: skip when no maximum moved
-#pragma unroll
-          for (int db = 0; db < DB; ++db) {
-#pragma unroll
-            for (int j = 0; j < 16; ++j) o[db][j] *= alpha;
-          }
-        }
-        half8_t pf[2];
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const float pj = fast_exp2(fmaf(acc[j], p.scale_log2, -m_new));  // masked: exp2(-3e38*scale - m) = 0
-          lsum += pj;
-          pf[j >> 3][j & 7] = static_cast<half_t>(pj);
-        }
-        // ---- O^T += V^T P^T -----------------------------------------------------------------
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-#pragma unroll
-          for (int kk = 0; kk < 2; ++kk) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[db][kk], pf[kk], o[db], 0, 0, 0);
-        }
+        for (int j = 0; j < 16; ++j) acc[j] = ((j >> 2) * 8 + (j & 3)) < rel ? acc[j] : -3.0e38f;
       }
+      rescale(advance_max(row_max(acc)));
+      probs(acc, pf);
+      pv(vf, pf);
     }
   }
 
@@ -339,8 +456,15 @@ template <int DQK, int DV, bool PAGED, int PS>
 static void launch_prefill(const PrefillParams& p, int64_t total_q, hipStream_t stream) {
   const int64_t slots = total_q * p.group / BM + p.batch_size;
   if (slots >= 65536) throw Error(TVMKV_EINVAL, "prefill: too many row tiles for one launch (65535 x 128 rows)");
-  hipLaunchKernelGGL((prefill_kernel<DQK, DV, PAGED, PS>), dim3(p.h_kv, static_cast<unsigned>(slots)), dim3(256), 0,
-                     stream, p);
+  constexpr size_t lds_bytes = 2 * BN * (DQK + DV) * sizeof(half_t);
+  static bool attr_set = false;  // per instantiation; the attribute is per function, not per device
+  if (lds_bytes > 48 * 1024 && !attr_set) {
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, PAGED, PS>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((prefill_kernel<DQK, DV, PAGED, PS>), dim3(p.h_kv, static_cast<unsigned>(slots)), dim3(256),
+                     lds_bytes, stream, p);
 }
 
 }  // namespace tvmkv
