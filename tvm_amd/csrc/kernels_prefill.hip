@@ -26,11 +26,15 @@
 // Workgroup -> (sequence, row tile) without a prologue kernel: sequence b owns tile slots
 //   [floor(q_indptr[b]*group/128) + b, floor(q_indptr[b+1]*group/128) + b + 1)
 // found by binary search on q_indptr; the grid is floor(total_q*group/128) + B slots.
+#include <type_traits>
+
 #include "kernels_common.cuh"
 
 namespace tvmkv {
 
-constexpr int BM = 128;  // rows per workgroup
+constexpr int NW = 4;        // wavefronts per workgroup, 32 rows each
+constexpr int BM = NW * 32;  // rows per workgroup
+constexpr int RPW = 64 / NW; // token rows of a tile copied by each wave
 constexpr int BN = 64;   // kv tokens per tile
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -114,8 +118,25 @@ __device__ __forceinline__ void interleave_mfma_valu() {
   }
 }
 
+// Pipeline depth: as many stages as fit next to a second workgroup (NW = 4) or alone (NW = 8).
+constexpr int prefill_stages(int dqk, int dv) {
+  const int stage_bytes = BN * (dqk + dv) * 2;
+  const int budget = (NW == 8 ? 160 : 80) * 1024;
+  return budget / stage_bytes >= 4 ? 4 : (budget / stage_bytes >= 3 ? 3 : 2);
+}
+
+constexpr size_t prefill_lds_bytes(int dqk, int dv) {
+  return static_cast<size_t>(prefill_stages(dqk, dv)) * BN * (dqk + dv) * 2;
+}
+
+// s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters at their maximum)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
 template <int DQK, int DV, bool PAGED, int PS>
-__global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(PrefillParams p) {
   static_assert(DQK % 64 == 0 && DV % 64 == 0, "feature dims must be multiples of 64");
   constexpr int KS = DQK / 16;                  // k-steps of the QK^T product
   constexpr int DB = DV / 32;                   // 32-wide output feature blocks
@@ -127,6 +148,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   constexpr int VBLK = DV / VW;
   constexpr int VCH = VW / 8;
   constexpr int STAGE = BN * (DQK + DV);        // halfs per pipeline stage
+  constexpr int NSTAGE = prefill_stages(DQK, DV);
+  constexpr int COPIES = (DQK + DV) / 8 / NW;   // copy instructions per wave per tile
   static_assert(!PAGED || PS % 16 == 0, "page size must be a multiple of 16");
 
   // two stages; the workgroup's 4 waves each copy 16 of the 64 token rows of a tile
@@ -215,13 +238,14 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds_tiles));
   const int last_tok = kv_len - 1;
-  // Page holding this wave's 16 rows of the tile at kv0.  The value is the same in every lane but
-  // is deliberately computed per lane: a wave-uniform load would be moved to a scalar register
-  // right away, and that wait would also wait for the tile copy issued just before it.
-  auto page_of = [&](int kv0) -> int {
-    if (!PAGED) return 0;
-    const int pslot = min(kv0 + wave * 16, last_tok) / PS;
-    return p.page_values[pbeg + pslot];
+  // Page ids of this wave's RPW rows for 64 consecutive tiles, one tile per lane, fetched once per
+  // 64 tiles: the wait for this load also waits for every tile copy in flight, so it must be rare.
+  int page_ids = 0;
+  auto load_page_ids = [&](int first_tile) {
+    if (PAGED) {
+      const int pslot = min((first_tile + lane) * BN + wave_u * RPW, last_tok) / PS;
+      page_ids = p.page_values[pbeg + pslot];
+    }
   };
   // Global addresses are a wave-uniform base (scalar registers) plus a 32-bit byte offset per lane.
   // Ragged: the base is the sequence's first K/V row of this head, the offset token * row stride,
@@ -231,12 +255,19 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   const half_t* v_seq = PAGED ? nullptr : uniform_ptr(p.v + (static_cast<int64_t>(kv_start) * p.h_kv + kvh) * DV);
   const uint32_t k_stride_bytes = static_cast<uint32_t>(p.h_kv) * DQK * 2;
   const uint32_t v_stride_bytes = static_cast<uint32_t>(p.h_kv) * DV * 2;
-  auto issue_tile = [&](int kv0, int page_v, int stage_index) {
-    const uint32_t stage = lds_base + stage_index * (STAGE * 2);  // LDS byte address
+  // Issues copy instructions [FIRST, FIRST + COUNT) of the wave's COPIES for `tile` (K blocks first,
+  // then V), so that the caller can spread them over its arithmetic: a burst of all copies of all
+  // waves right after the barrier queues up in front of the one address unit of the CU, and the
+  // waves stall in issue instead of computing.
+  auto issue_copies = [&](int tile, auto first_c, auto count_c) {
+    constexpr int FIRST = decltype(first_c)::value;
+    constexpr int COUNT = decltype(count_c)::value;
+    const int kv0 = tile * BN;
+    const uint32_t stage = lds_base + (tile % NSTAGE) * (STAGE * 2);  // LDS byte address
     const half_t* kbase = k_seq;
     const half_t* vbase = v_seq;
     if (PAGED) {
-      const int page = __builtin_amdgcn_readfirstlane(page_v);
+      const int page = __builtin_amdgcn_readlane(page_ids, tile & 63);
       kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * (PS * DQK);
       vbase = kbase + static_cast<int64_t>(p.h_kv) * (PS * DQK);
     }
@@ -244,26 +275,34 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
     for (int blk = 0; blk < KBLK; ++blk) {
       constexpr int RPI = 64 / KCH;  // rows per instruction
 #pragma unroll
-      for (int i = 0; i < 16 / RPI; ++i) {
-        const int row = wave_u * 16 + i * RPI + lane / KCH;
+      for (int i = 0; i < RPW / RPI; ++i) {
+        const int idx = blk * (RPW / RPI) + i;
+        if (idx < FIRST || idx >= FIRST + COUNT) continue;
+        const int row = wave_u * RPW + i * RPI + lane / KCH;
         const int piece = (lane % KCH) ^ k_swizzle<KW>(row);
         const uint32_t t = min(kv0 + row, last_tok);
         const uint32_t off = (PAGED ? (t % PS) * (DQK * 2) : __umul24(t, k_stride_bytes)) + (blk * KW + piece * 8) * 2;
-        copy16_to_lds(kbase, off, stage + (blk * (BN * KW) + (wave_u * 16 + i * RPI) * KW) * 2);
+        copy16_to_lds(kbase, off, stage + (blk * (BN * KW) + (wave_u * RPW + i * RPI) * KW) * 2);
       }
     }
 #pragma unroll
     for (int blk = 0; blk < VBLK; ++blk) {
       constexpr int RPI = 64 / VCH;
 #pragma unroll
-      for (int i = 0; i < 16 / RPI; ++i) {
-        const int row = wave_u * 16 + i * RPI + lane / VCH;
+      for (int i = 0; i < RPW / RPI; ++i) {
+        const int idx = DQK / 8 / NW + blk * (RPW / RPI) + i;
+        if (idx < FIRST || idx >= FIRST + COUNT) continue;
+        const int row = wave_u * RPW + i * RPI + lane / VCH;
         const int piece = (lane % VCH) ^ v_swizzle<VW>(row);
         const uint32_t t = min(kv0 + row, last_tok);
         const uint32_t off = (PAGED ? (t % PS) * (DV * 2) : __umul24(t, v_stride_bytes)) + (blk * VW + piece * 8) * 2;
-        copy16_to_lds(vbase, off, stage + (BN * DQK + blk * (BN * VW) + (wave_u * 16 + i * RPI) * VW) * 2);
+        copy16_to_lds(vbase, off, stage + (BN * DQK + blk * (BN * VW) + (wave_u * RPW + i * RPI) * VW) * 2);
       }
     }
+  };
+  auto issue_tile = [&](int tile) {
+    if (PAGED && (tile & 63) == 0) load_page_ids(tile);
+    issue_copies(tile, std::integral_constant<int, 0>{}, std::integral_constant<int, COPIES>{});
   };
 
   // ---- per-lane fragment addressing (halfs, relative to the K / V part of a stage) -----------
@@ -354,27 +393,36 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   };
 
   const int n_tiles = (kv_end + BN - 1) / BN;
-  int page_next = 0;
-  if (n_tiles > 0) {
-    issue_tile(0, page_of(0), 0);
-    if (n_tiles > 1) page_next = page_of(BN);
+  // Tiles tile .. tile+NSTAGE-2 are in flight or landed at the top of iteration `tile`.
+#pragma unroll
+  for (int s = 0; s < NSTAGE - 1; ++s) {
+    if (s < n_tiles) issue_tile(s);
   }
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int kv0 = tile * BN;
-    const half_t* Ks = lds_tiles + (tile & 1) * STAGE;
+    const half_t* Ks = lds_tiles + (tile % NSTAGE) * STAGE;
     const half_t* Vs = Ks + BN * DQK;
-    // this wave's part of the tile has landed; after the barrier everyone's has, and every wave
-    // is done reading the other stage (tile-1), which the next copy overwrites
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
-    if (tile + 1 < n_tiles) {
-      issue_tile(kv0 + BN, page_next, (tile + 1) & 1);
-      if (tile + 2 < n_tiles) page_next = page_of(kv0 + 2 * BN);
+    // Wait until this wave's part of the tile has landed (copies complete in order, so it is enough
+    // that no more than the later tiles' copies are outstanding); after the barrier everyone's
+    // has, and every wave is done reading the stage of tile-1, which the next copy overwrites.
+    // Copies complete in order, so it is enough that no more than the later tiles' copies (the
+    // NSTAGE-2 iterations before this one issued COPIES each, where those tiles exist) are
+    // outstanding.  The count passed to s_waitcnt must never exceed what was really issued.
+    if (NSTAGE > 2 && tile + NSTAGE - 2 < n_tiles) {
+      wait_vmcnt<(NSTAGE - 2) * COPIES>();
+    } else {
+      wait_vmcnt<0>();
     }
+    __syncthreads();
+    // no prefetch across a 64-tile window of page ids: the ids held are those of the last copy issued
+    const int next = tile + NSTAGE - 1;  // the tile whose copy this iteration issues
+    const bool has_next = next < n_tiles;
+    const bool unmasked = TB == 2 && kv0 < wave_limit_max && kv0 + BN <= wave_limit_min;  // wave-uniform
+    if (has_next) issue_tile(next);
 
     if (kv0 >= wave_limit_max) continue;  // wave-uniform: every row of this wave is masked out
 
-    if (TB == 2 && kv0 + BN <= wave_limit_min) {
+    if (unmasked) {
       // Every row of the wave sees the whole tile (all tiles left of the causal diagonal): no
       // masking, and the two 32-token halves are software-pipelined so that the wave's own matrix
       // and vector work overlap: S1 = K1 Q^T runs under the softmax of S0, and O += V0 P0 under the
@@ -455,15 +503,15 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
 template <int DQK, int DV, bool PAGED, int PS>
 static void launch_prefill(const PrefillParams& p, int64_t total_q, hipStream_t stream) {
   const int64_t slots = total_q * p.group / BM + p.batch_size;
-  if (slots >= 65536) throw Error(TVMKV_EINVAL, "prefill: too many row tiles for one launch (65535 x 128 rows)");
-  constexpr size_t lds_bytes = 2 * BN * (DQK + DV) * sizeof(half_t);
+  if (slots >= 65536) throw Error(TVMKV_EINVAL, "prefill: too many row tiles for one launch");
+  constexpr size_t lds_bytes = prefill_lds_bytes(DQK, DV);
   static bool attr_set = false;  // per instantiation; the attribute is per function, not per device
   if (lds_bytes > 48 * 1024 && !attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, PAGED, PS>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     attr_set = true;
   }
-  hipLaunchKernelGGL((prefill_kernel<DQK, DV, PAGED, PS>), dim3(p.h_kv, static_cast<unsigned>(slots)), dim3(256),
+  hipLaunchKernelGGL((prefill_kernel<DQK, DV, PAGED, PS>), dim3(p.h_kv, static_cast<unsigned>(slots)), dim3(NW * 64),
                      lds_bytes, stream, p);
 }
 
