@@ -116,6 +116,21 @@ def calibrate(num_bytes=2 << 30, iters=10):
     return out
 
 
+# HBM bytes per launch of the decode entry point on the default workload, from rocprofv3 counter runs
+# of this file (profiles/decode_mfma_kernel_cfg2_batched_decode.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
+# in KiB per dispatch, decode_mfma_kernel + decode_merge_kernel; the scales come from the plain copy
+# kernel of known size (profiles/stream_copy_kernel_2GiB_calibration.txt).  It is a property of the
+# workload, so it is only reported when the algorithmic bytes are those it was measured on.
+TRAFFIC_MEASURED_ON_BYTES = 1182904320
+TRAFFIC_KIB = {"decode_mfma_kernel": (578946.1 * 2.0, 5053.8), "decode_merge_kernel": (2666.0 * 2.0, 528.0)}
+
+
+def measured_traffic(algorithmic_bytes):
+    if algorithmic_bytes != TRAFFIC_MEASURED_ON_BYTES:
+        return None
+    return int(sum(r + w for r, w in TRAFFIC_KIB.values()) * 1024)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -216,8 +231,9 @@ def main():
         "tokens_per_s": round(B / (ms_step * 1e-3), 1),
         "host_wall_ms_per_step": round(wall_ms, 4),
         "roofline": {"bound": "hbm", "achieved": round(gbps_decode, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps_decode / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "tvmkv_batch_decode_paged_kv (decode_splitkv_kernel + decode_merge_kernel)",
+                     "frac": round(gbps_decode / HBM_PEAK_GBPS, 4),
+                     "traffic": measured_traffic(int(decode_bytes)),
+                     "kernel": "tvmkv_batch_decode_paged_kv (decode_mfma_kernel + decode_merge_kernel)",
                      "ms": round(ms_decode, 4), "algorithmic_bytes": int(decode_bytes)},
     }
 
