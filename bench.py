@@ -131,6 +131,78 @@ def measured_traffic(algorithmic_bytes):
     return int(sum(r + w for r, w in TRAFFIC_KIB.values()) * 1024)
 
 
+def extras(torch, K, dev):
+    """configs[3] and configs[4] of BASELINE.json, kernels only (inputs resident, HIP events)."""
+    out = {}
+
+    def i32(a):
+        return torch.tensor(np.asarray(a), dtype=torch.int32, device=dev)
+
+    # ---- configs[3]: long-context split-KV decode, 64 q heads / 8 kv heads, 8 sequences ---------
+    rng = np.random.default_rng(3)
+    hq, hkv, d, ps = 64, 8, 128, 16
+    ctx = rng.integers(32768, 131072, size=8, endpoint=True)
+    npages = (ctx + ps - 1) // ps
+    pool = int(npages.sum()) + 64
+    perm = rng.permutation(pool).astype(np.int32)
+    pages = torch.empty((pool, 2, hkv, ps, d), dtype=torch.float16, device=dev)
+    for lo in range(0, pool, 8192):
+        pages[lo:lo + 8192].normal_()
+    indptr = np.concatenate([[0], np.cumsum(npages)])
+    q = torch.randn((8, hq, d), device=dev).to(torch.float16)
+    o = torch.empty_like(q)
+    lse = torch.empty((8, hq), dtype=torch.float32, device=dev)
+    z = torch.zeros(8, dtype=torch.int32, device=dev)
+    args = (q, pages, i32(indptr), i32(perm[:indptr[-1]]), i32((ctx - 1) % ps + 1), z, z, o, lse, 0, 1.0, 1e4,
+            d ** -0.5)
+    K.batch_decode_paged_kv(*args)
+    ms = time_region(torch, lambda i: K.batch_decode_paged_kv(*args), 10)
+    nbytes = float(ctx.sum()) * 2 * hkv * d * 2 + 2 * 8 * hq * d * 2
+    out["long_context_decode"] = {"workload": "configs[3]: 8 seqs, ctx U[32768,131072] seed 3, Hq64/Hkv8/D128, page 16",
+                                  "kv_tokens": int(ctx.sum()), "ms": round(ms, 4),
+                                  "GBps": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    del pages
+    torch.cuda.empty_cache()
+
+    # ---- configs[4]: MLA, 128 heads, latent 512 + rope 64, page 64 ------------------------------
+    hq, dl, dr, ps = 128, 512, 64, 64
+    sm = (128 + 64) ** -0.5
+
+    def mla_case(name, prefix, chunk, seed, causal):
+        rng = np.random.default_rng(seed)
+        kv = prefix + chunk
+        npg = (kv + ps - 1) // ps
+        pool = int(npg.sum()) + 8
+        perm = rng.permutation(pool).astype(np.int32)
+        pg = (torch.randn((pool, ps, dl + dr), device=dev) * 0.5).to(torch.float16)
+        ip = np.concatenate([[0], np.cumsum(npg)])
+        qi = np.concatenate([[0], np.cumsum(chunk)])
+        n = int(qi[-1])
+        q = (torch.randn((n, hq, dl + dr), device=dev) * 0.5).to(torch.float16)
+        o = torch.empty((n, hq, dl), dtype=torch.float16, device=dev)
+        lse = torch.empty((n, hq), dtype=torch.float32, device=dev)
+        a = (q, i32(qi), pg, i32(ip), i32(perm[:ip[-1]]), i32((kv - 1) % ps + 1), o, lse, causal, sm)
+        K.batch_prefill_paged_kv_mla(*a)
+        ms = time_region(torch, lambda i: K.batch_prefill_paged_kv_mla(*a), 10)
+        if causal:
+            pairs = float(np.sum(chunk * prefix + chunk * (chunk + 1) / 2))
+        else:
+            pairs = float(np.sum(chunk * kv))
+        flops = 2.0 * hq * (2 * dl + dr) * pairs  # QK^T over 576 features + PV over 512
+        nbytes = float(kv.sum()) * (dl + dr) * 2 + n * hq * (2 * dl + dr) * 2
+        out[name] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                     "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                     "GBps": round(nbytes / ms / 1e6, 1)}
+
+    rng = np.random.default_rng(4)
+    ctx = rng.integers(2048, 8192, size=32, endpoint=True)
+    mla_case("mla_decode", ctx - 1, np.ones(32, dtype=np.int64), 5, 0)
+    out["mla_decode"]["workload"] = "configs[4] decode: batch 32, ctx U[2048,8192] seed 4, 128 heads, 576-wide latent rows, page 64"
+    mla_case("mla_prefill", np.full(4, 2048), np.full(4, 1024), 6, 1)
+    out["mla_prefill"]["workload"] = "configs[4] prefill: 4 seqs, 1024-token chunk on a 2048-token prefix (chunk already appended), causal"
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -138,6 +210,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (profiling runs)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the chunked-prefill leg (profiling runs)")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time configs[3] (long-context decode) and configs[4] (MLA decode / prefill); "
+                         "reported under \"extras\", not part of the headline value")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the plain 2 GiB streaming read and copy kernels (bandwidth calibration; "
                          "known-size dispatches for scaling rocprofv3 traffic counters)")
@@ -274,6 +349,11 @@ def main():
                              "tflops": round(tflops, 2), "ms": round(ms_prefill, 4),
                              "algorithmic_flops": pw["flops"],
                              "frac_of_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
+
+    if args.extras:
+        del pages, qkv
+        torch.cuda.empty_cache()
+        result["extras"] = extras(torch, K, dev)
 
     # ---- CPU baseline: the oracle's restatement of the reference's llvm decode kernel ---------
     if not args.no_cpu_baseline:

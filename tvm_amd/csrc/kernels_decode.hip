@@ -585,19 +585,6 @@ static void* get_workspace(size_t bytes) {
   return ws.ptr;
 }
 
-static int compute_units() {
-  static int cached[64] = {0};
-  int dev = 0;
-  HIP_CHECK(hipGetDevice(&dev));
-  if (dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    HIP_CHECK(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
-    cached[dev] = n > 0 ? n : 256;
-  }
-  return cached[dev];
-}
-
 // Pages per chunk from shapes only: aim at ~8K workgroups, keep a chunk between 4 and 64 pages.
 static int pick_chunk_pages(int64_t nnz_pages, int h_kv) {
   static const char* forced = getenv("TVMKV_DECODE_CHUNK_PAGES");  // tuning aid

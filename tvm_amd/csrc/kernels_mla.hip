@@ -45,38 +45,62 @@ struct MlaParams {
   float scale_log2;
 };
 
+// First row-tile slot of sequence b.  A sequence starts a new tile; when h_q is not a multiple of
+// the tile height the rows before it may end inside a tile, and one spare slot per sequence covers
+// that.  (With h_q a multiple of the tile height there are no spare slots: in decode-shaped calls
+// they would alternate with the real ones and leave half of the XCDs idle.)
 __device__ __forceinline__ int mla_tile_slot_begin(const int32_t* q_indptr, int b, int h_q) {
-  return static_cast<int>((static_cast<int64_t>(q_indptr[b]) * h_q) / MLA_BM) + b;
+  return static_cast<int>((static_cast<int64_t>(q_indptr[b]) * h_q) / MLA_BM) + (h_q % MLA_BM != 0 ? b : 0);
 }
 
 __device__ __forceinline__ int mla_num_chunks(int kv_len, int max_chunks) {
   return max(1, min(max_chunks, (kv_len + MLA_MIN_CHUNK - 1) / MLA_MIN_CHUNK));
 }
 
-template <int DQK, int DV>
-__global__ __launch_bounds__(256) void mla_paged_kernel(MlaParams p) {
-  constexpr int BN = MLA_BN;
-  constexpr int KS = DQK / 16;
-  constexpr int DB = DV / 32;
-  constexpr int KROW = DQK + 8;
-  constexpr int VROW = BN + 4;
-  constexpr int FCH = DQK / 8;            // 16-byte pieces per cached row
-  constexpr int VCH = DV / 8;             // of which the first VCH belong to the value part
-  constexpr int UNITS = (BN / 4) * FCH;   // (4 tokens x 8 features) units per tile
-  constexpr int ROUNDS = (UNITS + 255) / 256;
+constexpr int MLA_WAVES = 8;    // wavefronts per workgroup, 16 rows each
+constexpr int MLA_STAGES = 4;   // 4 x 36 KiB of LDS: three tiles in flight behind the one being multiplied
 
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  half_t* Ks = reinterpret_cast<half_t*>(smem_raw);  // [BN][KROW]
-  half_t* Vt = Ks + BN * KROW;                       // [DV][VROW]
+// LDS image of a tile: DQK/64 column blocks of [MLA_BN rows][64 features] (128-byte rows, 8 pieces
+// of 16 bytes).  The same bytes are the A-operand of S^T = KV Q^T (ds_read_b128: 16 lanes = 16
+// consecutive rows at one piece) and, for the latent part, of O^T = V^T P^T (ds_read_b64_tr_b16: 32
+// lanes = 8 consecutive rows x 32 bytes).  Piece c of row r sits at piece position
+// c ^ mla_swizzle(r), the bit reversal of (r >> 1) & 7: rows 2 and 4 apart land in other 32-byte
+// parts of the 256-byte bank line (odd rows are its other half anyway), and 16 consecutive rows
+// take 16 different positions.
+__device__ __forceinline__ int mla_swizzle(int row) {
+  return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);
+}
+
+template <int DQK, int DV>
+__global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) {
+  constexpr int BN = MLA_BN;
+  static_assert(BN == 32 && MLA_BM == MLA_WAVES * 16 && DQK % 64 == 0 && DV % 64 == 0 && DV <= DQK, "tile shape");
+  constexpr int KS = DQK / 32;               // k-steps of the score product (v_mfma_f32_16x16x32_f16)
+  constexpr int DB = DV / 16;                // 16-wide output feature blocks
+  constexpr int NBLK = DQK / 64;             // column blocks of a tile
+  constexpr int BLK = BN * 64;               // halfs per column block
+  constexpr int STAGE = NBLK * BLK;          // halfs per stage
+  constexpr int NSTAGE = MLA_STAGES;
+  constexpr int NCOPY = NBLK * (BN / 8);     // copy instructions (8 rows x 128 B) per tile
+  constexpr int COPIES_HI = (NCOPY + MLA_WAVES - 1) / MLA_WAVES;  // per wave: the first NCOPY % MLA_WAVES waves
+  constexpr int COPIES_LO = NCOPY / MLA_WAVES;                    // ... the others
+  constexpr int WAVES_HI = NCOPY % MLA_WAVES;
+
+  extern __shared__ __attribute__((aligned(16))) half_t lds_tiles[];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
-  const int col = lane & 31;
-  const int half = lane >> 5;
+  const int c16 = lane & 15;   // query row of the wave (MFMA column) / token row of an A-fragment
+  const int g4 = lane >> 4;    // lane group: contraction slots 8*g4 .. 8*g4+7
   const int h_q = p.h_q;
 
-  const int slot = blockIdx.x;
+  // Work item = (row-tile slot, KV chunk), chunk fastest.  Workgroups are dealt round-robin to the
+  // 8 XCDs: with the chunk fastest the chunks of one row tile spread over the XCDs, and so do the
+  // row tiles of one sequence, whose cost grows along the sequence under the causal mask.
+  const int item = blockIdx.x;
+  const int slot = item / p.max_chunks;
+  const int chunk = item - slot * p.max_chunks;
   int b;
   {
     int lo = 0, hi = p.batch_size - 1;
@@ -101,10 +125,9 @@ __global__ __launch_bounds__(256) void mla_paged_kernel(MlaParams p) {
   const int ps = p.page_size;
   const int kv_len = npages > 0 ? (npages - 1) * ps + p.last_page_len[b] : 0;
   const int nchunks = mla_num_chunks(kv_len, p.max_chunks);
-  const int chunk = blockIdx.y;
   if (chunk >= nchunks) return;
 
-  const int my_row = r0 + wave * 32 + col;
+  const int my_row = r0 + wave * 16 + c16;
   const bool row_valid = my_row < rows;
   const int my_pos = my_row / h_q;
   const int my_head = my_row % h_q;
@@ -112,8 +135,8 @@ __global__ __launch_bounds__(256) void mla_paged_kernel(MlaParams p) {
   const int my_limit = row_valid ? (p.causal ? min(kv_len, causal_shift + my_pos) : kv_len) : 0;
   const int last_row_wg = min(rows, r0 + MLA_BM) - 1;
   const int kv_end = p.causal ? max(0, min(kv_len, causal_shift + last_row_wg / h_q)) : kv_len;
-  const int first_row_wave = r0 + wave * 32;
-  const int last_row_wave = min(rows, first_row_wave + 32) - 1;
+  const int first_row_wave = r0 + wave * 16;
+  const int last_row_wave = min(rows, first_row_wave + 16) - 1;
   const bool wave_active = first_row_wave < rows;
   const int wave_limit_max = !wave_active ? 0 : (p.causal ? min(kv_len, causal_shift + last_row_wave / h_q) : kv_len);
   const int wave_limit_min = !wave_active ? 0 : (p.causal ? min(kv_len, causal_shift + first_row_wave / h_q) : kv_len);
@@ -123,161 +146,176 @@ __global__ __launch_bounds__(256) void mla_paged_kernel(MlaParams p) {
   const int tile_lo = static_cast<int>(static_cast<int64_t>(chunk) * tiles_all / nchunks);
   const int tile_hi = min(static_cast<int>(static_cast<int64_t>(chunk + 1) * tiles_all / nchunks), (kv_end + BN - 1) / BN);
 
+  // Q^T fragments (B operand): column = query c16, contraction slots = features ks*32 + g4*8 .. +7
   half8_t qf[KS];
   {
-    const half_t* qrow = p.q + (static_cast<int64_t>(q_start + my_pos) * h_q + my_head) * DQK + half * 8;
+    const half_t* qrow = p.q + (static_cast<int64_t>(q_start + my_pos) * h_q + my_head) * DQK + g4 * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_valid ? ld16(qrow + ks * 16).h8 : zero16().h8;
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_valid ? ld16(qrow + ks * 32).h8 : zero16().h8;
   }
-  float16_t o[DB];
+  // O^T accumulators: o[db][j] is feature db*16 + 4*g4 + j of query c16
+  float4_t o[DB];
 #pragma unroll
-  for (int db = 0; db < DB; ++db) {
-#pragma unroll
-    for (int j = 0; j < 16; ++j) o[db][j] = 0.f;
-  }
+  for (int db = 0; db < DB; ++db) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
   float m = kNegInit, lsum = 0.f;
 
-  Vec16 stage[ROUNDS][4];
-  auto load_tile = [&](int kv0) {
-#pragma unroll
-    for (int r = 0; r < ROUNDS; ++r) {
-      const int idx = r * 256 + tid;
-      const int piece = idx % FCH;
-      const int tgroup = idx / FCH;
-      const int t0 = kv0 + tgroup * 4;
-      const half_t* src = nullptr;
-      if (idx < UNITS && t0 < kv_len) {
-        const int page = p.page_values[pbeg + t0 / ps];  // 4 | page_size: the 4 tokens share a page
-        src = p.pages + (static_cast<int64_t>(page) * ps + t0 % ps) * DQK + piece * 8;
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) stage[r][e] = (src != nullptr && t0 + e < kv_len) ? ld16(src + e * DQK) : zero16();
+  // ---- tile copy: global -> LDS -------------------------------------------------------------
+  // Copy instruction n of a tile (n = 0 .. NCOPY-1, dealt out to the waves in consecutive runs)
+  // moves rows 8*(n%4) .. +7 of column block n/4.  Rows past the end of the sequence repeat its last
+  // token (masked scores; P = 0 times a finite value).  The page ids of 16 consecutive tiles (4 row
+  // groups each) are fetched by one vector load, lane = 4*tile + row group: the wait for that load
+  // also waits for every copy in flight, so it must be rare.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const bool copies_hi = wave_u < WAVES_HI;
+  const int copy_first = copies_hi ? wave_u * COPIES_HI : WAVES_HI * COPIES_HI + (wave_u - WAVES_HI) * COPIES_LO;
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds_tiles));
+  const int last_tok = kv_len - 1;
+  int page_ids = 0;
+  auto issue_tile = [&](int tile) {
+    const int w = tile - tile_lo;
+    if ((w & 15) == 0) {
+      const int t = min((tile + (lane >> 2)) * BN + (lane & 3) * 8, last_tok);
+      page_ids = p.page_values[pbeg + t / ps];
     }
-  };
-  auto store_tile = [&]() {
-#pragma unroll
-    for (int r = 0; r < ROUNDS; ++r) {
-      const int idx = r * 256 + tid;
-      if (idx < UNITS) {
-        const int piece = idx % FCH;
-        const int tgroup = idx / FCH;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) st16(Ks + (tgroup * 4 + e) * KROW + piece * 8, stage[r][e]);
-        if (piece < VCH) {
-#pragma unroll
-          for (int e2 = 0; e2 < 4; ++e2) {
-            const uint32_t w0 = stage[r][0].w[e2], w1 = stage[r][1].w[e2], w2 = stage[r][2].w[e2], w3 = stage[r][3].w[e2];
-            uint2 even, odd;
-            even.x = (w0 & 0xffffu) | (w1 << 16);
-            even.y = (w2 & 0xffffu) | (w3 << 16);
-            odd.x = (w0 >> 16) | (w1 & 0xffff0000u);
-            odd.y = (w2 >> 16) | (w3 & 0xffff0000u);
-            *reinterpret_cast<uint2*>(Vt + (piece * 8 + 2 * e2) * VROW + tgroup * 4) = even;
-            *reinterpret_cast<uint2*>(Vt + (piece * 8 + 2 * e2 + 1) * VROW + tgroup * 4) = odd;
-          }
-        }
-      }
-    }
-  };
-
-  if (tile_lo < tile_hi) load_tile(tile_lo * BN);
-  for (int tile = tile_lo; tile < tile_hi; ++tile) {
     const int kv0 = tile * BN;
-    __syncthreads();
-    store_tile();
-    __syncthreads();
-    if (tile + 1 < tile_hi) load_tile(kv0 + BN);
-
-    if (kv0 < wave_limit_max) {
-      float16_t acc;
+    const uint32_t stage = lds_base + (w % NSTAGE) * (STAGE * 2);
 #pragma unroll
-      for (int j = 0; j < 16; ++j) acc[j] = 0.f;
-      const half_t* krow = Ks + col * KROW + half * 8;
+    for (int j = 0; j < COPIES_HI; ++j) {
+      if (j < COPIES_LO || copies_hi) {  // wave-uniform
+        const int n = copy_first + j;
+        const int blk = n >> 2;
+        const int rg = n & 3;
+        const int page = __builtin_amdgcn_readlane(page_ids, (w & 15) * 4 + rg);
+        const half_t* base = p.pages + static_cast<int64_t>(page) * ps * DQK;
+        const int row = rg * 8 + (lane >> 3);
+        const int piece = (lane & 7) ^ mla_swizzle(row);
+        const uint32_t t = min(kv0 + row, last_tok);
+        const uint32_t off = (t % ps) * (DQK * 2) + (blk * 64 + piece * 8) * 2;
+        copy16_to_lds(base, off, stage + (blk * BLK + rg * 8 * 64) * 2);
+      }
+    }
+  };
+
+  // ---- per-lane fragment addressing (halfs, relative to a stage) ---------------------------------
+  // K A-fragment of k-step ks, token block tb: row tb*16 + c16, features ks*32 + g4*8 .. +7
+  const int k_lane_off = c16 * 64;
+  const int k_swz = mla_swizzle(c16);  // the same for row + 16
+  // V^T A-fragment via the transposing read: lane li of a 16-lane group points at 4 features of
+  // token (li >> 2) of the group's 4 tokens and receives feature li of the group's 16 for the 4
+  // tokens.  Contraction slot 8*g4 + i holds token (i/4)*16 + 4*g4 + i%4, the order in which the
+  // S^T accumulators of the two token blocks hold them.
+  const int li = lane & 15;
+  const int v_row = 4 * g4 + (li >> 2);               // + 16 for the second half of the fragment
+  const int v_swz = mla_swizzle(v_row);               // row + 16 does not change it
+  const int v_lane_off = v_row * 64 + (li & 1) * 4;
+  const int v_piece = (li & 3) >> 1;                   // + 2 * (feature block % 4)
+
+  const int n_tiles = tile_hi - tile_lo;
+#pragma unroll
+  for (int s = 0; s < NSTAGE - 1; ++s) {
+    if (s < n_tiles) issue_tile(tile_lo + s);
+  }
+  for (int w = 0; w < n_tiles; ++w) {
+    const int kv0 = (tile_lo + w) * BN;
+    const half_t* T = lds_tiles + (w % NSTAGE) * STAGE;
+    // copies complete in order: it is enough that no more than the later tiles' copies are outstanding
+    if (w + NSTAGE - 2 < n_tiles) {
+      if (copies_hi) {
+        wait_vmcnt<(NSTAGE - 2) * COPIES_HI>();
+      } else {
+        wait_vmcnt<(NSTAGE - 2) * COPIES_LO>();
+      }
+    } else {
+      wait_vmcnt<0>();
+    }
+    __syncthreads();  // everyone's part of this tile has landed; everyone is done with the stage of tile w-1
+    if (w + NSTAGE - 1 < n_tiles) issue_tile(tile_lo + w + NSTAGE - 1);
+
+    if (kv0 >= wave_limit_max) continue;  // wave-uniform: every row of this wave is masked out
+
+    // ---- S^T = KV Q^T over all DQK features: two blocks of 16 tokens ------------------------------
+    float4_t s[2];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) {
+      s[tb] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const half8_t a = ld16(krow + ks * 16).h8;
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], acc, 0, 0, 0);
+        const int piece = ((ks & 1) * 4 + g4) ^ k_swz;
+        const half8_t a = *reinterpret_cast<const half8_t*>(T + (ks >> 1) * BLK + tb * 16 * 64 + k_lane_off + piece * 8);
+        s[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[ks], s[tb], 0, 0, 0);
       }
-      const bool need_mask = kv0 + BN > wave_limit_min;
-      float mx = kNegInit;
+    }
+    // s[tb][j]: token kv0 + tb*16 + 4*g4 + j, query c16
+    if (kv0 + BN > wave_limit_min) {  // wave-uniform: the causal diagonal or the end of the sequence
+      asm volatile("" ::: "memory");
+      const int rel = my_limit - kv0 - 4 * g4;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        float s = acc[j] * p.scale_log2;
-        if (need_mask) {
-          const int t = kv0 + (j >> 2) * 8 + half * 4 + (j & 3);
-          s = t < my_limit ? s : kNegInit;
-        }
-        acc[j] = s;
-        mx = fmaxf(mx, s);
+      for (int tb = 0; tb < 2; ++tb) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[tb][j] = (tb * 16 + j) < rel ? s[tb][j] : -3.0e38f;
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m, mx);
-      const float alpha = fast_exp2(m - m_new);
-      m = m_new;
-      lsum *= alpha;
+    }
+    float mx = -3.0e38f;
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
+    for (int tb = 0; tb < 2; ++tb) {
 #pragma unroll
-        for (int j = 0; j < 16; ++j) o[db][j] *= alpha;
-      }
-      half8_t pf[2];
+      for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[tb][j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, fmaxf(mx * p.scale_log2, -1.0e30f));  // a fully masked row keeps its maximum
+    const float alpha = fast_exp2(m - m_new);
+    m = m_new;
+    lsum *= alpha;
+    if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {  // wave-uniform: skip when no maximum moved
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        float pj = fast_exp2(acc[j] - m_new);
-        if (need_mask) {
-          const int t = kv0 + (j >> 2) * 8 + half * 4 + (j & 3);
-          pj = t < my_limit ? pj : 0.f;
-        }
+      for (int db = 0; db < DB; ++db) o[db] *= alpha;
+    }
+    half8_t pf;
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float pj = fast_exp2(fmaf(s[tb][j], p.scale_log2, -m_new));  // masked: exp2(-huge) = 0
         lsum += pj;
-        pf[j >> 3][j & 7] = static_cast<half_t>(pj);
+        pf[tb * 4 + j] = static_cast<half_t>(pj);
       }
+    }
+    // ---- O^T += V^T P^T: the value is the first DV features of the same rows ---------------------
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const half_t* vrow = Vt + (db * 32 + col) * VROW + half * 4;
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-          const half4_t lo = *reinterpret_cast<const half4_t*>(vrow + kk * 16);
-          const half4_t hi = *reinterpret_cast<const half4_t*>(vrow + kk * 16 + 8);
-          half8_t a;
-          a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
-          a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[kk], o[db], 0, 0, 0);
-        }
-      }
+    for (int db = 0; db < DB; ++db) {
+      const half_t* vb = T + (db >> 2) * BLK + v_lane_off + (((db & 3) * 2 + v_piece) ^ v_swz) * 8;
+      const half4_t lo = lds_read_tr16(vb);
+      const half4_t hi = lds_read_tr16(vb + 16 * 64);
+      half8_t a;
+      a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
+      a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pf, o[db], 0, 0, 0);
     }
   }
 
+  // the row sums are per lane group: add them up; m is already common
+  lsum += __shfl_xor(lsum, 16, 64);
   lsum += __shfl_xor(lsum, 32, 64);
   if (!row_valid) return;
   const int64_t grow = static_cast<int64_t>(q_start + my_pos) * h_q + my_head;  // global row
   if (nchunks == 1) {
     const float denom = lsum + fast_exp2(kNegInit - m);
     const float inv = 1.0f / denom;
-    half_t* orow = p.output + grow * DV + half * 4;
+    half_t* orow = p.output + grow * DV + 4 * g4;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
+      half4_t out4;
 #pragma unroll
-      for (int j4 = 0; j4 < 4; ++j4) {
-        half4_t out4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) out4[e] = static_cast<half_t>(o[db][j4 * 4 + e] * inv);
-        *reinterpret_cast<half4_t*>(orow + db * 32 + j4 * 8) = out4;
-      }
+      for (int e = 0; e < 4; ++e) out4[e] = static_cast<half_t>(o[db][e] * inv);
+      *reinterpret_cast<half4_t*>(orow + db * 16) = out4;
     }
-    if (half == 0) p.lse[grow] = m + fast_log2(denom);
+    if (g4 == 0) p.lse[grow] = m + fast_log2(denom);
   } else {
-    float* prow = p.part_o + (grow * p.max_chunks + chunk) * DV + half * 4;
+    float* prow = p.part_o + (grow * p.max_chunks + chunk) * DV + 4 * g4;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-#pragma unroll
-      for (int j4 = 0; j4 < 4; ++j4) {
-        float4_t out4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) out4[e] = o[db][j4 * 4 + e];
-        *reinterpret_cast<float4_t*>(prow + db * 32 + j4 * 8) = out4;
-      }
-    }
-    if (half == 0) {
+    for (int db = 0; db < DB; ++db) *reinterpret_cast<float4_t*>(prow + db * 16) = o[db];
+    if (g4 == 0) {
       p.part_ml[(grow * p.max_chunks + chunk) * 2 + 0] = m;
       p.part_ml[(grow * p.max_chunks + chunk) * 2 + 1] = lsum;
     }
@@ -369,8 +407,8 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
   KV_UNSUPPORTED(d_latent != 512 || d_rope != 64)
       << "batch_prefill_paged_kv_mla: (d_latent, d_rope) = (" << d_latent << ", " << d_rope
       << ") is not built ((512, 64))";
-  KV_UNSUPPORTED(page_size <= 0 || page_size % 4 != 0)
-      << "batch_prefill_paged_kv_mla: page_size " << page_size << " must be a positive multiple of 4";
+  KV_UNSUPPORTED(page_size <= 0 || page_size % 8 != 0)
+      << "batch_prefill_paged_kv_mla: page_size " << page_size << " must be a positive multiple of 8";
   if (batch_size == 0 || total_q == 0) return TVMKV_OK;
   KV_CHECK(q && q_indptr && pages && page_indptr && length_info && output && lse)
       << "batch_prefill_paged_kv_mla: NULL tensor";
@@ -390,10 +428,11 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
   p.page_size = page_size;
   p.causal = causal > 0;
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
-  const int64_t slots = total_q * h_q / MLA_BM + batch_size;
+  const int64_t slots = total_q * h_q / MLA_BM + (h_q % MLA_BM != 0 ? batch_size : 0);
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_prefill_paged_kv_mla: too many row tiles";
   // split the KV only when the row tiles alone cannot fill the chip (decode-shaped calls)
-  int max_chunks = static_cast<int>(512 / slots);
+  // one workgroup per compute unit is resident (LDS): aim at one round of workgroups
+  int max_chunks = static_cast<int>(compute_units() / slots);
   max_chunks = max_chunks < 1 ? 1 : (max_chunks > 16 ? 16 : max_chunks);
   p.max_chunks = max_chunks;
   if (max_chunks > 1) {
@@ -403,7 +442,7 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
     p.part_o = reinterpret_cast<float*>(ws);
     p.part_ml = reinterpret_cast<float*>(ws + part_o_bytes);
   }
-  constexpr size_t lds_bytes = (MLA_BN * (DQK + 8) + DV * (MLA_BN + 4)) * sizeof(half_t);
+  constexpr size_t lds_bytes = static_cast<size_t>(MLA_STAGES) * MLA_BN * DQK * sizeof(half_t);
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_paged_kernel<DQK, DV>),
@@ -411,7 +450,10 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
     attr_set = true;
   }
   hipStream_t s = as_stream(stream);
-  hipLaunchKernelGGL((mla_paged_kernel<DQK, DV>), dim3(static_cast<unsigned>(slots), max_chunks), dim3(256), lds_bytes,
+  KV_CHECK(slots * max_chunks < (int64_t{1} << 31) - 8) << "batch_prefill_paged_kv_mla: too many row tiles";
+  const unsigned grid = static_cast<unsigned>(slots * max_chunks);
+  hipLaunchKernelGGL((mla_paged_kernel<DQK, DV>), dim3(grid), dim3(MLA_WAVES * 64),
+                     lds_bytes,
                      s, p);
   KV_LAUNCH_CHECK();
   if (max_chunks > 1) {

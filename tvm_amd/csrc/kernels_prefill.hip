@@ -37,38 +37,6 @@ constexpr int BM = NW * 32;  // rows per workgroup
 constexpr int RPW = 64 / NW; // token rows of a tile copied by each wave
 constexpr int BN = 64;   // kv tokens per tile
 
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-
-// One global_load_lds_dwordx4: lane L copies the 16 bytes at its own global address to LDS address
-// lds_addr + 16*L (lds_addr must be the same in every lane).  The copy is asynchronous and counted
-// by vmcnt.  It is issued from inline assembly on purpose: when the compiler knows of a copy in
-// flight it puts s_waitcnt vmcnt(0) in front of the next LDS read it cannot tell apart from the
-// copy's destination, which would serialise the two-stage pipeline; here the one wait per tile is
-// written by hand in front of the workgroup barrier.  The compiler sets M0 itself right before
-// each of its own uses, so the asm does not have to restore it.
-// src_base (the same in every lane) + byte_off (per lane, unsigned 32 bit) is the global address.
-__device__ __forceinline__ void copy16_to_lds(const void* src_base, uint32_t byte_off, uint32_t lds_addr) {
-  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               ::"v"(byte_off), "s"(src_base), "s"(lds_addr) : "memory");
-}
-
-// Tells the compiler that a pointer holds the same value in every lane.
-__device__ __forceinline__ const half_t* uniform_ptr(const half_t* p) {
-  const uint64_t v = reinterpret_cast<uint64_t>(p);
-  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
-  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
-  return reinterpret_cast<const half_t*>((static_cast<uint64_t>(hi) << 32) | lo);
-}
-typedef short short4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) short4_t* lds_short4_ptr_t;
-
-// ds_read_b64_tr_b16: within each group of 16 lanes, lane l receives element l%4 of the four
-// 8-byte rows addressed by lanes l/4, 4 + l/4, 8 + l/4 and 12 + l/4 of the group.
-__device__ __forceinline__ half4_t lds_read_tr16(const half_t* p) {
-  return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr_t)p));
-}
-
 struct PrefillParams {
   const half_t* q;
   const int32_t* q_indptr;
@@ -108,16 +76,6 @@ __device__ __forceinline__ int v_swizzle(int row) {
   return W == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
 }
 
-// Scheduling hint for the region it is placed in: N groups of (1 MFMA, then a few vector ALU ops).
-template <int N>
-__device__ __forceinline__ void interleave_mfma_valu() {
-#pragma unroll
-  for (int i = 0; i < N; ++i) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-    __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);  // VALU
-  }
-}
-
 // Pipeline depth: as many stages as fit next to a second workgroup (NW = 4) or alone (NW = 8).
 constexpr int prefill_stages(int dqk, int dv) {
   const int stage_bytes = BN * (dqk + dv) * 2;
@@ -127,12 +85,6 @@ constexpr int prefill_stages(int dqk, int dv) {
 
 constexpr size_t prefill_lds_bytes(int dqk, int dv) {
   return static_cast<size_t>(prefill_stages(dqk, dv)) * BN * (dqk + dv) * 2;
-}
-
-// s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters at their maximum)
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
 template <int DQK, int DV, bool PAGED, int PS>
