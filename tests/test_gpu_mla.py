@@ -68,6 +68,25 @@ def test_mla_decode_shaped_split_kv(ps):
     assert not go[6].any() and np.all(gl[6] == np.float32(-5e4))
 
 
+def test_mla_as_many_tokens_as_sequences_but_not_a_decode_step():
+    """total_q == batch makes the launcher split the KV; sequences that do not have exactly one
+    query token must still come out right (they are done unsplit by the workgroups of chunk 0)."""
+    rng = np.random.default_rng(33)
+    kv_lens, q_lens = [700, 50, 300, 420], [2, 0, 1, 1]
+    go, gl, eo, el = _mla_both(rng, kv_lens, q_lens, 64, npages=30)
+    assert_close(go, eo, what="mla mixed out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla mixed lse")
+
+
+def test_mla_decode_heads_not_a_multiple_of_the_row_tile():
+    rng = np.random.default_rng(34)
+    kv_lens = [900, 33, 257]
+    for heads in (16, 160):
+        go, gl, eo, el = _mla_both(rng, kv_lens, [1, 1, 1], 16, npages=80, heads=heads)
+        assert_close(go, eo, what=f"mla decode out, {heads} heads")
+        assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"mla decode lse, {heads} heads")
+
+
 @pytest.mark.parametrize("causal", [0, 1])
 def test_mla_prefill_shaped(causal):
     rng = np.random.default_rng(31)

@@ -8,16 +8,20 @@
 // same kernel for MLA decode (src/runtime/vm/paged_kv_cache.cc:954-956), and so does this one.
 // Numerics as in kernels_prefill.hip (base-2 online softmax, m = -5e4, d = 1 initial state).
 //
-// Tiling: 128 rows (position, head) per workgroup, 32 rows per wave with the query on the MFMA
-// N axis; 32-token KV tiles are read from HBM once per workgroup and written to LDS twice: row
-// major (A-operand of S^T = KV Q^T) and transposed (A-operand of O^T = V^T P^T).  O^T of one wave
-// is 512 x 32 fp32 = 256 accumulator registers, Q is 144 registers of B-fragments: one wave per
-// SIMD.
+// Tiling: 128 rows (position, head) per workgroup of 8 wavefronts, 16 rows per wave with the query
+// on the N axis of v_mfma_f32_16x16x32_f16: O^T of one wave is 512 x 16 fp32 = 128 accumulator
+// registers, Q is 72 registers of B-fragments, which leaves room for two waves per SIMD.  32-token
+// tiles of cached rows are copied from global memory straight into LDS (global_load_lds_dwordx4),
+// four stages deep; the same LDS bytes serve as A-operand of S^T = KV Q^T (ds_read_b128) and of
+// O^T = V^T P^T (ds_read_b64_tr_b16, which transposes on the way out of LDS).
 //
-// KV split: decode-shaped calls have too few row tiles to fill 256 CUs, so a sequence's KV may be
-// cut into up to `max_chunks` chunks (grid.y), each at least 128 tokens; partial (O, m, l) states
-// go to an fp32 buffer indexed by (global row, chunk) and a second kernel merges them.  The chunk
-// count of a sequence is a pure function of its kv_len, recomputed by both kernels.
+// KV split: decode-shaped calls (one token per sequence) have too few row tiles to fill 256 CUs,
+// so the KV of a sequence is cut into chunks of about `chunk_tokens` tokens; partial (O, m, l)
+// states go to an fp32 buffer indexed by (chunk slot, head) and a second kernel merges them.  The
+// chunk slots of a sequence are a pure function of the page table, recomputed by both kernels.
+#include <algorithm>
+#include <cstdlib>
+
 #include "kernels_common.cuh"
 
 namespace tvmkv {
@@ -35,13 +39,15 @@ struct MlaParams {
   const int32_t* last_page_len;
   half_t* output;
   float* lse;
-  float* part_o;   // (total_rows, max_chunks, DV)
-  float* part_ml;  // (total_rows, max_chunks, 2)
+  float* part_o;   // (chunk slots, h_q, DV)
+  float* part_ml;  // (chunk slots, h_q, 2)
   int batch_size;
   int h_q;
   int page_size;
   int causal;
-  int max_chunks;
+  int split;         // 1: decode-shaped call, the KV of a sequence is cut into chunks (see mla_chunk_slot_begin)
+  int chunk_tokens;  // target tokens per chunk
+  int row_tiles;     // split: row tiles of a one-token sequence, ceil(h_q / MLA_BM)
   float scale_log2;
 };
 
@@ -53,8 +59,12 @@ __device__ __forceinline__ int mla_tile_slot_begin(const int32_t* q_indptr, int 
   return static_cast<int>((static_cast<int64_t>(q_indptr[b]) * h_q) / MLA_BM) + (h_q % MLA_BM != 0 ? b : 0);
 }
 
-__device__ __forceinline__ int mla_num_chunks(int kv_len, int max_chunks) {
-  return max(1, min(max_chunks, (kv_len + MLA_MIN_CHUNK - 1) / MLA_MIN_CHUNK));
+// Split mode: sequence b owns the chunk slots [mla_chunk_slot_begin(b), mla_chunk_slot_begin(b+1)),
+// a function of the page table alone (so the grid can be sized from shapes: at most
+// floor(nnz_pages * page_size / chunk_tokens) + batch slots, every one of them in use), and its KV
+// tiles are divided evenly among them: about chunk_tokens tokens each.
+__device__ __forceinline__ int mla_chunk_slot_begin(const int32_t* page_indptr, int b, int page_size, int chunk_tokens) {
+  return static_cast<int>(static_cast<int64_t>(page_indptr[b]) * page_size / chunk_tokens) + b;
 }
 
 constexpr int MLA_WAVES = 8;    // wavefronts per workgroup, 16 rows each
@@ -95,14 +105,30 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
   const int g4 = lane >> 4;    // lane group: contraction slots 8*g4 .. 8*g4+7
   const int h_q = p.h_q;
 
-  // Work item = (row-tile slot, KV chunk), chunk fastest.  Workgroups are dealt round-robin to the
-  // 8 XCDs: with the chunk fastest the chunks of one row tile spread over the XCDs, and so do the
-  // row tiles of one sequence, whose cost grows along the sequence under the causal mask.
-  const int item = blockIdx.x;
-  const int slot = item / p.max_chunks;
-  const int chunk = item - slot * p.max_chunks;
-  int b;
-  {
+  // Work item.  Normal mode: a row-tile slot.  Split mode: (chunk slot, row tile of a one-token
+  // sequence), the grid holding exactly the items in use: a workgroup takes a whole compute unit
+  // (LDS, registers) and runs long, and workgroups that only find out they have nothing to do
+  // still disturb the placement of the others.
+  int b, r0, chunk = 0, nchunks = 1, cslot = 0, row_step = 0;
+  if (p.split) {
+    cslot = blockIdx.x / p.row_tiles;
+    r0 = (blockIdx.x - cslot * p.row_tiles) * MLA_BM;
+    row_step = p.row_tiles * MLA_BM;
+    int lo = 0, hi = p.batch_size - 1;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) >> 1;
+      if (mla_chunk_slot_begin(p.page_indptr, mid, p.page_size, p.chunk_tokens) <= cslot) {
+        lo = mid;
+      } else {
+        hi = mid - 1;
+      }
+    }
+    b = lo;
+    const int first = mla_chunk_slot_begin(p.page_indptr, b, p.page_size, p.chunk_tokens);
+    chunk = cslot - first;
+    nchunks = mla_chunk_slot_begin(p.page_indptr, b + 1, p.page_size, p.chunk_tokens) - first;
+  } else {
+    const int slot = blockIdx.x;
     int lo = 0, hi = p.batch_size - 1;
     while (lo < hi) {
       int mid = (lo + hi + 1) >> 1;
@@ -113,20 +139,24 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
       }
     }
     b = lo;
+    r0 = (slot - mla_tile_slot_begin(p.q_indptr, b, h_q)) * MLA_BM;
   }
   const int q_start = p.q_indptr[b];
   const int qo_len = p.q_indptr[b + 1] - q_start;
   const int rows = qo_len * h_q;
-  const int r0 = (slot - mla_tile_slot_begin(p.q_indptr, b, h_q)) * MLA_BM;
-  if (r0 >= rows) return;
+  if (p.split && qo_len != 1) {
+    // not a decode step after all: the workgroups of chunk 0 do the whole sequence, unsplit
+    if (chunk != 0) return;
+    nchunks = 1;
+  }
 
   const int pbeg = p.page_indptr[b];
   const int npages = p.page_indptr[b + 1] - pbeg;
   const int ps = p.page_size;
   const int kv_len = npages > 0 ? (npages - 1) * ps + p.last_page_len[b] : 0;
-  const int nchunks = mla_num_chunks(kv_len, p.max_chunks);
-  if (chunk >= nchunks) return;
 
+  // normal mode: one pass; split mode: one pass per row tile this workgroup owns (one, for a decode step)
+  for (; r0 < rows; r0 += row_step) {
   const int my_row = r0 + wave * 16 + c16;
   const bool row_valid = my_row < rows;
   const int my_pos = my_row / h_q;
@@ -297,7 +327,7 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
   // the row sums are per lane group: add them up; m is already common
   lsum += __shfl_xor(lsum, 16, 64);
   lsum += __shfl_xor(lsum, 32, 64);
-  if (!row_valid) return;
+  if (row_valid) {
   const int64_t grow = static_cast<int64_t>(q_start + my_pos) * h_q + my_head;  // global row
   if (nchunks == 1) {
     const float denom = lsum + fast_exp2(kNegInit - m);
@@ -312,13 +342,19 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
     }
     if (g4 == 0) p.lse[grow] = m + fast_log2(denom);
   } else {
-    float* prow = p.part_o + (grow * p.max_chunks + chunk) * DV + 4 * g4;
+    // only one-token sequences are split: the row is the head
+    const int64_t prow_idx = static_cast<int64_t>(cslot) * h_q + my_head;
+    float* prow = p.part_o + prow_idx * DV + 4 * g4;
 #pragma unroll
     for (int db = 0; db < DB; ++db) *reinterpret_cast<float4_t*>(prow + db * 16) = o[db];
     if (g4 == 0) {
-      p.part_ml[(grow * p.max_chunks + chunk) * 2 + 0] = m;
-      p.part_ml[(grow * p.max_chunks + chunk) * 2 + 1] = lsum;
+      p.part_ml[prow_idx * 2 + 0] = m;
+      p.part_ml[prow_idx * 2 + 1] = lsum;
     }
+  }
+  }
+  if (row_step == 0) break;
+  __syncthreads();  // the LDS stages are reused by the next pass
   }
 }
 
@@ -340,23 +376,25 @@ __global__ __launch_bounds__(DV / 4) void mla_merge_kernel(MlaParams p) {
     }
     b = lo;
   }
-  // skip sequences with qo_len == 0 that share the q_indptr value: the search above returns the
-  // last b with q_indptr[b] <= token, which is the one that owns the token
-  const int npages = p.page_indptr[b + 1] - p.page_indptr[b];
-  const int kv_len = npages > 0 ? (npages - 1) * p.page_size + p.last_page_len[b] : 0;
-  const int nchunks = mla_num_chunks(kv_len, p.max_chunks);
+  // (sequences with qo_len == 0 share their q_indptr value with the next one: the search returns
+  // the last b with q_indptr[b] <= token, which is the one that owns the token)
+  if (p.q_indptr[b + 1] - p.q_indptr[b] != 1) return;  // only one-token sequences are split
+  const int first = mla_chunk_slot_begin(p.page_indptr, b, p.page_size, p.chunk_tokens);
+  const int nchunks = mla_chunk_slot_begin(p.page_indptr, b + 1, p.page_size, p.chunk_tokens) - first;
   if (nchunks == 1) return;
   const int64_t grow = static_cast<int64_t>(token) * p.h_q + head;
-  const float* ml = p.part_ml + grow * p.max_chunks * 2;
+  const int64_t prow = static_cast<int64_t>(first) * p.h_q + head;  // + c * h_q for chunk c
+  const float* ml = p.part_ml + prow * 2;
+  const int64_t cstride = p.h_q;
   float mx = kNegInit;
-  for (int c = 0; c < nchunks; ++c) mx = fmaxf(mx, ml[c * 2]);
+  for (int c = 0; c < nchunks; ++c) mx = fmaxf(mx, ml[c * cstride * 2]);
   float lsum = 0.f;
   float4_t acc = {0.f, 0.f, 0.f, 0.f};
   const int d = threadIdx.x * 4;
   for (int c = 0; c < nchunks; ++c) {
-    const float sc = fast_exp2(ml[c * 2] - mx);
-    lsum += ml[c * 2 + 1] * sc;
-    const float4_t po = *reinterpret_cast<const float4_t*>(p.part_o + (grow * p.max_chunks + c) * DV + d);
+    const float sc = fast_exp2(ml[c * cstride * 2] - mx);
+    lsum += ml[c * cstride * 2 + 1] * sc;
+    const float4_t po = *reinterpret_cast<const float4_t*>(p.part_o + (prow + c * cstride) * DV + d);
     acc += po * sc;
   }
   const float denom = lsum + fast_exp2(kNegInit - mx);
@@ -430,15 +468,29 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
   const int64_t slots = total_q * h_q / MLA_BM + (h_q % MLA_BM != 0 ? batch_size : 0);
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_prefill_paged_kv_mla: too many row tiles";
-  // split the KV only when the row tiles alone cannot fill the chip (decode-shaped calls)
-  // one workgroup per compute unit is resident (LDS): aim at one round of workgroups
-  int max_chunks = static_cast<int>(compute_units() / slots);
-  max_chunks = max_chunks < 1 ? 1 : (max_chunks > 16 ? 16 : max_chunks);
-  p.max_chunks = max_chunks;
-  if (max_chunks > 1) {
-    const size_t rows = static_cast<size_t>(total_q) * h_q;
-    const size_t part_o_bytes = rows * max_chunks * DV * sizeof(float);
-    char* ws = static_cast<char*>(mla_workspace(part_o_bytes + rows * max_chunks * 2 * sizeof(float)));
+  // Decode-shaped calls (one token per sequence, as far as the shapes tell) have too few row
+  // tiles for the chip, so the KV of a sequence is cut into chunks of about chunk_tokens tokens.
+  // One workgroup per compute unit is resident (LDS), so aim at one round of workgroups:
+  // chunk slots = floor(tokens / chunk_tokens) + B, times the row tiles of a sequence, <= CUs.
+  const int cus = compute_units();
+  const int row_tiles = (h_q + MLA_BM - 1) / MLA_BM;
+  const int64_t tokens = nnz_pages * page_size;  // upper bound on the cached tokens
+  int64_t grid = slots;
+  if (total_q == batch_size && static_cast<int64_t>(batch_size) * row_tiles * 2 <= cus && tokens > 0) {
+    const int64_t room = cus / row_tiles - batch_size;
+    int64_t ct = (tokens + room - 1) / room;
+    ct = std::max<int64_t>(MLA_MIN_CHUNK, (ct + MLA_BN - 1) / MLA_BN * MLA_BN);
+    if (const char* e = getenv("TVMKV_MLA_CHUNK_TOKENS")) {  // tuning aid
+      if (atoi(e) >= MLA_BN) ct = atoi(e) / MLA_BN * MLA_BN;
+    }
+    const int64_t cslots = tokens / ct + batch_size;
+    p.split = 1;
+    p.chunk_tokens = static_cast<int>(ct);
+    p.row_tiles = row_tiles;
+    grid = cslots * row_tiles;
+    const size_t part_rows = static_cast<size_t>(cslots) * h_q;
+    const size_t part_o_bytes = part_rows * DV * sizeof(float);
+    char* ws = static_cast<char*>(mla_workspace(part_o_bytes + part_rows * 2 * sizeof(float)));
     p.part_o = reinterpret_cast<float*>(ws);
     p.part_ml = reinterpret_cast<float*>(ws + part_o_bytes);
   }
@@ -450,13 +502,11 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
     attr_set = true;
   }
   hipStream_t s = as_stream(stream);
-  KV_CHECK(slots * max_chunks < (int64_t{1} << 31) - 8) << "batch_prefill_paged_kv_mla: too many row tiles";
-  const unsigned grid = static_cast<unsigned>(slots * max_chunks);
-  hipLaunchKernelGGL((mla_paged_kernel<DQK, DV>), dim3(grid), dim3(MLA_WAVES * 64),
-                     lds_bytes,
+  KV_CHECK(grid < (int64_t{1} << 31)) << "batch_prefill_paged_kv_mla: too many work items";
+  hipLaunchKernelGGL((mla_paged_kernel<DQK, DV>), dim3(static_cast<unsigned>(grid)), dim3(MLA_WAVES * 64), lds_bytes,
                      s, p);
   KV_LAUNCH_CHECK();
-  if (max_chunks > 1) {
+  if (p.split) {
     hipLaunchKernelGGL(mla_merge_kernel<DV>, dim3(static_cast<unsigned>(total_q), h_q), dim3(DV / 4), 0, s, p);
     KV_LAUNCH_CHECK();
   }
