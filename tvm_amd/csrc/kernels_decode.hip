@@ -267,8 +267,9 @@ __global__ __launch_bounds__(256) void decode_splitkv_kernel(DecodeParams p) {
 // run on v_mfma_f32_16x16x32_f16 with the query heads of the group padded to the 16-wide N axis:
 //   S^T[token, head] = K Q^T   -- K fragments come straight from global memory in the MFMA
 //                                 A-layout (lane = token row, 16 bytes of features), no staging;
-//   O^T[d, head]     = V^T P^T -- V is loaded coalesced (16 lanes per 256-byte row), transposed
-//                                 through a wave-private LDS tile so that tokens run along the
+//   O^T[d, head]     = V^T P^T -- the V rows go from global memory straight into a wave-private
+//                                 LDS tile (global_load_lds_dwordx4, no registers) and come out
+//                                 of it transposed (ds_read_b64_tr_b16), tokens along the
 //                                 contraction axis; P stays in registers (the S^T accumulator
 //                                 layout is the B-operand layout).
 // A wave consumes two pages (32 tokens) per step: 16 KiB of K/V, 16 MFMAs, a handful of vector
@@ -277,12 +278,17 @@ __global__ __launch_bounds__(256) void decode_splitkv_kernel(DecodeParams p) {
 // ------------------------------------------------------------------------------------------
 constexpr int DM_D = 128;
 constexpr int DM_PS = 16;
-constexpr int DM_VROW = 36;  // halfs per row of the transposed V tile (32 tokens + padding)
+constexpr int DM_VTILE = 2 * DM_PS * DM_D;  // halfs of a wave's V tile: two pages, row-major
+
+// Piece (16 bytes) c of V row r sits at piece position c ^ dm_swizzle(r): the transposing read of
+// 32 lanes touches 8 consecutive rows x 32 bytes, which this spreads over the 8 32-byte parts of
+// a 256-byte bank line.
+__device__ __forceinline__ int dm_swizzle(int row) { return (row & 7) << 1; }
 
 __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int group, int num_items) {
-  constexpr int D = DM_D, PS = DM_PS, VROW = DM_VROW;
-  static_assert(D * VROW * sizeof(half_t) >= 16 * D * sizeof(float), "the merge buffer aliases the V tile");
-  __shared__ __attribute__((aligned(16))) half_t Vt_all[4][D * VROW];
+  constexpr int D = DM_D, PS = DM_PS;
+  static_assert(DM_VTILE * sizeof(half_t) >= 16 * D * sizeof(float), "the merge buffer aliases the V tile");
+  __shared__ __attribute__((aligned(16))) half_t Vt_all[4][DM_VTILE];
   __shared__ float sm_m[4][16];
   __shared__ float sm_l[4][16];
 
@@ -322,55 +328,48 @@ __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int
   for (int db = 0; db < 8; ++db) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
   float m = kNegInit, lsum = 0.f;
 
+  // V^T fragment via the transposing read: lane li of a 16-lane group points at 4 features of token
+  // (li >> 2) of the group's 4 tokens and receives feature li of the group's 16 for the 4 tokens
+  const uint32_t vt_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)Vt));
+  const int v_row = 4 * g4 + (c16 >> 2);             // + PS for the second page: same swizzle
+  const int v_swz = dm_swizzle(v_row);
+  const int v_lane_off = v_row * D + (c16 & 1) * 4;
+  const int v_piece = (c16 & 3) >> 1;                // + 2 * feature block
+
   // One step = pages (pi, pi+1).  K: lane reads row c16 of the page, features ks*32 + g4*8.
-  // V: lane reads rows 4*g4 + j of the page, features c16*8 (coalesced 256-byte rows).
+  // V: 8 copy instructions of 4 rows x 256 bytes each fill the wave's LDS tile; rows at or past
+  // kv_len repeat the last cached row of their page and a missing second page repeats the first
+  // (their P is 0, and 0 times cached data is 0, whereas unwritten memory could hold NaN patterns).
   struct Regs {
     Vec16 k[2][4];
-    Vec16 v[2][4];
   };
   auto issue = [&](int pi, Regs& r) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
+      const int pg = min(pi + h, page_hi - 1);
+      const int page = __builtin_amdgcn_readfirstlane(p.page_values[pbeg + pg]);
+      const half_t* kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * head_stride;
+      const half_t* vbase = kbase + static_cast<int64_t>(p.h_kv) * head_stride;
+      const int last_row = min(PS, kv_len - pg * PS) - 1;  // >= 0: every page of the table holds a token
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = i * 4 + (lane >> 4);
+        const int piece = (lane & 15) ^ dm_swizzle(h * PS + row);
+        copy16_to_lds(vbase, static_cast<uint32_t>(min(row, last_row) * (D * 2) + piece * 16),
+                      vt_lds + (h * PS + i * 4) * (D * 2));
+      }
       if (pi + h < page_hi) {
-        const int page = __builtin_amdgcn_readfirstlane(p.page_values[pbeg + pi + h]);
-        const half_t* kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * head_stride;
-        const half_t* vbase = kbase + static_cast<int64_t>(p.h_kv) * head_stride;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) r.v[h][j] = ld16(vbase + (4 * g4 + j) * D + c16 * 8);
       } else {
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = zero16();
-#pragma unroll
-        for (int j = 0; j < 4; ++j) r.v[h][j] = zero16();
       }
     }
   };
 
   auto consume = [&](int pi, Regs& r) {
     const bool partial = (pi + 2) * PS > kv_len;  // wave-uniform
-    // ---- V: zero the rows beyond kv_len, transpose into the wave's LDS tile ----------------
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      if (partial) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if ((pi + h) * PS + 4 * g4 + j >= kv_len) r.v[h][j] = zero16();
-        }
-      }
-#pragma unroll
-      for (int e2 = 0; e2 < 4; ++e2) {
-        const uint32_t w0 = r.v[h][0].w[e2], w1 = r.v[h][1].w[e2], w2 = r.v[h][2].w[e2], w3 = r.v[h][3].w[e2];
-        uint2 even, odd;
-        even.x = (w0 & 0xffffu) | (w1 << 16);
-        even.y = (w2 & 0xffffu) | (w3 << 16);
-        odd.x = (w0 >> 16) | (w1 & 0xffff0000u);
-        odd.y = (w2 >> 16) | (w3 & 0xffff0000u);
-        *reinterpret_cast<uint2*>(Vt + (c16 * 8 + 2 * e2) * VROW + h * 16 + 4 * g4) = even;
-        *reinterpret_cast<uint2*>(Vt + (c16 * 8 + 2 * e2 + 1) * VROW + h * 16 + 4 * g4) = odd;
-      }
-    }
     // ---- S^T = K Q^T for both pages ---------------------------------------------------------
     float4_t s[2];
 #pragma unroll
@@ -412,29 +411,26 @@ __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int
         pf[h * 4 + j] = static_cast<half_t>(pj);
       }
     }
-    // the LDS tile is written and read by this wave only: order the two without a block barrier
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     // ---- O^T += V^T P^T: contraction slot g4*8 + i <-> page i/4, token 4*g4 + i%4 ------------
+    // The tile is written (by the copies) and read by this wave only: the copies are done when
+    // vmcnt reaches 0, and the reads below are done before the MFMAs that use them are issued,
+    // which is before the next step's copies in program order.
+    wait_vmcnt<0>();
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
-      const half_t* vrow = Vt + (db * 16 + c16) * VROW + 4 * g4;
-      const half4_t lo = *reinterpret_cast<const half4_t*>(vrow);
-      const half4_t hi = *reinterpret_cast<const half4_t*>(vrow + 16);
+      const half_t* vb = Vt + v_lane_off + (((db * 2 + v_piece) ^ v_swz) * 8);
+      const half4_t lo = lds_read_tr16(vb);
+      const half4_t hi = lds_read_tr16(vb + PS * D);
       half8_t a;
       a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
       a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
       o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pf, o[db], 0, 0, 0);
     }
-    // next step's LDS writes must not overtake these reads
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
   };
 
   // No software pipelining: three waves per SIMD (twelve per CU, each with 16 KiB of loads in
-  // flight while it waits) hide the load latency; a second register buffer costs occupancy and
-  // measured slower.
+  // flight while it waits) hide the load latency; four per SIMD measured 4 % slower (more page
+  // streams at once than the memory system likes), two about the same.
   Regs ra;
   for (int pi = page_lo + 2 * wave; pi < page_hi; pi += 8) {
     issue(pi, ra);
