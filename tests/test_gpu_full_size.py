@@ -85,6 +85,17 @@ def test_decode_full_size_properties(name, batch, lo, hi, hq, pool):
     assert_close(host(out8), host(out128), atol=2e-3, rtol=2e-3, what=f"{name} chunk 8 vs 128")
     assert_close(host(lse8), host(lse128), atol=1e-3, rtol=1e-5, what=f"{name} lse chunk 8 vs 128")
     assert_close(host(out), host(out128), atol=2e-3, rtol=2e-3, what=f"{name} default chunk vs 128")
+    # the chunk merge done by the last workgroup of each (sequence, kv head) against the same
+    # arithmetic in a second kernel: bit-identical, every time (a stale read of another
+    # workgroup's partial state would show here)
+    os.environ["TVMKV_DECODE_SEPARATE_MERGE"] = "1"
+    try:
+        out_sep, lse_sep = _decode(q, pages, t)
+    finally:
+        os.environ.pop("TVMKV_DECODE_SEPARATE_MERGE", None)
+    for _ in range(20):
+        out_f, lse_f = _decode(q, pages, t)
+        assert torch.equal(out_f, out_sep) and torch.equal(lse_f, lse_sep), f"{name}: fused merge differs"
     # constant values come back unchanged
     feat = (torch.arange(128, device=DEV, dtype=torch.float32) / 64 - 1).to(F16)
     pages[:, 1] = feat

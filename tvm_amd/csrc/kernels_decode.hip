@@ -41,6 +41,8 @@ struct DecodeParams {
   float* lse;
   float* part_o;   // (slots, h_q, D) fp32, unnormalised, relative to part_ml[..][0]
   float* part_ml;  // (slots, h_q, 2) fp32: running max m, running sum l
+  int* arrivals;   // (batch, h_kv) chunk workgroups that have delivered their partial state; all zero
+                   // between calls (fused merge of decode_mfma_kernel), or NULL
   int batch_size;
   int h_q;
   int h_kv;
@@ -259,6 +261,99 @@ __global__ __launch_bounds__(256) void decode_splitkv_kernel(DecodeParams p) {
   }
 }
 
+// Merge of the per-chunk partial states of one (sequence, query head) row by one wavefront.
+// Lane c first fetches (m, l) of chunk c, a wave reduction gives the common maximum and the total
+// sum, and every lane keeps the rescale factor of "its" chunk; the second pass streams the partial
+// outputs (each lane owns D/64 features) with the factor broadcast by shuffle, loads of several
+// chunks in flight at once.
+//
+// COHERENT: the partial states were written by other workgroups of the SAME kernel, possibly on
+// another XCD (each XCD has its own L2): they are written with device-scope stores (write-through)
+// and must be read with device-scope loads, which do not hit lines another XCD may have changed.
+__device__ __forceinline__ float load_partial(const float* ptr, bool coherent) {
+  return coherent ? __hip_atomic_load(ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *ptr;
+}
+__device__ __forceinline__ void store_partial(float* ptr, float v) {
+  __hip_atomic_store(ptr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int D, bool COHERENT>
+__device__ __forceinline__ void merge_row(const DecodeParams& p, int b, int hq, int nchunks, int lane) {
+  constexpr int EPL = D / 64;  // features per lane
+  const int64_t row = static_cast<int64_t>(b) * p.h_q + hq;
+  half_t* out = p.output + row * D + lane * EPL;
+  const int s0 = slot_begin(p.page_indptr, b, p.chunk_pages);
+  float mx = kNegInit, lsum = 0.f;
+  float acc[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
+  for (int c0 = 0; c0 < nchunks; c0 += 64) {
+    const int c = c0 + lane;
+    float m_c = kNegInit, l_c = 0.f;
+    if (c < nchunks) {
+      const float* ml = p.part_ml + (static_cast<int64_t>(s0 + c) * p.h_q + hq) * 2;
+      m_c = load_partial(ml, COHERENT);
+      l_c = load_partial(ml + 1, COHERENT);
+    }
+    float mx_new = m_c;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx_new = fmaxf(mx_new, __shfl_xor(mx_new, off, 64));
+    mx_new = fmaxf(mx_new, mx);
+    const float rescale_old = fast_exp2(mx - mx_new);
+    const float sc = fast_exp2(m_c - mx_new);
+    float lpart = l_c * sc;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) lpart += __shfl_xor(lpart, off, 64);
+    lsum = lsum * rescale_old + lpart;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[e] *= rescale_old;
+    mx = mx_new;
+    const int n_here = min(64, nchunks - c0);
+    const float* po = p.part_o + (static_cast<int64_t>(s0 + c0) * p.h_q + hq) * D + lane * EPL;
+    const int64_t stride = static_cast<int64_t>(p.h_q) * D;
+#pragma unroll 8
+    for (int k = 0; k < n_here; ++k) {
+      const float w = __shfl(sc, k, 64);
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) acc[e] = fmaf(load_partial(po + k * stride + e, COHERENT), w, acc[e]);
+    }
+  }
+  const float denom = lsum + fast_exp2(kNegInit - mx);
+  const float inv = 1.0f / denom;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) out[e] = static_cast<half_t>(acc[e] * inv);
+  if (lane == 0) p.lse[row] = mx + fast_log2(denom);
+}
+
+// The empty-KV answer out = 0, lse = -5e4 (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:129-130,173-176).
+template <int D>
+__device__ __forceinline__ void empty_row(const DecodeParams& p, int b, int hq, int lane) {
+  constexpr int EPL = D / 64;
+  const int64_t row = static_cast<int64_t>(b) * p.h_q + hq;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) p.output[row * D + lane * EPL + e] = static_cast<half_t>(0.f);
+  if (lane == 0) p.lse[row] = kNegInit;
+}
+
+// Stand-alone merge for the kernels that do not merge themselves: one wavefront per (sequence,
+// query head), four per block.  Sequences with one chunk were finished by the main kernel.
+template <int D>
+__global__ __launch_bounds__(256) void decode_merge_kernel(DecodeParams p, int total_rows) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // (b, hq) flattened
+  if (row >= total_rows) return;
+  const int b = row / p.h_q;
+  const int hq = row % p.h_q;
+  const int npages = p.page_indptr[b + 1] - p.page_indptr[b];
+  const int nchunks = (npages + p.chunk_pages - 1) / p.chunk_pages;
+  if (nchunks == 1) return;
+  if (nchunks == 0) {
+    empty_row<D>(p, b, hq, lane);
+    return;
+  }
+  merge_row<D, false>(p, b, hq, nchunks, lane);
+}
+
 // ------------------------------------------------------------------------------------------
 // MFMA variant for head_dim 128 (any GQA group up to 16).
 //
@@ -291,6 +386,7 @@ __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int
   __shared__ __attribute__((aligned(16))) half_t Vt_all[4][DM_VTILE];
   __shared__ float sm_m[4][16];
   __shared__ float sm_l[4][16];
+  __shared__ int sm_last;
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -311,7 +407,12 @@ __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int
   const int npages = p.page_indptr[b + 1] - pbeg;
   const int chunk = slot - slot_begin(p.page_indptr, b, cp);
   const int nchunks = (npages + cp - 1) / cp;
-  if (chunk >= nchunks) continue;  // spare slot (uniform over the workgroup)
+  if (chunk >= nchunks) {  // spare slot (uniform over the workgroup)
+    if (p.arrivals != nullptr && npages == 0 && chunk == 0) {  // a sequence without pages: nobody else answers for it
+      for (int g = wave; g < group; g += 4) empty_row<D>(p, b, kvh * group + g, lane);
+    }
+    continue;
+  }
   const int kv_len = (npages - 1) * PS + p.last_page_len[b];
   const int page_lo = chunk * cp;
   const int page_hi = min(page_lo + cp, npages);
@@ -475,84 +576,34 @@ __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int
       p.output[(static_cast<int64_t>(b) * p.h_q + hq) * D + d] = static_cast<half_t>(acc / denom);
       if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = mx + fast_log2(denom);
     } else {
-      p.part_o[(static_cast<int64_t>(slot) * p.h_q + hq) * D + d] = acc;
+      store_partial(p.part_o + (static_cast<int64_t>(slot) * p.h_q + hq) * D + d, acc);
       if (d == 0) {
-        p.part_ml[(static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 0] = mx;
-        p.part_ml[(static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 1] = lt;
+        store_partial(p.part_ml + (static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 0, mx);
+        store_partial(p.part_ml + (static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 1, lt);
       }
+    }
+  }
+  // Fused chunk merge: the workgroup that delivers the last partial state of a (sequence, kv head)
+  // merges them all.  No device-scope fences (on this chip they write back and invalidate a whole
+  // L2 and made the kernel 2-4 x slower): the partial states are written with device-scope stores,
+  // every wave waits until its own have completed, the barrier collects the waves, one thread
+  // counts the workgroup in with a device-scope atomic, and the workgroup that completes the count
+  // reads the states with device-scope loads.  The counter is reset for the next call.
+  if (p.arrivals != nullptr && !single_chunk) {
+    wait_vmcnt<0>();
+    __syncthreads();
+    if (tid == 0) {
+      sm_last = __hip_atomic_fetch_add(p.arrivals + b * p.h_kv + kvh, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                nchunks - 1;
+    }
+    __syncthreads();
+    if (sm_last) {
+      for (int g = wave; g < group; g += 4) merge_row<D, true>(p, b, kvh * group + g, nchunks, lane);
+      if (tid == 0) __hip_atomic_store(p.arrivals + b * p.h_kv + kvh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
   __syncthreads();  // the merge buffers are the next item's V tiles
   }  // items
-}
-
-// Merge of the per-chunk partial states.  One wavefront per (sequence, query head), four per
-// block.  Lane c first fetches (m, l) of chunk c, a wave reduction gives the common maximum and
-// the total sum, and every lane keeps the rescale factor of "its" chunk; the second pass streams
-// the partial outputs (each lane owns D/64 features) with the factor broadcast by shuffle, loads
-// of several chunks in flight at once.  Sequences with one chunk were finished by the main
-// kernel; sequences without pages get the empty-KV answer out = 0, lse = -5e4
-// (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:129-130,173-176).
-template <int D>
-__global__ __launch_bounds__(256) void decode_merge_kernel(DecodeParams p, int total_rows) {
-  constexpr int EPL = D / 64;  // features per lane
-  const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // (b, hq) flattened
-  if (row >= total_rows) return;
-  const int b = row / p.h_q;
-  const int hq = row % p.h_q;
-  const int cp = p.chunk_pages;
-  const int npages = p.page_indptr[b + 1] - p.page_indptr[b];
-  const int nchunks = (npages + cp - 1) / cp;
-  if (nchunks == 1) return;
-  half_t* out = p.output + static_cast<int64_t>(row) * D + lane * EPL;
-  if (nchunks == 0) {
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) out[e] = static_cast<half_t>(0.f);
-    if (lane == 0) p.lse[row] = kNegInit;
-    return;
-  }
-  const int s0 = slot_begin(p.page_indptr, b, cp);
-  float mx = kNegInit, lsum = 0.f;
-  float acc[EPL];
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
-  for (int c0 = 0; c0 < nchunks; c0 += 64) {
-    const int c = c0 + lane;
-    float m_c = kNegInit, l_c = 0.f;
-    if (c < nchunks) {
-      const float2 ml = *reinterpret_cast<const float2*>(p.part_ml + (static_cast<int64_t>(s0 + c) * p.h_q + hq) * 2);
-      m_c = ml.x;
-      l_c = ml.y;
-    }
-    float mx_new = m_c;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx_new = fmaxf(mx_new, __shfl_xor(mx_new, off, 64));
-    mx_new = fmaxf(mx_new, mx);
-    const float rescale_old = fast_exp2(mx - mx_new);
-    const float sc = fast_exp2(m_c - mx_new);
-    float lpart = l_c * sc;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) lpart += __shfl_xor(lpart, off, 64);
-    lsum = lsum * rescale_old + lpart;
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) acc[e] *= rescale_old;
-    mx = mx_new;
-    const int n_here = min(64, nchunks - c0);
-    const float* po = p.part_o + (static_cast<int64_t>(s0 + c0) * p.h_q + hq) * D + lane * EPL;
-    const int64_t stride = static_cast<int64_t>(p.h_q) * D;
-#pragma unroll 8
-    for (int k = 0; k < n_here; ++k) {
-      const float w = __shfl(sc, k, 64);
-#pragma unroll
-      for (int e = 0; e < EPL; ++e) acc[e] = fmaf(po[k * stride + e], w, acc[e]);
-    }
-  }
-  const float denom = lsum + fast_exp2(kNegInit - mx);
-  const float inv = 1.0f / denom;
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) out[e] = static_cast<half_t>(acc[e] * inv);
-  if (lane == 0) p.lse[row] = mx + fast_log2(denom);
 }
 
 // ---- per-device workspace for the partial states, grown on demand --------------------------
@@ -561,6 +612,8 @@ struct Workspace {
   size_t bytes = 0;
 };
 static Workspace g_workspace[64];
+
+constexpr size_t kArrivalBytes = 256 * 1024;  // the first bytes of the workspace: arrival counters, zero between calls
 
 static void* get_workspace(size_t bytes) {
   int dev = 0;
@@ -577,13 +630,14 @@ static void* get_workspace(size_t bytes) {
     size_t want = bytes + bytes / 2;
     HIP_CHECK(hipMalloc(&ws.ptr, want));
     ws.bytes = want;
+    HIP_CHECK(hipMemset(ws.ptr, 0, kArrivalBytes));
   }
   return ws.ptr;
 }
 
 // Pages per chunk from shapes only: aim at ~8K workgroups, keep a chunk between 4 and 64 pages.
 static int pick_chunk_pages(int64_t nnz_pages, int h_kv) {
-  static const char* forced = getenv("TVMKV_DECODE_CHUNK_PAGES");  // tuning aid
+  const char* forced = getenv("TVMKV_DECODE_CHUNK_PAGES");  // tuning aid, read per call
   if (forced != nullptr && atoi(forced) >= 8 && atoi(forced) % 8 == 0) return atoi(forced);
   // ~2300 work items = three rounds of 3 workgroups x 256 CUs; every item pays ~2 us of fixed
   // cost (locating its sequence, q, the cross-wave merge), so chunks should not be smaller than
@@ -647,9 +701,10 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many chunks";
   const size_t part_o_bytes = static_cast<size_t>(slots) * h_q * d * sizeof(float);
   const size_t part_ml_bytes = static_cast<size_t>(slots) * h_q * 2 * sizeof(float);
-  char* ws = static_cast<char*>(get_workspace(part_o_bytes + part_ml_bytes));
-  p.part_o = reinterpret_cast<float*>(ws);
-  p.part_ml = reinterpret_cast<float*>(ws + part_o_bytes);
+  char* ws = static_cast<char*>(get_workspace(kArrivalBytes + part_o_bytes + part_ml_bytes));
+  p.part_o = reinterpret_cast<float*>(ws + kArrivalBytes);
+  p.part_ml = reinterpret_cast<float*>(ws + kArrivalBytes + part_o_bytes);
+  p.arrivals = nullptr;
 
   const dim3 grid(static_cast<unsigned>(slots), h_kv);
   const int group = h_q / h_kv;
@@ -664,10 +719,19 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
     if (wgs_env != nullptr && atoi(wgs_env) > 0) {
       grid_x = std::min<int64_t>(num_items, static_cast<int64_t>(compute_units()) * atoi(wgs_env));
     }
+    // the chunk merge is done by the last workgroup of each (sequence, kv head) when the arrival
+    // counters fit their region; TVMKV_DECODE_SEPARATE_MERGE=1 keeps the second kernel (tuning aid)
+    const char* sep_env = getenv("TVMKV_DECODE_SEPARATE_MERGE");  // read per call: tests switch it
+    const bool fused = static_cast<size_t>(batch_size) * h_kv * sizeof(int) <= kArrivalBytes &&
+                       !(sep_env != nullptr && atoi(sep_env) != 0);
+    if (fused) p.arrivals = reinterpret_cast<int*>(ws);
     hipLaunchKernelGGL(decode_mfma_kernel, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group,
                        static_cast<int>(num_items));
-    KV_LAUNCH_CHECK();
-    hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
+    if (!fused) {
+      KV_LAUNCH_CHECK();
+      hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p,
+                         batch_size * h_q);
+    }
   } else if (d == 128) {
     launch_decode<128, 16>(p, group, grid, s);
     KV_LAUNCH_CHECK();
