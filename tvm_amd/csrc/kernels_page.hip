@@ -24,6 +24,9 @@ struct RopeDivisors {
   float v[kMaxHalfDim];
 };
 
+// One workgroup per token: the D/2 (cos, sin) pairs of the token's position are computed once
+// (they are the same for every head; the precise sinf/cosf with their range reduction are by far
+// the most expensive part) and shared through LDS, then all heads of the token are streamed.
 template <int D>
 __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restrict__ qkv,
                                                          const int32_t* __restrict__ position_map,
@@ -32,42 +35,50 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
                                                          int num_kv_heads, int apply_rope, float scale,
                                                          RopeDivisors div) {
   constexpr int kThreadsPerHead = D / 16;  // a thread owns d-range [8c, 8c+8) and its partner +D/2
+  __shared__ float cs_lds[D / 2];
+  __shared__ float sn_lds[D / 2];
+  const int64_t s = blockIdx.x;  // token
   const int fused_heads = num_q_heads + 2 * num_kv_heads;
-  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int c = gid % kThreadsPerHead;
-  const int64_t row = gid / kThreadsPerHead;  // (token, fused head)
-  if (row >= seq_len * fused_heads) return;
-  const int64_t s = row / fused_heads;
-  const int h = row % fused_heads;
-  const half_t* src = qkv + row * D + c * 8;
-  Vec16 lo = ld16(src);
-  Vec16 hi = ld16(src + D / 2);
-  half_t* dst;
-  if (h < num_q_heads) {
-    dst = q + (s * num_q_heads + h) * D;
-  } else if (h < num_q_heads + num_kv_heads) {
-    dst = k + (s * num_kv_heads + (h - num_q_heads)) * D;
-  } else {
-    dst = v + (s * num_kv_heads + (h - num_q_heads - num_kv_heads)) * D;
-  }
-  if (apply_rope > 0 && h < num_q_heads + num_kv_heads) {
+  if (apply_rope > 0) {
     const float pos_scaled = static_cast<float>(position_map[s]) * scale;
-    Vec16 out_lo, out_hi;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float freq = pos_scaled / div.v[c * 8 + e];
-      const float cs = cosf(freq);
-      const float sn = sinf(freq);
-      const float xl = static_cast<float>(lo.h[e]);
-      const float xh = static_cast<float>(hi.h[e]);
-      out_lo.h[e] = static_cast<half_t>(cs * xl + sn * (-xh));
-      out_hi.h[e] = static_cast<half_t>(cs * xh + sn * xl);
+    for (int i = threadIdx.x; i < D / 2; i += 256) {
+      const float freq = pos_scaled / div.v[i];
+      cs_lds[i] = cosf(freq);
+      sn_lds[i] = sinf(freq);
     }
-    lo = out_lo;
-    hi = out_hi;
+    __syncthreads();
   }
-  st16(dst + c * 8, lo);
-  st16(dst + D / 2 + c * 8, hi);
+  for (int task = threadIdx.x; task < fused_heads * kThreadsPerHead; task += 256) {
+    const int c = task % kThreadsPerHead;
+    const int h = task / kThreadsPerHead;
+    const half_t* src = qkv + (s * fused_heads + h) * D + c * 8;
+    Vec16 lo = ld16(src);
+    Vec16 hi = ld16(src + D / 2);
+    half_t* dst;
+    if (h < num_q_heads) {
+      dst = q + (s * num_q_heads + h) * D;
+    } else if (h < num_q_heads + num_kv_heads) {
+      dst = k + (s * num_kv_heads + (h - num_q_heads)) * D;
+    } else {
+      dst = v + (s * num_kv_heads + (h - num_q_heads - num_kv_heads)) * D;
+    }
+    if (apply_rope > 0 && h < num_q_heads + num_kv_heads) {
+      Vec16 out_lo, out_hi;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float cs = cs_lds[c * 8 + e];
+        const float sn = sn_lds[c * 8 + e];
+        const float xl = static_cast<float>(lo.h[e]);
+        const float xh = static_cast<float>(hi.h[e]);
+        out_lo.h[e] = static_cast<half_t>(cs * xl + sn * (-xh));
+        out_hi.h[e] = static_cast<half_t>(cs * xh + sn * xl);
+      }
+      lo = out_lo;
+      hi = out_hi;
+    }
+    st16(dst + c * 8, lo);
+    st16(dst + D / 2 + c * 8, hi);
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -286,10 +297,10 @@ int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void
   for (int i = 0; i < head_dim / 2; ++i) {
     div.v[i] = powf(theta, static_cast<float>((i * 2) % head_dim) / static_cast<float>(head_dim));
   }
-  const int64_t threads = seq_len * (num_q_heads + 2 * num_kv_heads) * (head_dim / 16);
+  KV_CHECK(seq_len < (int64_t{1} << 31)) << "fused_rope: too many tokens for one launch";
   const float scale = static_cast<float>(rope_scale);
   auto launch = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid_for(threads), dim3(256), 0, as_stream(stream), static_cast<const half_t*>(qkv),
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(seq_len)), dim3(256), 0, as_stream(stream), static_cast<const half_t*>(qkv),
                        position_map, static_cast<half_t*>(q), static_cast<half_t*>(k), static_cast<half_t*>(v),
                        seq_len, num_q_heads, num_kv_heads, static_cast<int>(apply_rope > 0), scale, div);
   };
