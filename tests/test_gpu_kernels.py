@@ -190,12 +190,53 @@ def test_decode_ignores_garbage_beyond_last_page_len():
     assert_close(host(go), eo, what="decode with NaN padding")
 
 
+@pytest.mark.parametrize("rotary", [0, 1])
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (8, 8), (16, 1)])
+def test_decode_sliding_window_cache_and_inline_rope(hq, hkv, rotary):
+    """length_info (3, B) = [last_page_len; window offset; sink size] and rotary_mode = 1."""
+    from tests.test_oracle_kernels import SLIDING_SPEC, sliding_case
+    rng = np.random.default_rng(22)
+    d = 128
+    spec = SLIDING_SPEC + [(2300, 8, 40)]  # several chunks
+    pages, indptr, values, info, k_log, _ = sliding_case(rng, spec, hkv, d, npages=260)
+    b = len(spec)
+    q = rng.standard_normal((b, hq, d)).astype(F16)
+    k_off = rng.integers(0, 300, size=b).astype(np.int32)
+    q_pos = (k_off + np.array([len(k) for k in k_log]) - 1).astype(np.int32)
+    eo, el = np.zeros((b, hq, d), F16), np.zeros((b, hq), np.float32)
+    ok.decode(q, pages, indptr, values, info, k_off, q_pos, eo, el, rotary, 1.0, 1e4, d ** -0.5)
+    go = torch.full((b, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((b, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_decode_paged_kv(dev(q), dev(pages), i32(indptr), i32(values), i32(info), i32(k_off), i32(q_pos), go, gl,
+                            rotary, 1.0, 1e4, d ** -0.5)
+    assert_close(host(go), eo, what="sliding decode out")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="sliding decode lse")
+
+
+def test_decode_inline_rope_plain_cache_and_scaled_positions():
+    rng = np.random.default_rng(23)
+    hq, hkv, d = 32, 8, 128
+    pages, indptr, values, last, ks, vs = build_paged_kv(rng, [5, 130, 1000], 80, hkv, 16, d)
+    q = rng.standard_normal((3, hq, d)).astype(F16)
+    k_off = np.array([0, 7, 3000], np.int32)
+    q_pos = np.array([4, 136, 3999], np.int32)
+    for scale, theta in ((1.0, 1e4), (0.5, 5e5)):
+        eo, el = np.zeros((3, hq, d), F16), np.zeros((3, hq), np.float32)
+        ok.decode(q, pages, indptr, values, last, k_off, q_pos, eo, el, 1, scale, theta, d ** -0.5)
+        go = torch.zeros((3, hq, d), dtype=torch.float16, device=DEV)
+        gl = torch.zeros((3, hq), dtype=torch.float32, device=DEV)
+        K.batch_decode_paged_kv(dev(q), dev(pages), i32(indptr), i32(values), i32(last), i32(k_off), i32(q_pos), go,
+                                gl, 1, scale, theta, d ** -0.5)
+        assert_close(host(go), eo, what=f"inline rope decode out, scale {scale}")
+        assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"inline rope decode lse, scale {scale}")
+
+
 def test_decode_rejects_what_is_not_built():
-    t = torch.zeros((1, 8, 128), dtype=torch.float16, device=DEV)
-    pages = torch.zeros((2, 2, 2, 16, 128), dtype=torch.float16, device=DEV)
+    t = torch.zeros((1, 8, 64), dtype=torch.float16, device=DEV)
+    pages = torch.zeros((2, 2, 2, 16, 64), dtype=torch.float16, device=DEV)
     lse = torch.zeros((1, 8), dtype=torch.float32, device=DEV)
     one = i32([0, 1])
-    with pytest.raises(KVError, match="inline RoPE") as info:
+    with pytest.raises(KVError, match="inline RoPE") as info:  # head_dim 64 has no inline-RoPE kernel
         K.batch_decode_paged_kv(t, pages, one, i32([0]), i32([1]), i32([0]), i32([0]), t, lse, 1, 1.0, 1e4, 1.0)
     assert info.value.code == -2
 

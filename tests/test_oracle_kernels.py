@@ -255,6 +255,60 @@ def test_inline_rope_equals_rope_then_attend():
 
 
 # ----------------------------------------------------------------------------- merge
+def test_layer_sliding_window_mask_known_answer():
+    """The reference's own known-answer vector for the paged prefill kernel built with
+    sliding_window_size = 3 (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_tir.py:98-156):
+    zero queries, V = 1, 3, 5 in the first three slots, two query rows -> out[:, 0, 0] = [4, 5]."""
+    hq, hkv, d = 4, 2, 64
+    q = np.zeros((2, hq, d), F16)
+    pages = np.zeros((1, 2, hkv, 16, d), F16)
+    for position, value in enumerate([1, 3, 5]):
+        pages[0, 1, :, position, :] = value
+    out, lse = np.zeros_like(q), np.zeros((2, hq), np.float32)
+    ok.prefill_paged(q, np.array([0, 2], np.int32), pages, np.array([0, 1], np.int32), np.array([0], np.int32),
+                     np.array([[3], [0], [0]], np.int32), np.array([0], np.int32), np.array([3, 4], np.int32),
+                     out, lse, 1, 0, 1.0, 1e4, d ** -0.5, sliding_window_size=3)
+    assert_close(out[:, 0, 0], np.array([4, 5], F16), atol=1e-3, rtol=1e-3, what="sliding window known answer")
+    assert np.all(out == out[:, :1, :1])
+
+
+def sliding_case(rng, spec, hkv, d, ps=16, npages=96):
+    """spec: list of (physical_len, sink, window_offset).  Returns the page pool, tables, the (3, B)
+    length_info and, per sequence, the K/V rows in LOGICAL order (sink tokens, then the window)."""
+    pages, indptr, values, last, ks, vs = build_paged_kv(rng, [s[0] for s in spec], npages, hkv, ps, d)
+    info = np.array([last, [s[2] for s in spec], [s[1] for s in spec]], np.int32)
+    k_log = [np.concatenate([k[:sink], k[off:]]) for k, (n, sink, off) in zip(ks, spec)]
+    v_log = [np.concatenate([v[:sink], v[off:]]) for v, (n, sink, off) in zip(vs, spec)]
+    return pages, indptr, values, info, k_log, v_log
+
+
+SLIDING_SPEC = [(100, 4, 20), (257, 0, 0), (700, 16, 48), (33, 2, 2), (17, 0, 5), (1, 0, 0), (64, 16, 32)]
+
+
+def test_sliding_cache_decode_is_attention_over_sink_plus_window():
+    """length_info (3, B): the kernel attends to the first `sink` tokens and to the tokens from
+    `window_offset` on (python/tvm/relax/frontend/nn/llm/_kernel_common.py:155-170); with inline
+    RoPE the key with logical index t sits at position k_rope_pos_offset + t."""
+    rng = np.random.default_rng(21)
+    hq, hkv, d = 8, 2, 128
+    pages, indptr, values, info, k_log, v_log = sliding_case(rng, SLIDING_SPEC, hkv, d)
+    b = len(SLIDING_SPEC)
+    q = rng.standard_normal((b, hq, d)).astype(F16)
+    k_off = rng.integers(0, 300, size=b).astype(np.int32)
+    q_pos = (k_off + np.array([len(k) for k in k_log]) - 1).astype(np.int32)
+    for rotary in (0, 1):
+        out, lse = np.zeros((b, hq, d), F16), np.zeros((b, hq), np.float32)
+        ok.decode(q, pages, indptr, values, info, k_off, q_pos, out, lse, rotary, 1.0, 1e4, d ** -0.5)
+        for i in range(b):
+            kk, qq = k_log[i], q[i:i + 1]
+            if rotary:
+                kk = cf.apply_rotary(kk, k_off[i] + np.arange(len(kk))).astype(F16)
+                qq = cf.apply_rotary(qq, [q_pos[i]]).astype(F16)
+            eo, el = cf.attention(qq, kk, v_log[i], d ** -0.5, causal=False)
+            assert_close(out[i], eo[0], atol=3e-3, rtol=3e-3, what=f"sliding decode out seq {i} rotary {rotary}")
+            assert_close(lse[i], el[0], atol=2e-3, rtol=1e-4, what=f"sliding decode lse seq {i} rotary {rotary}")
+
+
 def test_merge_closed_form_and_special_cases():
     rng = np.random.default_rng(12)
     n, h, d = 6, 4, 64

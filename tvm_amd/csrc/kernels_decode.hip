@@ -25,6 +25,7 @@
 // which always holds ceil(npages_b/CP) chunks; a workgroup finds its sequence by binary search
 // on page_indptr, so the grid size depends on shapes only (floor(nnz_pages/CP) + B slots).
 #include <algorithm>
+#include <cmath>
 #include <cstdlib>
 
 #include "kernels_common.cuh"
@@ -41,6 +42,13 @@ struct DecodeParams {
   float* lse;
   float* part_o;   // (slots, h_q, D) fp32, unnormalised, relative to part_ml[..][0]
   float* part_ml;  // (slots, h_q, 2) fp32: running max m, running sum l
+  // extended form (decode_mfma_kernel<true>): sliding-window cache and inline RoPE
+  const int32_t* window_offset;   // (B) physical index of the first token of the window, or NULL
+  const int32_t* sink_size;       // (B) attention-sink tokens kept at the front, or NULL
+  const int32_t* k_rope_pos_offset;  // (B) position of logical token 0 (inline RoPE)
+  const int32_t* q_rope_position;    // (B) position of the query token (inline RoPE)
+  int rotary;                     // 1: rotate q and k inside the kernel
+  float rope_scale;
   int* arrivals;   // (batch, h_kv) chunk workgroups that have delivered their partial state; all zero
                    // between calls (fused merge of decode_mfma_kernel), or NULL
   int batch_size;
@@ -380,7 +388,45 @@ constexpr int DM_VTILE = 2 * DM_PS * DM_D;  // halfs of a wave's V tile: two pag
 // a 256-byte bank line.
 __device__ __forceinline__ int dm_swizzle(int row) { return (row & 7) << 1; }
 
-__global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int group, int num_items) {
+// theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
+struct DecodeRopeDivisors {
+  float v[DM_D / 2];
+};
+
+// sin and cos of an fp32 angle of any size: two-constant Cody-Waite reduction to [-pi, pi], then
+// the hardware functions (which take revolutions).  Absolute error ~1e-6 for |x| up to ~1e5.
+__device__ __forceinline__ void sincos_reduced(float x, float& sn, float& cs) {
+  const float k = rintf(x * 0.15915494309189535f);
+  float r = fmaf(-k, 6.2831854820251465f, x);    // fp32(2 pi)
+  r = fmaf(-k, -1.7484555314695172e-7f, r);      // 2 pi - fp32(2 pi)
+  const float t = r * 0.15915494309189535f;
+  sn = __builtin_amdgcn_sinf(t);
+  cs = __builtin_amdgcn_cosf(t);
+}
+
+// Rotate-half RoPE of the features (f, f + D/2) held by one lane in two fragments, as the reference
+// does it (python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-127): fp32 math, one rounding to fp16.
+__device__ __forceinline__ void rope_pair(Vec16& lo, Vec16& hi, float pos_scaled, const float* div8) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float sn, cs;
+    sincos_reduced(pos_scaled / div8[i], sn, cs);
+    const float xl = static_cast<float>(lo.h[i]);
+    const float xh = static_cast<float>(hi.h[i]);
+    lo.h[i] = static_cast<half_t>(cs * xl + sn * (-xh));
+    hi.h[i] = static_cast<half_t>(cs * xh + sn * xl);
+  }
+}
+
+// EXT = false: plain cache, q and k already rotated (or no RoPE).  EXT = true adds the sliding-window
+// cache (length_info (3, B): the page table covers `sink` tokens at the front, evicted tokens up to
+// `window_offset`, then the window, python/tvm/relax/frontend/nn/llm/_kernel_common.py:155-170) and
+// inline RoPE (q at q_rope_position[b], the key with logical index t at k_rope_pos_offset[b] + t,
+// _decode_kernels.py:141-156).  Attention does not depend on the order of the keys, so the pages are
+// still walked in physical order; evicted tokens are masked and logical indices only feed RoPE.
+template <bool EXT>
+__global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodeParams p, int group, int num_items,
+                                                             DecodeRopeDivisors div) {
   constexpr int D = DM_D, PS = DM_PS;
   static_assert(DM_VTILE * sizeof(half_t) >= 16 * D * sizeof(float), "the merge buffer aliases the V tile");
   __shared__ __attribute__((aligned(16))) half_t Vt_all[4][DM_VTILE];
@@ -413,16 +459,34 @@ __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int
     }
     continue;
   }
-  const int kv_len = (npages - 1) * PS + p.last_page_len[b];
+  const int kv_len = (npages - 1) * PS + p.last_page_len[b];  // physical end of the cached tokens
   const int page_lo = chunk * cp;
   const int page_hi = min(page_lo + cp, npages);
+  // physical token t is attended to iff t < sink or win_lo <= t < kv_len
+  const int sink = EXT && p.sink_size != nullptr ? p.sink_size[b] : 0;
+  const int win_lo = EXT && p.window_offset != nullptr ? p.window_offset[b] : 0;
+  float divr[16];  // RoPE divisors of this lane's features ks*32 + g4*8 + i, ks = 0, 1
+  float k_pos0 = 0.f;
+  if (EXT && p.rotary) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) divr[i] = div.v[(i >> 3) * 32 + g4 * 8 + (i & 7)];
+    k_pos0 = static_cast<float>(p.k_rope_pos_offset[b]);
+  }
 
   // Q^T fragments (B operand): column = head c16 of the group, contraction slots = 8 features.
   half8_t qf[4];
   {
     const half_t* qrow = p.q + (static_cast<int64_t>(b) * p.h_q + kvh * group + c16) * D + g4 * 8;
+    Vec16 qv[4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) qf[ks] = c16 < group ? ld16(qrow + ks * 32).h8 : zero16().h8;
+    for (int ks = 0; ks < 4; ++ks) qv[ks] = c16 < group ? ld16(qrow + ks * 32) : zero16();
+    if (EXT && p.rotary) {
+      const float q_pos = static_cast<float>(p.q_rope_position[b]) * p.rope_scale;
+      rope_pair(qv[0], qv[2], q_pos, divr);
+      rope_pair(qv[1], qv[3], q_pos, divr + 8);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) qf[ks] = qv[ks].h8;
   }
   float4_t o[8];
 #pragma unroll
@@ -470,7 +534,21 @@ __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int
   };
 
   auto consume = [&](int pi, Regs& r) {
-    const bool partial = (pi + 2) * PS > kv_len;  // wave-uniform
+    // wave-uniform: some token of the two pages is not attended to (end of the sequence, evicted)
+    const bool partial = EXT ? !((pi * PS >= win_lo && (pi + 2) * PS <= kv_len) || (pi + 2) * PS <= sink)
+                             : (pi + 2) * PS > kv_len;
+    auto attended = [&](int t) { return EXT ? (t < sink || (t >= win_lo && t < kv_len)) : t < kv_len; };
+    if (EXT && p.rotary) {
+      // the key of this lane in page h is physical token (pi+h)*PS + c16; logical index = position
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int t = (pi + h) * PS + c16;
+        const int logical = t < sink ? t : t - win_lo + sink;
+        const float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
+        rope_pair(r.k[h][0], r.k[h][2], pos, divr);
+        rope_pair(r.k[h][1], r.k[h][3], pos, divr + 8);
+      }
+    }
     // ---- S^T = K Q^T for both pages ---------------------------------------------------------
     float4_t s[2];
 #pragma unroll
@@ -486,7 +564,7 @@ __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float v = s[h][j] * p.scale_log2;
-        if (partial) v = ((pi + h) * PS + 4 * g4 + j < kv_len) ? v : kNegInit;
+        if (partial) v = attended((pi + h) * PS + 4 * g4 + j) ? v : kNegInit;
         s[h][j] = v;
         mx = fmaxf(mx, v);
       }
@@ -507,7 +585,7 @@ __global__ __launch_bounds__(256, 3) void decode_mfma_kernel(DecodeParams p, int
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float pj = fast_exp2(s[h][j] - m_new);
-        if (partial) pj = ((pi + h) * PS + 4 * g4 + j < kv_len) ? pj : 0.f;
+        if (partial) pj = attended((pi + h) * PS + 4 * g4 + j) ? pj : 0.f;
         lsum += pj;
         pf[h * 4 + j] = static_cast<half_t>(pj);
       }
@@ -675,9 +753,10 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && nnz_pages >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_decode_paged_kv: bad shape";
-  KV_UNSUPPORTED(rotary_mode != 0) << "batch_decode_paged_kv: inline RoPE (rotary_mode=1) is not built; the "
-                                      "cache applies RoPE before the append (RoPE mode NORMAL) or not at all";
-  KV_UNSUPPORTED(sliding_window != 0) << "batch_decode_paged_kv: sliding-window length_info (3, B) is not built";
+  const bool ext = rotary_mode != 0 || sliding_window != 0;
+  KV_UNSUPPORTED(ext && !(d == 128 && h_q / h_kv <= 16))
+      << "batch_decode_paged_kv: inline RoPE (rotary_mode=1) and sliding-window length_info (3, B) are built "
+         "for head_dim 128 and GQA groups up to 16 only";
   KV_UNSUPPORTED(page_size != 16) << "batch_decode_paged_kv: page_size " << page_size << " is not built (16)";
   KV_UNSUPPORTED(d != 64 && d != 128) << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 128)";
   if (batch_size == 0) return TVMKV_OK;
@@ -689,7 +768,13 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
   p.pages = static_cast<const half_t*>(pages);
   p.page_indptr = page_indptr;
   p.page_values = page_values;
-  p.last_page_len = length_info;
+  p.last_page_len = length_info;  // row 0 of the (3, B) form
+  p.window_offset = sliding_window != 0 ? length_info + batch_size : nullptr;
+  p.sink_size = sliding_window != 0 ? length_info + 2 * static_cast<int64_t>(batch_size) : nullptr;
+  p.k_rope_pos_offset = k_rope_pos_offset;
+  p.q_rope_position = q_rope_position;
+  p.rotary = rotary_mode != 0;
+  p.rope_scale = static_cast<float>(rope_scale);
   p.output = static_cast<half_t*>(output);
   p.lse = lse;
   p.batch_size = batch_size;
@@ -725,8 +810,19 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
     const bool fused = static_cast<size_t>(batch_size) * h_kv * sizeof(int) <= kArrivalBytes &&
                        !(sep_env != nullptr && atoi(sep_env) != 0);
     if (fused) p.arrivals = reinterpret_cast<int*>(ws);
-    hipLaunchKernelGGL(decode_mfma_kernel, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group,
-                       static_cast<int>(num_items));
+    DecodeRopeDivisors div{};
+    if (p.rotary) {
+      KV_CHECK(k_rope_pos_offset && q_rope_position) << "batch_decode_paged_kv: inline RoPE needs the position arrays";
+      const float theta = static_cast<float>(rope_theta);
+      for (int i = 0; i < DM_D / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DM_D));
+    }
+    if (ext) {
+      hipLaunchKernelGGL(decode_mfma_kernel<true>, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group,
+                         static_cast<int>(num_items), div);
+    } else {
+      hipLaunchKernelGGL(decode_mfma_kernel<false>, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group,
+                         static_cast<int>(num_items), div);
+    }
     if (!fused) {
       KV_LAUNCH_CHECK();
       hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p,
