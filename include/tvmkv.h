@@ -84,8 +84,9 @@ int tvmkv_kv_cache_transpose_append_mla(void* pages, const void* kv_data, const 
  * (q, qo_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_offset, out, lse, causal,
  *  rotary_mode, rope_scale, rope_theta, sm_scale).
  * q (total_q, h_q, d_qk), k (total_kv, h_kv, d_qk), v (total_kv, h_kv, d_v),
- * out (total_q, h_q, d_v) fp16, lse (total_q, h_q) fp32 base-2.  rotary_mode must be 0 (RoPE
- * applied up front); 1 (inline RoPE) returns TVMKV_EUNSUPPORTED. */
+ * out (total_q, h_q, d_v) fp16, lse (total_q, h_q) fp32 base-2.  rotary_mode 0: q and k are used
+ * as they are; 1 (inline RoPE): q is rotated at q_rope_position[token], key t of sequence b at
+ * k_rope_pos_offset[b] + t (built for head dims 64 and 128). */
 int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const void* k, const void* v,
                                   const int32_t* kv_indptr, const int32_t* q_rope_position,
                                   const int32_t* k_rope_pos_offset, void* output, float* lse,
@@ -100,7 +101,11 @@ int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const 
  *  q_rope_position, out, lse, causal, rotary_mode, rope_scale, rope_theta, sm_scale).
  * length_info is (batch,) = last_page_len, or (3, batch) = [last_page_len; sliding_window_offset;
  * sink_size] when sliding_window != 0 (python/tvm/relax/frontend/nn/llm/_kernel_common.py:147-170).
- * kv_len = (npages-1)*page_size + last_page_len, 0 without pages. */
+ * kv_len = (npages-1)*page_size + last_page_len, 0 without pages; in the (3, batch) form the keys
+ * are the first sink_size cached tokens followed by those from sliding_window_offset on, and with
+ * causal != 0 and sliding_window_size > 0 query row r sees only the last sliding_window_size - r - 1
+ * keys (_kernel_common.py:138-144).  rotary_mode as for the ragged kernel, key positions counted
+ * over the keys as just defined. */
 int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const void* pages,
                                  const int32_t* page_indptr, const int32_t* page_values,
                                  const int32_t* length_info, const int32_t* k_rope_pos_offset,
@@ -117,7 +122,9 @@ int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const v
  * (q, pages, page_indptr, page_indices, length_info, k_rope_pos_offset, q_rope_position, out,
  *  lse, rotary_mode, rope_scale, rope_theta, sm_scale).
  * q/out (B, h_q, d) fp16, lse (B, h_q) fp32.  Split-KV across workgroups with a merge pass;
- * the partition count is derived from B and nnz_pages only (no host read of the page table). */
+ * the partition count is derived from B and nnz_pages only (no host read of the page table).
+ * The (3, batch) length_info and rotary_mode = 1 are built for head_dim 128 and GQA groups up to
+ * 16; other shapes return TVMKV_EUNSUPPORTED for them. */
 int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t* page_indptr,
                                 const int32_t* page_values, const int32_t* length_info,
                                 const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,

@@ -47,6 +47,9 @@ class GpuCache:
     def fork_sequence(self, parent, child, pos=-1):
         gf("vm.builtin.kv_state_fork_sequence")(self.cache, parent, child, pos)
 
+    def enable_sliding_window_for_seq(self, sid, window, sink):
+        gf("vm.builtin.attention_kv_cache_enable_sliding_window_for_seq")(self.cache, sid, window, sink)
+
     def popn(self, sid, n):
         gf("vm.builtin.kv_state_popn")(self.cache, sid, n)
 

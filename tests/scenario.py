@@ -115,7 +115,30 @@ class Scenario:
                              what=f"attention output, layer {layer}, seq {sid}")
                 cursor += n
         cache.end_forward()
+        # the sliding window takes effect after the step: keep the attention sink and the newest tokens
+        # (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_cpu.py:566-590)
+        for sid in seq_ids:
+            window, sink = self.window.get(sid, (0, 0))
+            n = self.cached_k[sid].shape[1]
+            if window and n > window:
+                cut = sink + (n - window)
+                self.cached_k[sid] = np.concatenate([self.cached_k[sid][:, :sink], self.cached_k[sid][:, cut:]], axis=1)
+                self.cached_v[sid] = np.concatenate([self.cached_v[sid][:, :sink], self.cached_v[sid][:, cut:]], axis=1)
         self.verify_cached_kv(seq_ids)
+
+    def add_with_window(self, sid, window, sink):
+        self.cache.add_sequence(sid)
+        self.cache.enable_sliding_window_for_seq(sid, window, sink)
+        self.cached_k[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), np.float16)
+        self.cached_v[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), np.float16)
+        self.window[sid] = (window, sink)
+
+    def fork_with_window(self, parent, sid, pos, window, sink):
+        self.cache.fork_sequence(parent, sid, pos)
+        self.cache.enable_sliding_window_for_seq(sid, window, sink)
+        self.cached_k[sid] = self.cached_k[parent][:, :pos]
+        self.cached_v[sid] = self.cached_v[parent][:, :pos]
+        self.window[sid] = (window, sink)
 
     def remove(self, sid):
         self.cache.remove_sequence(sid)
@@ -217,3 +240,26 @@ def run_popn(sc):
         sc.remove(sid)
         sc.verify_cached_kv(list(range(sid + 1, 5)))
     assert sc.cache.empty()
+
+
+def run_sliding_window(sc):
+    """tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_cpu.py:912-955"""
+    for sid, (window, sink) in enumerate(zip([20, 25, 30, 35, 40], [6, 4, 8, 3, 7])):
+        sc.add_with_window(sid, window, sink)
+    batches = [[(0, 4)], [(1, 6)], [(2, 6), (3, 7), (4, 7)]]
+    batches += [[(0, 20), (1, 19), (2, 30), (3, 35), (4, 40)]]
+    batches += [[(0, 6), (1, 5), (2, 4), (3, 3), (4, 2)]]
+    batches += [[(i, 1) for i in range(5)]] * 20
+    for batch in batches:
+        sc.step(list(batch))
+
+
+def run_sliding_window_fork(sc):
+    """tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_cpu.py:958-1022"""
+    for sid, (window, sink) in enumerate(zip([30, 35, 40], [15, 20, 25])):
+        sc.add_with_window(sid, window, sink)
+    sc.step([(0, 12), (1, 18), (2, 28)])
+    sc.step([((3, 0, 10), 8), ((4, 1, -1), 20), ((5, 2, 18), 18)])
+    sc.step([(0, 9), (1, 15), (2, 4), (3, 10), (4, 3), (5, 7)])
+    sc.fork_with_window(3, 6, 18, 25, 24)
+    sc.step([(3, 10), (6, 12)])

@@ -142,11 +142,28 @@ def test_error_paths_on_the_device_cache():
     cache.add_sequence(1)
     with pytest.raises(tvm_amd.KVError, match="The KV cache is full"):
         cache.begin_forward([1], [80])
-    with pytest.raises(tvm_amd.KVError, match="not built"):  # sliding window forces inline RoPE
-        c2 = GpuCache([4, 64, 32, 16, 1], 1, 8, 2, 128, 128, rope_mode=1)
-        c2.add_sequence(0)
-        c2.begin_forward([0], [4])
-        attn(c2.cache, 0, 1.0, qkv, out)
+    # a sliding-window cache forces inline RoPE; the head_dim 64 decode kernel has none
+    c2 = GpuCache([4, 64, 32, 16, 1], 1, 8, 2, 64, 64, rope_mode=1)
+    c2.add_sequence(0)
+    qkv64 = torch.zeros((1, 12, 64), dtype=torch.float16, device=DEV)
+    out64 = torch.zeros((1, 8, 64), dtype=torch.float16, device=DEV)
+    c2.begin_forward([0], [1])
+    attn(c2.cache, 0, 1.0, qkv64, out64)  # nothing cached yet: the ragged prefill kernel alone
+    c2.end_forward()
+    c2.begin_forward([0], [1])
+    with pytest.raises(tvm_amd.KVError, match="inline RoPE"):
+        attn(c2.cache, 0, 1.0, qkv64, out64)
+
+
+@pytest.mark.parametrize("runner", [S.run_sliding_window, S.run_sliding_window_fork])
+def test_sliding_window_scenarios_on_the_gpu(runner):
+    """The reference's sliding-window tests (attention sinks, window trimming after every step,
+    forks inside the sink; tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_cpu.py:912-1022)
+    on the HIP cache: inline RoPE, length_info (3, B), prefill and decode kernels."""
+    layers, hq, hkv, d = 2, 8, 2, 128
+    cache = GpuCache([32, 2048, 512, 16, 1], layers, hq, hkv, d, d, rope_mode=S.ROPE_INLINE)
+    sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=S.ROPE_INLINE, seed=4)
+    runner(sc)
 
 
 def test_padded_qkv_rows_are_ignored():

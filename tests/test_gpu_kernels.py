@@ -303,6 +303,82 @@ def test_paged_prefill_against_oracle(hq, hkv, d, causal):
     assert_close(gl, el, atol=2e-3, rtol=1e-4, what="paged lse")
 
 
+def test_layer_sliding_window_mask_known_answer_on_the_gpu():
+    """The reference's known-answer vector for the paged prefill kernel with sliding_window_size = 3
+    (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_tir.py:98-156)."""
+    hq, hkv, d = 4, 2, 64
+    q = np.zeros((2, hq, d), F16)
+    pages = np.zeros((1, 2, hkv, 16, d), F16)
+    for position, value in enumerate([1, 3, 5]):
+        pages[0, 1, :, position, :] = value
+    go = torch.full((2, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.zeros((2, hq), dtype=torch.float32, device=DEV)
+    K.batch_prefill_paged_kv(dev(q), i32([0, 2]), dev(pages), i32([0, 1]), i32([0]), i32([[3], [0], [0]]), i32([0]),
+                             i32([3, 4]), go, gl, 1, 0, 1.0, 1e4, d ** -0.5, sliding_window_size=3)
+    assert_close(host(go)[:, 0, 0], np.array([4, 5], F16), atol=1e-3, rtol=1e-3, what="sliding window known answer")
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("rotary", [0, 1])
+@pytest.mark.parametrize("causal,window", [(0, 1024), (1, 0), (1, 5), (1, 40)])
+def test_paged_prefill_sliding_cache_layer_window_and_inline_rope(hq, hkv, d, rotary, causal, window):
+    """length_info (3, B), the per-layer window mask (window > 0 together with causal; with
+    window = 0 or without causal the reference falls back to the plain masks) and rotary_mode = 1."""
+    from tests.test_oracle_kernels import sliding_case
+    rng = np.random.default_rng(24)
+    spec = [(100, 4, 20), (257, 0, 0), (330, 16, 48), (33, 2, 2), (64, 16, 32), (90, 0, 17)]
+    q_lens = [7, 64, 33, 3, 1, 30]
+    pages, pindptr, pvalues, info, k_log, _ = sliding_case(rng, spec, hkv, d, npages=64)
+    n = sum(q_lens)
+    qindptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k_off = rng.integers(0, 200, size=len(spec)).astype(np.int32)
+    q_pos = np.concatenate([k_off[i] + len(k_log[i]) - q_lens[i] + np.arange(q_lens[i]) for i in range(len(spec))])
+    q_pos = q_pos.astype(np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    ok.prefill_paged(q, qindptr, pages, pindptr, pvalues, info, k_off, q_pos, eo, el, causal, rotary, 1.0, 1e4,
+                     d ** -0.5, sliding_window_size=window)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_paged_kv(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(info), i32(k_off),
+                             i32(q_pos), go, gl, causal, rotary, 1.0, 1e4, d ** -0.5, sliding_window_size=window)
+    assert_close(host(go), eo, what="sliding paged out")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="sliding paged lse")
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("causal", [1, 0])
+def test_prefill_inline_rope_plain_cache(hq, hkv, d, causal):
+    rng = np.random.default_rng(25)
+    # ragged
+    lens = [1, 33, 64, 130, 7]
+    n = sum(lens)
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    k_off = np.array([0, 17, 500, 3, 1000], np.int32)
+    q_pos = np.concatenate([k_off[i] + np.arange(lens[i]) for i in range(len(lens))]).astype(np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    ok.prefill_ragged(q, indptr, k, v, indptr, q_pos, k_off, eo, el, causal, 1, 1.0, 1e4, d ** -0.5)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_ragged_kv(dev(q), i32(indptr), dev(k), dev(v), i32(indptr), i32(q_pos), i32(k_off), go, gl,
+                              causal, 1, 1.0, 1e4, d ** -0.5)
+    assert_close(host(go), eo, what="inline rope ragged out")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="inline rope ragged lse")
+    # paged, plain length_info
+    kv_lens = [max(40, lens[0]), 75, 200, 130, 64]
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, kv_lens, 48, hkv, 16, d)
+    q_pos = np.concatenate([k_off[i] + kv_lens[i] - lens[i] + np.arange(lens[i]) for i in range(len(lens))])
+    q_pos = q_pos.astype(np.int32)
+    ok.prefill_paged(q, indptr, pages, pindptr, pvalues, last, k_off, q_pos, eo, el, causal, 1, 0.5, 5e5, d ** -0.5)
+    K.batch_prefill_paged_kv(dev(q), i32(indptr), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(k_off),
+                             i32(q_pos), go, gl, causal, 1, 0.5, 5e5, d ** -0.5)
+    assert_close(host(go), eo, what="inline rope paged out")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="inline rope paged lse")
+
+
 def test_chunked_prefill_composition_matches_oracle():
     """ragged(causal) + paged(non-causal) + merge_state: the chunked-prefill path of the cache."""
     rng = np.random.default_rng(12)

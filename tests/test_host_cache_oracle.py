@@ -241,3 +241,14 @@ def test_reference_scenarios_on_the_oracle(runner, rope_mode):
     sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=rope_mode, seed=3, on_step=on_step)
     runner(sc)
     check_pool_invariants(cache.host.state(), cache.host.num_total_pages, ps)
+
+
+@pytest.mark.parametrize("runner", [S.run_sliding_window, S.run_sliding_window_fork])
+def test_sliding_window_scenarios_on_the_oracle(runner):
+    """Sliding-window cache with attention sinks: RoPE is applied inside the kernels at positions
+    counted inside the cache (the reference switches such caches to INLINE mode,
+    src/runtime/vm/paged_kv_cache.cc:343-345)."""
+    layers, hq, hkv, d, ps = 2, 8, 2, 64, 16
+    cache = OraclePagedKVCache([32, 2048, 512, ps, 1], layers, hq, hkv, d, d, rope_mode=S.ROPE_INLINE)
+    sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=S.ROPE_INLINE, seed=4)
+    runner(sc)

@@ -115,6 +115,32 @@ __device__ __forceinline__ void interleave_mfma_valu() {
   }
 }
 
+// ---- inline RoPE (kernels that rotate q and k themselves) --------------------------------------
+// sin and cos of an fp32 angle of any size: two-constant Cody-Waite reduction to [-pi, pi], then
+// the hardware functions (which take revolutions).  Absolute error ~1e-6 for |x| up to ~1e5.
+__device__ __forceinline__ void sincos_reduced(float x, float& sn, float& cs) {
+  const float k = rintf(x * 0.15915494309189535f);
+  float r = fmaf(-k, 6.2831854820251465f, x);    // fp32(2 pi)
+  r = fmaf(-k, -1.7484555314695172e-7f, r);      // 2 pi - fp32(2 pi)
+  const float t = r * 0.15915494309189535f;
+  sn = __builtin_amdgcn_sinf(t);
+  cs = __builtin_amdgcn_cosf(t);
+}
+
+// Rotate-half RoPE of the features (f, f + D/2) held by one lane in two fragments, as the reference
+// does it (python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-127): fp32 math, one rounding to fp16.
+__device__ __forceinline__ void rope_pair(half8_t& lo, half8_t& hi, float pos_scaled, const float* div8) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float sn, cs;
+    sincos_reduced(pos_scaled / div8[i], sn, cs);
+    const float xl = static_cast<float>(lo[i]);
+    const float xh = static_cast<float>(hi[i]);
+    lo[i] = static_cast<half_t>(cs * xl + sn * (-xh));
+    hi[i] = static_cast<half_t>(cs * xh + sn * xl);
+  }
+}
+
 // Compute units of the current device (cached per device).
 inline int compute_units() {
   static int cached[64] = {0};

@@ -393,31 +393,6 @@ struct DecodeRopeDivisors {
   float v[DM_D / 2];
 };
 
-// sin and cos of an fp32 angle of any size: two-constant Cody-Waite reduction to [-pi, pi], then
-// the hardware functions (which take revolutions).  Absolute error ~1e-6 for |x| up to ~1e5.
-__device__ __forceinline__ void sincos_reduced(float x, float& sn, float& cs) {
-  const float k = rintf(x * 0.15915494309189535f);
-  float r = fmaf(-k, 6.2831854820251465f, x);    // fp32(2 pi)
-  r = fmaf(-k, -1.7484555314695172e-7f, r);      // 2 pi - fp32(2 pi)
-  const float t = r * 0.15915494309189535f;
-  sn = __builtin_amdgcn_sinf(t);
-  cs = __builtin_amdgcn_cosf(t);
-}
-
-// Rotate-half RoPE of the features (f, f + D/2) held by one lane in two fragments, as the reference
-// does it (python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-127): fp32 math, one rounding to fp16.
-__device__ __forceinline__ void rope_pair(Vec16& lo, Vec16& hi, float pos_scaled, const float* div8) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    float sn, cs;
-    sincos_reduced(pos_scaled / div8[i], sn, cs);
-    const float xl = static_cast<float>(lo.h[i]);
-    const float xh = static_cast<float>(hi.h[i]);
-    lo.h[i] = static_cast<half_t>(cs * xl + sn * (-xh));
-    hi.h[i] = static_cast<half_t>(cs * xh + sn * xl);
-  }
-}
-
 // EXT = false: plain cache, q and k already rotated (or no RoPE).  EXT = true adds the sliding-window
 // cache (length_info (3, B): the page table covers `sink` tokens at the front, evicted tokens up to
 // `window_offset`, then the window, python/tvm/relax/frontend/nn/llm/_kernel_common.py:155-170) and
@@ -482,8 +457,8 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
     for (int ks = 0; ks < 4; ++ks) qv[ks] = c16 < group ? ld16(qrow + ks * 32) : zero16();
     if (EXT && p.rotary) {
       const float q_pos = static_cast<float>(p.q_rope_position[b]) * p.rope_scale;
-      rope_pair(qv[0], qv[2], q_pos, divr);
-      rope_pair(qv[1], qv[3], q_pos, divr + 8);
+      rope_pair(qv[0].h8, qv[2].h8, q_pos, divr);
+      rope_pair(qv[1].h8, qv[3].h8, q_pos, divr + 8);
     }
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) qf[ks] = qv[ks].h8;
@@ -545,8 +520,8 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
         const int t = (pi + h) * PS + c16;
         const int logical = t < sink ? t : t - win_lo + sink;
         const float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
-        rope_pair(r.k[h][0], r.k[h][2], pos, divr);
-        rope_pair(r.k[h][1], r.k[h][3], pos, divr + 8);
+        rope_pair(r.k[h][0].h8, r.k[h][2].h8, pos, divr);
+        rope_pair(r.k[h][1].h8, r.k[h][3].h8, pos, divr + 8);
       }
     }
     // ---- S^T = K Q^T for both pages ---------------------------------------------------------

@@ -26,6 +26,7 @@
 // Workgroup -> (sequence, row tile) without a prologue kernel: sequence b owns tile slots
 //   [floor(q_indptr[b]*group/128) + b, floor(q_indptr[b+1]*group/128) + b + 1)
 // found by binary search on q_indptr; the grid is floor(total_q*group/128) + B slots.
+#include <cmath>
 #include <type_traits>
 
 #include "kernels_common.cuh"
@@ -55,6 +56,20 @@ struct PrefillParams {
   int group;
   int causal;
   float scale_log2;
+  // extended form (prefill_kernel<..., EXT = true>): sliding-window cache, per-layer sliding-window
+  // mask, inline RoPE
+  const int32_t* window_offset;      // paged, (B): physical index of the first token of the window, or NULL
+  const int32_t* sink_size;          // paged, (B): attention-sink tokens kept at the front, or NULL
+  int layer_window;                  // > 0 with causal: row r sees only the last layer_window - r - 1 keys
+  const int32_t* q_rope_position;    // (total_q) position of each query token (inline RoPE)
+  const int32_t* k_rope_pos_offset;  // (B) position of logical key 0 (inline RoPE)
+  int rotary;
+  float rope_scale;
+};
+
+// theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
+struct PrefillRopeDivisors {
+  float v[64];
 };
 
 __device__ __forceinline__ int tile_slot_begin(const int32_t* q_indptr, int b, int group) {
@@ -87,8 +102,18 @@ constexpr size_t prefill_lds_bytes(int dqk, int dv) {
   return static_cast<size_t>(prefill_stages(dqk, dv)) * BN * (dqk + dv) * 2;
 }
 
-template <int DQK, int DV, bool PAGED, int PS>
-__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(PrefillParams p) {
+// EXT = false: plain cache, q and k already rotated (or no RoPE).  EXT = true adds
+//  * the sliding-window cache, length_info (3, B): the page table covers `sink` tokens at the front,
+//    evicted tokens up to `window_offset`, then the window; keys have logical indices (sink tokens,
+//    then window tokens) that the masks and RoPE use
+//    (python/tvm/relax/frontend/nn/llm/_kernel_common.py:155-170);
+//  * the per-layer sliding-window mask of _kernel_common.py:138-144;
+//  * inline RoPE: q at q_rope_position[token], key t at k_rope_pos_offset[b] + t
+//    (_prefill_kernels.py:119-147).
+// Attention does not depend on the order of the keys, so the tiles are still walked in physical
+// order; every tile takes the masked path and masks are evaluated per element.
+template <int DQK, int DV, bool PAGED, int PS, bool EXT>
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
   static_assert(DQK % 64 == 0 && DV % 64 == 0, "feature dims must be multiples of 64");
   constexpr int KS = DQK / 16;                  // k-steps of the QK^T product
   constexpr int DB = DV / 32;                   // 32-wide output feature blocks
@@ -142,14 +167,27 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   if (local_slot >= n_row_tiles) return;
   const int r0 = (n_row_tiles - 1 - local_slot) * BM;
 
-  int kv_len, kv_start = 0, pbeg = 0;
+  // phys_len: tokens the K/V storage of the sequence covers; kv_len: keys attended to (logical)
+  int phys_len, kv_start = 0, pbeg = 0, sink = 0, win_lo = 0;
   if (PAGED) {
     pbeg = p.page_indptr[b];
     const int npages = p.page_indptr[b + 1] - pbeg;
-    kv_len = npages > 0 ? (npages - 1) * PS + p.last_page_len[b] : 0;
+    phys_len = npages > 0 ? (npages - 1) * PS + p.last_page_len[b] : 0;
+    if (EXT && p.sink_size != nullptr && npages > 0) {
+      sink = p.sink_size[b];
+      win_lo = p.window_offset[b];
+    }
   } else {
     kv_start = p.kv_indptr[b];
-    kv_len = p.kv_indptr[b + 1] - kv_start;
+    phys_len = p.kv_indptr[b + 1] - kv_start;
+  }
+  const int kv_len = phys_len - win_lo + sink;
+  // number of logical keys -> physical end of the tokens that hold them
+  auto to_phys = [&](int n) { return (!EXT || n <= sink) ? n : n - sink + win_lo; };
+  __shared__ float div_lds[64];
+  if (EXT && p.rotary) {
+    if (tid < DQK / 2) div_lds[tid] = div.v[tid];
+    __syncthreads();
   }
 
   // ---- this lane's query row -------------------------------------------------------------
@@ -158,23 +196,34 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   const int my_pos = my_row / group;
   const int my_head = kvh * group + my_row % group;
   const int causal_shift = kv_len - qo_len + 1;
-  // number of visible kv tokens for this row
-  const int my_limit = row_valid ? (p.causal ? min(kv_len, causal_shift + my_pos) : kv_len) : 0;
+  // number of visible kv tokens for this row (logical), and with the per-layer window the first one
+  const bool layer_mask = EXT && p.causal && p.layer_window > 0;
+  const int my_limit = !row_valid ? 0 : (layer_mask ? kv_len : (p.causal ? min(kv_len, causal_shift + my_pos) : kv_len));
+  const int my_lo = layer_mask ? max(kv_len - max(p.layer_window - my_pos - 1, 0), 0) : 0;
   // workgroup- and wave-level bounds (uniform)
   const int last_row_wg = min(rows, r0 + BM) - 1;
-  const int kv_end = p.causal ? max(0, min(kv_len, causal_shift + last_row_wg / group)) : kv_len;
+  const int kv_end = to_phys((p.causal && !layer_mask) ? max(0, min(kv_len, causal_shift + last_row_wg / group)) : kv_len);
   const int first_row_wave = r0 + wave * 32;
   const int last_row_wave = min(rows, first_row_wave + 32) - 1;  // < first_row_wave if the wave is empty
   const bool wave_active = first_row_wave < rows;
-  const int wave_limit_max = !wave_active ? 0 : (p.causal ? min(kv_len, causal_shift + last_row_wave / group) : kv_len);
-  const int wave_limit_min = !wave_active ? 0 : (p.causal ? min(kv_len, causal_shift + first_row_wave / group) : kv_len);
+  const bool causal_rows = p.causal && !layer_mask;
+  // physical bounds: beyond wave_limit_max nothing is visible to any row of the wave, below
+  // wave_limit_min everything is visible to all of them (plain cache only)
+  const int wave_limit_max = to_phys(!wave_active ? 0 : (causal_rows ? min(kv_len, causal_shift + last_row_wave / group) : kv_len));
+  const int wave_limit_min = !wave_active ? 0 : (causal_rows ? min(kv_len, causal_shift + first_row_wave / group) : kv_len);
 
   half8_t qf[KS];
   {
     const half_t* qrow = p.q + (static_cast<int64_t>(q_start + my_pos) * p.h_q + my_head) * DQK + half * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[ks] = row_valid ? ld16(qrow + ks * 16).h8 : zero16().h8;
+    if (EXT && p.rotary && row_valid) {
+      const float q_pos = static_cast<float>(p.q_rope_position[q_start + my_pos]) * p.rope_scale;
+#pragma unroll
+      for (int ks = 0; ks < KS / 2; ++ks) rope_pair(qf[ks], qf[ks + KS / 2], q_pos, div_lds + ks * 16 + half * 8);
+    }
   }
+  const float k_pos0 = (EXT && p.rotary) ? static_cast<float>(p.k_rope_pos_offset[b]) : 0.f;
 
   float16_t o[DB];
 #pragma unroll
@@ -189,7 +238,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   // times a finite V is 0 (unwritten page memory could hold NaN patterns).
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds_tiles));
-  const int last_tok = kv_len - 1;
+  const int last_tok = phys_len - 1;
   // Page ids of this wave's RPW rows for 64 consecutive tiles, one tile per lane, fetched once per
   // 64 tiles: the wait for this load also waits for every tile copy in flight, so it must be rare.
   int page_ids = 0;
@@ -369,7 +418,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     // no prefetch across a 64-tile window of page ids: the ids held are those of the last copy issued
     const int next = tile + NSTAGE - 1;  // the tile whose copy this iteration issues
     const bool has_next = next < n_tiles;
-    const bool unmasked = TB == 2 && kv0 < wave_limit_max && kv0 + BN <= wave_limit_min;  // wave-uniform
+    const bool unmasked = !EXT && TB == 2 && kv0 < wave_limit_max && kv0 + BN <= wave_limit_min;  // wave-uniform
     if (has_next) issue_tile(next);
 
     if (kv0 >= wave_limit_max) continue;  // wave-uniform: every row of this wave is masked out
@@ -416,11 +465,28 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
       half8_t vf[DB][2];
       half8_t pf[2];
       read_k(Ks, tb, kf);
+      if (EXT && p.rotary) {
+        // this lane's key row is physical token t0 + col; its logical index is its position
+        const int t = min(t0 + col, last_tok);
+        const int logical = t < sink ? t : t - win_lo + sink;
+        const float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
+#pragma unroll
+        for (int ks = 0; ks < KS / 2; ++ks) rope_pair(kf[ks], kf[ks + KS / 2], pos, div_lds + ks * 16 + half * 8);
+      }
       __builtin_amdgcn_sched_barrier(0);
       float16_t acc = qk(kf);
       read_v(Vs, tb, vf);
       __builtin_amdgcn_sched_barrier(0);
-      if (t0 + 32 > wave_limit_min) {  // wave-uniform
+      if (EXT) {
+        // element j is physical token t0 + half*4 + (j/4)*8 + j%4
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int t = t0 + half * 4 + (j >> 2) * 8 + (j & 3);
+          const bool cached = t < sink || (t >= win_lo && t < phys_len);
+          const int logical = t < sink ? t : t - win_lo + sink;
+          acc[j] = (cached && logical < my_limit && logical >= my_lo) ? acc[j] : -3.0e38f;
+        }
+      } else if (t0 + 32 > wave_limit_min) {  // wave-uniform
         asm volatile("" ::: "memory");  // keep this a branch: if-converted it costs 5 ops per element everywhere
         const int rel = my_limit - t0 - half * 4;  // element j is token t0 + half*4 + (j/4)*8 + j%4
 #pragma unroll
@@ -452,19 +518,38 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   }
 }
 
-template <int DQK, int DV, bool PAGED, int PS>
-static void launch_prefill(const PrefillParams& p, int64_t total_q, hipStream_t stream) {
+template <int DQK, int DV, bool PAGED, int PS, bool EXT>
+static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const PrefillRopeDivisors& div,
+                               hipStream_t stream) {
   const int64_t slots = total_q * p.group / BM + p.batch_size;
   if (slots >= 65536) throw Error(TVMKV_EINVAL, "prefill: too many row tiles for one launch");
   constexpr size_t lds_bytes = prefill_lds_bytes(DQK, DV);
   static bool attr_set = false;  // per instantiation; the attribute is per function, not per device
   if (lds_bytes > 48 * 1024 && !attr_set) {
-    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, PAGED, PS>),
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, PAGED, PS, EXT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     attr_set = true;
   }
-  hipLaunchKernelGGL((prefill_kernel<DQK, DV, PAGED, PS>), dim3(p.h_kv, static_cast<unsigned>(slots)), dim3(NW * 64),
-                     lds_bytes, stream, p);
+  hipLaunchKernelGGL((prefill_kernel<DQK, DV, PAGED, PS, EXT>), dim3(p.h_kv, static_cast<unsigned>(slots)),
+                     dim3(NW * 64), lds_bytes, stream, p, div);
+}
+
+// The extended kernels (sliding-window cache, per-layer window, inline RoPE) exist for the head
+// dims that RoPE models use here; d_qk 192 / d_v 128 is the MLA self-attention, which has neither.
+template <int DQK, int DV, bool PAGED, int PS>
+static void launch_prefill(const PrefillParams& p, int64_t total_q, bool ext, double rope_theta, hipStream_t stream) {
+  PrefillRopeDivisors div{};
+  if (!ext) {
+    launch_prefill_ext<DQK, DV, PAGED, PS, false>(p, total_q, div, stream);
+    return;
+  }
+  if constexpr (DQK == DV && DQK <= 128) {
+    const float theta = static_cast<float>(rope_theta);
+    for (int i = 0; i < DQK / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DQK));
+    launch_prefill_ext<DQK, DV, PAGED, PS, true>(p, total_q, div, stream);
+  } else {
+    throw Error(TVMKV_EUNSUPPORTED, "prefill: inline RoPE / sliding window are not built for this head shape");
+  }
 }
 
 }  // namespace tvmkv
@@ -482,9 +567,10 @@ int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const 
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_ragged_kv: bad shape";
-  KV_UNSUPPORTED(rotary_mode != 0) << "batch_prefill_ragged_kv: inline RoPE (rotary_mode=1) is not built";
   if (batch_size == 0 || total_q == 0) return TVMKV_OK;
   KV_CHECK(q && q_indptr && k && v && kv_indptr && output && lse) << "batch_prefill_ragged_kv: NULL tensor";
+  KV_CHECK(rotary_mode == 0 || (q_rope_position && k_rope_pos_offset))
+      << "batch_prefill_ragged_kv: inline RoPE needs the position arrays";
   PrefillParams p{};
   p.q = static_cast<const half_t*>(q);
   p.q_indptr = q_indptr;
@@ -499,13 +585,18 @@ int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const 
   p.group = h_q / h_kv;
   p.causal = causal > 0;
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
+  p.rotary = rotary_mode != 0;
+  p.rope_scale = static_cast<float>(rope_scale);
+  p.q_rope_position = q_rope_position;
+  p.k_rope_pos_offset = k_rope_pos_offset;
+  const bool ext = p.rotary != 0;
   hipStream_t s = as_stream(stream);
   if (d_qk == 128 && d_v == 128) {
-    launch_prefill<128, 128, false, 16>(p, total_q, s);
+    launch_prefill<128, 128, false, 16>(p, total_q, ext, rope_theta, s);
   } else if (d_qk == 64 && d_v == 64) {
-    launch_prefill<64, 64, false, 16>(p, total_q, s);
+    launch_prefill<64, 64, false, 16>(p, total_q, ext, rope_theta, s);
   } else if (d_qk == 192 && d_v == 128) {
-    launch_prefill<192, 128, false, 16>(p, total_q, s);
+    launch_prefill<192, 128, false, 16>(p, total_q, ext, rope_theta, s);
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_ragged_kv: (d_qk, d_v) = (" << d_qk << ", " << d_v
                          << ") is not built ((64,64), (128,128), (192,128))";
@@ -525,13 +616,13 @@ int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const v
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_paged_kv: bad shape";
-  KV_UNSUPPORTED(rotary_mode != 0) << "batch_prefill_paged_kv: inline RoPE (rotary_mode=1) is not built";
-  KV_UNSUPPORTED(sliding_window != 0) << "batch_prefill_paged_kv: sliding-window length_info (3, B) is not built";
   KV_UNSUPPORTED(page_size != 16) << "batch_prefill_paged_kv: page_size " << page_size << " is not built (16)";
   if (batch_size == 0 || total_q == 0) return TVMKV_OK;
   KV_CHECK(q && q_indptr && pages && page_indptr && length_info && output && lse)
       << "batch_prefill_paged_kv: NULL tensor";
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_prefill_paged_kv: NULL page table";
+  KV_CHECK(rotary_mode == 0 || (q_rope_position && k_rope_pos_offset))
+      << "batch_prefill_paged_kv: inline RoPE needs the position arrays";
   PrefillParams p{};
   p.q = static_cast<const half_t*>(q);
   p.q_indptr = q_indptr;
@@ -547,11 +638,21 @@ int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const v
   p.group = h_q / h_kv;
   p.causal = causal > 0;
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
+  p.rotary = rotary_mode != 0;
+  p.rope_scale = static_cast<float>(rope_scale);
+  p.q_rope_position = q_rope_position;
+  p.k_rope_pos_offset = k_rope_pos_offset;
+  if (sliding_window != 0) {  // length_info is (3, B): last_page_len, window offset, sink size
+    p.window_offset = length_info + batch_size;
+    p.sink_size = length_info + 2 * static_cast<int64_t>(batch_size);
+    p.layer_window = sliding_window_size;
+  }
+  const bool ext = p.rotary != 0 || sliding_window != 0;
   hipStream_t s = as_stream(stream);
   if (d == 128) {
-    launch_prefill<128, 128, true, 16>(p, total_q, s);
+    launch_prefill<128, 128, true, 16>(p, total_q, ext, rope_theta, s);
   } else if (d == 64) {
-    launch_prefill<64, 64, true, 16>(p, total_q, s);
+    launch_prefill<64, 64, true, 16>(p, total_q, ext, rope_theta, s);
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_paged_kv: head_dim " << d << " is not built (64, 128)";
   }

@@ -635,10 +635,6 @@ class PagedKVCache {
     KV_CHECK(total_seq_length <= prefill_chunk_size_)
         << "the batch appends " << total_seq_length << " tokens, more than prefill_chunk_size "
         << prefill_chunk_size_;
-    KV_UNSUPPORTED(rope_mode_ == TVMKV_ROPE_INLINE)
-        << "inline RoPE (and with it the sliding-window cache) is not built in the HIP kernels yet";
-    KV_UNSUPPORTED(attn_kinds_[layer_id] == TVMKV_ATTN_MHA_SLIDING)
-        << "per-layer sliding-window attention is not built in the HIP kernels yet";
     ComputeStreamWaitForCopyStream();
     KV_CHECK(!dirty_aux_data_device_) << "auxiliary data is not synchronised";
 
