@@ -118,11 +118,11 @@ def calibrate(num_bytes=2 << 30, iters=10):
 
 # HBM bytes per launch of the decode entry point on the default workload, from rocprofv3 counter runs
 # of this file (profiles/decode_mfma_kernel_cfg2_batched_decode.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
-# in KiB per dispatch, decode_mfma_kernel + decode_merge_kernel; the scales come from the plain copy
+# in KiB per dispatch of decode_mfma_kernel (it merges the chunks itself); the scales come from the plain copy
 # kernel of known size (profiles/stream_copy_kernel_2GiB_calibration.txt).  It is a property of the
 # workload, so it is only reported when the algorithmic bytes are those it was measured on.
 TRAFFIC_MEASURED_ON_BYTES = 1182904320
-TRAFFIC_KIB = {"decode_mfma_kernel": (578946.1 * 2.0, 5053.8), "decode_merge_kernel": (2666.0 * 2.0, 528.0)}
+TRAFFIC_KIB = {"decode_mfma_kernel": (581131.7 * 2.0, 6219.8)}
 
 
 def measured_traffic(algorithmic_bytes):
@@ -276,7 +276,7 @@ def main():
     t0 = time.perf_counter()
     ms_step = time_region(torch, lambda i: step(W + i), K_steps)
     wall_ms = (time.perf_counter() - t0) * 1e3 / K_steps
-    # the decode entry point alone (split-KV kernel + merge kernel), same page tables
+    # the decode entry point alone (split-KV kernel with the fused chunk merge), same page tables
     ms_decode = time_region(torch, lambda i: decode_only(W + i), K_steps)
 
     kv_tokens = np.array([t["kv_len"].sum() for t in wl["tables"][W:]], dtype=np.float64)
@@ -308,7 +308,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(gbps_decode, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps_decode / HBM_PEAK_GBPS, 4),
                      "traffic": measured_traffic(int(decode_bytes)),
-                     "kernel": "tvmkv_batch_decode_paged_kv (decode_mfma_kernel + decode_merge_kernel)",
+                     "kernel": "tvmkv_batch_decode_paged_kv (decode_mfma_kernel, chunk merge fused)",
                      "ms": round(ms_decode, 4), "algorithmic_bytes": int(decode_bytes)},
     }
 
@@ -350,11 +350,6 @@ def main():
                              "algorithmic_flops": pw["flops"],
                              "frac_of_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
 
-    if args.extras:
-        del pages, qkv
-        torch.cuda.empty_cache()
-        result["extras"] = extras(torch, K, dev)
-
     # ---- CPU baseline: the oracle's restatement of the reference's llvm decode kernel ---------
     if not args.no_cpu_baseline:
         from oracle import kernels as ok
@@ -382,6 +377,11 @@ def main():
                                             f"{cpu_s:.1f} s; the reference kernel is T.serial",
                                   "tokens_per_s": round(B / cpu_s, 2), "host_cpus": os.cpu_count(),
                                   "gpu_vs_cpu_max_abs_err": err}
+
+    if args.extras:
+        del pages, qkv
+        torch.cuda.empty_cache()
+        result["extras"] = extras(torch, K, dev)
     print(json.dumps(result))
 
 
