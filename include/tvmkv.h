@@ -133,6 +133,38 @@ int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t*
                                 int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
                                 int32_t d, int32_t page_size, int32_t sliding_window, void* stream);
 
+/* Slot 21 ragged prefill with a token-tree mask -- replaces `batch_tree_attn`
+ * (python/tvm/relax/frontend/nn/llm/tree_attn.py:264-603; llvm form :68-259), calling convention
+ * attn_backend.h:669-672:
+ * (q, qo_indptr, k, v, kv_indptr, q_rope_position, mn_indptr, mask, out, lse, rotary_mode,
+ *  rope_scale, rope_theta, sm_scale).
+ * mn_indptr (batch+1) gives the first tree node of each sequence, mask (nodes, 2) holds per node
+ * its pre-order number and the end of the range its subtree covers; the last
+ * mn_indptr[b+1]-mn_indptr[b] keys of sequence b are its tree nodes, and a query node sees the keys
+ * before the tree plus the nodes n with mask[n][0] <= mask[self][0] < mask[n][1]
+ * (tree_attn.py:48-65).  Under rotary_mode 1 key t is rotated at q_rope_position[kv_indptr[b]+t]. */
+int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                          const int32_t* kv_indptr, const int32_t* q_rope_position,
+                          const int32_t* mn_indptr, const int32_t* mask, void* output, float* lse,
+                          int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                          int32_t batch_size, int64_t total_q, int32_t h_q, int32_t h_kv, int32_t d,
+                          void* stream);
+
+/* Slot 20 paged prefill with a token-tree mask -- replaces `tree_attn_paged_kv`
+ * (tree_attn.py:798-1259; llvm form :606-797), calling convention attn_backend.h:623-626:
+ * (q, qo_indptr, pages, page_indptr, page_indices, length_info, k_rope_pos_offset,
+ *  q_rope_position, out, lse, rotary_mode, rope_scale, rope_theta, sm_scale, tree_order_indptr,
+ *  tree_order).  Like the reference kernel (tree_attn.py:700-702) it rejects rotary_mode != 0. */
+int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void* pages,
+                             const int32_t* page_indptr, const int32_t* page_values,
+                             const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                             const int32_t* q_rope_position, void* output, float* lse,
+                             int64_t rotary_mode, double rope_scale, double rope_theta,
+                             double sm_scale, const int32_t* tree_order_indptr,
+                             const int32_t* tree_order, int32_t batch_size, int64_t total_q,
+                             int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                             int32_t d, int32_t page_size, int32_t sliding_window, void* stream);
+
 /* Slot 22 MLA paged prefill (also used for MLA decode, paged_kv_cache.cc:954-956) -- replaces
  * `batch_prefill_paged_kv_mla` (_prefill_kernels.py:927-1071), calling convention
  * attn_backend.h:248-249: (q, qo_indptr, pages, page_indptr, page_indices, length_info, out, lse,

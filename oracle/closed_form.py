@@ -10,6 +10,8 @@ dropped term, a wrong sign or a transposed index in the C restatement fails a co
   query block aligned to the *end* of the keys (same file, :499-535 and :596-607); also
   returns the base-2 log-sum-exp the kernels expose
   (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:176).
+* ``tree_ancestor_mask`` -- the token-tree mask of speculative decoding from the parent
+  pointers (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_tir.py:614-627).
 * ``merge`` -- two-way log-sum-exp merge of partial attention states
   (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:441-450).
 * ``mla_expand`` -- MLA by its definition: expand the latent with ``w_kv`` and run plain MHA
@@ -31,8 +33,25 @@ def apply_rotary(x, positions, scale=1.0, theta=1e4):
     return np.einsum("ij,ikj->ikj", np.cos(emb), x) + np.einsum("ij,ikj->ikj", np.sin(emb), y)
 
 
-def attention(q, k, v, sm_scale, causal=True, window=None):
+def tree_ancestor_mask(parent_ptr):
+    """(n, n) bool: node i sees node j iff j is i or an ancestor of i.
+
+    Built the way the reference's test builds it: a node inherits its parent's row and adds
+    itself (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_tir.py:614-627).
+    """
+    n = len(parent_ptr)
+    mask = np.zeros((n, n), dtype=bool)
+    for i, parent in enumerate(parent_ptr):
+        if parent != -1:
+            mask[i] = mask[parent]
+        mask[i, i] = True
+    return mask
+
+
+def attention(q, k, v, sm_scale, causal=True, window=None, mask=None):
     """q: (Lq, Hq, Dqk), k: (Lk, Hkv, Dqk), v: (Lk, Hkv, Dv).
+
+    ``mask`` (Lq, Lk) bool, if given, replaces the causal / window masks.
 
     Query i sits at absolute position Lk - Lq + i.  Returns (out float64 (Lq, Hq, Dv),
     lse_base2 float64 (Lq, Hq)).  An all-masked row gives out 0 and lse -inf.
@@ -48,11 +67,13 @@ def attention(q, k, v, sm_scale, causal=True, window=None):
     scores = np.einsum("qhd,khd->hqk", q, k) * sm_scale
     qpos = lk - lq + np.arange(lq)
     kpos = np.arange(lk)
-    mask = np.ones((lq, lk), dtype=bool)
-    if causal:
-        mask &= kpos[None, :] <= qpos[:, None]
-    if window is not None:
-        mask &= kpos[None, :] > qpos[:, None] - window
+    if mask is None:
+        mask = np.ones((lq, lk), dtype=bool)
+        if causal:
+            mask &= kpos[None, :] <= qpos[:, None]
+        if window is not None:
+            mask &= kpos[None, :] > qpos[:, None] - window
+    mask = np.asarray(mask, dtype=bool)
     scores = np.where(mask[None], scores, -np.inf)
     with np.errstate(invalid="ignore", divide="ignore"):
         m = scores.max(axis=-1, keepdims=True)

@@ -161,6 +161,34 @@ def prefill_ragged(q, q_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_off
                              _c_f(rope_scale), _c_f(rope_theta), _c_f(sm_scale))
 
 
+def tree_attn_ragged(q, q_indptr, k, v, kv_indptr, q_rope_position, mn_indptr, mask, output, lse,
+                     rotary_mode, rope_scale, rope_theta, sm_scale):
+    """tree_attn_cpu; mask is (tree nodes, 2) int32 = (DFS order, end of the subtree's range)."""
+    _, hq, d = q.shape
+    _, hkv, _ = v.shape
+    qi, ki, qp = _i32(q_indptr), _i32(kv_indptr), _i32(q_rope_position)
+    mi, mk = _i32(mn_indptr), _i32(mask)
+    lib().orc_tree_attn_ragged(_p(q), _p(qi), _p(k), _p(v), _p(ki), _p(qp), _p(mi), _p(mk), _p(output),
+                               _p(lse), _c_int(len(qi) - 1), _c_int(hq), _c_int(hkv), _c_int(d),
+                               _c_int(rotary_mode), _c_f(rope_scale), _c_f(rope_theta), _c_f(sm_scale))
+
+
+def tree_attn_paged(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset,
+                    q_rope_position, output, lse, rotary_mode, rope_scale, rope_theta, sm_scale,
+                    tree_order_indptr, tree_order):
+    """tree_attn_paged_kv_cpu, argument order of the reference kernel."""
+    _, hq, d = q.shape
+    _, _, hkv, ps, _ = pages.shape
+    qi = _i32(q_indptr)
+    li = _i32(length_info)
+    args = [_i32(page_indptr), _i32(page_values), li, _i32(k_rope_pos_offset), _i32(q_rope_position)]
+    ti, to = _i32(tree_order_indptr), _i32(tree_order)
+    lib().orc_tree_attn_paged(_p(q), _p(qi), _p(pages), *[_p(a) for a in args], _p(output), _p(lse),
+                              _c_int(len(qi) - 1), _c_int(hq), _c_int(hkv), _c_int(d), _c_int(ps),
+                              _c_int(int(li.ndim == 2)), _c_int(rotary_mode), _c_f(rope_scale),
+                              _c_f(rope_theta), _c_f(sm_scale), _p(ti), _p(to))
+
+
 def prefill_paged_mla(q, q_indptr, pages, page_indptr, page_values, length_info, output, lse,
                       causal, sm_scale, d_latent=512):
     _, hq, dqk = q.shape

@@ -20,6 +20,8 @@
  *   orc_merge_state_inplace     _decode_kernels.py:414-452
  *   orc_prefill_paged           python/tvm/relax/frontend/nn/llm/_prefill_kernels.py:54-214
  *   orc_prefill_ragged          _prefill_kernels.py:677-791
+ *   orc_tree_attn_ragged        python/tvm/relax/frontend/nn/llm/tree_attn.py:93-259
+ *   orc_tree_attn_paged         tree_attn.py:634-797 (mask: tree_attn.py:48-65)
  *   orc_prefill_paged_mla       _prefill_kernels.py:927-1071 (GPU-only kernel in the
  *                               reference; restated here row by row, see below)
  *   helpers                     python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-170
@@ -91,6 +93,22 @@ static inline int causal_or_sliding_cross_mask(int causal, int row, int col, int
     return col < kv_len && col >= lo;
   }
   return causal_mask(causal, row, col, kv_len, qo_len);
+}
+
+/* tree_attn.py:48-65: the last tree_order_len keys of the sequence are the nodes of its token tree;
+ * tree_order holds (first, second) per node = its DFS order and the end of its subtree's range.
+ * A query node sees every key before the tree and the tree nodes that are its ancestors or itself. */
+static inline int check_tree_order(const int32_t* tree_order_indptr, const int32_t* tree_order,
+                                   int batch, int row, int col, int kv_len, int qo_len) {
+  int tree_order_len = tree_order_indptr[batch + 1] - tree_order_indptr[batch];
+  int tree_start = kv_len - tree_order_len;
+  int child_idx_in_tree = row + tree_order_len - qo_len;
+  int parent_idx_in_tree = col - tree_start;
+  if (!(col < kv_len)) return 0;
+  if (col < tree_start) return 1;
+  const int32_t* child = tree_order + 2 * (int64_t)(tree_order_indptr[batch] + child_idx_in_tree);
+  const int32_t* parent = tree_order + 2 * (int64_t)(tree_order_indptr[batch] + parent_idx_in_tree);
+  return child[0] >= parent[0] && child[0] < parent[1];
 }
 
 /* ---- RoPE (position_embedding.py:32-67 + _kernel_common.py:115-127) ----------- */
@@ -295,13 +313,16 @@ void orc_merge_state_inplace(f16* V, float* S, const f16* V_other, const float* 
 }
 
 /* ---- batch_prefill_paged_kv_cpu (_prefill_kernels.py:121-213) ------------------ */
-void orc_prefill_paged(const f16* q, const int32_t* q_indptr, const f16* pages,
-                       const int32_t* page_indptr, const int32_t* page_values,
-                       const int32_t* length_info, const int32_t* k_rope_pos_offset,
-                       const int32_t* q_rope_position, f16* output, float* lse, int batch_size,
-                       int h_q, int h_kv, int d, int page_size, int sliding_window,
-                       int sliding_window_size, int causal, int rotary_mode, float rope_scale,
-                       float rope_theta, float sm_scale) {
+/* tree_order_indptr == NULL: batch_prefill_paged_kv_cpu.  Otherwise tree_attn_paged_kv_cpu
+ * (tree_attn.py:634-797), which is the same loop nest with _check_tree_order as its mask. */
+static void prefill_paged_impl(const f16* q, const int32_t* q_indptr, const f16* pages,
+                               const int32_t* page_indptr, const int32_t* page_values,
+                               const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                               const int32_t* q_rope_position, f16* output, float* lse, int batch_size,
+                               int h_q, int h_kv, int d, int page_size, int sliding_window,
+                               int sliding_window_size, int causal, int rotary_mode, float rope_scale,
+                               float rope_theta, float sm_scale, const int32_t* tree_order_indptr,
+                               const int32_t* tree_order) {
   int group_size = h_q / h_kv;
   float* O_local = (float*)malloc(sizeof(float) * d * 4);
   float *Q_local = O_local + d, *K_local = Q_local + d, *V_local = K_local + d;
@@ -336,8 +357,11 @@ void orc_prefill_paged(const f16* q, const int32_t* q_indptr, const f16* pages,
           float S_val = 0.0f;
           for (int i = 0; i < d; ++i) S_val += Q_local[i] * K_local[i];
           S_val *= sm_scale * LOG2E_F;
-          if (causal_or_sliding_cross_mask(causal, q_idx, row_idx, kv_len, qo_len,
-                                           sliding_window ? sliding_window_size : 0)) {
+          int visible = tree_order_indptr
+                            ? check_tree_order(tree_order_indptr, tree_order, b_idx, q_idx, row_idx, kv_len, qo_len)
+                            : causal_or_sliding_cross_mask(causal, q_idx, row_idx, kv_len, qo_len,
+                                                           sliding_window ? sliding_window_size : 0);
+          if (visible) {
             new_m = fmaxf(m_val, S_val);
           } else {
             S_val = -5e4f;
@@ -361,12 +385,41 @@ void orc_prefill_paged(const f16* q, const int32_t* q_indptr, const f16* pages,
   free(O_local);
 }
 
-/* ---- batch_prefill_ragged_kv (cpu) (_prefill_kernels.py:715-790) ---------------- */
-void orc_prefill_ragged(const f16* q, const int32_t* q_indptr, const f16* k, const f16* v,
-                        const int32_t* kv_indptr, const int32_t* q_rope_position,
-                        const int32_t* k_rope_pos_offset, f16* output, float* lse, int batch_size,
-                        int h_q, int h_kv, int d_qk, int d_v, int causal, int rotary_mode,
-                        float rope_scale, float rope_theta, float sm_scale) {
+void orc_prefill_paged(const f16* q, const int32_t* q_indptr, const f16* pages,
+                       const int32_t* page_indptr, const int32_t* page_values,
+                       const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                       const int32_t* q_rope_position, f16* output, float* lse, int batch_size,
+                       int h_q, int h_kv, int d, int page_size, int sliding_window,
+                       int sliding_window_size, int causal, int rotary_mode, float rope_scale,
+                       float rope_theta, float sm_scale) {
+  prefill_paged_impl(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset,
+                     q_rope_position, output, lse, batch_size, h_q, h_kv, d, page_size, sliding_window,
+                     sliding_window_size, causal, rotary_mode, rope_scale, rope_theta, sm_scale, NULL, NULL);
+}
+
+/* tree_attn_paged_kv_cpu (tree_attn.py:634-797); the reference asserts rotary_mode == 0 (:700-702) */
+void orc_tree_attn_paged(const f16* q, const int32_t* q_indptr, const f16* pages,
+                         const int32_t* page_indptr, const int32_t* page_values,
+                         const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                         const int32_t* q_rope_position, f16* output, float* lse, int batch_size,
+                         int h_q, int h_kv, int d, int page_size, int sliding_window, int rotary_mode,
+                         float rope_scale, float rope_theta, float sm_scale,
+                         const int32_t* tree_order_indptr, const int32_t* tree_order) {
+  prefill_paged_impl(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset,
+                     q_rope_position, output, lse, batch_size, h_q, h_kv, d, page_size, sliding_window, 0, 0,
+                     rotary_mode, rope_scale, rope_theta, sm_scale, tree_order_indptr, tree_order);
+}
+
+/* ---- batch_prefill_ragged_kv (cpu) (_prefill_kernels.py:715-790) ----------------
+ * mn_indptr == NULL: the causal kernel.  Otherwise tree_attn_cpu (tree_attn.py:93-259): the same
+ * two-pass loop nest with _check_tree_order as its mask; under inline RoPE its keys are rotated to
+ * q_rope_position[kv_indptr[b] + k_idx] (:207-219) instead of k_rope_pos_offset[b] + k_idx. */
+static void prefill_ragged_impl(const f16* q, const int32_t* q_indptr, const f16* k, const f16* v,
+                                const int32_t* kv_indptr, const int32_t* q_rope_position,
+                                const int32_t* k_rope_pos_offset, f16* output, float* lse, int batch_size,
+                                int h_q, int h_kv, int d_qk, int d_v, int causal, int rotary_mode,
+                                float rope_scale, float rope_theta, float sm_scale,
+                                const int32_t* mn_indptr, const int32_t* mask) {
   int group_size = h_q / h_kv;
   int max_kv = 1;
   for (int b = 0; b < batch_size; ++b)
@@ -396,12 +449,16 @@ void orc_prefill_ragged(const f16* q, const int32_t* q_indptr, const f16* k, con
                         : h2f(qrow[i]);
         for (int k_idx = 0; k_idx < kv_len; ++k_idx) {
           float attention_score;
-          if (causal_mask(causal, q_idx, k_idx, kv_len, qo_len)) {
+          int visible = mn_indptr ? check_tree_order(mn_indptr, mask, b, q_idx, k_idx, kv_len, qo_len)
+                                  : causal_mask(causal, q_idx, k_idx, kv_len, qo_len);
+          if (visible) {
             const f16* krow = k + ((int64_t)(kv_indptr[b] + k_idx) * h_kv + h_kv_idx) * d_qk;
             float result = 0.0f;
+            int k_pos = rotary_mode != 1 ? 0
+                        : (mn_indptr ? q_rope_position[kv_indptr[b] + k_idx] : k_rope_pos_offset[b] + k_idx);
             for (int i = 0; i < d_qk; ++i) {
               float key_val = rotary_mode == 1
-                                  ? h2f(rope_elem(krow, i, d_qk, (float)(k_rope_pos_offset[b] + k_idx) * rope_scale, rope_theta))
+                                  ? h2f(rope_elem(krow, i, d_qk, (float)k_pos * rope_scale, rope_theta))
                                   : h2f(krow[i]);
               result += qbuf[i] * key_val;
             }
@@ -439,6 +496,25 @@ void orc_prefill_ragged(const f16* q, const int32_t* q_indptr, const f16* k, con
   }
   free(attention_scores);
   free(hbuf);
+}
+
+void orc_prefill_ragged(const f16* q, const int32_t* q_indptr, const f16* k, const f16* v,
+                        const int32_t* kv_indptr, const int32_t* q_rope_position,
+                        const int32_t* k_rope_pos_offset, f16* output, float* lse, int batch_size,
+                        int h_q, int h_kv, int d_qk, int d_v, int causal, int rotary_mode,
+                        float rope_scale, float rope_theta, float sm_scale) {
+  prefill_ragged_impl(q, q_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_offset, output, lse, batch_size,
+                      h_q, h_kv, d_qk, d_v, causal, rotary_mode, rope_scale, rope_theta, sm_scale, NULL, NULL);
+}
+
+/* tree_attn_cpu (tree_attn.py:93-259) */
+void orc_tree_attn_ragged(const f16* q, const int32_t* q_indptr, const f16* k, const f16* v,
+                          const int32_t* kv_indptr, const int32_t* q_rope_position,
+                          const int32_t* mn_indptr, const int32_t* mask, f16* output, float* lse,
+                          int batch_size, int h_q, int h_kv, int d, int rotary_mode, float rope_scale,
+                          float rope_theta, float sm_scale) {
+  prefill_ragged_impl(q, q_indptr, k, v, kv_indptr, q_rope_position, NULL, output, lse, batch_size, h_q, h_kv, d,
+                      d, 0, rotary_mode, rope_scale, rope_theta, sm_scale, mn_indptr, mask);
 }
 
 /* ---- batch_prefill_paged_kv_mla (_prefill_kernels.py:979-1064) ------------------

@@ -13,6 +13,7 @@ order the reference's cache object calls them:
   AttentionInternal / MHASelfAttnInternal / MHACrossAttnInternal / MLACrossAttnInternal
                              src/runtime/vm/paged_kv_cache.cc:2161-2335
   fork page copy             src/runtime/vm/paged_kv_cache.cc:721-734
+  commit of token-tree nodes src/runtime/vm/paged_kv_cache.cc:1566-1659, :736-770
 
 Arrays are numpy (fp16 data, int32 indices, fp32 lse).  Parity tests run the same seeded call
 sequence through this object and through the HIP-backed cache and compare outputs, cached
@@ -76,6 +77,16 @@ class OraclePagedKVCache:
         self.host.popn(seq_id, n)
         self._flush_copies()
 
+    def commit_accepted_token_tree_nodes(self, seq_ids, leaf_indices):
+        """CommitAcceptedTokenTreeNodes + CompactKVCopy (paged_kv_cache.cc:1566-1659, :736-770)."""
+        batch = len(self.host.cur_seq_ids)
+        copies = self.host.commit_accepted_token_tree_nodes(seq_ids, leaf_indices)
+        if copies is not None and copies[0][-1] > 0:
+            indptr, src, dst = copies
+            for layer in range(self.num_layers):
+                ok.compact_kv_copy(self.pages[layer], indptr, np.array([src, dst], np.int32), batch)
+        self._flush_copies()
+
     def enable_sliding_window_for_seq(self, seq_id, window, sink):
         self.host.enable_sliding_window_for_seq(seq_id, window, sink)
 
@@ -109,9 +120,14 @@ class OraclePagedKVCache:
 
     def _self_attn(self, q, k, v, out, lse, sm_scale, rope_mode):
         aux = self.host.aux
-        if not self.host.is_chain_on_depths[0]:
-            raise hc.CacheError("tree attention is not part of the oracle")
         indptr = self._i32(aux["cur_append_lengths_indptr"])
+        if not self.host.is_chain_on_depths[0]:
+            # the batch forms token trees (paged_kv_cache.cc:2192-2202)
+            mask = self._i32(aux["tree_attn_mask"][0]).reshape(-1, 2)
+            ok.tree_attn_ragged(q, indptr, k, v, indptr, self._i32(aux["q_rope_position_map"]),
+                                self._i32(aux["tree_attn_mn_indptr"][0]), mask, out, lse,
+                                int(rope_mode == hc.ROPE_INLINE), self.rope_scale, self.rope_theta, sm_scale)
+            return
         ok.prefill_ragged(q, indptr, k, v, indptr, self._i32(aux["q_rope_position_map"]),
                           self._i32(aux["k_ragged_rope_pos_offset"]), out, lse, 1,
                           int(rope_mode == hc.ROPE_INLINE), self.rope_scale, self.rope_theta, sm_scale)
@@ -140,8 +156,12 @@ class OraclePagedKVCache:
                 theta, scale = self.rope_theta, self.rope_scale
             rotary = int(self.rope_mode == hc.ROPE_INLINE)
             if host.append_before_attn and not host.is_chain_on_depths[d]:
-                raise hc.CacheError("tree attention is not part of the oracle")
-            if host.use_decode_kernel[d]:
+                # paged_kv_cache.cc:2266-2272
+                mask = self._i32(aux["tree_attn_mask"][d]).reshape(-1, 2)
+                ok.tree_attn_paged(q, aux["qo_indptr"][d], self.pages[layer], page_indptr, page_indices,
+                                   length_info, k_rope_pos, aux["q_rope_position_map"], o, s, rotary, scale,
+                                   theta, sm_scale, aux["tree_attn_mn_indptr"][d], mask)
+            elif host.use_decode_kernel[d]:
                 ok.decode(q, self.pages[layer], page_indptr, page_indices, length_info, k_rope_pos,
                           aux["q_rope_position_map"], o, s, rotary, scale, theta, sm_scale)
             else:

@@ -59,6 +59,9 @@ class GpuCache:
     def end_forward(self):
         gf("vm.builtin.kv_state_end_forward")(self.cache)
 
+    def commit_accepted_token_tree_nodes(self, ids, leaf_indices):
+        gf("vm.builtin.attention_kv_cache_commit_accepted_token_tree_nodes")(self.cache, ids, leaf_indices)
+
     def empty(self):
         return gf("vm.builtin.attention_kv_cache_empty")(self.cache)
 

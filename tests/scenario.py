@@ -50,8 +50,13 @@ class Scenario:
             assert_close(k, ek, atol=2e-3, rtol=2e-3, what=f"cached k of seq {sid}")
             assert np.array_equal(v, ev), f"cached v of seq {sid} differs"
 
-    def step(self, batch):
-        """batch: list of (seq_id, append_length) or ((seq_id, parent, fork_pos), append_length)."""
+    def step(self, batch, trees=None, accepted=None):
+        """batch: list of (seq_id, append_length) or ((seq_id, parent, fork_pos), append_length).
+
+        trees: per sequence the parent pointers of its whole token tree, whose last append_length
+        nodes are the new tokens; accepted: per sequence the leaf whose root path is kept when the
+        step is committed, -1 for none (test_runtime_builtin_paged_attention_kv_cache_tir.py:396-668).
+        """
         cache = self.cache
         seq_ids, append_lengths = [], []
         for item, n in batch:
@@ -73,19 +78,35 @@ class Scenario:
             seq_ids.append(sid)
             append_lengths.append(n)
 
-        cache.begin_forward(seq_ids, append_lengths)
+        depths = [None] * len(seq_ids)
+        if trees is not None:
+            assert self.rope_mode != ROPE_INLINE, "tree attention has no inline RoPE"
+            flat = []
+            for i, (tree, n) in enumerate(zip(trees, append_lengths)):
+                assert len(tree) >= n
+                flat += tree[-n:]
+                depths[i] = []
+                for parent in tree:
+                    depths[i].append(0 if parent == -1 else depths[i][parent] + 1)
+            cache.begin_forward(seq_ids, append_lengths, flat)
+        else:
+            cache.begin_forward(seq_ids, append_lengths)
         if self.on_step is not None:
             self.on_step(seq_ids, append_lengths)
 
-        new_q, new_k, new_v, offsets = [], [], [], []
-        for sid, n in zip(seq_ids, append_lengths):
+        new_q, new_k, new_v, positions = [], [], [], []
+        for i, (sid, n) in enumerate(zip(seq_ids, append_lengths)):
             q = self._rand(self.num_layers, n, self.hq, self.d)
             k = self._rand(self.num_layers, n, self.hkv, self.d)
             v = self._rand(self.num_layers, n, self.hkv, self.d)
-            off = self.cached_k[sid].shape[1]
-            offsets.append(off)
+            if trees is None:
+                pos = self.cached_k[sid].shape[1] + np.arange(n)
+            else:  # a tree node sits at its depth behind the tokens in front of the tree
+                tree_begin = self.cached_k[sid].shape[1] - (len(trees[i]) - n)
+                pos = tree_begin + np.array(depths[i][-n:])
+            positions.append(pos)
             if self.rope_mode == ROPE_NORMAL:
-                k_store = np.stack([cf.apply_rotary(k[l], off + np.arange(n), self.rope_scale, self.rope_theta)
+                k_store = np.stack([cf.apply_rotary(k[l], pos, self.rope_scale, self.rope_theta)
                                     for l in range(self.num_layers)]).astype(np.float16)
             else:
                 k_store = k
@@ -107,14 +128,34 @@ class Scenario:
                 q_seq = new_q[i][layer]
                 k_seq = self.cached_k[sid][layer]
                 if self.rope_mode != ROPE_NONE:
-                    q_seq = cf.apply_rotary(q_seq, offsets[i] + np.arange(n), self.rope_scale, self.rope_theta)
+                    q_seq = cf.apply_rotary(q_seq, positions[i], self.rope_scale, self.rope_theta)
                 if self.rope_mode == ROPE_INLINE:
                     k_seq = cf.apply_rotary(k_seq, np.arange(k_seq.shape[0]), self.rope_scale, self.rope_theta)
-                expected, _ = cf.attention(q_seq, k_seq, self.cached_v[sid][layer], self.sm_scale, causal=True)
+                mask = None
+                if trees is not None:
+                    total_kv, tree_size = k_seq.shape[0], len(trees[i])
+                    mask = np.ones((n, total_kv), bool)
+                    mask[:, total_kv - tree_size:] = cf.tree_ancestor_mask(trees[i])[tree_size - n:]
+                expected, _ = cf.attention(q_seq, k_seq, self.cached_v[sid][layer], self.sm_scale, causal=True,
+                                           mask=mask)
                 assert_close(out[cursor:cursor + n], expected, atol=self.tol, rtol=self.tol,
                              what=f"attention output, layer {layer}, seq {sid}")
                 cursor += n
         cache.end_forward()
+        if accepted is not None:
+            cache.commit_accepted_token_tree_nodes(seq_ids, accepted)
+            for i, (sid, n) in enumerate(zip(seq_ids, append_lengths)):
+                path, node = [], accepted[i]
+                while node != -1:
+                    path.append(node)
+                    node = trees[i][node]
+                begin = self.cached_k[sid].shape[1] - n
+                for dst, src in enumerate(reversed(path)):
+                    self.cached_k[sid][:, begin + dst] = self.cached_k[sid][:, begin + src]
+                    self.cached_v[sid][:, begin + dst] = self.cached_v[sid][:, begin + src]
+                if n - len(path) > 0:
+                    self.cached_k[sid] = self.cached_k[sid][:, :len(path) - n]
+                    self.cached_v[sid] = self.cached_v[sid][:, :len(path) - n]
         # the sliding window takes effect after the step: keep the attention sink and the newest tokens
         # (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_cpu.py:566-590)
         for sid in seq_ids:
@@ -263,3 +304,35 @@ def run_sliding_window_fork(sc):
     sc.step([(0, 9), (1, 15), (2, 4), (3, 10), (4, 3), (5, 7)])
     sc.fork_with_window(3, 6, 18, 25, 24)
     sc.step([(3, 10), (6, 12)])
+
+
+def run_tree_attn(sc):
+    """test_paged_attention_kv_cache_tree_attn
+    (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_tir.py:1053-1134)."""
+    from tests.util import REFERENCE_TREES
+    prefill = [(0, 10), (1, 20), (2, 30), (3, 40)]
+    tree_step = [(0, 7), (1, 15), (2, 10), (3, 14)]
+    decode = [(0, 1), (1, 1), (2, 1), (3, 1)]
+    # trees, one of them a chain; commit; plain decode
+    sc.step(list(prefill))
+    sc.step(list(tree_step), trees=[list(t) for t in REFERENCE_TREES], accepted=[6, 11, 6, 13])
+    for _ in range(5):
+        sc.step(list(decode))
+    # every tree is a chain
+    sc.cache.clear()
+    sc.cached_k.clear()
+    sc.cached_v.clear()
+    sc.step(list(prefill))
+    sc.step(list(tree_step), trees=[list(range(-1, n - 1)) for n in (7, 15, 10, 14)], accepted=[2, 6, -1, 4])
+    for _ in range(5):
+        sc.step(list(decode))
+    # trees grown level by level over five steps against the cached tokens, committed at the end
+    sc.cache.clear()
+    sc.cached_k.clear()
+    sc.cached_v.clear()
+    sc.step(list(prefill))
+    for i in range(5):
+        leaves = 2 ** i
+        parents = [(k - 1) // 2 for k in range(2 * leaves - 1)]
+        sc.step([(sid, leaves) for sid in range(4)], trees=[list(parents) for _ in range(4)],
+                accepted=None if i != 4 else [2, 6, -1, 4])

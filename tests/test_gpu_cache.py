@@ -166,6 +166,17 @@ def test_sliding_window_scenarios_on_the_gpu(runner):
     runner(sc)
 
 
+@pytest.mark.parametrize("d,rope_mode", [(128, S.ROPE_NORMAL), (64, S.ROPE_NORMAL), (128, S.ROPE_NONE)])
+def test_token_tree_scenario_on_the_gpu(d, rope_mode):
+    """test_paged_attention_kv_cache_tree_attn of the reference
+    (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_tir.py:1053-1134): tree attention
+    over new tokens and over appended tree nodes, commit with the compaction copy, decode after it."""
+    layers, hq, hkv = 2, 32, 4
+    cache = GpuCache([32, 2048, 512, 16, 0], layers, hq, hkv, d, d, rope_mode=rope_mode)
+    sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=rope_mode, seed=8, tol=4e-3)
+    S.run_tree_attn(sc)
+
+
 def test_padded_qkv_rows_are_ignored():
     """qkv / out may carry more rows than the batch appends (src/runtime/vm/paged_kv_cache.cc:1330-1354)."""
     layers, hq, hkv, d = 1, 8, 2, 128

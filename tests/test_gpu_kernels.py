@@ -379,6 +379,64 @@ def test_prefill_inline_rope_plain_cache(hq, hkv, d, causal):
     assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="inline rope paged lse")
 
 
+# ------------------------------------------------------------------------------ token trees
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("rotary", [0, 1])
+def test_tree_attn_ragged_against_oracle(hq, hkv, d, rotary):
+    from tests.util import REFERENCE_TREES, random_forest, tree_order
+    rng = np.random.default_rng(40)
+    trees = REFERENCE_TREES + [random_forest(rng, 200), [-1], list(range(-1, 69))]
+    lens = [len(t) for t in trees]
+    n = sum(lens)
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    mask = np.concatenate([tree_order(t) for t in trees])
+    # positions: the depth of the node in its tree on top of a per-sequence offset, as the cache hands out
+    depth = []
+    for i, t in enumerate(trees):
+        dep = []
+        for parent in t:
+            dep.append(0 if parent == -1 else dep[parent] + 1)
+        depth += [100 * i + x for x in dep]
+    q_pos = np.array(depth, np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    ok.tree_attn_ragged(q, indptr, k, v, indptr, q_pos, indptr, mask, eo, el, rotary, 1.0, 1e4, d ** -0.5)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_tree_attn(dev(q), i32(indptr), dev(k), dev(v), i32(indptr), i32(q_pos), i32(indptr), i32(mask), go, gl,
+                      rotary, 1.0, 1e4, d ** -0.5)
+    assert_close(host(go), eo, what="tree ragged out")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="tree ragged lse")
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+def test_tree_attn_paged_against_oracle(hq, hkv, d):
+    from tests.test_oracle_kernels import tree_paged_case
+    from tests.util import REFERENCE_TREES, random_forest
+    rng = np.random.default_rng(41)
+    prefix = [10, 20, 30, 40, 0, 700, 129]
+    trees = REFERENCE_TREES + [random_forest(rng, 50), random_forest(rng, 256), random_forest(rng, 31)]
+    new_lens = [7, 8, 10, 7, 50, 256, 16]  # some trees already had nodes from earlier steps
+    (pages, pindptr, pvalues, last, ks, vs, qindptr, q, tindptr, labels, masks) = tree_paged_case(
+        rng, prefix, trees, new_lens, hq, hkv, d, npages=128)
+    n = len(q)
+    zb, zq = np.zeros(len(trees), np.int32), np.zeros(n, np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    ok.tree_attn_paged(q, qindptr, pages, pindptr, pvalues, last, zb, zq, eo, el, 0, 1.0, 1e4, d ** -0.5,
+                       tindptr, labels)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.tree_attn_paged_kv(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(zb), i32(zq),
+                         go, gl, 0, 1.0, 1e4, d ** -0.5, i32(tindptr), i32(labels))
+    assert_close(host(go), eo, what="tree paged out")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="tree paged lse")
+    with pytest.raises(KVError, match="inline rotary mode is not supported in tree attention"):
+        K.tree_attn_paged_kv(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(zb),
+                             i32(zq), go, gl, 1, 1.0, 1e4, d ** -0.5, i32(tindptr), i32(labels))
+
+
 def test_chunked_prefill_composition_matches_oracle():
     """ragged(causal) + paged(non-causal) + merge_state: the chunked-prefill path of the cache."""
     rng = np.random.default_rng(12)

@@ -252,3 +252,18 @@ def test_sliding_window_scenarios_on_the_oracle(runner):
     cache = OraclePagedKVCache([32, 2048, 512, ps, 1], layers, hq, hkv, d, d, rope_mode=S.ROPE_INLINE)
     sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=S.ROPE_INLINE, seed=4)
     runner(sc)
+
+
+@pytest.mark.parametrize("rope_mode", [S.ROPE_NORMAL, S.ROPE_NONE])
+def test_token_tree_scenario_on_the_oracle(rope_mode):
+    """Speculative decoding: tree-masked attention over new tokens and over appended tree nodes,
+    commit of an accepted path (slots compacted, the rest popped), then plain decode."""
+    layers, hq, hkv, d, ps = 2, 8, 2, 64, 16
+    cache = OraclePagedKVCache([32, 2048, 512, ps, 0], layers, hq, hkv, d, d, rope_mode=rope_mode)
+
+    def on_step(seq_ids, lens):
+        check_pool_invariants(cache.host.state(), cache.host.num_total_pages, ps)
+
+    sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=rope_mode, seed=6, on_step=on_step)
+    S.run_tree_attn(sc)
+    check_pool_invariants(cache.host.state(), cache.host.num_total_pages, ps)

@@ -9,7 +9,7 @@ import pytest
 
 from oracle import closed_form as cf
 from oracle import kernels as ok
-from tests.util import assert_close, build_paged_kv
+from tests.util import REFERENCE_TREES, assert_close, build_paged_kv, random_forest, tree_order
 
 F16 = np.float16
 
@@ -252,6 +252,114 @@ def test_inline_rope_equals_rope_then_attend():
     q_rot = cf.apply_rotary(q_raw, [100 + n - 1]).astype(F16)
     eo, el = cf.attention(q_rot, k_rot, v, d ** -0.5, causal=False)
     assert_close(out_inline[0], eo[0], atol=3e-3, rtol=3e-3, what="inline rope out")
+
+
+# ----------------------------------------------------------------------------- token trees
+def test_tree_order_interval_test_is_the_ancestor_relation():
+    """What the kernels evaluate on the (first, second) labels equals the mask built from the parent
+    pointers, for the reference's trees and random forests."""
+    rng = np.random.default_rng(30)
+    trees = REFERENCE_TREES + [random_forest(rng, n) for n in (1, 2, 9, 40, 256)]
+    for parents in trees:
+        lab = tree_order(parents).astype(np.int64)
+        sees = (lab[:, None, 0] >= lab[None, :, 0]) & (lab[:, None, 0] < lab[None, :, 1])
+        assert np.array_equal(sees, cf.tree_ancestor_mask(parents)), parents
+
+
+def _tree_ragged_case(rng, trees, hq, hkv, d):
+    lens = [len(t) for t in trees]
+    n = sum(lens)
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    mask = np.concatenate([tree_order(t) for t in trees])
+    return indptr, q, k, v, mask
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (4, 4, 64)])
+def test_tree_attn_ragged_matches_closed_form(hq, hkv, d):
+    rng = np.random.default_rng(31)
+    trees = REFERENCE_TREES + [random_forest(rng, 70)]
+    indptr, q, k, v, mask = _tree_ragged_case(rng, trees, hq, hkv, d)
+    out = np.zeros_like(q)
+    lse = np.zeros(q.shape[:2], np.float32)
+    ok.tree_attn_ragged(q, indptr, k, v, indptr, np.zeros(len(q), np.int32), indptr, mask, out, lse,
+                        0, 1.0, 1e4, d ** -0.5)
+    for i, parents in enumerate(trees):
+        s, e = indptr[i], indptr[i + 1]
+        eo, el = cf.attention(q[s:e], k[s:e], v[s:e], d ** -0.5, mask=cf.tree_ancestor_mask(parents))
+        assert_close(out[s:e], eo, atol=2e-3, rtol=2e-3, what=f"tree out seq {i}")
+        assert_close(lse[s:e], el, atol=1e-3, rtol=1e-4, what=f"tree lse seq {i}")
+    # a root sees only itself
+    assert np.array_equal(out[0], np.repeat(v[0], hq // hkv, axis=0))
+
+
+def test_tree_attn_on_chains_is_causal_attention():
+    rng = np.random.default_rng(32)
+    hq, hkv, d = 8, 2, 64
+    trees = [list(range(-1, n - 1)) for n in (1, 7, 33)]
+    indptr, q, k, v, mask = _tree_ragged_case(rng, trees, hq, hkv, d)
+    zeros = np.zeros(len(q), np.int32)
+    o1, o2 = np.zeros_like(q), np.zeros_like(q)
+    l1, l2 = np.zeros(q.shape[:2], np.float32), np.zeros(q.shape[:2], np.float32)
+    ok.tree_attn_ragged(q, indptr, k, v, indptr, zeros, indptr, mask, o1, l1, 0, 1.0, 1e4, 0.125)
+    ok.prefill_ragged(q, indptr, k, v, indptr, zeros, np.zeros(3, np.int32), o2, l2, 1, 0, 1.0, 1e4, 0.125)
+    assert np.array_equal(o1, o2) and np.array_equal(l1, l2)
+
+
+def tree_paged_case(rng, prefix_lens, trees, new_lens, hq, hkv, d, ps=16, npages=64):
+    """Sequences whose pages hold a prefix followed by the nodes of a token tree; the queries are
+    the last new_lens[i] nodes of each tree (a tree can grow over several steps)."""
+    kv_lens = [p + len(t) for p, t in zip(prefix_lens, trees)]
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, kv_lens, npages, hkv, ps, d)
+    qindptr = np.concatenate([[0], np.cumsum(new_lens)]).astype(np.int32)
+    q = rng.standard_normal((int(qindptr[-1]), hq, d)).astype(F16)
+    tindptr = np.concatenate([[0], np.cumsum([len(t) for t in trees])]).astype(np.int32)
+    labels = np.concatenate([tree_order(t) for t in trees])
+    masks = []
+    for p, t, nq in zip(prefix_lens, trees, new_lens):
+        m = np.ones((nq, p + len(t)), bool)
+        m[:, p:] = cf.tree_ancestor_mask(t)[len(t) - nq:]
+        masks.append(m)
+    return pages, pindptr, pvalues, last, ks, vs, qindptr, q, tindptr, labels, masks
+
+
+def test_tree_attn_paged_matches_closed_form():
+    rng = np.random.default_rng(33)
+    hq, hkv, d = 8, 2, 128
+    prefix = [10, 20, 30, 40, 0]
+    trees = REFERENCE_TREES + [random_forest(rng, 50)]
+    new_lens = [7, 8, 10, 7, 50]  # sequences 1 and 3: the tree already had nodes from earlier steps
+    (pages, pindptr, pvalues, last, ks, vs, qindptr, q, tindptr, labels, masks) = tree_paged_case(
+        rng, prefix, trees, new_lens, hq, hkv, d)
+    out = np.zeros_like(q)
+    lse = np.zeros(q.shape[:2], np.float32)
+    zb = np.zeros(len(trees), np.int32)
+    ok.tree_attn_paged(q, qindptr, pages, pindptr, pvalues, last, zb, np.zeros(len(q), np.int32), out, lse,
+                       0, 1.0, 1e4, d ** -0.5, tindptr, labels)
+    for i in range(len(trees)):
+        s, e = qindptr[i], qindptr[i + 1]
+        eo, el = cf.attention(q[s:e], ks[i], vs[i], d ** -0.5, mask=masks[i])
+        assert_close(out[s:e], eo, atol=2e-3, rtol=2e-3, what=f"tree paged out seq {i}")
+        assert_close(lse[s:e], el, atol=1e-3, rtol=1e-4, what=f"tree paged lse seq {i}")
+
+
+def test_tree_attn_paged_on_chains_is_causal_paged_prefill():
+    rng = np.random.default_rng(34)
+    hq, hkv, d = 4, 2, 64
+    prefix = [5, 31]
+    trees = [list(range(-1, 8)), list(range(-1, 19))]
+    new_lens = [9, 4]
+    (pages, pindptr, pvalues, last, ks, vs, qindptr, q, tindptr, labels, masks) = tree_paged_case(
+        rng, prefix, trees, new_lens, hq, hkv, d)
+    zb, zq = np.zeros(2, np.int32), np.zeros(len(q), np.int32)
+    o1, o2 = np.zeros_like(q), np.zeros_like(q)
+    l1, l2 = np.zeros(q.shape[:2], np.float32), np.zeros(q.shape[:2], np.float32)
+    ok.tree_attn_paged(q, qindptr, pages, pindptr, pvalues, last, zb, zq, o1, l1, 0, 1.0, 1e4, 0.125,
+                       tindptr, labels)
+    ok.prefill_paged(q, qindptr, pages, pindptr, pvalues, last, zb, zq, o2, l2, 1, 0, 1.0, 1e4, 0.125)
+    assert np.array_equal(o1, o2) and np.array_equal(l1, l2)
 
 
 # ----------------------------------------------------------------------------- merge

@@ -49,3 +49,42 @@ def build_paged_kv(rng, kv_lens, num_pages, hkv, page_size, d, permute=True, sca
         vs.append(v)
     return (pages, np.array(indptr, np.int32), np.array(values, np.int32),
             np.array(last, np.int32), ks, vs)
+
+
+# Token trees of the reference's speculative-decoding test
+# (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_tir.py:1076-1081)
+REFERENCE_TREES = [
+    [-1, 0, 0, 1, 1, 2, 2],  # complete binary tree of height 3
+    [-1, 0, 0, 1, 1, 2, 2, 3, 3, 4, 4, 5, 5, 6, 6],  # complete binary tree of height 4
+    [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8],  # chain of length 10
+    [-1, 0, 0, 1, 1, 2, 2, -1, 7, 7, 8, 8, 9, 9],  # two complete binary trees of height 3
+]
+
+
+def random_forest(rng, n, p_root=0.15):
+    """Parent pointers of a random forest: parent[i] < i, -1 for roots."""
+    return [-1 if (i == 0 or rng.random() < p_root) else int(rng.integers(0, i)) for i in range(n)]
+
+
+def tree_order(parent_ptr):
+    """(n, 2) int32 labels a cache hands to the tree-attention kernels: the pre-order number of
+    each node (roots and children in index order) and the end of the range its subtree covers."""
+    n = len(parent_ptr)
+    children = {}
+    for node, parent in enumerate(parent_ptr):
+        children.setdefault(parent, []).append(node)
+    labels = np.zeros((n, 2), np.int32)
+    counter = 0
+    for root in children.get(-1, []):
+        stack = [(root, False)]
+        while stack:
+            node, done = stack.pop()
+            if done:
+                labels[node, 1] = counter
+                continue
+            labels[node, 0] = counter
+            counter += 1
+            stack.append((node, True))
+            for child in reversed(children.get(node, [])):
+                stack.append((child, False))
+    return labels

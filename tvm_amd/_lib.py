@@ -31,6 +31,9 @@ SIGNATURES = {
                                                    c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_decode_paged_kv": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32, c_i32,
                                                  c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_batch_tree_attn": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_tree_attn_paged_kv": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_vp, c_vp, c_i32, c_i64, c_i64, c_i64,
+                                               c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_prefill_paged_kv_mla": [c_vp] * 8 + [c_i64, c_f64, c_i32, c_i64, c_i64, c_i64, c_i32, c_i32,
                                                       c_i32, c_i32, c_vp],
     "tvmkv_merge_state_inplace": [c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_i32, c_vp],

@@ -65,6 +65,10 @@ struct PrefillParams {
   const int32_t* k_rope_pos_offset;  // (B) position of logical key 0 (inline RoPE)
   int rotary;
   float rope_scale;
+  // token-tree mask (python/tvm/relax/frontend/nn/llm/tree_attn.py:48-65), or NULL
+  const int32_t* tree_indptr;  // (B + 1) first tree node of each sequence
+  const int32_t* tree_order;   // (nodes, 2): pre-order number of the node, end of its subtree's range
+  int k_pos_from_q;            // ragged tree attention under inline RoPE: key t sits at q_rope_position[t]
 };
 
 // theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
@@ -109,9 +113,12 @@ constexpr size_t prefill_lds_bytes(int dqk, int dv) {
 //    (python/tvm/relax/frontend/nn/llm/_kernel_common.py:155-170);
 //  * the per-layer sliding-window mask of _kernel_common.py:138-144;
 //  * inline RoPE: q at q_rope_position[token], key t at k_rope_pos_offset[b] + t
-//    (_prefill_kernels.py:119-147).
+//    (_prefill_kernels.py:119-147);
+//  * the token-tree mask of speculative decoding: the last keys of a sequence are the nodes of its
+//    token tree, a query node sees the keys before the tree and its ancestors (tree_attn.py:48-65).
 // Attention does not depend on the order of the keys, so the tiles are still walked in physical
-// order; every tile takes the masked path and masks are evaluated per element.
+// order.  Masks are evaluated per element; only a plain cache without RoPE keeps the unmasked
+// path, for the tiles in front of the tree.
 template <int DQK, int DV, bool PAGED, int PS, bool EXT>
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
   static_assert(DQK % 64 == 0 && DV % 64 == 0, "feature dims must be multiples of 64");
@@ -211,6 +218,20 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   // wave_limit_min everything is visible to all of them (plain cache only)
   const int wave_limit_max = to_phys(!wave_active ? 0 : (causal_rows ? min(kv_len, causal_shift + last_row_wave / group) : kv_len));
   const int wave_limit_min = !wave_active ? 0 : (causal_rows ? min(kv_len, causal_shift + first_row_wave / group) : kv_len);
+
+  // token tree: keys from tree_start on are tree nodes; this row's node is my_pos + tree_len - qo_len
+  int tree_len = 0, tree_start = kv_len, child_first = 0;
+  const int32_t* tree_base = nullptr;
+  if (EXT && p.tree_order != nullptr) {
+    const int first_node = p.tree_indptr[b];
+    tree_len = p.tree_indptr[b + 1] - first_node;
+    tree_start = kv_len - tree_len;
+    tree_base = p.tree_order + 2 * static_cast<int64_t>(first_node);
+    if (tree_len > 0) child_first = tree_base[2 * min(max(my_pos + tree_len - qo_len, 0), tree_len - 1)];
+  }
+  // tiles that end at or before this (physical = logical) index need no mask at all
+  const bool plain_ext = EXT && !p.rotary && p.sink_size == nullptr;
+  const int unmasked_limit = !EXT ? wave_limit_min : (plain_ext ? min(wave_limit_min, max(tree_start, 0)) : 0);
 
   half8_t qf[KS];
   {
@@ -418,7 +439,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     // no prefetch across a 64-tile window of page ids: the ids held are those of the last copy issued
     const int next = tile + NSTAGE - 1;  // the tile whose copy this iteration issues
     const bool has_next = next < n_tiles;
-    const bool unmasked = !EXT && TB == 2 && kv0 < wave_limit_max && kv0 + BN <= wave_limit_min;  // wave-uniform
+    const bool unmasked = TB == 2 && kv0 < wave_limit_max && kv0 + BN <= unmasked_limit;  // wave-uniform
     if (has_next) issue_tile(next);
 
     if (kv0 >= wave_limit_max) continue;  // wave-uniform: every row of this wave is masked out
@@ -469,7 +490,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
         // this lane's key row is physical token t0 + col; its logical index is its position
         const int t = min(t0 + col, last_tok);
         const int logical = t < sink ? t : t - win_lo + sink;
-        const float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
+        float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
+        if (!PAGED && p.k_pos_from_q) pos = static_cast<float>(p.q_rope_position[kv_start + t]) * p.rope_scale;
 #pragma unroll
         for (int ks = 0; ks < KS / 2; ++ks) rope_pair(kf[ks], kf[ks + KS / 2], pos, div_lds + ks * 16 + half * 8);
       }
@@ -479,12 +501,20 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
       __builtin_amdgcn_sched_barrier(0);
       if (EXT) {
         // element j is physical token t0 + half*4 + (j/4)*8 + j%4
+        const int block_last = t0 + 31;
+        const bool in_tree = tree_len > 0 && (block_last < sink ? block_last : block_last - win_lo + sink) >= tree_start;  // wave-uniform
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
           const int t = t0 + half * 4 + (j >> 2) * 8 + (j & 3);
           const bool cached = t < sink || (t >= win_lo && t < phys_len);
           const int logical = t < sink ? t : t - win_lo + sink;
-          acc[j] = (cached && logical < my_limit && logical >= my_lo) ? acc[j] : -3.0e38f;
+          bool visible = cached && logical < my_limit && logical >= my_lo;
+          if (in_tree) {
+            const int node = min(max(logical - tree_start, 0), tree_len - 1);
+            const int first = tree_base[2 * node], second = tree_base[2 * node + 1];
+            visible = visible && (logical < tree_start || (child_first >= first && child_first < second));
+          }
+          acc[j] = visible ? acc[j] : -3.0e38f;
         }
       } else if (t0 + 32 > wave_limit_min) {  // wave-uniform
         asm volatile("" ::: "memory");  // keep this a branch: if-converted it costs 5 ops per element everywhere
@@ -655,6 +685,102 @@ int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const v
     launch_prefill<64, 64, true, 16>(p, total_q, ext, rope_theta, s);
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_paged_kv: head_dim " << d << " is not built (64, 128)";
+  }
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                          const int32_t* kv_indptr, const int32_t* q_rope_position, const int32_t* mn_indptr,
+                          const int32_t* mask, void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                          double rope_theta, double sm_scale, int32_t batch_size, int64_t total_q, int32_t h_q,
+                          int32_t h_kv, int32_t d, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0) << "batch_tree_attn: bad shape";
+  if (batch_size == 0 || total_q == 0) return TVMKV_OK;
+  KV_CHECK(q && q_indptr && k && v && kv_indptr && mn_indptr && mask && output && lse) << "batch_tree_attn: NULL tensor";
+  KV_CHECK(rotary_mode == 0 || q_rope_position) << "batch_tree_attn: inline RoPE needs the position array";
+  PrefillParams p{};
+  p.q = static_cast<const half_t*>(q);
+  p.q_indptr = q_indptr;
+  p.k = static_cast<const half_t*>(k);
+  p.v = static_cast<const half_t*>(v);
+  p.kv_indptr = kv_indptr;
+  p.output = static_cast<half_t*>(output);
+  p.lse = lse;
+  p.batch_size = batch_size;
+  p.h_q = h_q;
+  p.h_kv = h_kv;
+  p.group = h_q / h_kv;
+  p.causal = 0;
+  p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
+  p.rotary = rotary_mode != 0;
+  p.rope_scale = static_cast<float>(rope_scale);
+  p.q_rope_position = q_rope_position;
+  p.k_rope_pos_offset = q_indptr;  // not used: keys take their positions from q_rope_position
+  p.k_pos_from_q = 1;
+  p.tree_indptr = mn_indptr;
+  p.tree_order = mask;
+  hipStream_t s = as_stream(stream);
+  if (d == 128) {
+    launch_prefill<128, 128, false, 16>(p, total_q, true, rope_theta, s);
+  } else if (d == 64) {
+    launch_prefill<64, 64, false, 16>(p, total_q, true, rope_theta, s);
+  } else {
+    KV_UNSUPPORTED(true) << "batch_tree_attn: head_dim " << d << " is not built (64, 128)";
+  }
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void* pages, const int32_t* page_indptr,
+                             const int32_t* page_values, const int32_t* length_info,
+                             const int32_t* k_rope_pos_offset, const int32_t* q_rope_position, void* output,
+                             float* lse, int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                             const int32_t* tree_order_indptr, const int32_t* tree_order, int32_t batch_size,
+                             int64_t total_q, int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                             int32_t d, int32_t page_size, int32_t sliding_window, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
+      << "tree_attn_paged_kv: bad shape";
+  KV_UNSUPPORTED(page_size != 16) << "tree_attn_paged_kv: page_size " << page_size << " is not built (16)";
+  // the reference kernel asserts the same (tree_attn.py:700-702)
+  KV_UNSUPPORTED(rotary_mode != 0) << "tree_attn_paged_kv: inline rotary mode is not supported in tree attention";
+  if (batch_size == 0 || total_q == 0) return TVMKV_OK;
+  KV_CHECK(q && q_indptr && pages && page_indptr && length_info && output && lse && tree_order_indptr && tree_order)
+      << "tree_attn_paged_kv: NULL tensor";
+  KV_CHECK(nnz_pages == 0 || page_values) << "tree_attn_paged_kv: NULL page table";
+  PrefillParams p{};
+  p.q = static_cast<const half_t*>(q);
+  p.q_indptr = q_indptr;
+  p.pages = static_cast<const half_t*>(pages);
+  p.page_indptr = page_indptr;
+  p.page_values = page_values;
+  p.last_page_len = length_info;
+  p.output = static_cast<half_t*>(output);
+  p.lse = lse;
+  p.batch_size = batch_size;
+  p.h_q = h_q;
+  p.h_kv = h_kv;
+  p.group = h_q / h_kv;
+  p.causal = 0;
+  p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
+  p.rope_scale = static_cast<float>(rope_scale);
+  p.q_rope_position = q_rope_position;
+  p.k_rope_pos_offset = k_rope_pos_offset;
+  if (sliding_window != 0) {  // length_info is (3, B): last_page_len, window offset, sink size
+    p.window_offset = length_info + batch_size;
+    p.sink_size = length_info + 2 * static_cast<int64_t>(batch_size);
+  }
+  p.tree_indptr = tree_order_indptr;
+  p.tree_order = tree_order;
+  hipStream_t s = as_stream(stream);
+  if (d == 128) {
+    launch_prefill<128, 128, true, 16>(p, total_q, true, rope_theta, s);
+  } else if (d == 64) {
+    launch_prefill<64, 64, true, 16>(p, total_q, true, rope_theta, s);
+  } else {
+    KV_UNSUPPORTED(true) << "tree_attn_paged_kv: head_dim " << d << " is not built (64, 128)";
   }
   KV_LAUNCH_CHECK();
   KV_API_END();

@@ -660,7 +660,14 @@ class PagedKVCache {
     KV_CHECK(rows == total_seq_length) << "self_attention expects " << total_seq_length << " rows, got " << rows;
     ComputeStreamWaitForCopyStream();
     KV_CHECK(!dirty_aux_data_device_) << "auxiliary data is not synchronised";
-    KV_CHECK(is_chain_on_depths_[0]) << "tree attention is not built";
+    if (!is_chain_on_depths_[0]) {
+      KV_CHECK(attn_kinds_[layer_id] == TVMKV_ATTN_MHA) << "Tree attn not able for MLA for now.";
+      KV_CHECK(k_heads == num_kv_heads_ && qk_dim == qk_head_dim_ && v_dim == v_head_dim_)
+          << "self_attention: k/v shapes do not match the cache";
+      MHASelfAttnInternal(q, k, v, o, lse, total_seq_length, sm_scale);
+      RecordComputeEvent();
+      return;
+    }
     int rotary = attn_kinds_[layer_id] == TVMKV_ATTN_MHA ? (rope_mode_ == TVMKV_ROPE_INLINE) : 0;
     Launch(tvmkv_batch_prefill_ragged_kv(q, cur_append_length_indptr_view_.ptr, k, v,
                                          cur_append_length_indptr_view_.ptr, q_rope_position_map_view_.ptr,
@@ -1143,6 +1150,11 @@ class PagedKVCache {
         HIP_CHECK(hipHostMalloc(&aux_staging_[i], aux_capacity_ * sizeof(int32_t), hipHostMallocDefault));
         HIP_CHECK(hipEventCreateWithFlags(&aux_copied_[i], hipEventDisableTiming));
       }
+      // token-tree commit: copy_length_indptr + (2, copies) positions (attn_utils.h:1010-1021)
+      commit_capacity_ = (r + 1 + 3) / 4 * 4 + 2 * std::min<int64_t>(kTreeAttnMaxTreeSize * r, c) + 4;
+      HIP_CHECK(hipMalloc(&commit_device_, commit_capacity_ * sizeof(int32_t)));
+      HIP_CHECK(hipHostMalloc(&commit_staging_, commit_capacity_ * sizeof(int32_t), hipHostMallocDefault));
+      HIP_CHECK(hipEventCreateWithFlags(&commit_copied_, hipEventDisableTiming));
       HIP_CHECK(hipStreamCreateWithFlags(&copy_stream_, hipStreamNonBlocking));
       HIP_CHECK(hipEventCreateWithFlags(&compute_done_, hipEventDisableTiming));
     } catch (...) {
@@ -1170,6 +1182,12 @@ class PagedKVCache {
       aux_device_[i] = aux_staging_[i] = nullptr;
       aux_copied_[i] = nullptr;
     }
+    (void)hipFree(commit_device_);
+    if (commit_staging_) (void)hipHostFree(commit_staging_);
+    if (commit_copied_) (void)hipEventDestroy(commit_copied_);
+    commit_device_ = commit_staging_ = nullptr;
+    commit_copied_ = nullptr;
+    commit_staging_used_ = false;
     if (copy_stream_) (void)hipStreamDestroy(copy_stream_);
     if (compute_done_) (void)hipEventDestroy(compute_done_);
     copy_stream_ = nullptr;
@@ -1205,7 +1223,32 @@ class PagedKVCache {
     int total_copy_length = commit_copy_length_indptr_.back();
     KV_CHECK(total_copy_length >= 0) << "negative copy length";
     if (total_copy_length == 0 || device_ < 0) return;
-    KV_UNSUPPORTED(true) << "token-tree commit (compact KV copy) is not wired to the device yet";
+    HIP_CHECK(hipSetDevice(device_));
+    // one upload: [copy_length_indptr (batch + 1), padded to 16 bytes | src positions | dst positions]
+    const int64_t n_indptr = static_cast<int64_t>(commit_copy_length_indptr_.size());
+    const int64_t pos_begin = (n_indptr + 3) / 4 * 4;
+    KV_CHECK(pos_begin + 2 * static_cast<int64_t>(total_copy_length) <= commit_capacity_)
+        << "token-tree commit copies " << total_copy_length << " slots, more than the cache was sized for";
+    // the staging buffer is reused: wait until the previous commit's upload has read it
+    if (commit_staging_used_) HIP_CHECK(hipEventSynchronize(commit_copied_));
+    int32_t* staging = static_cast<int32_t*>(commit_staging_);
+    std::memcpy(staging, commit_copy_length_indptr_.data(), n_indptr * sizeof(int32_t));
+    std::memcpy(staging + pos_begin, commit_copy_src_pos_.data(), total_copy_length * sizeof(int32_t));
+    std::memcpy(staging + pos_begin + total_copy_length, commit_copy_dst_pos_.data(),
+                total_copy_length * sizeof(int32_t));
+    int32_t* device = static_cast<int32_t*>(commit_device_);
+    // after the attention kernels of the step that computed on these slots
+    if (compute_event_recorded_) HIP_CHECK(hipStreamWaitEvent(copy_stream_, compute_done_, 0));
+    HIP_CHECK(hipMemcpyAsync(device, staging, (pos_begin + 2 * total_copy_length) * sizeof(int32_t),
+                             hipMemcpyHostToDevice, copy_stream_));
+    HIP_CHECK(hipEventRecord(commit_copied_, copy_stream_));
+    commit_staging_used_ = true;
+    for (int64_t layer = 0; layer < num_layers_; ++layer) {
+      Launch(tvmkv_compact_kv_copy(pages_[layer], device, device + pos_begin, cur_batch_size_, total_copy_length,
+                                   num_total_pages_, num_kv_heads_, page_size_, qk_head_dim_, copy_stream_));
+    }
+    // The next BeginForward's first kernel waits for the copy stream (paged_kv_cache.cc:767-769).
+    copy_stream_has_work_ = true;
   }
 
   void AppendMHA(int64_t local_layer_id, int64_t total_seq_length) {
@@ -1221,13 +1264,7 @@ class PagedKVCache {
     bool is_first_kernel = true;
     if (!append_before_attn_) {
       is_first_kernel = false;
-      KV_CHECK(is_chain_on_depths_[0]) << "tree attention is not built";
-      Launch(tvmkv_batch_prefill_ragged_kv(q, cur_append_length_indptr_view_.ptr, k, v,
-                                           cur_append_length_indptr_view_.ptr, q_rope_position_map_view_.ptr,
-                                           k_ragged_rope_pos_offset_view_.ptr, output, merged_lse_, /*causal=*/1,
-                                           rope_mode_ == TVMKV_ROPE_INLINE, rotary_scale_, rotary_theta_, sm_scale,
-                                           cur_batch_size_, total_seq_length, num_qo_heads_, num_kv_heads_,
-                                           qk_head_dim_, v_head_dim_, compute_stream_));
+      MHASelfAttnInternal(q, k, v, output, merged_lse_, total_seq_length, sm_scale);
     }
     bool self_attn_computed = !is_first_kernel;
     bool cross_attn_computed = MHACrossAttnInternal(
@@ -1235,6 +1272,29 @@ class PagedKVCache {
         /*causal=*/!append_before_attn_ && attn_kinds_[layer_id] == TVMKV_ATTN_MHA_SLIDING);
     KV_CHECK(self_attn_computed || cross_attn_computed)
         << "Both self-attention and cross-attention are not computed.";
+  }
+
+  // :2182-2203
+  void MHASelfAttnInternal(const void* q, const void* k, const void* v, void* o, float* lse, int64_t total_seq_length,
+                           double sm_scale) {
+    if (is_chain_on_depths_[0]) {
+      Launch(tvmkv_batch_prefill_ragged_kv(q, cur_append_length_indptr_view_.ptr, k, v,
+                                           cur_append_length_indptr_view_.ptr, q_rope_position_map_view_.ptr,
+                                           k_ragged_rope_pos_offset_view_.ptr, o, lse, /*causal=*/1,
+                                           rope_mode_ == TVMKV_ROPE_INLINE, rotary_scale_, rotary_theta_, sm_scale,
+                                           cur_batch_size_, total_seq_length, num_qo_heads_, num_kv_heads_,
+                                           qk_head_dim_, v_head_dim_, compute_stream_));
+    } else {
+      // the batch forms token trees
+      KV_CHECK(tree_attn_mask_view_[0].ptr != nullptr && tree_attn_mn_indptr_view_[0].ptr != nullptr)
+          << "token-tree mask is not on the device";
+      KV_CHECK(qk_head_dim_ == v_head_dim_) << "tree attention needs equal qk and v head dims";
+      Launch(tvmkv_batch_tree_attn(q, cur_append_length_indptr_view_.ptr, k, v, cur_append_length_indptr_view_.ptr,
+                                   q_rope_position_map_view_.ptr, tree_attn_mn_indptr_view_[0].ptr,
+                                   tree_attn_mask_view_[0].ptr, o, lse, rope_mode_ == TVMKV_ROPE_INLINE,
+                                   rotary_scale_, rotary_theta_, sm_scale, cur_batch_size_, total_seq_length,
+                                   num_qo_heads_, num_kv_heads_, qk_head_dim_, compute_stream_));
+    }
   }
 
   // :2216-2299
@@ -1255,8 +1315,17 @@ class PagedKVCache {
       double rotary_theta = sliding_layer ? 10000 : rotary_theta_;
       double rotary_scale = sliding_layer ? 1 : rotary_scale_;
       int rotary_mode = rope_mode_ == TVMKV_ROPE_INLINE;
-      KV_CHECK(!(append_before_attn_ && !is_chain_on_depths_[d])) << "tree attention is not built";
-      if (use_decode_kernel_[d]) {
+      if (append_before_attn_ && !is_chain_on_depths_[d]) {
+        KV_CHECK(tree_attn_mask_view_[d].ptr != nullptr && tree_attn_mn_indptr_view_[d].ptr != nullptr)
+            << "token-tree mask is not on the device";
+        Launch(tvmkv_tree_attn_paged_kv(q, qo_indptr_view_[d].ptr, pages_[local_layer_id], page_indptr.ptr,
+                                        page_indices.ptr, length_info.ptr, k_rope_pos.ptr,
+                                        q_rope_position_map_view_.ptr, attn_output, attn_lse, rotary_mode,
+                                        rotary_scale, rotary_theta, sm_scale, tree_attn_mn_indptr_view_[d].ptr,
+                                        tree_attn_mask_view_[d].ptr, qo_indptr_view_[d].size - 1, total_seq_length,
+                                        page_indices.size, num_total_pages_, num_qo_heads_, num_kv_heads_,
+                                        qk_head_dim_, page_size_, sliding_window, compute_stream_));
+      } else if (use_decode_kernel_[d]) {
         Launch(tvmkv_batch_decode_paged_kv(q, pages_[local_layer_id], page_indptr.ptr, page_indices.ptr,
                                            length_info.ptr, k_rope_pos.ptr, q_rope_position_map_view_.ptr,
                                            attn_output, attn_lse, rotary_mode, rotary_scale, rotary_theta, sm_scale,
@@ -1437,6 +1506,11 @@ class PagedKVCache {
   hipEvent_t aux_copied_[2] = {nullptr, nullptr};
   bool aux_slot_used_[2] = {false, false};
   int aux_slot_ = 0;
+  int64_t commit_capacity_ = 0;
+  void* commit_device_ = nullptr;
+  void* commit_staging_ = nullptr;
+  hipEvent_t commit_copied_ = nullptr;
+  bool commit_staging_used_ = false;
   AuxView q_rope_position_map_view_, append_position_map_view_, cur_append_length_indptr_view_,
       k_ragged_rope_pos_offset_view_;
   AuxView qo_indptr_view_[kMaxBlockDepth], page_indptr_view_[kMaxBlockDepth], page_indices_view_[kMaxBlockDepth],

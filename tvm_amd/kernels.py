@@ -99,6 +99,30 @@ def batch_decode_paged_kv(q, pages, page_indptr, page_values, length_info, k_rop
         int(length_info.dim() == 2), _stream()))
 
 
+def batch_tree_attn(q, q_indptr, k, v, kv_indptr, q_rope_position, mn_indptr, mask, output, lse, rotary_mode,
+                    rope_scale, rope_theta, sm_scale):
+    _f16(q, k, v, output)
+    _i32(q_indptr, kv_indptr, q_rope_position, mn_indptr, mask)
+    check(lib().tvmkv_batch_tree_attn(
+        _p(q), _p(q_indptr), _p(k), _p(v), _p(kv_indptr), _p(q_rope_position), _p(mn_indptr), _p(mask), _p(output),
+        _p(lse), int(rotary_mode), float(rope_scale), float(rope_theta), float(sm_scale), q_indptr.shape[0] - 1,
+        q.shape[0], q.shape[1], k.shape[1], q.shape[2], _stream()))
+
+
+def tree_attn_paged_kv(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset,
+                       q_rope_position, output, lse, rotary_mode, rope_scale, rope_theta, sm_scale,
+                       tree_order_indptr, tree_order):
+    _f16(q, pages, output)
+    _i32(q_indptr, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, tree_order_indptr,
+         tree_order)
+    num_pages, _, hkv, ps, d = pages.shape
+    check(lib().tvmkv_tree_attn_paged_kv(
+        _p(q), _p(q_indptr), _p(pages), _p(page_indptr), _p(page_values), _p(length_info), _p(k_rope_pos_offset),
+        _p(q_rope_position), _p(output), _p(lse), int(rotary_mode), float(rope_scale), float(rope_theta),
+        float(sm_scale), _p(tree_order_indptr), _p(tree_order), q_indptr.shape[0] - 1, q.shape[0],
+        page_values.shape[0], num_pages, q.shape[1], hkv, d, ps, int(length_info.dim() == 2), _stream()))
+
+
 def batch_prefill_paged_kv_mla(q, q_indptr, pages, page_indptr, page_values, length_info, output, lse, causal,
                                sm_scale):
     _f16(q, pages, output)
