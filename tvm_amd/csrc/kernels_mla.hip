@@ -293,7 +293,11 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, fmaxf(mx * p.scale_log2, -1.0e30f));  // a fully masked row keeps its maximum
+    // The reference point only moves when the maximum exceeds it by more than 2^8 (p stays <= 256,
+    // same relative precision in fp16), so that after the first tiles no block rescales O; a fully
+    // masked row keeps its reference point.
+    const float cand = fmaxf(mx * p.scale_log2, -1.0e30f);
+    const float m_new = cand > m + 8.0f ? cand : m;
     const float alpha = fast_exp2(m - m_new);
     m = m_new;
     lsum *= alpha;

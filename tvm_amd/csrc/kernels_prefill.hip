@@ -380,9 +380,15 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     for (int j = 0; j < 16; ++j) mx = fmaxf(mx, acc[j]);
     return fmaxf(mx, __shfl_xor(mx, 32, 64));
   };
+  // The reference point m of the running softmax only has to bound the scores from above up to a
+  // factor that fp16 holds comfortably: it moves when a row's maximum exceeds it by more than
+  // kMaxSlack (p <= 2^kMaxSlack), so that after the first tiles almost no block rescales O.  Softmax
+  // is invariant to the shift, and p is rounded to fp16 with the same relative precision.
+  constexpr float kMaxSlack = 8.0f;
   auto advance_max = [&](float mx_raw) -> float {  // returns the factor that rescales the old state
     // a fully masked row keeps its old maximum (the scaled sentinel is far below -5e4)
-    const float m_new = fmaxf(m, fmaxf(mx_raw * p.scale_log2, -1.0e30f));
+    const float cand = fmaxf(mx_raw * p.scale_log2, -1.0e30f);
+    const float m_new = cand > m + kMaxSlack ? cand : m;
     const float alpha = fast_exp2(m - m_new);
     m = m_new;
     lsum *= alpha;
