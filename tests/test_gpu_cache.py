@@ -142,17 +142,14 @@ def test_error_paths_on_the_device_cache():
     cache.add_sequence(1)
     with pytest.raises(tvm_amd.KVError, match="The KV cache is full"):
         cache.begin_forward([1], [80])
-    # a sliding-window cache forces inline RoPE; the head_dim 64 decode kernel has none
-    c2 = GpuCache([4, 64, 32, 16, 1], 1, 8, 2, 64, 64, rope_mode=1)
+    # a kernel's refusal surfaces through the cache call: head_dim 96 is not built
+    c2 = GpuCache([4, 64, 32, 16, 0], 1, 8, 2, 96, 96, rope_mode=0)
     c2.add_sequence(0)
-    qkv64 = torch.zeros((1, 12, 64), dtype=torch.float16, device=DEV)
-    out64 = torch.zeros((1, 8, 64), dtype=torch.float16, device=DEV)
+    qkv96 = torch.zeros((1, 12, 96), dtype=torch.float16, device=DEV)
+    out96 = torch.zeros((1, 8, 96), dtype=torch.float16, device=DEV)
     c2.begin_forward([0], [1])
-    attn(c2.cache, 0, 1.0, qkv64, out64)  # nothing cached yet: the ragged prefill kernel alone
-    c2.end_forward()
-    c2.begin_forward([0], [1])
-    with pytest.raises(tvm_amd.KVError, match="inline RoPE"):
-        attn(c2.cache, 0, 1.0, qkv64, out64)
+    with pytest.raises(tvm_amd.KVError, match="is not built"):
+        attn(c2.cache, 0, 1.0, qkv96, out96)
 
 
 @pytest.mark.parametrize("runner", [S.run_sliding_window, S.run_sliding_window_fork])

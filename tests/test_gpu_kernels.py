@@ -232,13 +232,35 @@ def test_decode_inline_rope_plain_cache_and_scaled_positions():
 
 
 def test_decode_rejects_what_is_not_built():
-    t = torch.zeros((1, 8, 64), dtype=torch.float16, device=DEV)
-    pages = torch.zeros((2, 2, 2, 16, 64), dtype=torch.float16, device=DEV)
+    t = torch.zeros((1, 8, 96), dtype=torch.float16, device=DEV)
+    pages = torch.zeros((2, 2, 2, 16, 96), dtype=torch.float16, device=DEV)
     lse = torch.zeros((1, 8), dtype=torch.float32, device=DEV)
     one = i32([0, 1])
-    with pytest.raises(KVError, match="inline RoPE") as info:  # head_dim 64 has no inline-RoPE kernel
-        K.batch_decode_paged_kv(t, pages, one, i32([0]), i32([1]), i32([0]), i32([0]), t, lse, 1, 1.0, 1e4, 1.0)
+    with pytest.raises(KVError, match="head_dim 96 is not built") as info:
+        K.batch_decode_paged_kv(t, pages, one, i32([0]), i32([1]), i32([0]), i32([0]), t, lse, 0, 1.0, 1e4, 1.0)
     assert info.value.code == -2
+
+
+@pytest.mark.parametrize("rotary", [0, 1])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (16, 16, 64), (32, 1, 128)])
+def test_decode_sliding_cache_and_inline_rope_other_shapes(hq, hkv, d, rotary):
+    """Shapes outside the matrix-core decode kernel (head_dim 64, GQA groups above 16) take the paged
+    prefill kernel with one query per sequence."""
+    from tests.test_oracle_kernels import SLIDING_SPEC, sliding_case
+    rng = np.random.default_rng(26)
+    pages, pindptr, pvalues, length_info, ks, vs = sliding_case(rng, SLIDING_SPEC, hkv, d)
+    b = len(SLIDING_SPEC)
+    q = rng.standard_normal((b, hq, d)).astype(F16)
+    k_off = np.arange(b, dtype=np.int32) * 3
+    q_pos = np.array([k_off[i] + len(ks[i]) - 1 for i in range(b)], np.int32)
+    eo, el = np.zeros((b, hq, d), F16), np.zeros((b, hq), np.float32)
+    ok.decode(q, pages, pindptr, pvalues, length_info, k_off, q_pos, eo, el, rotary, 1.0, 1e4, d ** -0.5)
+    go = torch.full((b, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((b, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_decode_paged_kv(dev(q), dev(pages), i32(pindptr), i32(pvalues), i32(length_info), i32(k_off), i32(q_pos),
+                            go, gl, rotary, 1.0, 1e4, d ** -0.5)
+    assert_close(host(go), eo, what="decode (prefill path) out")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="decode (prefill path) lse")
 
 
 # ------------------------------------------------------------------------------ prefill

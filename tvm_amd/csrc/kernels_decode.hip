@@ -659,6 +659,11 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   }  // items
 }
 
+__global__ void iota_kernel(int32_t* out, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = i;
+}
+
 // ---- per-device workspace for the partial states, grown on demand --------------------------
 struct Workspace {
   void* ptr = nullptr;
@@ -729,14 +734,30 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
   KV_CHECK(batch_size >= 0 && nnz_pages >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_decode_paged_kv: bad shape";
   const bool ext = rotary_mode != 0 || sliding_window != 0;
-  KV_UNSUPPORTED(ext && !(d == 128 && h_q / h_kv <= 16))
-      << "batch_decode_paged_kv: inline RoPE (rotary_mode=1) and sliding-window length_info (3, B) are built "
-         "for head_dim 128 and GQA groups up to 16 only";
   KV_UNSUPPORTED(page_size != 16) << "batch_decode_paged_kv: page_size " << page_size << " is not built (16)";
   KV_UNSUPPORTED(d != 64 && d != 128) << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 128)";
   if (batch_size == 0) return TVMKV_OK;
   KV_CHECK(q && pages && page_indptr && length_info && output && lse) << "batch_decode_paged_kv: NULL tensor";
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_decode_paged_kv: NULL page table";
+
+  if (ext && !(d == 128 && h_q / h_kv <= 16)) {
+    // Inline RoPE and the sliding-window length_info (3, B) are built into the matrix-core kernel
+    // only (head_dim 128, GQA groups up to 16).  Other shapes run as a paged prefill with one query
+    // per sequence, which has both: one workgroup per (sequence, kv head), no split over the keys.
+    int32_t* q_indptr = reinterpret_cast<int32_t*>(
+        static_cast<char*>(get_workspace(kArrivalBytes + (static_cast<size_t>(batch_size) + 1) * sizeof(int32_t))) +
+        kArrivalBytes);
+    hipStream_t s = as_stream(stream);
+    hipLaunchKernelGGL(iota_kernel, dim3((batch_size + 256) / 256), dim3(256), 0, s, q_indptr, batch_size + 1);
+    KV_LAUNCH_CHECK();
+    const int rc = tvmkv_batch_prefill_paged_kv(q, q_indptr, pages, page_indptr, page_values, length_info,
+                                                k_rope_pos_offset, q_rope_position, output, lse, /*causal=*/0,
+                                                rotary_mode, rope_scale, rope_theta, sm_scale, batch_size, batch_size,
+                                                nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window,
+                                                /*sliding_window_size=*/0, stream);
+    if (rc != TVMKV_OK) return rc;
+    return TVMKV_OK;
+  }
 
   DecodeParams p;
   p.q = static_cast<const half_t*>(q);
