@@ -546,7 +546,9 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
+    // the reference point moves only when the maximum exceeds it by more than 2^8 (p stays <= 256):
+    // after the first steps almost no step rescales O
+    const float m_new = mx > m + 8.0f ? mx : m;
     const float alpha = fast_exp2(m - m_new);
     m = m_new;
     lsum *= alpha;
