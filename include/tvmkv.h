@@ -116,6 +116,23 @@ int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const v
                                  int32_t h_kv, int32_t d, int32_t page_size, int32_t sliding_window,
                                  int32_t sliding_window_size, void* stream);
 
+/* Slot 16 followed by slot 23 in one launch; no counterpart among the reference's kernels.
+ * `output` / `lse` already hold an attention state of the same query rows (what the ragged kernel
+ * wrote for the new tokens, paged_kv_cache.cc:2169-2172); the attention over the pages is merged
+ * into it in the kernel's epilogue with the arithmetic of `merge_state_inplace`
+ * (_decode_kernels.py:441-450), so the temporary output and the separate merge pass of
+ * paged_kv_cache.cc:2285-2292 are not needed.  Arguments as tvmkv_batch_prefill_paged_kv. */
+int tvmkv_batch_prefill_paged_kv_merge(const void* q, const int32_t* q_indptr, const void* pages,
+                                       const int32_t* page_indptr, const int32_t* page_values,
+                                       const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                                       const int32_t* q_rope_position, void* output, float* lse,
+                                       int64_t causal, int64_t rotary_mode, double rope_scale,
+                                       double rope_theta, double sm_scale, int32_t batch_size,
+                                       int64_t total_q, int64_t nnz_pages, int64_t num_pages,
+                                       int32_t h_q, int32_t h_kv, int32_t d, int32_t page_size,
+                                       int32_t sliding_window, int32_t sliding_window_size,
+                                       void* stream);
+
 /* Slots 17/19 paged decode -- replaces `batch_decode_paged_kv`
  * (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:181-411; llvm form :49-178), calling
  * convention attn_backend.h:511-514:

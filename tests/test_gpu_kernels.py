@@ -484,6 +484,13 @@ def test_chunked_prefill_composition_matches_oracle():
     K.batch_prefill_ragged_kv(qd, i32(ind), dev(k), dev(v), i32(ind), i32(zq), i32(zb), go, gl, 1, 0, 1.0, 1e4, d ** -0.5)
     K.batch_prefill_paged_kv(qd, i32(ind), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(zb), i32(zq), ho, hl,
                              0, 0, 1.0, 1e4, d ** -0.5)
+    go2, gl2 = go.clone(), gl.clone()
     K.merge_state_inplace(go, gl, ho, hl)
     assert_close(host(go), eo, what="chunked prefill out")
     assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="chunked prefill lse")
+    # the same with the merge done in the paged kernel's epilogue (sequence 1 has no pages: unchanged)
+    K.batch_prefill_paged_kv(qd, i32(ind), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(zb), i32(zq), go2,
+                             gl2, 0, 0, 1.0, 1e4, d ** -0.5, merge_into=True)
+    assert_close(host(go2), eo, what="chunked prefill out, merged in the epilogue")
+    assert_close(host(gl2), el, atol=2e-3, rtol=1e-4, what="chunked prefill lse, merged in the epilogue")
+    assert_close(host(go2), host(go), atol=2e-3, rtol=2e-3, what="epilogue merge vs separate merge")

@@ -69,6 +69,9 @@ struct PrefillParams {
   const int32_t* tree_indptr;  // (B + 1) first tree node of each sequence
   const int32_t* tree_order;   // (nodes, 2): pre-order number of the node, end of its subtree's range
   int k_pos_from_q;            // ragged tree attention under inline RoPE: key t sits at q_rope_position[t]
+  // != 0: output / lse already hold an attention state of the same rows, and this kernel's state is
+  // merged into it (the arithmetic of merge_state_inplace) instead of overwriting it
+  int merge_into;
 };
 
 // theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
@@ -540,17 +543,46 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   if (row_valid) {
     const float inv = 1.0f / denom;
     half_t* orow = p.output + (static_cast<int64_t>(q_start + my_pos) * p.h_q + my_head) * DV + half * 4;
+    float* lse_ptr = p.lse + static_cast<int64_t>(q_start + my_pos) * p.h_q + my_head;
+    const float my_lse = m + fast_log2(denom);
+    if (p.merge_into) {
+      // python/tvm/relax/frontend/nn/llm/_decode_kernels.py:441-450 with (v, s) = what the arrays
+      // hold and (v_other, s_other) = this kernel's state; both lanes of a row read s before lane
+      // `half == 0` overwrites it (one wavefront, program order)
+      const float s_prev = *lse_ptr;
+      const float s_max = fmaxf(s_prev, my_lse);
+      const float w_prev = fast_exp2(s_prev - s_max);
+      const float w_mine = fast_exp2(my_lse - s_max);
+      const float scale_prev = w_prev / (w_prev + w_mine);
+      const float scale_mine = w_mine / (w_prev + w_mine) * inv;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+      for (int db = 0; db < DB; ++db) {
 #pragma unroll
-      for (int j4 = 0; j4 < 4; ++j4) {
-        half4_t out4;
+        for (int j4 = 0; j4 < 4; ++j4) {
+          half4_t* dst = reinterpret_cast<half4_t*>(orow + db * 32 + j4 * 8);
+          const half4_t prev = *dst;
+          half4_t out4;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) out4[e] = static_cast<half_t>(o[db][j4 * 4 + e] * inv);
-        *reinterpret_cast<half4_t*>(orow + db * 32 + j4 * 8) = out4;
+          for (int e = 0; e < 4; ++e) {
+            out4[e] = static_cast<half_t>(static_cast<float>(prev[e]) * scale_prev + o[db][j4 * 4 + e] * scale_mine);
+          }
+          *dst = out4;
+        }
       }
+      if (half == 0) *lse_ptr = fast_log2(w_prev + w_mine) + s_max;
+    } else {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+#pragma unroll
+        for (int j4 = 0; j4 < 4; ++j4) {
+          half4_t out4;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out4[e] = static_cast<half_t>(o[db][j4 * 4 + e] * inv);
+          *reinterpret_cast<half4_t*>(orow + db * 32 + j4 * 8) = out4;
+        }
+      }
+      if (half == 0) *lse_ptr = my_lse;
     }
-    if (half == 0) p.lse[static_cast<int64_t>(q_start + my_pos) * p.h_q + my_head] = m + fast_log2(denom);
   }
 }
 
@@ -641,14 +673,13 @@ int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const 
   KV_API_END();
 }
 
-int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const void* pages,
-                                 const int32_t* page_indptr, const int32_t* page_values,
-                                 const int32_t* length_info, const int32_t* k_rope_pos_offset,
-                                 const int32_t* q_rope_position, void* output, float* lse, int64_t causal,
-                                 int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
-                                 int32_t batch_size, int64_t total_q, int64_t nnz_pages, int64_t num_pages,
-                                 int32_t h_q, int32_t h_kv, int32_t d, int32_t page_size, int32_t sliding_window,
-                                 int32_t sliding_window_size, void* stream) {
+static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pages, const int32_t* page_indptr,
+                         const int32_t* page_values, const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                         const int32_t* q_rope_position, void* output, float* lse, int64_t causal,
+                         int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                         int32_t batch_size, int64_t total_q, int64_t nnz_pages, int64_t num_pages, int32_t h_q,
+                         int32_t h_kv, int32_t d, int32_t page_size, int32_t sliding_window,
+                         int32_t sliding_window_size, bool merge_into, void* stream) {
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_paged_kv: bad shape";
@@ -678,6 +709,7 @@ int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const v
   p.rope_scale = static_cast<float>(rope_scale);
   p.q_rope_position = q_rope_position;
   p.k_rope_pos_offset = k_rope_pos_offset;
+  p.merge_into = merge_into;
   if (sliding_window != 0) {  // length_info is (3, B): last_page_len, window offset, sink size
     p.window_offset = length_info + batch_size;
     p.sink_size = length_info + 2 * static_cast<int64_t>(batch_size);
@@ -694,6 +726,34 @@ int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const v
   }
   KV_LAUNCH_CHECK();
   KV_API_END();
+}
+
+int tvmkv_batch_prefill_paged_kv(const void* q, const int32_t* q_indptr, const void* pages,
+                                 const int32_t* page_indptr, const int32_t* page_values,
+                                 const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                                 const int32_t* q_rope_position, void* output, float* lse, int64_t causal,
+                                 int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                                 int32_t batch_size, int64_t total_q, int64_t nnz_pages, int64_t num_pages,
+                                 int32_t h_q, int32_t h_kv, int32_t d, int32_t page_size, int32_t sliding_window,
+                                 int32_t sliding_window_size, void* stream) {
+  return paged_prefill(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position,
+                       output, lse, causal, rotary_mode, rope_scale, rope_theta, sm_scale, batch_size, total_q,
+                       nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window, sliding_window_size,
+                       /*merge_into=*/false, stream);
+}
+
+int tvmkv_batch_prefill_paged_kv_merge(const void* q, const int32_t* q_indptr, const void* pages,
+                                       const int32_t* page_indptr, const int32_t* page_values,
+                                       const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                                       const int32_t* q_rope_position, void* output, float* lse, int64_t causal,
+                                       int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                                       int32_t batch_size, int64_t total_q, int64_t nnz_pages, int64_t num_pages,
+                                       int32_t h_q, int32_t h_kv, int32_t d, int32_t page_size,
+                                       int32_t sliding_window, int32_t sliding_window_size, void* stream) {
+  return paged_prefill(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position,
+                       output, lse, causal, rotary_mode, rope_scale, rope_theta, sm_scale, batch_size, total_q,
+                       nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window, sliding_window_size,
+                       /*merge_into=*/true, stream);
 }
 
 int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k, const void* v,

@@ -1332,6 +1332,18 @@ class PagedKVCache {
                                            qo_indptr_view_[d].size - 1, page_indices.size, num_total_pages_,
                                            num_qo_heads_, num_kv_heads_, qk_head_dim_, page_size_, sliding_window,
                                            compute_stream_));
+      } else if (!is_first_kernel) {
+        // The prefill kernel merges its state into (o, lse) in its epilogue: one launch for the
+        // kernel and the merge of :2285-2292, and no temporary output.
+        Launch(tvmkv_batch_prefill_paged_kv_merge(q, qo_indptr_view_[d].ptr, pages_[local_layer_id], page_indptr.ptr,
+                                                  page_indices.ptr, length_info.ptr, k_rope_pos.ptr,
+                                                  q_rope_position_map_view_.ptr, o, lse, causal, rotary_mode,
+                                                  rotary_scale, rotary_theta, sm_scale, qo_indptr_view_[d].size - 1,
+                                                  total_seq_length, page_indices.size, num_total_pages_,
+                                                  num_qo_heads_, num_kv_heads_, qk_head_dim_, page_size_,
+                                                  sliding_window, layer_sliding_window_size_, compute_stream_));
+        cross_attn_computed = true;
+        continue;
       } else {
         Launch(tvmkv_batch_prefill_paged_kv(q, qo_indptr_view_[d].ptr, pages_[local_layer_id], page_indptr.ptr,
                                             page_indices.ptr, length_info.ptr, k_rope_pos.ptr,

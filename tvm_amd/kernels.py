@@ -76,11 +76,14 @@ def batch_prefill_ragged_kv(q, q_indptr, k, v, kv_indptr, q_rope_position, k_rop
 
 def batch_prefill_paged_kv(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset,
                            q_rope_position, output, lse, causal, rotary_mode, rope_scale, rope_theta, sm_scale,
-                           sliding_window_size=1024):
+                           sliding_window_size=1024, merge_into=False):
+    """merge_into: output / lse hold an attention state of the same rows; merge into it instead of
+    overwriting (one launch for the paged kernel and merge_state_inplace)."""
     _f16(q, pages, output)
     _i32(q_indptr, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position)
     num_pages, _, hkv, ps, d = pages.shape
-    check(lib().tvmkv_batch_prefill_paged_kv(
+    fn = lib().tvmkv_batch_prefill_paged_kv_merge if merge_into else lib().tvmkv_batch_prefill_paged_kv
+    check(fn(
         _p(q), _p(q_indptr), _p(pages), _p(page_indptr), _p(page_values), _p(length_info), _p(k_rope_pos_offset),
         _p(q_rope_position), _p(output), _p(lse), int(causal), int(rotary_mode), float(rope_scale),
         float(rope_theta), float(sm_scale), q_indptr.shape[0] - 1, q.shape[0], page_values.shape[0], num_pages,
