@@ -256,10 +256,9 @@ def main():
                                           "append_position_map")} for t in wl["tables"]]
     sm_scale = D ** -0.5
 
-    def rope_append(s):
+    def rope_append(s):  # split + RoPE and the append of the new k / v rows, one launch
         t = tabs[s]
-        K.fused_rope(qkv[s], t["q_rope_position"], q, k, v, 1, 1.0, 1e4)
-        K.tir_kv_cache_transpose_append(pages, k, v, t["append_position_map"])
+        K.fused_rope_append(qkv[s], t["q_rope_position"], q, k, v, 1, pages, t["append_position_map"], 1.0, 1e4)
 
     def decode_only(s):
         t = tabs[s]
@@ -301,7 +300,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "configs[1]: batched paged decode, 1 layer, B=64, ctx U[1024,8192] seed 1, "
                                "Hq32/Hkv8/D128 fp16, page 16, permuted 65536-page pool, append 1 token/seq/step "
-                               "(split+RoPE, append, split-KV decode + merge)",
+                               "(split+RoPE+append in one launch, split-KV decode with the chunk merge)",
                    "kv_tokens_per_step": int(kv_tokens.mean()), "bytes_per_step": int(step_bytes)},
         "tokens_per_s": round(B / (ms_step * 1e-3), 1),
         "host_wall_ms_per_step": round(wall_ms, 4),

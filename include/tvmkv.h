@@ -62,6 +62,17 @@ int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void
                      int64_t apply_rope, int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
                      int32_t head_dim, double rope_scale, double rope_theta, void* stream);
 
+/* Slot 24 followed by slot 13 in one launch; no counterpart among the reference's kernels.
+ * Besides the q / k / v outputs of tvmkv_fused_rope, the rotated k and the v rows are written into
+ * their page slots append_position_map[token] (-1 = none), which is what
+ * tvmkv_kv_cache_transpose_append would do from k and v afterwards (paged_kv_cache.cc:1360-1373).
+ * The cache uses it when it appends before attention; k and v stay available to the ragged kernel. */
+int tvmkv_fused_rope_append(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
+                            int64_t apply_rope, void* pages, const int32_t* append_position_map,
+                            int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
+                            int32_t head_dim, int64_t num_pages, int32_t page_size, double rope_scale,
+                            double rope_theta, void* stream);
+
 /* Slot 13 `f_transpose_append_mha` -- replaces `tir_kv_cache_transpose_append`
  * (python/tvm/relax/frontend/nn/llm/_page_kernels.py:40-74), called at paged_kv_cache.cc:1371
  * as (pages, k_data, v_data, position_map).  pages (num_pages, 2, num_kv_heads, page_size,

@@ -41,6 +41,31 @@ def test_fused_rope(d, hq, hkv, apply_rope):
     assert exact > 0.99, f"only {exact:.4f} of the rotated q elements are bit-identical to the oracle"
 
 
+def test_fused_rope_append_equals_rope_then_append():
+    """One launch for split + RoPE + append: bit-identical q, k, v and pages to the two kernels."""
+    rng = np.random.default_rng(42)
+    hq, hkv, d, ps, npages, n = 32, 8, 128, 16, 12, 70
+    qkv = dev(rng.standard_normal((n, hq + 2 * hkv, d)).astype(F16))
+    pos = i32(rng.integers(0, 5000, size=n))
+    slots = rng.permutation(npages * ps)[:n].astype(np.int32)
+    slots[[3, 17]] = -1
+    pages0 = rng.standard_normal((npages, 2, hkv, ps, d)).astype(F16)
+    outs = []
+    for fused in (False, True):
+        q = torch.zeros((n, hq, d), dtype=torch.float16, device=DEV)
+        k = torch.zeros((n, hkv, d), dtype=torch.float16, device=DEV)
+        v = torch.zeros((n, hkv, d), dtype=torch.float16, device=DEV)
+        pages = dev(pages0)
+        if fused:
+            K.fused_rope_append(qkv, pos, q, k, v, 1, pages, i32(slots), 1.0, 1e4)
+        else:
+            K.fused_rope(qkv, pos, q, k, v, 1, 1.0, 1e4)
+            K.tir_kv_cache_transpose_append(pages, k, v, i32(slots))
+        outs.append([host(t) for t in (q, k, v, pages)])
+    for a, b, name in zip(outs[0], outs[1], ("q", "k", "v", "pages")):
+        assert np.array_equal(a, b), name
+
+
 def test_transpose_append_bit_exact_with_skips():
     rng = np.random.default_rng(1)
     hkv, ps, d, npages, n = 8, 16, 128, 64, 300

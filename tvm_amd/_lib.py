@@ -23,6 +23,8 @@ class KVError(RuntimeError):
 # name -> argument ctypes, in the order of include/tvmkv.h
 SIGNATURES = {
     "tvmkv_fused_rope": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_i32, c_f64, c_f64, c_vp],
+    "tvmkv_fused_rope_append": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i64,
+                                c_i32, c_f64, c_f64, c_vp],
     "tvmkv_kv_cache_transpose_append": [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_kv_cache_transpose_append_mla": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_vp],
     "tvmkv_batch_prefill_ragged_kv": [c_vp] * 9 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i32, c_i32,

@@ -27,13 +27,17 @@ struct RopeDivisors {
 // One workgroup per token: the D/2 (cos, sin) pairs of the token's position are computed once
 // (they are the same for every head; the precise sinf/cosf with their range reduction are by far
 // the most expensive part) and shared through LDS, then all heads of the token are streamed.
-template <int D>
+// APPEND: the rotated k and the v rows also go into their page slots (what transpose_append
+// does from the k / v outputs), slot append_position_map[token], -1 = none.
+template <int D, bool APPEND>
 __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restrict__ qkv,
                                                          const int32_t* __restrict__ position_map,
                                                          half_t* __restrict__ q, half_t* __restrict__ k,
                                                          half_t* __restrict__ v, int64_t seq_len, int num_q_heads,
                                                          int num_kv_heads, int apply_rope, float scale,
-                                                         RopeDivisors div) {
+                                                         RopeDivisors div, half_t* __restrict__ pages,
+                                                         const int32_t* __restrict__ append_position_map,
+                                                         int page_size) {
   constexpr int kThreadsPerHead = D / 16;  // a thread owns d-range [8c, 8c+8) and its partner +D/2
   __shared__ float cs_lds[D / 2];
   __shared__ float sn_lds[D / 2];
@@ -78,6 +82,17 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
     }
     st16(dst + c * 8, lo);
     st16(dst + D / 2 + c * 8, hi);
+    if (APPEND && h >= num_q_heads) {
+      const int32_t slot = append_position_map[s];
+      if (slot != -1) {
+        const int kv = h >= num_q_heads + num_kv_heads;
+        const int head = h - num_q_heads - kv * num_kv_heads;
+        half_t* row = pages + ((static_cast<int64_t>(slot / page_size) * 2 + kv) * num_kv_heads + head) *
+                                  (static_cast<int64_t>(page_size) * D) + (slot % page_size) * D;
+        st16(row + c * 8, lo);
+        st16(row + D / 2 + c * 8, hi);
+      }
+    }
   }
 }
 
@@ -283,15 +298,21 @@ using namespace tvmkv;
 
 extern "C" {
 
-int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void* k, void* v, int64_t apply_rope,
-                     int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
-                     double rope_scale, double rope_theta, void* stream) {
+static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
+                           int64_t apply_rope, int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
+                           int32_t head_dim, double rope_scale, double rope_theta, void* pages,
+                           const int32_t* append_position_map, int64_t num_pages, int32_t page_size, void* stream) {
   KV_API_BEGIN();
   KV_CHECK(seq_len >= 0 && num_q_heads > 0 && num_kv_heads > 0) << "fused_rope: bad shape";
   KV_UNSUPPORTED(head_dim != 64 && head_dim != 128 && head_dim != 256)
       << "fused_rope: head_dim " << head_dim << " is not built (64, 128, 256)";
   if (seq_len == 0) return TVMKV_OK;
   KV_CHECK(qkv && position_map && q && k && v) << "fused_rope: NULL tensor";
+  const bool append = pages != nullptr;
+  if (append) {
+    KV_CHECK(append_position_map != nullptr && page_size > 0) << "fused_rope_append: NULL position map or bad page size";
+    KV_CHECK(num_pages * page_size <= INT32_MAX) << "fused_rope_append: slot ids do not fit int32";
+  }
   RopeDivisors div;
   const float theta = static_cast<float>(rope_theta);
   for (int i = 0; i < head_dim / 2; ++i) {
@@ -302,17 +323,37 @@ int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(seq_len)), dim3(256), 0, as_stream(stream), static_cast<const half_t*>(qkv),
                        position_map, static_cast<half_t*>(q), static_cast<half_t*>(k), static_cast<half_t*>(v),
-                       seq_len, num_q_heads, num_kv_heads, static_cast<int>(apply_rope > 0), scale, div);
+                       seq_len, num_q_heads, num_kv_heads, static_cast<int>(apply_rope > 0), scale, div,
+                       static_cast<half_t*>(pages), append_position_map, page_size);
   };
   if (head_dim == 64) {
-    launch(fused_rope_kernel<64>);
+    if (append) launch(fused_rope_kernel<64, true>); else launch(fused_rope_kernel<64, false>);
   } else if (head_dim == 128) {
-    launch(fused_rope_kernel<128>);
+    if (append) launch(fused_rope_kernel<128, true>); else launch(fused_rope_kernel<128, false>);
   } else {
-    launch(fused_rope_kernel<256>);
+    if (append) launch(fused_rope_kernel<256, true>); else launch(fused_rope_kernel<256, false>);
   }
   KV_LAUNCH_CHECK();
   KV_API_END();
+}
+
+int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void* k, void* v, int64_t apply_rope,
+                     int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                     double rope_scale, double rope_theta, void* stream) {
+  return fused_rope_impl(qkv, position_map, q, k, v, apply_rope, seq_len, num_q_heads, num_kv_heads, head_dim,
+                         rope_scale, rope_theta, nullptr, nullptr, 0, 0, stream);
+}
+
+int tvmkv_fused_rope_append(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
+                            int64_t apply_rope, void* pages, const int32_t* append_position_map, int64_t seq_len,
+                            int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int64_t num_pages,
+                            int32_t page_size, double rope_scale, double rope_theta, void* stream) {
+  if (seq_len > 0 && pages == nullptr) {
+    ::tvmkv::SetLastError("fused_rope_append: NULL pages");
+    return TVMKV_EINVAL;
+  }
+  return fused_rope_impl(qkv, position_map, q, k, v, apply_rope, seq_len, num_q_heads, num_kv_heads, head_dim,
+                         rope_scale, rope_theta, pages, append_position_map, num_pages, page_size, stream);
 }
 
 static void check_slot_layout(const char* what, int32_t page_size, int32_t head_dim) {

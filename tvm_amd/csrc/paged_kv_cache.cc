@@ -639,11 +639,19 @@ class PagedKVCache {
     KV_CHECK(!dirty_aux_data_device_) << "auxiliary data is not synchronised";
 
     // Part 2: split fused qkv, RoPE on q/k.
-    Launch(tvmkv_fused_rope(qkv, q_rope_position_map_view_.ptr, temp_q_, temp_k_, temp_v_,
-                            rope_mode_ == TVMKV_ROPE_NORMAL, total_seq_length, num_qo_heads_,
-                            num_kv_heads_, qk_head_dim_, rotary_scale_, rotary_theta_, compute_stream_));
-    // Part 3: append before attention when the decode kernel covers the new token itself.
-    if (append_before_attn_) AppendMHA(local_layer_id, total_seq_length);
+    // Part 3 with it when the new tokens are appended before attention (the decode kernel covers
+    // the new token itself): one launch writes q, k, v and the page slots.
+    if (append_before_attn_) {
+      Launch(tvmkv_fused_rope_append(qkv, q_rope_position_map_view_.ptr, temp_q_, temp_k_, temp_v_,
+                                     rope_mode_ == TVMKV_ROPE_NORMAL, pages_[local_layer_id],
+                                     append_position_map_view_.ptr, total_seq_length, num_qo_heads_, num_kv_heads_,
+                                     qk_head_dim_, num_total_pages_, page_size_, rotary_scale_, rotary_theta_,
+                                     compute_stream_));
+    } else {
+      Launch(tvmkv_fused_rope(qkv, q_rope_position_map_view_.ptr, temp_q_, temp_k_, temp_v_,
+                              rope_mode_ == TVMKV_ROPE_NORMAL, total_seq_length, num_qo_heads_,
+                              num_kv_heads_, qk_head_dim_, rotary_scale_, rotary_theta_, compute_stream_));
+    }
     // Part 5: attention.
     AttentionInternal(layer_id, temp_q_, temp_k_, temp_v_, out, total_seq_length, sm_scale);
     // Part 6.

@@ -48,6 +48,18 @@ def fused_rope(qkv, position_map, q, k, v, apply_rope, rope_scale=1.0, rope_thet
                                  k.shape[1], d, float(rope_scale), float(rope_theta), _stream()))
 
 
+def fused_rope_append(qkv, position_map, q, k, v, apply_rope, pages, append_position_map, rope_scale=1.0,
+                      rope_theta=1e4):
+    """fused_rope and tir_kv_cache_transpose_append in one launch."""
+    _f16(qkv, q, k, v, pages)
+    _i32(position_map, append_position_map)
+    n, _, d = qkv.shape
+    num_pages, _, hkv, ps, _ = pages.shape
+    check(lib().tvmkv_fused_rope_append(_p(qkv), _p(position_map), _p(q), _p(k), _p(v), int(apply_rope), _p(pages),
+                                        _p(append_position_map), n, q.shape[1], k.shape[1], d, num_pages, ps,
+                                        float(rope_scale), float(rope_theta), _stream()))
+
+
 def tir_kv_cache_transpose_append(pages, k_data, v_data, position_map):
     _f16(pages, k_data, v_data)
     _i32(position_map)
