@@ -153,9 +153,29 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   const int group = p.group;
 
   // ---- which (sequence, row tile) ---------------------------------------------------------
+  // Workgroups are dispatched in the order of their index, and the last ones to start decide when
+  // the kernel ends: the sequences are walked from the one with the most keys to the one with the
+  // fewest (up to 64 sequences: one lane per sequence ranks them), and inside a sequence from the
+  // last row tile to the first, since under the causal mask the last rows see the most keys.
   const int slot = blockIdx.y;
-  int b;
-  {
+  int b, local_slot;
+  if (p.batch_size <= 64) {
+    int my_tiles = 0, my_key = -1;
+    if (lane < p.batch_size) {
+      my_tiles = ((p.q_indptr[lane + 1] - p.q_indptr[lane]) * group + BM - 1) / BM;
+      my_key = PAGED ? p.page_indptr[lane + 1] - p.page_indptr[lane] : p.kv_indptr[lane + 1] - p.kv_indptr[lane];
+    }
+    int my_begin = 0;  // row tiles of the sequences ranked before this lane's
+    for (int j = 0; j < p.batch_size; ++j) {
+      const int key_j = __builtin_amdgcn_readlane(my_key, j);
+      const int tiles_j = __builtin_amdgcn_readlane(my_tiles, j);
+      if (key_j > my_key || (key_j == my_key && j < lane)) my_begin += tiles_j;
+    }
+    const uint64_t owner = __ballot(lane < p.batch_size && slot >= my_begin && slot < my_begin + my_tiles);
+    if (owner == 0) return;  // the grid is sized from shapes alone and has spare slots
+    b = __builtin_amdgcn_readfirstlane(__ffsll(static_cast<long long>(owner)) - 1);
+    local_slot = slot - __builtin_amdgcn_readlane(my_begin, b);
+  } else {
     int lo = 0, hi = p.batch_size - 1;
     while (lo < hi) {
       int mid = (lo + hi + 1) >> 1;
@@ -166,13 +186,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
       }
     }
     b = lo;
+    local_slot = slot - tile_slot_begin(p.q_indptr, b, group);
   }
   const int q_start = p.q_indptr[b];
   const int qo_len = p.q_indptr[b + 1] - q_start;
   const int rows = qo_len * group;
-  // tiles of a sequence are handed out last-first: under the causal mask the last rows see the
-  // most keys, and the longest workgroups should start first
-  const int local_slot = slot - tile_slot_begin(p.q_indptr, b, group);
   const int n_row_tiles = (rows + BM - 1) / BM;
   if (local_slot >= n_row_tiles) return;
   const int r0 = (n_row_tiles - 1 - local_slot) * BM;
