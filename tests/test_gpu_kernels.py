@@ -350,6 +350,22 @@ def test_paged_prefill_against_oracle(hq, hkv, d, causal):
     assert_close(gl, el, atol=2e-3, rtol=1e-4, what="paged lse")
 
 
+def test_prefill_more_than_64_sequences():
+    """Up to 64 sequences the kernels rank the sequences by length themselves; beyond that they
+    take them in batch order.  Both orders on one ragged and one paged call."""
+    rng = np.random.default_rng(43)
+    hq, hkv, d = 8, 2, 128
+    for nseq in (64, 70):
+        kv_lens = [int(x) for x in rng.integers(0, 90, size=nseq)]
+        q_lens = [int(x) for x in rng.integers(1, 40, size=nseq)]
+        go, gl, eo, el = _paged_both(rng, kv_lens, q_lens, hq, hkv, d, 0, 512)
+        assert_close(go, eo, what=f"paged out, {nseq} sequences")
+        assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"paged lse, {nseq} sequences")
+        go, gl, eo, el = _ragged_both(rng, q_lens, hq, hkv, d, d, 1)
+        assert_close(go, eo, what=f"ragged out, {nseq} sequences")
+        assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"ragged lse, {nseq} sequences")
+
+
 def test_layer_sliding_window_mask_known_answer_on_the_gpu():
     """The reference's known-answer vector for the paged prefill kernel with sliding_window_size = 3
     (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_tir.py:98-156)."""
