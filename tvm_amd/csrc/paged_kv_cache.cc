@@ -639,23 +639,17 @@ class PagedKVCache {
     KV_CHECK(!dirty_aux_data_device_) << "auxiliary data is not synchronised";
 
     // Part 2: split fused qkv, RoPE on q/k.
-    // Part 3 with it when the new tokens are appended before attention (the decode kernel covers
-    // the new token itself): one launch writes q, k, v and the page slots.
-    if (append_before_attn_) {
-      Launch(tvmkv_fused_rope_append(qkv, q_rope_position_map_view_.ptr, temp_q_, temp_k_, temp_v_,
-                                     rope_mode_ == TVMKV_ROPE_NORMAL, pages_[local_layer_id],
-                                     append_position_map_view_.ptr, total_seq_length, num_qo_heads_, num_kv_heads_,
-                                     qk_head_dim_, num_total_pages_, page_size_, rotary_scale_, rotary_theta_,
-                                     compute_stream_));
-    } else {
-      Launch(tvmkv_fused_rope(qkv, q_rope_position_map_view_.ptr, temp_q_, temp_k_, temp_v_,
-                              rope_mode_ == TVMKV_ROPE_NORMAL, total_seq_length, num_qo_heads_,
-                              num_kv_heads_, qk_head_dim_, rotary_scale_, rotary_theta_, compute_stream_));
-    }
+    // Part 3 (or 6) with it, in one launch: the new k / v rows go into their page slots while q, k, v
+    // are written.  When the reference appends after attention (chunked prefill) the earlier append
+    // changes nothing: the page tables of this step cover the tokens cached before it, the kernels
+    // never read a slot beyond them, and the slots of the new tokens are not shared with anyone.
+    Launch(tvmkv_fused_rope_append(qkv, q_rope_position_map_view_.ptr, temp_q_, temp_k_, temp_v_,
+                                   rope_mode_ == TVMKV_ROPE_NORMAL, pages_[local_layer_id],
+                                   append_position_map_view_.ptr, total_seq_length, num_qo_heads_, num_kv_heads_,
+                                   qk_head_dim_, num_total_pages_, page_size_, rotary_scale_, rotary_theta_,
+                                   compute_stream_));
     // Part 5: attention.
     AttentionInternal(layer_id, temp_q_, temp_k_, temp_v_, out, total_seq_length, sm_scale);
-    // Part 6.
-    if (!append_before_attn_) AppendMHA(local_layer_id, total_seq_length);
     RecordComputeEvent();
   }
 
@@ -1257,12 +1251,6 @@ class PagedKVCache {
     }
     // The next BeginForward's first kernel waits for the copy stream (paged_kv_cache.cc:767-769).
     copy_stream_has_work_ = true;
-  }
-
-  void AppendMHA(int64_t local_layer_id, int64_t total_seq_length) {
-    Launch(tvmkv_kv_cache_transpose_append(pages_[local_layer_id], temp_k_, temp_v_, append_position_map_view_.ptr,
-                                           total_seq_length, num_total_pages_, num_kv_heads_, page_size_,
-                                           qk_head_dim_, compute_stream_));
   }
 
   // :2161-2180
