@@ -144,6 +144,21 @@ int tvmkv_batch_prefill_paged_kv_merge(const void* q, const int32_t* q_indptr, c
                                        int32_t sliding_window, int32_t sliding_window_size,
                                        void* stream);
 
+/* Slots 15, 16 and 23 in one launch; no counterpart among the reference's kernels.  A chunked-
+ * prefill step of a plain (no sliding window, no inline RoPE, no token tree) cache in one pass: every
+ * query attends to the tokens its sequence has in the page pool (all visible) and to the new
+ * tokens k, v of the call under the causal mask, which is what the reference computes as ragged
+ * self-attention + paged cross-attention + merge_state_inplace (paged_kv_cache.cc:2161-2180,
+ * :2285-2292), without the temporary output, the second read of q and the merge pass.
+ * k, v (total_q, h_kv, d): the rows of the queries' own tokens, indexed by q_indptr. */
+int tvmkv_batch_prefill_cached_and_new_kv(const void* q, const int32_t* q_indptr, const void* k,
+                                          const void* v, const void* pages,
+                                          const int32_t* page_indptr, const int32_t* page_values,
+                                          const int32_t* last_page_len, void* output, float* lse,
+                                          double sm_scale, int32_t batch_size, int64_t total_q,
+                                          int64_t nnz_pages, int64_t num_pages, int32_t h_q,
+                                          int32_t h_kv, int32_t d, int32_t page_size, void* stream);
+
 /* Slots 17/19 paged decode -- replaces `batch_decode_paged_kv`
  * (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:181-411; llvm form :49-178), calling
  * convention attn_backend.h:511-514:

@@ -535,3 +535,37 @@ def test_chunked_prefill_composition_matches_oracle():
     assert_close(host(go2), eo, what="chunked prefill out, merged in the epilogue")
     assert_close(host(gl2), el, atol=2e-3, rtol=1e-4, what="chunked prefill lse, merged in the epilogue")
     assert_close(host(go2), host(go), atol=2e-3, rtol=2e-3, what="epilogue merge vs separate merge")
+    # and as one pass over the cached and the new tokens
+    go3 = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl3 = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_cached_and_new_kv(qd, i32(ind), dev(k), dev(v), dev(pages), i32(pindptr), i32(pvalues), i32(last),
+                                      go3, gl3, d ** -0.5)
+    assert_close(host(go3), eo, what="chunked prefill out, one pass")
+    assert_close(host(gl3), el, atol=2e-3, rtol=1e-4, what="chunked prefill lse, one pass")
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 8, 128)])
+def test_prefill_cached_and_new_in_one_pass(hq, hkv, d):
+    """Prefix lengths around the tile size (the padded end of the cached part), no prefix, chunks of one
+    token and of several row tiles; against ragged + paged + merge of the oracle."""
+    rng = np.random.default_rng(44)
+    prefix = [0, 1, 63, 64, 65, 128, 200, 700, 16, 330]
+    chunk = [5, 130, 1, 64, 33, 300, 2, 40, 129, 64]
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, prefix, 128, hkv, 16, d)
+    n = sum(chunk)
+    ind = np.concatenate([[0], np.cumsum(chunk)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    zq, zb = np.zeros(n, np.int32), np.zeros(len(prefix), np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    to, tl = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    ok.prefill_ragged(q, ind, k, v, ind, zq, zb, eo, el, 1, 0, 1.0, 1e4, d ** -0.5)
+    ok.prefill_paged(q, ind, pages, pindptr, pvalues, last, zb, zq, to, tl, 0, 0, 1.0, 1e4, d ** -0.5)
+    ok.merge_state_inplace(eo, el, to, tl)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_cached_and_new_kv(dev(q), i32(ind), dev(k), dev(v), dev(pages), i32(pindptr), i32(pvalues),
+                                      i32(last), go, gl, d ** -0.5)
+    assert_close(host(go), eo, what="one-pass chunked prefill out")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="one-pass chunked prefill lse")

@@ -33,6 +33,8 @@ SIGNATURES = {
                                                    c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_prefill_paged_kv_merge": [c_vp] * 10 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64,
                                                          c_i64, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_batch_prefill_cached_and_new_kv": [c_vp] * 10 + [c_f64, c_i32, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32,
+                                                            c_i32, c_vp],
     "tvmkv_batch_decode_paged_kv": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32, c_i32,
                                                  c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_tree_attn": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i32, c_i32, c_i32, c_vp],

@@ -122,8 +122,15 @@ constexpr size_t prefill_lds_bytes(int dqk, int dv) {
 // Attention does not depend on the order of the keys, so the tiles are still walked in physical
 // order.  Masks are evaluated per element; only a plain cache without RoPE keeps the unmasked
 // path, for the tiles in front of the tree.
-template <int DQK, int DV, bool PAGED, int PS, bool EXT>
+// SRC: where the keys come from.  kRagged: k / v rows of the call; kPaged: the page pool; kBoth: the
+// cached tokens of the page pool, all visible, followed by the k / v rows of the call under the
+// causal mask -- a chunked-prefill step in one pass, on one key axis whose paged part is padded to
+// a whole number of tiles (the padding is masked like the end of a sequence).
+constexpr int kRagged = 0, kPaged = 1, kBoth = 2;
+template <int DQK, int DV, int SRC, int PS, bool EXT>
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
+  constexpr bool PAGED = SRC == kPaged, BOTH = SRC == kBoth;
+  static_assert(!(BOTH && EXT), "the combined pass exists for the plain cache only");
   static_assert(DQK % 64 == 0 && DV % 64 == 0, "feature dims must be multiples of 64");
   constexpr int KS = DQK / 16;                  // k-steps of the QK^T product
   constexpr int DB = DV / 32;                   // 32-wide output feature blocks
@@ -137,7 +144,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   constexpr int STAGE = BN * (DQK + DV);        // halfs per pipeline stage
   constexpr int NSTAGE = prefill_stages(DQK, DV);
   constexpr int COPIES = (DQK + DV) / 8 / NW;   // copy instructions per wave per tile
-  static_assert(!PAGED || PS % 16 == 0, "page size must be a multiple of 16");
+  static_assert(SRC == kRagged || PS % 16 == 0, "page size must be a multiple of 16");
 
   // two stages; the workgroup's 4 waves each copy 16 of the 64 token rows of a tile
   extern __shared__ __attribute__((aligned(16))) half_t lds_tiles[];
@@ -163,7 +170,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     int my_tiles = 0, my_key = -1;
     if (lane < p.batch_size) {
       my_tiles = ((p.q_indptr[lane + 1] - p.q_indptr[lane]) * group + BM - 1) / BM;
-      my_key = PAGED ? p.page_indptr[lane + 1] - p.page_indptr[lane] : p.kv_indptr[lane + 1] - p.kv_indptr[lane];
+      my_key = 0;
+      if (PAGED || BOTH) my_key += (p.page_indptr[lane + 1] - p.page_indptr[lane]) * PS;
+      if (!PAGED) my_key += p.kv_indptr[lane + 1] - p.kv_indptr[lane];
     }
     int my_begin = 0;  // row tiles of the sequences ranked before this lane's
     for (int j = 0; j < p.batch_size; ++j) {
@@ -196,8 +205,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   const int r0 = (n_row_tiles - 1 - local_slot) * BM;
 
   // phys_len: tokens the K/V storage of the sequence covers; kv_len: keys attended to (logical)
-  int phys_len, kv_start = 0, pbeg = 0, sink = 0, win_lo = 0;
-  if (PAGED) {
+  // kBoth: the key axis is [cached tokens, padded to prefix_pad][new tokens]
+  int phys_len = 0, kv_start = 0, pbeg = 0, sink = 0, win_lo = 0, prefix_len = 0, prefix_pad = 0;
+  if (PAGED || BOTH) {
     pbeg = p.page_indptr[b];
     const int npages = p.page_indptr[b + 1] - pbeg;
     phys_len = npages > 0 ? (npages - 1) * PS + p.last_page_len[b] : 0;
@@ -205,10 +215,17 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
       sink = p.sink_size[b];
       win_lo = p.window_offset[b];
     }
-  } else {
-    kv_start = p.kv_indptr[b];
-    phys_len = p.kv_indptr[b + 1] - kv_start;
   }
+  if (!PAGED) {
+    kv_start = p.kv_indptr[b];
+    if (BOTH) {
+      prefix_len = phys_len;
+      prefix_pad = (prefix_len + BN - 1) / BN * BN;
+    }
+    phys_len = prefix_pad + p.kv_indptr[b + 1] - kv_start;
+  }
+  const int prefix_tiles = prefix_pad / BN;
+  const int hole_tile = (BOTH && prefix_len < prefix_pad) ? prefix_tiles - 1 : -1;  // its end is padding
   const int kv_len = phys_len - win_lo + sink;
   // number of logical keys -> physical end of the tokens that hold them
   auto to_phys = [&](int n) { return (!EXT || n <= sink) ? n : n - sink + win_lo; };
@@ -280,12 +297,13 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   // times a finite V is 0 (unwritten page memory could hold NaN patterns).
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds_tiles));
-  const int last_tok = phys_len - 1;
+  const int last_tok = BOTH ? prefix_len - 1 : phys_len - 1;               // last row of the (paged) source
+  const int last_new = BOTH ? phys_len - prefix_pad - 1 : 0;              // kBoth: last row of k / v
   // Page ids of this wave's RPW rows for 64 consecutive tiles, one tile per lane, fetched once per
   // 64 tiles: the wait for this load also waits for every tile copy in flight, so it must be rare.
   int page_ids = 0;
   auto load_page_ids = [&](int first_tile) {
-    if (PAGED) {
+    if (PAGED || BOTH) {
       const int pslot = min((first_tile + lane) * BN + wave_u * RPW, last_tok) / PS;
       page_ids = p.page_values[pbeg + pslot];
     }
@@ -305,11 +323,13 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   auto issue_copies = [&](int tile, auto first_c, auto count_c) {
     constexpr int FIRST = decltype(first_c)::value;
     constexpr int COUNT = decltype(count_c)::value;
-    const int kv0 = tile * BN;
+    const bool from_pages = BOTH ? tile < prefix_tiles : PAGED;  // wave-uniform
+    const int kv0 = tile * BN - (from_pages ? 0 : prefix_pad);
+    const int last_row = (BOTH && !from_pages) ? last_new : last_tok;
     const uint32_t stage = lds_base + (tile % NSTAGE) * (STAGE * 2);  // LDS byte address
     const half_t* kbase = k_seq;
     const half_t* vbase = v_seq;
-    if (PAGED) {
+    if (from_pages) {
       const int page = __builtin_amdgcn_readlane(page_ids, tile & 63);
       kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * (PS * DQK);
       vbase = kbase + static_cast<int64_t>(p.h_kv) * (PS * DQK);
@@ -323,8 +343,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
         if (idx < FIRST || idx >= FIRST + COUNT) continue;
         const int row = wave_u * RPW + i * RPI + lane / KCH;
         const int piece = (lane % KCH) ^ k_swizzle<KW>(row);
-        const uint32_t t = min(kv0 + row, last_tok);
-        const uint32_t off = (PAGED ? (t % PS) * (DQK * 2) : __umul24(t, k_stride_bytes)) + (blk * KW + piece * 8) * 2;
+        const uint32_t t = min(kv0 + row, last_row);
+        const uint32_t off = (from_pages ? (t % PS) * (DQK * 2) : __umul24(t, k_stride_bytes)) + (blk * KW + piece * 8) * 2;
         copy16_to_lds(kbase, off, stage + (blk * (BN * KW) + (wave_u * RPW + i * RPI) * KW) * 2);
       }
     }
@@ -337,14 +357,14 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
         if (idx < FIRST || idx >= FIRST + COUNT) continue;
         const int row = wave_u * RPW + i * RPI + lane / VCH;
         const int piece = (lane % VCH) ^ v_swizzle<VW>(row);
-        const uint32_t t = min(kv0 + row, last_tok);
-        const uint32_t off = (PAGED ? (t % PS) * (DV * 2) : __umul24(t, v_stride_bytes)) + (blk * VW + piece * 8) * 2;
+        const uint32_t t = min(kv0 + row, last_row);
+        const uint32_t off = (from_pages ? (t % PS) * (DV * 2) : __umul24(t, v_stride_bytes)) + (blk * VW + piece * 8) * 2;
         copy16_to_lds(vbase, off, stage + (BN * DQK + blk * (BN * VW) + (wave_u * RPW + i * RPI) * VW) * 2);
       }
     }
   };
   auto issue_tile = [&](int tile) {
-    if (PAGED && (tile & 63) == 0) load_page_ids(tile);
+    if ((PAGED || (BOTH && tile < prefix_tiles)) && (tile & 63) == 0) load_page_ids(tile);
     issue_copies(tile, std::integral_constant<int, 0>{}, std::integral_constant<int, COPIES>{});
   };
 
@@ -466,10 +486,16 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     // no prefetch across a 64-tile window of page ids: the ids held are those of the last copy issued
     const int next = tile + NSTAGE - 1;  // the tile whose copy this iteration issues
     const bool has_next = next < n_tiles;
-    const bool unmasked = TB == 2 && kv0 < wave_limit_max && kv0 + BN <= unmasked_limit;  // wave-uniform
+    // bounds of this tile: those of the wave and the lane, except in the tile that ends in the
+    // padding between the cached and the new tokens, which ends at the last cached token for all
+    const bool hole = BOTH && tile == hole_tile;
+    const int t_limit_max = hole ? (wave_active ? prefix_len : 0) : wave_limit_max;
+    const int t_limit_min = hole ? t_limit_max : wave_limit_min;
+    const int t_my_limit = hole ? (row_valid ? prefix_len : 0) : my_limit;
+    const bool unmasked = TB == 2 && kv0 < t_limit_max && kv0 + BN <= (hole ? t_limit_max : unmasked_limit);  // wave-uniform
     if (has_next) issue_tile(next);
 
-    if (kv0 >= wave_limit_max) continue;  // wave-uniform: every row of this wave is masked out
+    if (kv0 >= t_limit_max) continue;  // wave-uniform: every row of this wave is masked out
 
     if (unmasked) {
       // Every row of the wave sees the whole tile (all tiles left of the causal diagonal): no
@@ -508,7 +534,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) {
       const int t0 = kv0 + tb * 32;
-      if (t0 >= wave_limit_max) break;  // wave-uniform
+      if (t0 >= t_limit_max) break;  // wave-uniform
       half8_t kf[KS];
       half8_t vf[DB][2];
       half8_t pf[2];
@@ -543,9 +569,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
           }
           acc[j] = visible ? acc[j] : -3.0e38f;
         }
-      } else if (t0 + 32 > wave_limit_min) {  // wave-uniform
+      } else if (t0 + 32 > t_limit_min) {  // wave-uniform
         asm volatile("" ::: "memory");  // keep this a branch: if-converted it costs 5 ops per element everywhere
-        const int rel = my_limit - t0 - half * 4;  // element j is token t0 + half*4 + (j/4)*8 + j%4
+        const int rel = t_my_limit - t0 - half * 4;  // element j is token t0 + half*4 + (j/4)*8 + j%4
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[j] = ((j >> 2) * 8 + (j & 3)) < rel ? acc[j] : -3.0e38f;
       }
@@ -604,7 +630,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   }
 }
 
-template <int DQK, int DV, bool PAGED, int PS, bool EXT>
+template <int DQK, int DV, int SRC, int PS, bool EXT>
 static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const PrefillRopeDivisors& div,
                                hipStream_t stream) {
   const int64_t slots = total_q * p.group / BM + p.batch_size;
@@ -612,27 +638,27 @@ static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const Pr
   constexpr size_t lds_bytes = prefill_lds_bytes(DQK, DV);
   static bool attr_set = false;  // per instantiation; the attribute is per function, not per device
   if (lds_bytes > 48 * 1024 && !attr_set) {
-    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, PAGED, PS, EXT>),
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, SRC, PS, EXT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     attr_set = true;
   }
-  hipLaunchKernelGGL((prefill_kernel<DQK, DV, PAGED, PS, EXT>), dim3(p.h_kv, static_cast<unsigned>(slots)),
+  hipLaunchKernelGGL((prefill_kernel<DQK, DV, SRC, PS, EXT>), dim3(p.h_kv, static_cast<unsigned>(slots)),
                      dim3(NW * 64), lds_bytes, stream, p, div);
 }
 
 // The extended kernels (sliding-window cache, per-layer window, inline RoPE) exist for the head
 // dims that RoPE models use here; d_qk 192 / d_v 128 is the MLA self-attention, which has neither.
-template <int DQK, int DV, bool PAGED, int PS>
+template <int DQK, int DV, int SRC, int PS>
 static void launch_prefill(const PrefillParams& p, int64_t total_q, bool ext, double rope_theta, hipStream_t stream) {
   PrefillRopeDivisors div{};
   if (!ext) {
-    launch_prefill_ext<DQK, DV, PAGED, PS, false>(p, total_q, div, stream);
+    launch_prefill_ext<DQK, DV, SRC, PS, false>(p, total_q, div, stream);
     return;
   }
-  if constexpr (DQK == DV && DQK <= 128) {
+  if constexpr (DQK == DV && DQK <= 128 && SRC != kBoth) {
     const float theta = static_cast<float>(rope_theta);
     for (int i = 0; i < DQK / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DQK));
-    launch_prefill_ext<DQK, DV, PAGED, PS, true>(p, total_q, div, stream);
+    launch_prefill_ext<DQK, DV, SRC, PS, true>(p, total_q, div, stream);
   } else {
     throw Error(TVMKV_EUNSUPPORTED, "prefill: inline RoPE / sliding window are not built for this head shape");
   }
@@ -678,11 +704,11 @@ int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const 
   const bool ext = p.rotary != 0;
   hipStream_t s = as_stream(stream);
   if (d_qk == 128 && d_v == 128) {
-    launch_prefill<128, 128, false, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<128, 128, kRagged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d_qk == 64 && d_v == 64) {
-    launch_prefill<64, 64, false, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<64, 64, kRagged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d_qk == 192 && d_v == 128) {
-    launch_prefill<192, 128, false, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<192, 128, kRagged, 16>(p, total_q, ext, rope_theta, s);
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_ragged_kv: (d_qk, d_v) = (" << d_qk << ", " << d_v
                          << ") is not built ((64,64), (128,128), (192,128))";
@@ -736,9 +762,9 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
   const bool ext = p.rotary != 0 || sliding_window != 0;
   hipStream_t s = as_stream(stream);
   if (d == 128) {
-    launch_prefill<128, 128, true, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<128, 128, kPaged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d == 64) {
-    launch_prefill<64, 64, true, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<64, 64, kPaged, 16>(p, total_q, ext, rope_theta, s);
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_paged_kv: head_dim " << d << " is not built (64, 128)";
   }
@@ -774,6 +800,51 @@ int tvmkv_batch_prefill_paged_kv_merge(const void* q, const int32_t* q_indptr, c
                        /*merge_into=*/true, stream);
 }
 
+int tvmkv_batch_prefill_cached_and_new_kv(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                                          const void* pages, const int32_t* page_indptr,
+                                          const int32_t* page_values, const int32_t* last_page_len, void* output,
+                                          float* lse, double sm_scale, int32_t batch_size, int64_t total_q,
+                                          int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                                          int32_t d, int32_t page_size, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
+      << "batch_prefill_cached_and_new_kv: bad shape";
+  KV_UNSUPPORTED(page_size != 16) << "batch_prefill_cached_and_new_kv: page_size " << page_size
+                                  << " is not built (16)";
+  if (batch_size == 0 || total_q == 0) return TVMKV_OK;
+  KV_CHECK(q && q_indptr && k && v && pages && page_indptr && last_page_len && output && lse)
+      << "batch_prefill_cached_and_new_kv: NULL tensor";
+  KV_CHECK(nnz_pages == 0 || page_values) << "batch_prefill_cached_and_new_kv: NULL page table";
+  PrefillParams p{};
+  p.q = static_cast<const half_t*>(q);
+  p.q_indptr = q_indptr;
+  p.k = static_cast<const half_t*>(k);
+  p.v = static_cast<const half_t*>(v);
+  p.kv_indptr = q_indptr;  // the new tokens are the queries' own
+  p.pages = static_cast<const half_t*>(pages);
+  p.page_indptr = page_indptr;
+  p.page_values = page_values;
+  p.last_page_len = last_page_len;
+  p.output = static_cast<half_t*>(output);
+  p.lse = lse;
+  p.batch_size = batch_size;
+  p.h_q = h_q;
+  p.h_kv = h_kv;
+  p.group = h_q / h_kv;
+  p.causal = 1;
+  p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
+  hipStream_t s = as_stream(stream);
+  if (d == 128) {
+    launch_prefill<128, 128, kBoth, 16>(p, total_q, false, 0.0, s);
+  } else if (d == 64) {
+    launch_prefill<64, 64, kBoth, 16>(p, total_q, false, 0.0, s);
+  } else {
+    KV_UNSUPPORTED(true) << "batch_prefill_cached_and_new_kv: head_dim " << d << " is not built (64, 128)";
+  }
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
 int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k, const void* v,
                           const int32_t* kv_indptr, const int32_t* q_rope_position, const int32_t* mn_indptr,
                           const int32_t* mask, void* output, float* lse, int64_t rotary_mode, double rope_scale,
@@ -807,9 +878,9 @@ int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k,
   p.tree_order = mask;
   hipStream_t s = as_stream(stream);
   if (d == 128) {
-    launch_prefill<128, 128, false, 16>(p, total_q, true, rope_theta, s);
+    launch_prefill<128, 128, kRagged, 16>(p, total_q, true, rope_theta, s);
   } else if (d == 64) {
-    launch_prefill<64, 64, false, 16>(p, total_q, true, rope_theta, s);
+    launch_prefill<64, 64, kRagged, 16>(p, total_q, true, rope_theta, s);
   } else {
     KV_UNSUPPORTED(true) << "batch_tree_attn: head_dim " << d << " is not built (64, 128)";
   }
@@ -860,9 +931,9 @@ int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void*
   p.tree_order = tree_order;
   hipStream_t s = as_stream(stream);
   if (d == 128) {
-    launch_prefill<128, 128, true, 16>(p, total_q, true, rope_theta, s);
+    launch_prefill<128, 128, kPaged, 16>(p, total_q, true, rope_theta, s);
   } else if (d == 64) {
-    launch_prefill<64, 64, true, 16>(p, total_q, true, rope_theta, s);
+    launch_prefill<64, 64, kPaged, 16>(p, total_q, true, rope_theta, s);
   } else {
     KV_UNSUPPORTED(true) << "tree_attn_paged_kv: head_dim " << d << " is not built (64, 128)";
   }

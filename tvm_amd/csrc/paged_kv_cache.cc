@@ -1257,6 +1257,20 @@ class PagedKVCache {
   void AttentionInternal(int64_t layer_id, const void* q, const void* k, const void* v, void* output,
                          int64_t total_seq_length, double sm_scale) {
     int64_t local_layer_id = layer_id - layer_id_begin_offset_;
+    // A chunked-prefill step of a plain cache (one depth, no sliding window, no inline RoPE, no
+    // token tree): self-attention over the new tokens, attention over the cached ones and their
+    // merge (:2169-2177, :2285-2292) in one pass over both key sets.
+    if (!append_before_attn_ && num_depths_ == 1 && is_chain_on_depths_[0] && !use_decode_kernel_[0] &&
+        page_indices_view_[0].size > 0 && !support_sliding_window_ && attn_kinds_[layer_id] == TVMKV_ATTN_MHA &&
+        rope_mode_ != TVMKV_ROPE_INLINE && qk_head_dim_ == v_head_dim_ && (qk_head_dim_ == 64 || qk_head_dim_ == 128)) {
+      Launch(tvmkv_batch_prefill_cached_and_new_kv(q, cur_append_length_indptr_view_.ptr, k, v, pages_[local_layer_id],
+                                                   page_indptr_view_[0].ptr, page_indices_view_[0].ptr,
+                                                   length_info_view_[0].ptr, output, merged_lse_, sm_scale,
+                                                   cur_batch_size_, total_seq_length, page_indices_view_[0].size,
+                                                   num_total_pages_, num_qo_heads_, num_kv_heads_, qk_head_dim_,
+                                                   page_size_, compute_stream_));
+      return;
+    }
     bool is_first_kernel = true;
     if (!append_before_attn_) {
       is_first_kernel = false;

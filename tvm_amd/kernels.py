@@ -102,6 +102,19 @@ def batch_prefill_paged_kv(q, q_indptr, pages, page_indptr, page_values, length_
         q.shape[1], hkv, d, ps, int(length_info.dim() == 2), int(sliding_window_size), _stream()))
 
 
+def batch_prefill_cached_and_new_kv(q, q_indptr, k, v, pages, page_indptr, page_values, last_page_len, output, lse,
+                                    sm_scale):
+    """Ragged causal self-attention over the new tokens, paged attention over the cached ones and
+    the merge of the two, in one pass."""
+    _f16(q, k, v, pages, output)
+    _i32(q_indptr, page_indptr, page_values, last_page_len)
+    num_pages, _, hkv, ps, d = pages.shape
+    check(lib().tvmkv_batch_prefill_cached_and_new_kv(
+        _p(q), _p(q_indptr), _p(k), _p(v), _p(pages), _p(page_indptr), _p(page_values), _p(last_page_len),
+        _p(output), _p(lse), float(sm_scale), q_indptr.shape[0] - 1, q.shape[0], page_values.shape[0], num_pages,
+        q.shape[1], hkv, d, ps, _stream()))
+
+
 def batch_decode_paged_kv(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position,
                           output, lse, rotary_mode, rope_scale, rope_theta, sm_scale):
     _f16(q, pages, output)
