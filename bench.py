@@ -108,9 +108,12 @@ def calibrate(num_bytes=2 << 30, iters=10):
     K.stream_read(src, sink)
     K.stream_copy(src, dst)
     ms_read = time_region(torch, lambda i: K.stream_read(src, sink), iters)
+    K.stream_read_nt(src, sink)
+    ms_read_nt = time_region(torch, lambda i: K.stream_read_nt(src, sink), iters)
     ms_copy = time_region(torch, lambda i: K.stream_copy(src, dst), iters)
     out = {"calibration": "plain streaming kernels", "bytes": num_bytes,
            "read_GBps": round(num_bytes / ms_read / 1e6, 1), "read_ms": round(ms_read, 4),
+           "read_nt_GBps": round(num_bytes / ms_read_nt / 1e6, 1), "read_nt_ms": round(ms_read_nt, 4),
            "copy_GBps_read_plus_write": round(2 * num_bytes / ms_copy / 1e6, 1), "copy_ms": round(ms_copy, 4)}
     print(json.dumps(out))
     return out

@@ -263,6 +263,8 @@ int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr,
  * benchmark uses them to calibrate the achievable HBM bandwidth of the box, and the profiling
  * notes use the copy to scale the FETCH_SIZE / WRITE_SIZE counters. `sink` is 4 writable bytes. */
 int tvmkv_stream_read(const void* src, int64_t num_bytes, void* sink, void* stream);
+/* the same read with non-temporal loads, the kind the decode kernel issues */
+int tvmkv_stream_read_nt(const void* src, int64_t num_bytes, void* sink, void* stream);
 int tvmkv_stream_copy(const void* src, void* dst, int64_t num_bytes, void* stream);
 
 /* ======================================================================================

@@ -143,8 +143,8 @@ __global__ __launch_bounds__(256) void decode_splitkv_kernel(DecodeParams p) {
     const half_t* vbase = kbase + static_cast<int64_t>(p.h_kv) * head_stride;
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
-      kreg[j] = ld16(kbase + j * TPL * D);
-      vreg[j] = ld16(vbase + j * TPL * D);
+      kreg[j] = ld16_nt(kbase + j * TPL * D);
+      vreg[j] = ld16_nt(vbase + j * TPL * D);
     }
   };
 
@@ -495,12 +495,12 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
       for (int i = 0; i < 4; ++i) {
         const int row = i * 4 + (lane >> 4);
         const int piece = (lane & 15) ^ dm_swizzle(h * PS + row);
-        copy16_to_lds(vbase, static_cast<uint32_t>(min(row, last_row) * (D * 2) + piece * 16),
+        copy16_to_lds_nt(vbase, static_cast<uint32_t>(min(row, last_row) * (D * 2) + piece * 16),
                       vt_lds + (h * PS + i * 4) * (D * 2));
       }
       if (pi + h < page_hi) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
+        for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = ld16_nt(kbase + c16 * D + ks * 32 + g4 * 8);
       } else {
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = zero16();

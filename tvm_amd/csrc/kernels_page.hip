@@ -273,13 +273,14 @@ __global__ __launch_bounds__(256) void merge_state_inplace_kernel(half_t* __rest
 // Measurement utilities: a plain streaming read and a plain copy of known size, used to
 // calibrate what the memory system delivers and to scale hardware traffic counters.
 // ------------------------------------------------------------------------------------------
+template <bool NT>  // NT: loads carry the non-temporal hint, as the decode kernel's do
 __global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ src, int64_t n16,
                                                           uint32_t* __restrict__ sink) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   uint32_t acc = 0;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride) {
-    const uint4 v = src[i];
-    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    const Vec16 v = NT ? ld16_nt(src + i) : ld16(src + i);
+    acc ^= v.w[0] ^ v.w[1] ^ v.w[2] ^ v.w[3];
   }
   if (acc == 0x9e3779b9u) sink[0] = acc;  // keeps the loads alive; practically never taken
 }
@@ -468,11 +469,21 @@ int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr, const 
   KV_API_END();
 }
 
+int tvmkv_stream_read_nt(const void* src, int64_t num_bytes, void* sink, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(src && sink && num_bytes >= 0 && num_bytes % 16 == 0) << "stream_read_nt: bad arguments";
+  if (num_bytes == 0) return TVMKV_OK;
+  hipLaunchKernelGGL(stream_read_kernel<true>, dim3(256 * 16), dim3(256), 0, as_stream(stream),
+                     static_cast<const uint4*>(src), num_bytes / 16, static_cast<uint32_t*>(sink));
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
 int tvmkv_stream_read(const void* src, int64_t num_bytes, void* sink, void* stream) {
   KV_API_BEGIN();
   KV_CHECK(src && sink && num_bytes >= 0 && num_bytes % 16 == 0) << "stream_read: bad arguments";
   if (num_bytes == 0) return TVMKV_OK;
-  hipLaunchKernelGGL(stream_read_kernel, dim3(256 * 16), dim3(256), 0, as_stream(stream),
+  hipLaunchKernelGGL(stream_read_kernel<false>, dim3(256 * 16), dim3(256), 0, as_stream(stream),
                      static_cast<const uint4*>(src), num_bytes / 16, static_cast<uint32_t*>(sink));
   KV_LAUNCH_CHECK();
   KV_API_END();

@@ -207,6 +207,11 @@ def compact_kv_copy(pages, copy_length_indptr, copy_src_dst_pos, batch_size):
                                       copy_src_dst_pos.shape[1], num_pages, hkv, ps, d, _stream()))
 
 
+def stream_read_nt(src, sink):
+    """stream_read with non-temporal loads."""
+    check(lib().tvmkv_stream_read_nt(_p(src), src.numel() * src.element_size(), _p(sink), _stream()))
+
+
 def stream_read(src, sink):
     """Plain streaming read of the whole tensor (bandwidth calibration)."""
     check(lib().tvmkv_stream_read(_p(src), src.numel() * src.element_size(), _p(sink), _stream()))
