@@ -476,7 +476,10 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   const int v_lane_off = v_row * D + (c16 & 1) * 4;
   const int v_piece = (c16 & 3) >> 1;                // + 2 * feature block
 
-  // One step = pages (pi, pi+1).  K: lane reads row c16 of the page, features ks*32 + g4*8.
+  // One step = pages (pi, pi+1).  K: lane reads row c16 of the page, features ks*32 + g4*8, with
+  // ordinary loads: each request is a quarter of a 256-byte row, and partial rows with the streaming
+  // hint measured 10-15 % less bandwidth than without it (whole rows: 8 % more).  K through LDS
+  // with whole-row copies like V measured slower than this (two workgroups per CU instead of three).
   // V: 8 copy instructions of 4 rows x 256 bytes each fill the wave's LDS tile; rows at or past
   // kv_len repeat the last cached row of their page and a missing second page repeats the first
   // (their P is 0, and 0 times cached data is 0, whereas unwritten memory could hold NaN patterns).
@@ -500,7 +503,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
       }
       if (pi + h < page_hi) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = ld16_nt(kbase + c16 * D + ks * 32 + g4 * 8);
+        for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
       } else {
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = zero16();
