@@ -266,6 +266,16 @@ def test_decode_rejects_what_is_not_built():
     assert info.value.code == -2
 
 
+def test_decode_large_gqa_groups_plain_cache():
+    """Multi-query shapes (one kv head for 32 or 12 query heads) on a plain cache: groups the decode
+    kernels are not built for take the paged prefill kernel."""
+    for hq, hkv, d in ((32, 1, 128), (12, 1, 64), (24, 2, 64)):
+        rng = np.random.default_rng(27)
+        go, gl, eo, el = _decode_both(rng, [5, 130, 1000, 16], hq, hkv, d, 80)
+        assert_close(go, eo, what=f"decode out {hq}/{hkv}/{d}")
+        assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"decode lse {hq}/{hkv}/{d}")
+
+
 @pytest.mark.parametrize("rotary", [0, 1])
 @pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (16, 16, 64), (32, 1, 128)])
 def test_decode_sliding_cache_and_inline_rope_other_shapes(hq, hkv, d, rotary):

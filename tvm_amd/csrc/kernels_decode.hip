@@ -745,10 +745,14 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
   KV_CHECK(q && pages && page_indptr && length_info && output && lse) << "batch_decode_paged_kv: NULL tensor";
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_decode_paged_kv: NULL page table";
 
-  if (ext && !(d == 128 && h_q / h_kv <= 16)) {
+  const int gqa = h_q / h_kv;
+  const bool mfma_shape = d == 128 && gqa <= 16;
+  const bool valu_shape = gqa == 1 || gqa == 2 || gqa == 4 || gqa == 8;
+  if (!mfma_shape && (ext || !valu_shape)) {
     // Inline RoPE and the sliding-window length_info (3, B) are built into the matrix-core kernel
-    // only (head_dim 128, GQA groups up to 16).  Other shapes run as a paged prefill with one query
-    // per sequence, which has both: one workgroup per (sequence, kv head), no split over the keys.
+    // only (head_dim 128, GQA groups up to 16), and the vector kernel for the other shapes has GQA
+    // groups 1, 2, 4, 8.  What neither covers runs as a paged prefill with one query per sequence:
+    // one workgroup per (sequence, kv head), no split over the keys.
     int32_t* q_indptr = reinterpret_cast<int32_t*>(
         static_cast<char*>(get_workspace(kArrivalBytes + (static_cast<size_t>(batch_size) + 1) * sizeof(int32_t))) +
         kArrivalBytes);
