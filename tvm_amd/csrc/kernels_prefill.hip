@@ -363,8 +363,52 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
       }
     }
   };
+  // The same copies for head dim 128 and a tile whose 64 rows all exist in the source (every tile
+  // but the last of a source): nothing to clamp, the wave's 16 rows are one page or 16 consecutive
+  // k / v rows, the 4 rows of a copy instruction are selected through the scalar base, and per lane
+  // only the row inside the instruction and the swizzled piece remain -- a handful of vector
+  // instructions per tile instead of five per copy, and no branches.
+  auto issue_full_tile = [&](int tile) {
+    const bool from_pages = BOTH ? tile < prefix_tiles : PAGED;  // wave-uniform
+    const uint32_t stage = lds_base + (tile % NSTAGE) * (STAGE * 2) + wave_u * (RPW * 128 * 2);
+    const half_t* kbase;
+    const half_t* vbase;
+    uint32_t row_bytes;
+    if (from_pages) {
+      const int page = __builtin_amdgcn_readlane(page_ids, tile & 63);
+      kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * (PS * 128);
+      vbase = kbase + static_cast<int64_t>(p.h_kv) * (PS * 128);
+      row_bytes = 256;
+    } else {
+      const int64_t first_row = static_cast<int64_t>(tile) * BN - prefix_pad + wave_u * RPW;
+      kbase = k_seq + first_row * p.h_kv * 128;
+      vbase = v_seq + first_row * p.h_kv * 128;
+      row_bytes = k_stride_bytes;
+    }
+    const uint32_t row_off = (lane >> 4) * row_bytes;
+    const uint32_t k_piece = (lane & 15) ^ (lane >> 4);              // copy i: ^ (i << 2), see k_swizzle
+    const uint32_t v_off = row_off + (((lane & 15) ^ (((lane >> 4) & 3) << 2)) << 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      copy16_to_lds(kbase + static_cast<int64_t>(i) * 2 * row_bytes, row_off + ((k_piece ^ (i << 2)) << 4),
+                    stage + i * (4 * 128 * 2));
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      copy16_to_lds(vbase + static_cast<int64_t>(i) * 2 * row_bytes, v_off, stage + BN * 128 * 2 + i * (4 * 128 * 2));
+    }
+  };
   auto issue_tile = [&](int tile) {
     if ((PAGED || (BOTH && tile < prefix_tiles)) && (tile & 63) == 0) load_page_ids(tile);
+    if constexpr (DQK == 128 && DV == 128 && NW == 4 && PS == 16) {
+      const bool from_pages = BOTH ? tile < prefix_tiles : PAGED;
+      const int rows_left = from_pages ? last_tok + 1 - tile * BN : (BOTH ? last_new + 1 - (tile * BN - prefix_pad)
+                                                                          : last_tok + 1 - tile * BN);
+      if (rows_left >= BN) {  // wave-uniform
+        issue_full_tile(tile);
+        return;
+      }
+    }
     issue_copies(tile, std::integral_constant<int, 0>{}, std::integral_constant<int, COPIES>{});
   };
 
