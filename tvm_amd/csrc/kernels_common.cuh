@@ -66,6 +66,27 @@ __device__ __forceinline__ float group_sum(float x) {
   return x;
 }
 
+// Reductions over the lane pairs (l, l ^ 32) and (l, l ^ 16) with the gfx950 lane-swap
+// instructions (vector ALU; a __shfl_xor goes through LDS and its latency).  With both operands
+// equal to x, v_permlane32_swap leaves x[l & 31] in one result and x[(l & 31) + 32] in the other
+// in every lane, and v_permlane16_swap likewise for the 16-lane rows (0, 1) and (2, 3).
+__device__ __forceinline__ float max_xor32(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_xor32(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float max_xor16(float x) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_xor16(float x) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // ---- asynchronous global -> LDS copies, transposing LDS reads (gfx950) -----------------------
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 

@@ -547,8 +547,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
         mx = fmaxf(mx, v);
       }
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_xor32(max_xor16(mx));
     // the reference point moves only when the maximum exceeds it by more than 2^8 (p stays <= 256):
     // after the first steps almost no step rescales O
     const float m_new = mx > m + 8.0f ? mx : m;
@@ -597,8 +596,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   }
 
   // ---- the row sums are per lane group: add them up; m is already common -----------------------
-  lsum += __shfl_xor(lsum, 16, 64);
-  lsum += __shfl_xor(lsum, 32, 64);
+  lsum = sum_xor32(sum_xor16(lsum));
 
   // ---- merge the 4 waves through LDS: o[db][j] is feature db*16 + 4*g4 + j of head c16 ---------
   // (the wave's V tile is dead now and becomes its [16][D] fp32 output buffer)

@@ -291,8 +291,7 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
 #pragma unroll
       for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[tb][j]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_xor32(max_xor16(mx));
     // The reference point only moves when the maximum exceeds it by more than 2^8 (p stays <= 256,
     // same relative precision in fp16), so that after the first tiles no block rescales O; a fully
     // masked row keeps its reference point.
@@ -329,8 +328,7 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
   }
 
   // the row sums are per lane group: add them up; m is already common
-  lsum += __shfl_xor(lsum, 16, 64);
-  lsum += __shfl_xor(lsum, 32, 64);
+  lsum = sum_xor32(sum_xor16(lsum));
   if (row_valid) {
   const int64_t grow = static_cast<int64_t>(q_start + my_pos) * h_q + my_head;  // global row
   if (nchunks == 1) {

@@ -463,7 +463,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     float mx = -3.0e38f;
 #pragma unroll
     for (int j = 0; j < 16; ++j) mx = fmaxf(mx, acc[j]);
-    return fmaxf(mx, __shfl_xor(mx, 32, 64));
+    return max_xor32(mx);
   };
   // The reference point m of the running softmax only has to bound the scores from above up to a
   // factor that fp16 holds comfortably: it moves when a row's maximum exceeds it by more than
@@ -626,7 +626,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   }
 
   // ---- epilogue ------------------------------------------------------------------------------
-  lsum += __shfl_xor(lsum, 32, 64);
+  lsum = sum_xor32(lsum);
   const float denom = lsum + fast_exp2(kNegInit - m);  // the d = 1 of the initial state
   if (row_valid) {
     const float inv = 1.0f / denom;
