@@ -561,7 +561,10 @@ def test_prefill_cached_and_new_in_one_pass(hq, hkv, d):
     rng = np.random.default_rng(44)
     prefix = [0, 1, 63, 64, 65, 128, 200, 700, 16, 330]
     chunk = [5, 130, 1, 64, 33, 300, 2, 40, 129, 64]
-    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, prefix, 128, hkv, 16, d)
+    if d == 64:  # more than 64 sequences: the kernel takes them in batch order
+        prefix += [int(x) for x in rng.integers(0, 100, size=60)]
+        chunk += [int(x) for x in rng.integers(1, 50, size=60)]
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, prefix, 512, hkv, 16, d)
     n = sum(chunk)
     ind = np.concatenate([[0], np.cumsum(chunk)]).astype(np.int32)
     q = rng.standard_normal((n, hq, d)).astype(F16)
