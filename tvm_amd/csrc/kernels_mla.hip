@@ -73,12 +73,15 @@ constexpr int MLA_STAGES = 4;   // 4 x 36 KiB of LDS: three tiles in flight behi
 // LDS image of a tile: DQK/64 column blocks of [MLA_BN rows][64 features] (128-byte rows, 8 pieces
 // of 16 bytes).  The same bytes are the A-operand of S^T = KV Q^T (ds_read_b128: 16 lanes = 16
 // consecutive rows at one piece) and, for the latent part, of O^T = V^T P^T (ds_read_b64_tr_b16: 32
-// lanes = 8 consecutive rows x 32 bytes).  Piece c of row r sits at piece position
-// c ^ mla_swizzle(r), the bit reversal of (r >> 1) & 7: rows 2 and 4 apart land in other 32-byte
-// parts of the 256-byte bank line (odd rows are its other half anyway), and 16 consecutive rows
-// take 16 different positions.
+// lanes = 8 consecutive rows x 32 bytes).  Piece c of row r sits at piece position c ^ (r & 7).
+// A ds_read_b128 is served in four passes of 16 lanes, and the passes are not the four quarters of
+// the wave: within each half of it, the 4-lane blocks {0, 3, 5, 6} form one pass and {1, 2, 4, 7} the
+// other (measured: two such blocks on the same banks cost a cycle, two blocks of different passes do
+// not).  For the K fragment that is rows {0-3, 12-15} at one piece and rows {4-11} at the next one;
+// with this swizzle the 16 lanes of a pass cover all 64 banks, and so do the 32 lanes of a pass of
+// the transposing read.
 __device__ __forceinline__ int mla_swizzle(int row) {
-  return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);
+  return row & 7;
 }
 
 template <int DQK, int DV>
