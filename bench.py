@@ -135,7 +135,8 @@ def measured_traffic(algorithmic_bytes):
 
 
 def extras(torch, K, dev):
-    """configs[3] and configs[4] of BASELINE.json, kernels only (inputs resident, HIP events)."""
+    """configs[3] and configs[4] of BASELINE.json, and the sliding-window and token-tree variants of the
+    attention kernels on configs[1]'s shape; kernels only (inputs resident, HIP events)."""
     out = {}
 
     def i32(a):
@@ -164,6 +165,72 @@ def extras(torch, K, dev):
     out["long_context_decode"] = {"workload": "configs[3]: 8 seqs, ctx U[32768,131072] seed 3, Hq64/Hkv8/D128, page 16",
                                   "kv_tokens": int(ctx.sum()), "ms": round(ms, 4),
                                   "GBps": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    del pages
+    torch.cuda.empty_cache()
+
+    # ---- sliding window + attention sinks, and a token-tree verify step, on configs[1]'s shape ----
+    hq, hkv, d, ps, nseq = 32, 8, 128, 16, 64
+    rng = np.random.default_rng(7)
+    sink, window = 4, 4096
+    offset = rng.integers(sink, sink + ps, size=nseq)           # physical slot of the first window token
+    phys = offset + window                                       # slots in use: sinks, a gap, the window
+    npages = (phys + ps - 1) // ps
+    pool = 65536
+    perm = rng.permutation(pool).astype(np.int32)
+    pages = torch.empty((pool, 2, hkv, ps, d), dtype=torch.float16, device=dev)
+    for lo in range(0, pool, 8192):
+        pages[lo:lo + 8192].normal_()
+    indptr = np.concatenate([[0], np.cumsum(npages)])
+    q = torch.randn((nseq, hq, d), device=dev).to(torch.float16)
+    o = torch.empty_like(q)
+    lse = torch.empty((nseq, hq), dtype=torch.float32, device=dev)
+    z = torch.zeros(nseq, dtype=torch.int32, device=dev)
+    info = i32(np.stack([(phys - 1) % ps + 1, offset, np.full(nseq, sink)]))
+    args = (q, pages, i32(indptr), i32(perm[:indptr[-1]]), info, z, z, o, lse, 0, 1.0, 1e4, d ** -0.5)
+    K.batch_decode_paged_kv(*args)
+    ms = time_region(torch, lambda i: K.batch_decode_paged_kv(*args), 10)
+    nbytes = float(nseq * (sink + window)) * 2 * hkv * d * 2 + 2 * nseq * hq * d * 2
+    out["sliding_window_decode"] = {"workload": "64 seqs, 4 sink tokens + a 4096-token window each (length_info with 3 rows), "
+                                                "Hq32/Hkv8/D128, page 16",
+                                    "ms": round(ms, 4), "GBps": round(nbytes / ms / 1e6, 1),
+                                    "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+
+    def preorder(depth):  # (first, second) labels of a complete binary tree listed in depth-first order
+        labels = []
+
+        def walk(level):
+            me = len(labels)
+            labels.append([me, 0])
+            if level + 1 < depth:
+                walk(level + 1)
+                walk(level + 1)
+            labels[me][1] = len(labels)
+        walk(0)
+        return np.asarray(labels, dtype=np.int32)
+
+    labels = preorder(6)                                          # 63 draft tokens per sequence
+    nodes = len(labels)
+    ctx = rng.integers(1024, 8192, size=nseq, endpoint=True)    # cached tokens before the tree
+    kv = ctx + nodes                                              # the tree's tokens are appended already
+    npages = (kv + ps - 1) // ps
+    indptr = np.concatenate([[0], np.cumsum(npages)])
+    qi = np.arange(nseq + 1) * nodes
+    q = torch.randn((nseq * nodes, hq, d), device=dev).to(torch.float16)
+    o = torch.empty_like(q)
+    lse = torch.empty((nseq * nodes, hq), dtype=torch.float32, device=dev)
+    zq = torch.zeros(nseq * nodes, dtype=torch.int32, device=dev)
+    args = (q, i32(qi), pages, i32(indptr), i32(perm[:indptr[-1]]), i32((kv - 1) % ps + 1), z, zq, o, lse, 0, 1.0, 1e4,
+            d ** -0.5, i32(qi), i32(np.tile(labels, (nseq, 1)).reshape(-1)))
+    K.tree_attn_paged_kv(*args)
+    ms = time_region(torch, lambda i: K.tree_attn_paged_kv(*args), 10)
+    depth_sum = float(sum((lv + 1) * 2 ** lv for lv in range(6)))  # visible tree tokens summed over the nodes
+    flops = 4.0 * hq * d * (float(ctx.sum()) * nodes + nseq * depth_sum)
+    nbytes = float(kv.sum()) * 2 * hkv * d * 2 + 2 * nseq * nodes * hq * d * 2
+    out["token_tree_verify"] = {"workload": "64 seqs, ctx U[1024,8192], a 63-node binary draft tree each (appended), "
+                                            "one launch of the tree-masked paged kernel, Hq32/Hkv8/D128",
+                                "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                                "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                                "GBps": round(nbytes / ms / 1e6, 1)}
     del pages
     torch.cuda.empty_cache()
 
