@@ -443,6 +443,7 @@ def main():
             cpu_bytes += float(t["kv_len"].sum()) * TOKEN_BYTES + qo_bytes
             steps_done += 1
             if s == last:  # the GPU buffers hold the last step's result
+                eo_last = eo
                 err = float(np.max(np.abs(out.cpu().numpy().astype(np.float32) - eo.astype(np.float32))))
             if cpu_s > 12.0:
                 break
@@ -453,6 +454,36 @@ def main():
                                             f"kv tokens each), 1 thread, {cpu_s:.1f} s; the reference kernel is T.serial",
                                   "tokens_per_s": round(B * steps_done / cpu_s, 2), "host_cpus": os.cpu_count(),
                                   "gpu_vs_cpu_max_abs_err": err}
+
+        # The same kernel on all of the box's host cores: one task per sequence (sequences are
+        # independent in the reference kernel), the C calls run outside the interpreter lock.
+        from concurrent.futures import ThreadPoolExecutor
+        threads = max(1, min(16, len(os.sched_getaffinity(0))))
+        par_s, par_bytes, par_steps = 0.0, 0.0, 0
+        with ThreadPoolExecutor(threads) as pool:
+            for s in range(last, last - steps_done, -1):
+                t = wl["tables"][s]
+                values = np.array([renumber[int(pid)] for pid in t["page_values"]], np.int32)
+                qh = np.zeros((B, HQ, D), np.float16)
+                kh = np.zeros((B, HKV, D), np.float16)
+                vh = np.zeros((B, HKV, D), np.float16)
+                po = np.zeros((B, HQ, D), np.float16)
+                pl = np.zeros((B, HQ), np.float32)
+                order = np.argsort(-t["kv_len"])  # longest first
+                c0 = time.perf_counter()
+                ok.fused_rope(qkv_host[s - W], t["q_rope_position"], qh, kh, vh, 1)
+                list(pool.map(lambda b: ok.decode_range(qh, host_pages, t["page_indptr"], values, t["last_page_len"], z, z,
+                                                        po, pl, int(b), int(b) + 1, sm_scale), order))
+                par_s += time.perf_counter() - c0
+                par_bytes += float(t["kv_len"].sum()) * TOKEN_BYTES + qo_bytes
+                par_steps += 1
+                if s == last:
+                    assert np.array_equal(po, eo_last), "threaded CPU run differs from the serial one"
+        result["cpu_baseline_all_cores"] = {"value": round(par_bytes / par_s / 1e9, 3), "unit": "GB/s", "cores": threads,
+                                            "kind": "port",
+                                            "sample": f"the same {par_steps} decode steps, one task per sequence on "
+                                                      f"{threads} threads, {par_s:.1f} s",
+                                            "tokens_per_s": round(B * par_steps / par_s, 2)}
 
     if args.extras:
         del pages, qkv
