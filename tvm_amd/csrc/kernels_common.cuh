@@ -139,6 +139,17 @@ __device__ __forceinline__ half4_t lds_read_tr16(const half_t* p) {
   return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr_t)p));
 }
 
+// The same reads from an LDS byte address held in a register (plus what the compiler folds into
+// the instruction's immediate offset).
+typedef __attribute__((address_space(3))) const half8_t* lds_half8_cptr_t;
+__device__ __forceinline__ half8_t lds_read_b128_at(uint32_t addr) {
+  return *reinterpret_cast<lds_half8_cptr_t>(static_cast<uintptr_t>(addr));
+}
+__device__ __forceinline__ half4_t lds_read_tr16_at(uint32_t addr) {
+  return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                         reinterpret_cast<lds_short4_ptr_t>(static_cast<uintptr_t>(addr))));
+}
+
 // s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters at their maximum)
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {

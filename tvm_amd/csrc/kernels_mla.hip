@@ -8,12 +8,14 @@
 // same kernel for MLA decode (src/runtime/vm/paged_kv_cache.cc:954-956), and so does this one.
 // Numerics as in kernels_prefill.hip (base-2 online softmax, m = -5e4, d = 1 initial state).
 //
-// Tiling: 128 rows (position, head) per workgroup of 8 wavefronts, 16 rows per wave with the query
-// on the N axis of v_mfma_f32_16x16x32_f16: O^T of one wave is 512 x 16 fp32 = 128 accumulator
-// registers, Q is 72 registers of B-fragments, which leaves room for two waves per SIMD.  32-token
-// tiles of cached rows are copied from global memory straight into LDS (global_load_lds_dwordx4),
-// four stages deep; the same LDS bytes serve as A-operand of S^T = KV Q^T (ds_read_b128) and of
-// O^T = V^T P^T (ds_read_b64_tr_b16, which transposes on the way out of LDS).
+// Tiling: 128 rows (position, head) per workgroup of 4 wavefronts, 32 rows per wave with the query
+// on the N axis of v_mfma_f32_32x32x16_f16: O^T of one wave is 512 x 32 fp32 = 256 accumulator
+// registers and Q is 144 registers of B-fragments, so a wave has a SIMD's whole register file (one
+// workgroup per compute unit) and overlaps its own matrix and vector work.  32-token tiles of cached
+// rows are copied from global memory straight into LDS (global_load_lds_dwordx4), four stages; the
+// same LDS bytes serve as A-operand of S^T = KV Q^T (ds_read_b128) and of O^T = V^T P^T
+// (ds_read_b64_tr_b16, which transposes on the way out of LDS).  Per matrix instruction the LDS
+// delivers half as many bytes as with 16-row waves, which were bound by it.
 //
 // KV split: decode-shaped calls (one token per sequence) have too few row tiles to fill 256 CUs,
 // so the KV of a sequence is cut into chunks of about `chunk_tokens` tokens; partial (O, m, l)
@@ -21,6 +23,8 @@
 // chunk slots of a sequence are a pure function of the page table, recomputed by both kernels.
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
+#include <utility>
 
 #include "kernels_common.cuh"
 
@@ -67,45 +71,82 @@ __device__ __forceinline__ int mla_chunk_slot_begin(const int32_t* page_indptr, 
   return static_cast<int>(static_cast<int64_t>(page_indptr[b]) * page_size / chunk_tokens) + b;
 }
 
-constexpr int MLA_WAVES = 8;    // wavefronts per workgroup, 16 rows each
-constexpr int MLA_STAGES = 4;   // 4 x 36 KiB of LDS: three tiles in flight behind the one being multiplied
+constexpr int MLA_WAVES = 4;    // wavefronts per workgroup, 32 rows each, one per SIMD
+constexpr int MLA_STAGES = 4;   // 4 x 36 KiB of LDS: the tile whose V is in use, the one whose K is, two in flight
 
 // LDS image of a tile: DQK/64 column blocks of [MLA_BN rows][64 features] (128-byte rows, 8 pieces
-// of 16 bytes).  The same bytes are the A-operand of S^T = KV Q^T (ds_read_b128: 16 lanes = 16
-// consecutive rows at one piece) and, for the latent part, of O^T = V^T P^T (ds_read_b64_tr_b16: 32
-// lanes = 8 consecutive rows x 32 bytes).  Piece c of row r sits at piece position c ^ (r & 7).
-// A ds_read_b128 is served in four passes of 16 lanes, and the passes are not the four quarters of
-// the wave: within each half of it, the 4-lane blocks {0, 3, 5, 6} form one pass and {1, 2, 4, 7} the
-// other (measured: two such blocks on the same banks cost a cycle, two blocks of different passes do
-// not).  For the K fragment that is rows {0-3, 12-15} at one piece and rows {4-11} at the next one;
-// with this swizzle the 16 lanes of a pass cover all 64 banks, and so do the 32 lanes of a pass of
-// the transposing read.
+// of 16 bytes).  The same bytes are the A-operand of S^T = KV Q^T (ds_read_b128: lane = key row, one
+// piece) and, for the latent part, of O^T = V^T P^T (ds_read_b64_tr_b16: 32 lanes = 4 consecutive
+// rows x 64 bytes).  Piece c of row r sits at piece position c ^ mla_swizzle(r).  The LDS serves a
+// ds_read_b128 in four passes of 16 lanes, and within each half of the wave the 4-lane blocks
+// {0, 3, 5, 6} form one pass and {1, 2, 4, 7} the other (measured: two such blocks on the same banks
+// cost a cycle, blocks of different passes do not); the transposing read takes two passes of 32
+// consecutive lanes.  With this swizzle the rows of every pass of either read cover all 64 banks.
 __device__ __forceinline__ int mla_swizzle(int row) {
-  return row & 7;
+  return (((row >> 1) & 1) << 2) | ((row >> 3) & 3);
+}
+
+// ---- O in fixed accumulation registers ------------------------------------------------------------
+// O^T of a wave is 512 x 32 fp32 = all 256 accumulation registers of the SIMD.  They are addressed by
+// number from assembly and never handed to the register allocator (which, asked to keep 16 tuples
+// of 16 in that file across a loop that also touches them from the vector ALU, moves them into
+// ordinary registers and spills the Q fragments): block db is a[16*db : 16*db+15].  The compiler
+// therefore knows nothing of the matrix instructions on them, and the wait states it would insert
+// around accumulation-register reads and writes are written out where they are needed.  The file
+// must be compiled with -mllvm -amdgpu-spill-vgpr-to-agpr=0 so that no spill lands in these
+// registers.
+template <int R>
+__device__ __forceinline__ void acc_mfma_32x32x16(half8_t a, half8_t b) {  // a[R:R+15] += a * b
+  asm volatile("v_mfma_f32_32x32x16_f16 a[%2:%3], %0, %1, a[%2:%3]" : : "v"(a), "v"(b), "n"(R), "n"(R + 15));
+}
+template <int R>
+__device__ __forceinline__ void acc_zero() {
+  asm volatile("v_accvgpr_write_b32 a[%0], 0" : : "n"(R));
+}
+template <int R>
+__device__ __forceinline__ float acc_read() {
+  float x;
+  asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(R));
+  return x;
+}
+template <int R>
+__device__ __forceinline__ void acc_scale(float factor) {
+  float t;
+  asm volatile("v_accvgpr_read_b32 %0, a[%2]\n\tv_mul_f32 %0, %0, %1\n\tv_accvgpr_write_b32 a[%2], %0"
+               : "=&v"(t) : "v"(factor), "n"(R));
+}
+// wait states between the last matrix instruction that writes an accumulation register and a vector
+// instruction that reads it (or the reverse), more than any case needs
+__device__ __forceinline__ void acc_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {  // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 template <int DQK, int DV>
-__global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) {
+__global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams p) {
   constexpr int BN = MLA_BN;
-  static_assert(BN == 32 && MLA_BM == MLA_WAVES * 16 && DQK % 64 == 0 && DV % 64 == 0 && DV <= DQK, "tile shape");
-  constexpr int KS = DQK / 32;               // k-steps of the score product (v_mfma_f32_16x16x32_f16)
-  constexpr int DB = DV / 16;                // 16-wide output feature blocks
+  static_assert(BN == 32 && MLA_BM == MLA_WAVES * 32 && DQK % 64 == 0 && DV % 64 == 0 && DV <= DQK, "tile shape");
+  constexpr int KS = DQK / 16;               // k-steps of the score product (v_mfma_f32_32x32x16_f16)
+  constexpr int DB = DV / 32;                // 32-wide output feature blocks
   constexpr int NBLK = DQK / 64;             // column blocks of a tile
   constexpr int BLK = BN * 64;               // halfs per column block
   constexpr int STAGE = NBLK * BLK;          // halfs per stage
   constexpr int NSTAGE = MLA_STAGES;
   constexpr int NCOPY = NBLK * (BN / 8);     // copy instructions (8 rows x 128 B) per tile
-  constexpr int COPIES_HI = (NCOPY + MLA_WAVES - 1) / MLA_WAVES;  // per wave: the first NCOPY % MLA_WAVES waves
-  constexpr int COPIES_LO = NCOPY / MLA_WAVES;                    // ... the others
-  constexpr int WAVES_HI = NCOPY % MLA_WAVES;
+  static_assert(NCOPY % MLA_WAVES == 0 && NSTAGE == 4, "copy split / pipeline depth");
+  constexpr int COPIES = NCOPY / MLA_WAVES;  // per wave and tile
 
   extern __shared__ __attribute__((aligned(16))) half_t lds_tiles[];
+  asm volatile("" ::: "a0", "a255");  // the kernel uses every accumulation register (by number, see above)
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
-  const int lane = tid & 63;
-  const int c16 = lane & 15;   // query row of the wave (MFMA column) / token row of an A-fragment
-  const int g4 = lane >> 4;    // lane group: contraction slots 8*g4 .. 8*g4+7
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // a scalar: the bounds derived from it steer wave-uniform branches
   const int h_q = p.h_q;
 
   // Work item.  Normal mode: a row-tile slot.  Split mode: (chunk slot, row tile of a one-token
@@ -160,7 +201,14 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
 
   // normal mode: one pass; split mode: one pass per row tile this workgroup owns (one, for a decode step)
   for (; r0 < rows; r0 += row_step) {
-  const int my_row = r0 + wave * 16 + c16;
+  // Everything that depends on the lane is derived inside the pass from a value the compiler
+  // cannot see through: hoisted out of this (rarely taken) loop, the per-lane addresses would stay
+  // live across the epilogue, be spilled there, and be reloaded in the tile loop.
+  int lane = tid & 63;
+  asm volatile("" : "+v"(lane));
+  const int col = lane & 31;   // query row of the wave (MFMA column) / key row of an A-fragment
+  const int half = lane >> 5;  // contraction slots 8*half .. 8*half+7
+  const int my_row = r0 + wave * 32 + col;
   const bool row_valid = my_row < rows;
   const int my_pos = my_row / h_q;
   const int my_head = my_row % h_q;
@@ -168,8 +216,8 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
   const int my_limit = row_valid ? (p.causal ? min(kv_len, causal_shift + my_pos) : kv_len) : 0;
   const int last_row_wg = min(rows, r0 + MLA_BM) - 1;
   const int kv_end = p.causal ? max(0, min(kv_len, causal_shift + last_row_wg / h_q)) : kv_len;
-  const int first_row_wave = r0 + wave * 16;
-  const int last_row_wave = min(rows, first_row_wave + 16) - 1;
+  const int first_row_wave = r0 + wave * 32;
+  const int last_row_wave = min(rows, first_row_wave + 32) - 1;
   const bool wave_active = first_row_wave < rows;
   const int wave_limit_max = !wave_active ? 0 : (p.causal ? min(kv_len, causal_shift + last_row_wave / h_q) : kv_len);
   const int wave_limit_min = !wave_active ? 0 : (p.causal ? min(kv_len, causal_shift + first_row_wave / h_q) : kv_len);
@@ -179,28 +227,25 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
   const int tile_lo = static_cast<int>(static_cast<int64_t>(chunk) * tiles_all / nchunks);
   const int tile_hi = min(static_cast<int>(static_cast<int64_t>(chunk + 1) * tiles_all / nchunks), (kv_end + BN - 1) / BN);
 
-  // Q^T fragments (B operand): column = query c16, contraction slots = features ks*32 + g4*8 .. +7
+  // Q^T fragments (B operand): column = query col, contraction slots = features ks*16 + half*8 .. +7
   half8_t qf[KS];
   {
-    const half_t* qrow = p.q + (static_cast<int64_t>(q_start + my_pos) * h_q + my_head) * DQK + g4 * 8;
+    const half_t* qrow = p.q + (static_cast<int64_t>(q_start + my_pos) * h_q + my_head) * DQK + half * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_valid ? ld16(qrow + ks * 32).h8 : zero16().h8;
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_valid ? ld16(qrow + ks * 16).h8 : zero16().h8;
   }
-  // O^T accumulators: o[db][j] is feature db*16 + 4*g4 + j of query c16
-  float4_t o[DB];
-#pragma unroll
-  for (int db = 0; db < DB; ++db) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
+  // O^T accumulators: register 16*db + j is feature db*32 + (j/4)*8 + half*4 + j%4 of query col
+  static_assert(DB * 16 == 256, "O fills the accumulation registers");
+  static_for<DB * 16>([&](auto r) { acc_zero<decltype(r)::value>(); });
   float m = kNegInit, lsum = 0.f;
 
   // ---- tile copy: global -> LDS -------------------------------------------------------------
-  // Copy instruction n of a tile (n = 0 .. NCOPY-1, dealt out to the waves in consecutive runs)
-  // moves rows 8*(n%4) .. +7 of column block n/4.  Rows past the end of the sequence repeat its last
-  // token (masked scores; P = 0 times a finite value).  The page ids of 16 consecutive tiles (4 row
+  // Copy instruction n of a tile (n = 0 .. NCOPY-1, COPIES consecutive ones per wave) moves rows
+  // 8*(n%4) .. +7 of column block n/4.  Rows past the end of the sequence repeat its last token
+  // (masked scores; P = 0 times a finite value).  The page ids of 16 consecutive tiles (4 row
   // groups each) are fetched by one vector load, lane = 4*tile + row group: the wait for that load
   // also waits for every copy in flight, so it must be rare.
-  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  const bool copies_hi = wave_u < WAVES_HI;
-  const int copy_first = copies_hi ? wave_u * COPIES_HI : WAVES_HI * COPIES_HI + (wave_u - WAVES_HI) * COPIES_LO;
+  const int copy_first = wave * COPIES;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds_tiles));
   const int last_tok = kv_len - 1;
   int page_ids = 0;
@@ -213,146 +258,231 @@ __global__ __launch_bounds__(MLA_WAVES * 64) void mla_paged_kernel(MlaParams p) 
     const int kv0 = tile * BN;
     const uint32_t stage = lds_base + (w % NSTAGE) * (STAGE * 2);
 #pragma unroll
-    for (int j = 0; j < COPIES_HI; ++j) {
-      if (j < COPIES_LO || copies_hi) {  // wave-uniform
-        const int n = copy_first + j;
-        const int blk = n >> 2;
-        const int rg = n & 3;
-        const int page = __builtin_amdgcn_readlane(page_ids, (w & 15) * 4 + rg);
-        const half_t* base = p.pages + static_cast<int64_t>(page) * ps * DQK;
-        const int row = rg * 8 + (lane >> 3);
-        const int piece = (lane & 7) ^ mla_swizzle(row);
-        const uint32_t t = min(kv0 + row, last_tok);
-        const uint32_t off = (t % ps) * (DQK * 2) + (blk * 64 + piece * 8) * 2;
-        copy16_to_lds(base, off, stage + (blk * BLK + rg * 8 * 64) * 2);
-      }
+    for (int j = 0; j < COPIES; ++j) {
+      const int n = copy_first + j;
+      const int blk = n >> 2;
+      const int rg = n & 3;
+      const int page = __builtin_amdgcn_readlane(page_ids, (w & 15) * 4 + rg);
+      const half_t* base = p.pages + static_cast<int64_t>(page) * ps * DQK;
+      const int row = rg * 8 + (lane >> 3);
+      const int piece = (lane & 7) ^ mla_swizzle(row);
+      const uint32_t t = min(kv0 + row, last_tok);
+      const uint32_t off = (t % ps) * (DQK * 2) + (blk * 64 + piece * 8) * 2;
+      copy16_to_lds(base, off, stage + (blk * BLK + rg * 8 * 64) * 2);
     }
   };
 
-  // ---- per-lane fragment addressing (halfs, relative to a stage) ---------------------------------
-  // K A-fragment of k-step ks, token block tb: row tb*16 + c16, features ks*32 + g4*8 .. +7
-  const int k_lane_off = c16 * 64;
-  const int k_swz = mla_swizzle(c16);  // the same for row + 16
+  // ---- per-lane fragment addressing (LDS byte addresses) -------------------------------------------
+  // A fragment's 16-byte piece sits at (logical piece ^ swizzle of its row); the logical piece is a
+  // lane part XOR a part known at compile time, and every other term of the address is a multiple
+  // of the 128-byte row.  So each product keeps ONE per-lane offset, adds the stage's base once per
+  // tile, and reaches every fragment with an XOR of bits 4..6 and an immediate offset (registers
+  // are what this kernel is short of).
+  // K A-fragment of k-step ks: key row col, features ks*16 + half*8 .. +7: column block ks/4,
+  // logical piece (ks%4)*2 + half.
+  const uint32_t k_rel = col * 128 + ((mla_swizzle(col) ^ half) << 4);
   // V^T A-fragment via the transposing read: lane li of a 16-lane group points at 4 features of
   // token (li >> 2) of the group's 4 tokens and receives feature li of the group's 16 for the 4
-  // tokens.  Contraction slot 8*g4 + i holds token (i/4)*16 + 4*g4 + i%4, the order in which the
-  // S^T accumulators of the two token blocks hold them.
+  // tokens.  Contraction slot half*8 + i of fragment kk holds token kk*16 + (i/4)*8 + half*4 + i%4,
+  // the order in which the S^T accumulator registers hold the tokens.  Feature block db: column
+  // block db/2, logical piece (db%2)*4 + gg*2 + (li%4)/2; rows v_row + kk*16 + e*8, whose swizzle is
+  // that of v_row XOR (kk*2 + e).
   const int li = lane & 15;
-  const int v_row = 4 * g4 + (li >> 2);               // + 16 for the second half of the fragment
-  const int v_swz = mla_swizzle(v_row);               // row + 16 does not change it
-  const int v_lane_off = v_row * 64 + (li & 1) * 4;
-  const int v_piece = (li & 3) >> 1;                   // + 2 * (feature block % 4)
+  const int gg = (lane >> 4) & 1;
+  const int v_row = half * 4 + (li >> 2);
+  const uint32_t v_rel = v_row * 128 + (li & 1) * 8 + (((gg * 2 + ((li & 3) >> 1)) ^ mla_swizzle(v_row)) << 4);
 
+  // Both products read their A-fragments from LDS in groups, one group ahead of the matrix
+  // instructions that use them; scheduling fences between the groups keep the compiler from
+  // hoisting all reads of a product (which would not fit the register file).
+  constexpr int KG = 4;              // k-steps per group of the score product
+  constexpr int NKG = KS / KG;
+  constexpr int VG = 2;              // feature blocks per group of the PV product (2 fragments each)
+  constexpr int NVG = DB / VG;
+  static_assert(KS % KG == 0 && DB % VG == 0 && NVG >= 6, "fragment groups");
+  auto read_k_group = [&](uint32_t k_at, int g, half8_t (&a)[KG]) {  // k_at: stage base + k_rel
+#pragma unroll
+    for (int i = 0; i < KG; ++i) {
+      const int ks = g * KG + i;
+      a[i] = lds_read_b128_at((k_at ^ (((ks & 3) * 2) << 4)) + (ks >> 2) * (BLK * 2));
+    }
+  };
+  auto read_v_group = [&](uint32_t v_at, int g, half8_t (&a)[VG][2]) {  // v_at: stage base + v_rel
+#pragma unroll
+    for (int i = 0; i < VG; ++i) {
+      const int db = g * VG + i;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int c = ((db & 1) << 2) | (kk * 2 + e);
+          const half4_t part = lds_read_tr16_at((v_at ^ (c << 4)) + (db >> 1) * (BLK * 2) + (kk * 16 + e * 8) * 128);
+          a[i][kk][e * 4 + 0] = part[0]; a[i][kk][e * 4 + 1] = part[1];
+          a[i][kk][e * 4 + 2] = part[2]; a[i][kk][e * 4 + 3] = part[3];
+        }
+      }
+    }
+  };
+  // S^T = KV Q^T over all DQK features for the 32 tokens of a tile
+  auto qk = [&](uint32_t stage_at) -> float16_t {
+    float16_t acc;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+    half8_t a[2][KG];
+    const uint32_t k_at = stage_at + k_rel;
+    read_k_group(k_at, 0, a[0]);
+#pragma unroll
+    for (int g = 0; g < NKG; ++g) {
+      if (g + 1 < NKG) read_k_group(k_at, g + 1, a[(g + 1) & 1]);
+#pragma unroll
+      for (int i = 0; i < KG; ++i) {
+        // Written as assembly to put S into ordinary vector registers: with a whole register file
+        // per wave the compiler selects the form of the matrix instructions whose results live in
+        // accumulation registers, and O fills all 256 of those.
+        if (g == NKG - 1 && i == KG - 1) {
+          // the compiler does not know this is a matrix instruction: the wait states it would put
+          // between the last one and the first vector instruction that reads S are spelled out
+          asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7"
+              : "+v"(acc) : "v"(a[g & 1][i]), "v"(qf[g * KG + i]));
+        } else {
+          asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a[g & 1][i]), "v"(qf[g * KG + i]));
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    return acc;
+  };
+  // Online softmax of a tile's scores, cut into steps that are spread over the groups of the PV
+  // product running beside it.  s[j]: token kv0 + (j/4)*8 + half*4 + j%4, query col.  The reference
+  // point only moves when the maximum exceeds it by more than 2^8 (p stays <= 256, same relative
+  // precision in fp16), so that after the first tiles no block rescales O; a fully masked row keeps
+  // its reference point.  Step 0: mask and row maximum; 1: new reference point and the factor for
+  // the old state; 2..5: four probabilities each, as the B-operand of the next PV product.
+  float alpha = 1.0f, row_mx = 0.f;
+  auto softmax_step = [&](int step, float16_t& s, int kv0, half8_t (&pf)[2]) {
+    if (step == 0) {
+      if (kv0 + BN > wave_limit_min) {  // wave-uniform: the causal diagonal or the end of the sequence
+        asm volatile("" ::: "memory");
+        const int rel = my_limit - kv0 - half * 4;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) s[j] = ((j >> 2) * 8 + (j & 3)) < rel ? s[j] : -3.0e38f;
+      }
+      float mx = -3.0e38f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[j]);
+      row_mx = max_xor32(mx);
+    } else if (step == 1) {
+      const float cand = fmaxf(row_mx * p.scale_log2, -1.0e30f);
+      const float m_new = cand > m + 8.0f ? cand : m;
+      alpha = fast_exp2(m - m_new);
+      m = m_new;
+      lsum *= alpha;
+    } else if (step < 6) {
+#pragma unroll
+      for (int j = (step - 2) * 4; j < (step - 1) * 4; ++j) {
+        const float pj = fast_exp2(fmaf(s[j], p.scale_log2, -m));  // masked: exp2(-huge) = 0
+        lsum += pj;
+        pf[j >> 3][j & 7] = static_cast<half_t>(pj);
+      }
+    }
+  };
+  // O^T += V^T P^T (the value is the first DV features of the same rows), optionally with the
+  // softmax of the next tile's scores on the vector ALU beside it
+  auto pv = [&](uint32_t stage_at, const half8_t (&pf_in)[2], auto with_softmax, float16_t& s, int kv0, half8_t (&pf_out)[2]) {
+    half8_t a[2][VG][2];
+    const uint32_t v_at = stage_at + v_rel;
+    read_v_group(v_at, 0, a[0]);
+    static_for<NVG>([&](auto gc) {
+      constexpr int g = decltype(gc)::value;
+      if (g + 1 < NVG) read_v_group(v_at, g + 1, a[(g + 1) & 1]);
+      static_for<VG>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        acc_mfma_32x32x16<(g * VG + i) * 16>(a[g & 1][i][0], pf_in[0]);
+        acc_mfma_32x32x16<(g * VG + i) * 16>(a[g & 1][i][1], pf_in[1]);
+      });
+      if (decltype(with_softmax)::value) softmax_step(g, s, kv0, pf_out);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  auto rescale = [&]() {
+    if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {  // wave-uniform: skip when no maximum moved
+      acc_settle();
+      static_for<DB * 16>([&](auto r) { acc_scale<decltype(r)::value>(alpha); });
+      acc_settle();
+    }
+  };
+
+  // The wave is alone on its SIMD, so it overlaps its own matrix and vector work: the PV product of
+  // a tile runs one iteration late, beside the softmax of the next tile's scores.  Iteration w:
+  // S(w) = K(w) Q^T; then O += V(w-1) P(w-1) on the matrix pipe while the vector ALU turns S(w) into
+  // P(w); the rescale of O that a moved reference point asks for (rare) follows the product.
+  // Stages: tile w-1 (V in use), tile w, and tiles w+1 / w+2 in flight.  Every wave walks all tiles
+  // of the workgroup (a tile beyond a wave's own causal bound is masked like the diagonal one):
+  // with 128 heads a workgroup is a single position anyway.
   const int n_tiles = tile_hi - tile_lo;
 #pragma unroll
-  for (int s = 0; s < NSTAGE - 1; ++s) {
+  for (int s = 0; s < 2; ++s) {
     if (s < n_tiles) issue_tile(tile_lo + s);
   }
-  for (int w = 0; w < n_tiles; ++w) {
-    const int kv0 = (tile_lo + w) * BN;
-    const half_t* T = lds_tiles + (w % NSTAGE) * STAGE;
-    // copies complete in order: it is enough that no more than the later tiles' copies are outstanding
-    if (w + NSTAGE - 2 < n_tiles) {
-      if (copies_hi) {
-        wait_vmcnt<(NSTAGE - 2) * COPIES_HI>();
-      } else {
-        wait_vmcnt<(NSTAGE - 2) * COPIES_LO>();
-      }
+  auto tile_ready = [&](int w) {
+    // copies complete in order: it is enough that no more than the next tile's copies are outstanding
+    if (w + 1 < n_tiles) {
+      wait_vmcnt<COPIES>();
     } else {
       wait_vmcnt<0>();
     }
-    __syncthreads();  // everyone's part of this tile has landed; everyone is done with the stage of tile w-1
-    if (w + NSTAGE - 1 < n_tiles) issue_tile(tile_lo + w + NSTAGE - 1);
-
-    if (kv0 >= wave_limit_max) continue;  // wave-uniform: every row of this wave is masked out
-
-    // ---- S^T = KV Q^T over all DQK features: two blocks of 16 tokens ------------------------------
-    float4_t s[2];
+    __syncthreads();  // everyone's part of tile w has landed; everyone is done with the stage of tile w-2
+    if (w + 2 < n_tiles) issue_tile(tile_lo + w + 2);
+  };
+  if (n_tiles > 0) {
+    half8_t pf_prev[2];
+    float16_t s;
+    tile_ready(0);
+    s = qk(lds_base);
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb) {
-      s[tb] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int piece = ((ks & 1) * 4 + g4) ^ k_swz;
-        const half8_t a = *reinterpret_cast<const half8_t*>(T + (ks >> 1) * BLK + tb * 16 * 64 + k_lane_off + piece * 8);
-        s[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[ks], s[tb], 0, 0, 0);
-      }
+    for (int step = 0; step < 6; ++step) softmax_step(step, s, tile_lo * BN, pf_prev);  // nothing accumulated yet: no rescale
+    for (int w = 1; w < n_tiles; ++w) {
+      tile_ready(w);
+      half8_t pf[2];
+      s = qk(lds_base + (w % NSTAGE) * (STAGE * 2));
+      pv(lds_base + ((w - 1) % NSTAGE) * (STAGE * 2), pf_prev, std::true_type{}, s, (tile_lo + w) * BN, pf);
+      rescale();
+      pf_prev[0] = pf[0];
+      pf_prev[1] = pf[1];
     }
-    // s[tb][j]: token kv0 + tb*16 + 4*g4 + j, query c16
-    if (kv0 + BN > wave_limit_min) {  // wave-uniform: the causal diagonal or the end of the sequence
-      asm volatile("" ::: "memory");
-      const int rel = my_limit - kv0 - 4 * g4;
-#pragma unroll
-      for (int tb = 0; tb < 2; ++tb) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) s[tb][j] = (tb * 16 + j) < rel ? s[tb][j] : -3.0e38f;
-      }
-    }
-    float mx = -3.0e38f;
-#pragma unroll
-    for (int tb = 0; tb < 2; ++tb) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[tb][j]);
-    }
-    mx = max_xor32(max_xor16(mx));
-    // The reference point only moves when the maximum exceeds it by more than 2^8 (p stays <= 256,
-    // same relative precision in fp16), so that after the first tiles no block rescales O; a fully
-    // masked row keeps its reference point.
-    const float cand = fmaxf(mx * p.scale_log2, -1.0e30f);
-    const float m_new = cand > m + 8.0f ? cand : m;
-    const float alpha = fast_exp2(m - m_new);
-    m = m_new;
-    lsum *= alpha;
-    if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {  // wave-uniform: skip when no maximum moved
-#pragma unroll
-      for (int db = 0; db < DB; ++db) o[db] *= alpha;
-    }
-    half8_t pf;
-#pragma unroll
-    for (int tb = 0; tb < 2; ++tb) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float pj = fast_exp2(fmaf(s[tb][j], p.scale_log2, -m_new));  // masked: exp2(-huge) = 0
-        lsum += pj;
-        pf[tb * 4 + j] = static_cast<half_t>(pj);
-      }
-    }
-    // ---- O^T += V^T P^T: the value is the first DV features of the same rows ---------------------
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const half_t* vb = T + (db >> 2) * BLK + v_lane_off + (((db & 3) * 2 + v_piece) ^ v_swz) * 8;
-      const half4_t lo = lds_read_tr16(vb);
-      const half4_t hi = lds_read_tr16(vb + 16 * 64);
-      half8_t a;
-      a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
-      a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pf, o[db], 0, 0, 0);
-    }
+    half8_t pf_unused[2];
+    pv(lds_base + ((n_tiles - 1) % NSTAGE) * (STAGE * 2), pf_prev, std::false_type{}, s, 0, pf_unused);
   }
 
-  // the row sums are per lane group: add them up; m is already common
-  lsum = sum_xor32(sum_xor16(lsum));
+  // the row sums are per half of the wave: add them up; m is already common
+  lsum = sum_xor32(lsum);
+  acc_settle();  // the last PV product's results, before the vector ALU reads them
   if (row_valid) {
   const int64_t grow = static_cast<int64_t>(q_start + my_pos) * h_q + my_head;  // global row
   if (nchunks == 1) {
     const float denom = lsum + fast_exp2(kNegInit - m);
     const float inv = 1.0f / denom;
-    half_t* orow = p.output + grow * DV + 4 * g4;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
+    half_t* orow = p.output + grow * DV + half * 4;
+    static_for<DB * 4>([&](auto qc) {
+      constexpr int q4 = decltype(qc)::value;  // registers 4*q4 .. 4*q4+3: block q4/4, feature group q4%4
       half4_t out4;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) out4[e] = static_cast<half_t>(o[db][e] * inv);
-      *reinterpret_cast<half4_t*>(orow + db * 16) = out4;
-    }
-    if (g4 == 0) p.lse[grow] = m + fast_log2(denom);
+      out4[0] = static_cast<half_t>(acc_read<q4 * 4 + 0>() * inv);
+      out4[1] = static_cast<half_t>(acc_read<q4 * 4 + 1>() * inv);
+      out4[2] = static_cast<half_t>(acc_read<q4 * 4 + 2>() * inv);
+      out4[3] = static_cast<half_t>(acc_read<q4 * 4 + 3>() * inv);
+      *reinterpret_cast<half4_t*>(orow + (q4 / 4) * 32 + (q4 % 4) * 8) = out4;
+    });
+    if (half == 0) p.lse[grow] = m + fast_log2(denom);
   } else {
     // only one-token sequences are split: the row is the head
     const int64_t prow_idx = static_cast<int64_t>(cslot) * h_q + my_head;
-    float* prow = p.part_o + prow_idx * DV + 4 * g4;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) *reinterpret_cast<float4_t*>(prow + db * 16) = o[db];
-    if (g4 == 0) {
+    float* prow = p.part_o + prow_idx * DV + half * 4;
+    static_for<DB * 4>([&](auto qc) {
+      constexpr int q4 = decltype(qc)::value;
+      const float4_t v4 = {acc_read<q4 * 4 + 0>(), acc_read<q4 * 4 + 1>(), acc_read<q4 * 4 + 2>(), acc_read<q4 * 4 + 3>()};
+      *reinterpret_cast<float4_t*>(prow + (q4 / 4) * 32 + (q4 % 4) * 8) = v4;
+    });
+    if (half == 0) {
       p.part_ml[prow_idx * 2 + 0] = m;
       p.part_ml[prow_idx * 2 + 1] = lsum;
     }
