@@ -48,6 +48,7 @@ struct MlaParams {
   int batch_size;
   int h_q;
   int page_size;
+  int page_shift;    // log2(page_size) when it is a power of two, else -1
   int causal;
   int split;         // 1: decode-shaped call, the KV of a sequence is cut into chunks (see mla_chunk_slot_begin)
   int chunk_tokens;  // target tokens per chunk
@@ -99,6 +100,17 @@ template <int R>
 __device__ __forceinline__ void acc_mfma_32x32x16(half8_t a, half8_t b) {  // a[R:R+15] += a * b
   asm volatile("v_mfma_f32_32x32x16_f16 a[%2:%3], %0, %1, a[%2:%3]" : : "v"(a), "v"(b), "n"(R), "n"(R + 15));
 }
+// The same with an order token: `tok` is an operand the instruction does not touch.  Vector work that
+// is made to depend on it (pin_after) cannot be scheduled before this matrix instruction, and a
+// matrix instruction whose token depends on that work's result cannot be scheduled before the work:
+// program order then alternates matrix and vector instructions, which a single wave needs in order
+// to use both pipes at once (it issues in order).
+template <int R>
+__device__ __forceinline__ void acc_mfma_32x32x16(half8_t a, half8_t b, float& tok) {
+  asm volatile("v_mfma_f32_32x32x16_f16 a[%3:%4], %1, %2, a[%3:%4]" : "+v"(tok) : "v"(a), "v"(b), "n"(R), "n"(R + 15));
+}
+__device__ __forceinline__ void pin_after(float& x, float on) { asm("" : "+v"(x) : "v"(on)); }  // no instruction
+
 template <int R>
 __device__ __forceinline__ void acc_zero() {
   asm volatile("v_accvgpr_write_b32 a[%0], 0" : : "n"(R));
@@ -128,7 +140,10 @@ __device__ __forceinline__ void static_for(F&& f) {  // f(integral_constant<int,
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-template <int DQK, int DV>
+// POW2: the page size is a power of two (p.page_shift), so that a token's page and slot are a shift
+// and a mask; the general form divides, per copy instruction, and costs about as much again as the
+// matrix work of a tile.
+template <int DQK, int DV, bool POW2>
 __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams p) {
   constexpr int BN = MLA_BN;
   static_assert(BN == 32 && MLA_BM == MLA_WAVES * 32 && DQK % 64 == 0 && DV % 64 == 0 && DV <= DQK, "tile shape");
@@ -253,7 +268,7 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
     const int w = tile - tile_lo;
     if ((w & 15) == 0) {
       const int t = min((tile + (lane >> 2)) * BN + (lane & 3) * 8, last_tok);
-      page_ids = p.page_values[pbeg + t / ps];
+      page_ids = p.page_values[pbeg + (POW2 ? t >> p.page_shift : t / ps)];
     }
     const int kv0 = tile * BN;
     const uint32_t stage = lds_base + (w % NSTAGE) * (STAGE * 2);
@@ -267,7 +282,7 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
       const int row = rg * 8 + (lane >> 3);
       const int piece = (lane & 7) ^ mla_swizzle(row);
       const uint32_t t = min(kv0 + row, last_tok);
-      const uint32_t off = (t % ps) * (DQK * 2) + (blk * 64 + piece * 8) * 2;
+      const uint32_t off = (POW2 ? t & (ps - 1) : t % ps) * (DQK * 2) + (blk * 64 + piece * 8) * 2;
       copy16_to_lds(base, off, stage + (blk * BLK + rg * 8 * 64) * 2);
     }
   };
@@ -292,115 +307,125 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   const int v_row = half * 4 + (li >> 2);
   const uint32_t v_rel = v_row * 128 + (li & 1) * 8 + (((gg * 2 + ((li & 3) >> 1)) ^ mla_swizzle(v_row)) << 4);
 
-  // Both products read their A-fragments from LDS in groups, one group ahead of the matrix
-  // instructions that use them; scheduling fences between the groups keep the compiler from
-  // hoisting all reads of a product (which would not fit the register file).
-  constexpr int KG = 4;              // k-steps per group of the score product
-  constexpr int NKG = KS / KG;
-  constexpr int VG = 2;              // feature blocks per group of the PV product (2 fragments each)
-  constexpr int NVG = DB / VG;
-  static_assert(KS % KG == 0 && DB % VG == 0 && NVG >= 6, "fragment groups");
-  auto read_k_group = [&](uint32_t k_at, int g, half8_t (&a)[KG]) {  // k_at: stage base + k_rel
-#pragma unroll
-    for (int i = 0; i < KG; ++i) {
-      const int ks = g * KG + i;
-      a[i] = lds_read_b128_at((k_at ^ (((ks & 3) * 2) << 4)) + (ks >> 2) * (BLK * 2));
-    }
+  // Both products read their A-fragments from LDS through a ring of RING fragments: the read of
+  // fragment t + RING - 1 is issued right after matrix instruction t, i.e. RING - 1 instructions
+  // (of 32 cycles each) ahead of its use, which is what the LDS takes under the load of four waves.
+  // A scheduling fence after every step keeps the compiler from hoisting all reads of a product
+  // (which would not fit the register file).
+  constexpr int RING = 8;
+  auto read_k_frag = [&](uint32_t k_at, int ks) -> half8_t {  // k_at: stage base + k_rel
+    return lds_read_b128_at((k_at ^ (((ks & 3) * 2) << 4)) + (ks >> 2) * (BLK * 2));
   };
-  auto read_v_group = [&](uint32_t v_at, int g, half8_t (&a)[VG][2]) {  // v_at: stage base + v_rel
+  auto read_v_frag = [&](uint32_t v_at, int t) -> half8_t {  // v_at: stage base + v_rel; t = 2*db + kk
+    const int db = t >> 1, kk = t & 1;
+    half8_t a;
 #pragma unroll
-    for (int i = 0; i < VG; ++i) {
-      const int db = g * VG + i;
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const int c = ((db & 1) << 2) | (kk * 2 + e);
-          const half4_t part = lds_read_tr16_at((v_at ^ (c << 4)) + (db >> 1) * (BLK * 2) + (kk * 16 + e * 8) * 128);
-          a[i][kk][e * 4 + 0] = part[0]; a[i][kk][e * 4 + 1] = part[1];
-          a[i][kk][e * 4 + 2] = part[2]; a[i][kk][e * 4 + 3] = part[3];
-        }
-      }
+    for (int e = 0; e < 2; ++e) {
+      const int c = ((db & 1) << 2) | (kk * 2 + e);
+      const half4_t part = lds_read_tr16_at((v_at ^ (c << 4)) + (db >> 1) * (BLK * 2) + (kk * 16 + e * 8) * 128);
+      a[e * 4 + 0] = part[0]; a[e * 4 + 1] = part[1];
+      a[e * 4 + 2] = part[2]; a[e * 4 + 3] = part[3];
     }
+    return a;
   };
   // S^T = KV Q^T over all DQK features for the 32 tokens of a tile
   auto qk = [&](uint32_t stage_at) -> float16_t {
     float16_t acc;
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[j] = 0.f;
-    half8_t a[2][KG];
+    half8_t a[RING];
     const uint32_t k_at = stage_at + k_rel;
-    read_k_group(k_at, 0, a[0]);
 #pragma unroll
-    for (int g = 0; g < NKG; ++g) {
-      if (g + 1 < NKG) read_k_group(k_at, g + 1, a[(g + 1) & 1]);
+    for (int t = 0; t < RING - 1; ++t) a[t] = read_k_frag(k_at, t);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < KG; ++i) {
-        // Written as assembly to put S into ordinary vector registers: with a whole register file
-        // per wave the compiler selects the form of the matrix instructions whose results live in
-        // accumulation registers, and O fills all 256 of those.
-        if (g == NKG - 1 && i == KG - 1) {
-          // the compiler does not know this is a matrix instruction: the wait states it would put
-          // between the last one and the first vector instruction that reads S are spelled out
-          asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7"
-              : "+v"(acc) : "v"(a[g & 1][i]), "v"(qf[g * KG + i]));
-        } else {
-          asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a[g & 1][i]), "v"(qf[g * KG + i]));
-        }
+    for (int t = 0; t < KS; ++t) {
+      // Written as assembly to put S into ordinary vector registers: with a whole register file per
+      // wave the compiler selects the form of the matrix instructions whose results live in
+      // accumulation registers, and O fills all 256 of those.
+      if (t == KS - 1) {
+        // the compiler does not know this is a matrix instruction: the wait states it would put
+        // between the last one and the first vector instruction that reads S are spelled out
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(acc) : "v"(a[t % RING]), "v"(qf[t]));
+      } else {
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a[t % RING]), "v"(qf[t]));
       }
+      if (t + RING - 1 < KS) a[(t + RING - 1) % RING] = read_k_frag(k_at, t + RING - 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     return acc;
   };
-  // Online softmax of a tile's scores, cut into steps that are spread over the groups of the PV
-  // product running beside it.  s[j]: token kv0 + (j/4)*8 + half*4 + j%4, query col.  The reference
-  // point only moves when the maximum exceeds it by more than 2^8 (p stays <= 256, same relative
-  // precision in fp16), so that after the first tiles no block rescales O; a fully masked row keeps
-  // its reference point.  Step 0: mask and row maximum; 1: new reference point and the factor for
-  // the old state; 2..5: four probabilities each, as the B-operand of the next PV product.
+  // Online softmax of a tile's scores, cut into slots that sit between the matrix instructions of
+  // the PV product running beside it (vec_slot<t> follows instruction t).  s[j]: token kv0 + (j/4)*8 +
+  // half*4 + j%4, query col.  The reference point only moves when the maximum exceeds it by more
+  // than 2^8 (p stays <= 256, same relative precision in fp16), so that after the first tiles no
+  // block rescales O; a fully masked row keeps its reference point.  Slots 0, 1: row maximum of the
+  // lane's 16 scores; 2: the other half's maximum, new reference point, factor for the old state;
+  // 3, 5, .., 17: two probabilities each, as the B-operand of the next PV product.
   float alpha = 1.0f, row_mx = 0.f;
-  auto softmax_step = [&](int step, float16_t& s, int kv0, half8_t (&pf)[2]) {
-    if (step == 0) {
-      if (kv0 + BN > wave_limit_min) {  // wave-uniform: the causal diagonal or the end of the sequence
-        asm volatile("" ::: "memory");
-        const int rel = my_limit - kv0 - half * 4;
+  auto mask_scores = [&](float16_t& s, int kv0) {
+    if (kv0 + BN > wave_limit_min) {  // wave-uniform: the causal diagonal or the end of the sequence
+      asm volatile("" ::: "memory");
+      const int rel = my_limit - kv0 - half * 4;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) s[j] = ((j >> 2) * 8 + (j & 3)) < rel ? s[j] : -3.0e38f;
+      for (int j = 0; j < 16; ++j) s[j] = ((j >> 2) * 8 + (j & 3)) < rel ? s[j] : -3.0e38f;
+    }
+  };
+  auto vec_slot = [&](auto tc, float16_t& s, half8_t (&pf)[2], float& tok) {
+    constexpr int t = decltype(tc)::value;
+    if constexpr (t == 0 || t == 1) {
+      float mx = t == 0 ? -3.0e38f : row_mx;
+#pragma unroll
+      for (int j = t * 8; j < t * 8 + 8; ++j) {
+        float x = s[j];
+        pin_after(x, tok);
+        mx = fmaxf(mx, x);
       }
-      float mx = -3.0e38f;
-#pragma unroll
-      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[j]);
-      row_mx = max_xor32(mx);
-    } else if (step == 1) {
+      row_mx = mx;
+      pin_after(tok, row_mx);
+    } else if constexpr (t == 2) {
+      pin_after(row_mx, tok);
+      row_mx = max_xor32(row_mx);
       const float cand = fmaxf(row_mx * p.scale_log2, -1.0e30f);
       const float m_new = cand > m + 8.0f ? cand : m;
       alpha = fast_exp2(m - m_new);
       m = m_new;
       lsum *= alpha;
-    } else if (step < 6) {
-#pragma unroll
-      for (int j = (step - 2) * 4; j < (step - 1) * 4; ++j) {
-        const float pj = fast_exp2(fmaf(s[j], p.scale_log2, -m));  // masked: exp2(-huge) = 0
-        lsum += pj;
-        pf[j >> 3][j & 7] = static_cast<half_t>(pj);
-      }
+      pin_after(tok, lsum);
+    } else if constexpr (t >= 3 && t <= 17 && (t & 1) == 1) {
+      constexpr int j = t - 3;  // elements j, j + 1
+      float x0 = s[j], x1 = s[j + 1];
+      pin_after(x0, tok);
+      pin_after(x1, tok);
+      const float p0 = fast_exp2(fmaf(x0, p.scale_log2, -m));  // masked: exp2(-huge) = 0
+      const float p1 = fast_exp2(fmaf(x1, p.scale_log2, -m));
+      lsum += p0;
+      lsum += p1;
+      pf[j >> 3][j & 7] = static_cast<half_t>(p0);
+      pf[j >> 3][(j & 7) + 1] = static_cast<half_t>(p1);
+      pin_after(tok, lsum);
     }
+  };
+  auto softmax_alone = [&](float16_t& s, int kv0, half8_t (&pf)[2]) {
+    float tok = 0.f;
+    mask_scores(s, kv0);
+    static_for<18>([&](auto tc) { vec_slot(tc, s, pf, tok); });
   };
   // O^T += V^T P^T (the value is the first DV features of the same rows), optionally with the
   // softmax of the next tile's scores on the vector ALU beside it
   auto pv = [&](uint32_t stage_at, const half8_t (&pf_in)[2], auto with_softmax, float16_t& s, int kv0, half8_t (&pf_out)[2]) {
-    half8_t a[2][VG][2];
+    half8_t a[RING];
     const uint32_t v_at = stage_at + v_rel;
-    read_v_group(v_at, 0, a[0]);
-    static_for<NVG>([&](auto gc) {
-      constexpr int g = decltype(gc)::value;
-      if (g + 1 < NVG) read_v_group(v_at, g + 1, a[(g + 1) & 1]);
-      static_for<VG>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        acc_mfma_32x32x16<(g * VG + i) * 16>(a[g & 1][i][0], pf_in[0]);
-        acc_mfma_32x32x16<(g * VG + i) * 16>(a[g & 1][i][1], pf_in[1]);
-      });
-      if (decltype(with_softmax)::value) softmax_step(g, s, kv0, pf_out);
+    float tok = 0.f;
+    if (decltype(with_softmax)::value) mask_scores(s, kv0);
+#pragma unroll
+    for (int t = 0; t < RING - 1; ++t) a[t] = read_v_frag(v_at, t);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<DB * 2>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;  // instruction t: feature block t/2, tokens (t%2)*16 .. +15
+      acc_mfma_32x32x16<(t / 2) * 16>(a[t % RING], pf_in[t & 1], tok);
+      if constexpr (t + RING - 1 < DB * 2) a[(t + RING - 1) % RING] = read_v_frag(v_at, t + RING - 1);
+      if constexpr (decltype(with_softmax)::value) vec_slot(tc, s, pf_out, tok);
       __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -439,8 +464,7 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
     float16_t s;
     tile_ready(0);
     s = qk(lds_base);
-#pragma unroll
-    for (int step = 0; step < 6; ++step) softmax_step(step, s, tile_lo * BN, pf_prev);  // nothing accumulated yet: no rescale
+    softmax_alone(s, tile_lo * BN, pf_prev);  // nothing accumulated yet: no rescale
     for (int w = 1; w < n_tiles; ++w) {
       tile_ready(w);
       half8_t pf[2];
@@ -632,14 +656,24 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
   constexpr size_t lds_bytes = static_cast<size_t>(MLA_STAGES) * MLA_BN * DQK * sizeof(half_t);
   static bool attr_set = false;
   if (!attr_set) {
-    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_paged_kernel<DQK, DV>),
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_paged_kernel<DQK, DV, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_paged_kernel<DQK, DV, false>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     attr_set = true;
   }
   hipStream_t s = as_stream(stream);
   KV_CHECK(grid < (int64_t{1} << 31)) << "batch_prefill_paged_kv_mla: too many work items";
-  hipLaunchKernelGGL((mla_paged_kernel<DQK, DV>), dim3(static_cast<unsigned>(grid)), dim3(MLA_WAVES * 64), lds_bytes,
-                     s, p);
+  p.page_shift = -1;
+  if ((page_size & (page_size - 1)) == 0) {
+    p.page_shift = 0;
+    while ((1 << p.page_shift) < page_size) ++p.page_shift;
+    hipLaunchKernelGGL((mla_paged_kernel<DQK, DV, true>), dim3(static_cast<unsigned>(grid)), dim3(MLA_WAVES * 64),
+                       lds_bytes, s, p);
+  } else {
+    hipLaunchKernelGGL((mla_paged_kernel<DQK, DV, false>), dim3(static_cast<unsigned>(grid)), dim3(MLA_WAVES * 64),
+                       lds_bytes, s, p);
+  }
   KV_LAUNCH_CHECK();
   if (p.split) {
     hipLaunchKernelGGL(mla_merge_kernel<DV>, dim3(static_cast<unsigned>(total_q), h_q), dim3(DV / 4), 0, s, p);
