@@ -264,12 +264,19 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds_tiles));
   const int last_tok = kv_len - 1;
   int page_ids = 0;
-  auto issue_tile = [&](int tile) {
-    const int w = tile - tile_lo;
-    if ((w & 15) == 0) {
+  // Per-lane part of a copy's source offset for rows that need no clamping: row lane/8 of the
+  // 8-row group rg, piece (lane%8) ^ swizzle(rg*8 + lane/8) = this value ^ (rg << 4).
+  const uint32_t copy_lane_off = (lane >> 3) * (DQK * 2) + (((lane & 7) ^ ((((lane >> 3) >> 1) & 1) << 2)) << 4);
+  // General form of a tile's copies: a page id per 8-row group, rows past the end clamped.
+  auto load_page_ids = [&](int tile) {
+    if (((tile - tile_lo) & 15) == 0) {
       const int t = min((tile + (lane >> 2)) * BN + (lane & 3) * 8, last_tok);
       page_ids = p.page_values[pbeg + (POW2 ? t >> p.page_shift : t / ps)];
     }
+  };
+  auto issue_tile = [&](int tile) {
+    load_page_ids(tile);
+    const int w = tile - tile_lo;
     const int kv0 = tile * BN;
     const uint32_t stage = lds_base + (w % NSTAGE) * (STAGE * 2);
 #pragma unroll
@@ -285,6 +292,31 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
       const uint32_t off = (POW2 ? t & (ps - 1) : t % ps) * (DQK * 2) + (blk * 64 + piece * 8) * 2;
       copy16_to_lds(base, off, stage + (blk * BLK + rg * 8 * 64) * 2);
     }
+  };
+  // Fast form, for a tile that lies inside one page (pages of 32 tokens or more) and inside the
+  // sequence: one scalar base per tile, and a copy is two vector and a few scalar instructions,
+  // which fit beside one matrix instruction of the score product.
+  const bool tile_in_page = POW2 && ps >= BN;
+  const half_t* tile_base = p.pages;
+  uint32_t tile_stage = lds_base;
+  uint32_t tile_lane_off = 0;
+  auto fast_copy_prepare = [&](int tile) {
+    // a copy of the per-lane offset that the compiler cannot see through: the nine offsets derived
+    // from it are then computed where they are used instead of being kept in nine registers
+    tile_lane_off = copy_lane_off;
+    asm volatile("" : "+v"(tile_lane_off));
+    load_page_ids(tile);
+    const int w = tile - tile_lo;
+    const int page = __builtin_amdgcn_readlane(page_ids, (w & 15) * 4);
+    tile_base = p.pages + (static_cast<int64_t>(page) * ps + ((tile * BN) & (ps - 1))) * DQK;
+    tile_stage = lds_base + (w % NSTAGE) * (STAGE * 2);
+  };
+  auto fast_copy_step = [&](auto jc) {  // copy instruction j (of COPIES) of this wave
+    constexpr int j = decltype(jc)::value;
+    const int n = copy_first + j;
+    const int blk = n >> 2;
+    const int rg = n & 3;
+    copy16_to_lds(tile_base, (tile_lane_off ^ (rg << 4)) + (rg * 8 * DQK + blk * 64) * 2, tile_stage + (blk * BLK + rg * 8 * 64) * 2);
   };
 
   // ---- per-lane fragment addressing (LDS byte addresses) -------------------------------------------
@@ -329,7 +361,7 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
     return a;
   };
   // S^T = KV Q^T over all DQK features for the 32 tokens of a tile
-  auto qk = [&](uint32_t stage_at) -> float16_t {
+  auto qk = [&](uint32_t stage_at, auto&& beside) -> float16_t {  // beside(t): scalar / vector work placed after instruction t
     float16_t acc;
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[j] = 0.f;
@@ -338,21 +370,22 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
 #pragma unroll
     for (int t = 0; t < RING - 1; ++t) a[t] = read_k_frag(k_at, t);
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int t = 0; t < KS; ++t) {
+    static_for<KS>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
       // Written as assembly to put S into ordinary vector registers: with a whole register file per
       // wave the compiler selects the form of the matrix instructions whose results live in
       // accumulation registers, and O fills all 256 of those.
-      if (t == KS - 1) {
+      if constexpr (t == KS - 1) {
         // the compiler does not know this is a matrix instruction: the wait states it would put
         // between the last one and the first vector instruction that reads S are spelled out
         asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(acc) : "v"(a[t % RING]), "v"(qf[t]));
       } else {
         asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a[t % RING]), "v"(qf[t]));
       }
-      if (t + RING - 1 < KS) a[(t + RING - 1) % RING] = read_k_frag(k_at, t + RING - 1);
+      if constexpr (t + RING - 1 < KS) a[(t + RING - 1) % RING] = read_k_frag(k_at, t + RING - 1);
+      beside(tc);
       __builtin_amdgcn_sched_barrier(0);
-    }
+    });
     return acc;
   };
   // Online softmax of a tile's scores, cut into slots that sit between the matrix instructions of
@@ -375,12 +408,9 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
     constexpr int t = decltype(tc)::value;
     if constexpr (t == 0 || t == 1) {
       float mx = t == 0 ? -3.0e38f : row_mx;
+      pin_after(mx, tok);  // everything below hangs on it
 #pragma unroll
-      for (int j = t * 8; j < t * 8 + 8; ++j) {
-        float x = s[j];
-        pin_after(x, tok);
-        mx = fmaxf(mx, x);
-      }
+      for (int j = t * 8; j < t * 8 + 8; ++j) mx = fmaxf(mx, s[j]);
       row_mx = mx;
       pin_after(tok, row_mx);
     } else if constexpr (t == 2) {
@@ -394,11 +424,10 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
       pin_after(tok, lsum);
     } else if constexpr (t >= 3 && t <= 17 && (t & 1) == 1) {
       constexpr int j = t - 3;  // elements j, j + 1
-      float x0 = s[j], x1 = s[j + 1];
-      pin_after(x0, tok);
-      pin_after(x1, tok);
-      const float p0 = fast_exp2(fmaf(x0, p.scale_log2, -m));  // masked: exp2(-huge) = 0
-      const float p1 = fast_exp2(fmaf(x1, p.scale_log2, -m));
+      float mm = m;
+      pin_after(mm, tok);
+      const float p0 = fast_exp2(fmaf(s[j], p.scale_log2, -mm));  // masked: exp2(-huge) = 0
+      const float p1 = fast_exp2(fmaf(s[j + 1], p.scale_log2, -mm));
       lsum += p0;
       lsum += p1;
       pf[j >> 3][j & 7] = static_cast<half_t>(p0);
@@ -457,18 +486,37 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
       wait_vmcnt<0>();
     }
     __syncthreads();  // everyone's part of tile w has landed; everyone is done with the stage of tile w-2
-    if (w + 2 < n_tiles) issue_tile(tile_lo + w + 2);
+  };
+  // Where the fast form applies, the copies of tile w+2 go out one by one between the matrix
+  // instructions of S(w), which leave the scalar and vector units idle; otherwise before them.
+  auto qk_and_copies = [&](int w) -> float16_t {
+    const uint32_t stage_at = lds_base + (w % NSTAGE) * (STAGE * 2);
+    if (w + 2 < n_tiles) {
+      const int tile = tile_lo + w + 2;
+      if (tile_in_page && (tile + 1) * BN <= kv_len) {  // wave-uniform
+        return qk(stage_at, [&](auto tc) {
+          constexpr int t = decltype(tc)::value;
+          if constexpr (t == 0) {
+            fast_copy_prepare(tile);
+          } else if constexpr (t % 3 == 0 && t / 3 <= COPIES) {
+            fast_copy_step(std::integral_constant<int, t / 3 - 1>{});
+          }
+        });
+      }
+      issue_tile(tile);
+    }
+    return qk(stage_at, [&](auto) {});
   };
   if (n_tiles > 0) {
     half8_t pf_prev[2];
     float16_t s;
     tile_ready(0);
-    s = qk(lds_base);
+    s = qk_and_copies(0);
     softmax_alone(s, tile_lo * BN, pf_prev);  // nothing accumulated yet: no rescale
     for (int w = 1; w < n_tiles; ++w) {
       tile_ready(w);
       half8_t pf[2];
-      s = qk(lds_base + (w % NSTAGE) * (STAGE * 2));
+      s = qk_and_copies(w);
       pv(lds_base + ((w - 1) % NSTAGE) * (STAGE * 2), pf_prev, std::true_type{}, s, (tile_lo + w) * BN, pf);
       rescale();
       pf_prev[0] = pf[0];
