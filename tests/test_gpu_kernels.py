@@ -332,6 +332,33 @@ def test_ragged_prefill_longer_chunk():
     assert_close(gl, el, atol=2e-3, rtol=1e-4, what="ragged lse")
 
 
+@pytest.mark.parametrize("causal", [1, 0])
+def test_ragged_prefill_scores_that_keep_growing(causal):
+    """The running softmax moves its reference point (and rescales O) only when a score exceeds it by
+    more than 2^8; random inputs do that in the first tile only.  Here the score grows by ~10 in the
+    exponent per 32 keys, so the rescale runs in every tile."""
+    rng = np.random.default_rng(19)
+    hq, hkv, d = 8, 2, 128
+    lens = [300, 64, 130]
+    n = sum(lens)
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    q[:, :, :16] = 1
+    for b in range(len(lens)):
+        k[indptr[b]:indptr[b + 1], :, :16] = (0.153 * np.arange(lens[b], dtype=np.float32))[:, None, None].astype(F16)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    zq, zb = np.zeros(n, np.int32), np.zeros(len(lens), np.int32)
+    ok.prefill_ragged(q, indptr, k, v, indptr, zq, zb, eo, el, causal, 0, 1.0, 1e4, d ** -0.5)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_ragged_kv(dev(q), i32(indptr), dev(k), dev(v), i32(indptr), i32(zq), i32(zb), go, gl, causal, 0,
+                              1.0, 1e4, d ** -0.5)
+    assert_close(host(go), eo, what="ragged growing scores out")
+    assert_close(host(gl), el, atol=5e-3, rtol=1e-4, what="ragged growing scores lse")
+
+
 def _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages):
     pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, kv_lens, npages, hkv, 16, d)
     n = sum(q_lens)

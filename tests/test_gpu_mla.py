@@ -24,7 +24,9 @@ H, D_LAT, D_ROPE, D_NOPE, D_V = 128, 512, 64, 128, 128
 D_QK = D_LAT + D_ROPE
 
 
-def _latent_pool(rng, kv_lens, ps, npages):
+def _latent_pool(rng, kv_lens, ps, npages, ramp=0.0):
+    """ramp > 0: the rope part of token t is ramp * t in every feature, so that against a query
+    whose rope part is all ones the scores grow along the sequence without bound."""
     pages = np.zeros((npages, ps, D_QK), F16)
     order = rng.permutation(npages)
     indptr, values, last, rows = [0], [], [], []
@@ -34,6 +36,8 @@ def _latent_pool(rng, kv_lens, ps, npages):
         ids = order[cursor:cursor + npg]
         cursor += npg
         lat = (rng.standard_normal((n, D_QK)) * 0.5).astype(F16)
+        if ramp:
+            lat[:, D_LAT:] = (ramp * np.arange(n, dtype=np.float32))[:, None].astype(F16)
         for t in range(n):
             pages[ids[t // ps], t % ps] = lat[t]
         values.extend(int(x) for x in ids)
@@ -43,11 +47,13 @@ def _latent_pool(rng, kv_lens, ps, npages):
     return pages, np.array(indptr, np.int32), np.array(values, np.int32), np.array(last, np.int32), rows
 
 
-def _mla_both(rng, kv_lens, q_lens, ps, npages, causal=0, heads=H):
-    pages, pindptr, pvalues, last, _ = _latent_pool(rng, kv_lens, ps, npages)
+def _mla_both(rng, kv_lens, q_lens, ps, npages, causal=0, heads=H, ramp=0.0):
+    pages, pindptr, pvalues, last, _ = _latent_pool(rng, kv_lens, ps, npages, ramp)
     n = sum(q_lens)
     qindptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
     q = (rng.standard_normal((n, heads, D_QK)) * 0.5).astype(F16)
+    if ramp:
+        q[:, :, D_LAT:] = 1
     eo, el = np.zeros((n, heads, D_LAT), F16), np.zeros((n, heads), np.float32)
     sm = (D_NOPE + D_ROPE) ** -0.5
     ok.prefill_paged_mla(q, qindptr, pages, pindptr, pvalues, last, eo, el, causal, sm, d_latent=D_LAT)
@@ -96,6 +102,34 @@ def test_mla_prefill_shaped(causal):
     go, gl, eo, el = _mla_both(rng, kv_lens, q_lens, 64, npages=16, causal=causal, heads=16)
     assert_close(go, eo, what="mla prefill out")
     assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla prefill lse")
+
+
+@pytest.mark.parametrize("causal", [0, 1])
+def test_mla_scores_that_keep_growing_move_the_reference_point(causal):
+    """The running softmax only moves its reference point (and rescales O, which the kernel does on
+    the accumulation registers from assembly) when a score exceeds it by more than 2^8.  Random
+    inputs do that in the first tile only; here the score grows by ~10 in the exponent per 32-token
+    tile, so every tile rescales, in prefill- and in decode-shaped (split-KV) calls."""
+    rng = np.random.default_rng(35)
+    kv_lens, q_lens = [330, 96, 64, 200], [40, 1, 3, 200]
+    go, gl, eo, el = _mla_both(rng, kv_lens, q_lens, 64, npages=16, causal=causal, heads=16, ramp=0.047)
+    assert_close(go, eo, what="mla growing scores out")
+    assert_close(gl, el, atol=5e-3, rtol=1e-4, what="mla growing scores lse")
+    kv_lens = [700, 1300, 129]
+    go, gl, eo, el = _mla_both(rng, kv_lens, [1, 1, 1], 64, npages=40, ramp=0.02)
+    assert_close(go, eo, what="mla growing scores decode out")
+    assert_close(gl, el, atol=5e-3, rtol=1e-4, what="mla growing scores decode lse")
+
+
+def test_mla_page_size_that_is_not_a_power_of_two():
+    rng = np.random.default_rng(36)
+    kv_lens, q_lens = [300, 47, 0, 100], [33, 5, 2, 100]
+    go, gl, eo, el = _mla_both(rng, kv_lens, q_lens, 24, npages=24, causal=1, heads=16)
+    assert_close(go, eo, what="mla page 24 out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla page 24 lse")
+    go, gl, eo, el = _mla_both(rng, [500, 90], [1, 1], 40, npages=20)
+    assert_close(go, eo, what="mla page 40 decode out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla page 40 decode lse")
 
 
 def test_mla_cache_flow_matches_the_definition():
