@@ -94,9 +94,10 @@ def time_region(torch, fn, iters):
     return start.elapsed_time(stop) / iters
 
 
-def calibrate(num_bytes=2 << 30, iters=10):
-    """Plain streaming read and copy of `num_bytes`: what the memory system of this box delivers
-    to the simplest possible kernel.  Prints one JSON line."""
+def calibrate(num_bytes=2 << 30, iters=10, quiet=False):
+    """Plain streaming read and copy of `num_bytes`, and a loop of nothing but fp16 MFMA: what the
+    memory system and the matrix cores of this box deliver to the simplest possible kernels.
+    Prints one JSON line unless `quiet`."""
     import torch
 
     from tvm_amd import kernels as K
@@ -111,11 +112,22 @@ def calibrate(num_bytes=2 << 30, iters=10):
     K.stream_read_nt(src, sink)
     ms_read_nt = time_region(torch, lambda i: K.stream_read_nt(src, sink), iters)
     ms_copy = time_region(torch, lambda i: K.stream_copy(src, dst), iters)
-    out = {"calibration": "plain streaming kernels", "bytes": num_bytes,
+    # matrix cores: a loop of nothing but fp16 MFMA, one round of workgroups per wave slot
+    wgs, mfma_iters = 256 * 2, 4096
+    sums = torch.empty((wgs, 256), dtype=torch.float32, device=dev)
+    mfma = {}
+    for name, ops in (("constant", torch.full((256, 16), 0.5, dtype=torch.float16, device=dev)),
+                      ("random", torch.randn((256, 16), device=dev).to(torch.float16))):
+        K.mfma_loop(ops, sums, 16)
+        ms = time_region(torch, lambda i: K.mfma_loop(ops, sums, mfma_iters), 5)
+        mfma[name] = round(2.0 * 32 * 32 * 16 * 8 * mfma_iters * 4 * wgs / ms / 1e9, 1)
+    out = {"calibration": "plain streaming kernels and an MFMA-only loop", "bytes": num_bytes,
+           "mfma_f16_TFLOPs_constant_operands": mfma["constant"], "mfma_f16_TFLOPs_random_operands": mfma["random"],
            "read_GBps": round(num_bytes / ms_read / 1e6, 1), "read_ms": round(ms_read, 4),
            "read_nt_GBps": round(num_bytes / ms_read_nt / 1e6, 1), "read_nt_ms": round(ms_read_nt, 4),
            "copy_GBps_read_plus_write": round(2 * num_bytes / ms_copy / 1e6, 1), "copy_ms": round(ms_copy, 4)}
-    print(json.dumps(out))
+    if not quiet:
+        print(json.dumps(out))
     return out
 
 
@@ -288,7 +300,8 @@ def main():
                          "known-size dispatches for scaling rocprofv3 traffic counters)")
     args = ap.parse_args()
     if args.calibrate:
-        return calibrate()
+        calibrate()
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; the path shards per kv head without any exchange "
                  "step, and no multi-GPU figure is produced. Use --gpus 1.")
@@ -412,6 +425,18 @@ def main():
                              "tflops": round(tflops, 2), "ms": round(ms_prefill, 4),
                              "algorithmic_flops": pw["flops"],
                              "frac_of_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
+
+    # What the simplest kernels reach on this box, next to the datasheet peaks.  After the timed legs:
+    # the MFMA loop heats the chip and the clock of what follows drops.
+    cal = calibrate(num_bytes=1 << 30, iters=5, quiet=True)
+    result["calibration"] = {"hbm_read_GBps": cal["read_GBps"], "hbm_read_nontemporal_GBps": cal["read_nt_GBps"],
+                             "mfma_f16_TFLOPs_constant_operands": cal["mfma_f16_TFLOPs_constant_operands"],
+                             "mfma_f16_TFLOPs_random_operands": cal["mfma_f16_TFLOPs_random_operands"],
+                             "what": "1 GiB streaming read (plain / non-temporal loads); a loop of fp16 MFMA only"}
+    result["roofline"]["frac_of_calibrated_read"] = round(gbps_decode / cal["read_nt_GBps"], 4)
+    if "prefill" in result:
+        result["prefill"]["frac_of_calibrated_mfma_random_operands"] = round(
+            result["prefill"]["tflops"] / cal["mfma_f16_TFLOPs_random_operands"], 4)
 
     # ---- CPU baseline: the oracle's restatement of the reference's llvm decode kernel ---------
     if not args.no_cpu_baseline:

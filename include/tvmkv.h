@@ -267,6 +267,11 @@ int tvmkv_stream_read(const void* src, int64_t num_bytes, void* sink, void* stre
 /* the same read with non-temporal loads, the kind the decode kernel issues */
 int tvmkv_stream_read_nt(const void* src, int64_t num_bytes, void* sink, void* stream);
 int tvmkv_stream_copy(const void* src, void* dst, int64_t num_bytes, void* stream);
+/* Matrix-core calibration (no counterpart in the reference): `workgroups` workgroups of 4 waves run
+ * `iters` rounds of 8 v_mfma_f32_32x32x16_f16 each (4 accumulators, nothing else in the loop) on the
+ * A and B fragments read from `operands` (256 lanes x 16 halfs); `out` gets workgroups x 256
+ * floats.  2 * 32 * 32 * 16 * 8 * iters * 4 * workgroups flop per launch. */
+int tvmkv_mfma_loop(const void* operands, float* out, int32_t iters, int32_t workgroups, void* stream);
 
 /* ======================================================================================
  * (2) Cache object

@@ -291,6 +291,34 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restric
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
 
+// Matrix-core calibration: every wave runs `iters` rounds of 8 independent-enough
+// v_mfma_f32_32x32x16_f16 (4 accumulators) on operands it read once from `operands` (8 halfs per lane
+// for A and for B).  Nothing else is in the loop: this is what the matrix pipes of the box deliver,
+// and it depends on the operand values (the clock drops with random data).
+__global__ __launch_bounds__(256) void mfma_loop_kernel(const half_t* __restrict__ operands, float* __restrict__ out,
+                                                        int iters) {
+  const int tid = threadIdx.x;
+  const half8_t a = *reinterpret_cast<const half8_t*>(operands + tid * 16);
+  const half8_t b = *reinterpret_cast<const half8_t*>(operands + tid * 16 + 8);
+  float16_t acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+  }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[j & 3], 0, 0, 0);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sum += acc[j][i];
+  }
+  out[static_cast<int64_t>(blockIdx.x) * 256 + tid] = sum;
+}
+
 inline dim3 grid_for(int64_t threads, int block = 256) { return dim3(static_cast<unsigned>((threads + block - 1) / block)); }
 
 }  // namespace tvmkv
@@ -495,6 +523,15 @@ int tvmkv_stream_copy(const void* src, void* dst, int64_t num_bytes, void* strea
   if (num_bytes == 0) return TVMKV_OK;
   hipLaunchKernelGGL(stream_copy_kernel, dim3(256 * 16), dim3(256), 0, as_stream(stream),
                      static_cast<const uint4*>(src), static_cast<uint4*>(dst), num_bytes / 16);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
+
+int tvmkv_mfma_loop(const void* operands, float* out, int32_t iters, int32_t workgroups, void* stream) {
+  KV_API_BEGIN();
+  KV_CHECK(operands && out && iters >= 0 && workgroups > 0) << "mfma_loop: bad arguments";
+  hipLaunchKernelGGL(mfma_loop_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0, as_stream(stream),
+                     static_cast<const half_t*>(operands), out, iters);
   KV_LAUNCH_CHECK();
   KV_API_END();
 }

@@ -207,6 +207,13 @@ def compact_kv_copy(pages, copy_length_indptr, copy_src_dst_pos, batch_size):
                                       copy_src_dst_pos.shape[1], num_pages, hkv, ps, d, _stream()))
 
 
+def mfma_loop(operands, out, iters):
+    """Matrix-core calibration loop: operands (256, 16) fp16, out (workgroups, 256) fp32."""
+    _f16(operands)
+    assert operands.numel() == 256 * 16 and out.dtype == torch.float32 and out.shape[1] == 256
+    check(lib().tvmkv_mfma_loop(_p(operands), _p(out), int(iters), out.shape[0], _stream()))
+
+
 def stream_read_nt(src, sink):
     """stream_read with non-temporal loads."""
     check(lib().tvmkv_stream_read_nt(_p(src), src.numel() * src.element_size(), _p(sink), _stream()))
