@@ -609,3 +609,23 @@ def test_prefill_cached_and_new_in_one_pass(hq, hkv, d):
                                       i32(last), go, gl, d ** -0.5)
     assert_close(host(go), eo, what="one-pass chunked prefill out")
     assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="one-pass chunked prefill lse")
+
+
+def test_measurement_utilities():
+    """The calibration kernels of the benchmark: the copy copies, the reads leave their input alone,
+    and the MFMA loop adds up what its instruction count says (integers in fp32, so exactly)."""
+    src = torch.arange(1 << 16, dtype=torch.int32, device=DEV)
+    dst = torch.zeros_like(src)
+    sink = torch.zeros(4, dtype=torch.int32, device=DEV)
+    K.stream_copy(src, dst)
+    K.stream_read(src, sink)
+    K.stream_read_nt(src, sink)
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst) and torch.equal(src, torch.arange(1 << 16, dtype=torch.int32, device=DEV))
+    ops = torch.full((256, 16), 0.5, dtype=torch.float16, device=DEV)
+    out = torch.zeros((3, 256), dtype=torch.float32, device=DEV)
+    iters = 5
+    K.mfma_loop(ops, out, iters)
+    torch.cuda.synchronize()
+    # one instruction adds 16 * 0.5 * 0.5 = 4 to each of its 16 results per lane; 8 instructions a round
+    assert torch.all(out == 4.0 * 16 * 8 * iters)
