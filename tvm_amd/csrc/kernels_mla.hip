@@ -363,8 +363,6 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   // S^T = KV Q^T over all DQK features for the 32 tokens of a tile
   auto qk = [&](uint32_t stage_at, auto&& beside) -> float16_t {  // beside(t): scalar / vector work placed after instruction t
     float16_t acc;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
     half8_t a[RING];
     const uint32_t k_at = stage_at + k_rel;
 #pragma unroll
@@ -375,7 +373,11 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
       // Written as assembly to put S into ordinary vector registers: with a whole register file per
       // wave the compiler selects the form of the matrix instructions whose results live in
       // accumulation registers, and O fills all 256 of those.
-      if constexpr (t == KS - 1) {
+      if constexpr (t == 0) {
+        // C = 0 as a literal instead of sixteen zeroed registers; the result must not share
+        // registers with the operands
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a[0]), "v"(qf[0]));
+      } else if constexpr (t == KS - 1) {
         // the compiler does not know this is a matrix instruction: the wait states it would put
         // between the last one and the first vector instruction that reads S are spelled out
         asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(acc) : "v"(a[t % RING]), "v"(qf[t]));
