@@ -276,8 +276,50 @@ def extras(torch, K, dev):
                      "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
                      "GBps": round(nbytes / ms / 1e6, 1)}
 
+    def mla_prefill_step(name, prefix_len, chunk_len, nseq, seed):
+        """A chunked-prefill step of an MLA layer as the reference composes it
+        (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_mla_tir.py:293-349):
+        causal self-attention of the chunk on expanded heads (d_qk 192, d_v 128, ragged kernel),
+        attention of the absorbed query over the cached latent prefix (paged MLA kernel, all
+        visible), and the merge of the two states in the 128-wide value space (the projection of
+        the latent output that sits between them in a model is not part of the path)."""
+        rng = np.random.default_rng(seed)
+        n = nseq * chunk_len
+        qi = i32(np.arange(nseq + 1) * chunk_len)
+        qe = (torch.randn((n, hq, 192), device=dev) * 0.5).to(torch.float16)
+        ke = (torch.randn((n, hq, 192), device=dev) * 0.5).to(torch.float16)
+        ve = (torch.randn((n, hq, 128), device=dev) * 0.5).to(torch.float16)
+        o_self = torch.empty((n, hq, 128), dtype=torch.float16, device=dev)
+        l_self = torch.empty((n, hq), dtype=torch.float32, device=dev)
+        zq, zb = torch.zeros(n, dtype=torch.int32, device=dev), torch.zeros(nseq, dtype=torch.int32, device=dev)
+        npg = (prefix_len + ps - 1) // ps
+        pool = nseq * npg + 8
+        perm = rng.permutation(pool).astype(np.int32)
+        pg = (torch.randn((pool, ps, dl + dr), device=dev) * 0.5).to(torch.float16)
+        ip = i32(np.arange(nseq + 1) * npg)
+        qa = (torch.randn((n, hq, dl + dr), device=dev) * 0.5).to(torch.float16)
+        o_lat = torch.empty((n, hq, dl), dtype=torch.float16, device=dev)
+        l_lat = torch.empty((n, hq), dtype=torch.float32, device=dev)
+        o_cross = torch.empty((n, hq, 128), dtype=torch.float16, device=dev).normal_()
+        pv_ = i32(perm[:nseq * npg])
+        last = i32(np.full(nseq, (prefix_len - 1) % ps + 1))
+
+        def step(_):
+            K.batch_prefill_ragged_kv(qe, qi, ke, ve, qi, zq, zb, o_self, l_self, 1, 0, 1.0, 1e4, sm)
+            K.batch_prefill_paged_kv_mla(qa, qi, pg, ip, pv_, last, o_lat, l_lat, 0, sm)
+            K.merge_state_inplace(o_self, l_self, o_cross, l_lat)
+
+        step(0)
+        ms = time_region(torch, step, 10)
+        flops = float(hq) * nseq * (640.0 * chunk_len * (chunk_len + 1) / 2 + 2176.0 * chunk_len * prefix_len)
+        out[name] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                     "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                     "workload": f"configs[4] prefill step: {nseq} seqs, {chunk_len}-token chunk on a {prefix_len}-token "
+                                 "prefix: ragged causal (192/128) + absorbed paged (576->512) + merge, three launches"}
+
     rng = np.random.default_rng(4)
     ctx = rng.integers(2048, 8192, size=32, endpoint=True)
+    mla_prefill_step("mla_prefill_step", 2048, 1024, 4, 8)
     mla_case("mla_decode", ctx - 1, np.ones(32, dtype=np.int64), 5, 0)
     out["mla_decode"]["workload"] = "configs[4] decode: batch 32, ctx U[2048,8192] seed 4, 128 heads, 576-wide latent rows, page 64"
     mla_case("mla_prefill", np.full(4, 2048), np.full(4, 1024), 6, 1)
