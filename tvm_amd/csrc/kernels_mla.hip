@@ -394,9 +394,11 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   // the PV product running beside it (vec_slot<t> follows instruction t).  s[j]: token kv0 + (j/4)*8 +
   // half*4 + j%4, query col.  The reference point only moves when the maximum exceeds it by more
   // than 2^8 (p stays <= 256, same relative precision in fp16), so that after the first tiles no
-  // block rescales O; a fully masked row keeps its reference point.  Slots 0, 1: row maximum of the
-  // lane's 16 scores; 2: the other half's maximum, new reference point, factor for the old state;
-  // 3, 5, .., 17: two probabilities each, as the B-operand of the next PV product.
+  // block rescales O; a fully masked row keeps its reference point.  Slots 0 .. 3: row maximum of the
+  // lane's 16 scores; 4: the other half's maximum; 5: new reference point, factor for the old
+  // state; 6 .. 21: one probability each (a slot must not take longer than the 32 cycles of a matrix
+  // instruction, or the matrix pipe waits for the wave), packed in pairs as the B-operand of the
+  // next PV product.
   float alpha = 1.0f, row_mx = 0.f;
   auto mask_scores = [&](float16_t& s, int kv0) {
     if (kv0 + BN > wave_limit_min) {  // wave-uniform: the causal diagonal or the end of the sequence
@@ -408,39 +410,44 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   };
   auto vec_slot = [&](auto tc, float16_t& s, half8_t (&pf)[2], float& tok) {
     constexpr int t = decltype(tc)::value;
-    if constexpr (t == 0 || t == 1) {
+    if constexpr (t < 4) {  // a quarter of the lane's 16 scores each
       float mx = t == 0 ? -3.0e38f : row_mx;
       pin_after(mx, tok);  // everything below hangs on it
 #pragma unroll
-      for (int j = t * 8; j < t * 8 + 8; ++j) mx = fmaxf(mx, s[j]);
+      for (int j = t * 4; j < t * 4 + 4; ++j) mx = fmaxf(mx, s[j]);
       row_mx = mx;
       pin_after(tok, row_mx);
-    } else if constexpr (t == 2) {
+    } else if constexpr (t == 4) {
       pin_after(row_mx, tok);
       row_mx = max_xor32(row_mx);
+      pin_after(tok, row_mx);
+    } else if constexpr (t == 5) {
+      pin_after(row_mx, tok);
       const float cand = fmaxf(row_mx * p.scale_log2, -1.0e30f);
       const float m_new = cand > m + 8.0f ? cand : m;
       alpha = fast_exp2(m - m_new);
       m = m_new;
       lsum *= alpha;
       pin_after(tok, lsum);
-    } else if constexpr (t >= 3 && t <= 17 && (t & 1) == 1) {
-      constexpr int j = t - 3;  // elements j, j + 1
+    } else if constexpr (t >= 6 && t < 6 + 16) {
+      constexpr int j = t - 6;  // one probability per slot, two of them packed in the odd ones
       float mm = m;
       pin_after(mm, tok);
-      const float p0 = fast_exp2(fmaf(s[j], p.scale_log2, -mm));  // masked: exp2(-huge) = 0
-      const float p1 = fast_exp2(fmaf(s[j + 1], p.scale_log2, -mm));
-      lsum += p0;
-      lsum += p1;
-      pf[j >> 3][j & 7] = static_cast<half_t>(p0);
-      pf[j >> 3][(j & 7) + 1] = static_cast<half_t>(p1);
+      const float pj = fast_exp2(fmaf(s[j], p.scale_log2, -mm));  // masked: exp2(-huge) = 0
+      lsum += pj;
+      if constexpr ((j & 1) == 0) {
+        s[j] = pj;  // kept until its neighbour is there
+      } else {
+        pf[j >> 3][(j & 7) - 1] = static_cast<half_t>(s[j - 1]);
+        pf[j >> 3][j & 7] = static_cast<half_t>(pj);
+      }
       pin_after(tok, lsum);
     }
   };
   auto softmax_alone = [&](float16_t& s, int kv0, half8_t (&pf)[2]) {
     float tok = 0.f;
     mask_scores(s, kv0);
-    static_for<18>([&](auto tc) { vec_slot(tc, s, pf, tok); });
+    static_for<22>([&](auto tc) { vec_slot(tc, s, pf, tok); });
   };
   // O^T += V^T P^T (the value is the first DV features of the same rows), optionally with the
   // softmax of the next tile's scores on the vector ALU beside it
