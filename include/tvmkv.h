@@ -348,6 +348,15 @@ int tvmkv_attention_kv_cache_self_attention(tvmkv_cache* cache, int64_t layer_id
 /* (cache, layer_id, sm_scale, q, o, lse). */
 int tvmkv_attention_kv_cache_cross_attention(tvmkv_cache* cache, int64_t layer_id, double sm_scale,
                                              const void* q, void* o, float* lse, int64_t rows);
+/* `vm.builtin.attention_kv_cache_attention_with_shared_kv` (src/runtime/vm/kv_state.cc:97-105,
+ * paged_kv_cache.cc:1487-1525): (cache, source_layer_id, sm_scale, q, current_k, current_v, o).
+ * The step's queries attend to the K/V that layer `source_layer_id` holds in its pages plus the
+ * rows current_k / current_v (rows, Hkv, D) of the step's own tokens; nothing is appended and q is
+ * used as it is handed in.  rows must equal the batch's total append length. */
+int tvmkv_attention_kv_cache_attention_with_shared_kv(tvmkv_cache* cache, int64_t source_layer_id,
+                                                      double sm_scale, const void* q,
+                                                      const void* current_k, const void* current_v,
+                                                      void* o, int64_t rows);
 /* (cache, layer_id, kv): kv (rows, qk_head_dim). */
 int tvmkv_attention_kv_cache_append_mla_kv(tvmkv_cache* cache, int64_t layer_id, const void* kv,
                                            int64_t rows);

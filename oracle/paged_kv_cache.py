@@ -7,6 +7,7 @@ order the reference's cache object calls them:
   attention_with_fused_qkv   src/runtime/vm/paged_kv_cache.cc:1303-1402
   self_attention             src/runtime/vm/paged_kv_cache.cc:1404-1445
   cross_attention            src/runtime/vm/paged_kv_cache.cc:1447-1485
+  attention_with_shared_kv   src/runtime/vm/paged_kv_cache.cc:1487-1525
   append_mla_kv              src/runtime/vm/paged_kv_cache.cc:1527-1551
   merge_attn_output_inplace  src/runtime/vm/paged_kv_cache.cc:1553-1559
   debug_get_kv(_mla)         src/runtime/vm/paged_kv_cache.cc:1669-1766
@@ -211,6 +212,14 @@ class OraclePagedKVCache:
         out[:total] = o_view
         if not host.append_before_attn:
             ok.transpose_append(self.pages[layer_id], k, v, aux["append_position_map"])
+
+    def attention_with_shared_kv(self, source_layer_id, sm_scale, q, current_k, current_v, out):
+        if self.attn_kinds[source_layer_id] not in (hc.ATTN_MHA, hc.ATTN_MHA_SLIDING):
+            raise hc.CacheError("Querying K/V from another logical layer is only supported for MHA caches.")
+        total = sum(self.host.cur_append_lengths)
+        if not (q.shape[0] == current_k.shape[0] == current_v.shape[0] == out.shape[0] == total):
+            raise hc.CacheError("attention_with_shared_kv: row counts do not match the batch")
+        self._attention_internal(source_layer_id, q, current_k, current_v, out, sm_scale)
 
     def self_attention(self, layer_id, sm_scale, q, k, v, out, lse):
         if self.attn_kinds[layer_id] == hc.ATTN_MHA:

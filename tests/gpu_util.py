@@ -70,6 +70,12 @@ class GpuCache:
         gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")(self.cache, layer, sm_scale, dev(qkv), o)
         out[...] = host(o)
 
+    def attention_with_shared_kv(self, source_layer, sm_scale, q, current_k, current_v, out):
+        o = torch.zeros(out.shape, dtype=torch.float16, device=DEV)
+        gf("vm.builtin.attention_kv_cache_attention_with_shared_kv")(self.cache, source_layer, sm_scale, dev(q),
+                                                                     dev(current_k), dev(current_v), o)
+        out[...] = host(o)
+
     def self_attention(self, layer, sm_scale, q, k, v, out, lse):
         o = torch.zeros(out.shape, dtype=torch.float16, device=DEV)
         s = torch.zeros(lse.shape, dtype=torch.float32, device=DEV)

@@ -306,6 +306,18 @@ def run_sliding_window_fork(sc):
     sc.step([(3, 10), (6, 12)])
 
 
+def run_sliding_window_page_reuse(sc):
+    """Four sequences with a 40-token window and 4 sink tokens, six steps of 17 tokens each: from the
+    third step on every sequence slides its window while the step's slots are reserved, the pages it
+    frees go to the next sequence of the same batch, and that sequence's new tokens land on slots the
+    step's page table of the first one still attends to.  Only a cache that writes the new rows after
+    attention (src/runtime/vm/paged_kv_cache.cc:1396-1401) computes this batch correctly."""
+    for sid in range(4):
+        sc.add_with_window(sid, 40, 4)
+    for _ in range(6):
+        sc.step([(sid, 17) for sid in range(4)])
+
+
 def run_tree_attn(sc):
     """test_paged_attention_kv_cache_tree_attn
     (tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_tir.py:1053-1134)."""

@@ -152,7 +152,7 @@ def test_error_paths_on_the_device_cache():
         attn(c2.cache, 0, 1.0, qkv96, out96)
 
 
-@pytest.mark.parametrize("runner", [S.run_sliding_window, S.run_sliding_window_fork])
+@pytest.mark.parametrize("runner", [S.run_sliding_window, S.run_sliding_window_fork, S.run_sliding_window_page_reuse])
 def test_sliding_window_scenarios_on_the_gpu(runner):
     """The reference's sliding-window tests (attention sinks, window trimming after every step,
     forks inside the sink; tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_cpu.py:912-1022)
@@ -190,3 +190,52 @@ def test_padded_qkv_rows_are_ignored():
     o_pad = np.full((16, hq, d), 3.0, np.float16)
     b.attention_with_fused_qkv(0, d ** -0.5, padded, o_pad)
     assert np.array_equal(o_pad[:10], o_exact)
+
+
+def test_attention_with_shared_kv_reads_the_source_layer():
+    """vm.builtin.attention_kv_cache_attention_with_shared_kv (src/runtime/vm/kv_state.cc:97-105,
+    paged_kv_cache.cc:1487-1525): a second set of queries attends to the K/V that layer 0 caches plus
+    the step's own rows, nothing is appended.  Prefill (self + cross), a second chunk, then decode;
+    checked against the oracle cache and against the closed form over layer 0's K/V."""
+    from oracle import closed_form as cf
+    layers, hq, hkv, d = 2, 8, 2, 128
+    cfg = [4, 512, 128, 16, 0]
+    gpu = GpuCache(cfg, layers, hq, hkv, d, d, rope_mode=S.ROPE_NONE)
+    cpu = OraclePagedKVCache(cfg, layers, hq, hkv, d, d, rope_mode=S.ROPE_NONE)
+    rng = np.random.default_rng(17)
+    cached_k = {0: np.zeros((0, hkv, d), np.float16), 1: np.zeros((0, hkv, d), np.float16)}
+    cached_v = {0: np.zeros((0, hkv, d), np.float16), 1: np.zeros((0, hkv, d), np.float16)}
+    for cache in (gpu, cpu):
+        cache.add_sequence(0)
+        cache.add_sequence(1)
+    for lens in ([40, 23], [9, 30], [1, 1], [1, 1]):
+        total = sum(lens)
+        qkv = rng.standard_normal((total, hq + 2 * hkv, d)).astype(np.float16)
+        q2 = rng.standard_normal((total, hq, d)).astype(np.float16)
+        k_cur = np.ascontiguousarray(qkv[:, hq:hq + hkv])
+        v_cur = np.ascontiguousarray(qkv[:, hq + hkv:])
+        outs = []
+        for cache in (gpu, cpu):
+            cache.begin_forward([0, 1], lens)
+            o1 = np.zeros((total, hq, d), np.float16)
+            cache.attention_with_fused_qkv(0, d ** -0.5, qkv, o1)
+            o2 = np.zeros((total, hq, d), np.float16)
+            cache.attention_with_shared_kv(0, d ** -0.5, q2, k_cur, v_cur, o2)
+            cache.end_forward()
+            outs.append(o2)
+        assert_close(outs[0], outs[1], what=f"shared-kv attention vs oracle cache, step {lens}")
+        cursor = 0
+        for sid, n in enumerate(lens):
+            cached_k[sid] = np.concatenate([cached_k[sid], k_cur[cursor:cursor + n]])
+            cached_v[sid] = np.concatenate([cached_v[sid], v_cur[cursor:cursor + n]])
+            expected, _ = cf.attention(q2[cursor:cursor + n], cached_k[sid], cached_v[sid], d ** -0.5, causal=True)
+            assert_close(outs[0][cursor:cursor + n], expected, atol=4e-3, rtol=4e-3,
+                         what=f"shared-kv attention vs closed form, seq {sid}")
+            cursor += n
+    # layer 1 never received anything
+    with pytest.raises(tvm_amd.KVError, match="rows"):
+        gf("vm.builtin.attention_kv_cache_attention_with_shared_kv")(
+            gpu.cache, 0, 1.0, torch.zeros((5, hq, d), dtype=torch.float16, device=DEV),
+            torch.zeros((5, hkv, d), dtype=torch.float16, device=DEV),
+            torch.zeros((5, hkv, d), dtype=torch.float16, device=DEV),
+            torch.zeros((5, hq, d), dtype=torch.float16, device=DEV))

@@ -16,6 +16,7 @@ from oracle import host_cache as hc
 from oracle.paged_kv_cache import OraclePagedKVCache
 from tests import scenario as S
 from tests.invariants import check_pool_invariants
+from tests.util import assert_close
 
 
 def make(capacity=16368, reserved=32, chunk=8192, ps=16, sliding=0):
@@ -243,7 +244,46 @@ def test_reference_scenarios_on_the_oracle(runner, rope_mode):
     check_pool_invariants(cache.host.state(), cache.host.num_total_pages, ps)
 
 
-@pytest.mark.parametrize("runner", [S.run_sliding_window, S.run_sliding_window_fork])
+def _attended_slots(aux, depth, row, page_size):
+    """Slots the step's page table lets sequence `row` attend to at `depth`: sink tokens, then the
+    window (python/tvm/relax/frontend/nn/llm/_kernel_common.py:155-170)."""
+    lo, hi = aux["page_indptr"][depth][row], aux["page_indptr"][depth][row + 1]
+    pages = aux["page_indices"][depth][lo:hi]
+    if not pages:
+        return set()
+    phys_len = (len(pages) - 1) * page_size + aux["last_page_len"][depth][row]
+    sink, win_lo = aux["sink_size"][depth][row], aux["sliding_window_offset"][depth][row]
+    tokens = list(range(sink)) + list(range(win_lo, phys_len))
+    return {pages[t // page_size] * page_size + t % page_size for t in tokens}
+
+
+def test_sliding_window_reuses_attended_slots_within_a_step():
+    """Why a sliding-window cache must append AFTER attention: in this batch the new tokens of one
+    sequence are given slots that the same step's page table of another sequence attends to.  The
+    oracle (which follows the reference's order) and the closed form still agree on every output."""
+    ps = 16
+    host = hc.HostCache([32, 2048, 512, ps, 1], [hc.ATTN_MHA], hc.ROPE_NORMAL)
+    for sid in range(4):
+        host.add_sequence(sid)
+        host.enable_sliding_window_for_seq(sid, 40, 4)
+    clashes = []
+    for _ in range(6):
+        host.begin_forward([0, 1, 2, 3], [17] * 4)
+        assert not host.aux["append_before_attn"]
+        attended = [_attended_slots(host.aux, 0, row, ps) for row in range(4)]
+        new = [s for s in host.aux["append_position_map"] if s != -1]
+        indptr = host.aux["cur_append_lengths_indptr"]
+        clash = 0
+        for row in range(4):
+            mine = set(host.aux["append_position_map"][indptr[row]:indptr[row + 1]]) - {-1}
+            clash += sum(len(mine & attended[other]) for other in range(4) if other != row)
+        clashes.append(clash)
+        assert len(new) == len(set(new)), "two new tokens share a slot"
+        host.end_forward()
+    assert clashes[:3] == [0, 0, 0] and all(c > 0 for c in clashes[3:]), clashes
+
+
+@pytest.mark.parametrize("runner", [S.run_sliding_window, S.run_sliding_window_fork, S.run_sliding_window_page_reuse])
 def test_sliding_window_scenarios_on_the_oracle(runner):
     """Sliding-window cache with attention sinks: RoPE is applied inside the kernels at positions
     counted inside the cache (the reference switches such caches to INLINE mode,
@@ -267,3 +307,26 @@ def test_token_tree_scenario_on_the_oracle(rope_mode):
     sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=rope_mode, seed=6, on_step=on_step)
     S.run_tree_attn(sc)
     check_pool_invariants(cache.host.state(), cache.host.num_total_pages, ps)
+
+
+def test_attention_with_shared_kv_on_the_oracle():
+    """src/runtime/vm/paged_kv_cache.cc:1487-1525: queries of another layer attend to layer 0's cached
+    K/V plus the step's own rows; equals the closed form over layer 0's K/V, in prefill and decode."""
+    from oracle import closed_form as cf
+    layers, hq, hkv, d = 2, 4, 2, 64
+    cache = OraclePagedKVCache([4, 256, 64, 16, 0], layers, hq, hkv, d, d, rope_mode=S.ROPE_NONE)
+    rng = np.random.default_rng(5)
+    cache.add_sequence(0)
+    ks, vs = np.zeros((0, hkv, d), np.float16), np.zeros((0, hkv, d), np.float16)
+    for n in (21, 12, 1, 1):
+        qkv = rng.standard_normal((n, hq + 2 * hkv, d)).astype(np.float16)
+        q2 = rng.standard_normal((n, hq, d)).astype(np.float16)
+        k_cur, v_cur = np.ascontiguousarray(qkv[:, hq:hq + hkv]), np.ascontiguousarray(qkv[:, hq + hkv:])
+        cache.begin_forward([0], [n])
+        o1, o2 = np.zeros((n, hq, d), np.float16), np.zeros((n, hq, d), np.float16)
+        cache.attention_with_fused_qkv(0, d ** -0.5, qkv, o1)
+        cache.attention_with_shared_kv(0, d ** -0.5, q2, k_cur, v_cur, o2)
+        cache.end_forward()
+        ks, vs = np.concatenate([ks, k_cur]), np.concatenate([vs, v_cur])
+        expected, _ = cf.attention(q2, ks, vs, d ** -0.5, causal=True)
+        assert_close(o2, expected, atol=2e-3, rtol=2e-3, what=f"shared-kv attention, append {n}")

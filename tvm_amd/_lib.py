@@ -72,6 +72,7 @@ SIGNATURES = {
     "tvmkv_attention_kv_cache_self_attention": [c_vp, c_i64, c_f64, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i32,
                                                 c_i32, c_i32],
     "tvmkv_attention_kv_cache_cross_attention": [c_vp, c_i64, c_f64, c_vp, c_vp, c_vp, c_i64],
+    "tvmkv_attention_kv_cache_attention_with_shared_kv": [c_vp, c_i64, c_f64, c_vp, c_vp, c_vp, c_vp, c_i64],
     "tvmkv_attention_kv_cache_append_mla_kv": [c_vp, c_i64, c_vp, c_i64],
     "tvmkv_attention_kv_cache_merge_attn_output_inplace": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_i32],
     "tvmkv_attention_kv_cache_debug_get_kv": [c_vp, c_i64, c_i64, c_i64, c_vp, c_vp],

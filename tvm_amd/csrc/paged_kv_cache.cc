@@ -638,18 +638,51 @@ class PagedKVCache {
     ComputeStreamWaitForCopyStream();
     KV_CHECK(!dirty_aux_data_device_) << "auxiliary data is not synchronised";
 
-    // Part 2: split fused qkv, RoPE on q/k.
-    // Part 3 (or 6) with it, in one launch: the new k / v rows go into their page slots while q, k, v
-    // are written.  When the reference appends after attention (chunked prefill) the earlier append
-    // changes nothing: the page tables of this step cover the tokens cached before it, the kernels
-    // never read a slot beyond them, and the slots of the new tokens are not shared with anyone.
-    Launch(tvmkv_fused_rope_append(qkv, q_rope_position_map_view_.ptr, temp_q_, temp_k_, temp_v_,
-                                   rope_mode_ == TVMKV_ROPE_NORMAL, pages_[local_layer_id],
-                                   append_position_map_view_.ptr, total_seq_length, num_qo_heads_, num_kv_heads_,
-                                   qk_head_dim_, num_total_pages_, page_size_, rotary_scale_, rotary_theta_,
-                                   compute_stream_));
+    // Part 2: split fused qkv, RoPE on q/k.  Part 3 with it, in one launch, when the new k / v rows may
+    // go into their page slots before attention: always when the reference appends first, and in a
+    // cache without sliding windows also when the reference appends afterwards (:1396-1401) -- there
+    // the step's page tables cover only the tokens cached before it, the new slots lie on pages
+    // that were free or beyond their sequence's cached tokens, and no kernel of the step reads them.
+    // A sliding-window cache frees pages while it reserves the step's slots and hands them out again
+    // in the same step (:1935-1992, :2004-2044): a new token's slot can be one that the step's page
+    // table of another sequence still attends to, so there the rows are written after attention.
+    const bool append_early = append_before_attn_ || !support_sliding_window_;
+    if (append_early) {
+      Launch(tvmkv_fused_rope_append(qkv, q_rope_position_map_view_.ptr, temp_q_, temp_k_, temp_v_,
+                                     rope_mode_ == TVMKV_ROPE_NORMAL, pages_[local_layer_id],
+                                     append_position_map_view_.ptr, total_seq_length, num_qo_heads_, num_kv_heads_,
+                                     qk_head_dim_, num_total_pages_, page_size_, rotary_scale_, rotary_theta_,
+                                     compute_stream_));
+    } else {
+      Launch(tvmkv_fused_rope(qkv, q_rope_position_map_view_.ptr, temp_q_, temp_k_, temp_v_,
+                              rope_mode_ == TVMKV_ROPE_NORMAL, total_seq_length, num_qo_heads_, num_kv_heads_,
+                              qk_head_dim_, rotary_scale_, rotary_theta_, compute_stream_));
+    }
     // Part 5: attention.
     AttentionInternal(layer_id, temp_q_, temp_k_, temp_v_, out, total_seq_length, sm_scale);
+    // Part 6: append after attention (:1396-1401).
+    if (!append_early) {
+      Launch(tvmkv_kv_cache_transpose_append(pages_[local_layer_id], temp_k_, temp_v_, append_position_map_view_.ptr,
+                                             total_seq_length, num_total_pages_, num_kv_heads_, page_size_,
+                                             qk_head_dim_, compute_stream_));
+    }
+    RecordComputeEvent();
+  }
+
+  // :1487-1525: attention of this step's queries against the K/V of another layer (the new tokens'
+  // rows are handed in; nothing is appended).
+  void AttentionWithSharedKV(int64_t source_layer_id, const void* q, const void* k, const void* v, void* o,
+                             int64_t rows, double sm_scale) {
+    RequireDevice();
+    CheckLayer(source_layer_id);
+    KV_CHECK(attn_kinds_[source_layer_id] == TVMKV_ATTN_MHA || attn_kinds_[source_layer_id] == TVMKV_ATTN_MHA_SLIDING)
+        << "Querying K/V from another logical layer is only supported for MHA caches.";
+    int64_t total_seq_length = TotalAppendLength();
+    KV_CHECK(rows == total_seq_length)
+        << "attention_with_shared_kv expects " << total_seq_length << " rows, got " << rows;
+    ComputeStreamWaitForCopyStream();
+    KV_CHECK(!dirty_aux_data_device_) << "auxiliary data is not synchronised";
+    AttentionInternal(source_layer_id, q, k, v, o, total_seq_length, sm_scale);
     RecordComputeEvent();
   }
 
@@ -1151,6 +1184,7 @@ class PagedKVCache {
         HIP_CHECK(hipMalloc(&aux_device_[i], aux_capacity_ * sizeof(int32_t)));
         HIP_CHECK(hipHostMalloc(&aux_staging_[i], aux_capacity_ * sizeof(int32_t), hipHostMallocDefault));
         HIP_CHECK(hipEventCreateWithFlags(&aux_copied_[i], hipEventDisableTiming));
+      HIP_CHECK(hipEventCreateWithFlags(&aux_consumed_[i], hipEventDisableTiming));
       }
       // token-tree commit: copy_length_indptr + (2, copies) positions (attn_utils.h:1010-1021)
       commit_capacity_ = (r + 1 + 3) / 4 * 4 + 2 * std::min<int64_t>(kTreeAttnMaxTreeSize * r, c) + 4;
@@ -1181,8 +1215,10 @@ class PagedKVCache {
       (void)hipFree(aux_device_[i]);
       if (aux_staging_[i]) (void)hipHostFree(aux_staging_[i]);
       if (aux_copied_[i]) (void)hipEventDestroy(aux_copied_[i]);
+      if (aux_consumed_[i]) (void)hipEventDestroy(aux_consumed_[i]);
       aux_device_[i] = aux_staging_[i] = nullptr;
-      aux_copied_[i] = nullptr;
+      aux_copied_[i] = aux_consumed_[i] = nullptr;
+      aux_consumed_recorded_[i] = false;
     }
     (void)hipFree(commit_device_);
     if (commit_staging_) (void)hipHostFree(commit_staging_);
@@ -1199,6 +1235,9 @@ class PagedKVCache {
   void RecordComputeEvent() {
     HIP_CHECK(hipEventRecord(compute_done_, compute_stream_));
     compute_event_recorded_ = true;
+    // the kernels enqueued so far are the last readers of the auxiliary buffer in use
+    HIP_CHECK(hipEventRecord(aux_consumed_[aux_slot_], compute_stream_));
+    aux_consumed_recorded_[aux_slot_] = true;
   }
 
   // :721-734.  The copy runs on the copy stream, after everything enqueued on the compute
@@ -1469,6 +1508,9 @@ class PagedKVCache {
       }
     }
     if (cursor) {
+      // A host that runs ahead of the device must not overwrite arrays that kernels of the step
+      // two uploads ago, still queued on the compute stream, have yet to read.
+      if (aux_consumed_recorded_[aux_slot_]) HIP_CHECK(hipStreamWaitEvent(copy_stream_, aux_consumed_[aux_slot_], 0));
       HIP_CHECK(hipMemcpyAsync(device, staging, cursor * sizeof(int32_t), hipMemcpyHostToDevice, copy_stream_));
     }
     aux_slot_used_[aux_slot_] = true;
@@ -1526,6 +1568,8 @@ class PagedKVCache {
   void* aux_device_[2] = {nullptr, nullptr};
   void* aux_staging_[2] = {nullptr, nullptr};
   hipEvent_t aux_copied_[2] = {nullptr, nullptr};
+  hipEvent_t aux_consumed_[2] = {nullptr, nullptr};  // recorded on the compute stream behind a slot's last readers
+  bool aux_consumed_recorded_[2] = {false, false};
   bool aux_slot_used_[2] = {false, false};
   int aux_slot_ = 0;
   int64_t commit_capacity_ = 0;
@@ -1639,6 +1683,11 @@ int tvmkv_attention_kv_cache_self_attention(tvmkv_cache* cache, int64_t layer_id
 int tvmkv_attention_kv_cache_cross_attention(tvmkv_cache* cache, int64_t layer_id, double sm_scale, const void* q,
                                              void* o, float* lse, int64_t rows) {
   KV_CACHE_FN(cache->impl->CrossAttention(layer_id, q, o, lse, rows, sm_scale));
+}
+int tvmkv_attention_kv_cache_attention_with_shared_kv(tvmkv_cache* cache, int64_t source_layer_id, double sm_scale,
+                                                      const void* q, const void* current_k, const void* current_v,
+                                                      void* o, int64_t rows) {
+  KV_CACHE_FN(cache->impl->AttentionWithSharedKV(source_layer_id, q, current_k, current_v, o, rows, sm_scale));
 }
 int tvmkv_attention_kv_cache_append_mla_kv(tvmkv_cache* cache, int64_t layer_id, const void* kv, int64_t rows) {
   KV_CACHE_FN(cache->impl->AppendMLAKV(layer_id, kv, rows));

@@ -224,6 +224,18 @@ def _cross_attention(cache, layer_id, sm_scale, q, o, lse):
         cache.handle, layer_id, float(sm_scale), _ptr(q), _ptr(o), _ptr(lse), q.shape[0]))
 
 
+def _attention_with_shared_kv(cache, source_layer_id, sm_scale, q, current_k, current_v, o):
+    _require_contiguous(q, current_k, current_v, o)
+    if not (q.shape[0] == current_k.shape[0] == current_v.shape[0] == o.shape[0]):
+        raise KVError(-1, "attention_with_shared_kv: q, current_k, current_v, o must have the same number of rows")
+    if current_k.shape[1] != cache.num_kv_heads or current_k.shape[2] != cache.qk_head_dim or \
+            current_v.shape[2] != cache.v_head_dim:
+        raise KVError(-1, "attention_with_shared_kv: current_k / current_v do not have the cache's head shape")
+    check(lib().tvmkv_attention_kv_cache_attention_with_shared_kv(
+        cache.handle, source_layer_id, float(sm_scale), _ptr(q), _ptr(current_k), _ptr(current_v), _ptr(o),
+        q.shape[0]))
+
+
 def _append_mla_kv(cache, layer_id, kv):
     _require_contiguous(kv)
     check(lib().tvmkv_attention_kv_cache_append_mla_kv(cache.handle, layer_id, _ptr(kv), kv.shape[0]))
@@ -294,6 +306,7 @@ _GLOBAL_FUNCS = {
     "vm.builtin.attention_kv_cache_attention_with_fused_qkv": _attention_with_fused_qkv,
     "vm.builtin.attention_kv_cache_self_attention": _self_attention,
     "vm.builtin.attention_kv_cache_cross_attention": _cross_attention,
+    "vm.builtin.attention_kv_cache_attention_with_shared_kv": _attention_with_shared_kv,
     "vm.builtin.attention_kv_cache_append_mla_kv": _append_mla_kv,
     "vm.builtin.attention_kv_cache_merge_attn_output_inplace": _merge_attn_output_inplace,
     "vm.builtin.attention_kv_cache_debug_get_kv": _debug_get_kv,
