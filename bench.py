@@ -174,12 +174,13 @@ def extras(torch, K, dev):
     K.batch_decode_paged_kv(*args)
     ms = time_region(torch, lambda i: K.batch_decode_paged_kv(*args), 10)
     nbytes = float(ctx.sum()) * 2 * hkv * d * 2 + 2 * 8 * hq * d * 2
-    # the same call with the chunk merge as a second kernel (the library reads the switch per call):
-    # the difference is what merging inside the kernel saves
-    os.environ["TVMKV_DECODE_SEPARATE_MERGE"] = "1"
+    # the same call with the chunk merge as a second kernel: the difference is what merging inside
+    # the kernel saves
+    import tvm_amd
+    tvm_amd.set_option("decode_separate_merge", 1)
     K.batch_decode_paged_kv(*args)
     ms_two_kernels = time_region(torch, lambda i: K.batch_decode_paged_kv(*args), 10)
-    del os.environ["TVMKV_DECODE_SEPARATE_MERGE"]
+    tvm_amd.set_option("decode_separate_merge", 0)
     out["long_context_decode"] = {"workload": "configs[3]: 8 seqs, ctx U[32768,131072] seed 3, Hq64/Hkv8/D128, page 16",
                                   "kv_tokens": int(ctx.sum()), "ms": round(ms, 4),
                                   "ms_with_separate_merge_kernel": round(ms_two_kernels, 4),

@@ -25,8 +25,10 @@
  * text of the reference's failed check where one exists).  Nothing throws across the ABI.
  *
  * Threading: a cache object is not thread-safe (neither is the reference's).  The split-KV
- * decode launcher uses one lazily grown workspace per device: calls on the same device must
- * be ordered on one stream.
+ * launchers (decode, MLA decode) keep their scratch memory per (device, stream): calls on one
+ * stream are ordered and share it, calls on different streams never do, and the table of buffers
+ * is guarded by a mutex.  A buffer grows with hipMalloc when a call needs more than any before it
+ * on that stream (after synchronising that stream only).
  */
 #ifndef TVMKV_H_
 #define TVMKV_H_
@@ -258,6 +260,25 @@ int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr,
                           const int32_t* copy_src_dst_pos, int32_t batch_size,
                           int32_t total_copy_length, int64_t num_pages, int32_t num_kv_heads,
                           int32_t page_size, int32_t head_dim, void* stream);
+
+/* Tuning options (no counterpart in the reference).  Each starts from an environment variable read
+ * once when the library is loaded (TVMKV_ + the upper-case name) and defaults to 0:
+ *   decode_chunk_pages     pages per split-KV chunk of the decode kernel (a multiple of 8); 0 = from shapes
+ *   decode_separate_merge  != 0: merge the decode chunks in a second launch instead of inside the kernel
+ *   decode_wgs_per_cu      > 0: cap the decode grid at this many workgroups per compute unit
+ *   mla_chunk_tokens       tokens per split-KV chunk of MLA decode; 0 = from shapes
+ *   mla_separate_merge     != 0: merge the MLA decode chunks in a second launch */
+int tvmkv_set_option(const char* name, int64_t value);
+int tvmkv_get_option(const char* name, int64_t* value);
+
+/* Host view of the decode split (no counterpart in the reference; the tests check the arithmetic the
+ * kernel repeats on the device).  page_indptr_host is a HOST array (batch_size + 1).  Writes the
+ * chunk size in pages and the number of chunk slots of the launch; when slot_seq and slot_chunk are
+ * not NULL (room for slot_capacity entries each) also the sequence and chunk index every slot
+ * resolves to, -1 for a spare slot. */
+int tvmkv_decode_split_plan(const int32_t* page_indptr_host, int32_t batch_size, int64_t nnz_pages,
+                            int32_t h_kv, int32_t* chunk_pages, int64_t* num_slots, int32_t* slot_seq,
+                            int32_t* slot_chunk, int64_t slot_capacity);
 
 /* Measurement utilities (no counterpart in the reference): a plain streaming read (XOR-folded,
  * the result is discarded) and a plain copy of `num_bytes` (a multiple of 16) bytes.  The

@@ -15,6 +15,7 @@ import pytest
 import torch
 
 import bench
+import tvm_amd
 from oracle import kernels as ok
 from tests.gpu_util import DEV, host, i32
 from tests.util import assert_close
@@ -71,28 +72,24 @@ def test_decode_full_size_properties(name, batch, lo, hi, hq, pool):
         assert_close(host(out[b]), eo, what=f"{name} seq {b} out")
         assert_close(host(lse[b]), el, atol=2e-3, rtol=1e-4, what=f"{name} seq {b} lse")
     # chunk-size independence of the split-KV path
-    prev = os.environ.get("TVMKV_DECODE_CHUNK_PAGES")
+    prev = tvm_amd.set_option("decode_chunk_pages", 8)
     try:
-        os.environ["TVMKV_DECODE_CHUNK_PAGES"] = "8"
         out8, lse8 = _decode(q, pages, t)
-        os.environ["TVMKV_DECODE_CHUNK_PAGES"] = "128"
+        tvm_amd.set_option("decode_chunk_pages", 128)
         out128, lse128 = _decode(q, pages, t)
     finally:
-        if prev is None:
-            os.environ.pop("TVMKV_DECODE_CHUNK_PAGES", None)
-        else:
-            os.environ["TVMKV_DECODE_CHUNK_PAGES"] = prev
+        tvm_amd.set_option("decode_chunk_pages", prev)
     assert_close(host(out8), host(out128), atol=2e-3, rtol=2e-3, what=f"{name} chunk 8 vs 128")
     assert_close(host(lse8), host(lse128), atol=1e-3, rtol=1e-5, what=f"{name} lse chunk 8 vs 128")
     assert_close(host(out), host(out128), atol=2e-3, rtol=2e-3, what=f"{name} default chunk vs 128")
     # the chunk merge done by the last workgroup of each (sequence, kv head) against the same
     # arithmetic in a second kernel: bit-identical, every time (a stale read of another
     # workgroup's partial state would show here)
-    os.environ["TVMKV_DECODE_SEPARATE_MERGE"] = "1"
+    prev = tvm_amd.set_option("decode_separate_merge", 1)
     try:
         out_sep, lse_sep = _decode(q, pages, t)
     finally:
-        os.environ.pop("TVMKV_DECODE_SEPARATE_MERGE", None)
+        tvm_amd.set_option("decode_separate_merge", prev)
     for _ in range(20):
         out_f, lse_f = _decode(q, pages, t)
         assert torch.equal(out_f, out_sep) and torch.equal(lse_f, lse_sep), f"{name}: fused merge differs"

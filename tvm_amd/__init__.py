@@ -8,5 +8,5 @@ and friends return callables with the reference's argument order
 (src/runtime/vm/kv_state.cc:33-116 of the reference), and ``tvm_amd.kernels`` exposes the
 kernel launchers with the argument order of the reference's kernel slots.
 """
-from ._lib import LIB_PATH, KVError, lib  # noqa: F401
+from ._lib import LIB_PATH, KVError, decode_split_plan, lib, set_option  # noqa: F401
 from .runtime import AttnKind, RopeMode, Shape, get_global_func  # noqa: F401

@@ -48,6 +48,9 @@ SIGNATURES = {
     "tvmkv_kv_cache_debug_get_kv": [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_kv_cache_debug_get_kv_mla": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
     "tvmkv_compact_kv_copy": [c_vp, c_vp, c_vp, c_i32, c_i32, c_i64, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_set_option": [ctypes.c_char_p, c_i64],
+    "tvmkv_get_option": [ctypes.c_char_p, p_i64],
+    "tvmkv_decode_split_plan": [p_i32, c_i32, c_i64, c_i32, p_i32, p_i64, p_i32, p_i32, c_i64],
     "tvmkv_stream_read": [c_vp, c_i64, c_vp, c_vp],
     "tvmkv_stream_read_nt": [c_vp, c_i64, c_vp, c_vp],
     "tvmkv_mfma_loop": [c_vp, c_vp, c_i32, c_i32, c_vp],
@@ -111,3 +114,25 @@ def lib():
 def check(rc):
     if rc != 0:
         raise KVError(rc, lib().tvmkv_last_error().decode())
+
+
+def set_option(name, value):
+    """Sets a tuning option of the library (see tvmkv_set_option in include/tvmkv.h); returns the old value."""
+    old = ctypes.c_int64()
+    check(lib().tvmkv_get_option(name.encode(), ctypes.byref(old)))
+    check(lib().tvmkv_set_option(name.encode(), int(value)))
+    return old.value
+
+
+def decode_split_plan(page_indptr, nnz_pages, h_kv):
+    """(chunk_pages, slot_seq, slot_chunk) of a decode launch with these shapes; host arithmetic only."""
+    batch = len(page_indptr) - 1
+    indptr = (ctypes.c_int32 * (batch + 1))(*[int(v) for v in page_indptr])
+    cp, slots = ctypes.c_int32(), ctypes.c_int64()
+    check(lib().tvmkv_decode_split_plan(indptr, batch, int(nnz_pages), int(h_kv), ctypes.byref(cp),
+                                        ctypes.byref(slots), None, None, 0))
+    seq = (ctypes.c_int32 * max(slots.value, 1))()
+    chunk = (ctypes.c_int32 * max(slots.value, 1))()
+    check(lib().tvmkv_decode_split_plan(indptr, batch, int(nnz_pages), int(h_kv), ctypes.byref(cp),
+                                        ctypes.byref(slots), seq, chunk, slots.value))
+    return cp.value, list(seq[:slots.value]), list(chunk[:slots.value])

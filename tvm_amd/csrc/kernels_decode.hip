@@ -29,6 +29,8 @@
 #include <cstdlib>
 
 #include "kernels_common.cuh"
+#include "runtime_support.h"
+#include "split_plan.h"
 
 namespace tvmkv {
 
@@ -49,32 +51,18 @@ struct DecodeParams {
   const int32_t* q_rope_position;    // (B) position of the query token (inline RoPE)
   int rotary;                     // 1: rotate q and k inside the kernel
   float rope_scale;
-  int* arrivals;   // (batch, h_kv) chunk workgroups that have delivered their partial state; all zero
-                   // between calls (fused merge of decode_mfma_kernel), or NULL
+  // (batch, h_kv) arrival counters of the fused chunk merge of decode_mfma_kernel, or NULL.  A counter
+  // is epoch << 32 | workgroups that have delivered their partial state in the launch with that epoch;
+  // a word with an older epoch is what an earlier launch left behind and counts as zero, so nothing
+  // has to be reset between launches, not even after one that failed half way.
+  unsigned long long* arrivals;
+  uint32_t epoch;
   int batch_size;
   int h_q;
   int h_kv;
   int chunk_pages;
   float scale_log2;  // sm_scale * log2(e)
 };
-
-__device__ __forceinline__ int slot_begin(const int32_t* page_indptr, int b, int cp) {
-  return page_indptr[b] / cp + b;
-}
-
-// Largest b in [0, batch) with slot_begin(b) <= slot.
-__device__ __forceinline__ int find_sequence(const int32_t* page_indptr, int batch, int cp, int slot) {
-  int lo = 0, hi = batch - 1;
-  while (lo < hi) {
-    int mid = (lo + hi + 1) >> 1;
-    if (slot_begin(page_indptr, mid, cp) <= slot) {
-      lo = mid;
-    } else {
-      hi = mid - 1;
-    }
-  }
-  return lo;
-}
 
 // Same answer as find_sequence, computed by one wavefront with one round trip per 64 sequences:
 // lane i evaluates slot_begin(base + i) <= slot, and because slot_begin is increasing the number
@@ -644,18 +632,22 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   // L2 and made the kernel 2-4 x slower): the partial states are written with device-scope stores,
   // every wave waits until its own have completed, the barrier collects the waves, one thread
   // counts the workgroup in with a device-scope atomic, and the workgroup that completes the count
-  // reads the states with device-scope loads.  The counter is reset for the next call.
+  // reads the states with device-scope loads.  The counter carries the launch's epoch in its upper
+  // half: the maximum brings a word of an older launch to (epoch, 0) and leaves this launch's alone.
   if (p.arrivals != nullptr && !single_chunk) {
     wait_vmcnt<0>();
     __syncthreads();
     if (tid == 0) {
-      sm_last = __hip_atomic_fetch_add(p.arrivals + b * p.h_kv + kvh, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
-                nchunks - 1;
+      unsigned long long* counter = p.arrivals + b * p.h_kv + kvh;
+      __hip_atomic_fetch_max(counter, static_cast<unsigned long long>(p.epoch) << 32, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned long long before =
+          __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      sm_last = static_cast<uint32_t>(before) == static_cast<uint32_t>(nchunks - 1);
     }
     __syncthreads();
     if (sm_last) {
       for (int g = wave; g < group; g += 4) merge_row<D, true>(p, b, kvh * group + g, nchunks, lane);
-      if (tid == 0) __hip_atomic_store(p.arrivals + b * p.h_kv + kvh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
   __syncthreads();  // the merge buffers are the next item's V tiles
@@ -667,47 +659,7 @@ __global__ void iota_kernel(int32_t* out, int n) {
   if (i < n) out[i] = i;
 }
 
-// ---- per-device workspace for the partial states, grown on demand --------------------------
-struct Workspace {
-  void* ptr = nullptr;
-  size_t bytes = 0;
-};
-static Workspace g_workspace[64];
-
-constexpr size_t kArrivalBytes = 256 * 1024;  // the first bytes of the workspace: arrival counters, zero between calls
-
-static void* get_workspace(size_t bytes) {
-  int dev = 0;
-  HIP_CHECK(hipGetDevice(&dev));
-  KV_CHECK(dev >= 0 && dev < 64) << "device ordinal " << dev << " out of range";
-  Workspace& ws = g_workspace[dev];
-  if (ws.bytes < bytes) {
-    if (ws.ptr) {
-      HIP_CHECK(hipDeviceSynchronize());  // kernels of earlier calls may still read the old buffer
-      HIP_CHECK(hipFree(ws.ptr));
-      ws.ptr = nullptr;
-      ws.bytes = 0;
-    }
-    size_t want = bytes + bytes / 2;
-    HIP_CHECK(hipMalloc(&ws.ptr, want));
-    ws.bytes = want;
-    HIP_CHECK(hipMemset(ws.ptr, 0, kArrivalBytes));
-  }
-  return ws.ptr;
-}
-
-// Pages per chunk from shapes only: aim at ~8K workgroups, keep a chunk between 4 and 64 pages.
-static int pick_chunk_pages(int64_t nnz_pages, int h_kv) {
-  const char* forced = getenv("TVMKV_DECODE_CHUNK_PAGES");  // tuning aid, read per call
-  if (forced != nullptr && atoi(forced) >= 8 && atoi(forced) % 8 == 0) return atoi(forced);
-  // ~2300 work items = three rounds of 3 workgroups x 256 CUs; every item pays ~2 us of fixed
-  // cost (locating its sequence, q, the cross-wave merge), so chunks should not be smaller than
-  // that buys.  One step of the MFMA kernel is 2 pages per wave, 8 per workgroup.
-  const int64_t cp = nnz_pages * h_kv / 2304;
-  int pow2 = 8;
-  while (pow2 < 128 && pow2 * 3 / 2 <= cp) pow2 *= 2;  // nearest power of two
-  return pow2;
-}
+constexpr size_t kArrivalBytes = 256 * 1024;  // the first bytes of the scratch buffer: arrival counters
 
 template <int D, int PS>
 static void launch_decode(const DecodeParams& p, int group, dim3 grid, hipStream_t stream) {
@@ -726,22 +678,24 @@ static void launch_decode(const DecodeParams& p, int group, dim3 grid, hipStream
 
 using namespace tvmkv;
 
-extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t* page_indptr,
-                                           const int32_t* page_values, const int32_t* length_info,
-                                           const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,
-                                           void* output, float* lse, int64_t rotary_mode, double rope_scale,
-                                           double rope_theta, double sm_scale, int32_t batch_size,
-                                           int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
-                                           int32_t d, int32_t page_size, int32_t sliding_window, void* stream) {
-  KV_API_BEGIN();
+// Body of the decode entry point.  lease(bytes) hands out the scratch memory of the call: arrival
+// counters in the first kArrivalBytes, partial states behind them.
+template <class Lease>
+static void decode_entry(Lease&& lease, const void* q, const void* pages, const int32_t* page_indptr, const int32_t* page_values,
+                         const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                         const int32_t* q_rope_position, void* output, float* lse, int64_t rotary_mode,
+                         double rope_scale, double rope_theta, double sm_scale, int32_t batch_size,
+                         int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv, int32_t d,
+                         int32_t page_size, int32_t sliding_window, void* stream) {
   KV_CHECK(batch_size >= 0 && nnz_pages >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_decode_paged_kv: bad shape";
   const bool ext = rotary_mode != 0 || sliding_window != 0;
   KV_UNSUPPORTED(page_size != 16) << "batch_decode_paged_kv: page_size " << page_size << " is not built (16)";
   KV_UNSUPPORTED(d != 64 && d != 128) << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 128)";
-  if (batch_size == 0) return TVMKV_OK;
+  if (batch_size == 0) return;
   KV_CHECK(q && pages && page_indptr && length_info && output && lse) << "batch_decode_paged_kv: NULL tensor";
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_decode_paged_kv: NULL page table";
+  hipStream_t s = as_stream(stream);
 
   const int gqa = h_q / h_kv;
   const bool mfma_shape = d == 128 && gqa <= 16;
@@ -751,10 +705,8 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
     // only (head_dim 128, GQA groups up to 16), and the vector kernel for the other shapes has GQA
     // groups 1, 2, 4, 8.  What neither covers runs as a paged prefill with one query per sequence:
     // one workgroup per (sequence, kv head), no split over the keys.
-    int32_t* q_indptr = reinterpret_cast<int32_t*>(
-        static_cast<char*>(get_workspace(kArrivalBytes + (static_cast<size_t>(batch_size) + 1) * sizeof(int32_t))) +
-        kArrivalBytes);
-    hipStream_t s = as_stream(stream);
+    const ScratchLease ws = lease(kArrivalBytes + (static_cast<size_t>(batch_size) + 1) * sizeof(int32_t));
+    int32_t* q_indptr = reinterpret_cast<int32_t*>(ws.ptr + kArrivalBytes);
     hipLaunchKernelGGL(iota_kernel, dim3((batch_size + 256) / 256), dim3(256), 0, s, q_indptr, batch_size + 1);
     KV_LAUNCH_CHECK();
     const int rc = tvmkv_batch_prefill_paged_kv(q, q_indptr, pages, page_indptr, page_values, length_info,
@@ -762,8 +714,8 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
                                                 rotary_mode, rope_scale, rope_theta, sm_scale, batch_size, batch_size,
                                                 nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window,
                                                 /*sliding_window_size=*/0, stream);
-    if (rc != TVMKV_OK) return rc;
-    return TVMKV_OK;
+    if (rc != TVMKV_OK) throw Error(rc, tvmkv_last_error());
+    return;
   }
 
   DecodeParams p;
@@ -783,36 +735,33 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
   p.batch_size = batch_size;
   p.h_q = h_q;
   p.h_kv = h_kv;
-  p.chunk_pages = pick_chunk_pages(nnz_pages, h_kv);
+  p.chunk_pages = decode_pick_chunk_pages(nnz_pages, h_kv);
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
   const int64_t slots = nnz_pages / p.chunk_pages + batch_size;
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many chunks";
   const size_t part_o_bytes = static_cast<size_t>(slots) * h_q * d * sizeof(float);
   const size_t part_ml_bytes = static_cast<size_t>(slots) * h_q * 2 * sizeof(float);
-  char* ws = static_cast<char*>(get_workspace(kArrivalBytes + part_o_bytes + part_ml_bytes));
-  p.part_o = reinterpret_cast<float*>(ws + kArrivalBytes);
-  p.part_ml = reinterpret_cast<float*>(ws + kArrivalBytes + part_o_bytes);
+  const ScratchLease ws = lease(kArrivalBytes + part_o_bytes + part_ml_bytes);
+  p.part_o = reinterpret_cast<float*>(ws.ptr + kArrivalBytes);
+  p.part_ml = reinterpret_cast<float*>(ws.ptr + kArrivalBytes + part_o_bytes);
   p.arrivals = nullptr;
+  p.epoch = ws.epoch;
 
   const dim3 grid(static_cast<unsigned>(slots), h_kv);
   const int group = h_q / h_kv;
-  hipStream_t s = as_stream(stream);
   if (d == 128 && group <= 16) {
     const int64_t num_items = slots * h_kv;
     KV_CHECK(num_items < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many work items";
     // One item per workgroup by default (measured a little faster than a resident-size grid
-    // striding over the items); TVMKV_DECODE_WGS_PER_CU=n caps the grid at n workgroups per CU.
-    static const char* wgs_env = getenv("TVMKV_DECODE_WGS_PER_CU");
+    // striding over the items); the option decode_wgs_per_cu = n caps the grid at n workgroups per CU.
+    const int64_t wgs_per_cu = option(kOptDecodeWgsPerCu);
     int64_t grid_x = num_items;
-    if (wgs_env != nullptr && atoi(wgs_env) > 0) {
-      grid_x = std::min<int64_t>(num_items, static_cast<int64_t>(compute_units()) * atoi(wgs_env));
-    }
+    if (wgs_per_cu > 0) grid_x = std::min<int64_t>(num_items, static_cast<int64_t>(compute_units()) * wgs_per_cu);
     // the chunk merge is done by the last workgroup of each (sequence, kv head) when the arrival
-    // counters fit their region; TVMKV_DECODE_SEPARATE_MERGE=1 keeps the second kernel (tuning aid)
-    const char* sep_env = getenv("TVMKV_DECODE_SEPARATE_MERGE");  // read per call: tests switch it
-    const bool fused = static_cast<size_t>(batch_size) * h_kv * sizeof(int) <= kArrivalBytes &&
-                       !(sep_env != nullptr && atoi(sep_env) != 0);
-    if (fused) p.arrivals = reinterpret_cast<int*>(ws);
+    // counters fit their region; the option decode_separate_merge keeps the second kernel
+    const bool fused = static_cast<size_t>(batch_size) * h_kv * sizeof(unsigned long long) <= kArrivalBytes &&
+                       option(kOptDecodeSeparateMerge) == 0;
+    if (fused) p.arrivals = reinterpret_cast<unsigned long long*>(ws.ptr);
     DecodeRopeDivisors div{};
     if (p.rotary) {
       KV_CHECK(k_rope_pos_offset && q_rope_position) << "batch_decode_paged_kv: inline RoPE needs the position arrays";
@@ -841,5 +790,45 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
     hipLaunchKernelGGL(decode_merge_kernel<64>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
   }
   KV_LAUNCH_CHECK();
+}
+
+extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t* page_indptr,
+                                           const int32_t* page_values, const int32_t* length_info,
+                                           const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,
+                                           void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                                           double rope_theta, double sm_scale, int32_t batch_size,
+                                           int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                                           int32_t d, int32_t page_size, int32_t sliding_window, void* stream) {
+  KV_API_BEGIN();
+  hipStream_t s = as_stream(stream);
+  decode_entry([&](size_t bytes) { return lease_scratch(kScratchDecode, s, bytes, kArrivalBytes); }, q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode,
+               rope_scale, rope_theta, sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d, page_size,
+               sliding_window, stream);
+  KV_API_END();
+}
+
+// Host view of the split: which chunk size a launch of these shapes uses, how many chunk slots its
+// grid has, and which (sequence, chunk) every slot resolves to (-1, -1 for a spare slot).
+extern "C" int tvmkv_decode_split_plan(const int32_t* page_indptr_host, int32_t batch_size, int64_t nnz_pages,
+                                       int32_t h_kv, int32_t* chunk_pages, int64_t* num_slots, int32_t* slot_seq,
+                                       int32_t* slot_chunk, int64_t slot_capacity) {
+  KV_API_BEGIN();
+  KV_CHECK(page_indptr_host && chunk_pages && num_slots && batch_size > 0 && h_kv > 0 && nnz_pages >= 0)
+      << "decode_split_plan: bad argument";
+  const int cp = decode_pick_chunk_pages(nnz_pages, h_kv);
+  const int64_t slots = nnz_pages / cp + batch_size;
+  *chunk_pages = cp;
+  *num_slots = slots;
+  if (slot_seq == nullptr || slot_chunk == nullptr) return TVMKV_OK;
+  KV_CHECK(slots <= slot_capacity) << "decode_split_plan: " << slots << " slots, room for " << slot_capacity;
+  for (int64_t slot = 0; slot < slots; ++slot) {
+    const int b = find_sequence(page_indptr_host, batch_size, cp, static_cast<int>(slot));
+    const int npages = page_indptr_host[b + 1] - page_indptr_host[b];
+    const int chunk = static_cast<int>(slot) - slot_begin(page_indptr_host, b, cp);
+    const int nchunks = (npages + cp - 1) / cp;
+    const bool in_use = chunk < nchunks;
+    slot_seq[slot] = in_use ? b : -1;
+    slot_chunk[slot] = in_use ? chunk : -1;
+  }
   KV_API_END();
 }

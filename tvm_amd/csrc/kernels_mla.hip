@@ -27,6 +27,8 @@
 #include <utility>
 
 #include "kernels_common.cuh"
+#include "runtime_support.h"
+#include "split_plan.h"
 
 namespace tvmkv {
 
@@ -62,14 +64,6 @@ struct MlaParams {
 // they would alternate with the real ones and leave half of the XCDs idle.)
 __device__ __forceinline__ int mla_tile_slot_begin(const int32_t* q_indptr, int b, int h_q) {
   return static_cast<int>((static_cast<int64_t>(q_indptr[b]) * h_q) / MLA_BM) + (h_q % MLA_BM != 0 ? b : 0);
-}
-
-// Split mode: sequence b owns the chunk slots [mla_chunk_slot_begin(b), mla_chunk_slot_begin(b+1)),
-// a function of the page table alone (so the grid can be sized from shapes: at most
-// floor(nnz_pages * page_size / chunk_tokens) + batch slots, every one of them in use), and its KV
-// tiles are divided evenly among them: about chunk_tokens tokens each.
-__device__ __forceinline__ int mla_chunk_slot_begin(const int32_t* page_indptr, int b, int page_size, int chunk_tokens) {
-  return static_cast<int>(static_cast<int64_t>(page_indptr[b]) * page_size / chunk_tokens) + b;
 }
 
 constexpr int MLA_WAVES = 4;    // wavefronts per workgroup, 32 rows each, one per SIMD
@@ -622,30 +616,6 @@ __global__ __launch_bounds__(DV / 4) void mla_merge_kernel(MlaParams p) {
   if (threadIdx.x == 0) p.lse[grow] = mx + fast_log2(denom);
 }
 
-struct MlaWorkspace {
-  void* ptr = nullptr;
-  size_t bytes = 0;
-};
-static MlaWorkspace g_mla_workspace[64];
-
-static void* mla_workspace(size_t bytes) {
-  int dev = 0;
-  HIP_CHECK(hipGetDevice(&dev));
-  KV_CHECK(dev >= 0 && dev < 64) << "device ordinal " << dev << " out of range";
-  MlaWorkspace& ws = g_mla_workspace[dev];
-  if (ws.bytes < bytes) {
-    if (ws.ptr) {
-      HIP_CHECK(hipDeviceSynchronize());
-      HIP_CHECK(hipFree(ws.ptr));
-      ws.ptr = nullptr;
-      ws.bytes = 0;
-    }
-    HIP_CHECK(hipMalloc(&ws.ptr, bytes + bytes / 2));
-    ws.bytes = bytes + bytes / 2;
-  }
-  return ws.ptr;
-}
-
 }  // namespace tvmkv
 
 using namespace tvmkv;
@@ -696,9 +666,7 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
     const int64_t room = cus / row_tiles - batch_size;
     int64_t ct = (tokens + room - 1) / room;
     ct = std::max<int64_t>(MLA_MIN_CHUNK, (ct + MLA_BN - 1) / MLA_BN * MLA_BN);
-    if (const char* e = getenv("TVMKV_MLA_CHUNK_TOKENS")) {  // tuning aid
-      if (atoi(e) >= MLA_BN) ct = atoi(e) / MLA_BN * MLA_BN;
-    }
+    if (option(kOptMlaChunkTokens) >= MLA_BN) ct = option(kOptMlaChunkTokens) / MLA_BN * MLA_BN;  // tuning aid
     const int64_t cslots = tokens / ct + batch_size;
     p.split = 1;
     p.chunk_tokens = static_cast<int>(ct);
@@ -706,7 +674,7 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
     grid = cslots * row_tiles;
     const size_t part_rows = static_cast<size_t>(cslots) * h_q;
     const size_t part_o_bytes = part_rows * DV * sizeof(float);
-    char* ws = static_cast<char*>(mla_workspace(part_o_bytes + part_rows * 2 * sizeof(float)));
+    char* ws = lease_scratch(kScratchMla, as_stream(stream), part_o_bytes + part_rows * 2 * sizeof(float), 0).ptr;
     p.part_o = reinterpret_cast<float*>(ws);
     p.part_ml = reinterpret_cast<float*>(ws + part_o_bytes);
   }

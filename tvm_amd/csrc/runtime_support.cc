@@ -1,0 +1,118 @@
+// Tuning options and the scratch-buffer pool of the split-KV launchers (see runtime_support.h).
+#include "runtime_support.h"
+
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "common.h"
+
+namespace tvmkv {
+
+namespace {
+
+struct OptionTable {
+  std::atomic<int64_t> value[kNumOptions];
+  OptionTable() {
+    static const char* const env_names[kNumOptions] = {"TVMKV_DECODE_CHUNK_PAGES", "TVMKV_DECODE_SEPARATE_MERGE",
+                                                       "TVMKV_DECODE_WGS_PER_CU", "TVMKV_MLA_CHUNK_TOKENS",
+                                                       "TVMKV_MLA_SEPARATE_MERGE"};
+    for (int i = 0; i < kNumOptions; ++i) {
+      const char* text = std::getenv(env_names[i]);  // once, when the library is loaded
+      value[i].store(text != nullptr ? std::atoll(text) : 0, std::memory_order_relaxed);
+    }
+  }
+};
+OptionTable g_options;
+
+const char* const kOptionNames[kNumOptions] = {"decode_chunk_pages", "decode_separate_merge", "decode_wgs_per_cu",
+                                               "mla_chunk_tokens", "mla_separate_merge"};
+
+struct Scratch {
+  char* ptr = nullptr;
+  size_t bytes = 0;
+  size_t counter_bytes = 0;
+  uint32_t epoch = 0;
+};
+std::mutex g_scratch_mutex;
+std::map<std::tuple<int, hipStream_t, int>, Scratch> g_scratch;
+
+}  // namespace
+
+int64_t option(Option id) { return g_options.value[id].load(std::memory_order_relaxed); }
+
+ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, size_t counter_bytes) {
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  Scratch& s = g_scratch[std::make_tuple(dev, stream, static_cast<int>(user))];
+  if (s.bytes < bytes || s.counter_bytes < counter_bytes) {
+    if (s.ptr != nullptr) {
+      // launches still queued on this stream read the old buffer; nobody else ever does
+      HIP_CHECK(hipStreamSynchronize(stream));
+      HIP_CHECK(hipFree(s.ptr));
+      s = Scratch{};
+    }
+    const size_t want = bytes + bytes / 2;
+    void* ptr = nullptr;
+    HIP_CHECK(hipMalloc(&ptr, want));
+    s.ptr = static_cast<char*>(ptr);
+    s.bytes = want;
+    s.counter_bytes = counter_bytes;
+    s.epoch = 0;
+    HIP_CHECK(hipMemsetAsync(s.ptr, 0, counter_bytes, stream));
+  }
+  if (++s.epoch == 0) {
+    // 2^32 launches on this buffer: start the epochs over from clean counters
+    HIP_CHECK(hipMemsetAsync(s.ptr, 0, s.counter_bytes, stream));
+    s.epoch = 1;
+  }
+  return ScratchLease{s.ptr, s.epoch};
+}
+
+// ~2300 work items = three rounds of 3 workgroups x 256 CUs; every item pays ~2 us of fixed cost
+// (locating its sequence, q, the cross-wave merge), so chunks should not be smaller than that buys.
+// One step of the matrix-core decode kernel is 2 pages per wave, 8 per workgroup.
+int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv) {
+  const int64_t forced = option(kOptDecodeChunkPages);
+  if (forced >= 8 && forced % 8 == 0) return static_cast<int>(forced);
+  const int64_t cp = nnz_pages * h_kv / 2304;
+  int pow2 = 8;
+  while (pow2 < 128 && pow2 * 3 / 2 <= cp) pow2 *= 2;  // nearest power of two
+  return pow2;
+}
+
+}  // namespace tvmkv
+
+extern "C" {
+
+int tvmkv_set_option(const char* name, int64_t value) {
+  KV_API_BEGIN();
+  KV_CHECK(name != nullptr) << "tvmkv_set_option: name is NULL";
+  for (int i = 0; i < tvmkv::kNumOptions; ++i) {
+    if (std::strcmp(name, tvmkv::kOptionNames[i]) == 0) {
+      tvmkv::g_options.value[i].store(value, std::memory_order_relaxed);
+      return TVMKV_OK;
+    }
+  }
+  KV_CHECK(false) << "tvmkv_set_option: unknown option \"" << name << "\"";
+  KV_API_END();
+}
+
+int tvmkv_get_option(const char* name, int64_t* value) {
+  KV_API_BEGIN();
+  KV_CHECK(name != nullptr && value != nullptr) << "tvmkv_get_option: NULL argument";
+  for (int i = 0; i < tvmkv::kNumOptions; ++i) {
+    if (std::strcmp(name, tvmkv::kOptionNames[i]) == 0) {
+      *value = tvmkv::option(static_cast<tvmkv::Option>(i));
+      return TVMKV_OK;
+    }
+  }
+  KV_CHECK(false) << "tvmkv_get_option: unknown option \"" << name << "\"";
+  KV_API_END();
+}
+
+}  // extern "C"
