@@ -81,6 +81,38 @@ def prefill_workload(batch=8, prefix_hi=4096, chunk_lo=128, chunk_hi=2048, seed=
                 last_page_len=np.where(prefix == 0, 0, (prefix - 1) % PS + 1).astype(np.int32), flops=flops)
 
 
+def make_prefill_step(torch, K, pw, gen, dev):
+    """The chunked-prefill step that this file times, on the workload `pw` of prefill_workload():
+    returns (step, tensors).  step(_) runs split + RoPE + append of the new K/V rows (one launch) and
+    causal attention over the cached prefix and the new chunk in one pass (one launch); `tensors`
+    holds every device array it reads and writes (the full-size parity test checks `out` / `lse`)."""
+    def i32(a):
+        return torch.tensor(np.asarray(a), dtype=torch.int32, device=dev)
+
+    n = int(pw["q_indptr"][-1])
+    t = dict(
+        pages=torch.randn((pw["pool_pages"], 2, HKV, PS, D), generator=gen, device=dev).to(torch.float16),
+        qkv=torch.randn((n, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16),
+        q=torch.empty((n, HQ, D), dtype=torch.float16, device=dev),
+        k=torch.empty((n, HKV, D), dtype=torch.float16, device=dev),
+        v=torch.empty((n, HKV, D), dtype=torch.float16, device=dev),
+        out=torch.empty((n, HQ, D), dtype=torch.float16, device=dev),
+        lse=torch.empty((n, HQ), dtype=torch.float32, device=dev),
+        q_indptr=i32(pw["q_indptr"]), page_indptr=i32(pw["page_indptr"]), page_values=i32(pw["page_values"]),
+        last_page_len=i32(pw["last_page_len"]),
+        q_rope_position=i32(np.concatenate([p + np.arange(c) for p, c in zip(pw["prefix"], pw["chunk"])])),
+        append_position_map=i32(pw["append_position_map"]))
+    sm_scale = D ** -0.5
+
+    def prefill_step(_):
+        K.fused_rope_append(t["qkv"], t["q_rope_position"], t["q"], t["k"], t["v"], 1, t["pages"],
+                            t["append_position_map"], 1.0, 1e4)
+        K.batch_prefill_cached_and_new_kv(t["q"], t["q_indptr"], t["k"], t["v"], t["pages"], t["page_indptr"],
+                                          t["page_values"], t["last_page_len"], t["out"], t["lse"], sm_scale)
+
+    return prefill_step, t
+
+
 # --------------------------------------------------------------------------------------------
 def time_region(torch, fn, iters):
     """Milliseconds per call of fn, by HIP events on the stream the kernels run on."""
@@ -131,19 +163,21 @@ def calibrate(num_bytes=2 << 30, iters=10, quiet=False):
     return out
 
 
-# HBM bytes per launch of the decode entry point on the default workload, from rocprofv3 counter runs
-# of this file (profiles/decode_mfma_kernel_cfg2_batched_decode.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
-# in KiB per dispatch of decode_mfma_kernel (it merges the chunks itself); the scales come from the plain copy
-# kernel of known size (profiles/stream_copy_kernel_2GiB_calibration.txt).  It is a property of the
-# workload, so it is only reported when the algorithmic bytes are those it was measured on.
+# HBM bytes per launch of the decode entry point, from rocprofv3 counter runs of this file
+# (profiles/decode_mfma_kernel_cfg2_batched_decode.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 in KiB per
+# dispatch of decode_mfma_kernel (it merges the chunks itself); the scales come from the plain copy
+# kernel of known size (profiles/stream_copy_kernel_2GiB_calibration.txt).  Measured on the default
+# workload (--steps 16 --warmup 3, 1 182 904 320 algorithmic bytes per launch) and kept as bytes of
+# traffic per algorithmic byte: the kernel reads every K/V row once whatever the context lengths are,
+# and the rest (q, outputs, split-KV partial states) scales with the same page tables, so the ratio
+# carries over to the page tables of any --steps / --warmup of this workload.
 TRAFFIC_MEASURED_ON_BYTES = 1182904320
 TRAFFIC_KIB = {"decode_mfma_kernel": (581061.0 * 2.0, 6219.8)}
+TRAFFIC_PER_ALGORITHMIC_BYTE = sum(r + w for r, w in TRAFFIC_KIB.values()) * 1024 / TRAFFIC_MEASURED_ON_BYTES
 
 
 def measured_traffic(algorithmic_bytes):
-    if algorithmic_bytes != TRAFFIC_MEASURED_ON_BYTES:
-        return None
-    return int(sum(r + w for r, w in TRAFFIC_KIB.values()) * 1024)
+    return int(round(TRAFFIC_PER_ALGORITHMIC_BYTE * algorithmic_bytes))
 
 
 def extras(torch, K, dev):
@@ -182,7 +216,7 @@ def extras(torch, K, dev):
     ms_two_kernels = time_region(torch, lambda i: K.batch_decode_paged_kv(*args), 10)
     tvm_amd.set_option("decode_separate_merge", 0)
     out["long_context_decode"] = {"workload": "configs[3]: 8 seqs, ctx U[32768,131072] seed 3, Hq64/Hkv8/D128, page 16",
-                                  "kv_tokens": int(ctx.sum()), "ms": round(ms, 4),
+                                  "kv_tokens": int(ctx.sum()), "algorithmic_bytes": int(nbytes), "ms": round(ms, 4),
                                   "ms_with_separate_merge_kernel": round(ms_two_kernels, 4),
                                   "GBps": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     del pages
@@ -280,9 +314,11 @@ def extras(torch, K, dev):
             pairs = float(np.sum(chunk * kv))
         flops = 2.0 * hq * (2 * dl + dr) * pairs  # QK^T over 576 features + PV over 512
         nbytes = float(kv.sum()) * (dl + dr) * 2 + n * hq * (2 * dl + dr) * 2
-        out[name] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+        out[name] = {"ms": round(ms, 4), "algorithmic_flops": flops, "algorithmic_bytes": int(nbytes),
+                     "tflops": round(flops / ms / 1e9, 1),
                      "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
-                     "GBps": round(nbytes / ms / 1e6, 1)}
+                     "GBps": round(nbytes / ms / 1e6, 1),
+                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
 
     def mla_prefill_step(name, prefix_len, chunk_len, nseq, seed):
         """A chunked-prefill step of an MLA layer as the reference composes it
@@ -320,7 +356,7 @@ def extras(torch, K, dev):
         step(0)
         ms = time_region(torch, step, 10)
         flops = float(hq) * nseq * (640.0 * chunk_len * (chunk_len + 1) / 2 + 2176.0 * chunk_len * prefix_len)
-        out[name] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+        out[name] = {"ms": round(ms, 4), "algorithmic_flops": flops, "tflops": round(flops / ms / 1e9, 1),
                      "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
                      "workload": f"configs[4] prefill step: {nseq} seqs, {chunk_len}-token chunk on a {prefix_len}-token "
                                  "prefix: ragged causal (192/128) + absorbed paged (576->512) + merge, three launches"}
@@ -342,9 +378,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (profiling runs)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the chunked-prefill leg (profiling runs)")
-    ap.add_argument("--extras", action="store_true",
-                    help="also time configs[3] (long-context decode) and configs[4] (MLA decode / prefill); "
-                         "reported under \"extras\", not part of the headline value")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip configs[3] (long-context decode), configs[4] (MLA decode / prefill) and the "
+                         "sliding-window / token-tree variants, which are otherwise reported under \"extras\" "
+                         "(not part of the headline value)")
+    ap.add_argument("--extras", action="store_true", help="accepted for compatibility: the extras run by default")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the plain 2 GiB streaming read and copy kernels (bandwidth calibration; "
                          "known-size dispatches for scaling rocprofv3 traffic counters)")
@@ -440,6 +478,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(gbps_decode, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps_decode / HBM_PEAK_GBPS, 4),
                      "traffic": measured_traffic(int(decode_bytes)),
+                     "traffic_per_algorithmic_byte": round(TRAFFIC_PER_ALGORITHMIC_BYTE, 4),
                      "kernel": "tvmkv_batch_decode_paged_kv (decode_mfma_kernel, chunk merge fused)",
                      "ms": round(ms_decode, 4), "algorithmic_bytes": int(decode_bytes)},
     }
@@ -447,24 +486,7 @@ def main():
     # ---- chunked prefill (configs[2]): ragged causal + paged non-causal + merge + append -------
     if not args.no_prefill:
         pw = prefill_workload()
-        n = int(pw["q_indptr"][-1])
-        ppages = torch.randn((pw["pool_pages"], 2, HKV, PS, D), generator=gen, device=dev).to(torch.float16)
-        pq = torch.randn((n, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16)
-        q2 = torch.empty((n, HQ, D), dtype=torch.float16, device=dev)
-        k2 = torch.empty((n, HKV, D), dtype=torch.float16, device=dev)
-        v2 = torch.empty((n, HKV, D), dtype=torch.float16, device=dev)
-        o1 = torch.empty((n, HQ, D), dtype=torch.float16, device=dev)
-        l1 = torch.empty((n, HQ), dtype=torch.float32, device=dev)
-        q_indptr, page_indptr = i32(pw["q_indptr"]), i32(pw["page_indptr"])
-        page_values, last = i32(pw["page_values"]), i32(pw["last_page_len"])
-        qpos = i32(np.concatenate([p + np.arange(c) for p, c in zip(pw["prefix"], pw["chunk"])]))
-        amap = i32(pw["append_position_map"])
-
-        def prefill_step(_):
-            # split + RoPE + append, then attention over the cached prefix and the new chunk in one pass
-            K.fused_rope_append(pq, qpos, q2, k2, v2, 1, ppages, amap, 1.0, 1e4)
-            K.batch_prefill_cached_and_new_kv(q2, q_indptr, k2, v2, ppages, page_indptr, page_values, last, o1, l1,
-                                              sm_scale)
+        prefill_step, _ = make_prefill_step(torch, K, pw, gen, dev)
 
         for _ in range(3):
             prefill_step(0)
@@ -560,7 +582,7 @@ def main():
                                                       f"{threads} threads, {par_s:.1f} s",
                                             "tokens_per_s": round(B * par_steps / par_s, 2)}
 
-    if args.extras:
+    if not args.no_extras:
         del pages, qkv
         torch.cuda.empty_cache()
         result["extras"] = extras(torch, K, dev)

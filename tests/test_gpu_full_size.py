@@ -155,6 +155,72 @@ def test_chunked_prefill_full_size_properties():
     assert_close(host(outc), np.broadcast_to(host(feat), outc.shape), atol=2e-3, rtol=2e-3, what="configs[2] constant V")
 
 
+def test_chunked_prefill_step_of_the_benchmark_full_size():
+    """configs[2] through exactly the two launches bench.py times (split + RoPE + append, then the
+    one-pass kernel over cached prefix and new chunk): against the three-kernel composition of the
+    reference (ragged causal + paged + merge) on every row, against the oracle on the cheapest
+    sequence (from the raw qkv: RoPE, self, cross, merge), the appended page slots bit for bit, and
+    constant values in, constant values out."""
+    pw = bench.prefill_workload()
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(1)
+    step, t = bench.make_prefill_step(torch, K, pw, gen, DEV)
+    hq, hkv, d, ps = bench.HQ, bench.HKV, bench.D, bench.PS
+    n = int(pw["q_indptr"][-1])
+    nb = len(pw["chunk"])
+    sm = d ** -0.5
+    pages_before = t["pages"].clone()
+    step(0)
+    out, lse = t["out"].clone(), t["lse"].clone()
+    # (1) the reference's composition on the same rotated q / k / v
+    z, zn = torch.zeros(nb, dtype=torch.int32, device=DEV), torch.zeros(n, dtype=torch.int32, device=DEV)
+    o1, o2 = torch.empty_like(out), torch.empty_like(out)
+    l1, l2 = torch.empty_like(lse), torch.empty_like(lse)
+    K.batch_prefill_ragged_kv(t["q"], t["q_indptr"], t["k"], t["v"], t["q_indptr"], zn, z, o1, l1, 1, 0, 1.0, 1e4, sm)
+    K.batch_prefill_paged_kv(t["q"], t["q_indptr"], t["pages"], t["page_indptr"], t["page_values"], t["last_page_len"],
+                             z, zn, o2, l2, 0, 0, 1.0, 1e4, sm)
+    K.merge_state_inplace(o1, l1, o2, l2)
+    assert_close(host(out), host(o1), atol=2e-3, rtol=2e-3, what="one pass vs ragged + paged + merge, out")
+    assert_close(host(lse), host(l1), atol=1e-3, rtol=1e-5, what="one pass vs ragged + paged + merge, lse")
+    # (2) the cheapest sequence from the raw inputs through the oracle
+    b = int(np.argmin(pw["chunk"] * (pw["chunk"] + pw["prefix"])))
+    s, e = int(pw["q_indptr"][b]), int(pw["q_indptr"][b + 1])
+    lo, hi = int(pw["page_indptr"][b]), int(pw["page_indptr"][b + 1])
+    c = e - s
+    pos = np.arange(c, dtype=np.int32) + int(pw["prefix"][b])
+    qh, kh, vh = np.zeros((c, hq, d), np.float16), np.zeros((c, hkv, d), np.float16), np.zeros((c, hkv, d), np.float16)
+    ok.fused_rope(host(t["qkv"][s:e]), pos, qh, kh, vh, 1)
+    hp = host(pages_before[torch.tensor(pw["page_values"][lo:hi], dtype=torch.int64, device=DEV)]) if hi > lo else \
+        np.zeros((1, 2, hkv, ps, d), np.float16)
+    eo1, el1 = np.zeros((c, hq, d), np.float16), np.zeros((c, hq), np.float32)
+    eo2, el2 = np.zeros_like(eo1), np.zeros_like(el1)
+    ind = np.array([0, c], np.int32)
+    z1, zc = np.zeros(1, np.int32), np.zeros(c, np.int32)
+    ok.prefill_ragged(qh, ind, kh, vh, ind, zc, z1, eo1, el1, 1, 0, 1.0, 1e4, sm)
+    if hi > lo:
+        ok.prefill_paged(qh, ind, hp, np.array([0, hi - lo], np.int32), np.arange(hi - lo, dtype=np.int32),
+                         pw["last_page_len"][b:b + 1], z1, zc, eo2, el2, 0, 0, 1.0, 1e4, sm)
+        ok.merge_state_inplace(eo1, el1, eo2, el2)
+    assert_close(host(out[s:e]), eo1, what=f"configs[2] one pass, seq {b} out vs oracle")
+    assert_close(host(lse[s:e]), el1, atol=2e-3, rtol=1e-4, what=f"configs[2] one pass, seq {b} lse vs oracle")
+    # (3) the appended slots hold the rotated k and the v rows, every other slot is untouched
+    slots = torch.tensor(pw["append_position_map"], dtype=torch.int64, device=DEV)
+    flat = t["pages"].permute(0, 3, 1, 2, 4).reshape(-1, 2, hkv, d)  # (slot, k|v, head, d)
+    assert torch.equal(flat[slots, 0], t["k"]) and torch.equal(flat[slots, 1], t["v"])
+    untouched = torch.ones(flat.shape[0], dtype=torch.bool, device=DEV)
+    untouched[slots] = False
+    flat_before = pages_before.permute(0, 3, 1, 2, 4).reshape(-1, 2, hkv, d)
+    assert torch.equal(flat[untouched], flat_before[untouched])
+    # (4) constant values (cached prefix and new tokens alike) come back unchanged; lse does not move
+    feat = (torch.arange(d, device=DEV, dtype=torch.float32) / 64 - 1).to(F16)
+    t["pages"][:, 1] = feat
+    t["qkv"][:, hq + hkv:] = feat
+    step(0)
+    assert_close(host(t["lse"]), host(lse), atol=1e-4, rtol=1e-6, what="lse must not depend on the values")
+    assert_close(host(t["out"]), np.broadcast_to(host(feat), t["out"].shape), atol=2e-3, rtol=2e-3,
+                 what="configs[2] one pass, constant V")
+
+
 def test_mla_full_size_properties():
     """configs[4]: decode batch 32 (split-KV route) and a 1024-token chunk on a 2048-token prefix."""
     hq, dl, dr, ps = 128, 512, 64, 64

@@ -485,3 +485,48 @@ def test_mla_absorbed_equals_expanded_definition():
     got = np.einsum("qhl,lhv->qhv", out.astype(np.float64), w_uv)
     assert_close(got, eo, atol=1e-2, rtol=1e-2, what="mla out")
     assert_close(lse, el, atol=2e-2, rtol=1e-3, what="mla lse")
+
+
+def test_mla_absorbed_causal_equals_expanded_definition():
+    """The causal form of the paged MLA kernel (the chunk's own rows are in the pages already,
+    python/tvm/relax/frontend/nn/llm/_prefill_kernels.py:1021-1031): query row r of nq sees the first
+    kv_len - nq + r + 1 cached rows; against the expanded definition with the causal mask, two
+    sequences of different lengths, one of them with as many queries as cached rows."""
+    rng = np.random.default_rng(15)
+    h, d_lat, d_rope, d_nope, d_v, ps = 4, 32, 8, 16, 12, 8
+    kv_lens, nqs = [21, 6], [5, 6]
+    w_kv = (rng.standard_normal((d_lat, h * (d_nope + d_v))) * 0.3).astype(np.float64)
+    w = w_kv.reshape(d_lat, h, d_nope + d_v)
+    w_uk, w_uv = w[..., :d_nope], w[..., d_nope:]
+    pages = np.zeros((6, ps, d_lat + d_rope), F16)
+    page_ids = np.array([3, 0, 4, 5], np.int32)  # 3 pages for sequence 0, 1 for sequence 1
+    page_indptr = np.array([0, 3, 4], np.int32)
+    latents, q_abs_all, qs = [], [], []
+    for b, (n, nq) in enumerate(zip(kv_lens, nqs)):
+        latent = (rng.standard_normal((n, d_lat + d_rope)) * 0.5).astype(F16)
+        ids = page_ids[page_indptr[b]:page_indptr[b + 1]]
+        slots = np.array([ids[t // ps] * ps + t % ps for t in range(n)], np.int32)
+        ok.transpose_append_mla(pages, latent, slots)
+        q = (rng.standard_normal((nq, h, d_nope + d_rope)) * 0.5).astype(np.float64)
+        q_abs_all.append(np.concatenate([np.einsum("qhn,lhn->qhl", q[..., :d_nope], w_uk), q[..., d_nope:]], axis=-1))
+        latents.append(latent)
+        qs.append(q)
+    q_abs = np.concatenate(q_abs_all).astype(F16)
+    total = sum(nqs)
+    out, lse = np.zeros((total, h, d_lat), F16), np.zeros((total, h), np.float32)
+    sm = (d_nope + d_rope) ** -0.5
+    last = np.array([(n - 1) % ps + 1 for n in kv_lens], np.int32)
+    ok.prefill_paged_mla(q_abs, np.array([0, nqs[0], total], np.int32), pages, page_indptr, page_ids, last, out, lse,
+                         1, sm, d_latent=d_lat)
+    cursor = 0
+    for b, nq in enumerate(nqs):
+        k_full, v_full = cf.mla_expand(latents[b], w_kv, h, d_nope, d_v)
+        eo, el = cf.attention(qs[b], k_full, v_full, sm, causal=True)
+        got = np.einsum("qhl,lhv->qhv", out[cursor:cursor + nq].astype(np.float64), w_uv)
+        assert_close(got, eo, atol=1e-2, rtol=1e-2, what=f"causal mla out, seq {b}")
+        assert_close(lse[cursor:cursor + nq], el, atol=2e-2, rtol=1e-3, what=f"causal mla lse, seq {b}")
+        cursor += nq
+    # the first query row of sequence 1 sees exactly one cached row: its value comes back
+    first = out[nqs[0]].astype(np.float64)
+    assert_close(first, np.broadcast_to(latents[1][0, :d_lat].astype(np.float64), first.shape), atol=2e-3, rtol=2e-3,
+                 what="a row that sees one key returns that key's latent")
