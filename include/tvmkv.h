@@ -180,6 +180,25 @@ int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t*
                                 int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
                                 int32_t d, int32_t page_size, int32_t sliding_window, void* stream);
 
+/* tvmkv_batch_decode_paged_kv for callers that cannot allocate.  It has no counterpart in the
+ * reference; it is for code under HIP graph capture, tight serving loops and harnesses that
+ * forbid hipMalloc.  Arguments and results as tvmkv_batch_decode_paged_kv.  Its scratch memory
+ * (arrival counters and split-KV partial states) is an array of 24 MiB built into the library, one
+ * per device, held until the process ends; the call makes no hipMalloc / hipFree and returns
+ * TVMKV_EINVAL with a message when the shapes need more: 256 KiB + (nnz_pages / chunk_pages +
+ * batch_size) * h_q * (head_dim + 2) * 4 bytes, chunk_pages as tvmkv_decode_split_plan reports
+ * (configs of 64 x 8k-token and 8 x 128k-token sequences need 6 and 11 MiB).  All calls on a device
+ * share the array: calls that overlap on one device (different streams) race, stream-ordered
+ * calls do not. */
+int tvmkv_batch_decode_paged_kv_noalloc(const void* q, const void* pages, const int32_t* page_indptr,
+                                        const int32_t* page_values, const int32_t* length_info,
+                                        const int32_t* k_rope_pos_offset,
+                                        const int32_t* q_rope_position, void* output, float* lse,
+                                        int64_t rotary_mode, double rope_scale, double rope_theta,
+                                        double sm_scale, int32_t batch_size, int64_t nnz_pages,
+                                        int64_t num_pages, int32_t h_q, int32_t h_kv, int32_t d,
+                                        int32_t page_size, int32_t sliding_window, void* stream);
+
 /* Slot 21 ragged prefill with a token-tree mask -- replaces `batch_tree_attn`
  * (python/tvm/relax/frontend/nn/llm/tree_attn.py:264-603; llvm form :68-259), calling convention
  * attn_backend.h:669-672:

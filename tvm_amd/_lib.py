@@ -37,6 +37,8 @@ SIGNATURES = {
                                                             c_i32, c_vp],
     "tvmkv_batch_decode_paged_kv": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32, c_i32,
                                                  c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_batch_decode_paged_kv_noalloc": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32,
+                                                         c_i32, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_tree_attn": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_tree_attn_paged_kv": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_vp, c_vp, c_i32, c_i64, c_i64, c_i64,
                                                c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],

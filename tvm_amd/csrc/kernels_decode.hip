@@ -27,6 +27,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
+#include <mutex>
 
 #include "kernels_common.cuh"
 #include "runtime_support.h"
@@ -678,6 +679,38 @@ static void launch_decode(const DecodeParams& p, int group, dim3 grid, hipStream
 
 using namespace tvmkv;
 
+// ---- scratch memory of the entry point that allocates nothing --------------------------------
+// One array per device that loads this library, held until the process ends: arrival counters, then
+// the partial states.  The name below is a host-side handle of the symbol, not a device address:
+// host code only ever uses the address hipGetSymbolAddress returns for the current device.
+constexpr size_t kStaticScratchBytes = 24u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+struct StaticScratch {
+  char* ptr = nullptr;   // device address of `scratch` on this device
+  uint32_t epoch = 0;
+};
+static StaticScratch g_static_scratch[64];
+static std::mutex g_static_scratch_mutex;
+
+static ScratchLease lease_static_scratch(size_t bytes) {
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  KV_CHECK(dev >= 0 && dev < 64) << "device ordinal " << dev << " out of range";
+  KV_CHECK(bytes <= kStaticScratchBytes)
+      << "batch_decode_paged_kv_noalloc: the call needs " << bytes << " bytes of scratch memory, the built-in "
+      << "buffer has " << kStaticScratchBytes << "; use tvmkv_batch_decode_paged_kv for this shape";
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  StaticScratch& s = g_static_scratch[dev];
+  if (s.ptr == nullptr) {
+    void* ptr = nullptr;
+    HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    s.ptr = static_cast<char*>(ptr);  // device memory of a loaded code object starts out zeroed
+  }
+  KV_CHECK(s.epoch != 0xffffffffu) << "batch_decode_paged_kv_noalloc: 2^32 calls on this device; counters exhausted";
+  return ScratchLease{s.ptr, ++s.epoch};
+}
+
 // Body of the decode entry point.  lease(bytes) hands out the scratch memory of the call: arrival
 // counters in the first kArrivalBytes, partial states behind them.
 template <class Lease>
@@ -804,6 +837,25 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
   decode_entry([&](size_t bytes) { return lease_scratch(kScratchDecode, s, bytes, kArrivalBytes); }, q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode,
                rope_scale, rope_theta, sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d, page_size,
                sliding_window, stream);
+  KV_API_END();
+}
+
+// The same entry point for callers that must not allocate (code under HIP graph capture, serving
+// loops and harnesses that forbid hipMalloc): scratch memory is the built-in per-device array, and a
+// call that needs more than it holds is refused.  Every call on a device shares that array, so calls
+// that overlap on one device (two streams) race; stream-ordered calls do not.
+extern "C" int tvmkv_batch_decode_paged_kv_noalloc(const void* q, const void* pages, const int32_t* page_indptr,
+                                                   const int32_t* page_values, const int32_t* length_info,
+                                                   const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,
+                                                   void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                                                   double rope_theta, double sm_scale, int32_t batch_size,
+                                                   int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                                                   int32_t d, int32_t page_size, int32_t sliding_window,
+                                                   void* stream) {
+  KV_API_BEGIN();
+  decode_entry([&](size_t bytes) { return lease_static_scratch(bytes); }, q, pages, page_indptr, page_values,
+               length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode, rope_scale, rope_theta,
+               sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window, stream);
   KV_API_END();
 }
 

@@ -116,11 +116,14 @@ def batch_prefill_cached_and_new_kv(q, q_indptr, k, v, pages, page_indptr, page_
 
 
 def batch_decode_paged_kv(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position,
-                          output, lse, rotary_mode, rope_scale, rope_theta, sm_scale):
+                          output, lse, rotary_mode, rope_scale, rope_theta, sm_scale, noalloc=False):
+    """noalloc=True calls the entry point that takes its scratch memory from the library's built-in
+    per-device array instead of allocating (tvmkv_batch_decode_paged_kv_noalloc)."""
     _f16(q, pages, output)
     _i32(page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position)
     num_pages, _, hkv, ps, d = pages.shape
-    check(lib().tvmkv_batch_decode_paged_kv(
+    entry = lib().tvmkv_batch_decode_paged_kv_noalloc if noalloc else lib().tvmkv_batch_decode_paged_kv
+    check(entry(
         _p(q), _p(pages), _p(page_indptr), _p(page_values), _p(length_info), _p(k_rope_pos_offset),
         _p(q_rope_position), _p(output), _p(lse), int(rotary_mode), float(rope_scale), float(rope_theta),
         float(sm_scale), q.shape[0], page_values.shape[0], num_pages, q.shape[1], hkv, d, ps,
