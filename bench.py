@@ -83,9 +83,11 @@ def prefill_workload(batch=8, prefix_hi=4096, chunk_lo=128, chunk_hi=2048, seed=
 
 def make_prefill_step(torch, K, pw, gen, dev):
     """The chunked-prefill step that this file times, on the workload `pw` of prefill_workload():
-    returns (step, tensors).  step(_) runs split + RoPE + append of the new K/V rows (one launch) and
-    causal attention over the cached prefix and the new chunk in one pass (one launch); `tensors`
-    holds every device array it reads and writes (the full-size parity test checks `out` / `lse`)."""
+    returns (step, tensors).  step(_) runs RoPE of k and the append of the new K/V rows (one launch) and
+    causal attention over the cached prefix and the new chunk in one pass, with the queries read from
+    the fused qkv tensor and rotated inside the kernel (one launch) -- what the cache object runs for
+    such a step; `tensors` holds every device array it reads and writes (the full-size parity test
+    checks `out` / `lse`)."""
     def i32(a):
         return torch.tensor(np.asarray(a), dtype=torch.int32, device=dev)
 
@@ -105,10 +107,11 @@ def make_prefill_step(torch, K, pw, gen, dev):
     sm_scale = D ** -0.5
 
     def prefill_step(_):
-        K.fused_rope_append(t["qkv"], t["q_rope_position"], t["q"], t["k"], t["v"], 1, t["pages"],
+        K.fused_rope_append(t["qkv"], t["q_rope_position"], None, t["k"], t["v"], 1, t["pages"],
                             t["append_position_map"], 1.0, 1e4)
-        K.batch_prefill_cached_and_new_kv(t["q"], t["q_indptr"], t["k"], t["v"], t["pages"], t["page_indptr"],
-                                          t["page_values"], t["last_page_len"], t["out"], t["lse"], sm_scale)
+        K.batch_prefill_cached_and_new_kv_fused_q(t["qkv"], t["q_rope_position"], 1, 1.0, 1e4, t["q_indptr"], t["k"],
+                                                  t["v"], t["pages"], t["page_indptr"], t["page_values"],
+                                                  t["last_page_len"], t["out"], t["lse"], sm_scale)
 
     return prefill_step, t
 
@@ -493,7 +496,7 @@ def main():
         ms_prefill = time_region(torch, prefill_step, 10)
         tflops = pw["flops"] / (ms_prefill * 1e-3) / 1e12
         result["prefill"] = {"workload": "configs[2]: chunked causal prefill, 8 seqs, prefix U[0,4096], chunk "
-                                         "U[128,2048] seed 2 (split+RoPE+append in one launch; causal attention over the new chunk and attention over the cached prefix in one pass)",
+                                         "U[128,2048] seed 2 (RoPE of k + append of the new K/V rows in one launch; causal attention over the new chunk and attention over the cached prefix in one pass that rotates q itself)",
                              "tflops": round(tflops, 2), "ms": round(ms_prefill, 4),
                              "algorithmic_flops": pw["flops"],
                              "frac_of_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}

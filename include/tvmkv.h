@@ -75,6 +75,9 @@ int tvmkv_fused_rope_append(const void* qkv, const int32_t* position_map, void* 
                             int32_t head_dim, int64_t num_pages, int32_t page_size, double rope_scale,
                             double rope_theta, void* stream);
 
+/* (q may be NULL in tvmkv_fused_rope_append: the q rows are then not written; the caller hands the
+ * fused qkv tensor to tvmkv_batch_prefill_cached_and_new_kv_fused_q, which rotates them itself.) */
+
 /* Slot 13 `f_transpose_append_mha` -- replaces `tir_kv_cache_transpose_append`
  * (python/tvm/relax/frontend/nn/llm/_page_kernels.py:40-74), called at paged_kv_cache.cc:1371
  * as (pages, k_data, v_data, position_map).  pages (num_pages, 2, num_kv_heads, page_size,
@@ -160,6 +163,24 @@ int tvmkv_batch_prefill_cached_and_new_kv(const void* q, const int32_t* q_indptr
                                           double sm_scale, int32_t batch_size, int64_t total_q,
                                           int64_t nnz_pages, int64_t num_pages, int32_t h_q,
                                           int32_t h_kv, int32_t d, int32_t page_size, void* stream);
+
+/* The same pass with the queries taken from the fused qkv tensor of the step (rows of
+ * (h_q + 2*h_kv) * d elements whose first h_q heads are q), rotated inside the kernel at
+ * q_rope_position[token] when apply_rope != 0 (rotate-half RoPE in fp32, rounded once to fp16, as
+ * slot 24 does it): together with tvmkv_fused_rope_append(q = NULL) a chunked-prefill step never
+ * writes the rotated q rows to memory or reads them back.  k, v: the rotated k and the v rows of the
+ * new tokens, as tvmkv_fused_rope_append leaves them. */
+int tvmkv_batch_prefill_cached_and_new_kv_fused_q(const void* qkv, const int32_t* q_rope_position,
+                                                  int64_t apply_rope, double rope_scale,
+                                                  double rope_theta, const int32_t* q_indptr,
+                                                  const void* k, const void* v, const void* pages,
+                                                  const int32_t* page_indptr,
+                                                  const int32_t* page_values,
+                                                  const int32_t* last_page_len, void* output,
+                                                  float* lse, double sm_scale, int32_t batch_size,
+                                                  int64_t total_q, int64_t nnz_pages, int64_t num_pages,
+                                                  int32_t h_q, int32_t h_kv, int32_t d,
+                                                  int32_t page_size, void* stream);
 
 /* Slots 17/19 paged decode -- replaces `batch_decode_paged_kv`
  * (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:181-411; llvm form :49-178), calling

@@ -611,6 +611,53 @@ def test_prefill_cached_and_new_in_one_pass(hq, hkv, d):
     assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="one-pass chunked prefill lse")
 
 
+@pytest.mark.parametrize("apply_rope", [1, 0])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+def test_prefill_one_pass_with_queries_from_the_fused_qkv(hq, hkv, d, apply_rope):
+    """The step of the cache object for a chunked prefill: k rotated and appended without writing q
+    (fused_rope_append with q = None), then the one-pass kernel that reads q from qkv and rotates it
+    itself.  Against the oracle from the raw qkv (fused_rope, ragged + paged + merge), with positions
+    that continue each sequence's prefix, a scaled position and a theta other than the default; the
+    appended slots against the k / v rows bit for bit."""
+    rng = np.random.default_rng(45)
+    prefix = [0, 63, 200, 700, 16]
+    chunk = [130, 1, 33, 40, 129]
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, prefix, 512, hkv, 16, d)
+    n = sum(chunk)
+    ind = np.concatenate([[0], np.cumsum(chunk)]).astype(np.int32)
+    qkv = rng.standard_normal((n, hq + 2 * hkv, d)).astype(F16)
+    pos = np.concatenate([p0 + np.arange(c) for p0, c in zip(prefix, chunk)]).astype(np.int32)
+    scale, theta = 0.5, 5e5
+    # free slots for the new rows: pages beyond the ones the prefixes use
+    used = set(int(x) for x in pvalues)
+    free = [pg for pg in range(512) if pg not in used]
+    slots = np.array([free[i // 16] * 16 + i % 16 for i in range(n)], np.int32)
+    q, k, v = np.zeros((n, hq, d), F16), np.zeros((n, hkv, d), F16), np.zeros((n, hkv, d), F16)
+    ok.fused_rope(qkv, pos, q, k, v, apply_rope, theta=theta, scale=scale)
+    zq, zb = np.zeros(n, np.int32), np.zeros(len(prefix), np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    to, tl = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    ok.prefill_ragged(q, ind, k, v, ind, zq, zb, eo, el, 1, 0, 1.0, 1e4, d ** -0.5)
+    ok.prefill_paged(q, ind, pages, pindptr, pvalues, last, zb, zq, to, tl, 0, 0, 1.0, 1e4, d ** -0.5)
+    ok.merge_state_inplace(eo, el, to, tl)
+    gp, gqkv = dev(pages), dev(qkv)
+    gk = torch.zeros((n, hkv, d), dtype=torch.float16, device=DEV)
+    gv = torch.zeros_like(gk)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.fused_rope_append(gqkv, i32(pos), None, gk, gv, apply_rope, gp, i32(slots), scale, theta)
+    K.batch_prefill_cached_and_new_kv_fused_q(gqkv, i32(pos), apply_rope, scale, theta, i32(ind), gk, gv, gp,
+                                              i32(pindptr), i32(pvalues), i32(last), go, gl, d ** -0.5)
+    assert_close(host(go), eo, what="one-pass chunked prefill with fused q, out")
+    assert_close(host(gl), el, atol=4e-3, rtol=1e-4, what="one-pass chunked prefill with fused q, lse")
+    assert np.array_equal(host(gv), v)
+    assert_close(host(gk), k, atol=2e-3, rtol=2e-3, what="rotated k")
+    flat = gp.permute(0, 3, 1, 2, 4).reshape(-1, 2, hkv, d)
+    sl = torch.tensor(slots, dtype=torch.int64, device=DEV)
+    assert torch.equal(flat[sl, 0], gk) and torch.equal(flat[sl, 1], gv)
+    assert torch.equal(gqkv, dev(qkv)), "qkv must be left alone"
+
+
 def test_measurement_utilities():
     """The calibration kernels of the benchmark: the copy copies, the reads leave their input alone,
     and the MFMA loop adds up what its instruction count says (integers in fp32, so exactly)."""

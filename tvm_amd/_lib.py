@@ -35,6 +35,8 @@ SIGNATURES = {
                                                          c_i64, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_prefill_cached_and_new_kv": [c_vp] * 10 + [c_f64, c_i32, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32,
                                                             c_i32, c_vp],
+    "tvmkv_batch_prefill_cached_and_new_kv_fused_q": [c_vp, c_vp, c_i64, c_f64, c_f64] + [c_vp] * 9 + [
+        c_f64, c_i32, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_decode_paged_kv": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32, c_i32,
                                                  c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_decode_paged_kv_noalloc": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32,

@@ -52,7 +52,9 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
     }
     __syncthreads();
   }
-  for (int task = threadIdx.x; task < fused_heads * kThreadsPerHead; task += 256) {
+  // q == NULL: the q rows are left alone (an attention kernel that reads them from qkv rotates them itself)
+  const int first_task = q == nullptr ? num_q_heads * kThreadsPerHead : 0;
+  for (int task = first_task + threadIdx.x; task < fused_heads * kThreadsPerHead; task += 256) {
     const int c = task % kThreadsPerHead;
     const int h = task / kThreadsPerHead;
     const half_t* src = qkv + (s * fused_heads + h) * D + c * 8;
@@ -336,8 +338,8 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
   KV_UNSUPPORTED(head_dim != 64 && head_dim != 128 && head_dim != 256)
       << "fused_rope: head_dim " << head_dim << " is not built (64, 128, 256)";
   if (seq_len == 0) return TVMKV_OK;
-  KV_CHECK(qkv && position_map && q && k && v) << "fused_rope: NULL tensor";
   const bool append = pages != nullptr;
+  KV_CHECK(qkv && position_map && (q || append) && k && v) << "fused_rope: NULL tensor";
   if (append) {
     KV_CHECK(append_position_map != nullptr && page_size > 0) << "fused_rope_append: NULL position map or bad page size";
     KV_CHECK(num_pages * page_size <= INT32_MAX) << "fused_rope_append: slot ids do not fit int32";

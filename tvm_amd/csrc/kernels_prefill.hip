@@ -29,74 +29,9 @@
 #include <cmath>
 #include <type_traits>
 
-#include "kernels_common.cuh"
+#include "prefill_common.cuh"
 
 namespace tvmkv {
-
-constexpr int NW = 4;        // wavefronts per workgroup, 32 rows each
-constexpr int BM = NW * 32;  // rows per workgroup
-constexpr int RPW = 64 / NW; // token rows of a tile copied by each wave
-constexpr int BN = 64;   // kv tokens per tile
-
-struct PrefillParams {
-  const half_t* q;
-  const int32_t* q_indptr;
-  const half_t* k;  // ragged
-  const half_t* v;
-  const int32_t* kv_indptr;
-  const half_t* pages;  // paged
-  const int32_t* page_indptr;
-  const int32_t* page_values;
-  const int32_t* last_page_len;
-  half_t* output;
-  float* lse;
-  int batch_size;
-  int h_q;
-  int h_kv;
-  int group;
-  int causal;
-  float scale_log2;
-  // extended form (prefill_kernel<..., EXT = true>): sliding-window cache, per-layer sliding-window
-  // mask, inline RoPE
-  const int32_t* window_offset;      // paged, (B): physical index of the first token of the window, or NULL
-  const int32_t* sink_size;          // paged, (B): attention-sink tokens kept at the front, or NULL
-  int layer_window;                  // > 0 with causal: row r sees only the last layer_window - r - 1 keys
-  const int32_t* q_rope_position;    // (total_q) position of each query token (inline RoPE)
-  const int32_t* k_rope_pos_offset;  // (B) position of logical key 0 (inline RoPE)
-  int rotary;
-  float rope_scale;
-  // token-tree mask (python/tvm/relax/frontend/nn/llm/tree_attn.py:48-65), or NULL
-  const int32_t* tree_indptr;  // (B + 1) first tree node of each sequence
-  const int32_t* tree_order;   // (nodes, 2): pre-order number of the node, end of its subtree's range
-  int k_pos_from_q;            // ragged tree attention under inline RoPE: key t sits at q_rope_position[t]
-  // != 0: output / lse already hold an attention state of the same rows, and this kernel's state is
-  // merged into it (the arithmetic of merge_state_inplace) instead of overwriting it
-  int merge_into;
-};
-
-// theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
-struct PrefillRopeDivisors {
-  float v[64];
-};
-
-__device__ __forceinline__ int tile_slot_begin(const int32_t* q_indptr, int b, int group) {
-  return static_cast<int>((static_cast<int64_t>(q_indptr[b]) * group) / BM) + b;
-}
-
-// LDS image of a tile of BN token rows x W features (W = 64 or 128), pieces of 8 features.
-// Piece c of row r is kept at piece position c ^ swz(r).
-//  * K is read as MFMA A-fragments with ds_read_b128, 16 lanes = 16 consecutive rows at the same
-//    piece: swz spreads 16 consecutive rows over the 16 piece positions of a 256-byte bank line.
-//  * V is read with ds_read_b64_tr_b16, 32 lanes = 4 consecutive rows x 64 bytes: swz moves the 4
-//    rows to the 4 different 64-byte quarters of the bank line.
-template <int W>
-__device__ __forceinline__ int k_swizzle(int row) {
-  return W == 128 ? (row & 15) : ((row >> 1) & 7);
-}
-template <int W>
-__device__ __forceinline__ int v_swizzle(int row) {
-  return W == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
-}
 
 // Pipeline depth: as many stages as fit next to a second workgroup (NW = 4) or alone (NW = 8).
 constexpr int prefill_stages(int dqk, int dv) {
@@ -126,7 +61,6 @@ constexpr size_t prefill_lds_bytes(int dqk, int dv) {
 // cached tokens of the page pool, all visible, followed by the k / v rows of the call under the
 // causal mask -- a chunked-prefill step in one pass, on one key axis whose paged part is padded to
 // a whole number of tiles (the padding is masked like the end of a sequence).
-constexpr int kRagged = 0, kPaged = 1, kBoth = 2;
 template <int DQK, int DV, int SRC, int PS, bool EXT>
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
   constexpr bool PAGED = SRC == kPaged, BOTH = SRC == kBoth;
@@ -230,7 +164,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   // number of logical keys -> physical end of the tokens that hold them
   auto to_phys = [&](int n) { return (!EXT || n <= sink) ? n : n - sink + win_lo; };
   __shared__ float div_lds[64];
-  if (EXT && p.rotary) {
+  const bool q_rope = (EXT && p.rotary) || (BOTH && p.q_inline_rope != 0);  // uniform over the launch
+  if (q_rope) {
     if (tid < DQK / 2) div_lds[tid] = div.v[tid];
     __syncthreads();
   }
@@ -273,10 +208,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
 
   half8_t qf[KS];
   {
-    const half_t* qrow = p.q + (static_cast<int64_t>(q_start + my_pos) * p.h_q + my_head) * DQK + half * 8;
+    const int64_t q_token_stride = p.q_token_stride != 0 ? p.q_token_stride : static_cast<int64_t>(p.h_q) * DQK;
+    const half_t* qrow = p.q + static_cast<int64_t>(q_start + my_pos) * q_token_stride + my_head * DQK + half * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[ks] = row_valid ? ld16(qrow + ks * 16).h8 : zero16().h8;
-    if (EXT && p.rotary && row_valid) {
+    if (q_rope && row_valid) {
       const float q_pos = static_cast<float>(p.q_rope_position[q_start + my_pos]) * p.rope_scale;
 #pragma unroll
       for (int ks = 0; ks < KS / 2; ++ks) rope_pair(qf[ks], qf[ks + KS / 2], q_pos, div_lds + ks * 16 + half * 8);
@@ -696,6 +632,10 @@ template <int DQK, int DV, int SRC, int PS>
 static void launch_prefill(const PrefillParams& p, int64_t total_q, bool ext, double rope_theta, hipStream_t stream) {
   PrefillRopeDivisors div{};
   if (!ext) {
+    if (p.q_inline_rope) {
+      const float theta = static_cast<float>(rope_theta);
+      for (int i = 0; i < DQK / 2 && i < 64; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DQK));
+    }
     launch_prefill_ext<DQK, DV, SRC, PS, false>(p, total_q, div, stream);
     return;
   }
@@ -844,12 +784,12 @@ int tvmkv_batch_prefill_paged_kv_merge(const void* q, const int32_t* q_indptr, c
                        /*merge_into=*/true, stream);
 }
 
-int tvmkv_batch_prefill_cached_and_new_kv(const void* q, const int32_t* q_indptr, const void* k, const void* v,
-                                          const void* pages, const int32_t* page_indptr,
-                                          const int32_t* page_values, const int32_t* last_page_len, void* output,
-                                          float* lse, double sm_scale, int32_t batch_size, int64_t total_q,
-                                          int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
-                                          int32_t d, int32_t page_size, void* stream) {
+static int cached_and_new(const void* q, int64_t q_token_stride, const int32_t* q_rope_position, int64_t apply_rope,
+                          double rope_scale, double rope_theta, const int32_t* q_indptr, const void* k, const void* v,
+                          const void* pages, const int32_t* page_indptr, const int32_t* page_values,
+                          const int32_t* last_page_len, void* output, float* lse, double sm_scale, int32_t batch_size,
+                          int64_t total_q, int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv, int32_t d,
+                          int32_t page_size, void* stream) {
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_cached_and_new_kv: bad shape";
@@ -859,8 +799,13 @@ int tvmkv_batch_prefill_cached_and_new_kv(const void* q, const int32_t* q_indptr
   KV_CHECK(q && q_indptr && k && v && pages && page_indptr && last_page_len && output && lse)
       << "batch_prefill_cached_and_new_kv: NULL tensor";
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_prefill_cached_and_new_kv: NULL page table";
+  KV_CHECK(apply_rope == 0 || q_rope_position) << "batch_prefill_cached_and_new_kv: RoPE needs the position array";
   PrefillParams p{};
   p.q = static_cast<const half_t*>(q);
+  p.q_token_stride = q_token_stride;
+  p.q_inline_rope = apply_rope != 0;
+  p.q_rope_position = q_rope_position;
+  p.rope_scale = static_cast<float>(rope_scale);
   p.q_indptr = q_indptr;
   p.k = static_cast<const half_t*>(k);
   p.v = static_cast<const half_t*>(v);
@@ -879,14 +824,38 @@ int tvmkv_batch_prefill_cached_and_new_kv(const void* q, const int32_t* q_indptr
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
   hipStream_t s = as_stream(stream);
   if (d == 128) {
-    launch_prefill<128, 128, kBoth, 16>(p, total_q, false, 0.0, s);
+    launch_prefill<128, 128, kBoth, 16>(p, total_q, false, rope_theta, s);
   } else if (d == 64) {
-    launch_prefill<64, 64, kBoth, 16>(p, total_q, false, 0.0, s);
+    launch_prefill<64, 64, kBoth, 16>(p, total_q, false, rope_theta, s);
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_cached_and_new_kv: head_dim " << d << " is not built (64, 128)";
   }
   KV_LAUNCH_CHECK();
   KV_API_END();
+}
+
+int tvmkv_batch_prefill_cached_and_new_kv(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                                          const void* pages, const int32_t* page_indptr,
+                                          const int32_t* page_values, const int32_t* last_page_len, void* output,
+                                          float* lse, double sm_scale, int32_t batch_size, int64_t total_q,
+                                          int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                                          int32_t d, int32_t page_size, void* stream) {
+  return cached_and_new(q, 0, nullptr, 0, 1.0, 1e4, q_indptr, k, v, pages, page_indptr, page_values, last_page_len,
+                        output, lse, sm_scale, batch_size, total_q, nnz_pages, num_pages, h_q, h_kv, d, page_size,
+                        stream);
+}
+
+int tvmkv_batch_prefill_cached_and_new_kv_fused_q(const void* qkv, const int32_t* q_rope_position, int64_t apply_rope,
+                                                  double rope_scale, double rope_theta, const int32_t* q_indptr,
+                                                  const void* k, const void* v, const void* pages,
+                                                  const int32_t* page_indptr, const int32_t* page_values,
+                                                  const int32_t* last_page_len, void* output, float* lse,
+                                                  double sm_scale, int32_t batch_size, int64_t total_q,
+                                                  int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                                                  int32_t d, int32_t page_size, void* stream) {
+  return cached_and_new(qkv, static_cast<int64_t>(h_q + 2 * h_kv) * d, q_rope_position, apply_rope, rope_scale,
+                        rope_theta, q_indptr, k, v, pages, page_indptr, page_values, last_page_len, output, lse, sm_scale,
+                        batch_size, total_q, nnz_pages, num_pages, h_q, h_kv, d, page_size, stream);
 }
 
 int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k, const void* v,

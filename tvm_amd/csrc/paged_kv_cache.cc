@@ -638,6 +638,24 @@ class PagedKVCache {
     ComputeStreamWaitForCopyStream();
     KV_CHECK(!dirty_aux_data_device_) << "auxiliary data is not synchronised";
 
+    // A chunked-prefill step of a plain cache in two launches: k is rotated and the new k / v rows go
+    // into their page slots (part 2 without q, part 3), then one pass over the cached and the new
+    // tokens that reads the queries from qkv and rotates them itself (parts 2 and 5).
+    if (OnePassPrefillApplies(layer_id)) {
+      Launch(tvmkv_fused_rope_append(qkv, q_rope_position_map_view_.ptr, /*q=*/nullptr, temp_k_, temp_v_,
+                                     rope_mode_ == TVMKV_ROPE_NORMAL, pages_[local_layer_id],
+                                     append_position_map_view_.ptr, total_seq_length, num_qo_heads_, num_kv_heads_,
+                                     qk_head_dim_, num_total_pages_, page_size_, rotary_scale_, rotary_theta_,
+                                     compute_stream_));
+      Launch(tvmkv_batch_prefill_cached_and_new_kv_fused_q(
+          qkv, q_rope_position_map_view_.ptr, rope_mode_ == TVMKV_ROPE_NORMAL, rotary_scale_, rotary_theta_,
+          cur_append_length_indptr_view_.ptr, temp_k_, temp_v_, pages_[local_layer_id], page_indptr_view_[0].ptr,
+          page_indices_view_[0].ptr, length_info_view_[0].ptr, out, merged_lse_, sm_scale, cur_batch_size_,
+          total_seq_length, page_indices_view_[0].size, num_total_pages_, num_qo_heads_, num_kv_heads_, qk_head_dim_,
+          page_size_, compute_stream_));
+      RecordComputeEvent();
+      return;
+    }
     // Part 2: split fused qkv, RoPE on q/k.  Part 3 with it, in one launch, when the new k / v rows may
     // go into their page slots before attention: always when the reference appends first, and in a
     // cache without sliding windows also when the reference appends afterwards (:1396-1401) -- there
@@ -1292,6 +1310,15 @@ class PagedKVCache {
     copy_stream_has_work_ = true;
   }
 
+  // A chunked-prefill step of a plain cache (one depth, no sliding window, no inline RoPE, no token
+  // tree) can run as one pass over the cached and the new tokens.
+  bool OnePassPrefillApplies(int64_t layer_id) const {
+    return !append_before_attn_ && num_depths_ == 1 && is_chain_on_depths_[0] && !use_decode_kernel_[0] &&
+           page_indices_view_[0].size > 0 && !support_sliding_window_ && attn_kinds_[layer_id] == TVMKV_ATTN_MHA &&
+           rope_mode_ != TVMKV_ROPE_INLINE && qk_head_dim_ == v_head_dim_ &&
+           (qk_head_dim_ == 64 || qk_head_dim_ == 128);
+  }
+
   // :2161-2180
   void AttentionInternal(int64_t layer_id, const void* q, const void* k, const void* v, void* output,
                          int64_t total_seq_length, double sm_scale) {
@@ -1299,9 +1326,7 @@ class PagedKVCache {
     // A chunked-prefill step of a plain cache (one depth, no sliding window, no inline RoPE, no
     // token tree): self-attention over the new tokens, attention over the cached ones and their
     // merge (:2169-2177, :2285-2292) in one pass over both key sets.
-    if (!append_before_attn_ && num_depths_ == 1 && is_chain_on_depths_[0] && !use_decode_kernel_[0] &&
-        page_indices_view_[0].size > 0 && !support_sliding_window_ && attn_kinds_[layer_id] == TVMKV_ATTN_MHA &&
-        rope_mode_ != TVMKV_ROPE_INLINE && qk_head_dim_ == v_head_dim_ && (qk_head_dim_ == 64 || qk_head_dim_ == 128)) {
+    if (OnePassPrefillApplies(layer_id)) {
       Launch(tvmkv_batch_prefill_cached_and_new_kv(q, cur_append_length_indptr_view_.ptr, k, v, pages_[local_layer_id],
                                                    page_indptr_view_[0].ptr, page_indices_view_[0].ptr,
                                                    length_info_view_[0].ptr, output, merged_lse_, sm_scale,

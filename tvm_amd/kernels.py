@@ -50,14 +50,17 @@ def fused_rope(qkv, position_map, q, k, v, apply_rope, rope_scale=1.0, rope_thet
 
 def fused_rope_append(qkv, position_map, q, k, v, apply_rope, pages, append_position_map, rope_scale=1.0,
                       rope_theta=1e4):
-    """fused_rope and tir_kv_cache_transpose_append in one launch."""
-    _f16(qkv, q, k, v, pages)
+    """fused_rope and tir_kv_cache_transpose_append in one launch.  q=None: the q rows are not written
+    (batch_prefill_cached_and_new_kv_fused_q reads and rotates them from qkv)."""
+    _f16(qkv, k, v, pages)
+    if q is not None:
+        _f16(q)
     _i32(position_map, append_position_map)
     n, _, d = qkv.shape
     num_pages, _, hkv, ps, _ = pages.shape
     check(lib().tvmkv_fused_rope_append(_p(qkv), _p(position_map), _p(q), _p(k), _p(v), int(apply_rope), _p(pages),
-                                        _p(append_position_map), n, q.shape[1], k.shape[1], d, num_pages, ps,
-                                        float(rope_scale), float(rope_theta), _stream()))
+                                        _p(append_position_map), n, qkv.shape[1] - 2 * k.shape[1], k.shape[1], d,
+                                        num_pages, ps, float(rope_scale), float(rope_theta), _stream()))
 
 
 def tir_kv_cache_transpose_append(pages, k_data, v_data, position_map):
@@ -113,6 +116,20 @@ def batch_prefill_cached_and_new_kv(q, q_indptr, k, v, pages, page_indptr, page_
         _p(q), _p(q_indptr), _p(k), _p(v), _p(pages), _p(page_indptr), _p(page_values), _p(last_page_len),
         _p(output), _p(lse), float(sm_scale), q_indptr.shape[0] - 1, q.shape[0], page_values.shape[0], num_pages,
         q.shape[1], hkv, d, ps, _stream()))
+
+
+def batch_prefill_cached_and_new_kv_fused_q(qkv, q_rope_position, apply_rope, rope_scale, rope_theta, q_indptr, k, v,
+                                            pages, page_indptr, page_values, last_page_len, output, lse, sm_scale):
+    """batch_prefill_cached_and_new_kv with the queries read from the fused qkv tensor and rotated inside
+    the kernel."""
+    _f16(qkv, k, v, pages, output)
+    _i32(q_rope_position, q_indptr, page_indptr, page_values, last_page_len)
+    num_pages, _, hkv, ps, d = pages.shape
+    hq = qkv.shape[1] - 2 * hkv
+    check(lib().tvmkv_batch_prefill_cached_and_new_kv_fused_q(
+        _p(qkv), _p(q_rope_position), int(apply_rope), float(rope_scale), float(rope_theta), _p(q_indptr), _p(k),
+        _p(v), _p(pages), _p(page_indptr), _p(page_values), _p(last_page_len), _p(output), _p(lse), float(sm_scale),
+        q_indptr.shape[0] - 1, qkv.shape[0], page_values.shape[0], num_pages, hq, hkv, d, ps, _stream()))
 
 
 def batch_decode_paged_kv(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position,
