@@ -64,6 +64,43 @@ int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void
                      int64_t apply_rope, int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
                      int32_t head_dim, double rope_scale, double rope_theta, void* stream);
 
+/* The frequency variants of slot 24 (`switch_rope_freq_func`, position_embedding.py:258-299), which the
+ * reference bakes into the kernel it compiles for a model.  rope_type DEFAULT: angle = pos * scale /
+ * theta^(2i/D).  LLAMA3 (:130-161): smoothed inverse frequencies from factor, low_freq_factor,
+ * high_freq_factor, original_max_position_embeddings.  LONGROPE (:164-188): the default divisors times a
+ * per-dimension factor tensor, cos and sin scaled by sqrt(1 + ln(max / original_max) / ln(original_max)).
+ * YARN (:191-255): interpolated / extrapolated inverse frequencies blended over the dimensions between
+ * the correction dims of beta_fast and beta_slow.  Rotation is over the whole head (rotary_dim ==
+ * head_dim) with the rotate-half pairing; the gptj / llama4 interleaved pairings are not built. */
+enum {
+  TVMKV_ROPE_FREQ_DEFAULT = 0,
+  TVMKV_ROPE_FREQ_LLAMA3 = 1,
+  TVMKV_ROPE_FREQ_LONGROPE = 2,
+  TVMKV_ROPE_FREQ_YARN = 3
+};
+typedef struct tvmkv_rope_scaling {
+  int32_t rope_type;
+  int32_t reserved;
+  double factor;          /* llama3, yarn */
+  double low_freq_factor; /* llama3 */
+  double high_freq_factor;
+  double beta_fast; /* yarn */
+  double beta_slow;
+  int64_t max_position_embeddings; /* longrope */
+  int64_t original_max_position_embeddings;
+} tvmkv_rope_scaling;
+
+/* tvmkv_fused_rope with a frequency variant.  scaling NULL = DEFAULT.  rope_ext_factors: device tensor of
+ * head_dim float32, LONGROPE only: the long factors (head_dim / 2), then the short ones; as in the
+ * reference's kernel (position_embedding.py:582-668) the long ones apply when the call has more rows
+ * than original_max_position_embeddings.  The tables are computed on the host in float32 in the
+ * reference's order of operations and travel as a kernel argument. */
+int tvmkv_fused_rope_scaled(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
+                            int64_t apply_rope, const float* rope_ext_factors,
+                            const tvmkv_rope_scaling* scaling, int64_t seq_len, int32_t num_q_heads,
+                            int32_t num_kv_heads, int32_t head_dim, double rope_scale, double rope_theta,
+                            void* stream);
+
 /* Slot 24 followed by slot 13 in one launch; no counterpart among the reference's kernels.
  * Besides the q / k / v outputs of tvmkv_fused_rope, the rotated k and the v rows are written into
  * their page slots append_position_map[token] (-1 = none), which is what

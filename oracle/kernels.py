@@ -57,6 +57,48 @@ def fused_rope(qkv, position_map, q, k, v, apply_rope, *, theta=1e4, scale=1.0, 
                          _c_f(scale))
 
 
+class RopeScaling(ctypes.Structure):
+    """orc_rope_scaling; `from_dict` takes the reference's rope_scaling dictionary (position_embedding.py:258-299)."""
+    _fields_ = [("rope_type", ctypes.c_int32), ("reserved", ctypes.c_int32), ("factor", ctypes.c_double),
+                ("low_freq_factor", ctypes.c_double), ("high_freq_factor", ctypes.c_double),
+                ("beta_fast", ctypes.c_double), ("beta_slow", ctypes.c_double),
+                ("max_position_embeddings", ctypes.c_int64), ("original_max_position_embeddings", ctypes.c_int64)]
+    TYPES = {"default": 0, "llama3": 1, "longrope": 2, "yarn": 3}
+
+    @classmethod
+    def from_dict(cls, rope_scaling):
+        out = cls()
+        out.rope_type = cls.TYPES[rope_scaling.get("rope_type", "default")]
+        for key in ("factor", "low_freq_factor", "high_freq_factor", "beta_fast", "beta_slow",
+                    "max_position_embeddings", "original_max_position_embeddings"):
+            if key in rope_scaling:
+                setattr(out, key, rope_scaling[key])
+        return out
+
+
+def rope_angle(rope_scaling, pos_scaled, d, rotary_dim, theta, ext=None):
+    """(angle, magnitude) of element d at scaled position pos_scaled, float32 as the reference computes it."""
+    sc = RopeScaling.from_dict(rope_scaling)
+    fn = lib().orc_rope_angle
+    fn.restype = ctypes.c_float
+    mag = ctypes.c_float()
+    ext_p = None if ext is None else _p(np.ascontiguousarray(ext, dtype=np.float32))
+    angle = fn(ctypes.byref(sc), _c_f(pos_scaled), _c_int(d), _c_int(rotary_dim), _c_f(theta), ext_p, ctypes.byref(mag))
+    return float(angle), float(mag.value)
+
+
+def fused_rope_scaled(qkv, position_map, q, k, v, apply_rope, rope_scaling, *, theta=1e4, scale=1.0, ext_factors=None):
+    n, fused, d = qkv.shape
+    hq, hkv = q.shape[1], k.shape[1]
+    assert fused == hq + 2 * hkv
+    pm = _i32(position_map)
+    sc = RopeScaling.from_dict(rope_scaling)
+    ext = None if ext_factors is None else np.ascontiguousarray(ext_factors, dtype=np.float32)
+    lib().orc_fused_rope_scaled(_p(qkv), _p(pm), _p(q), _p(k), _p(v), _c_i64(n), _c_int(hq), _c_int(hkv), _c_int(d),
+                                _c_i64(int(apply_rope)), _c_f(theta), _c_f(scale), ctypes.byref(sc),
+                                None if ext is None else _p(ext))
+
+
 def transpose_append(pages, k_data, v_data, position_map):
     _, two, hkv, ps, d = pages.shape
     assert two == 2

@@ -148,6 +148,98 @@ void orc_fused_rope(const f16* qkv, const int32_t* position_map, f16* q, f16* k,
   }
 }
 
+/* ---- RoPE frequency variants (position_embedding.py:130-299) ------------------------
+ * The reference compiles one of these into the kernel of a model.  Everything is float32 as in the
+ * TIR expression (python constants become float32 immediates); the angle of element d at scaled
+ * position s:
+ *   default   s / theta^((2d mod R)/R)                                                      (:32-67)
+ *   llama3    s * ((1-smooth)*f/factor + smooth*f), f = 1/theta^(..),
+ *             smooth = clip(alpha*f - beta, 0, 1)                                           (:130-161)
+ *   longrope  s / (ext[d mod R/2] * theta^(..)); cos and sin times
+ *             sqrt(1 + ln(max/orig)/ln(orig)) when max > orig                               (:164-188)
+ *   yarn      s * (inter*(1-mask) + extra*mask), extra = 1/theta^(..), inter = extra/factor,
+ *             mask = 1 - clip((d - low)/(high - low), 0, 1) with d the ELEMENT index and the
+ *             correction dims low/high not rounded (:191-255; the published YaRN code floors and
+ *             ceils them and ramps over R/2 frequencies, the reference does neither)
+ * Pins (tests/test_oracle_kernels.py): llama3 against the piecewise form of the Llama-3.1 release
+ * (unchanged above the high-frequency wavelength, divided by `factor` below the low one, linear in
+ * between); yarn against the published formula with its rounding removed and, for factor = 1,
+ * against default; longrope with unit factors and max = orig against default, bit for bit. */
+typedef struct {
+  int32_t rope_type; /* 0 default, 1 llama3, 2 longrope, 3 yarn */
+  int32_t reserved;
+  double factor, low_freq_factor, high_freq_factor, beta_fast, beta_slow;
+  int64_t max_position_embeddings, original_max_position_embeddings;
+} orc_rope_scaling;
+
+/* angle and magnitude of element d; ext = the factor half to use or NULL */
+float orc_rope_angle(const orc_rope_scaling* sc, float s, int d, int R, float theta, const float* ext,
+                     float* magnitude) {
+  float power = powf(theta, (float)((d * 2) % R) / (float)R);
+  *magnitude = 1.0f;
+  if (sc == NULL || sc->rope_type == 0) return s / power;
+  if (sc->rope_type == 1) {
+    float orig = 1.0f / power;
+    double inv_diff = 1.0 / (sc->high_freq_factor - sc->low_freq_factor);
+    float inv_factor = (float)(1.0 / sc->factor);
+    float alpha = (float)((double)sc->original_max_position_embeddings / (2 * M_PI) * inv_diff);
+    float beta = (float)(sc->low_freq_factor * inv_diff);
+    float smooth = fmaxf(0.0f, fminf(1.0f, alpha * orig - beta));
+    return s * ((1.0f - smooth) * orig * inv_factor + smooth * orig);
+  }
+  if (sc->rope_type == 2) {
+    double scale = (double)sc->max_position_embeddings / (double)sc->original_max_position_embeddings;
+    if (scale > 1.0)
+      *magnitude = (float)sqrt(1.0 + log(scale) / log((double)sc->original_max_position_embeddings));
+    float divisor = power;
+    if (ext != NULL) divisor = ext[d % (R / 2)] * divisor;
+    return s / divisor;
+  }
+  double inv_theta_log_scale = 1.0 / (2.0 * log((double)theta)); /* kv_cache.py:363-365 */
+  double lo = R * log((double)sc->original_max_position_embeddings / (sc->beta_fast * 2 * M_PI)) * inv_theta_log_scale;
+  double hi = R * log((double)sc->original_max_position_embeddings / (sc->beta_slow * 2 * M_PI)) * inv_theta_log_scale;
+  float low = (float)(lo > 0 ? lo : 0), high = (float)(hi < R - 1 ? hi : R - 1);
+  if (low == high) high += 0.001f;
+  float extra = 1.0f / power;
+  float inter = 1.0f / ((float)sc->factor * power);
+  float mask = 1.0f - fmaxf(fminf(((float)d - low) / (high - low), 1.0f), 0.0f);
+  return s * (inter * (1.0f - mask) + extra * mask);
+}
+
+/* fused_rope / fused_rope_longrope_scaling (position_embedding.py:525-667) with a frequency variant.
+ * ext_factors: NULL or R floats, long factors then short ones; the long ones apply when
+ * seq_len > original_max_position_embeddings (:601). */
+void orc_fused_rope_scaled(const f16* qkv, const int32_t* position_map, f16* q, f16* k, f16* v,
+                           int64_t seq_len, int num_q_heads, int num_kv_heads, int head_dim,
+                           int64_t apply_rope, float theta, float scale, const orc_rope_scaling* sc,
+                           const float* ext_factors) {
+  int fused_heads = num_q_heads + 2 * num_kv_heads;
+  int R = head_dim;
+  const float* ext = ext_factors;
+  if (ext != NULL && sc != NULL && !(seq_len > sc->original_max_position_embeddings)) ext += R / 2;
+  for (int64_t s = 0; s < seq_len; ++s) {
+    for (int h = 0; h < fused_heads; ++h) {
+      const f16* x = qkv + (s * fused_heads + h) * head_dim;
+      f16* dst = h < num_q_heads ? q + (s * num_q_heads + h) * head_dim
+                 : h < num_q_heads + num_kv_heads
+                     ? k + (s * num_kv_heads + (h - num_q_heads)) * head_dim
+                     : v + (s * num_kv_heads + (h - num_q_heads - num_kv_heads)) * head_dim;
+      for (int d = 0; d < head_dim; ++d) {
+        if (h >= num_q_heads + num_kv_heads || !(apply_rope > 0)) {
+          dst[d] = x[d];
+          continue;
+        }
+        float magnitude;
+        float freq = orc_rope_angle(sc, (float)position_map[s] * scale, d, R, theta, ext, &magnitude);
+        float c = (cosf(freq) * magnitude) * h2f(x[d]);
+        f16 other = d < R / 2 ? (f16)(x[d + R / 2] ^ 0x8000u) : x[d - R / 2];
+        float sn = (sinf(freq) * magnitude) * h2f(other);
+        dst[d] = f2h(c + sn);
+      }
+    }
+  }
+}
+
 /* ---- page kernels ------------------------------------------------------------ */
 #define PAGE_AT(pages, Hkv, ps, D, page, kv, h, slot) \
   ((pages) + ((((int64_t)(page) * 2 + (kv)) * (Hkv) + (h)) * (ps) + (slot)) * (int64_t)(D))

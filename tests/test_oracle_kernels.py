@@ -530,3 +530,117 @@ def test_mla_absorbed_causal_equals_expanded_definition():
     first = out[nqs[0]].astype(np.float64)
     assert_close(first, np.broadcast_to(latents[1][0, :d_lat].astype(np.float64), first.shape), atol=2e-3, rtol=2e-3,
                  what="a row that sees one key returns that key's latent")
+
+
+# ------------------------------------------------------------------------ RoPE frequency variants
+LLAMA3 = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+          "original_max_position_embeddings": 8192}
+YARN = {"rope_type": "yarn", "factor": 40.0, "beta_fast": 32, "beta_slow": 1, "original_max_position_embeddings": 4096}
+
+
+def test_llama3_angles_match_the_published_piecewise_rule():
+    """Llama-3.1's rule as published with the model: frequencies whose wavelength is below
+    original_max / high_freq_factor stay, those above original_max / low_freq_factor are divided by
+    `factor`, those in between blend linearly in original_max / wavelength.  float64 numpy, a
+    different structure (where / masks) from the reference's clip expression."""
+    D, theta = 128, 5e5
+    i = np.arange(D // 2, dtype=np.float64)
+    inv_freq = 1.0 / theta ** (2 * i / D)
+    wavelen = 2 * np.pi / inv_freq
+    old, low, high, factor = 8192.0, 1.0, 4.0, 8.0
+    expect = np.where(wavelen > old / low, inv_freq / factor, inv_freq)
+    smooth = (old / wavelen - low) / (high - low)
+    medium = ~(wavelen < old / high) & ~(wavelen > old / low)
+    expect = np.where(medium, (1 - smooth) * inv_freq / factor + smooth * inv_freq, expect)
+    assert medium.any() and (wavelen > old / low).any() and (wavelen < old / high).any()
+    pos = 1000.0
+    for d in range(D):
+        angle, mag = ok.rope_angle(LLAMA3, pos, d, D, theta)
+        assert mag == 1.0
+        np.testing.assert_allclose(angle, pos * expect[d % (D // 2)], rtol=2e-6)
+
+
+def test_yarn_angles_match_the_published_blend_without_rounding():
+    """YaRN as published (find_correction_dim, linear ramp, blend of interpolated and extrapolated
+    frequencies) with the two deviations of the reference: the correction dims are not floored / ceiled
+    (position_embedding.py:203-217) and the ramp is indexed by the element, so the upper half of the
+    head (d >= D/2) gets the ramp value of d, not of d - D/2 (:244-247)."""
+    D, theta = 128, 1e4
+    factor, beta_fast, beta_slow, orig = 40.0, 32.0, 1.0, 4096.0
+
+    def correction_dim(rot):
+        return D * np.log(orig / (rot * 2 * np.pi)) / (2 * np.log(theta))
+
+    low, high = max(correction_dim(beta_fast), 0.0), min(correction_dim(beta_slow), D - 1.0)
+    d = np.arange(D, dtype=np.float64)
+    pos_freqs = theta ** ((2 * d % D) / D)
+    ramp = np.clip((d - low) / (high - low), 0, 1)
+    expect = (1.0 / (factor * pos_freqs)) * ramp + (1.0 / pos_freqs) * (1 - ramp)
+    assert 0 < low < high < D / 2  # the ramp is inside the lower half; the upper half is fully interpolated
+    pos = 777.0
+    for e in range(D):
+        angle, mag = ok.rope_angle(YARN, pos, e, D, theta)
+        assert mag == 1.0
+        np.testing.assert_allclose(angle, pos * expect[e], rtol=3e-6)
+    # every element of the upper half is interpolated: its angle is the default one over `factor`
+    for e in (D // 2, D // 2 + 5, D - 1):
+        plain, _ = ok.rope_angle({}, pos, e, D, theta)
+        np.testing.assert_allclose(ok.rope_angle(YARN, pos, e, D, theta)[0], plain / factor, rtol=3e-6)
+
+
+def test_rope_variants_reduce_to_default():
+    D, theta = 64, 1e4
+    rng = np.random.default_rng(3)
+    n, hq, hkv = 6, 4, 2
+    qkv = rng.standard_normal((n, hq + 2 * hkv, D)).astype(np.float16)
+    pos = np.array([0, 1, 17, 300, 4095, 70000], np.int32)
+
+    def run(scaling, ext=None, apply_rope=1):
+        q, k, v = np.zeros((n, hq, D), np.float16), np.zeros((n, hkv, D), np.float16), np.zeros((n, hkv, D), np.float16)
+        ok.fused_rope_scaled(qkv, pos, q, k, v, apply_rope, scaling, theta=theta, ext_factors=ext)
+        return q, k, v
+
+    eq, ek, ev = np.zeros((n, hq, D), np.float16), np.zeros((n, hkv, D), np.float16), np.zeros((n, hkv, D), np.float16)
+    ok.fused_rope(qkv, pos, eq, ek, ev, 1, theta=theta)
+    # no scaling, and longrope with unit factors and no extension: bit for bit the plain kernel
+    for scaling, ext in (({}, None), ({"rope_type": "longrope", "max_position_embeddings": 4096,
+                                       "original_max_position_embeddings": 4096}, np.ones(D, np.float32))):
+        q, k, v = run(scaling, ext)
+        assert np.array_equal(q, eq) and np.array_equal(k, ek) and np.array_equal(v, ev)
+    # yarn with factor 1 and llama3 with factor 1 are the plain frequencies up to float32 rounding
+    for scaling in (dict(YARN, factor=1.0), dict(LLAMA3, factor=1.0)):
+        q, k, v = run(scaling)
+        assert np.array_equal(v, ev)
+        assert_close(q, eq, atol=2e-2, rtol=1e-2, what="factor-1 scaling q")  # angles of ~7e4 rad carry ~1e-2 abs error in float32
+        assert np.mean(q == eq) > 0.9
+    # apply_rope = 0 copies
+    q, k, v = run(LLAMA3, apply_rope=0)
+    assert np.array_equal(q, qkv[:, :hq]) and np.array_equal(k, qkv[:, hq:hq + hkv])
+
+
+def test_longrope_factors_and_magnitude():
+    """The angle is the default one over the factor of the dimension; cos and sin carry
+    sqrt(1 + ln(max/orig)/ln(orig)); the long factors apply only to calls with more rows than orig."""
+    D, theta = 64, 1e4
+    scaling = {"rope_type": "longrope", "max_position_embeddings": 131072, "original_max_position_embeddings": 4}
+    ext = np.concatenate([np.linspace(1.0, 4.0, D // 2), np.linspace(1.0, 1.5, D // 2)]).astype(np.float32)
+    plain, _ = ok.rope_angle({}, 33.0, 7, D, theta)
+    angle, mag = ok.rope_angle(scaling, 33.0, 7, D, theta, ext[:D // 2])
+    np.testing.assert_allclose(angle, plain / ext[7], rtol=1e-6)
+    np.testing.assert_allclose(mag, np.sqrt(1 + np.log(131072 / 4) / np.log(4)), rtol=1e-6)
+    angle_hi, _ = ok.rope_angle(scaling, 33.0, 7 + D // 2, D, theta, ext[:D // 2])
+    assert angle_hi == angle  # both halves of a pair share the factor (index d mod D/2)
+    rng = np.random.default_rng(4)
+    hq, hkv = 2, 1
+    for n, half in ((3, ext[D // 2:]), (5, ext[:D // 2])):  # 3 rows <= orig: short factors; 5 rows > orig: long
+        qkv = rng.standard_normal((n, hq + 2 * hkv, D)).astype(np.float16)
+        pos = np.arange(10, 10 + n, dtype=np.int32)
+        q, k, v = np.zeros((n, hq, D), np.float16), np.zeros((n, hkv, D), np.float16), np.zeros((n, hkv, D), np.float16)
+        ok.fused_rope_scaled(qkv, pos, q, k, v, 1, scaling, theta=theta, ext_factors=ext)
+        x = qkv[:, 0].astype(np.float64)
+        i = np.arange(D // 2)
+        ang = pos[:, None].astype(np.float64) / (half.astype(np.float64) * theta ** (2 * i / D))
+        m = np.sqrt(1 + np.log(131072 / 4) / np.log(4))
+        lo = m * (np.cos(ang) * x[:, :D // 2] - np.sin(ang) * x[:, D // 2:])
+        hi = m * (np.cos(ang) * x[:, D // 2:] + np.sin(ang) * x[:, :D // 2])
+        assert_close(q[:, 0], np.concatenate([lo, hi], axis=1).astype(np.float16), atol=2e-3, rtol=2e-3, what="longrope q")

@@ -23,6 +23,8 @@ class KVError(RuntimeError):
 # name -> argument ctypes, in the order of include/tvmkv.h
 SIGNATURES = {
     "tvmkv_fused_rope": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_i32, c_f64, c_f64, c_vp],
+    "tvmkv_fused_rope_scaled": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_f64,
+                                c_f64, c_vp],
     "tvmkv_fused_rope_append": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i64,
                                 c_i32, c_f64, c_f64, c_vp],
     "tvmkv_kv_cache_transpose_append": [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_i32, c_vp],
@@ -89,6 +91,21 @@ SIGNATURES = {
     "tvmkv_cache_dump_state": [c_vp, p_i64, c_i64, p_i64],
     "tvmkv_cache_get_copy_log": [c_vp, ctypes.POINTER(p_i64), p_i64],
     "tvmkv_cache_get_pages": [c_vp, c_i64, ctypes.POINTER(c_vp), p_i64],
+    # include/tvmkv_dlpack.h: DLTensor* arguments in the order of the reference's kernel slots
+    "tvmkv_dl_fused_rope": [c_vp] * 5 + [c_i64, c_vp, c_vp, c_f64, c_f64, c_vp],
+    "tvmkv_dl_transpose_append": [c_vp] * 5,
+    "tvmkv_dl_transpose_append_mla": [c_vp] * 4,
+    "tvmkv_dl_batch_prefill_ragged_kv": [c_vp] * 9 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_vp],
+    "tvmkv_dl_batch_prefill_paged_kv": [c_vp] * 10 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_i64, c_vp],
+    "tvmkv_dl_batch_decode_paged_kv": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_vp],
+    "tvmkv_dl_tree_attn_paged_kv": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_vp, c_vp, c_vp],
+    "tvmkv_dl_batch_tree_attn": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_vp],
+    "tvmkv_dl_batch_prefill_paged_kv_mla": [c_vp] * 8 + [c_i64, c_f64, c_vp],
+    "tvmkv_dl_merge_state_inplace": [c_vp] * 5,
+    "tvmkv_dl_copy_single_page": [c_vp, c_i64, c_i64, c_i64, c_vp],
+    "tvmkv_dl_debug_get_kv": [c_vp] * 4 + [c_i64, c_vp],
+    "tvmkv_dl_debug_get_kv_mla": [c_vp] * 3 + [c_i64, c_vp],
+    "tvmkv_dl_compact_kv_copy": [c_vp] * 3 + [c_i64, c_vp],
 }
 
 _lib = None

@@ -19,9 +19,12 @@ namespace tvmkv {
 // The D/2 divisors pow(theta, 2i/D) are computed on the host with the same libm call the CPU
 // kernels use and travel as a kernel argument, so the angle is formed by one IEEE division.
 // ------------------------------------------------------------------------------------------
-constexpr int kMaxHalfDim = 128;
+// One entry per element of the head: element d and its rotation partner d + D/2 share an angle in
+// every variant but yarn, whose blend between interpolated and extrapolated frequencies is indexed
+// by the element (position_embedding.py:244-247).
+constexpr int kMaxHeadDim = 256;
 struct RopeDivisors {
-  float v[kMaxHalfDim];
+  float v[kMaxHeadDim];
 };
 
 // One workgroup per token: the D/2 (cos, sin) pairs of the token's position are computed once
@@ -35,20 +38,35 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
                                                          half_t* __restrict__ q, half_t* __restrict__ k,
                                                          half_t* __restrict__ v, int64_t seq_len, int num_q_heads,
                                                          int num_kv_heads, int apply_rope, float scale,
-                                                         RopeDivisors div, half_t* __restrict__ pages,
+                                                         RopeDivisors div, int table_is_inverse, int halves_differ,
+                                                         float magnitude,
+                                                         const float* __restrict__ ext_factors,
+                                                         half_t* __restrict__ pages,
                                                          const int32_t* __restrict__ append_position_map,
                                                          int page_size) {
   constexpr int kThreadsPerHead = D / 16;  // a thread owns d-range [8c, 8c+8) and its partner +D/2
-  __shared__ float cs_lds[D / 2];
-  __shared__ float sn_lds[D / 2];
+  __shared__ float cs_lds[D];  // [0, D/2): for the elements of the lower half, [D/2, D): of the upper half
+  __shared__ float sn_lds[D];
   const int64_t s = blockIdx.x;  // token
   const int fused_heads = num_q_heads + 2 * num_kv_heads;
   if (apply_rope > 0) {
     const float pos_scaled = static_cast<float>(position_map[s]) * scale;
-    for (int i = threadIdx.x; i < D / 2; i += 256) {
-      const float freq = pos_scaled / div.v[i];
-      cs_lds[i] = cosf(freq);
-      sn_lds[i] = sinf(freq);
+    for (int i = threadIdx.x; i < (halves_differ ? D : D / 2); i += 256) {
+      // default / longrope: position over a divisor (times the model's per-dimension factor, if any);
+      // llama3 / yarn: position times an inverse frequency (position_embedding.py:130-255)
+      float freq;
+      if (table_is_inverse) {
+        freq = pos_scaled * div.v[i];
+      } else {
+        freq = pos_scaled / (ext_factors != nullptr ? ext_factors[i] * div.v[i] : div.v[i]);
+      }
+      const float cs = cosf(freq) * magnitude, sn = sinf(freq) * magnitude;
+      cs_lds[i] = cs;
+      sn_lds[i] = sn;
+      if (!halves_differ) {
+        cs_lds[i + D / 2] = cs;
+        sn_lds[i + D / 2] = sn;
+      }
     }
     __syncthreads();
   }
@@ -72,12 +90,10 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
       Vec16 out_lo, out_hi;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float cs = cs_lds[c * 8 + e];
-        const float sn = sn_lds[c * 8 + e];
         const float xl = static_cast<float>(lo.h[e]);
         const float xh = static_cast<float>(hi.h[e]);
-        out_lo.h[e] = static_cast<half_t>(cs * xl + sn * (-xh));
-        out_hi.h[e] = static_cast<half_t>(cs * xh + sn * xl);
+        out_lo.h[e] = static_cast<half_t>(cs_lds[c * 8 + e] * xl + sn_lds[c * 8 + e] * (-xh));
+        out_hi.h[e] = static_cast<half_t>(cs_lds[D / 2 + c * 8 + e] * xh + sn_lds[D / 2 + c * 8 + e] * xl);
       }
       lo = out_lo;
       hi = out_hi;
@@ -329,8 +345,78 @@ using namespace tvmkv;
 
 extern "C" {
 
+// The table of floats a RoPE variant needs (head_dim / 2, or head_dim when the two halves differ), in
+// float32 arithmetic in the reference's order of operations (position_embedding.py:32-67 default,
+// :130-161 llama3, :164-188 longrope, :191-255 yarn).  Returns whether the table holds inverse
+// frequencies (multiply) or divisors.
+static bool rope_table(const tvmkv_rope_scaling* scaling, int head_dim, double rope_theta, int64_t seq_len,
+                       const float** ext_factors, RopeDivisors* table, float* magnitude, bool* halves_differ) {
+  *halves_differ = false;
+  const float theta = static_cast<float>(rope_theta);
+  const int type = scaling == nullptr ? TVMKV_ROPE_FREQ_DEFAULT : scaling->rope_type;
+  const float d_range = static_cast<float>(head_dim);
+  *magnitude = 1.0f;
+  auto power = [&](int i) { return powf(theta, static_cast<float>((i * 2) % head_dim) / d_range); };
+  if (type == TVMKV_ROPE_FREQ_DEFAULT || type == TVMKV_ROPE_FREQ_LONGROPE) {
+    for (int i = 0; i < head_dim / 2; ++i) table->v[i] = power(i);
+    if (type == TVMKV_ROPE_FREQ_LONGROPE) {
+      KV_CHECK(scaling->original_max_position_embeddings > 0 && scaling->max_position_embeddings > 0)
+          << "fused_rope: longrope needs max_position_embeddings and original_max_position_embeddings";
+      const double scale = static_cast<double>(scaling->max_position_embeddings) /
+                           static_cast<double>(scaling->original_max_position_embeddings);
+      if (scale > 1.0) {
+        *magnitude = static_cast<float>(
+            std::sqrt(1.0 + std::log(scale) / std::log(static_cast<double>(scaling->original_max_position_embeddings))));
+      }
+      // the factor tensor holds the long factors, then the short ones (position_embedding.py:601-668)
+      if (*ext_factors != nullptr && seq_len <= scaling->original_max_position_embeddings) *ext_factors += head_dim / 2;
+    } else {
+      KV_CHECK(*ext_factors == nullptr) << "fused_rope: rope_ext_factors needs a longrope scaling description";
+    }
+    return false;
+  }
+  KV_CHECK(*ext_factors == nullptr) << "fused_rope: rope_ext_factors needs a longrope scaling description";
+  if (type == TVMKV_ROPE_FREQ_LLAMA3) {
+    KV_CHECK(scaling->high_freq_factor != scaling->low_freq_factor && scaling->factor != 0)
+        << "fused_rope: llama3 scaling needs factor != 0 and high_freq_factor != low_freq_factor";
+    const double inv_diff = 1.0 / (scaling->high_freq_factor - scaling->low_freq_factor);
+    const float inv_factor = static_cast<float>(1.0 / scaling->factor);
+    const float alpha = static_cast<float>(static_cast<double>(scaling->original_max_position_embeddings) / (2 * M_PI) * inv_diff);
+    const float beta = static_cast<float>(scaling->low_freq_factor * inv_diff);
+    for (int i = 0; i < head_dim / 2; ++i) {
+      const float orig = 1.0f / power(i);
+      const float smooth = fmaxf(0.0f, fminf(1.0f, alpha * orig - beta));
+      table->v[i] = (1.0f - smooth) * orig * inv_factor + smooth * orig;
+    }
+    return true;
+  }
+  KV_UNSUPPORTED(type != TVMKV_ROPE_FREQ_YARN)
+      << "fused_rope: rope type " << type << " is not built (default, llama3, longrope, yarn)";
+  KV_CHECK(scaling->factor != 0 && rope_theta > 1.0) << "fused_rope: yarn scaling needs factor != 0 and theta > 1";
+  const double inv_theta_log_scale = 1.0 / (2.0 * std::log(rope_theta));  // kv_cache.py:363-365
+  auto correction_dim = [&](double rotations) {
+    return head_dim * std::log(static_cast<double>(scaling->original_max_position_embeddings) / (rotations * 2 * M_PI)) *
+           inv_theta_log_scale;
+  };
+  const float low = static_cast<float>(std::max(correction_dim(scaling->beta_fast), 0.0));
+  float high = static_cast<float>(std::min(correction_dim(scaling->beta_slow), static_cast<double>(head_dim - 1)));
+  if (low == high) high += 0.001f;
+  const float factor = static_cast<float>(scaling->factor);
+  // the blend is indexed by the element, not by its frequency: the two halves get different angles
+  *halves_differ = true;
+  for (int d = 0; d < head_dim; ++d) {
+    const float freq_power = power(d);
+    const float extra = 1.0f / freq_power;
+    const float inter = 1.0f / (factor * freq_power);
+    const float mask = 1.0f - fmaxf(fminf((static_cast<float>(d) - low) / (high - low), 1.0f), 0.0f);
+    table->v[d] = inter * (1.0f - mask) + extra * mask;
+  }
+  return true;
+}
+
 static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
-                           int64_t apply_rope, int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
+                           int64_t apply_rope, const float* ext_factors, const tvmkv_rope_scaling* scaling,
+                           int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
                            int32_t head_dim, double rope_scale, double rope_theta, void* pages,
                            const int32_t* append_position_map, int64_t num_pages, int32_t page_size, void* stream) {
   KV_API_BEGIN();
@@ -345,17 +431,19 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
     KV_CHECK(num_pages * page_size <= INT32_MAX) << "fused_rope_append: slot ids do not fit int32";
   }
   RopeDivisors div;
-  const float theta = static_cast<float>(rope_theta);
-  for (int i = 0; i < head_dim / 2; ++i) {
-    div.v[i] = powf(theta, static_cast<float>((i * 2) % head_dim) / static_cast<float>(head_dim));
-  }
+  float magnitude = 1.0f;
+  bool halves_differ = false;
+  const bool table_is_inverse =
+      rope_table(scaling, head_dim, rope_theta, seq_len, &ext_factors, &div, &magnitude, &halves_differ);
   KV_CHECK(seq_len < (int64_t{1} << 31)) << "fused_rope: too many tokens for one launch";
   const float scale = static_cast<float>(rope_scale);
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(seq_len)), dim3(256), 0, as_stream(stream), static_cast<const half_t*>(qkv),
                        position_map, static_cast<half_t*>(q), static_cast<half_t*>(k), static_cast<half_t*>(v),
                        seq_len, num_q_heads, num_kv_heads, static_cast<int>(apply_rope > 0), scale, div,
-                       static_cast<half_t*>(pages), append_position_map, page_size);
+                       static_cast<int>(table_is_inverse), static_cast<int>(halves_differ), magnitude, ext_factors,
+                       static_cast<half_t*>(pages),
+                       append_position_map, page_size);
   };
   if (head_dim == 64) {
     if (append) launch(fused_rope_kernel<64, true>); else launch(fused_rope_kernel<64, false>);
@@ -371,8 +459,16 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
 int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void* k, void* v, int64_t apply_rope,
                      int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                      double rope_scale, double rope_theta, void* stream) {
-  return fused_rope_impl(qkv, position_map, q, k, v, apply_rope, seq_len, num_q_heads, num_kv_heads, head_dim,
-                         rope_scale, rope_theta, nullptr, nullptr, 0, 0, stream);
+  return fused_rope_impl(qkv, position_map, q, k, v, apply_rope, nullptr, nullptr, seq_len, num_q_heads, num_kv_heads,
+                         head_dim, rope_scale, rope_theta, nullptr, nullptr, 0, 0, stream);
+}
+
+int tvmkv_fused_rope_scaled(const void* qkv, const int32_t* position_map, void* q, void* k, void* v, int64_t apply_rope,
+                            const float* rope_ext_factors, const tvmkv_rope_scaling* scaling, int64_t seq_len,
+                            int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, double rope_scale,
+                            double rope_theta, void* stream) {
+  return fused_rope_impl(qkv, position_map, q, k, v, apply_rope, rope_ext_factors, scaling, seq_len, num_q_heads,
+                         num_kv_heads, head_dim, rope_scale, rope_theta, nullptr, nullptr, 0, 0, stream);
 }
 
 int tvmkv_fused_rope_append(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
@@ -383,8 +479,8 @@ int tvmkv_fused_rope_append(const void* qkv, const int32_t* position_map, void* 
     ::tvmkv::SetLastError("fused_rope_append: NULL pages");
     return TVMKV_EINVAL;
   }
-  return fused_rope_impl(qkv, position_map, q, k, v, apply_rope, seq_len, num_q_heads, num_kv_heads, head_dim,
-                         rope_scale, rope_theta, pages, append_position_map, num_pages, page_size, stream);
+  return fused_rope_impl(qkv, position_map, q, k, v, apply_rope, nullptr, nullptr, seq_len, num_q_heads, num_kv_heads,
+                         head_dim, rope_scale, rope_theta, pages, append_position_map, num_pages, page_size, stream);
 }
 
 static void check_slot_layout(const char* what, int32_t page_size, int32_t head_dim) {

@@ -48,6 +48,23 @@ def fused_rope(qkv, position_map, q, k, v, apply_rope, rope_scale=1.0, rope_thet
                                  k.shape[1], d, float(rope_scale), float(rope_theta), _stream()))
 
 
+def fused_rope_scaled(qkv, position_map, q, k, v, apply_rope, rope_scaling, rope_scale=1.0, rope_theta=1e4,
+                      rope_ext_factors=None):
+    """fused_rope with one of the reference's frequency variants: rope_scaling is the reference's dictionary
+    (rope_type llama3 / longrope / yarn and its parameters, position_embedding.py:258-299); rope_ext_factors the
+    float32 device tensor of a longrope model (long factors, then short ones)."""
+    from .dlpack import RopeScaling
+    _f16(qkv, q, k, v)
+    _i32(position_map)
+    if rope_ext_factors is not None and rope_ext_factors.dtype != torch.float32:
+        raise KVError(-1, "rope_ext_factors must be float32")
+    n, _, d = qkv.shape
+    scaling = RopeScaling.from_dict(rope_scaling)
+    check(lib().tvmkv_fused_rope_scaled(_p(qkv), _p(position_map), _p(q), _p(k), _p(v), int(apply_rope),
+                                        _p(rope_ext_factors), ctypes.c_void_p(ctypes.addressof(scaling)), n, q.shape[1],
+                                        k.shape[1], d, float(rope_scale), float(rope_theta), _stream()))
+
+
 def fused_rope_append(qkv, position_map, q, k, v, apply_rope, pages, append_position_map, rope_scale=1.0,
                       rope_theta=1e4):
     """fused_rope and tir_kv_cache_transpose_append in one launch.  q=None: the q rows are not written
