@@ -343,8 +343,8 @@ int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr,
  *   decode_chunk_pages     pages per split-KV chunk of the decode kernel (a multiple of 8); 0 = from shapes
  *   decode_separate_merge  != 0: merge the decode chunks in a second launch instead of inside the kernel
  *   decode_wgs_per_cu      > 0: cap the decode grid at this many workgroups per compute unit
- *   mla_chunk_tokens       tokens per split-KV chunk of MLA decode; 0 = from shapes
- *   mla_separate_merge     != 0: merge the MLA decode chunks in a second launch */
+ *   mla_chunk_tokens       lower bound of the tokens per split-KV chunk of MLA decode; 0 = 128
+ *   mla_separate_merge     accepted and ignored: the MLA decode chunks are always merged in a second launch */
 int tvmkv_set_option(const char* name, int64_t value);
 int tvmkv_get_option(const char* name, int64_t* value);
 

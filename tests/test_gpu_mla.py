@@ -74,6 +74,25 @@ def test_mla_decode_shaped_split_kv(ps):
     assert not go[6].any() and np.all(gl[6] == np.float32(-5e4))
 
 
+def test_mla_decode_one_long_sequence_many_chunks():
+    """One sequence over all workgroups: more than a hundred chunks, merged several at a time."""
+    rng = np.random.default_rng(31)
+    go, gl, eo, el = _mla_both(rng, [20000], [1], 64, npages=320)
+    assert_close(go, eo, what="mla long decode out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla long decode lse")
+
+
+def test_mla_decode_batch_beyond_one_sequence_per_lane():
+    """100 sequences: the split plan keeps two sequences per lane; lengths from empty to a few chunks."""
+    rng = np.random.default_rng(32)
+    kv_lens = [int(x) for x in rng.integers(0, 700, size=100)]
+    kv_lens[3], kv_lens[64], kv_lens[99] = 0, 1, 2500
+    go, gl, eo, el = _mla_both(rng, kv_lens, [1] * 100, 64, npages=700)
+    assert_close(go, eo, what="mla wide decode out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla wide decode lse")
+    assert not go[3].any() and np.all(gl[3] == np.float32(-5e4))
+
+
 def test_mla_as_many_tokens_as_sequences_but_not_a_decode_step():
     """total_q == batch makes the launcher split the KV; sequences that do not have exactly one
     query token must still come out right (they are done unsplit by the workgroups of chunk 0)."""

@@ -17,10 +17,17 @@
 // (ds_read_b64_tr_b16, which transposes on the way out of LDS).  Per matrix instruction the LDS
 // delivers half as many bytes as with 16-row waves, which were bound by it.
 //
-// KV split: decode-shaped calls (one token per sequence) have too few row tiles to fill 256 CUs,
-// so the KV of a sequence is cut into chunks of about `chunk_tokens` tokens; partial (O, m, l)
-// states go to an fp32 buffer indexed by (chunk slot, head) and a second kernel merges them.  The
-// chunk slots of a sequence are a pure function of the page table, recomputed by both kernels.
+// KV split: decode-shaped calls (one token per sequence) have too few row tiles to fill 256 CUs, so
+// the KV tiles of the sequences are cut into chunks, one workgroup each, of a common maximum length:
+// the smallest one with which the chunks fit the grid.  Every workgroup derives that length and its
+// own (sequence, chunk) from the page table alone, with the sequences spread over the lanes (one
+// round of loads; mla_split_plan).  A chunk's state leaves the kernel normalised, in fp16, with its
+// log-sum-exp in fp32, as whole rows put together in LDS; workgroup ids are mapped to chunk slots so
+// that the chunks of a sequence run on one XCD (they share the sequence's q rows in its L2); a second
+// kernel merges the states.  (Merging inside the kernel -- the workgroups of a sequence counting
+// themselves in and sharing the merge -- was built and measured: the states then have to cross between
+// workgroups with device-scope stores and loads, which move 33 + 33 MB at under 4 TB/s while every
+// workgroup waits for them, and the step took 102 us against 83 us with the second kernel.)
 #include <algorithm>
 #include <cstdlib>
 #include <type_traits>
@@ -45,15 +52,16 @@ struct MlaParams {
   const int32_t* last_page_len;
   half_t* output;
   float* lse;
-  float* part_o;   // (chunk slots, h_q, DV)
-  float* part_ml;  // (chunk slots, h_q, 2)
+  half_t* part_o;    // (chunk slots, h_q, DV): a chunk's attention output (normalised)
+  float* part_lse;   // (chunk slots, h_q): its log-sum-exp, base 2
+  int4* slot_plan;   // (chunk slots): {token row of the sequence, chunk, chunks of the sequence, its first slot}, for the merge
   int batch_size;
   int h_q;
   int page_size;
   int page_shift;    // log2(page_size) when it is a power of two, else -1
   int causal;
-  int split;         // 1: decode-shaped call, the KV of a sequence is cut into chunks (see mla_chunk_slot_begin)
-  int chunk_tokens;  // target tokens per chunk
+  int split;         // 1: decode-shaped call, the KV of the sequences is cut into chunks (see mla_split_plan)
+  int min_chunk_tiles;  // split: lower bound of the chunk length
   int row_tiles;     // split: row tiles of a one-token sequence, ceil(h_q / MLA_BM)
   float scale_log2;
 };
@@ -90,9 +98,29 @@ __device__ __forceinline__ int mla_swizzle(int row) {
 // around accumulation-register reads and writes are written out where they are needed.  The file
 // must be compiled with -mllvm -amdgpu-spill-vgpr-to-agpr=0 so that no spill lands in these
 // registers.
+// Every statement that touches them names all 256 as clobbered: a value of the compiler's own can then
+// not sit in one across such a statement (under register pressure it parks values there otherwise), and
+// check_mla_isa.py verifies on the generated assembly that none does in between either.
+#define MLA_ACC_REGS \
+  "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", \
+  "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31", \
+  "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47", \
+  "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63", \
+  "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79", \
+  "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95", \
+  "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111", \
+  "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127", \
+  "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143", \
+  "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159", \
+  "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", \
+  "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", \
+  "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207", \
+  "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223", \
+  "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", \
+  "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
 template <int R>
 __device__ __forceinline__ void acc_mfma_32x32x16(half8_t a, half8_t b) {  // a[R:R+15] += a * b
-  asm volatile("v_mfma_f32_32x32x16_f16 a[%2:%3], %0, %1, a[%2:%3]" : : "v"(a), "v"(b), "n"(R), "n"(R + 15));
+  asm volatile("v_mfma_f32_32x32x16_f16 a[%2:%3], %0, %1, a[%2:%3]" : : "v"(a), "v"(b), "n"(R), "n"(R + 15) : MLA_ACC_REGS);
 }
 // The same with an order token: `tok` is an operand the instruction does not touch.  Vector work that
 // is made to depend on it (pin_after) cannot be scheduled before this matrix instruction, and a
@@ -101,25 +129,25 @@ __device__ __forceinline__ void acc_mfma_32x32x16(half8_t a, half8_t b) {  // a[
 // to use both pipes at once (it issues in order).
 template <int R>
 __device__ __forceinline__ void acc_mfma_32x32x16(half8_t a, half8_t b, float& tok) {
-  asm volatile("v_mfma_f32_32x32x16_f16 a[%3:%4], %1, %2, a[%3:%4]" : "+v"(tok) : "v"(a), "v"(b), "n"(R), "n"(R + 15));
+  asm volatile("v_mfma_f32_32x32x16_f16 a[%3:%4], %1, %2, a[%3:%4]" : "+v"(tok) : "v"(a), "v"(b), "n"(R), "n"(R + 15) : MLA_ACC_REGS);
 }
 __device__ __forceinline__ void pin_after(float& x, float on) { asm("" : "+v"(x) : "v"(on)); }  // no instruction
 
 template <int R>
 __device__ __forceinline__ void acc_zero() {
-  asm volatile("v_accvgpr_write_b32 a[%0], 0" : : "n"(R));
+  asm volatile("v_accvgpr_write_b32 a[%0], 0" : : "n"(R) : MLA_ACC_REGS);
 }
 template <int R>
 __device__ __forceinline__ float acc_read() {
   float x;
-  asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(R));
+  asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(R) : MLA_ACC_REGS);
   return x;
 }
 template <int R>
 __device__ __forceinline__ void acc_scale(float factor) {
   float t;
   asm volatile("v_accvgpr_read_b32 %0, a[%2]\n\tv_mul_f32 %0, %0, %1\n\tv_accvgpr_write_b32 a[%2], %0"
-               : "=&v"(t) : "v"(factor), "n"(R));
+               : "=&v"(t) : "v"(factor), "n"(R) : MLA_ACC_REGS);
 }
 // wait states between the last matrix instruction that writes an accumulation register and a vector
 // instruction that reads it (or the reverse), more than any case needs
@@ -132,6 +160,153 @@ __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int
 template <int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {  // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
   static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// ---- the split of a decode-shaped call ---------------------------------------------------------------
+constexpr int MLA_MAX_SPLIT_BATCH = 128;  // two sequences per lane
+
+// What a lane knows of the two sequences it looks after (lane and lane + 64).
+struct MlaSeqInfo {
+  int q_start, qo_len, pbeg, npages, kv_len;
+  int cost;  // KV tiles a split launch has to walk: 0 for a sequence that is empty or not a decode step
+};
+__device__ __forceinline__ MlaSeqInfo mla_seq_info(const MlaParams& p, int b) {
+  MlaSeqInfo s{0, 0, 0, 0, 0, 0};
+  if (b < p.batch_size) {
+    s.q_start = p.q_indptr[b];
+    s.qo_len = p.q_indptr[b + 1] - s.q_start;
+    s.pbeg = p.page_indptr[b];
+    s.npages = p.page_indptr[b + 1] - s.pbeg;
+    s.kv_len = s.npages > 0 ? (s.npages - 1) * p.page_size + p.last_page_len[b] : 0;
+    s.cost = s.qo_len == 1 ? (s.kv_len + MLA_BN - 1) / MLA_BN : 0;
+  }
+  return s;
+}
+// ceil(a / c) for 0 <= a < 2^22, c >= 1, rc = 1.0f / c: the float product is off by less than one
+__device__ __forceinline__ int mla_ceil_div(int a, int c, float rc) {
+  const int x = a + c - 1;
+  int q = static_cast<int>(static_cast<float>(x) * rc);
+  const int r = x - q * c;
+  q += r >= c ? 1 : 0;
+  q -= r < 0 ? 1 : 0;
+  return q;
+}
+__device__ __forceinline__ int mla_lane_value(int v0, int v1, int b) {  // b is the same in every lane
+  return b < 64 ? __builtin_amdgcn_readlane(v0, b) : __builtin_amdgcn_readlane(v1, b - 64);
+}
+
+struct MlaSplit {
+  int b, chunk, nchunks;  // nchunks == 0: the slot is not in use
+  int first;              // first chunk slot of the sequence
+};
+// Sum over the wave of small non-negative integers (exact: the total stays below 2^24).
+__device__ __forceinline__ int mla_wave_sum(int x) {
+  const uint32_t rows = __float_as_uint(group_sum<16>(static_cast<float>(x)));  // every lane: the sum of its row of 16
+  return static_cast<int>(__uint_as_float(__builtin_amdgcn_readlane(rows, 0)) + __uint_as_float(__builtin_amdgcn_readlane(rows, 16)) +
+                          __uint_as_float(__builtin_amdgcn_readlane(rows, 32)) + __uint_as_float(__builtin_amdgcn_readlane(rows, 48)));
+}
+// Chunk slots: sequence b gets n_b = max(1, ceil(cost_b / c)) consecutive slots, c being the smallest
+// chunk length (in tiles, at least p.min_chunk_tiles) for which all of them fit into `slots`; its tiles
+// are divided evenly among its n_b chunks.  The total cost T bounds c from both sides, ceil(T / slots) <= c
+// <= ceil(T / (slots - batch)), and a bisection of that (narrow) range finds it, every lane working out the
+// chunks of its own two sequences.  Integer arithmetic on values every workgroup reads alike: all
+// workgroups, and the merge kernel, arrive at the same plan.
+__device__ __forceinline__ MlaSplit mla_split_plan(const MlaParams& p, const MlaSeqInfo& s0, const MlaSeqInfo& s1,
+                                                   int slots, int cslot, int lane) {
+  const int batch = p.batch_size;
+  const bool have0 = lane < batch, have1 = lane + 64 < batch;
+  int n0 = 0, n1 = 0;
+  auto chunks_with = [&](int c) {
+    const float rc = 1.0f / static_cast<float>(c);
+    n0 = have0 ? max(1, mla_ceil_div(s0.cost, c, rc)) : 0;
+    n1 = have1 ? max(1, mla_ceil_div(s1.cost, c, rc)) : 0;
+    return mla_wave_sum(n0 + n1);
+  };
+  const int total = mla_wave_sum(s0.cost + s1.cost);
+  int lo = max(p.min_chunk_tiles, (total + slots - 1) / slots);
+  int hi = max(lo, (total + (slots - batch) - 1) / (slots - batch));  // fits: at most total / hi + batch chunks
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (chunks_with(mid) <= slots) {
+      hi = mid;
+    } else {
+      lo = mid + 1;
+    }
+  }
+  chunks_with(hi);
+  int first = 0;
+  for (int b = 0; b < batch; ++b) {
+    const int n = mla_lane_value(n0, n1, b);
+    if (cslot < first + n) return MlaSplit{b, cslot - first, n, first};
+    first += n;
+  }
+  return MlaSplit{0, 0, 0, 0};
+}
+
+// Merge of the chunk states of heads [h_lo, h_hi) of a one-token sequence: out = sum_c w_c O_c / sum_c w_c
+// with w_c = 2^(lse_c - max lse), the arithmetic of merge_state_inplace (_decode_kernels.py:441-450) over
+// all chunks, CB at a time with a running maximum.  A wave takes four heads at once, 16 lanes and 32
+// features per lane each, and every lane works out the weights of its head for itself: no exchange
+// between lanes, and the loads of CB chunks (CB log-sum-exps and 4 CB x 16 bytes per lane) are in
+// flight together -- the merge is a chain of memory round trips and nothing else.
+template <int DV, int CB>
+__device__ __forceinline__ void mla_merge_heads(const MlaParams& p, int q_row, int first, int nchunks, int h_lo, int h_hi,
+                                                int wave, int waves, int lane) {
+  static_assert(DV == 512, "16 lanes x 32 features");
+  const int sub = lane >> 4;   // which of the wave's four heads
+  const int part = lane & 15;  // features part*32 .. +31
+  for (int h0 = h_lo; h0 < h_hi; h0 += waves * 4) {
+    const int h = h0 + wave * 4 + sub;
+    const bool valid = h < h_hi;
+    const int hh = valid ? h : h_lo;  // lanes without a head repeat a valid one and drop the result
+    float acc[32];
+#pragma unroll
+    for (int e = 0; e < 32; ++e) acc[e] = 0.f;
+    float top = -3.0e38f, wsum = 0.f;
+    for (int c0 = 0; c0 < nchunks; c0 += CB) {
+      float lse_c[CB];
+      half8_t o_c[CB][4];
+#pragma unroll
+      for (int k = 0; k < CB; ++k) {
+        const int c = min(c0 + k, nchunks - 1);  // past the end: the last chunk again, with weight 0
+        const int64_t row = static_cast<int64_t>(first + c) * p.h_q + hh;
+        lse_c[k] = p.part_lse[row];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o_c[k][j] = *reinterpret_cast<const half8_t*>(p.part_o + row * DV + part * 32 + j * 8);
+      }
+      float block_top = top;
+#pragma unroll
+      for (int k = 0; k < CB; ++k) block_top = fmaxf(block_top, c0 + k < nchunks ? lse_c[k] : -3.0e38f);
+      const float keep = fast_exp2(top - block_top);  // 0 in the first round
+      top = block_top;
+      wsum *= keep;
+#pragma unroll
+      for (int e = 0; e < 32; ++e) acc[e] *= keep;
+#pragma unroll
+      for (int k = 0; k < CB; ++k) {
+        const float w = c0 + k < nchunks ? fast_exp2(lse_c[k] - top) : 0.f;
+        wsum += w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[j * 8 + e] = fmaf(static_cast<float>(o_c[k][j][e]), w, acc[j * 8 + e]);
+        }
+      }
+    }
+    if (valid) {
+      const float inv = 1.0f / wsum;  // the chunk that holds the maximum weighs 1
+      const int64_t grow = static_cast<int64_t>(q_row) * p.h_q + h;
+      half_t* out = p.output + grow * DV + part * 32;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        half8_t out8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out8[e] = static_cast<half_t>(acc[j * 8 + e] * inv);
+        *reinterpret_cast<half8_t*>(out + j * 8) = out8;
+      }
+      if (part == 0) p.lse[grow] = top + fast_log2(wsum);
+    }
+  }
 }
 
 // POW2: the page size is a power of two (p.page_shift), so that a token's page and slot are a shift
@@ -152,6 +327,7 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   constexpr int COPIES = NCOPY / MLA_WAVES;  // per wave and tile
 
   extern __shared__ __attribute__((aligned(16))) half_t lds_tiles[];
+  // (no static LDS beside it: the fragment addressing XORs address bits and needs the stages at offset 0)
   asm volatile("" ::: "a0", "a255");  // the kernel uses every accumulation register (by number, see above)
 
   const int tid = threadIdx.x;
@@ -162,24 +338,32 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   // sequence), the grid holding exactly the items in use: a workgroup takes a whole compute unit
   // (LDS, registers) and runs long, and workgroups that only find out they have nothing to do
   // still disturb the placement of the others.
-  int b, r0, chunk = 0, nchunks = 1, cslot = 0, row_step = 0;
+  int b, r0, chunk = 0, nchunks = 1, cslot = 0, row_step = 0, first_slot = 0;
+  int q_start, qo_len, pbeg, npages, kv_len;
   if (p.split) {
-    cslot = blockIdx.x / p.row_tiles;
-    r0 = (blockIdx.x - cslot * p.row_tiles) * MLA_BM;
+    // Workgroup ids go round the XCDs; chunk slots are numbered so that consecutive ones -- the chunks
+    // of a sequence -- land on one XCD.
+    const int slots = gridDim.x / p.row_tiles;
+    const int wg = blockIdx.x / p.row_tiles;
+    cslot = slots % 8 == 0 ? (wg % 8) * (slots / 8) + wg / 8 : wg;
+    r0 = (blockIdx.x - wg * p.row_tiles) * MLA_BM;
     row_step = p.row_tiles * MLA_BM;
-    int lo = 0, hi = p.batch_size - 1;
-    while (lo < hi) {
-      int mid = (lo + hi + 1) >> 1;
-      if (mla_chunk_slot_begin(p.page_indptr, mid, p.page_size, p.chunk_tokens) <= cslot) {
-        lo = mid;
-      } else {
-        hi = mid - 1;
-      }
+    const int plan_lane = tid & 63;
+    const MlaSeqInfo s0 = mla_seq_info(p, plan_lane), s1 = mla_seq_info(p, plan_lane + 64);
+    const MlaSplit plan = mla_split_plan(p, s0, s1, slots, cslot, plan_lane);
+    if (tid == 0 && r0 == 0) {  // what the merge kernel needs to know of this slot (nchunks <= 1: nothing to merge)
+      p.slot_plan[cslot] = make_int4(mla_lane_value(s0.q_start, s1.q_start, plan.b), plan.chunk, plan.nchunks, plan.first);
     }
-    b = lo;
-    const int first = mla_chunk_slot_begin(p.page_indptr, b, p.page_size, p.chunk_tokens);
-    chunk = cslot - first;
-    nchunks = mla_chunk_slot_begin(p.page_indptr, b + 1, p.page_size, p.chunk_tokens) - first;
+    if (plan.nchunks == 0) return;  // a slot the plan does not use
+    b = plan.b;
+    chunk = plan.chunk;
+    nchunks = plan.nchunks;
+    first_slot = plan.first;
+    q_start = mla_lane_value(s0.q_start, s1.q_start, b);
+    qo_len = mla_lane_value(s0.qo_len, s1.qo_len, b);
+    pbeg = mla_lane_value(s0.pbeg, s1.pbeg, b);
+    npages = mla_lane_value(s0.npages, s1.npages, b);
+    kv_len = mla_lane_value(s0.kv_len, s1.kv_len, b);
   } else {
     const int slot = blockIdx.x;
     int lo = 0, hi = p.batch_size - 1;
@@ -193,20 +377,16 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
     }
     b = lo;
     r0 = (slot - mla_tile_slot_begin(p.q_indptr, b, h_q)) * MLA_BM;
+    q_start = p.q_indptr[b];
+    qo_len = p.q_indptr[b + 1] - q_start;
+    pbeg = p.page_indptr[b];
+    npages = p.page_indptr[b + 1] - pbeg;
+    kv_len = npages > 0 ? (npages - 1) * p.page_size + p.last_page_len[b] : 0;
   }
-  const int q_start = p.q_indptr[b];
-  const int qo_len = p.q_indptr[b + 1] - q_start;
   const int rows = qo_len * h_q;
-  if (p.split && qo_len != 1) {
-    // not a decode step after all: the workgroups of chunk 0 do the whole sequence, unsplit
-    if (chunk != 0) return;
-    nchunks = 1;
-  }
+  // (a sequence of a split call that is not a decode step is one chunk: its workgroup walks all its row tiles)
 
-  const int pbeg = p.page_indptr[b];
-  const int npages = p.page_indptr[b + 1] - pbeg;
   const int ps = p.page_size;
-  const int kv_len = npages > 0 ? (npages - 1) * ps + p.last_page_len[b] : 0;
 
   // normal mode: one pass; split mode: one pass per row tile this workgroup owns (one, for a decode step)
   for (; r0 < rows; r0 += row_step) {
@@ -236,6 +416,16 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   const int tile_lo = static_cast<int>(static_cast<int64_t>(chunk) * tiles_all / nchunks);
   const int tile_hi = min(static_cast<int>(static_cast<int64_t>(chunk + 1) * tiles_all / nchunks), (kv_end + BN - 1) / BN);
 
+  // The page ids of the first tiles are asked for ahead of the query rows: the first copies wait for them,
+  // and a wait for a load is a wait for every load issued before it.
+  const int last_tok = kv_len - 1;
+  int page_ids = 0;
+  auto load_page_ids = [&](int tile) {  // of 16 consecutive tiles (4 row groups each), lane = 4*tile + row group
+    const int t = min((tile + (lane >> 2)) * BN + (lane & 3) * 8, last_tok);
+    page_ids = p.page_values[pbeg + (POW2 ? t >> p.page_shift : t / ps)];
+  };
+  if (tile_lo < tile_hi) load_page_ids(tile_lo);
+  __builtin_amdgcn_sched_barrier(0);
   // Q^T fragments (B operand): column = query col, contraction slots = features ks*16 + half*8 .. +7
   half8_t qf[KS];
   {
@@ -256,21 +446,13 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   // also waits for every copy in flight, so it must be rare.
   const int copy_first = wave * COPIES;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds_tiles));
-  const int last_tok = kv_len - 1;
-  int page_ids = 0;
   // Per-lane part of a copy's source offset for rows that need no clamping: row lane/8 of the
   // 8-row group rg, piece (lane%8) ^ swizzle(rg*8 + lane/8) = this value ^ (rg << 4).
   const uint32_t copy_lane_off = (lane >> 3) * (DQK * 2) + (((lane & 7) ^ ((((lane >> 3) >> 1) & 1) << 2)) << 4);
   // General form of a tile's copies: a page id per 8-row group, rows past the end clamped.
-  auto load_page_ids = [&](int tile) {
-    if (((tile - tile_lo) & 15) == 0) {
-      const int t = min((tile + (lane >> 2)) * BN + (lane & 3) * 8, last_tok);
-      page_ids = p.page_values[pbeg + (POW2 ? t >> p.page_shift : t / ps)];
-    }
-  };
   auto issue_tile = [&](int tile) {
-    load_page_ids(tile);
     const int w = tile - tile_lo;
+    if (w != 0 && (w & 15) == 0) load_page_ids(tile);  // the wait for it also waits for every copy in flight: rare
     const int kv0 = tile * BN;
     const uint32_t stage = lds_base + (w % NSTAGE) * (STAGE * 2);
 #pragma unroll
@@ -299,8 +481,8 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
     // from it are then computed where they are used instead of being kept in nine registers
     tile_lane_off = copy_lane_off;
     asm volatile("" : "+v"(tile_lane_off));
-    load_page_ids(tile);
     const int w = tile - tile_lo;
+    if ((w & 15) == 0) load_page_ids(tile);
     const int page = __builtin_amdgcn_readlane(page_ids, (w & 15) * 4);
     tile_base = p.pages + (static_cast<int64_t>(page) * ps + ((tile * BN) & (ps - 1))) * DQK;
     tile_stage = lds_base + (w % NSTAGE) * (STAGE * 2);
@@ -370,13 +552,13 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
       if constexpr (t == 0) {
         // C = 0 as a literal instead of sixteen zeroed registers; the result must not share
         // registers with the operands
-        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a[0]), "v"(qf[0]));
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a[0]), "v"(qf[0]) : MLA_ACC_REGS);
       } else if constexpr (t == KS - 1) {
         // the compiler does not know this is a matrix instruction: the wait states it would put
         // between the last one and the first vector instruction that reads S are spelled out
-        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(acc) : "v"(a[t % RING]), "v"(qf[t]));
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(acc) : "v"(a[t % RING]), "v"(qf[t]) : MLA_ACC_REGS);
       } else {
-        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a[t % RING]), "v"(qf[t]));
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a[t % RING]), "v"(qf[t]) : MLA_ACC_REGS);
       }
       if constexpr (t + RING - 1 < KS) a[(t + RING - 1) % RING] = read_k_frag(k_at, t + RING - 1);
       beside(tc);
@@ -532,88 +714,72 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   // the row sums are per half of the wave: add them up; m is already common
   lsum = sum_xor32(lsum);
   acc_settle();  // the last PV product's results, before the vector ALU reads them
-  if (row_valid) {
-  const int64_t grow = static_cast<int64_t>(q_start + my_pos) * h_q + my_head;  // global row
   if (nchunks == 1) {
-    const float denom = lsum + fast_exp2(kNegInit - m);
-    const float inv = 1.0f / denom;
-    half_t* orow = p.output + grow * DV + half * 4;
+    if (row_valid) {
+      const int64_t grow = static_cast<int64_t>(q_start + my_pos) * h_q + my_head;  // global row
+      const float denom = lsum + fast_exp2(kNegInit - m);
+      const float inv = 1.0f / denom;
+      half_t* orow = p.output + grow * DV + half * 4;
+      static_for<DB * 4>([&](auto qc) {
+        constexpr int q4 = decltype(qc)::value;  // registers 4*q4 .. 4*q4+3: block q4/4, feature group q4%4
+        half4_t out4;
+        out4[0] = static_cast<half_t>(acc_read<q4 * 4 + 0>() * inv);
+        out4[1] = static_cast<half_t>(acc_read<q4 * 4 + 1>() * inv);
+        out4[2] = static_cast<half_t>(acc_read<q4 * 4 + 2>() * inv);
+        out4[3] = static_cast<half_t>(acc_read<q4 * 4 + 3>() * inv);
+        *reinterpret_cast<half4_t*>(orow + (q4 / 4) * 32 + (q4 % 4) * 8) = out4;
+      });
+      if (half == 0) p.lse[grow] = m + fast_log2(denom);
+    }
+  } else {
+    // A chunk of a one-token sequence (the row is the head).  Its state goes out normalised, in fp16,
+    // with the log-sum-exp beside it.  A lane holds 4 features of a head here and there; the rows are
+    // put together in LDS (the tile stages are free by now) and leave as whole 1 KiB rows.
+    constexpr int PSTRIDE = DV + 8;  // halfs: consecutive rows start 4 banks apart
+    static_assert(MLA_WAVES * 32 * PSTRIDE <= NSTAGE * STAGE, "the tile stages hold the rows of all waves");
+    __syncthreads();  // every wave is done with the tiles
+    half_t* wave_rows = lds_tiles + wave * (32 * PSTRIDE);
+    const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;  // a chunk without a visible token weighs nothing
     static_for<DB * 4>([&](auto qc) {
-      constexpr int q4 = decltype(qc)::value;  // registers 4*q4 .. 4*q4+3: block q4/4, feature group q4%4
+      constexpr int q4 = decltype(qc)::value;
       half4_t out4;
       out4[0] = static_cast<half_t>(acc_read<q4 * 4 + 0>() * inv);
       out4[1] = static_cast<half_t>(acc_read<q4 * 4 + 1>() * inv);
       out4[2] = static_cast<half_t>(acc_read<q4 * 4 + 2>() * inv);
       out4[3] = static_cast<half_t>(acc_read<q4 * 4 + 3>() * inv);
-      *reinterpret_cast<half4_t*>(orow + (q4 / 4) * 32 + (q4 % 4) * 8) = out4;
+      *reinterpret_cast<half4_t*>(wave_rows + col * PSTRIDE + (q4 / 4) * 32 + (q4 % 4) * 8 + half * 4) = out4;
     });
-    if (half == 0) p.lse[grow] = m + fast_log2(denom);
-  } else {
-    // only one-token sequences are split: the row is the head
-    const int64_t prow_idx = static_cast<int64_t>(cslot) * h_q + my_head;
-    float* prow = p.part_o + prow_idx * DV + half * 4;
-    static_for<DB * 4>([&](auto qc) {
-      constexpr int q4 = decltype(qc)::value;
-      const float4_t v4 = {acc_read<q4 * 4 + 0>(), acc_read<q4 * 4 + 1>(), acc_read<q4 * 4 + 2>(), acc_read<q4 * 4 + 3>()};
-      *reinterpret_cast<float4_t*>(prow + (q4 / 4) * 32 + (q4 % 4) * 8) = v4;
-    });
-    if (half == 0) {
-      p.part_ml[prow_idx * 2 + 0] = m;
-      p.part_ml[prow_idx * 2 + 1] = lsum;
+    // the rows are read back below through another type: keep the reads behind the writes
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const int head0 = r0 + wave * 32;
+    const int nrows = min(32, rows - head0);
+    half_t* dst = p.part_o + (static_cast<int64_t>(cslot) * h_q + head0) * DV + lane * 8;
+    for (int r4 = 0; r4 < nrows; r4 += 4) {  // four rows at a time: their LDS reads are in flight together
+      Vec16 v[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k].u = *reinterpret_cast<const uint4*>(wave_rows + min(r4 + k, 31) * PSTRIDE + lane * 8);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (r4 + k < nrows) st16(dst + (r4 + k) * DV, v[k]);
+      }
     }
-  }
+    if (row_valid && half == 0) p.part_lse[static_cast<int64_t>(cslot) * h_q + my_head] = lsum > 0.f ? m + fast_log2(lsum) : kNegInit;
   }
   if (row_step == 0) break;
   __syncthreads();  // the LDS stages are reused by the next pass
   }
 }
 
-// One block per (query token, head); DV/4 threads, 4 features each.
+// The merge of a split call: block i merges the i-th slice of the heads of the sequence that chunk slot i
+// belongs to (the kernel above left a note of the plan for every slot).
 template <int DV>
-__global__ __launch_bounds__(DV / 4) void mla_merge_kernel(MlaParams p) {
-  const int token = blockIdx.x;
-  const int head = blockIdx.y;
-  int b;
-  {
-    int lo = 0, hi = p.batch_size - 1;
-    while (lo < hi) {
-      int mid = (lo + hi + 1) >> 1;
-      if (p.q_indptr[mid] <= token) {
-        lo = mid;
-      } else {
-        hi = mid - 1;
-      }
-    }
-    b = lo;
-  }
-  // (sequences with qo_len == 0 share their q_indptr value with the next one: the search returns
-  // the last b with q_indptr[b] <= token, which is the one that owns the token)
-  if (p.q_indptr[b + 1] - p.q_indptr[b] != 1) return;  // only one-token sequences are split
-  const int first = mla_chunk_slot_begin(p.page_indptr, b, p.page_size, p.chunk_tokens);
-  const int nchunks = mla_chunk_slot_begin(p.page_indptr, b + 1, p.page_size, p.chunk_tokens) - first;
-  if (nchunks == 1) return;
-  const int64_t grow = static_cast<int64_t>(token) * p.h_q + head;
-  const int64_t prow = static_cast<int64_t>(first) * p.h_q + head;  // + c * h_q for chunk c
-  const float* ml = p.part_ml + prow * 2;
-  const int64_t cstride = p.h_q;
-  float mx = kNegInit;
-  for (int c = 0; c < nchunks; ++c) mx = fmaxf(mx, ml[c * cstride * 2]);
-  float lsum = 0.f;
-  float4_t acc = {0.f, 0.f, 0.f, 0.f};
-  const int d = threadIdx.x * 4;
-  for (int c = 0; c < nchunks; ++c) {
-    const float sc = fast_exp2(ml[c * cstride * 2] - mx);
-    lsum += ml[c * cstride * 2 + 1] * sc;
-    const float4_t po = *reinterpret_cast<const float4_t*>(p.part_o + (prow + c * cstride) * DV + d);
-    acc += po * sc;
-  }
-  const float denom = lsum + fast_exp2(kNegInit - mx);
-  const float inv = 1.0f / denom;
-  half4_t out4;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) out4[e] = static_cast<half_t>(acc[e] * inv);
-  *reinterpret_cast<half4_t*>(p.output + grow * DV + d) = out4;
-  if (threadIdx.x == 0) p.lse[grow] = mx + fast_log2(denom);
+__global__ __launch_bounds__(256) void mla_merge_kernel(MlaParams p) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int4 plan = p.slot_plan[blockIdx.x];  // {token row, chunk, nchunks, first slot}
+  if (plan.z <= 1) return;
+  mla_merge_heads<DV, 8>(p, plan.x, plan.w, plan.z, static_cast<int>(static_cast<int64_t>(plan.y) * p.h_q / plan.z),
+                         static_cast<int>(static_cast<int64_t>(plan.y + 1) * p.h_q / plan.z), wave, 4, lane);
 }
 
 }  // namespace tvmkv
@@ -654,29 +820,27 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
   const int64_t slots = total_q * h_q / MLA_BM + (h_q % MLA_BM != 0 ? batch_size : 0);
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_prefill_paged_kv_mla: too many row tiles";
-  // Decode-shaped calls (one token per sequence, as far as the shapes tell) have too few row
-  // tiles for the chip, so the KV of a sequence is cut into chunks of about chunk_tokens tokens.
-  // One workgroup per compute unit is resident (LDS), so aim at one round of workgroups:
-  // chunk slots = floor(tokens / chunk_tokens) + B, times the row tiles of a sequence, <= CUs.
+  // Decode-shaped calls (one token per sequence, as far as the shapes tell) have too few row tiles
+  // for the chip, so the KV of the sequences is cut into chunks.  One workgroup per compute unit is
+  // resident (LDS): the grid is one round of workgroups, and the kernel fits the chunks to it.
   const int cus = compute_units();
   const int row_tiles = (h_q + MLA_BM - 1) / MLA_BM;
-  const int64_t tokens = nnz_pages * page_size;  // upper bound on the cached tokens
   int64_t grid = slots;
-  if (total_q == batch_size && static_cast<int64_t>(batch_size) * row_tiles * 2 <= cus && tokens > 0) {
-    const int64_t room = cus / row_tiles - batch_size;
-    int64_t ct = (tokens + room - 1) / room;
-    ct = std::max<int64_t>(MLA_MIN_CHUNK, (ct + MLA_BN - 1) / MLA_BN * MLA_BN);
-    if (option(kOptMlaChunkTokens) >= MLA_BN) ct = option(kOptMlaChunkTokens) / MLA_BN * MLA_BN;  // tuning aid
-    const int64_t cslots = tokens / ct + batch_size;
+  if (total_q == batch_size && static_cast<int64_t>(batch_size) * row_tiles * 2 <= cus && batch_size <= MLA_MAX_SPLIT_BATCH &&
+      nnz_pages > 0 && nnz_pages * page_size < (int64_t{1} << 26)) {
+    const int64_t cslots = cus / row_tiles;
     p.split = 1;
-    p.chunk_tokens = static_cast<int>(ct);
     p.row_tiles = row_tiles;
+    p.min_chunk_tiles = MLA_MIN_CHUNK / MLA_BN;
+    if (option(kOptMlaChunkTokens) >= MLA_BN) p.min_chunk_tiles = static_cast<int>(option(kOptMlaChunkTokens) / MLA_BN);  // tuning aid
     grid = cslots * row_tiles;
     const size_t part_rows = static_cast<size_t>(cslots) * h_q;
-    const size_t part_o_bytes = part_rows * DV * sizeof(float);
-    char* ws = lease_scratch(kScratchMla, as_stream(stream), part_o_bytes + part_rows * 2 * sizeof(float), 0).ptr;
-    p.part_o = reinterpret_cast<float*>(ws);
-    p.part_ml = reinterpret_cast<float*>(ws + part_o_bytes);
+    const size_t part_o_bytes = part_rows * DV * sizeof(half_t);
+    const size_t part_lse_bytes = (part_rows * sizeof(float) + 15) / 16 * 16;
+    char* ws = lease_scratch(kScratchMla, as_stream(stream), part_o_bytes + part_lse_bytes + cslots * sizeof(int4), 0).ptr;
+    p.part_o = reinterpret_cast<half_t*>(ws);
+    p.part_lse = reinterpret_cast<float*>(ws + part_o_bytes);
+    p.slot_plan = reinterpret_cast<int4*>(ws + part_o_bytes + part_lse_bytes);
   }
   constexpr size_t lds_bytes = static_cast<size_t>(MLA_STAGES) * MLA_BN * DQK * sizeof(half_t);
   static bool attr_set = false;
@@ -701,7 +865,7 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
   }
   KV_LAUNCH_CHECK();
   if (p.split) {
-    hipLaunchKernelGGL(mla_merge_kernel<DV>, dim3(static_cast<unsigned>(total_q), h_q), dim3(DV / 4), 0, s, p);
+    hipLaunchKernelGGL(mla_merge_kernel<DV>, dim3(static_cast<unsigned>(grid / row_tiles)), dim3(256), 0, s, p);
     KV_LAUNCH_CHECK();
   }
   KV_API_END();

@@ -14,8 +14,8 @@ enum Option {
   kOptDecodeChunkPages = 0,   // pages per split-KV chunk of the decode kernel, 0 = derived from the shapes
   kOptDecodeSeparateMerge,    // != 0: merge the chunks in a second launch instead of inside the kernel
   kOptDecodeWgsPerCu,         // > 0: cap the decode grid at this many workgroups per compute unit
-  kOptMlaChunkTokens,         // tokens per split-KV chunk of the MLA kernel, 0 = derived from the shapes
-  kOptMlaSeparateMerge,       // != 0: merge the MLA chunks in a second launch
+  kOptMlaChunkTokens,         // lower bound of the tokens per split-KV chunk of the MLA kernel, 0 = 128
+  kOptMlaSeparateMerge,       // unused (the MLA chunks are always merged in a second launch)
   kNumOptions
 };
 int64_t option(Option id);

@@ -32,13 +32,6 @@ TVMKV_HD int find_sequence(const int32_t* page_indptr, int batch, int cp, int sl
   return lo;
 }
 
-// MLA decode: sequence b owns the chunk slots [mla_chunk_slot_begin(b), mla_chunk_slot_begin(b + 1)),
-// a function of the page table alone (at most floor(nnz_pages * page_size / chunk_tokens) + batch
-// slots, every one of them in use), and its KV tiles are divided evenly among them.
-TVMKV_HD int mla_chunk_slot_begin(const int32_t* page_indptr, int b, int page_size, int chunk_tokens) {
-  return static_cast<int>(static_cast<int64_t>(page_indptr[b]) * page_size / chunk_tokens) + b;
-}
-
 }  // namespace tvmkv
 
 #endif  // TVMKV_CSRC_SPLIT_PLAN_H_
