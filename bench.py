@@ -252,6 +252,37 @@ def extras(torch, K, dev):
                                     "ms": round(ms, 4), "GBps": round(nbytes / ms / 1e6, 1),
                                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
 
+    # ---- paged prefill through the sliding-window form of the kernel (three-row length_info, per-layer
+    # window) against the plain form on the same keys: configs[2]'s sequences, every key visible --------
+    rng2 = np.random.default_rng(2)
+    pre = rng2.integers(0, 4096, size=8, endpoint=True)
+    chunk = rng2.integers(128, 2048, size=8, endpoint=True)
+    kvp = pre + chunk
+    npg = (kvp + ps - 1) // ps
+    ipp = np.concatenate([[0], np.cumsum(npg)])
+    qip = np.concatenate([[0], np.cumsum(chunk)])
+    nq = int(qip[-1])
+    qp = torch.randn((nq, hq, d), device=dev).to(torch.float16)
+    op = torch.empty_like(qp)
+    lp = torch.empty((nq, hq), dtype=torch.float32, device=dev)
+    z8, zq = torch.zeros(8, dtype=torch.int32, device=dev), torch.zeros(nq, dtype=torch.int32, device=dev)
+    last = (kvp - 1) % ps + 1
+    plain = (qp, i32(qip), pages, i32(ipp), i32(perm[:ipp[-1]]), i32(last), z8, zq, op, lp, 0, 0, 1.0, 1e4, d ** -0.5)
+    three = i32(np.stack([last, np.zeros(8, dtype=np.int64), np.zeros(8, dtype=np.int64)]))
+    slid = (qp, i32(qip), pages, i32(ipp), i32(perm[:ipp[-1]]), three, z8, zq, op, lp, 1, 0, 1.0, 1e4, d ** -0.5)
+    K.batch_prefill_paged_kv(*plain)
+    ms_plain = time_region(torch, lambda i: K.batch_prefill_paged_kv(*plain), 10)
+    K.batch_prefill_paged_kv(*slid, sliding_window_size=1 << 20)
+    ms_slid = time_region(torch, lambda i: K.batch_prefill_paged_kv(*slid, sliding_window_size=1 << 20), 10)
+    flops = 4.0 * hq * d * float(np.sum(chunk * kvp))
+    out["sliding_window_prefill"] = {"workload": "configs[2]'s 8 sequences (prefix U[0,4096] + chunk U[128,2048], seed 2), the chunk's "
+                                                 "queries against all cached keys: plain kernel, and the sliding-window form "
+                                                 "(length_info with 3 rows, per-layer window mask) with a window that covers them",
+                                     "ms_plain": round(ms_plain, 4), "ms_sliding_form": round(ms_slid, 4),
+                                     "sliding_over_plain": round(ms_slid / ms_plain, 3),
+                                     "tflops_sliding_form": round(flops / ms_slid / 1e9, 1),
+                                     "frac_of_mfma_peak": round(flops / ms_slid / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+
     def preorder(depth):  # (first, second) labels of a complete binary tree listed in depth-first order
         labels = []
 

@@ -202,9 +202,14 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     tree_base = p.tree_order + 2 * static_cast<int64_t>(first_node);
     if (tree_len > 0) child_first = tree_base[2 * min(max(my_pos + tree_len - qo_len, 0), tree_len - 1)];
   }
-  // tiles that end at or before this (physical = logical) index need no mask at all
-  const bool plain_ext = EXT && !p.rotary && p.sink_size == nullptr;
-  const int unmasked_limit = !EXT ? wave_limit_min : (plain_ext ? min(wave_limit_min, max(tree_start, 0)) : 0);
+  // Tiles whose keys every row of the wave sees need no mask at all.  Plain cache: the tiles that end
+  // at or before unmasked_limit.  EXT without in-kernel RoPE: a tile that lies wholly among the attention
+  // sinks or wholly in the window, in front of the tree nodes and of the causal bound of the wave's first
+  // row, and behind the per-layer window start of its last row (logical key indices ext_lo .. ext_hi).
+  const int unmasked_limit = !EXT ? wave_limit_min : 0;
+  const bool ext_fast = EXT && !p.rotary;
+  const int ext_hi = min(wave_limit_min, max(tree_start, 0));
+  const int ext_lo = (layer_mask && wave_active) ? max(kv_len - max(p.layer_window - last_row_wave / group - 1, 0), 0) : 0;
 
   half8_t qf[KS];
   {
@@ -472,7 +477,14 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     const int t_limit_max = hole ? (wave_active ? prefix_len : 0) : wave_limit_max;
     const int t_limit_min = hole ? t_limit_max : wave_limit_min;
     const int t_my_limit = hole ? (row_valid ? prefix_len : 0) : my_limit;
-    const bool unmasked = TB == 2 && kv0 < t_limit_max && kv0 + BN <= (hole ? t_limit_max : unmasked_limit);  // wave-uniform
+    bool unmasked = TB == 2 && kv0 < t_limit_max && kv0 + BN <= (hole ? t_limit_max : unmasked_limit);  // wave-uniform
+    if (EXT) {
+      const bool in_sink = kv0 + BN <= sink;
+      const bool in_window = kv0 >= win_lo && kv0 + BN <= phys_len;
+      const int first_key = in_sink ? kv0 : kv0 - win_lo + sink;  // logical index of the tile's first key
+      unmasked = TB == 2 && ext_fast && kv0 < t_limit_max && (in_sink || in_window) && first_key >= ext_lo &&
+                 first_key + BN <= ext_hi;
+    }
     if (has_next) issue_tile(next);
 
     if (kv0 >= t_limit_max) continue;  // wave-uniform: every row of this wave is masked out
