@@ -226,10 +226,8 @@ int tvmkv_batch_prefill_cached_and_new_kv_fused_q(const void* qkv, const int32_t
  *  lse, rotary_mode, rope_scale, rope_theta, sm_scale).
  * q/out (B, h_q, d) fp16, lse (B, h_q) fp32.  Split-KV across workgroups with a merge pass;
  * the partition count is derived from B and nnz_pages only (no host read of the page table).
- * The (3, batch) length_info and rotary_mode = 1 are built into the kernel for head_dim 128 and GQA
- * groups up to 16; for them other shapes take the paged prefill kernel with one query per
- * sequence (same results, no split over the keys), and so do GQA groups other than 1, 2, 4, 8
- * with head_dim 64 or above 16 with head_dim 128 on a plain cache. */
+ * Head dims 64 and 128, any GQA group (groups above 16 are walked in blocks of 16 heads), with the
+ * (3, batch) length_info and rotary_mode = 1 built in for all of them. */
 int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t* page_indptr,
                                 const int32_t* page_values, const int32_t* length_info,
                                 const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,

@@ -267,11 +267,12 @@ def test_decode_rejects_what_is_not_built():
 
 
 def test_decode_large_gqa_groups_plain_cache():
-    """Multi-query shapes (one kv head for 32 or 12 query heads) on a plain cache: groups the decode
-    kernels are not built for take the paged prefill kernel."""
-    for hq, hkv, d in ((32, 1, 128), (12, 1, 64), (24, 2, 64)):
+    """Multi-query shapes (one kv head for 32 or 12 query heads) on a plain cache: groups above 16 heads
+    are walked in blocks of 16, groups that are not a power of two leave columns of the tile empty."""
+    for hq, hkv, d in ((32, 1, 128), (12, 1, 64), (24, 2, 64), (40, 1, 128), (80, 2, 64)):
         rng = np.random.default_rng(27)
-        go, gl, eo, el = _decode_both(rng, [5, 130, 1000, 16], hq, hkv, d, 80)
+        # 5000 tokens: several chunks, merged per block of 16 heads by the last workgroup to arrive
+        go, gl, eo, el = _decode_both(rng, [5, 130, 5000, 16], hq, hkv, d, 330)
         assert_close(go, eo, what=f"decode out {hq}/{hkv}/{d}")
         assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"decode lse {hq}/{hkv}/{d}")
 
@@ -279,8 +280,7 @@ def test_decode_large_gqa_groups_plain_cache():
 @pytest.mark.parametrize("rotary", [0, 1])
 @pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (16, 16, 64), (32, 1, 128)])
 def test_decode_sliding_cache_and_inline_rope_other_shapes(hq, hkv, d, rotary):
-    """Shapes outside the matrix-core decode kernel (head_dim 64, GQA groups above 16) take the paged
-    prefill kernel with one query per sequence."""
+    """Head dim 64 and GQA groups above 16 through the sliding-window / inline-RoPE form of the decode kernel."""
     from tests.test_oracle_kernels import SLIDING_SPEC, sliding_case
     rng = np.random.default_rng(26)
     pages, pindptr, pvalues, length_info, ks, vs = sliding_case(rng, SLIDING_SPEC, hkv, d)

@@ -8,17 +8,11 @@
 // sm_scale*log2(e), base-2 online softmax with m = -5e4, d = 1 as the initial state, fp32
 // accumulation, output O/d rounded once to fp16, lse = m + log2(d).
 //
-// Data path of one workgroup (4 wavefronts, one kv head, all `GROUP` query heads of it):
-//   * wave w takes pages w, w+4, ... of the chunk; a page of one kv head is 4 KiB of K and
-//     4 KiB of V, each contiguous, read with 16-byte loads: 16 lanes cover one 256-byte row,
-//     one wave-wide load covers 4 rows = 1 KiB, fully coalesced; the next page's loads are
-//     issued before the current page is consumed;
-//   * q.k: packed fp16 dot products accumulate in fp32 per lane, then a 4-step DPP reduction
-//     inside the 16-lane row; every 16-lane group keeps its own online-softmax state, so the
-//     inner loop has no cross-group traffic;
-//   * at the end the four lane groups are merged with wavefront shuffles, the four waves
-//     through LDS, and the chunk result goes either straight to the output (single-chunk
-//     sequence) or to the fp32 partial buffer.
+// One workgroup (4 wavefronts) takes one chunk of one kv head and up to 16 of the query heads that
+// share it (a larger GQA group is walked in blocks of 16 heads by neighbouring workgroups, which read
+// the same pages); decode_mfma_kernel below describes the data path.  The chunk result goes either
+// straight to the output (single-chunk sequence) or to the fp32 partial buffer, and the workgroup
+// that delivers the last partial state of a (sequence, kv head, head block) merges them.
 //
 // Chunk slots without a prologue kernel: sequence b owns slots
 //   [floor(page_indptr[b]/CP) + b, floor(page_indptr[b+1]/CP) + b + 1)
@@ -79,183 +73,6 @@ __device__ __forceinline__ int find_sequence_wave(const int32_t* page_indptr, in
     if (count < 64) break;
   }
   return b;
-}
-
-template <int D, int GROUP, int PS>
-__global__ __launch_bounds__(256) void decode_splitkv_kernel(DecodeParams p) {
-  constexpr int LPR = D / 8;         // lanes per K/V row
-  constexpr int TPL = 64 / LPR;      // rows (tokens) covered by one wave-wide 16-byte load
-  constexpr int LOADS = PS / TPL;    // loads per page for K (and as many for V)
-  constexpr int NGRP = TPL;          // independent lane groups per wave
-  static_assert(PS % TPL == 0, "page must be a whole number of wave-wide loads");
-
-  const int slot = blockIdx.x;
-  const int kvh = blockIdx.y;
-  const int tid = threadIdx.x;
-  const int wave = tid >> 6;
-  const int lane = tid & 63;
-  const int grp = lane / LPR;   // which row of a wave-wide load this lane reads
-  const int sub = lane % LPR;   // which 16-byte piece of the row
-
-  const int cp = p.chunk_pages;
-  const int b = find_sequence(p.page_indptr, p.batch_size, cp, slot);
-  const int pbeg = p.page_indptr[b];
-  const int pend = p.page_indptr[b + 1];
-  const int npages = pend - pbeg;
-  const int chunk = slot - slot_begin(p.page_indptr, b, cp);
-  const int nchunks = (npages + cp - 1) / cp;
-  if (chunk >= nchunks) return;  // spare slot
-  const int kv_len = (npages - 1) * PS + p.last_page_len[b];
-  const int page_lo = chunk * cp;
-  const int page_hi = min(page_lo + cp, npages);
-
-  // q of the GROUP heads sharing this kv head: the 8 features this lane owns, packed fp16.
-  Vec16 qv[GROUP];
-#pragma unroll
-  for (int g = 0; g < GROUP; ++g) {
-    qv[g] = ld16(p.q + (static_cast<int64_t>(b) * p.h_q + kvh * GROUP + g) * D + sub * 8);
-  }
-
-  float m[GROUP], l[GROUP], o[GROUP][8];
-#pragma unroll
-  for (int g = 0; g < GROUP; ++g) {
-    m[g] = kNegInit;
-    l[g] = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) o[g][e] = 0.f;
-  }
-
-  const int64_t head_stride = static_cast<int64_t>(PS) * D;  // elements of one (page, k|v, head)
-  auto issue = [&](int page_idx, Vec16* kreg, Vec16* vreg) {
-    const int page = __builtin_amdgcn_readfirstlane(p.page_values[pbeg + page_idx]);
-    const half_t* kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * head_stride + lane * 8;
-    const half_t* vbase = kbase + static_cast<int64_t>(p.h_kv) * head_stride;
-#pragma unroll
-    for (int j = 0; j < LOADS; ++j) {
-      kreg[j] = ld16_nt(kbase + j * TPL * D);
-      vreg[j] = ld16_nt(vbase + j * TPL * D);
-    }
-  };
-
-  auto consume = [&](int page_idx, const Vec16* kreg, Vec16* vreg) {
-    const int tok0 = page_idx * PS + grp;  // token of load j is tok0 + j*TPL
-    const bool partial = (page_idx + 1) * PS > kv_len;  // wave-uniform: only the last page
-    bool valid[LOADS];
-#pragma unroll
-    for (int j = 0; j < LOADS; ++j) {
-      valid[j] = !partial || (tok0 + j * TPL < kv_len);
-      if (partial && !valid[j]) vreg[j] = zero16();  // slots beyond kv_len hold arbitrary bits
-    }
-#pragma unroll
-    for (int g = 0; g < GROUP; ++g) {
-      float s[LOADS];
-      float mx = m[g];
-#pragma unroll
-      for (int j = 0; j < LOADS; ++j) {
-        float acc = 0.f;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2(qv[g].h2[e], kreg[j].h2[e], acc, false);
-        acc = group_sum<LPR>(acc) * p.scale_log2;
-        s[j] = valid[j] ? acc : kNegInit;
-        mx = fmaxf(mx, s[j]);
-      }
-      const float alpha = fast_exp2(m[g] - mx);
-      m[g] = mx;
-      l[g] *= alpha;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) o[g][e] *= alpha;
-#pragma unroll
-      for (int j = 0; j < LOADS; ++j) {
-        const float pj = valid[j] ? fast_exp2(s[j] - mx) : 0.f;
-        l[g] += pj;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[g][e] = fmaf(pj, static_cast<float>(vreg[j].h[e]), o[g][e]);
-      }
-    }
-  };
-
-  // Two register buffers: the loads of the next page are in flight while this one is consumed.
-  Vec16 k0[LOADS], v0[LOADS], k1[LOADS], v1[LOADS];
-  int pi = page_lo + wave;
-  if (pi < page_hi) issue(pi, k0, v0);
-  while (pi < page_hi) {
-    const int pn = pi + 4;
-    if (pn < page_hi) issue(pn, k1, v1);
-    consume(pi, k0, v0);
-    pi = pn;
-    if (pi >= page_hi) break;
-    const int pn2 = pi + 4;
-    if (pn2 < page_hi) issue(pn2, k0, v0);
-    consume(pi, k1, v1);
-    pi = pn2;
-  }
-
-  // ---- merge the NGRP lane groups of this wave (butterfly over the group index) -------------
-#pragma unroll
-  for (int g = 0; g < GROUP; ++g) {
-#pragma unroll
-    for (int off = LPR; off < 64; off <<= 1) {
-      const float m_o = __shfl_xor(m[g], off, 64);
-      const float l_o = __shfl_xor(l[g], off, 64);
-      const float mx = fmaxf(m[g], m_o);
-      const float a = fast_exp2(m[g] - mx);
-      const float bsc = fast_exp2(m_o - mx);
-      l[g] = l[g] * a + l_o * bsc;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float o_o = __shfl_xor(o[g][e], off, 64);
-        o[g][e] = o[g][e] * a + o_o * bsc;
-      }
-      m[g] = mx;
-    }
-  }
-  (void)NGRP;
-
-  // ---- merge the 4 waves through LDS --------------------------------------------------------
-  __shared__ float sm_o[4][GROUP][D];
-  __shared__ float sm_m[4][GROUP];
-  __shared__ float sm_l[4][GROUP];
-  if (grp == 0) {
-#pragma unroll
-    for (int g = 0; g < GROUP; ++g) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) sm_o[wave][g][sub * 8 + e] = o[g][e];
-      if (sub == 0) {
-        sm_m[wave][g] = m[g];
-        sm_l[wave][g] = l[g];
-      }
-    }
-  }
-  __syncthreads();
-
-  const bool single_chunk = nchunks == 1;
-  for (int idx = tid; idx < GROUP * D; idx += 256) {
-    const int g = idx / D;
-    const int d = idx % D;
-    float mx = sm_m[0][g];
-#pragma unroll
-    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, sm_m[w][g]);
-    float lsum = 0.f, acc = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float sc = fast_exp2(sm_m[w][g] - mx);
-      lsum += sm_l[w][g] * sc;
-      acc += sm_o[w][g][d] * sc;
-    }
-    const int hq = kvh * GROUP + g;
-    if (single_chunk) {
-      // the reference's initial state (m=-5e4, d=1) leaves a term exp2(-5e4 - m) in the sum
-      const float denom = lsum + fast_exp2(kNegInit - mx);
-      p.output[(static_cast<int64_t>(b) * p.h_q + hq) * D + d] = static_cast<half_t>(acc / denom);
-      if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = mx + fast_log2(denom);
-    } else {
-      p.part_o[(static_cast<int64_t>(slot) * p.h_q + hq) * D + d] = acc;
-      if (d == 0) {
-        p.part_ml[(static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 0] = mx;
-        p.part_ml[(static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 1] = lsum;
-      }
-    }
-  }
 }
 
 // Merge of the per-chunk partial states of one (sequence, query head) row by one wavefront.
@@ -352,11 +169,11 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeParams p, int t
 }
 
 // ------------------------------------------------------------------------------------------
-// MFMA variant for head_dim 128 (any GQA group up to 16).
+// The decode kernel, for head dims 64 and 128 and any GQA group.
 //
-// The VALU kernel above spends ~90*GROUP vector instructions per 8 KiB page, which for groups of
+// A vector-ALU formulation spends ~90 instructions per query head and 8 KiB page, which for groups of
 // 4-8 query heads is about as much issue time as the page's HBM time.  Here the two contractions
-// run on v_mfma_f32_16x16x32_f16 with the query heads of the group padded to the 16-wide N axis:
+// run on v_mfma_f32_16x16x32_f16 with (a block of 16 of) the query heads of the group on the N axis:
 //   S^T[token, head] = K Q^T   -- K fragments come straight from global memory in the MFMA
 //                                 A-layout (lane = token row, 16 bytes of features), no staging;
 //   O^T[d, head]     = V^T P^T -- the V rows go from global memory straight into a wave-private
@@ -368,18 +185,20 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeParams p, int t
 // instructions for the softmax.  Per-head state (m, l) is lane-local; the running maximum is
 // shared across the four lane groups with two shuffles per step.
 // ------------------------------------------------------------------------------------------
-constexpr int DM_D = 128;
 constexpr int DM_PS = 16;
-constexpr int DM_VTILE = 2 * DM_PS * DM_D;  // halfs of a wave's V tile: two pages, row-major
 
 // Piece (16 bytes) c of V row r sits at piece position c ^ dm_swizzle(r): the transposing read of
-// 32 lanes touches 8 consecutive rows x 32 bytes, which this spreads over the 8 32-byte parts of
-// a 256-byte bank line.
-__device__ __forceinline__ int dm_swizzle(int row) { return (row & 7) << 1; }
+// 32 lanes touches 8 consecutive rows x 32 bytes, which this spreads over the 8 32-byte parts of a
+// 256-byte bank line (head dim 128: one row per line) or over the 4 parts of each half of two lines
+// (head dim 64: two rows per line, the rows of equal parity share a half).
+template <int D>
+__device__ __forceinline__ int dm_swizzle(int row) {
+  return D == 128 ? (row & 7) << 1 : ((row >> 1) & 3) << 1;
+}
 
 // theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
 struct DecodeRopeDivisors {
-  float v[DM_D / 2];
+  float v[64];
 };
 
 // EXT = false: plain cache, q and k already rotated (or no RoPE).  EXT = true adds the sliding-window
@@ -388,10 +207,16 @@ struct DecodeRopeDivisors {
 // inline RoPE (q at q_rope_position[b], the key with logical index t at k_rope_pos_offset[b] + t,
 // _decode_kernels.py:141-156).  Attention does not depend on the order of the keys, so the pages are
 // still walked in physical order; evicted tokens are masked and logical indices only feed RoPE.
-template <bool EXT>
+template <bool EXT, int D>
 __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodeParams p, int group, int num_items,
                                                              DecodeRopeDivisors div) {
-  constexpr int D = DM_D, PS = DM_PS;
+  constexpr int PS = DM_PS;
+  constexpr int KS = D / 32;                // k-steps of the score product
+  constexpr int DB = D / 16;                // 16-wide output feature blocks
+  constexpr int PPR = D / 8;                // 16-byte pieces per row
+  constexpr int RPI = 64 / PPR;             // rows one copy instruction covers
+  constexpr int DM_VTILE = 2 * PS * D;      // halfs of a wave's V tile: two pages, row-major
+  static_assert(D == 64 || D == 128, "head dim");
   static_assert(DM_VTILE * sizeof(half_t) >= 16 * D * sizeof(float), "the merge buffer aliases the V tile");
   __shared__ __attribute__((aligned(16))) half_t Vt_all[4][DM_VTILE];
   __shared__ float sm_m[4][16];
@@ -407,11 +232,16 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   half_t* Vt = Vt_all[wave];
   const int64_t head_stride = static_cast<int64_t>(PS) * D;
 
-  // Persistent workgroups: item = (chunk slot, kv head), strided over the grid.  Neighbouring
-  // workgroups take the kv heads of one slot, i.e. the same pages.
+  // Persistent workgroups: item = (chunk slot, kv head, block of 16 heads of the group), strided over
+  // the grid.  Neighbouring workgroups take the head blocks and kv heads of one slot, i.e. the same pages.
+  const int head_blocks = (group + 15) >> 4;
   for (int item = blockIdx.x; item < num_items; item += gridDim.x) {
-  const int slot = item / p.h_kv;
-  const int kvh = item - slot * p.h_kv;
+  const int slot = item / (p.h_kv * head_blocks);
+  const int rest = item - slot * (p.h_kv * head_blocks);
+  const int kvh = rest / head_blocks;
+  const int hb = rest - kvh * head_blocks;
+  const int hq0 = kvh * group + hb * 16;      // first query head of this item
+  const int heads = min(16, group - hb * 16);  // and how many
   const int b = find_sequence_wave(p.page_indptr, p.batch_size, cp, slot, lane);
   const int pbeg = p.page_indptr[b];
   const int npages = p.page_indptr[b + 1] - pbeg;
@@ -419,7 +249,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   const int nchunks = (npages + cp - 1) / cp;
   if (chunk >= nchunks) {  // spare slot (uniform over the workgroup)
     if (p.arrivals != nullptr && npages == 0 && chunk == 0) {  // a sequence without pages: nobody else answers for it
-      for (int g = wave; g < group; g += 4) empty_row<D>(p, b, kvh * group + g, lane);
+      for (int g = wave; g < heads; g += 4) empty_row<D>(p, b, hq0 + g, lane);
     }
     continue;
   }
@@ -429,39 +259,40 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   // physical token t is attended to iff t < sink or win_lo <= t < kv_len
   const int sink = EXT && p.sink_size != nullptr ? p.sink_size[b] : 0;
   const int win_lo = EXT && p.window_offset != nullptr ? p.window_offset[b] : 0;
-  float divr[16];  // RoPE divisors of this lane's features ks*32 + g4*8 + i, ks = 0, 1
+  float divr[4 * KS];  // RoPE divisors of this lane's features ks*32 + g4*8 + i, ks < KS/2
   float k_pos0 = 0.f;
   if (EXT && p.rotary) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) divr[i] = div.v[(i >> 3) * 32 + g4 * 8 + (i & 7)];
+    for (int i = 0; i < 4 * KS; ++i) divr[i] = div.v[(i >> 3) * 32 + g4 * 8 + (i & 7)];
     k_pos0 = static_cast<float>(p.k_rope_pos_offset[b]);
   }
 
   // Q^T fragments (B operand): column = head c16 of the group, contraction slots = 8 features.
-  half8_t qf[4];
+  half8_t qf[KS];
   {
-    const half_t* qrow = p.q + (static_cast<int64_t>(b) * p.h_q + kvh * group + c16) * D + g4 * 8;
-    Vec16 qv[4];
+    const half_t* qrow = p.q + (static_cast<int64_t>(b) * p.h_q + hq0 + c16) * D + g4 * 8;
+    Vec16 qv[KS];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) qv[ks] = c16 < group ? ld16(qrow + ks * 32) : zero16();
+    for (int ks = 0; ks < KS; ++ks) qv[ks] = c16 < heads ? ld16(qrow + ks * 32) : zero16();
     if (EXT && p.rotary) {
+      // feature f < D/2 rotates with f + D/2: k-step ks with ks + KS/2
       const float q_pos = static_cast<float>(p.q_rope_position[b]) * p.rope_scale;
-      rope_pair(qv[0].h8, qv[2].h8, q_pos, divr);
-      rope_pair(qv[1].h8, qv[3].h8, q_pos, divr + 8);
+#pragma unroll
+      for (int ks = 0; ks < KS / 2; ++ks) rope_pair(qv[ks].h8, qv[ks + KS / 2].h8, q_pos, divr + 8 * ks);
     }
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) qf[ks] = qv[ks].h8;
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = qv[ks].h8;
   }
-  float4_t o[8];
+  float4_t o[DB];
 #pragma unroll
-  for (int db = 0; db < 8; ++db) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
+  for (int db = 0; db < DB; ++db) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
   float m = kNegInit, lsum = 0.f;
 
   // V^T fragment via the transposing read: lane li of a 16-lane group points at 4 features of token
   // (li >> 2) of the group's 4 tokens and receives feature li of the group's 16 for the 4 tokens
   const uint32_t vt_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)Vt));
   const int v_row = 4 * g4 + (c16 >> 2);             // + PS for the second page: same swizzle
-  const int v_swz = dm_swizzle(v_row);
+  const int v_swz = dm_swizzle<D>(v_row);
   const int v_lane_off = v_row * D + (c16 & 1) * 4;
   const int v_piece = (c16 & 3) >> 1;                // + 2 * feature block
 
@@ -469,11 +300,11 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   // ordinary loads: each request is a quarter of a 256-byte row, and partial rows with the streaming
   // hint measured 10-15 % less bandwidth than without it (whole rows: 8 % more).  K through LDS
   // with whole-row copies like V measured slower than this (two workgroups per CU instead of three).
-  // V: 8 copy instructions of 4 rows x 256 bytes each fill the wave's LDS tile; rows at or past
+  // V: copy instructions of 1 KiB each (4 rows of head dim 128, 8 of head dim 64) fill the wave's LDS tile; rows at or past
   // kv_len repeat the last cached row of their page and a missing second page repeats the first
   // (their P is 0, and 0 times cached data is 0, whereas unwritten memory could hold NaN patterns).
   struct Regs {
-    Vec16 k[2][4];
+    Vec16 k[2][KS];
   };
   auto issue = [&](int pi, Regs& r) {
 #pragma unroll
@@ -484,18 +315,18 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
       const half_t* vbase = kbase + static_cast<int64_t>(p.h_kv) * head_stride;
       const int last_row = min(PS, kv_len - pg * PS) - 1;  // >= 0: every page of the table holds a token
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = i * 4 + (lane >> 4);
-        const int piece = (lane & 15) ^ dm_swizzle(h * PS + row);
+      for (int i = 0; i < PS / RPI; ++i) {
+        const int row = i * RPI + lane / PPR;
+        const int piece = (lane % PPR) ^ dm_swizzle<D>(h * PS + row);
         copy16_to_lds_nt(vbase, static_cast<uint32_t>(min(row, last_row) * (D * 2) + piece * 16),
-                      vt_lds + (h * PS + i * 4) * (D * 2));
+                      vt_lds + (h * PS + i * RPI) * (D * 2));
       }
       if (pi + h < page_hi) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
+        for (int ks = 0; ks < KS; ++ks) r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
       } else {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) r.k[h][ks] = zero16();
+        for (int ks = 0; ks < KS; ++ks) r.k[h][ks] = zero16();
       }
     }
   };
@@ -512,8 +343,8 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
         const int t = (pi + h) * PS + c16;
         const int logical = t < sink ? t : t - win_lo + sink;
         const float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
-        rope_pair(r.k[h][0].h8, r.k[h][2].h8, pos, divr);
-        rope_pair(r.k[h][1].h8, r.k[h][3].h8, pos, divr + 8);
+#pragma unroll
+        for (int ks = 0; ks < KS / 2; ++ks) rope_pair(r.k[h][ks].h8, r.k[h][ks + KS / 2].h8, pos, divr + 8 * ks);
       }
     }
     // ---- S^T = K Q^T for both pages ---------------------------------------------------------
@@ -522,7 +353,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
     for (int h = 0; h < 2; ++h) {
       s[h] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) s[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][ks].h8, qf[ks], s[h], 0, 0, 0);
+      for (int ks = 0; ks < KS; ++ks) s[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][ks].h8, qf[ks], s[h], 0, 0, 0);
     }
     // s[h][j]: token (pi+h)*PS + 4*g4 + j, head c16
     float mx = kNegInit;
@@ -545,7 +376,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
     lsum *= alpha;
     if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {
 #pragma unroll
-      for (int db = 0; db < 8; ++db) o[db] *= alpha;
+      for (int db = 0; db < DB; ++db) o[db] *= alpha;
     }
     half8_t pf;
 #pragma unroll
@@ -564,7 +395,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
     // which is before the next step's copies in program order.
     wait_vmcnt<0>();
 #pragma unroll
-    for (int db = 0; db < 8; ++db) {
+    for (int db = 0; db < DB; ++db) {
       const half_t* vb = Vt + v_lane_off + (((db * 2 + v_piece) ^ v_swz) * 8);
       const half4_t lo = lds_read_tr16(vb);
       const half4_t hi = lds_read_tr16(vb + PS * D);
@@ -591,7 +422,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   // (the wave's V tile is dead now and becomes its [16][D] fp32 output buffer)
   float* sm_o_w = reinterpret_cast<float*>(Vt_all[wave]);
 #pragma unroll
-  for (int db = 0; db < 8; ++db) {
+  for (int db = 0; db < DB; ++db) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) sm_o_w[c16 * D + db * 16 + 4 * g4 + j] = o[db][j];
   }
@@ -602,7 +433,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   __syncthreads();
 
   const bool single_chunk = nchunks == 1;
-  for (int idx = tid; idx < group * D; idx += 256) {
+  for (int idx = tid; idx < heads * D; idx += 256) {
     const int g = idx / D;
     const int d = idx % D;
     float mx = sm_m[0][g];
@@ -615,7 +446,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
       lt += sm_l[w][g] * sc;
       acc += reinterpret_cast<const float*>(Vt_all[w])[g * D + d] * sc;
     }
-    const int hq = kvh * group + g;
+    const int hq = hq0 + g;
     if (single_chunk) {
       const float denom = lt + fast_exp2(kNegInit - mx);
       p.output[(static_cast<int64_t>(b) * p.h_q + hq) * D + d] = static_cast<half_t>(acc / denom);
@@ -639,7 +470,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
     wait_vmcnt<0>();
     __syncthreads();
     if (tid == 0) {
-      unsigned long long* counter = p.arrivals + b * p.h_kv + kvh;
+      unsigned long long* counter = p.arrivals + (static_cast<int64_t>(b) * p.h_kv + kvh) * head_blocks + hb;
       __hip_atomic_fetch_max(counter, static_cast<unsigned long long>(p.epoch) << 32, __ATOMIC_RELAXED,
                              __HIP_MEMORY_SCOPE_AGENT);
       const unsigned long long before =
@@ -648,32 +479,14 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
     }
     __syncthreads();
     if (sm_last) {
-      for (int g = wave; g < group; g += 4) merge_row<D, true>(p, b, kvh * group + g, nchunks, lane);
+      for (int g = wave; g < heads; g += 4) merge_row<D, true>(p, b, hq0 + g, nchunks, lane);
     }
   }
   __syncthreads();  // the merge buffers are the next item's V tiles
   }  // items
 }
 
-__global__ void iota_kernel(int32_t* out, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) out[i] = i;
-}
-
 constexpr size_t kArrivalBytes = 256 * 1024;  // the first bytes of the scratch buffer: arrival counters
-
-template <int D, int PS>
-static void launch_decode(const DecodeParams& p, int group, dim3 grid, hipStream_t stream) {
-  switch (group) {
-    case 1: hipLaunchKernelGGL((decode_splitkv_kernel<D, 1, PS>), grid, dim3(256), 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((decode_splitkv_kernel<D, 2, PS>), grid, dim3(256), 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((decode_splitkv_kernel<D, 4, PS>), grid, dim3(256), 0, stream, p); break;
-    case 8: hipLaunchKernelGGL((decode_splitkv_kernel<D, 8, PS>), grid, dim3(256), 0, stream, p); break;
-    default:
-      throw Error(TVMKV_EUNSUPPORTED, "batch_decode_paged_kv: GQA group size " + std::to_string(group) +
-                                          " is not built (1, 2, 4, 8)");
-  }
-}
 
 }  // namespace tvmkv
 
@@ -730,27 +543,6 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_decode_paged_kv: NULL page table";
   hipStream_t s = as_stream(stream);
 
-  const int gqa = h_q / h_kv;
-  const bool mfma_shape = d == 128 && gqa <= 16;
-  const bool valu_shape = gqa == 1 || gqa == 2 || gqa == 4 || gqa == 8;
-  if (!mfma_shape && (ext || !valu_shape)) {
-    // Inline RoPE and the sliding-window length_info (3, B) are built into the matrix-core kernel
-    // only (head_dim 128, GQA groups up to 16), and the vector kernel for the other shapes has GQA
-    // groups 1, 2, 4, 8.  What neither covers runs as a paged prefill with one query per sequence:
-    // one workgroup per (sequence, kv head), no split over the keys.
-    const ScratchLease ws = lease(kArrivalBytes + (static_cast<size_t>(batch_size) + 1) * sizeof(int32_t));
-    int32_t* q_indptr = reinterpret_cast<int32_t*>(ws.ptr + kArrivalBytes);
-    hipLaunchKernelGGL(iota_kernel, dim3((batch_size + 256) / 256), dim3(256), 0, s, q_indptr, batch_size + 1);
-    KV_LAUNCH_CHECK();
-    const int rc = tvmkv_batch_prefill_paged_kv(q, q_indptr, pages, page_indptr, page_values, length_info,
-                                                k_rope_pos_offset, q_rope_position, output, lse, /*causal=*/0,
-                                                rotary_mode, rope_scale, rope_theta, sm_scale, batch_size, batch_size,
-                                                nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window,
-                                                /*sliding_window_size=*/0, stream);
-    if (rc != TVMKV_OK) throw Error(rc, tvmkv_last_error());
-    return;
-  }
-
   DecodeParams p;
   p.q = static_cast<const half_t*>(q);
   p.pages = static_cast<const half_t*>(pages);
@@ -780,47 +572,41 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   p.arrivals = nullptr;
   p.epoch = ws.epoch;
 
-  const dim3 grid(static_cast<unsigned>(slots), h_kv);
   const int group = h_q / h_kv;
-  if (d == 128 && group <= 16) {
-    const int64_t num_items = slots * h_kv;
-    KV_CHECK(num_items < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many work items";
-    // One item per workgroup by default (measured a little faster than a resident-size grid
-    // striding over the items); the option decode_wgs_per_cu = n caps the grid at n workgroups per CU.
-    const int64_t wgs_per_cu = option(kOptDecodeWgsPerCu);
-    int64_t grid_x = num_items;
-    if (wgs_per_cu > 0) grid_x = std::min<int64_t>(num_items, static_cast<int64_t>(compute_units()) * wgs_per_cu);
-    // the chunk merge is done by the last workgroup of each (sequence, kv head) when the arrival
-    // counters fit their region; the option decode_separate_merge keeps the second kernel
-    const bool fused = static_cast<size_t>(batch_size) * h_kv * sizeof(unsigned long long) <= kArrivalBytes &&
-                       option(kOptDecodeSeparateMerge) == 0;
-    if (fused) p.arrivals = reinterpret_cast<unsigned long long*>(ws.ptr);
-    DecodeRopeDivisors div{};
-    if (p.rotary) {
-      KV_CHECK(k_rope_pos_offset && q_rope_position) << "batch_decode_paged_kv: inline RoPE needs the position arrays";
-      const float theta = static_cast<float>(rope_theta);
-      for (int i = 0; i < DM_D / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DM_D));
-    }
-    if (ext) {
-      hipLaunchKernelGGL(decode_mfma_kernel<true>, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group,
-                         static_cast<int>(num_items), div);
-    } else {
-      hipLaunchKernelGGL(decode_mfma_kernel<false>, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group,
-                         static_cast<int>(num_items), div);
-    }
-    if (!fused) {
-      KV_LAUNCH_CHECK();
-      hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p,
-                         batch_size * h_q);
-    }
-  } else if (d == 128) {
-    launch_decode<128, 16>(p, group, grid, s);
-    KV_LAUNCH_CHECK();
-    hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
+  const int head_blocks = (group + 15) / 16;
+  const int64_t num_items = slots * h_kv * head_blocks;
+  KV_CHECK(num_items < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many work items";
+  // One item per workgroup by default (measured a little faster than a resident-size grid
+  // striding over the items); the option decode_wgs_per_cu = n caps the grid at n workgroups per CU.
+  const int64_t wgs_per_cu = option(kOptDecodeWgsPerCu);
+  int64_t grid_x = num_items;
+  if (wgs_per_cu > 0) grid_x = std::min<int64_t>(num_items, static_cast<int64_t>(compute_units()) * wgs_per_cu);
+  // the chunk merge is done by the last workgroup of each (sequence, kv head, head block) when the
+  // arrival counters fit their region; the option decode_separate_merge keeps the second kernel
+  const bool fused = static_cast<size_t>(batch_size) * h_kv * head_blocks * sizeof(unsigned long long) <= kArrivalBytes &&
+                     option(kOptDecodeSeparateMerge) == 0;
+  if (fused) p.arrivals = reinterpret_cast<unsigned long long*>(ws.ptr);
+  DecodeRopeDivisors div{};
+  if (p.rotary) {
+    KV_CHECK(k_rope_pos_offset && q_rope_position) << "batch_decode_paged_kv: inline RoPE needs the position arrays";
+    const float theta = static_cast<float>(rope_theta);
+    for (int i = 0; i < d / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(d));
+  }
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group, static_cast<int>(num_items), div);
+  };
+  if (d == 128) {
+    if (ext) launch(decode_mfma_kernel<true, 128>); else launch(decode_mfma_kernel<false, 128>);
   } else {
-    launch_decode<64, 16>(p, group, grid, s);
+    if (ext) launch(decode_mfma_kernel<true, 64>); else launch(decode_mfma_kernel<false, 64>);
+  }
+  if (!fused) {
     KV_LAUNCH_CHECK();
-    hipLaunchKernelGGL(decode_merge_kernel<64>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
+    if (d == 128) {
+      hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
+    } else {
+      hipLaunchKernelGGL(decode_merge_kernel<64>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
+    }
   }
   KV_LAUNCH_CHECK();
 }
