@@ -101,6 +101,14 @@ int tvmkv_fused_rope_scaled(const void* qkv, const int32_t* position_map, void* 
                             int32_t num_kv_heads, int32_t head_dim, double rope_scale, double rope_theta,
                             void* stream);
 
+/* tvmkv_fused_rope_append (below) with a frequency variant. */
+int tvmkv_fused_rope_append_scaled(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
+                                   int64_t apply_rope, const float* rope_ext_factors,
+                                   const tvmkv_rope_scaling* scaling, void* pages,
+                                   const int32_t* append_position_map, int64_t seq_len, int32_t num_q_heads,
+                                   int32_t num_kv_heads, int32_t head_dim, int64_t num_pages,
+                                   int32_t page_size, double rope_scale, double rope_theta, void* stream);
+
 /* Slot 24 followed by slot 13 in one launch; no counterpart among the reference's kernels.
  * Besides the q / k / v outputs of tvmkv_fused_rope, the rotated k and the v rows are written into
  * their page slots append_position_map[token] (-1 = none), which is what
@@ -400,6 +408,14 @@ int tvmkv_cache_create(const int64_t* cache_config, int32_t n_config, const int6
                        double rope_scale, double rope_theta, int32_t dtype_bits, int32_t device_id,
                        tvmkv_cache** out);
 void tvmkv_cache_destroy(tvmkv_cache* cache);
+/* The RoPE frequency variant of the model (what the reference bakes into the f_split_rotary kernel it is
+ * created with, paged_kv_cache.cc:2583) and, for longrope, the factor tensor the reference's create call
+ * takes as `rope_ext_factors` (device memory, head_dim float32, kept by reference: it must outlive the
+ * cache).  scaling NULL or rope_type DEFAULT: back to plain frequencies.  Caches that rotate inside the
+ * attention kernels (RoPE mode inline, i.e. sliding-window caches) only have the plain frequencies:
+ * TVMKV_EUNSUPPORTED. */
+int tvmkv_cache_set_rope_scaling(tvmkv_cache* cache, const tvmkv_rope_scaling* scaling,
+                                 const float* rope_ext_factors);
 /* Stream on which the cache enqueues kernels (the reference uses the device's current stream,
  * paged_kv_cache.cc:524).  Default: the null stream. */
 int tvmkv_cache_set_stream(tvmkv_cache* cache, void* stream);

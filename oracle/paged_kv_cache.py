@@ -29,7 +29,7 @@ from . import kernels as ok
 class OraclePagedKVCache:
     def __init__(self, cache_config, num_layers, num_qo_heads, num_kv_heads, qk_head_dim, v_head_dim,
                  attn_kinds=None, rope_mode=hc.ROPE_NORMAL, rope_scale=1.0, rope_theta=1e4,
-                 dtype=np.float16):
+                 dtype=np.float16, rope_scaling=None, rope_ext_factors=None):
         attn_kinds = list(attn_kinds) if attn_kinds is not None else [hc.ATTN_MHA] * num_layers
         self.host = hc.HostCache(cache_config, attn_kinds, rope_mode)
         self.num_layers = num_layers
@@ -38,6 +38,8 @@ class OraclePagedKVCache:
         self.attn_kinds = attn_kinds
         self.rope_mode = self.host.rope_mode
         self.rope_scale, self.rope_theta = rope_scale, rope_theta
+        # the frequency variant the reference bakes into its split-rotary kernel (position_embedding.py:258-299)
+        self.rope_scaling, self.rope_ext_factors = rope_scaling, rope_ext_factors
         self.dtype = dtype
         ps, npages = self.host.page_size, self.host.num_total_pages
         self.pages = []
@@ -203,8 +205,14 @@ class OraclePagedKVCache:
         q = np.zeros((total, self.hq, self.dqk), self.dtype)
         k = np.zeros((total, self.hkv, self.dqk), self.dtype)
         v = np.zeros((total, self.hkv, self.dqk), self.dtype)
-        ok.fused_rope(qkv_view, aux["q_rope_position_map"], q, k, v, int(self.rope_mode == hc.ROPE_NORMAL),
-                      theta=self.rope_theta, scale=self.rope_scale)
+        if self.rope_scaling:
+            # the longrope kernel has no apply_rope argument and always rotates (position_embedding.py:582-667)
+            apply = 1 if self.rope_ext_factors is not None else int(self.rope_mode == hc.ROPE_NORMAL)
+            ok.fused_rope_scaled(qkv_view, aux["q_rope_position_map"], q, k, v, apply, self.rope_scaling,
+                                 theta=self.rope_theta, scale=self.rope_scale, ext_factors=self.rope_ext_factors)
+        else:
+            ok.fused_rope(qkv_view, aux["q_rope_position_map"], q, k, v, int(self.rope_mode == hc.ROPE_NORMAL),
+                          theta=self.rope_theta, scale=self.rope_scale)
         if host.append_before_attn:
             ok.transpose_append(self.pages[layer_id], k, v, aux["append_position_map"])
         o_view = np.zeros((total, self.hq, self.dqk), self.dtype)

@@ -28,11 +28,12 @@ class GpuCache:
     """The library's cache behind the interface of oracle.paged_kv_cache.OraclePagedKVCache."""
 
     def __init__(self, cache_config, num_layers, hq, hkv, dqk, dv, attn_kinds=None, rope_mode=1, rope_scale=1.0,
-                 rope_theta=1e4):
+                 rope_theta=1e4, rope_scaling=None, rope_ext_factors=None):
         attn_kinds = list(attn_kinds) if attn_kinds is not None else [0] * num_layers
+        ext = None if rope_ext_factors is None else dev(np.asarray(rope_ext_factors, dtype=np.float32))
         self.cache = gf("vm.builtin.paged_attention_kv_cache_create")(
             list(cache_config), [0, num_layers], hq, hkv, dqk, dv, attn_kinds, False, rope_mode, rope_scale,
-            rope_theta, None, torch.empty((), dtype=torch.float16, device=DEV))
+            rope_theta, ext, torch.empty((), dtype=torch.float16, device=DEV), rope_scaling=rope_scaling)
         self.num_layers, self.hq, self.hkv, self.dqk, self.dv = num_layers, hq, hkv, dqk, dv
 
     def clear(self):

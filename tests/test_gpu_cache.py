@@ -32,9 +32,9 @@ def test_reference_scenarios_on_the_gpu(runner, d, rope_mode):
 class Mirror:
     """Feeds the oracle cache and the GPU cache the same calls and the same tensors."""
 
-    def __init__(self, cache_config, layers, hq, hkv, d, rope_mode=1):
-        self.o = OraclePagedKVCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode)
-        self.g = GpuCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode)
+    def __init__(self, cache_config, layers, hq, hkv, d, rope_mode=1, **rope):
+        self.o = OraclePagedKVCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode, **rope)
+        self.g = GpuCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode, **rope)
         self.layers, self.hq, self.hkv, self.d = layers, hq, hkv, d
         self.rng = np.random.default_rng(21)
         self.lengths = {}
@@ -108,6 +108,31 @@ def test_identical_inputs_through_oracle_and_gpu_caches():
     m.lengths[6] -= 30
     m.step([(6, 1), (1, 200)])
     m.step([(i, 1) for i in (0, 1, 2, 4, 5, 6)])
+
+
+@pytest.mark.parametrize("rope", [
+    dict(rope_theta=5e5, rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                                       "original_max_position_embeddings": 8192}),
+    dict(rope_scaling={"rope_type": "yarn", "factor": 40.0, "beta_fast": 32, "beta_slow": 1,
+                       "original_max_position_embeddings": 4096}),
+    dict(rope_scaling={"rope_type": "longrope", "max_position_embeddings": 131072, "original_max_position_embeddings": 64},
+         rope_ext_factors=np.concatenate([np.linspace(1.0, 8.0, 64), np.linspace(1.0, 1.3, 64)]).astype(np.float32)),
+])
+def test_rope_frequency_variants_through_the_cache(rope):
+    """The model's RoPE variant (what the reference compiles into the split-rotary kernel it hands to the
+    cache): prefill, decode and a fork, cached K compared with the oracle cache that rotates the same way.
+    The longrope steps have fewer and more rows than original_max_position_embeddings (short / long factors)."""
+    m = Mirror([8, 2048, 512, 16, 0], 1, 32, 8, 128, **rope)
+    m.step([(0, 60), (1, 88), (2, 17)])   # 165 rows
+    m.step([(0, 1), (1, 1), (2, 1)])      # 3 rows
+    m.step([((3, 1, 40), 25), (0, 2)])
+
+
+def test_rope_variants_need_a_cache_that_rotates_up_front():
+    with pytest.raises(tvm_amd.KVError, match="inline RoPE") as info:
+        GpuCache([8, 2048, 512, 16, 1], 1, 32, 8, 128, 128, rope_scaling={"rope_type": "llama3", "factor": 8.0,
+                 "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 8192})
+    assert info.value.code == -2
 
 
 def test_cfg1_decode_through_the_cache_verbs():

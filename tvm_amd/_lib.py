@@ -25,6 +25,8 @@ SIGNATURES = {
     "tvmkv_fused_rope": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_i32, c_f64, c_f64, c_vp],
     "tvmkv_fused_rope_scaled": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_f64,
                                 c_f64, c_vp],
+    "tvmkv_fused_rope_append_scaled": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_i32,
+                                       c_i32, c_i64, c_i32, c_f64, c_f64, c_vp],
     "tvmkv_fused_rope_append": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i64,
                                 c_i32, c_f64, c_f64, c_vp],
     "tvmkv_kv_cache_transpose_append": [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_i32, c_vp],
@@ -64,6 +66,7 @@ SIGNATURES = {
     "tvmkv_cache_create": [p_i64, c_i32, p_i64, c_i32, c_i64, c_i64, c_i64, c_i64, p_i64, c_i32, c_i32, c_i32,
                            c_f64, c_f64, c_i32, c_i32, ctypes.POINTER(c_vp)],
     "tvmkv_cache_set_stream": [c_vp, c_vp],
+    "tvmkv_cache_set_rope_scaling": [c_vp, c_vp, c_vp],
     "tvmkv_kv_state_clear": [c_vp],
     "tvmkv_kv_state_add_sequence": [c_vp, c_i64],
     "tvmkv_kv_state_remove_sequence": [c_vp, c_i64],

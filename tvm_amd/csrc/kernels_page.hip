@@ -471,6 +471,20 @@ int tvmkv_fused_rope_scaled(const void* qkv, const int32_t* position_map, void* 
                          num_kv_heads, head_dim, rope_scale, rope_theta, nullptr, nullptr, 0, 0, stream);
 }
 
+int tvmkv_fused_rope_append_scaled(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
+                                   int64_t apply_rope, const float* rope_ext_factors, const tvmkv_rope_scaling* scaling,
+                                   void* pages, const int32_t* append_position_map, int64_t seq_len, int32_t num_q_heads,
+                                   int32_t num_kv_heads, int32_t head_dim, int64_t num_pages, int32_t page_size,
+                                   double rope_scale, double rope_theta, void* stream) {
+  if (seq_len > 0 && pages == nullptr) {
+    ::tvmkv::SetLastError("fused_rope_append: NULL pages");
+    return TVMKV_EINVAL;
+  }
+  return fused_rope_impl(qkv, position_map, q, k, v, apply_rope, rope_ext_factors, scaling, seq_len, num_q_heads,
+                         num_kv_heads, head_dim, rope_scale, rope_theta, pages, append_position_map, num_pages, page_size,
+                         stream);
+}
+
 int tvmkv_fused_rope_append(const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
                             int64_t apply_rope, void* pages, const int32_t* append_position_map, int64_t seq_len,
                             int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int64_t num_pages,

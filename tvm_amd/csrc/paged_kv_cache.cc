@@ -159,6 +159,31 @@ class PagedKVCache {
     // A chunked-prefill step of a plain cache in two launches: k is rotated and the new k / v rows go
     // into their page slots (part 2 without q, part 3), then one pass over the cached and the new
     // tokens that reads the queries from qkv and rotates them itself (parts 2 and 5).
+    if (has_rope_scaling_) {
+      // the model's frequency variant lives in the split-rotary kernel only: q, k and v take the round trip
+      const bool early = s.append_before_attn || !support_sliding_window_;
+      // the reference's kernel for a factor tensor has no apply_rope argument: it always rotates
+      const bool rotate = rope_normal || rope_ext_factors_ != nullptr;
+      if (early) {
+        Launch(tvmkv_fused_rope_append_scaled(qkv, Dev(s.q_rope_position_map), temp_q_, temp_k_, temp_v_, rotate,
+                                              rope_ext_factors_, &rope_scaling_, pages_[local_layer_id],
+                                              Dev(s.append_position_map), total_seq_length, num_qo_heads_, num_kv_heads_,
+                                              qk_head_dim_, num_total_pages_, page_size_, rotary_scale_, rotary_theta_,
+                                              compute_stream_));
+      } else {
+        Launch(tvmkv_fused_rope_scaled(qkv, Dev(s.q_rope_position_map), temp_q_, temp_k_, temp_v_, rotate,
+                                       rope_ext_factors_, &rope_scaling_, total_seq_length, num_qo_heads_, num_kv_heads_,
+                                       qk_head_dim_, rotary_scale_, rotary_theta_, compute_stream_));
+      }
+      AttentionInternal(layer_id, temp_q_, temp_k_, temp_v_, out, total_seq_length, sm_scale);
+      if (!early) {
+        Launch(tvmkv_kv_cache_transpose_append(pages_[local_layer_id], temp_k_, temp_v_, Dev(s.append_position_map),
+                                               total_seq_length, num_total_pages_, num_kv_heads_, page_size_,
+                                               qk_head_dim_, compute_stream_));
+      }
+      RecordComputeEvent();
+      return;
+    }
     if (OnePassPrefillApplies(layer_id)) {
       Launch(tvmkv_fused_rope_append(qkv, Dev(s.q_rope_position_map), /*q=*/nullptr, temp_k_, temp_v_, rope_normal,
                                      pages_[local_layer_id], Dev(s.append_position_map), total_seq_length,
@@ -358,6 +383,14 @@ class PagedKVCache {
     return pages_[local_layer];
   }
   void SetStream(hipStream_t stream) { compute_stream_ = stream; }
+  void SetRopeScaling(const tvmkv_rope_scaling* scaling, const float* rope_ext_factors) {
+    has_rope_scaling_ = scaling != nullptr && scaling->rope_type != TVMKV_ROPE_FREQ_DEFAULT;
+    KV_UNSUPPORTED(has_rope_scaling_ && rope_mode_ == TVMKV_ROPE_INLINE)
+        << "RoPE scaling variants are not built for caches that rotate inside the attention kernels (inline RoPE)";
+    KV_CHECK(has_rope_scaling_ || rope_ext_factors == nullptr) << "rope_ext_factors needs a longrope scaling description";
+    if (has_rope_scaling_) rope_scaling_ = *scaling;
+    rope_ext_factors_ = rope_ext_factors;
+  }
 
  private:
   // ---------------------------------------------------------------- device layer
@@ -713,6 +746,10 @@ class PagedKVCache {
   int rope_mode_ = TVMKV_ROPE_NORMAL;
   double rotary_scale_, rotary_theta_;
 
+  bool has_rope_scaling_ = false;
+  tvmkv_rope_scaling rope_scaling_{};
+  const float* rope_ext_factors_ = nullptr;
+
   std::unique_ptr<KVBookkeeper> book_;
   size_t page_copies_issued_ = 0;  // elements of the bookkeeper's copy log already on the copy stream
 
@@ -785,6 +822,9 @@ void tvmkv_cache_destroy(tvmkv_cache* cache) { delete cache; }
 
 int tvmkv_cache_set_stream(tvmkv_cache* cache, void* stream) {
   KV_CACHE_FN(cache->impl->SetStream(static_cast<hipStream_t>(stream)));
+}
+int tvmkv_cache_set_rope_scaling(tvmkv_cache* cache, const tvmkv_rope_scaling* scaling, const float* rope_ext_factors) {
+  KV_CACHE_FN(cache->impl->SetRopeScaling(scaling, rope_ext_factors));
 }
 int tvmkv_kv_state_clear(tvmkv_cache* cache) { KV_CACHE_FN(cache->impl->Clear()); }
 int tvmkv_kv_state_add_sequence(tvmkv_cache* cache, int64_t seq_id) { KV_CACHE_FN(cache->impl->AddSequence(seq_id)); }

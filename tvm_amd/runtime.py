@@ -164,12 +164,16 @@ def _dtype_bits(init):
 
 
 def _create(cache_config, layer_indptr, num_qo_heads, num_kv_heads, qk_head_dim, v_head_dim, attn_kinds,
-            enable_kv_transfer, rope_mode, rope_scale, rope_theta, rope_ext_factors, init, *kernel_slots):
+            enable_kv_transfer, rope_mode, rope_scale, rope_theta, rope_ext_factors, init, *kernel_slots,
+            rope_scaling=None):
     """(cache_config, layer_indptr, Hq, Hkv, qk_dim, v_dim, attn_kinds, enable_kv_transfer, rope_mode,
     rope_scale, rope_theta, rope_ext_factors, init_tensor, <15 kernel slots>).  The kernel slots of the
-    reference's signature are accepted and ignored: the kernels are the library's own."""
-    if rope_ext_factors is not None:
-        raise KVError(-2, "rope_ext_factors (RoPE scaling variants) are not built")
+    reference's signature are accepted and ignored: the kernels are the library's own.  What the reference
+    bakes into its split-rotary kernel slot travels as the keyword rope_scaling: the model's dictionary
+    (rope_type llama3 / longrope / yarn and its parameters, position_embedding.py:258-299 of the reference);
+    rope_ext_factors is the float32 device tensor of a longrope model."""
+    if rope_ext_factors is not None and (rope_scaling or {}).get("rope_type") != "longrope":
+        raise KVError(-1, "rope_ext_factors needs rope_scaling = {'rope_type': 'longrope', ...}")
     cfg = _i64_array(cache_config)
     lip = _i64_array(layer_indptr)
     kinds = _i64_array(attn_kinds)
@@ -178,8 +182,15 @@ def _create(cache_config, layer_indptr, num_qo_heads, num_kv_heads, qk_head_dim,
                                    qk_head_dim, v_head_dim, kinds, len(attn_kinds), int(bool(enable_kv_transfer)),
                                    int(rope_mode), float(rope_scale), float(rope_theta), _dtype_bits(init),
                                    _device_index(init), ctypes.byref(out)))
-    return PagedAttentionKVCache(out.value, layer_indptr[-1] - layer_indptr[0], num_kv_heads, qk_head_dim,
-                                 v_head_dim)
+    cache = PagedAttentionKVCache(out.value, layer_indptr[-1] - layer_indptr[0], num_kv_heads, qk_head_dim,
+                                  v_head_dim)
+    if rope_scaling:
+        from .dlpack import RopeScaling
+        scaling = RopeScaling.from_dict(rope_scaling)
+        ext = ctypes.c_void_p(rope_ext_factors.data_ptr()) if rope_ext_factors is not None else None
+        check(lib().tvmkv_cache_set_rope_scaling(cache.handle, ctypes.c_void_p(ctypes.addressof(scaling)), ext))
+        cache._rope_ext_factors = rope_ext_factors  # the library keeps the pointer, not the tensor
+    return cache
 
 
 def _begin_forward(cache, seq_ids, append_lengths, token_tree_parent_ptr=None):
