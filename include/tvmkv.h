@@ -376,6 +376,17 @@ int tvmkv_stream_copy(const void* src, void* dst, int64_t num_bytes, void* strea
  * A and B fragments read from `operands` (256 lanes x 16 halfs); `out` gets workgroups x 256
  * floats.  2 * 32 * 32 * 16 * 8 * iters * 4 * workgroups flop per launch. */
 int tvmkv_mfma_loop(const void* operands, float* out, int32_t iters, int32_t workgroups, void* stream);
+/* Clock probe of the prefill kernels (no counterpart in the reference; a measurement aid).  The
+ * shader clock of this chip follows the power the kernel draws, so a fraction of the datasheet
+ * matrix peak (quoted at 2.4 GHz) says little without the clock the kernel really ran at.  After
+ * tvmkv_prefill_clock_probe(1) every workgroup of every prefill / tree-attention launch of this
+ * process adds three numbers to counters on its device: the shader cycles and the 100 MHz ticks
+ * between its start and its end, and 1.  tvmkv_prefill_clock_probe_read synchronizes the current
+ * device, copies the three sums to counters[0..2] (cycles, ticks, workgroups) and clears them if
+ * reset != 0: cycles / ticks * 100 MHz is the average shader clock.  Not thread-safe against
+ * concurrent launches; costs two timestamp reads and three atomics per workgroup while enabled. */
+int tvmkv_prefill_clock_probe(int32_t enable);
+int tvmkv_prefill_clock_probe_read(uint64_t* counters, int32_t reset);
 
 /* ======================================================================================
  * (2) Cache object

@@ -676,3 +676,26 @@ def test_measurement_utilities():
     torch.cuda.synchronize()
     # one instruction adds 16 * 0.5 * 0.5 = 4 to each of its 16 results per lane; 8 instructions a round
     assert torch.all(out == 4.0 * 16 * 8 * iters)
+
+
+def test_prefill_clock_probe_counts_workgroups_and_leaves_results_alone():
+    """The clock probe adds (shader cycles, 100 MHz ticks, 1) per workgroup while it is switched on,
+    nothing while it is off, and does not change what the kernel computes."""
+    rng = np.random.default_rng(77)
+    lens = [300, 5, 200]
+    K.prefill_clock_probe(False)
+    K.prefill_clock_probe_read(reset=True)
+    base_out, base_lse, eo, el = _ragged_both(rng, lens, 32, 8, 128, 128, 1)
+    assert K.prefill_clock_probe_read(reset=True) == (0, 0, 0)
+    K.prefill_clock_probe(True)
+    try:
+        rng = np.random.default_rng(77)
+        out, lse, _, _ = _ragged_both(rng, lens, 32, 8, 128, 128, 1)
+        cycles, ticks, workgroups = K.prefill_clock_probe_read(reset=True)
+    finally:
+        K.prefill_clock_probe(False)
+    assert np.array_equal(out, base_out) and np.array_equal(lse, base_lse)
+    # row tiles: ceil(len * group / 128) per sequence and kv head, group 4, 8 kv heads
+    assert workgroups == 8 * sum((n * 4 + 127) // 128 for n in lens)
+    assert ticks > 0 and 200.0 < cycles / ticks * 100.0 < 4000.0, (cycles, ticks)
+    assert K.prefill_clock_probe_read(reset=False) == (0, 0, 0)

@@ -62,6 +62,8 @@ SIGNATURES = {
     "tvmkv_stream_read": [c_vp, c_i64, c_vp, c_vp],
     "tvmkv_stream_read_nt": [c_vp, c_i64, c_vp, c_vp],
     "tvmkv_mfma_loop": [c_vp, c_vp, c_i32, c_i32, c_vp],
+    "tvmkv_prefill_clock_probe": [c_i32],
+    "tvmkv_prefill_clock_probe_read": [c_vp, c_i32],
     "tvmkv_stream_copy": [c_vp, c_vp, c_i64, c_vp],
     "tvmkv_cache_create": [p_i64, c_i32, p_i64, c_i32, c_i64, c_i64, c_i64, c_i64, p_i64, c_i32, c_i32, c_i32,
                            c_f64, c_f64, c_i32, c_i32, ctypes.POINTER(c_vp)],

@@ -50,6 +50,7 @@ struct PrefillParams {
   // rotates them at q_rope_position[token] itself (with rope_scale and the divisors of the launch)
   int64_t q_token_stride;
   int q_inline_rope;
+  int clock_probe;  // != 0: add this workgroup's shader cycles and 100 MHz ticks to the probe counters
 };
 
 // theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use

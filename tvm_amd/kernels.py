@@ -251,6 +251,20 @@ def mfma_loop(operands, out, iters):
     check(lib().tvmkv_mfma_loop(_p(operands), _p(out), int(iters), out.shape[0], _stream()))
 
 
+def prefill_clock_probe(enable):
+    """Switches the clock probe of the prefill kernels on or off (a measurement aid)."""
+    check(lib().tvmkv_prefill_clock_probe(int(bool(enable))))
+
+
+def prefill_clock_probe_read(reset=True):
+    """(shader cycles, 100 MHz ticks, workgroups) summed over the prefill launches since the last
+    reset on the current device; cycles / ticks * 100 is the average shader clock in MHz."""
+    import ctypes
+    buf = (ctypes.c_uint64 * 3)()
+    check(lib().tvmkv_prefill_clock_probe_read(ctypes.cast(buf, ctypes.c_void_p), int(bool(reset))))
+    return int(buf[0]), int(buf[1]), int(buf[2])
+
+
 def stream_read_nt(src, sink):
     """stream_read with non-temporal loads."""
     check(lib().tvmkv_stream_read_nt(_p(src), src.numel() * src.element_size(), _p(sink), _stream()))
