@@ -195,7 +195,7 @@ def calibrate(num_bytes=2 << 30, iters=10, quiet=False):
 # and the rest (q, outputs, split-KV partial states) scales with the same page tables, so the ratio
 # carries over to the page tables of any --steps / --warmup of this workload.
 TRAFFIC_MEASURED_ON_BYTES = 1182904320
-TRAFFIC_KIB = {"decode_mfma_kernel": (581061.0 * 2.0, 6219.8)}
+TRAFFIC_KIB = {"decode_mfma_kernel": (581458.0 * 2.0, 6281.5)}
 TRAFFIC_PER_ALGORITHMIC_BYTE = sum(r + w for r, w in TRAFFIC_KIB.values()) * 1024 / TRAFFIC_MEASURED_ON_BYTES
 
 
