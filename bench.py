@@ -186,6 +186,76 @@ def calibrate(num_bytes=2 << 30, iters=10, quiet=False):
     return out
 
 
+def cache_object_decode(torch, dev, layers=32, seed=1):
+    """configs[1] through the cache OBJECT, the way a model drives it (the reference's call order,
+    src/runtime/vm/kv_state.cc:33-116): per decode step one begin_forward for all layers, then
+    attention_with_fused_qkv layer by layer, then end_forward.  The cache is filled through the same
+    interface (chunked prefill steps).  What this leg shows beside the kernel legs: the host
+    bookkeeping, the single auxiliary upload per step and the launches of `layers` layers do not
+    slow the kernels down."""
+    from tvm_amd import get_global_func as gf
+
+    rng = np.random.default_rng(seed)
+    B = 64
+    ctx = rng.integers(1024, 8192, size=B, endpoint=True)
+    steps = 12
+    capacity = int(ctx.sum()) + B * (steps + 4) + B * PS
+    cache = gf("vm.builtin.paged_attention_kv_cache_create")(
+        [B, capacity, 4096, PS, 0], [0, layers], HQ, HKV, D, D, [0] * layers, False, 1, 1.0, 1e4, None,
+        torch.empty((), dtype=torch.float16, device=dev))
+    cache.set_stream(torch.cuda.current_stream().cuda_stream)
+    f_add = gf("vm.builtin.kv_state_add_sequence")
+    f_begin = gf("vm.builtin.kv_state_begin_forward")
+    f_end = gf("vm.builtin.kv_state_end_forward")
+    f_attn = gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")
+    sm_scale = D ** -0.5
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    chunk_qkv = torch.randn((4096, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16)
+    chunk_out = torch.empty((4096, HQ, D), dtype=torch.float16, device=dev)
+    for b in range(B):
+        f_add(cache, b)
+        left = int(ctx[b])
+        while left > 0:
+            n = min(left, 4096)
+            f_begin(cache, [b], [n], None)
+            for layer in range(layers):
+                f_attn(cache, layer, sm_scale, chunk_qkv[:n], chunk_out[:n])
+            f_end(cache)
+            left -= n
+    qkv = torch.randn((B, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16)
+    out = torch.empty((B, HQ, D), dtype=torch.float16, device=dev)
+    ids, ones = list(range(B)), [1] * B
+
+    def step():
+        f_begin(cache, ids, ones, None)
+        for layer in range(layers):
+            f_attn(cache, layer, sm_scale, qkv, out)
+        f_end(cache)
+
+    for _ in range(4):
+        step()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps - 4):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / (steps - 4)
+    gpu_ms = start.elapsed_time(stop) / (steps - 4)
+    kv_tokens = float(ctx.sum()) + B * (4 + (steps - 4) / 2.0)  # cached tokens an average timed step attends to
+    step_bytes = layers * (kv_tokens * TOKEN_BYTES + B * HQ * D * 2 * 2 + B * (HQ + 2 * HKV) * D * 2 + B * TOKEN_BYTES)
+    return {"workload": f"configs[1] through the cache object: {layers} layers, B=64, ctx U[1024,8192], one begin_forward + "
+                        f"{layers} x attention_with_fused_qkv + end_forward per decode step, cache filled by chunked prefill "
+                        "steps through the same interface",
+            "layers": layers, "ms_per_step": round(gpu_ms, 4), "ms_per_layer": round(gpu_ms / layers, 4),
+            "host_wall_ms_per_step": round(wall_ms, 4), "GBps": round(step_bytes / gpu_ms / 1e6, 1),
+            "frac_of_hbm_peak": round(step_bytes / gpu_ms / 1e6 / HBM_PEAK_GBPS, 4),
+            "tokens_per_s": round(B / (gpu_ms * 1e-3), 1)}
+
+
 # HBM bytes per launch of the decode entry point, from rocprofv3 counter runs of this file
 # (profiles/decode_mfma_kernel_cfg2_batched_decode.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 in KiB per
 # dispatch of decode_mfma_kernel (it merges the chunks itself); the scales come from the plain copy
@@ -660,6 +730,8 @@ def main():
         del pages, qkv
         torch.cuda.empty_cache()
         result["extras"] = extras(torch, K, dev)
+        torch.cuda.empty_cache()
+        result["extras"]["cache_object_decode"] = cache_object_decode(torch, dev)
     print(json.dumps(result))
 
 

@@ -116,6 +116,13 @@ class PagedKVCache {
   void BeginForward(const int64_t* seq_ids, const int64_t* append_lengths, int64_t batch_size,
                     const int64_t* token_tree_parent_ptr, int64_t n_tree) {
     if (device_ >= 0) {
+      // the kernels enqueued since the last step began were the last readers of the buffer in use
+      if (aux_read_since_event_[aux_slot_]) {
+        HIP_CHECK(hipSetDevice(device_));
+        HIP_CHECK(hipEventRecord(aux_consumed_[aux_slot_], compute_stream_));
+        aux_consumed_recorded_[aux_slot_] = true;
+        aux_read_since_event_[aux_slot_] = false;
+      }
       const int next = aux_slot_ ^ 1;
       // this slot's staging memory was last read by the upload two steps ago
       if (aux_slot_used_[next]) HIP_CHECK(hipEventSynchronize(aux_copied_[next]));
@@ -382,7 +389,24 @@ class PagedKVCache {
     *bytes = PageBytes(local_layer);
     return pages_[local_layer];
   }
-  void SetStream(hipStream_t stream) { compute_stream_ = stream; }
+  void SetStream(hipStream_t stream) {
+    if (stream == compute_stream_) return;
+    if (device_ >= 0 && (compute_work_since_event_ || aux_read_since_event_[aux_slot_])) {
+      // the events that later waits rely on belong on the stream the work was enqueued on
+      HIP_CHECK(hipSetDevice(device_));
+      if (compute_work_since_event_) {
+        HIP_CHECK(hipEventRecord(compute_done_, compute_stream_));
+        compute_event_recorded_ = true;
+        compute_work_since_event_ = false;
+      }
+      if (aux_read_since_event_[aux_slot_]) {
+        HIP_CHECK(hipEventRecord(aux_consumed_[aux_slot_], compute_stream_));
+        aux_consumed_recorded_[aux_slot_] = true;
+        aux_read_since_event_[aux_slot_] = false;
+      }
+    }
+    compute_stream_ = stream;
+  }
   void SetRopeScaling(const tvmkv_rope_scaling* scaling, const float* rope_ext_factors) {
     has_rope_scaling_ = scaling != nullptr && scaling->rope_type != TVMKV_ROPE_FREQ_DEFAULT;
     KV_UNSUPPORTED(has_rope_scaling_ && rope_mode_ == TVMKV_ROPE_INLINE)
@@ -478,7 +502,7 @@ class PagedKVCache {
       if (aux_consumed_[i]) (void)hipEventDestroy(aux_consumed_[i]);
       aux_device_[i] = aux_staging_[i] = nullptr;
       aux_copied_[i] = aux_consumed_[i] = nullptr;
-      aux_consumed_recorded_[i] = aux_slot_used_[i] = false;
+      aux_consumed_recorded_[i] = aux_slot_used_[i] = aux_read_since_event_[i] = false;
     }
     (void)hipFree(commit_device_);
     if (commit_staging_) (void)hipHostFree(commit_staging_);
@@ -492,12 +516,23 @@ class PagedKVCache {
     compute_done_ = nullptr;
   }
 
+  // Kernels of the step were enqueued on the compute stream.  Nothing is recorded here: an event
+  // record between the launches of two layers costs the device ~5 us of idle time each, so the
+  // events are recorded where somebody is about to wait for them (CopyStreamWaitsForCompute,
+  // BeginForward).
   void RecordComputeEvent() {
-    HIP_CHECK(hipEventRecord(compute_done_, compute_stream_));
-    compute_event_recorded_ = true;
-    // the kernels enqueued so far are the last readers of the auxiliary buffer in use
-    HIP_CHECK(hipEventRecord(aux_consumed_[aux_slot_], compute_stream_));
-    aux_consumed_recorded_[aux_slot_] = true;
+    compute_work_since_event_ = true;
+    aux_read_since_event_[aux_slot_] = true;  // by kernels that read the auxiliary buffer in use
+  }
+
+  // Orders what is enqueued on the copy stream next after everything enqueued on the compute stream so far.
+  void CopyStreamWaitsForCompute() {
+    if (compute_work_since_event_) {
+      HIP_CHECK(hipEventRecord(compute_done_, compute_stream_));
+      compute_event_recorded_ = true;
+      compute_work_since_event_ = false;
+    }
+    if (compute_event_recorded_) HIP_CHECK(hipStreamWaitEvent(copy_stream_, compute_done_, 0));
   }
 
   // The partial-page copies that forks have asked for since the last call (:721-734).  They run on the
@@ -511,7 +546,7 @@ class PagedKVCache {
       return;
     }
     HIP_CHECK(hipSetDevice(device_));
-    if (compute_event_recorded_) HIP_CHECK(hipStreamWaitEvent(copy_stream_, compute_done_, 0));
+    CopyStreamWaitsForCompute();
     for (; page_copies_issued_ < log.size(); page_copies_issued_ += 3) {
       const int32_t src = static_cast<int32_t>(log[page_copies_issued_]);
       const int32_t tgt = static_cast<int32_t>(log[page_copies_issued_ + 1]);
@@ -550,7 +585,7 @@ class PagedKVCache {
                 total_copy_length * sizeof(int32_t));
     int32_t* device = static_cast<int32_t*>(commit_device_);
     // after the attention kernels of the step that computed on these slots
-    if (compute_event_recorded_) HIP_CHECK(hipStreamWaitEvent(copy_stream_, compute_done_, 0));
+    CopyStreamWaitsForCompute();
     HIP_CHECK(hipMemcpyAsync(device, staging, (pos_begin + 2 * total_copy_length) * sizeof(int32_t),
                              hipMemcpyHostToDevice, copy_stream_));
     HIP_CHECK(hipEventRecord(commit_copied_, copy_stream_));
@@ -759,6 +794,7 @@ class PagedKVCache {
   hipStream_t copy_stream_ = nullptr;
   hipEvent_t compute_done_ = nullptr;
   bool compute_event_recorded_ = false;
+  bool compute_work_since_event_ = false;
   bool copy_stream_has_work_ = false;
   std::vector<void*> pages_;
   void *temp_q_ = nullptr, *temp_k_ = nullptr, *temp_v_ = nullptr, *temp_out_ = nullptr;
@@ -769,6 +805,7 @@ class PagedKVCache {
   hipEvent_t aux_copied_[2] = {nullptr, nullptr};
   hipEvent_t aux_consumed_[2] = {nullptr, nullptr};  // recorded on the compute stream behind a slot's last readers
   bool aux_consumed_recorded_[2] = {false, false};
+  bool aux_read_since_event_[2] = {false, false};
   bool aux_slot_used_[2] = {false, false};
   bool aux_needs_upload_ = false;
   int aux_slot_ = 0;
