@@ -256,6 +256,59 @@ def cache_object_decode(torch, dev, layers=32, seed=1):
             "tokens_per_s": round(B / (gpu_ms * 1e-3), 1)}
 
 
+def cache_object_prefill(torch, dev, layers=8):
+    """configs[2] through the cache object: the prefixes are cached by chunked-prefill steps, then every
+    timed step appends the 8 chunks in one begin_forward, runs attention_with_fused_qkv on every layer
+    and pops the chunks again (popn), so that all timed steps see the same cache."""
+    from tvm_amd import get_global_func as gf
+
+    pw = prefill_workload()
+    prefix, chunk = [int(x) for x in pw["prefix"]], [int(x) for x in pw["chunk"]]
+    B = len(prefix)
+    total = sum(chunk)
+    capacity = sum(prefix) + total + 2 * B * PS
+    chunk_cap = (total + 255) // 256 * 256
+    cache = gf("vm.builtin.paged_attention_kv_cache_create")(
+        [B, capacity, chunk_cap, PS, 0], [0, layers], HQ, HKV, D, D, [0] * layers, False, 1, 1.0, 1e4, None,
+        torch.empty((), dtype=torch.float16, device=dev))
+    cache.set_stream(torch.cuda.current_stream().cuda_stream)
+    f_add = gf("vm.builtin.kv_state_add_sequence")
+    f_begin = gf("vm.builtin.kv_state_begin_forward")
+    f_end = gf("vm.builtin.kv_state_end_forward")
+    f_popn = gf("vm.builtin.kv_state_popn")
+    f_attn = gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")
+    sm_scale = D ** -0.5
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2)
+    qkv = torch.randn((chunk_cap, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16)
+    out = torch.empty((chunk_cap, HQ, D), dtype=torch.float16, device=dev)
+    for b in range(B):
+        f_add(cache, b)
+        if prefix[b] > 0:
+            f_begin(cache, [b], [prefix[b]], None)
+            for layer in range(layers):
+                f_attn(cache, layer, sm_scale, qkv[:prefix[b]], out[:prefix[b]])
+            f_end(cache)
+    ids = list(range(B))
+
+    def step(_):
+        f_begin(cache, ids, chunk, None)
+        for layer in range(layers):
+            f_attn(cache, layer, sm_scale, qkv[:total], out[:total])
+        f_end(cache)
+        for b in range(B):
+            f_popn(cache, b, chunk[b])
+
+    for _ in range(2):
+        step(0)
+    ms = time_region(torch, step, 10, SETTLE_S)
+    tflops = layers * pw["flops"] / (ms * 1e-3) / 1e12
+    return {"workload": f"configs[2] through the cache object: {layers} layers; per step one begin_forward that appends the 8 "
+                        f"chunks, {layers} x attention_with_fused_qkv, end_forward, and popn of the chunks",
+            "layers": layers, "ms_per_step": round(ms, 4), "ms_per_layer": round(ms / layers, 4),
+            "tflops": round(tflops, 1), "frac_of_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
+
+
 # HBM bytes per launch of the decode entry point, from rocprofv3 counter runs of this file
 # (profiles/decode_mfma_kernel_cfg2_batched_decode.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 in KiB per
 # dispatch of decode_mfma_kernel (it merges the chunks itself); the scales come from the plain copy
@@ -732,6 +785,8 @@ def main():
         result["extras"] = extras(torch, K, dev)
         torch.cuda.empty_cache()
         result["extras"]["cache_object_decode"] = cache_object_decode(torch, dev)
+        torch.cuda.empty_cache()
+        result["extras"]["cache_object_prefill"] = cache_object_prefill(torch, dev)
     print(json.dumps(result))
 
 
