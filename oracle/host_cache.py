@@ -363,6 +363,11 @@ class HostCache:
             _check(block.sliding_window_offset == 0, "offset")
             block.sink_length = seq.last_block_attn_sink_size
             block.sliding_window_offset = seq.last_block_attn_sink_size
+        # the reference erases pages without looking (:1966-1972): undefined behaviour when a shared
+        # prefix alone is longer than the window; an error here and in the library
+        _check(length_to_slide <= block.seq_length - block.sink_length,
+               f"The sliding window has to drop {length_to_slide} tokens, but the last block of the sequence holds only "
+               f"{block.seq_length - block.sink_length} behind its attention sink.")
         num_sink_pages = (block.sink_length + ps - 1) // ps
         page_idx_after = (block.sliding_window_offset + length_to_slide) // ps
         page_start_offset_after = (block.sliding_window_offset + length_to_slide) % ps

@@ -276,6 +276,12 @@ void KVBookkeeper::SlideWindow(SeqRecord& seq) {
     blocks_.sink_length[b] = seq.last_block_sink;
     blocks_.window_offset[b] = seq.last_block_sink;
   }
+  // Only the last block slides.  The reference erases pages without looking (:1966-1972) and runs off
+  // the end of the block's page list when a shared prefix alone is longer than the window; here
+  // that is an error like any other.
+  KV_CHECK(to_slide <= blocks_.seq_length[b] - blocks_.sink_length[b])
+      << "The sliding window has to drop " << to_slide << " tokens, but the last block of the sequence holds only "
+      << blocks_.seq_length[b] - blocks_.sink_length[b] << " behind its attention sink.";
   const int32_t sink_pages = (blocks_.sink_length[b] + ps - 1) / ps;
   int32_t first_page = (blocks_.window_offset[b] + to_slide) / ps;
   const int32_t first_slot = (blocks_.window_offset[b] + to_slide) % ps;
