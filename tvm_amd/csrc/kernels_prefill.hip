@@ -112,24 +112,48 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   // last row tile to the first, since under the causal mask the last rows see the most keys.
   const int slot = blockIdx.y;
   int b, local_slot;
+  // the sequence's entries of the index arrays: from the lanes that ranked the sequences where they
+  // did (no second round trip to memory), loaded otherwise
+  int seq_q0, seq_q1, seq_p0 = 0, seq_p1 = 0, seq_last = 0, seq_k0 = 0, seq_k1 = 0;
   if (p.batch_size <= 64) {
     int my_tiles = 0, my_key = -1;
+    int lq0 = 0, lq1 = 0, lp0 = 0, lp1 = 0, llast = 0, lk0 = 0, lk1 = 0;
     if (lane < p.batch_size) {
-      my_tiles = ((p.q_indptr[lane + 1] - p.q_indptr[lane]) * group + BM - 1) / BM;
-      my_key = 0;
-      if (PAGED || BOTH) my_key += (p.page_indptr[lane + 1] - p.page_indptr[lane]) * PS;
-      if (!PAGED) my_key += p.kv_indptr[lane + 1] - p.kv_indptr[lane];
+      lq0 = p.q_indptr[lane];
+      lq1 = p.q_indptr[lane + 1];
+      if (PAGED || BOTH) {
+        lp0 = p.page_indptr[lane];
+        lp1 = p.page_indptr[lane + 1];
+        llast = p.last_page_len[lane];
+      }
+      if (!PAGED) {
+        lk0 = p.kv_indptr[lane];
+        lk1 = p.kv_indptr[lane + 1];
+      }
+      my_tiles = ((lq1 - lq0) * group + BM - 1) / BM;
+      my_key = (lp1 - lp0) * PS + (lk1 - lk0);
     }
     int my_begin = 0;  // row tiles of the sequences ranked before this lane's
+    // (key, index) as one sortable number, compared without branches: every workgroup runs this
+    // loop, and with short sequences it is a visible part of its life
+    const long long my_rank = (static_cast<long long>(my_key) << 8) | (63 - lane);
     for (int j = 0; j < p.batch_size; ++j) {
       const int key_j = __builtin_amdgcn_readlane(my_key, j);
       const int tiles_j = __builtin_amdgcn_readlane(my_tiles, j);
-      if (key_j > my_key || (key_j == my_key && j < lane)) my_begin += tiles_j;
+      const long long rank_j = (static_cast<long long>(key_j) << 8) | (63 - j);
+      my_begin += rank_j > my_rank ? tiles_j : 0;
     }
     const uint64_t owner = __ballot(lane < p.batch_size && slot >= my_begin && slot < my_begin + my_tiles);
     if (owner == 0) return;  // the grid is sized from shapes alone and has spare slots
     b = __builtin_amdgcn_readfirstlane(__ffsll(static_cast<long long>(owner)) - 1);
     local_slot = slot - __builtin_amdgcn_readlane(my_begin, b);
+    seq_q0 = __builtin_amdgcn_readlane(lq0, b);
+    seq_q1 = __builtin_amdgcn_readlane(lq1, b);
+    seq_p0 = __builtin_amdgcn_readlane(lp0, b);
+    seq_p1 = __builtin_amdgcn_readlane(lp1, b);
+    seq_last = __builtin_amdgcn_readlane(llast, b);
+    seq_k0 = __builtin_amdgcn_readlane(lk0, b);
+    seq_k1 = __builtin_amdgcn_readlane(lk1, b);
   } else {
     int lo = 0, hi = p.batch_size - 1;
     while (lo < hi) {
@@ -142,9 +166,20 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     }
     b = lo;
     local_slot = slot - tile_slot_begin(p.q_indptr, b, group);
+    seq_q0 = p.q_indptr[b];
+    seq_q1 = p.q_indptr[b + 1];
+    if (PAGED || BOTH) {
+      seq_p0 = p.page_indptr[b];
+      seq_p1 = p.page_indptr[b + 1];
+      seq_last = p.last_page_len[b];
+    }
+    if (!PAGED) {
+      seq_k0 = p.kv_indptr[b];
+      seq_k1 = p.kv_indptr[b + 1];
+    }
   }
-  const int q_start = p.q_indptr[b];
-  const int qo_len = p.q_indptr[b + 1] - q_start;
+  const int q_start = seq_q0;
+  const int qo_len = seq_q1 - q_start;
   const int rows = qo_len * group;
   const int n_row_tiles = (rows + BM - 1) / BM;
   if (local_slot >= n_row_tiles) return;
@@ -154,21 +189,21 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   // kBoth: the key axis is [cached tokens, padded to prefix_pad][new tokens]
   int phys_len = 0, kv_start = 0, pbeg = 0, sink = 0, win_lo = 0, prefix_len = 0, prefix_pad = 0;
   if (PAGED || BOTH) {
-    pbeg = p.page_indptr[b];
-    const int npages = p.page_indptr[b + 1] - pbeg;
-    phys_len = npages > 0 ? (npages - 1) * PS + p.last_page_len[b] : 0;
+    pbeg = seq_p0;
+    const int npages = seq_p1 - pbeg;
+    phys_len = npages > 0 ? (npages - 1) * PS + seq_last : 0;
     if (EXT && p.sink_size != nullptr && npages > 0) {
       sink = p.sink_size[b];
       win_lo = p.window_offset[b];
     }
   }
   if (!PAGED) {
-    kv_start = p.kv_indptr[b];
+    kv_start = seq_k0;
     if (BOTH) {
       prefix_len = phys_len;
       prefix_pad = (prefix_len + BN - 1) / BN * BN;
     }
-    phys_len = prefix_pad + p.kv_indptr[b + 1] - kv_start;
+    phys_len = prefix_pad + seq_k1 - kv_start;
   }
   const int prefix_tiles = prefix_pad / BN;
   const int hole_tile = (BOTH && prefix_len < prefix_pad) ? prefix_tiles - 1 : -1;  // its end is padding
@@ -501,11 +536,57 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
 
     if (kv0 >= t_limit_max) continue;  // wave-uniform: every row of this wave is masked out
 
-    if (unmasked) {
-      // Every row of the wave sees the whole tile (all tiles left of the causal diagonal): no
-      // masking, and the two 32-token halves are software-pipelined so that the wave's own matrix
-      // and vector work overlap: S1 = K1 Q^T runs under the softmax of S0, and O += V0 P0 under the
-      // softmax of S1.
+    // The two 32-token halves of a tile, software-pipelined so that the wave's own matrix and vector
+    // work overlap: S1 = K1 Q^T runs under the softmax of S0, and O += V0 P0 under the softmax of S1.
+    // MASKED: rows of the wave see different parts of the tile (plain cache: the tiles on the causal
+    // diagonal and at the end of a source), each lane masks its row's scores against its own bound.
+    auto two_halves = [&](auto masked_c) {
+      constexpr bool MASKED = decltype(masked_c)::value;
+      auto mask = [&](float16_t& acc, int t0) {
+        const int rel = t_my_limit - t0 - half * 4;  // element j is token t0 + half*4 + (j/4)*8 + j%4
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[j] = ((j >> 2) * 8 + (j & 3)) < rel ? acc[j] : -3.0e38f;
+      };
+      half8_t kf[KS];
+      half8_t vf[DB][2];
+      half8_t pf[2];
+      read_k(Ks, 0, kf);
+      __builtin_amdgcn_sched_barrier(0);
+      float16_t s0 = qk(kf);
+      read_k(Ks, 1, kf);
+      read_v(Vs, 0, vf);
+      if (MASKED) mask(s0, kv0);
+      const float a0 = advance_max(row_max(s0));
+      rescale(a0);
+      __builtin_amdgcn_sched_barrier(0);
+      float16_t s1 = qk(kf);
+      probs(s0, pf);
+      interleave_mfma_valu<KS>();
+      __builtin_amdgcn_sched_barrier(0);
+      if (MASKED) mask(s1, kv0 + 32);
+      const float a1 = advance_max(row_max(s1));
+      pv(vf, pf);
+      probs(s1, pf);
+      interleave_mfma_valu<2 * DB>();
+      __builtin_amdgcn_sched_barrier(0);
+      read_v(Vs, 1, vf);
+      rescale(a1);
+      pv(vf, pf);
+    };
+    if constexpr (DQK <= 128) {
+      if (unmasked) {  // every row of the wave sees the whole tile (all tiles left of the causal diagonal)
+        two_halves(std::false_type{});
+        continue;
+      }
+      if constexpr (!EXT && TB == 2) {
+        if (kv0 + 32 < t_limit_max) {  // wave-uniform: both halves hold keys that some row sees
+          two_halves(std::true_type{});
+          continue;
+        }
+      }
+    } else if (unmasked) {
+      // d_qk 192 has no register to spare: the same unmasked pipeline written out, which the compiler
+      // allocates without spilling (as a call of the generic form above it spills ten registers)
       half8_t kf[KS];
       half8_t vf[DB][2];
       half8_t pf[2];
