@@ -133,16 +133,22 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
       my_tiles = ((lq1 - lq0) * group + BM - 1) / BM;
       my_key = (lp1 - lp0) * PS + (lk1 - lk0);
     }
-    int my_begin = 0;  // row tiles of the sequences ranked before this lane's
-    // (key, index) as one sortable number, compared without branches: every workgroup runs this
-    // loop, and with short sequences it is a visible part of its life
-    const long long my_rank = (static_cast<long long>(my_key) << 8) | (63 - lane);
-    for (int j = 0; j < p.batch_size; ++j) {
-      const int key_j = __builtin_amdgcn_readlane(my_key, j);
-      const int tiles_j = __builtin_amdgcn_readlane(my_tiles, j);
-      const long long rank_j = (static_cast<long long>(key_j) << 8) | (63 - j);
-      my_begin += rank_j > my_rank ? tiles_j : 0;
+    // Row tiles of the sequences ranked before this lane's.  (key, index) is one sortable 32-bit
+    // number (keys beyond 2^24 tokens rank equal), compared without branches, four sequences per
+    // round with separate sums: every workgroup runs this loop alone on its SIMDs, one dependent
+    // instruction after the other, and with short sequences it is a visible part of its life.
+    const int my_rank = min(my_key, (1 << 24) - 1) * 64 + (63 - lane);  // negative for the lanes past the batch
+    int begin4[4] = {0, 0, 0, 0};
+    for (int j = 0; j < p.batch_size; j += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        // lanes past the batch rank below every sequence and have no tiles
+        const int rank_j = __builtin_amdgcn_readlane(my_rank, (j + u) & 63);
+        const int tiles_j = __builtin_amdgcn_readlane(my_tiles, (j + u) & 63);
+        begin4[u] += rank_j > my_rank ? tiles_j : 0;
+      }
     }
+    const int my_begin = (begin4[0] + begin4[1]) + (begin4[2] + begin4[3]);
     const uint64_t owner = __ballot(lane < p.batch_size && slot >= my_begin && slot < my_begin + my_tiles);
     if (owner == 0) return;  // the grid is sized from shapes alone and has spare slots
     b = __builtin_amdgcn_readfirstlane(__ffsll(static_cast<long long>(owner)) - 1);
