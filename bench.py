@@ -554,6 +554,42 @@ def extras(torch, K, dev):
     return out
 
 
+def hold(which, seconds):
+    """Runs one kernel back to back for `seconds` and prints its rate over the last second."""
+    import torch
+
+    from tvm_amd import kernels as K
+
+    dev = "cuda:0"
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    if which == "prefill":
+        pw = prefill_workload()
+        fn, _ = make_prefill_step(torch, K, pw, gen, dev)
+        unit, work = "TFLOP/s", pw["flops"] / 1e12
+    elif which == "mfma":
+        ops = torch.randn((256, 16), device=dev).to(torch.float16)
+        sums = torch.empty((512, 256), dtype=torch.float32, device=dev)
+        fn = lambda i: K.mfma_loop(ops, sums, 4096)
+        unit, work = "TFLOP/s (random operands)", 2.0 * 32 * 32 * 16 * 8 * 4096 * 4 * 512 / 1e12
+    else:
+        wl = decode_workload(steps=1)
+        t = wl["tables"][0]
+        B = wl["batch"]
+        pages = torch.randn((wl["pool_pages"], 2, HKV, PS, D), generator=gen, device=dev, dtype=torch.float16)
+        q = torch.randn((B, HQ, D), generator=gen, device=dev, dtype=torch.float16)
+        out = torch.empty_like(q)
+        lse = torch.empty((B, HQ), dtype=torch.float32, device=dev)
+        z = torch.zeros(B, dtype=torch.int32, device=dev)
+        tabs = {k: torch.tensor(t[k], dtype=torch.int32, device=dev) for k in ("page_indptr", "page_values", "last_page_len")}
+        fn = lambda i: K.batch_decode_paged_kv(q, pages, tabs["page_indptr"], tabs["page_values"], tabs["last_page_len"],
+                                               z, z, out, lse, 0, 1.0, 1e4, D ** -0.5)
+        unit, work = "TB/s", (float(t["kv_len"].sum()) * TOKEN_BYTES + B * HQ * D * 4) / 1e12
+    settle(torch, fn, max(seconds - 1.0, 0.5))
+    ms = time_region(torch, fn, 200)
+    print(json.dumps({"held": which, "seconds": seconds, "ms": round(ms, 4), "rate": round(work / (ms * 1e-3), 2), "unit": unit}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -569,9 +605,16 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the plain 2 GiB streaming read and copy kernels (bandwidth calibration; "
                          "known-size dispatches for scaling rocprofv3 traffic counters)")
+    ap.add_argument("--hold", choices=["prefill", "mfma", "decode"],
+                    help="only run one kernel back to back for --hold-seconds and print its rate: a steady load to "
+                         "read the board's power and clocks under from another shell (rocm-smi)")
+    ap.add_argument("--hold-seconds", type=float, default=6.0)
     args = ap.parse_args()
     if args.calibrate:
         calibrate()
+        return
+    if args.hold:
+        hold(args.hold, args.hold_seconds)
         return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; the path shards per kv head without any exchange "
