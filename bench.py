@@ -439,35 +439,40 @@ def extras(torch, K, dev):
         walk(0)
         return np.asarray(labels, dtype=np.int32)
 
-    labels = preorder(6)                                          # 63 draft tokens per sequence
-    nodes = len(labels)
     ctx = rng.integers(1024, 8192, size=nseq, endpoint=True)    # cached tokens before the tree
-    kv = ctx + nodes                                              # the tree's tokens are appended already
-    npages = (kv + ps - 1) // ps
-    indptr = np.concatenate([[0], np.cumsum(npages)])
-    qi = np.arange(nseq + 1) * nodes
-    q = torch.randn((nseq * nodes, hq, d), device=dev).to(torch.float16)
-    o = torch.empty_like(q)
-    lse = torch.empty((nseq * nodes, hq), dtype=torch.float32, device=dev)
-    zq = torch.zeros(nseq * nodes, dtype=torch.int32, device=dev)
-    args = (q, i32(qi), pages, i32(indptr), i32(perm[:indptr[-1]]), i32((kv - 1) % ps + 1), z, zq, o, lse, 0, 1.0, 1e4,
-            d ** -0.5, i32(qi), i32(np.tile(labels, (nseq, 1)).reshape(-1)))
-    K.tree_attn_paged_kv(*args)
-    K.prefill_clock_probe(True)
-    settle(torch, lambda i: K.tree_attn_paged_kv(*args))
-    K.prefill_clock_probe_read(reset=True)
-    ms = time_region(torch, lambda i: K.tree_attn_paged_kv(*args), 20)
-    cycles, ticks, _ = K.prefill_clock_probe_read(reset=True)
-    K.prefill_clock_probe(False)
-    depth_sum = float(sum((lv + 1) * 2 ** lv for lv in range(6)))  # visible tree tokens summed over the nodes
-    flops = 4.0 * hq * d * (float(ctx.sum()) * nodes + nseq * depth_sum)
-    nbytes = float(kv.sum()) * 2 * hkv * d * 2 + 2 * nseq * nodes * hq * d * 2
-    out["token_tree_verify"] = {"workload": "64 seqs, ctx U[1024,8192], a 63-node binary draft tree each (appended), "
-                                            "one launch of the tree-masked paged kernel, Hq32/Hkv8/D128",
-                                "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
-                                "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
-                                "GBps": round(nbytes / ms / 1e6, 1),
-                                "shader_clock_MHz": round(cycles / max(ticks, 1) * 100.0, 1)}
+
+    def tree_verify(depth):
+        labels = preorder(depth)                                  # 2^depth - 1 draft tokens per sequence
+        nodes = len(labels)
+        kv = ctx + nodes                                          # the tree's tokens are appended already
+        npages = (kv + ps - 1) // ps
+        indptr = np.concatenate([[0], np.cumsum(npages)])
+        qi = np.arange(nseq + 1) * nodes
+        q = torch.randn((nseq * nodes, hq, d), device=dev).to(torch.float16)
+        o = torch.empty_like(q)
+        lse = torch.empty((nseq * nodes, hq), dtype=torch.float32, device=dev)
+        zq = torch.zeros(nseq * nodes, dtype=torch.int32, device=dev)
+        args = (q, i32(qi), pages, i32(indptr), i32(perm[:indptr[-1]]), i32((kv - 1) % ps + 1), z, zq, o, lse, 0, 1.0,
+                1e4, d ** -0.5, i32(qi), i32(np.tile(labels, (nseq, 1)).reshape(-1)))
+        K.tree_attn_paged_kv(*args)
+        K.prefill_clock_probe(True)
+        settle(torch, lambda i: K.tree_attn_paged_kv(*args))
+        K.prefill_clock_probe_read(reset=True)
+        ms = time_region(torch, lambda i: K.tree_attn_paged_kv(*args), 20)
+        cycles, ticks, _ = K.prefill_clock_probe_read(reset=True)
+        K.prefill_clock_probe(False)
+        depth_sum = float(sum((lv + 1) * 2 ** lv for lv in range(depth)))  # visible tree tokens summed over the nodes
+        flops = 4.0 * hq * d * (float(ctx.sum()) * nodes + nseq * depth_sum)
+        nbytes = float(kv.sum()) * 2 * hkv * d * 2 + 2 * nseq * nodes * hq * d * 2
+        return {"workload": f"64 seqs, ctx U[1024,8192], a {nodes}-node binary draft tree each (appended), one launch of the "
+                            f"tree-masked paged kernel, Hq32/Hkv8/D128: {nodes * hq // hkv} query rows per kv head",
+                "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                "GBps": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                "shader_clock_MHz": round(cycles / max(ticks, 1) * 100.0, 1)}
+
+    out["token_tree_verify"] = tree_verify(6)            # 63 nodes: 252 rows per kv head, two row tiles, compute-bound
+    out["token_tree_verify_15_nodes"] = tree_verify(4)   # 60 rows per kv head: one row tile, the K/V stream decides
     del pages
     torch.cuda.empty_cache()
 
