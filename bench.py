@@ -577,6 +577,29 @@ def hold(which, seconds):
         sums = torch.empty((512, 256), dtype=torch.float32, device=dev)
         fn = lambda i: K.mfma_loop(ops, sums, 4096)
         unit, work = "TFLOP/s (random operands)", 2.0 * 32 * 32 * 16 * 8 * 4096 * 4 * 512 / 1e12
+    elif which in ("mla_prefill", "mla_decode"):
+        hq, dl, dr, ps = 128, 512, 64, 64
+        rng = np.random.default_rng(4)
+        if which == "mla_decode":
+            prefix, chunk, causal = rng.integers(2048, 8192, size=32, endpoint=True) - 1, np.ones(32, dtype=np.int64), 0
+        else:
+            prefix, chunk, causal = np.full(4, 2048), np.full(4, 1024), 1
+        kv = prefix + chunk
+        npg = (kv + ps - 1) // ps
+        pool = int(npg.sum()) + 8
+        perm = rng.permutation(pool).astype(np.int32)
+        pg = (torch.randn((pool, ps, dl + dr), device=dev) * 0.5).to(torch.float16)
+        ip = np.concatenate([[0], np.cumsum(npg)])
+        qi = np.concatenate([[0], np.cumsum(chunk)])
+        n = int(qi[-1])
+        i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=dev)
+        q = (torch.randn((n, hq, dl + dr), device=dev) * 0.5).to(torch.float16)
+        o = torch.empty((n, hq, dl), dtype=torch.float16, device=dev)
+        lse = torch.empty((n, hq), dtype=torch.float32, device=dev)
+        a = (q, i32(qi), pg, i32(ip), i32(perm[:ip[-1]]), i32((kv - 1) % ps + 1), o, lse, causal, (128 + 64) ** -0.5)
+        fn = lambda i: K.batch_prefill_paged_kv_mla(*a)
+        pairs = float(np.sum(chunk * prefix + chunk * (chunk + 1) / 2)) if causal else float(np.sum(chunk * kv))
+        unit, work = "TFLOP/s", 2.0 * hq * (2 * dl + dr) * pairs / 1e12
     else:
         wl = decode_workload(steps=1)
         t = wl["tables"][0]
@@ -610,7 +633,7 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the plain 2 GiB streaming read and copy kernels (bandwidth calibration; "
                          "known-size dispatches for scaling rocprofv3 traffic counters)")
-    ap.add_argument("--hold", choices=["prefill", "mfma", "decode"],
+    ap.add_argument("--hold", choices=["prefill", "mfma", "decode", "mla_prefill", "mla_decode"],
                     help="only run one kernel back to back for --hold-seconds and print its rate: a steady load to "
                          "read the board's power and clocks under from another shell (rocm-smi)")
     ap.add_argument("--hold-seconds", type=float, default=6.0)
