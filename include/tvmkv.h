@@ -358,7 +358,8 @@ int tvmkv_get_option(const char* name, int64_t* value);
  * kernel repeats on the device).  page_indptr_host is a HOST array (batch_size + 1).  Writes the
  * chunk size in pages and the number of chunk slots of the launch; when slot_seq and slot_chunk are
  * not NULL (room for slot_capacity entries each) also the sequence and chunk index every slot
- * resolves to, -1 for a spare slot. */
+ * resolves to, -1 for a spare slot.  The figures are those of a cache with 16-token pages; with pages
+ * of 16 << s tokens (s = 1, 2, 3) the launch uses chunks of max(1, chunk_pages(nnz_pages << s) >> s) pages. */
 int tvmkv_decode_split_plan(const int32_t* page_indptr_host, int32_t batch_size, int64_t nnz_pages,
                             int32_t h_kv, int32_t* chunk_pages, int64_t* num_slots, int32_t* slot_seq,
                             int32_t* slot_chunk, int64_t slot_capacity);

@@ -95,8 +95,9 @@ class Mirror:
             assert_close(gk, ek, atol=1e-3, rtol=2e-3, what=f"cached K of seq {sid}")
 
 
-def test_identical_inputs_through_oracle_and_gpu_caches():
-    m = Mirror([16, 4096, 1024, 16, 0], 2, 32, 8, 128)
+@pytest.mark.parametrize("page_size", [16, 32, 64])
+def test_identical_inputs_through_oracle_and_gpu_caches(page_size):
+    m = Mirror([16, 4096, 1024, page_size, 0], 2, 32, 8, 128)
     m.step([(0, 60), (1, 88), (2, 17), (3, 4)])
     m.step([((4, 3, -1), 35)])
     m.step([((5, 0, 33), 20)])            # fork inside a page -> page copy on the device
@@ -264,3 +265,15 @@ def test_attention_with_shared_kv_reads_the_source_layer():
             torch.zeros((5, hkv, d), dtype=torch.float16, device=DEV),
             torch.zeros((5, hkv, d), dtype=torch.float16, device=DEV),
             torch.zeros((5, hq, d), dtype=torch.float16, device=DEV))
+
+
+@pytest.mark.parametrize("runner,rope_mode,sliding", [(S.run_fork_sequence, S.ROPE_NORMAL, 0), (S.run_tree_attn, S.ROPE_NORMAL, 0),
+                                                      (S.run_sliding_window_fork, S.ROPE_INLINE, 1),
+                                                      (S.run_sliding_window_page_reuse, S.ROPE_INLINE, 1)])
+def test_reference_scenarios_with_pages_of_32_tokens(runner, rope_mode, sliding):
+    """The reference's scenarios on a cache whose pages hold 32 tokens (the kernels walk such pages as
+    two runs of 16): forks inside a page, token trees with their commit, sliding windows."""
+    layers, hq, hkv, d = 2, 8, 2, 128
+    cache = GpuCache([32, 2048, 512, 32, sliding], layers, hq, hkv, d, d, rope_mode=rope_mode)
+    sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=rope_mode, seed=9, tol=4e-3)
+    runner(sc)

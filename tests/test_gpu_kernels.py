@@ -153,8 +153,8 @@ def test_merge_state_inplace(h, d):
 
 
 # ------------------------------------------------------------------------------ decode
-def _decode_both(rng, kv_lens, hq, hkv, d, npages, scale=1.0):
-    pages, indptr, values, last, ks, vs = build_paged_kv(rng, kv_lens, npages, hkv, 16, d, scale=scale)
+def _decode_both(rng, kv_lens, hq, hkv, d, npages, scale=1.0, page_size=16):
+    pages, indptr, values, last, ks, vs = build_paged_kv(rng, kv_lens, npages, hkv, page_size, d, scale=scale)
     b = len(kv_lens)
     q = rng.standard_normal((b, hq, d)).astype(F16)
     eo, el = np.zeros((b, hq, d), F16), np.zeros((b, hq), np.float32)
@@ -178,6 +178,19 @@ def test_decode_ragged_lengths_against_oracle(hq, hkv, d):
     for i, n in enumerate(kv_lens):
         if n == 0:
             assert not go[i].any() and np.all(gl[i] == np.float32(-5e4))
+
+
+@pytest.mark.parametrize("page_size", [32, 64, 128])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 4, 64)])
+def test_decode_other_page_sizes(page_size, hq, hkv, d):
+    """Pages of 32, 64 and 128 tokens (the kernel walks them as runs of 16-token pages): partly filled
+    last pages at every position inside a page, several chunks, empty sequences."""
+    rng = np.random.default_rng(50 + page_size)
+    kv_lens = [0, 1, 15, 16, 17, page_size - 1, page_size, page_size + 1, 3 * page_size + 5, 700, 2500, 33]
+    go, gl, eo, el = _decode_both(rng, kv_lens, hq, hkv, d, npages=3 + sum((n + page_size - 1) // page_size for n in kv_lens),
+                                  page_size=page_size)
+    assert_close(go, eo, what=f"decode out, page size {page_size}")
+    assert_close(gl, el, atol=1e-3, rtol=1e-4, what=f"decode lse, page size {page_size}")
 
 
 def test_decode_cfg1_shapes_against_oracle():
@@ -359,8 +372,8 @@ def test_ragged_prefill_scores_that_keep_growing(causal):
     assert_close(host(gl), el, atol=5e-3, rtol=1e-4, what="ragged growing scores lse")
 
 
-def _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages):
-    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, kv_lens, npages, hkv, 16, d)
+def _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages, page_size=16):
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, kv_lens, npages, hkv, page_size, d)
     n = sum(q_lens)
     qindptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
     q = rng.standard_normal((n, hq, d)).astype(F16)
@@ -385,6 +398,100 @@ def test_paged_prefill_against_oracle(hq, hkv, d, causal):
     go, gl, eo, el = _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages=64)
     assert_close(go, eo, what="paged out")
     assert_close(gl, el, atol=2e-3, rtol=1e-4, what="paged lse")
+
+
+@pytest.mark.parametrize("page_size", [32, 64, 128])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+def test_paged_kernels_with_other_page_sizes(page_size, hq, hkv, d):
+    """Pages of 32, 64 and 128 tokens through every kernel that reads the page pool with 16-token steps:
+    plain and causal paged prefill, the sliding-window / inline-RoPE forms of prefill and decode, the
+    tree-masked kernel, and the one-pass chunked prefill."""
+    from tests.test_oracle_kernels import sliding_case, tree_paged_case
+    from tests.util import REFERENCE_TREES, random_forest
+    rng = np.random.default_rng(60 + page_size)
+    ps = page_size
+    # last pages filled to every kind of boundary: one token, a 16-token run, a tile of 64, the page
+    kv_lens = [40, 16, 0, 75, 200, ps, 1, ps + 1, 2 * ps - 1, 700]
+    q_lens = [7, 16, 3, 30, 64, 1, 1, 20, 5, 130]
+    need = lambda lens: 4 + sum((n + ps - 1) // ps for n in lens)
+    for causal in (0, 1):
+        lens = [max(k, q) for k, q in zip(kv_lens, q_lens)] if causal else kv_lens
+        go, gl, eo, el = _paged_both(rng, lens, q_lens, hq, hkv, d, causal, need(lens), page_size=ps)
+        assert_close(go, eo, what=f"paged out, page size {ps}, causal {causal}")
+        assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"paged lse, page size {ps}, causal {causal}")
+
+    # sliding-window cache + inline RoPE: prefill with the per-layer window mask, and decode
+    spec = [(100, 4, 20), (257, 0, 0), (330, 16, 48), (33, 2, 2), (ps, 16, 32), (90, 0, 17), (2300, 8, 40)]
+    sq_lens = [7, 64, 33, 3, 1, 30, 40]
+    pages, pindptr, pvalues, info, k_log, _ = sliding_case(rng, spec, hkv, d, ps=ps, npages=need([x[0] for x in spec]))
+    n = sum(sq_lens)
+    qindptr = np.concatenate([[0], np.cumsum(sq_lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k_off = rng.integers(0, 200, size=len(spec)).astype(np.int32)
+    q_pos = np.concatenate([k_off[i] + len(k_log[i]) - sq_lens[i] + np.arange(sq_lens[i]) for i in range(len(spec))])
+    q_pos = q_pos.astype(np.int32)
+    for causal, window in ((0, 0), (1, 40)):
+        eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+        ok.prefill_paged(q, qindptr, pages, pindptr, pvalues, info, k_off, q_pos, eo, el, causal, 1, 1.0, 1e4,
+                         d ** -0.5, sliding_window_size=window)
+        go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+        gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+        K.batch_prefill_paged_kv(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(info), i32(k_off),
+                                 i32(q_pos), go, gl, causal, 1, 1.0, 1e4, d ** -0.5, sliding_window_size=window)
+        assert_close(host(go), eo, what=f"sliding paged out, page size {ps}, window {window}")
+        assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"sliding paged lse, page size {ps}, window {window}")
+    b = len(spec)
+    qd = rng.standard_normal((b, hq, d)).astype(F16)
+    qd_pos = (k_off + np.array([len(k) for k in k_log]) - 1).astype(np.int32)
+    for rotary in (0, 1):
+        eo, el = np.zeros((b, hq, d), F16), np.zeros((b, hq), np.float32)
+        ok.decode(qd, pages, pindptr, pvalues, info, k_off, qd_pos, eo, el, rotary, 1.0, 1e4, d ** -0.5)
+        go = torch.full((b, hq, d), 7.0, dtype=torch.float16, device=DEV)
+        gl = torch.full((b, hq), 7.0, dtype=torch.float32, device=DEV)
+        K.batch_decode_paged_kv(dev(qd), dev(pages), i32(pindptr), i32(pvalues), i32(info), i32(k_off), i32(qd_pos),
+                                go, gl, rotary, 1.0, 1e4, d ** -0.5)
+        assert_close(host(go), eo, what=f"sliding decode out, page size {ps}, rotary {rotary}")
+        assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"sliding decode lse, page size {ps}, rotary {rotary}")
+
+    # token trees behind a cached prefix
+    prefix = [10, 20, 30, 40, 0, 700, ps - 3]
+    trees = REFERENCE_TREES + [random_forest(rng, 50), random_forest(rng, 256), random_forest(rng, 31)]
+    new_lens = [7, 8, 10, 7, 50, 256, 16]
+    (pages, pindptr, pvalues, last, ks, vs, qindptr, q, tindptr, labels, masks) = tree_paged_case(
+        rng, prefix, trees, new_lens, hq, hkv, d, ps=ps, npages=need([a + len(t) for a, t in zip(prefix, trees)]))
+    n = len(q)
+    zb, zq = np.zeros(len(trees), np.int32), np.zeros(n, np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    ok.tree_attn_paged(q, qindptr, pages, pindptr, pvalues, last, zb, zq, eo, el, 0, 1.0, 1e4, d ** -0.5,
+                       tindptr, labels)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.tree_attn_paged_kv(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(zb), i32(zq),
+                         go, gl, 0, 1.0, 1e4, d ** -0.5, i32(tindptr), i32(labels))
+    assert_close(host(go), eo, what=f"tree paged out, page size {ps}")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"tree paged lse, page size {ps}")
+
+    # cached prefix + new chunk in one pass, against ragged + paged + merge of the oracle
+    prefix = [0, 1, 63, 64, 65, ps, ps + 1, 700, 16, 330]
+    chunk = [5, 130, 1, 64, 33, 300, 2, 40, 129, 64]
+    pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, prefix, need(prefix), hkv, ps, d)
+    n = sum(chunk)
+    ind = np.concatenate([[0], np.cumsum(chunk)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k = rng.standard_normal((n, hkv, d)).astype(F16)
+    v = rng.standard_normal((n, hkv, d)).astype(F16)
+    zq, zb = np.zeros(n, np.int32), np.zeros(len(prefix), np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    to, tl = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    ok.prefill_ragged(q, ind, k, v, ind, zq, zb, eo, el, 1, 0, 1.0, 1e4, d ** -0.5)
+    ok.prefill_paged(q, ind, pages, pindptr, pvalues, last, zb, zq, to, tl, 0, 0, 1.0, 1e4, d ** -0.5)
+    ok.merge_state_inplace(eo, el, to, tl)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_cached_and_new_kv(dev(q), i32(ind), dev(k), dev(v), dev(pages), i32(pindptr), i32(pvalues),
+                                      i32(last), go, gl, d ** -0.5)
+    assert_close(host(go), eo, what=f"one-pass chunked prefill out, page size {ps}")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"one-pass chunked prefill lse, page size {ps}")
 
 
 def test_prefill_more_than_64_sequences():

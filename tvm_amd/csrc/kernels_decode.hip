@@ -56,6 +56,7 @@ struct DecodeParams {
   int h_q;
   int h_kv;
   int chunk_pages;
+  int page_shift;  // pages hold 16 << page_shift tokens; the kernel walks them as runs of 16-token pages
   float scale_log2;  // sm_scale * log2(e)
 };
 
@@ -230,7 +231,8 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   const int g4 = lane >> 4;    // lane group 0..3
   const int cp = p.chunk_pages;
   half_t* Vt = Vt_all[wave];
-  const int64_t head_stride = static_cast<int64_t>(PS) * D;
+  const int psh = p.page_shift;  // a page of the table is 1 << psh of the 16-token pages the steps consume
+  const int64_t head_stride = static_cast<int64_t>(PS << psh) * D;
 
   // Persistent workgroups: item = (chunk slot, kv head, block of 16 heads of the group), strided over
   // the grid.  Neighbouring workgroups take the head blocks and kv heads of one slot, i.e. the same pages.
@@ -253,9 +255,10 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
     }
     continue;
   }
-  const int kv_len = (npages - 1) * PS + p.last_page_len[b];  // physical end of the cached tokens
-  const int page_lo = chunk * cp;
-  const int page_hi = min(page_lo + cp, npages);
+  const int kv_len = (npages - 1) * (PS << psh) + p.last_page_len[b];  // physical end of the cached tokens
+  // the chunk's 16-token pages (chunks are counted in pages of the table; the last one may be partly filled)
+  const int page_lo = (chunk * cp) << psh;
+  const int page_hi = min(min(chunk * cp + cp, npages) << psh, (kv_len + PS - 1) / PS);
   // physical token t is attended to iff t < sink or win_lo <= t < kv_len
   const int sink = EXT && p.sink_size != nullptr ? p.sink_size[b] : 0;
   const int win_lo = EXT && p.window_offset != nullptr ? p.window_offset[b] : 0;
@@ -310,8 +313,9 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int pg = min(pi + h, page_hi - 1);
-      const int page = __builtin_amdgcn_readfirstlane(p.page_values[pbeg + pg]);
-      const half_t* kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * head_stride;
+      const int page = __builtin_amdgcn_readfirstlane(p.page_values[pbeg + (pg >> psh)]);
+      const half_t* kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * head_stride +
+                            __builtin_amdgcn_readfirstlane(pg & ((1 << psh) - 1)) * (PS * D);
       const half_t* vbase = kbase + static_cast<int64_t>(p.h_kv) * head_stride;
       const int last_row = min(PS, kv_len - pg * PS) - 1;  // >= 0: every page of the table holds a token
 #pragma unroll
@@ -536,7 +540,8 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   KV_CHECK(batch_size >= 0 && nnz_pages >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_decode_paged_kv: bad shape";
   const bool ext = rotary_mode != 0 || sliding_window != 0;
-  KV_UNSUPPORTED(page_size != 16) << "batch_decode_paged_kv: page_size " << page_size << " is not built (16)";
+  KV_UNSUPPORTED(page_size < 16 || page_size > 128 || (page_size & (page_size - 1)) != 0)
+      << "batch_decode_paged_kv: page_size " << page_size << " is not built (16, 32, 64, 128)";
   KV_UNSUPPORTED(d != 64 && d != 128) << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 128)";
   if (batch_size == 0) return;
   KV_CHECK(q && pages && page_indptr && length_info && output && lse) << "batch_decode_paged_kv: NULL tensor";
@@ -560,7 +565,11 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   p.batch_size = batch_size;
   p.h_q = h_q;
   p.h_kv = h_kv;
-  p.chunk_pages = decode_pick_chunk_pages(nnz_pages, h_kv);
+  // the kernel walks a page of 16 << page_shift tokens as 1 << page_shift pages of 16: chunks are
+  // sized in those and counted in pages of the table
+  p.page_shift = 0;
+  while ((16 << p.page_shift) < page_size) ++p.page_shift;
+  p.chunk_pages = std::max(1, decode_pick_chunk_pages(nnz_pages << p.page_shift, h_kv) >> p.page_shift);
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
   const int64_t slots = nnz_pages / p.chunk_pages + batch_size;
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many chunks";

@@ -131,7 +131,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
         lk1 = p.kv_indptr[lane + 1];
       }
       my_tiles = ((lq1 - lq0) * group + BM - 1) / BM;
-      my_key = (lp1 - lp0) * PS + (lk1 - lk0);
+      my_key = (lp1 - lp0) * (PS << p.page_shift) + (lk1 - lk0);
     }
     // Row tiles of the sequences ranked before this lane's.  (key, index) is one sortable 32-bit
     // number (keys beyond 2^24 tokens rank equal), compared without branches, four sequences per
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   if (PAGED || BOTH) {
     pbeg = seq_p0;
     const int npages = seq_p1 - pbeg;
-    phys_len = npages > 0 ? (npages - 1) * PS + seq_last : 0;
+    phys_len = npages > 0 ? (npages - 1) * (PS << p.page_shift) + seq_last : 0;
     if (EXT && p.sink_size != nullptr && npages > 0) {
       sink = p.sink_size[b];
       win_lo = p.window_offset[b];
@@ -296,10 +296,13 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   // Page ids of this wave's RPW rows for 64 consecutive tiles, one tile per lane, fetched once per
   // 64 tiles: the wait for this load also waits for every tile copy in flight, so it must be rare.
   int page_ids = 0;
+  const int psh = p.page_shift;
   auto load_page_ids = [&](int first_tile) {
     if (PAGED || BOTH) {
+      // a page of PS << page_shift tokens is walked as 1 << page_shift runs of PS tokens: the lane
+      // keeps (page id, run inside the page), the run in the low 3 bits
       const int pslot = min((first_tile + lane) * BN + wave_u * RPW, last_tok) / PS;
-      page_ids = p.page_values[pbeg + pslot];
+      page_ids = (p.page_values[pbeg + (pslot >> psh)] << 3) | (pslot & ((1 << psh) - 1));
     }
   };
   // Global addresses are a wave-uniform base (scalar registers) plus a 32-bit byte offset per lane.
@@ -325,8 +328,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     const half_t* vbase = v_seq;
     if (from_pages) {
       const int page = __builtin_amdgcn_readlane(page_ids, tile & 63);
-      kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * (PS * DQK);
-      vbase = kbase + static_cast<int64_t>(p.h_kv) * (PS * DQK);
+      kbase = p.pages + (((static_cast<int64_t>(page >> 3) * 2 * p.h_kv + kvh) << psh) + (page & 7)) * (PS * DQK);
+      vbase = kbase + (static_cast<int64_t>(p.h_kv) << psh) * (PS * DQK);
     }
 #pragma unroll
     for (int blk = 0; blk < KBLK; ++blk) {
@@ -370,8 +373,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
     uint32_t row_bytes;
     if (from_pages) {
       const int page = __builtin_amdgcn_readlane(page_ids, tile & 63);
-      kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * (PS * 128);
-      vbase = kbase + static_cast<int64_t>(p.h_kv) * (PS * 128);
+      kbase = p.pages + (((static_cast<int64_t>(page >> 3) * 2 * p.h_kv + kvh) << psh) + (page & 7)) * (PS * 128);
+      vbase = kbase + (static_cast<int64_t>(p.h_kv) << psh) * (PS * 128);
       row_bytes = 256;
     } else {
       const int64_t first_row = static_cast<int64_t>(tile) * BN - prefix_pad + wave_u * RPW;
@@ -727,6 +730,14 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   }
 }
 
+// Page sizes the paged kernels take: 16 << shift tokens, walked as 1 << shift runs of 16.  -1: not built.
+static int paged_page_shift(int32_t page_size) {
+  if (page_size < 16 || page_size > 128 || (page_size & (page_size - 1)) != 0) return -1;
+  int shift = 0;
+  while ((16 << shift) < page_size) ++shift;
+  return shift;
+}
+
 template <int DQK, int DV, int SRC, int PS, bool EXT>
 static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const PrefillRopeDivisors& div,
                                hipStream_t stream) {
@@ -850,7 +861,9 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_paged_kv: bad shape";
-  KV_UNSUPPORTED(page_size != 16) << "batch_prefill_paged_kv: page_size " << page_size << " is not built (16)";
+  const int page_shift = paged_page_shift(page_size);
+  KV_UNSUPPORTED(page_shift < 0) << "batch_prefill_paged_kv: page_size " << page_size << " is not built (16, 32, 64, 128)";
+  KV_CHECK(num_pages < (int64_t{1} << 28)) << "batch_prefill_paged_kv: page ids must stay below 2^28";
   if (batch_size == 0 || total_q == 0) return TVMKV_OK;
   KV_CHECK(q && q_indptr && pages && page_indptr && length_info && output && lse)
       << "batch_prefill_paged_kv: NULL tensor";
@@ -858,6 +871,7 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
   KV_CHECK(rotary_mode == 0 || (q_rope_position && k_rope_pos_offset))
       << "batch_prefill_paged_kv: inline RoPE needs the position arrays";
   PrefillParams p{};
+  p.page_shift = page_shift;
   p.q = static_cast<const half_t*>(q);
   p.q_indptr = q_indptr;
   p.pages = static_cast<const half_t*>(pages);
@@ -932,14 +946,16 @@ static int cached_and_new(const void* q, int64_t q_token_stride, const int32_t* 
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_cached_and_new_kv: bad shape";
-  KV_UNSUPPORTED(page_size != 16) << "batch_prefill_cached_and_new_kv: page_size " << page_size
-                                  << " is not built (16)";
+  const int page_shift = paged_page_shift(page_size);
+  KV_UNSUPPORTED(page_shift < 0) << "batch_prefill_cached_and_new_kv: page_size " << page_size << " is not built (16, 32, 64, 128)";
+  KV_CHECK(num_pages < (int64_t{1} << 28)) << "batch_prefill_cached_and_new_kv: page ids must stay below 2^28";
   if (batch_size == 0 || total_q == 0) return TVMKV_OK;
   KV_CHECK(q && q_indptr && k && v && pages && page_indptr && last_page_len && output && lse)
       << "batch_prefill_cached_and_new_kv: NULL tensor";
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_prefill_cached_and_new_kv: NULL page table";
   KV_CHECK(apply_rope == 0 || q_rope_position) << "batch_prefill_cached_and_new_kv: RoPE needs the position array";
   PrefillParams p{};
+  p.page_shift = page_shift;
   p.q = static_cast<const half_t*>(q);
   p.q_token_stride = q_token_stride;
   p.q_inline_rope = apply_rope != 0;
@@ -1050,7 +1066,9 @@ int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void*
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "tree_attn_paged_kv: bad shape";
-  KV_UNSUPPORTED(page_size != 16) << "tree_attn_paged_kv: page_size " << page_size << " is not built (16)";
+  const int page_shift = paged_page_shift(page_size);
+  KV_UNSUPPORTED(page_shift < 0) << "tree_attn_paged_kv: page_size " << page_size << " is not built (16, 32, 64, 128)";
+  KV_CHECK(num_pages < (int64_t{1} << 28)) << "tree_attn_paged_kv: page ids must stay below 2^28";
   // the reference kernel asserts the same (tree_attn.py:700-702)
   KV_UNSUPPORTED(rotary_mode != 0) << "tree_attn_paged_kv: inline rotary mode is not supported in tree attention";
   if (batch_size == 0 || total_q == 0) return TVMKV_OK;
@@ -1058,6 +1076,7 @@ int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void*
       << "tree_attn_paged_kv: NULL tensor";
   KV_CHECK(nnz_pages == 0 || page_values) << "tree_attn_paged_kv: NULL page table";
   PrefillParams p{};
+  p.page_shift = page_shift;
   p.q = static_cast<const half_t*>(q);
   p.q_indptr = q_indptr;
   p.pages = static_cast<const half_t*>(pages);

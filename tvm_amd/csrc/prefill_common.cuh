@@ -50,6 +50,7 @@ struct PrefillParams {
   // rotates them at q_rope_position[token] itself (with rope_scale and the divisors of the launch)
   int64_t q_token_stride;
   int q_inline_rope;
+  int page_shift;   // pages hold 16 << page_shift tokens; the kernel walks them as runs of 16-token pages
   int clock_probe;  // != 0: add this workgroup's shader cycles and 100 MHz ticks to the probe counters
 };
 
