@@ -147,7 +147,7 @@ int tvmkv_kv_cache_transpose_append_mla(void* pages, const void* kv_data, const 
  * q (total_q, h_q, d_qk), k (total_kv, h_kv, d_qk), v (total_kv, h_kv, d_v),
  * out (total_q, h_q, d_v) fp16, lse (total_q, h_q) fp32 base-2.  rotary_mode 0: q and k are used
  * as they are; 1 (inline RoPE): q is rotated at q_rope_position[token], key t of sequence b at
- * k_rope_pos_offset[b] + t (built for head dims 64 and 128). */
+ * k_rope_pos_offset[b] + t (built for head dims 64, 128 and 256). */
 int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const void* k, const void* v,
                                   const int32_t* kv_indptr, const int32_t* q_rope_position,
                                   const int32_t* k_rope_pos_offset, void* output, float* lse,
@@ -234,7 +234,7 @@ int tvmkv_batch_prefill_cached_and_new_kv_fused_q(const void* qkv, const int32_t
  *  lse, rotary_mode, rope_scale, rope_theta, sm_scale).
  * q/out (B, h_q, d) fp16, lse (B, h_q) fp32.  Split-KV across workgroups with a merge pass;
  * the partition count is derived from B and nnz_pages only (no host read of the page table).
- * Head dims 64 and 128, any GQA group (groups above 16 are walked in blocks of 16 heads), with the
+ * Head dims 64, 128 and 256, any GQA group (groups above 16 are walked in blocks of 16 heads), with the
  * (3, batch) length_info and rotary_mode = 1 built in for all of them. */
 int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t* page_indptr,
                                 const int32_t* page_values, const int32_t* length_info,

@@ -17,7 +17,7 @@ from tvm_amd import get_global_func as gf
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("d,rope_mode", [(128, S.ROPE_NORMAL), (64, S.ROPE_NORMAL), (128, S.ROPE_NONE)])
+@pytest.mark.parametrize("d,rope_mode", [(128, S.ROPE_NORMAL), (64, S.ROPE_NORMAL), (128, S.ROPE_NONE), (256, S.ROPE_NORMAL)])
 @pytest.mark.parametrize("runner", [S.run_prefill_and_decode, S.run_remove_sequence, S.run_fork_sequence,
                                     S.run_unlimited_depth, S.run_popn])
 def test_reference_scenarios_on_the_gpu(runner, d, rope_mode):

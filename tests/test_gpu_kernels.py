@@ -167,7 +167,8 @@ def _decode_both(rng, kv_lens, hq, hkv, d, npages, scale=1.0, page_size=16):
     return host(go), host(gl), eo, el
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (64, 8, 128), (8, 8, 128), (8, 4, 64), (16, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (64, 8, 128), (8, 8, 128), (8, 4, 64), (16, 2, 64), (8, 2, 256),
+                                      (16, 16, 256)])
 def test_decode_ragged_lengths_against_oracle(hq, hkv, d):
     rng = np.random.default_rng(5)
     # empty, single token, page boundaries, several chunks, spare slots
@@ -291,7 +292,7 @@ def test_decode_large_gqa_groups_plain_cache():
 
 
 @pytest.mark.parametrize("rotary", [0, 1])
-@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (16, 16, 64), (32, 1, 128)])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (16, 16, 64), (32, 1, 128), (8, 2, 256)])
 def test_decode_sliding_cache_and_inline_rope_other_shapes(hq, hkv, d, rotary):
     """Head dim 64 and GQA groups above 16 through the sliding-window / inline-RoPE form of the decode kernel."""
     from tests.test_oracle_kernels import SLIDING_SPEC, sliding_case
@@ -328,7 +329,8 @@ def _ragged_both(rng, lens, hq, hkv, dqk, dv, causal, scale=1.0):
     return host(go), host(gl), eo, el
 
 
-@pytest.mark.parametrize("hq,hkv,dqk,dv", [(32, 8, 128, 128), (8, 8, 128, 128), (8, 2, 64, 64), (16, 16, 192, 128)])
+@pytest.mark.parametrize("hq,hkv,dqk,dv", [(32, 8, 128, 128), (8, 8, 128, 128), (8, 2, 64, 64), (16, 16, 192, 128),
+                                           (8, 2, 256, 256)])
 @pytest.mark.parametrize("causal", [1, 0])
 def test_ragged_prefill_against_oracle(hq, hkv, dqk, dv, causal):
     rng = np.random.default_rng(9)
@@ -387,7 +389,7 @@ def _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages, page_size=16):
     return host(go), host(gl), eo, el
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
 @pytest.mark.parametrize("causal", [0, 1])
 def test_paged_prefill_against_oracle(hq, hkv, d, causal):
     rng = np.random.default_rng(11)
@@ -525,7 +527,7 @@ def test_layer_sliding_window_mask_known_answer_on_the_gpu():
     assert_close(host(go)[:, 0, 0], np.array([4, 5], F16), atol=1e-3, rtol=1e-3, what="sliding window known answer")
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
 @pytest.mark.parametrize("rotary", [0, 1])
 @pytest.mark.parametrize("causal,window", [(0, 1024), (1, 0), (1, 5), (1, 40)])
 def test_paged_prefill_sliding_cache_layer_window_and_inline_rope(hq, hkv, d, rotary, causal, window):
@@ -553,7 +555,7 @@ def test_paged_prefill_sliding_cache_layer_window_and_inline_rope(hq, hkv, d, ro
     assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="sliding paged lse")
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
 @pytest.mark.parametrize("causal", [1, 0])
 def test_prefill_inline_rope_plain_cache(hq, hkv, d, causal):
     rng = np.random.default_rng(25)
@@ -587,7 +589,7 @@ def test_prefill_inline_rope_plain_cache(hq, hkv, d, causal):
 
 
 # ------------------------------------------------------------------------------ token trees
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
 @pytest.mark.parametrize("rotary", [0, 1])
 def test_tree_attn_ragged_against_oracle(hq, hkv, d, rotary):
     from tests.util import REFERENCE_TREES, random_forest, tree_order
@@ -618,7 +620,7 @@ def test_tree_attn_ragged_against_oracle(hq, hkv, d, rotary):
     assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="tree ragged lse")
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
 def test_tree_attn_paged_against_oracle(hq, hkv, d):
     from tests.test_oracle_kernels import tree_paged_case
     from tests.util import REFERENCE_TREES, random_forest
@@ -688,7 +690,7 @@ def test_chunked_prefill_composition_matches_oracle():
     assert_close(host(gl3), el, atol=2e-3, rtol=1e-4, what="chunked prefill lse, one pass")
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 8, 128)])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 8, 128), (8, 2, 256)])
 def test_prefill_cached_and_new_in_one_pass(hq, hkv, d):
     """Prefix lengths around the tile size (the padded end of the cached part), no prefix, chunks of one
     token and of several row tiles; against ragged + paged + merge of the oracle."""
@@ -719,7 +721,7 @@ def test_prefill_cached_and_new_in_one_pass(hq, hkv, d):
 
 
 @pytest.mark.parametrize("apply_rope", [1, 0])
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
 def test_prefill_one_pass_with_queries_from_the_fused_qkv(hq, hkv, d, apply_rope):
     """The step of the cache object for a chunked prefill: k rotated and appended without writing q
     (fused_rope_append with q = None), then the one-pass kernel that reads q from qkv and rotates it

@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeParams p, int t
 }
 
 // ------------------------------------------------------------------------------------------
-// The decode kernel, for head dims 64 and 128 and any GQA group.
+// The decode kernel, for head dims 64, 128 and 256 and any GQA group.
 //
 // A vector-ALU formulation spends ~90 instructions per query head and 8 KiB page, which for groups of
 // 4-8 query heads is about as much issue time as the page's HBM time.  Here the two contractions
@@ -194,12 +194,12 @@ constexpr int DM_PS = 16;
 // (head dim 64: two rows per line, the rows of equal parity share a half).
 template <int D>
 __device__ __forceinline__ int dm_swizzle(int row) {
-  return D == 128 ? (row & 7) << 1 : ((row >> 1) & 3) << 1;
+  return D >= 128 ? (row & 7) << 1 : ((row >> 1) & 3) << 1;
 }
 
 // theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
 struct DecodeRopeDivisors {
-  float v[64];
+  float v[128];
 };
 
 // EXT = false: plain cache, q and k already rotated (or no RoPE).  EXT = true adds the sliding-window
@@ -209,7 +209,7 @@ struct DecodeRopeDivisors {
 // _decode_kernels.py:141-156).  Attention does not depend on the order of the keys, so the pages are
 // still walked in physical order; evicted tokens are masked and logical indices only feed RoPE.
 template <bool EXT, int D>
-__global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodeParams p, int group, int num_items,
+__global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_kernel(DecodeParams p, int group, int num_items,
                                                              DecodeRopeDivisors div) {
   constexpr int PS = DM_PS;
   constexpr int KS = D / 32;                // k-steps of the score product
@@ -217,7 +217,7 @@ __global__ __launch_bounds__(256, EXT ? 2 : 3) void decode_mfma_kernel(DecodePar
   constexpr int PPR = D / 8;                // 16-byte pieces per row
   constexpr int RPI = 64 / PPR;             // rows one copy instruction covers
   constexpr int DM_VTILE = 2 * PS * D;      // halfs of a wave's V tile: two pages, row-major
-  static_assert(D == 64 || D == 128, "head dim");
+  static_assert(D == 64 || D == 128 || D == 256, "head dim");
   static_assert(DM_VTILE * sizeof(half_t) >= 16 * D * sizeof(float), "the merge buffer aliases the V tile");
   __shared__ __attribute__((aligned(16))) half_t Vt_all[4][DM_VTILE];
   __shared__ float sm_m[4][16];
@@ -542,7 +542,7 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   const bool ext = rotary_mode != 0 || sliding_window != 0;
   KV_UNSUPPORTED(page_size < 16 || page_size > 128 || (page_size & (page_size - 1)) != 0)
       << "batch_decode_paged_kv: page_size " << page_size << " is not built (16, 32, 64, 128)";
-  KV_UNSUPPORTED(d != 64 && d != 128) << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 128)";
+  KV_UNSUPPORTED(d != 64 && d != 128 && d != 256) << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 128, 256)";
   if (batch_size == 0) return;
   KV_CHECK(q && pages && page_indptr && length_info && output && lse) << "batch_decode_paged_kv: NULL tensor";
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_decode_paged_kv: NULL page table";
@@ -606,6 +606,8 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   };
   if (d == 128) {
     if (ext) launch(decode_mfma_kernel<true, 128>); else launch(decode_mfma_kernel<false, 128>);
+  } else if (d == 256) {
+    if (ext) launch(decode_mfma_kernel<true, 256>); else launch(decode_mfma_kernel<false, 256>);
   } else {
     if (ext) launch(decode_mfma_kernel<true, 64>); else launch(decode_mfma_kernel<false, 64>);
   }
@@ -613,6 +615,8 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
     KV_LAUNCH_CHECK();
     if (d == 128) {
       hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
+    } else if (d == 256) {
+      hipLaunchKernelGGL(decode_merge_kernel<256>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
     } else {
       hipLaunchKernelGGL(decode_merge_kernel<64>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
     }

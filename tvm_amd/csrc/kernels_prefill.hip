@@ -69,7 +69,7 @@ constexpr size_t prefill_lds_bytes(int dqk, int dv) {
 // causal mask -- a chunked-prefill step in one pass, on one key axis whose paged part is padded to
 // a whole number of tiles (the padding is masked like the end of a sequence).
 template <int DQK, int DV, int SRC, int PS, bool EXT>
-__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
+__global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : 2) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
   constexpr bool PAGED = SRC == kPaged, BOTH = SRC == kBoth;
   static_assert(!(BOTH && EXT), "the combined pass exists for the plain cache only");
   static_assert(DQK % 64 == 0 && DV % 64 == 0, "feature dims must be multiples of 64");
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void prefill_kernel(Prefi
   const int kv_len = phys_len - win_lo + sink;
   // number of logical keys -> physical end of the tokens that hold them
   auto to_phys = [&](int n) { return (!EXT || n <= sink) ? n : n - sink + win_lo; };
-  __shared__ float div_lds[64];
+  __shared__ float div_lds[DQK > 128 ? 128 : 64];
   const bool q_rope = (EXT && p.rotary) || (BOTH && p.q_inline_rope != 0);  // uniform over the launch
   if (q_rope) {
     if (tid < DQK / 2) div_lds[tid] = div.v[tid];
@@ -764,12 +764,12 @@ static void launch_prefill(const PrefillParams& p, int64_t total_q, bool ext, do
   if (!ext) {
     if (p.q_inline_rope) {
       const float theta = static_cast<float>(rope_theta);
-      for (int i = 0; i < DQK / 2 && i < 64; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DQK));
+      for (int i = 0; i < DQK / 2 && i < 128; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DQK));
     }
     launch_prefill_ext<DQK, DV, SRC, PS, false>(p, total_q, div, stream);
     return;
   }
-  if constexpr (DQK == DV && DQK <= 128 && SRC != kBoth) {
+  if constexpr (DQK == DV && SRC != kBoth) {
     const float theta = static_cast<float>(rope_theta);
     for (int i = 0; i < DQK / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DQK));
     launch_prefill_ext<DQK, DV, SRC, PS, true>(p, total_q, div, stream);
@@ -841,11 +841,13 @@ int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const 
     launch_prefill<128, 128, kRagged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d_qk == 64 && d_v == 64) {
     launch_prefill<64, 64, kRagged, 16>(p, total_q, ext, rope_theta, s);
+  } else if (d_qk == 256 && d_v == 256) {
+    launch_prefill<256, 256, kRagged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d_qk == 192 && d_v == 128) {
     launch_prefill<192, 128, kRagged, 16>(p, total_q, ext, rope_theta, s);
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_ragged_kv: (d_qk, d_v) = (" << d_qk << ", " << d_v
-                         << ") is not built ((64,64), (128,128), (192,128))";
+                         << ") is not built ((64,64), (128,128), (192,128), (256,256))";
   }
   KV_LAUNCH_CHECK();
   KV_API_END();
@@ -902,8 +904,10 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
     launch_prefill<128, 128, kPaged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d == 64) {
     launch_prefill<64, 64, kPaged, 16>(p, total_q, ext, rope_theta, s);
+  } else if (d == 256) {
+    launch_prefill<256, 256, kPaged, 16>(p, total_q, ext, rope_theta, s);
   } else {
-    KV_UNSUPPORTED(true) << "batch_prefill_paged_kv: head_dim " << d << " is not built (64, 128)";
+    KV_UNSUPPORTED(true) << "batch_prefill_paged_kv: head_dim " << d << " is not built (64, 128, 256)";
   }
   KV_LAUNCH_CHECK();
   KV_API_END();
@@ -982,8 +986,10 @@ static int cached_and_new(const void* q, int64_t q_token_stride, const int32_t* 
     launch_prefill<128, 128, kBoth, 16>(p, total_q, false, rope_theta, s);
   } else if (d == 64) {
     launch_prefill<64, 64, kBoth, 16>(p, total_q, false, rope_theta, s);
+  } else if (d == 256) {
+    launch_prefill<256, 256, kBoth, 16>(p, total_q, false, rope_theta, s);
   } else {
-    KV_UNSUPPORTED(true) << "batch_prefill_cached_and_new_kv: head_dim " << d << " is not built (64, 128)";
+    KV_UNSUPPORTED(true) << "batch_prefill_cached_and_new_kv: head_dim " << d << " is not built (64, 128, 256)";
   }
   KV_LAUNCH_CHECK();
   KV_API_END();
@@ -1049,8 +1055,10 @@ int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k,
     launch_prefill<128, 128, kRagged, 16>(p, total_q, true, rope_theta, s);
   } else if (d == 64) {
     launch_prefill<64, 64, kRagged, 16>(p, total_q, true, rope_theta, s);
+  } else if (d == 256) {
+    launch_prefill<256, 256, kRagged, 16>(p, total_q, true, rope_theta, s);
   } else {
-    KV_UNSUPPORTED(true) << "batch_tree_attn: head_dim " << d << " is not built (64, 128)";
+    KV_UNSUPPORTED(true) << "batch_tree_attn: head_dim " << d << " is not built (64, 128, 256)";
   }
   KV_LAUNCH_CHECK();
   KV_API_END();
@@ -1105,8 +1113,10 @@ int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void*
     launch_prefill<128, 128, kPaged, 16>(p, total_q, true, rope_theta, s);
   } else if (d == 64) {
     launch_prefill<64, 64, kPaged, 16>(p, total_q, true, rope_theta, s);
+  } else if (d == 256) {
+    launch_prefill<256, 256, kPaged, 16>(p, total_q, true, rope_theta, s);
   } else {
-    KV_UNSUPPORTED(true) << "tree_attn_paged_kv: head_dim " << d << " is not built (64, 128)";
+    KV_UNSUPPORTED(true) << "tree_attn_paged_kv: head_dim " << d << " is not built (64, 128, 256)";
   }
   KV_LAUNCH_CHECK();
   KV_API_END();

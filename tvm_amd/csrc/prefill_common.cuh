@@ -56,7 +56,7 @@ struct PrefillParams {
 
 // theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
 struct PrefillRopeDivisors {
-  float v[64];
+  float v[128];
 };
 
 __device__ __forceinline__ int tile_slot_begin(const int32_t* q_indptr, int b, int group) {
