@@ -423,6 +423,10 @@ static void prefill_paged_impl(const f16* q, const int32_t* q_indptr, const f16*
       int begin = page_indptr[b_idx], end = page_indptr[b_idx + 1];
       int kv_len = kv_chunk_len(end - begin, page_size, b_idx, length_info, batch_size, sliding_window);
       int qo_len = q_indptr[b_idx + 1] - q_indptr[b_idx];
+      /* new_m lives across the query rows of a sequence as in the reference (_prefill_kernels.py:192-201
+       * never resets it): a row that sees no key at all -- rows from sliding_window_size - 1 on under the
+       * per-layer window mask -- is scaled by the previous row's maximum and ends as 0 / 0.  The tests
+       * leave such rows out of the comparison and pin the library's answer for them (out 0, lse -5e4). */
       float new_m = -5e4f;
       for (int q_idx = 0; q_idx < qo_len; ++q_idx) {
         float m_val = -5e4f, d_val = 1.0f;

@@ -8,6 +8,10 @@ def assert_close(actual, expected, atol=ATOL, rtol=RTOL, what=""):
     actual = np.asarray(actual, dtype=np.float64)
     expected = np.asarray(expected, dtype=np.float64)
     assert actual.shape == expected.shape, f"{what}: shape {actual.shape} vs {expected.shape}"
+    for name, a in (("actual", actual), ("expected", expected)):  # NaN would compare as "not greater than the tolerance"
+        if not np.isfinite(a).all():
+            idx = tuple(np.argwhere(~np.isfinite(a))[0])
+            raise AssertionError(f"{what}: {name} holds {a[idx]!r} at {idx} ({(~np.isfinite(a)).sum()} non-finite elements)")
     err = np.abs(actual - expected)
     tol = atol + rtol * np.abs(expected)
     bad = err > tol
@@ -16,6 +20,27 @@ def assert_close(actual, expected, atol=ATOL, rtol=RTOL, what=""):
         raise AssertionError(
             f"{what}: {bad.sum()} / {bad.size} elements out of tolerance; worst at {idx}: "
             f"actual {actual[idx]!r} expected {expected[idx]!r}")
+
+
+def rows_without_keys(q_lens, causal, window):
+    """Boolean mask over the query rows of a paged prefill call: under the per-layer window mask row r of
+    a sequence sees the last max(window - r - 1, 0) keys (python/tvm/relax/frontend/nn/llm/
+    _kernel_common.py:138-144), so rows from window - 1 on see none.  For such a row the reference's CPU
+    kernel divides 0 by 0 (its running maximum is the previous row's, _prefill_kernels.py:192-201, and
+    the oracle restates that) and its GPU kernel averages V over the masked keys; the library returns
+    what a sequence without keys returns, out = 0 and lse = -5e4, and the tests pin that."""
+    if not (causal and window > 0):
+        return np.zeros(sum(q_lens), bool)
+    return np.concatenate([np.arange(n) >= window - 1 for n in q_lens])
+
+
+def assert_close_where_keys(actual_out, actual_lse, expected_out, expected_lse, no_keys, lse_atol, what):
+    """assert_close on the rows that see keys; out = 0 and lse = -5e4 on the others."""
+    assert not np.asarray(actual_out)[no_keys].any(), f"{what}: rows without keys must be 0"
+    assert np.all(np.asarray(actual_lse)[no_keys] == np.float32(-5e4)), f"{what}: lse of rows without keys must be -5e4"
+    assert_close(np.asarray(actual_out)[~no_keys], np.asarray(expected_out)[~no_keys], what=f"{what} out")
+    assert_close(np.asarray(actual_lse)[~no_keys], np.asarray(expected_lse)[~no_keys], atol=lse_atol, rtol=1e-4,
+                 what=f"{what} lse")
 
 
 def build_paged_kv(rng, kv_lens, num_pages, hkv, page_size, d, permute=True, scale=1.0,
