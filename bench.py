@@ -473,6 +473,30 @@ def extras(torch, K, dev):
 
     out["token_tree_verify"] = tree_verify(6)            # 63 nodes: 252 rows per kv head, two row tiles, compute-bound
     out["token_tree_verify_15_nodes"] = tree_verify(4)   # 60 rows per kv head: one row tile, the K/V stream decides
+
+    # ---- a short chunk against a long cached sequence: few row tiles, split over the keys ----------
+    plen, clen = 100000, 64
+    npg = (plen + ps - 1) // ps
+    qs = torch.randn((clen, hq, d), device=dev).to(torch.float16)
+    ks_ = torch.randn((clen, hkv, d), device=dev).to(torch.float16)
+    vs_ = torch.randn((clen, hkv, d), device=dev).to(torch.float16)
+    os_ = torch.empty_like(qs)
+    ls_ = torch.empty((clen, hq), dtype=torch.float32, device=dev)
+    sargs = (qs, i32([0, clen]), ks_, vs_, pages, i32([0, npg]), i32(perm[:npg]), i32([(plen - 1) % ps + 1]), os_, ls_,
+             d ** -0.5)
+    ms_split = time_region(torch, lambda i: K.batch_prefill_cached_and_new_kv(*sargs), 20, SETTLE_S)
+    prev = tvm_amd.set_option("prefill_kv_splits", 1)
+    try:
+        ms_whole = time_region(torch, lambda i: K.batch_prefill_cached_and_new_kv(*sargs), 20, SETTLE_S)
+    finally:
+        tvm_amd.set_option("prefill_kv_splits", prev)
+    nbytes = float(plen) * 2 * hkv * d * 2
+    out["short_chunk_long_context"] = {
+        "workload": f"one sequence, a {clen}-token chunk on {plen} cached tokens, Hq32/Hkv8/D128, one-pass chunked prefill: "
+                    "2 row tiles per kv head, their keys split over the workgroups of the launch and merged",
+        "ms": round(ms_split, 4), "ms_one_workgroup_per_row_tile": round(ms_whole, 4),
+        "speedup": round(ms_whole / ms_split, 2), "GBps": round(nbytes / ms_split / 1e6, 1),
+        "frac_of_hbm_peak": round(nbytes / ms_split / 1e6 / HBM_PEAK_GBPS, 4)}
     del pages
     torch.cuda.empty_cache()
 

@@ -350,7 +350,11 @@ int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr,
  *   decode_separate_merge  != 0: merge the decode chunks in a second launch instead of inside the kernel
  *   decode_wgs_per_cu      > 0: cap the decode grid at this many workgroups per compute unit
  *   mla_chunk_tokens       lower bound of the tokens per split-KV chunk of MLA decode; 0 = 128
- *   mla_separate_merge     accepted and ignored: the MLA decode chunks are always merged in a second launch */
+ *   mla_separate_merge     accepted and ignored: the MLA decode chunks are always merged in a second launch
+ *   prefill_kv_splits      > 0: the paged prefill, one-pass chunked prefill and paged tree-attention launches
+ *                          split the keys of every row tile over this many workgroups (at most 64) and merge
+ *                          the states in a second launch; 0 = derived from the shapes (launches with few row
+ *                          tiles and long cached sequences are split, all others are not) */
 int tvmkv_set_option(const char* name, int64_t value);
 int tvmkv_get_option(const char* name, int64_t* value);
 

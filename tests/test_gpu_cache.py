@@ -111,6 +111,18 @@ def test_identical_inputs_through_oracle_and_gpu_caches(page_size):
     m.step([(i, 1) for i in (0, 1, 2, 4, 5, 6)])
 
 
+def test_short_chunk_against_a_long_cached_sequence():
+    """A chunk of a few tokens against thousands of cached ones is one or two row tiles per kv head: the
+    launch splits their keys over several workgroups and merges the states.  Through the cache's one-pass
+    chunked prefill and its mixed prefill / decode batches, against the oracle cache."""
+    m = Mirror([4, 8192, 2048, 16, 0], 2, 8, 2, 64)
+    m.step([(0, 2000), (1, 40)])
+    m.step([(0, 1500)])
+    m.step([(0, 20), (1, 3)])       # 3520 cached tokens, 20 new ones
+    m.step([(0, 1), (1, 2)])        # not a pure decode batch: the prefill kernels again
+    m.step([((2, 0, 3000), 7)])     # a fork deep inside the long sequence
+
+
 @pytest.mark.parametrize("rope", [
     dict(rope_theta=5e5, rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
                                        "original_max_position_embeddings": 8192}),

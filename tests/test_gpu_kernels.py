@@ -496,6 +496,92 @@ def test_paged_kernels_with_other_page_sizes(page_size, hq, hkv, d):
     assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"one-pass chunked prefill lse, page size {ps}")
 
 
+@pytest.mark.parametrize("hq,hkv,d,splits", [(32, 8, 128, 0), (32, 8, 128, 3), (8, 2, 64, 5), (8, 2, 64, 64), (8, 2, 256, 2)])
+def test_prefill_split_over_the_keys(hq, hkv, d, splits):
+    """Launches with few row tiles split every row tile's keys over several workgroups and merge the
+    states: the derived split (few queries against long cached sequences) and forced ones (more shares
+    than some sequences have tiles, so that shares are empty; sequences without cached tokens; rows that
+    see no key), through the paged kernel with every mask, the tree-masked kernel and the one-pass
+    chunked prefill."""
+    import tvm_amd
+    from tests.test_oracle_kernels import sliding_case, tree_paged_case
+    from tests.util import REFERENCE_TREES, random_forest
+    rng = np.random.default_rng(70 + splits)
+    prev = tvm_amd.set_option("prefill_kv_splits", splits)
+    try:
+        if splits == 0:  # long enough for the derived split: 8 shares
+            go, gl, eo, el = _paged_both(rng, [6000, 3000], [5, 3], hq, hkv, d, 1, 600)
+            assert_close(go, eo, what="paged out, derived split")
+            assert_close(gl, el, atol=2e-3, rtol=1e-4, what="paged lse, derived split")
+        kv_lens = [1500, 16, 0, 75, 700, 64, 1, 65, 400, 129]
+        q_lens = [7, 16, 3, 30, 64, 1, 1, 20, 5, 40]
+        for causal in (0, 1):
+            lens = [max(k, q) for k, q in zip(kv_lens, q_lens)] if causal else kv_lens
+            go, gl, eo, el = _paged_both(rng, lens, q_lens, hq, hkv, d, causal, 8 + sum((n + 15) // 16 for n in lens))
+            assert_close(go, eo, what=f"paged out, {splits} splits, causal {causal}")
+            assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"paged lse, {splits} splits, causal {causal}")
+
+        spec = [(100, 4, 20), (1300, 0, 0), (800, 16, 48), (33, 2, 2), (64, 16, 32), (500, 0, 17)]
+        sq_lens = [7, 64, 33, 3, 1, 50]
+        pages, pindptr, pvalues, info, k_log, _ = sliding_case(rng, spec, hkv, d, npages=8 + sum((x[0] + 15) // 16 for x in spec))
+        n = sum(sq_lens)
+        qindptr = np.concatenate([[0], np.cumsum(sq_lens)]).astype(np.int32)
+        q = rng.standard_normal((n, hq, d)).astype(F16)
+        k_off = rng.integers(0, 200, size=len(spec)).astype(np.int32)
+        q_pos = np.concatenate([k_off[i] + len(k_log[i]) - sq_lens[i] + np.arange(sq_lens[i]) for i in range(len(spec))])
+        q_pos = q_pos.astype(np.int32)
+        for causal, window, rotary in ((0, 0, 1), (1, 40, 0), (1, 0, 1)):
+            eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+            ok.prefill_paged(q, qindptr, pages, pindptr, pvalues, info, k_off, q_pos, eo, el, causal, rotary, 1.0, 1e4,
+                             d ** -0.5, sliding_window_size=window)
+            go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+            gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+            K.batch_prefill_paged_kv(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(info), i32(k_off),
+                                     i32(q_pos), go, gl, causal, rotary, 1.0, 1e4, d ** -0.5, sliding_window_size=window)
+            assert_close_where_keys(host(go), host(gl), eo, el, rows_without_keys(sq_lens, causal, window), 2e-3,
+                                    f"sliding paged, {splits} splits, window {window}")
+
+        prefix = [10, 1200, 30, 640, 0, 300]
+        trees = REFERENCE_TREES + [random_forest(rng, 50), random_forest(rng, 15)]
+        new_lens = [7, 8, 10, 7, 50, 15]
+        (pages, pindptr, pvalues, last, ks, vs, qindptr, q, tindptr, labels, masks) = tree_paged_case(
+            rng, prefix, trees, new_lens, hq, hkv, d, npages=8 + sum((a + len(t) + 15) // 16 for a, t in zip(prefix, trees)))
+        n = len(q)
+        zb, zq = np.zeros(len(trees), np.int32), np.zeros(n, np.int32)
+        eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+        ok.tree_attn_paged(q, qindptr, pages, pindptr, pvalues, last, zb, zq, eo, el, 0, 1.0, 1e4, d ** -0.5,
+                           tindptr, labels)
+        go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+        gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+        K.tree_attn_paged_kv(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(zb), i32(zq),
+                             go, gl, 0, 1.0, 1e4, d ** -0.5, i32(tindptr), i32(labels))
+        assert_close(host(go), eo, what=f"tree paged out, {splits} splits")
+        assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"tree paged lse, {splits} splits")
+
+        prefix = [0, 1, 63, 64, 65, 1500, 200, 700]
+        chunk = [5, 130, 1, 64, 33, 40, 2, 129]
+        pages, pindptr, pvalues, last, ks, vs = build_paged_kv(rng, prefix, 8 + sum((x + 15) // 16 for x in prefix), hkv, 16, d)
+        n = sum(chunk)
+        ind = np.concatenate([[0], np.cumsum(chunk)]).astype(np.int32)
+        q = rng.standard_normal((n, hq, d)).astype(F16)
+        k = rng.standard_normal((n, hkv, d)).astype(F16)
+        v = rng.standard_normal((n, hkv, d)).astype(F16)
+        zq, zb = np.zeros(n, np.int32), np.zeros(len(prefix), np.int32)
+        eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+        to, tl = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+        ok.prefill_ragged(q, ind, k, v, ind, zq, zb, eo, el, 1, 0, 1.0, 1e4, d ** -0.5)
+        ok.prefill_paged(q, ind, pages, pindptr, pvalues, last, zb, zq, to, tl, 0, 0, 1.0, 1e4, d ** -0.5)
+        ok.merge_state_inplace(eo, el, to, tl)
+        go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+        gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+        K.batch_prefill_cached_and_new_kv(dev(q), i32(ind), dev(k), dev(v), dev(pages), i32(pindptr), i32(pvalues),
+                                          i32(last), go, gl, d ** -0.5)
+        assert_close(host(go), eo, what=f"one-pass chunked prefill out, {splits} splits")
+        assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"one-pass chunked prefill lse, {splits} splits")
+    finally:
+        tvm_amd.set_option("prefill_kv_splits", prev)
+
+
 def test_prefill_more_than_64_sequences():
     """Up to 64 sequences the kernels rank the sequences by length themselves; beyond that they
     take them in batch order.  Both orders on one ragged and one paged call."""

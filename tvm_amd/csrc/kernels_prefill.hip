@@ -30,6 +30,7 @@
 #include <type_traits>
 
 #include "prefill_common.cuh"
+#include "runtime_support.h"
 
 namespace tvmkv {
 
@@ -502,13 +503,21 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : 2) void 
     }
   };
 
-  const int n_tiles = (kv_end + BN - 1) / BN;
+  // This workgroup's key tiles [tile_lo, n_tiles): all of the row tile's, or its share of them
+  int tile_lo = 0, n_tiles = (kv_end + BN - 1) / BN;
+  if (SRC != kRagged && p.kv_splits > 1) {  // (ragged launches are never split)
+    const int per_split = (n_tiles + p.kv_splits - 1) / p.kv_splits;
+    tile_lo = min(static_cast<int>(blockIdx.z) * per_split, n_tiles);
+    n_tiles = min(tile_lo + per_split, n_tiles);
+    // the page ids are held for windows of 64 tiles that start at multiples of 64
+    if ((PAGED || (BOTH && tile_lo < prefix_tiles)) && (tile_lo & 63) != 0 && tile_lo < n_tiles) load_page_ids(tile_lo & ~63);
+  }
   // Tiles tile .. tile+NSTAGE-2 are in flight or landed at the top of iteration `tile`.
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s) {
-    if (s < n_tiles) issue_tile(s);
+    if (tile_lo + s < n_tiles) issue_tile(tile_lo + s);
   }
-  for (int tile = 0; tile < n_tiles; ++tile) {
+  for (int tile = tile_lo; tile < n_tiles; ++tile) {
     const int kv0 = tile * BN;
     const half_t* Ks = lds_tiles + (tile % NSTAGE) * STAGE;
     const half_t* Vs = Ks + BN * DQK;
@@ -686,8 +695,9 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : 2) void 
   const float denom = lsum + fast_exp2(kNegInit - m);  // the d = 1 of the initial state
   if (row_valid) {
     const float inv = 1.0f / denom;
-    half_t* orow = p.output + (static_cast<int64_t>(q_start + my_pos) * p.h_q + my_head) * DV + half * 4;
-    float* lse_ptr = p.lse + static_cast<int64_t>(q_start + my_pos) * p.h_q + my_head;
+    const int64_t out_row = (SRC != kRagged && p.kv_splits > 1 ? blockIdx.z * p.split_rows : 0) + static_cast<int64_t>(q_start + my_pos) * p.h_q + my_head;
+    half_t* orow = p.output + out_row * DV + half * 4;
+    float* lse_ptr = p.lse + out_row;
     const float my_lse = m + fast_log2(denom);
     if (p.merge_into) {
       // python/tvm/relax/frontend/nn/llm/_decode_kernels.py:441-450 with (v, s) = what the arrays
@@ -752,9 +762,99 @@ static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const Pr
   }
   PrefillParams launch = p;
   launch.clock_probe = g_prefill_clock_probe;
-  hipLaunchKernelGGL((prefill_kernel<DQK, DV, SRC, PS, EXT>), dim3(p.h_kv, static_cast<unsigned>(slots)),
+  hipLaunchKernelGGL((prefill_kernel<DQK, DV, SRC, PS, EXT>),
+                     dim3(p.h_kv, static_cast<unsigned>(slots), static_cast<unsigned>(std::max(1, p.kv_splits))),
                      dim3(NW * 64), lds_bytes, stream, launch, div);
 }
+
+// ---- split over the keys ---------------------------------------------------------------------
+// A launch with few row tiles and long key ranges (a token tree or a short chunk against long cached
+// sequences) neither fills the chip nor balances it: a row tile is one workgroup that walks all its
+// keys.  Such a launch is split: kv_splits workgroups share a row tile, each writes the attention state
+// of its share of the key tiles (normalised output in fp16, lse) to scratch memory, and a second kernel
+// merges the states of a row with the arithmetic of merge_state_inplace
+// (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:441-450) over kv_splits states at once.  A row
+// whose states are all empty (lse = -5e4) stays the empty state: out 0, lse -5e4.
+template <int DV>
+__global__ __launch_bounds__(256) void prefill_split_merge_kernel(const half_t* __restrict__ part_o,
+                                                                  const float* __restrict__ part_lse, half_t* __restrict__ output,
+                                                                  float* __restrict__ lse, int64_t rows, int splits) {
+  constexpr int TPR = DV / 8;  // threads per row, 8 features each
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * (256 / TPR) + threadIdx.x / TPR;
+  const int piece = threadIdx.x % TPR;
+  if (row >= rows) return;
+  float s_max = kNegInit;
+  for (int i = 0; i < splits; ++i) s_max = fmaxf(s_max, part_lse[i * rows + row]);
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float w_sum = 0.f;
+  if (s_max > kNegInit) {
+    for (int i = 0; i < splits; ++i) {
+      const float w = fast_exp2(part_lse[i * rows + row] - s_max);
+      const Vec16 v = ld16(part_o + (i * rows + row) * DV + piece * 8);
+      w_sum += w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += w * static_cast<float>(v.h8[e]);
+    }
+  }
+  const float inv = w_sum > 0.f ? 1.0f / w_sum : 0.f;
+  Vec16 out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out.h8[e] = static_cast<half_t>(acc[e] * inv);
+  *reinterpret_cast<Vec16*>(output + row * DV + piece * 8) = out;
+  if (piece == 0) lse[row] = w_sum > 0.f ? s_max + fast_log2(w_sum) : kNegInit;
+}
+
+// How many ways to split the keys of a launch with `workgroups` row-tile workgroups (an upper bound:
+// spare slots included) whose sequences hold avg_keys keys on average.  Enough workgroups for two
+// rounds of the chip's two per compute unit, no share shorter than 8 tiles, at most 64 shares.  More
+// shares than that cost more in start-up, epilogue and merge traffic than they gain in balance
+// (64 sequences of 1024-8192 keys with a 4-token chain each, 576 workgroups: 0.241 ms unsplit, 0.217 ms
+// with 2 shares, 0.226 with 4, 0.239 with 8; a 63-node tree per sequence, 1520 workgroups, matrix-bound:
+// 0.409 ms unsplit, 0.442 with 2 shares).
+static int pick_kv_splits(int64_t workgroups, int64_t avg_keys) {
+  const int64_t forced = option(kOptPrefillKvSplits);
+  if (forced > 0) return static_cast<int>(std::min<int64_t>(forced, 64));
+  const int64_t target = static_cast<int64_t>(compute_units()) * 2 * 2;
+  if (workgroups >= target) return 1;
+  const int64_t by_work = (target + workgroups - 1) / std::max<int64_t>(workgroups, 1);
+  const int64_t by_length = avg_keys / (8 * BN);
+  return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(std::min(by_work, by_length), 64)));
+}
+
+// Redirects the launch described by p to scratch memory when it is to be split; finish() merges.
+struct KvSplit {
+  half_t* output;
+  float* lse;
+  int64_t rows;
+  int splits;
+  KvSplit(PrefillParams& p, int64_t total_q, int64_t avg_keys, int dv, hipStream_t stream)
+      : output(p.output), lse(p.lse), rows(total_q * p.h_q), splits(1) {
+    if (p.merge_into) return;  // the epilogue merges into the caller's state: one workgroup per row tile
+    const int64_t slots = total_q * p.group / BM + p.batch_size;
+    splits = pick_kv_splits(slots * p.h_kv, avg_keys);
+    if (splits <= 1) return;
+    const size_t o_bytes = static_cast<size_t>(splits) * rows * dv * sizeof(half_t);
+    const size_t lse_bytes = static_cast<size_t>(splits) * rows * sizeof(float);
+    char* ws = lease_scratch(kScratchPrefill, stream, o_bytes + lse_bytes, 0).ptr;
+    p.output = reinterpret_cast<half_t*>(ws);
+    p.lse = reinterpret_cast<float*>(ws + o_bytes);
+    p.kv_splits = splits;
+    p.split_rows = rows;
+  }
+  void finish(const PrefillParams& p, int dv, hipStream_t stream) const {
+    if (splits <= 1) return;
+    KV_LAUNCH_CHECK();
+    const unsigned rows_per_block = 256 / (dv / 8);
+    const dim3 grid(static_cast<unsigned>((rows + rows_per_block - 1) / rows_per_block));
+    if (dv == 128) {
+      hipLaunchKernelGGL(prefill_split_merge_kernel<128>, grid, dim3(256), 0, stream, p.output, p.lse, output, lse, rows, splits);
+    } else if (dv == 64) {
+      hipLaunchKernelGGL(prefill_split_merge_kernel<64>, grid, dim3(256), 0, stream, p.output, p.lse, output, lse, rows, splits);
+    } else {
+      hipLaunchKernelGGL(prefill_split_merge_kernel<256>, grid, dim3(256), 0, stream, p.output, p.lse, output, lse, rows, splits);
+    }
+  }
+};
 
 // The extended kernels (sliding-window cache, per-layer window, inline RoPE) exist for the head
 // dims that RoPE models use here; d_qk 192 / d_v 128 is the MLA self-attention, which has neither.
@@ -900,6 +1000,7 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
   }
   const bool ext = p.rotary != 0 || sliding_window != 0;
   hipStream_t s = as_stream(stream);
+  const KvSplit split(p, total_q, nnz_pages * page_size / batch_size, d, s);
   if (d == 128) {
     launch_prefill<128, 128, kPaged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d == 64) {
@@ -909,6 +1010,7 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_paged_kv: head_dim " << d << " is not built (64, 128, 256)";
   }
+  split.finish(p, d, s);
   KV_LAUNCH_CHECK();
   KV_API_END();
 }
@@ -982,6 +1084,7 @@ static int cached_and_new(const void* q, int64_t q_token_stride, const int32_t* 
   p.causal = 1;
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
   hipStream_t s = as_stream(stream);
+  const KvSplit split(p, total_q, (nnz_pages * page_size + total_q) / batch_size, d, s);
   if (d == 128) {
     launch_prefill<128, 128, kBoth, 16>(p, total_q, false, rope_theta, s);
   } else if (d == 64) {
@@ -991,6 +1094,7 @@ static int cached_and_new(const void* q, int64_t q_token_stride, const int32_t* 
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_cached_and_new_kv: head_dim " << d << " is not built (64, 128, 256)";
   }
+  split.finish(p, d, s);
   KV_LAUNCH_CHECK();
   KV_API_END();
 }
@@ -1109,6 +1213,7 @@ int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void*
   p.tree_indptr = tree_order_indptr;
   p.tree_order = tree_order;
   hipStream_t s = as_stream(stream);
+  const KvSplit split(p, total_q, nnz_pages * page_size / batch_size, d, s);
   if (d == 128) {
     launch_prefill<128, 128, kPaged, 16>(p, total_q, true, rope_theta, s);
   } else if (d == 64) {
@@ -1118,6 +1223,7 @@ int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void*
   } else {
     KV_UNSUPPORTED(true) << "tree_attn_paged_kv: head_dim " << d << " is not built (64, 128, 256)";
   }
+  split.finish(p, d, s);
   KV_LAUNCH_CHECK();
   KV_API_END();
 }

@@ -50,6 +50,10 @@ struct PrefillParams {
   // rotates them at q_rope_position[token] itself (with rope_scale and the divisors of the launch)
   int64_t q_token_stride;
   int q_inline_rope;
+  // > 1: gridDim.z workgroups share a row tile, each taking an equal share of its key tiles and writing
+  // its own attention state: output / lse then point at kv_splits arrays of split_rows rows each
+  int kv_splits;
+  int64_t split_rows;
   int page_shift;   // pages hold 16 << page_shift tokens; the kernel walks them as runs of 16-token pages
   int clock_probe;  // != 0: add this workgroup's shader cycles and 100 MHz ticks to the probe counters
 };

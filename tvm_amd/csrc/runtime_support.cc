@@ -17,9 +17,10 @@ namespace {
 struct OptionTable {
   std::atomic<int64_t> value[kNumOptions];
   OptionTable() {
-    static const char* const env_names[kNumOptions] = {"TVMKV_DECODE_CHUNK_PAGES", "TVMKV_DECODE_SEPARATE_MERGE",
+    static const char* const env_names[] = {"TVMKV_DECODE_CHUNK_PAGES", "TVMKV_DECODE_SEPARATE_MERGE",
                                                        "TVMKV_DECODE_WGS_PER_CU", "TVMKV_MLA_CHUNK_TOKENS",
-                                                       "TVMKV_MLA_SEPARATE_MERGE"};
+                                                       "TVMKV_MLA_SEPARATE_MERGE", "TVMKV_PREFILL_KV_SPLITS"};
+    static_assert(sizeof(env_names) / sizeof(env_names[0]) == kNumOptions, "one environment variable per option");
     for (int i = 0; i < kNumOptions; ++i) {
       const char* text = std::getenv(env_names[i]);  // once, when the library is loaded
       value[i].store(text != nullptr ? std::atoll(text) : 0, std::memory_order_relaxed);
@@ -28,8 +29,9 @@ struct OptionTable {
 };
 OptionTable g_options;
 
-const char* const kOptionNames[kNumOptions] = {"decode_chunk_pages", "decode_separate_merge", "decode_wgs_per_cu",
-                                               "mla_chunk_tokens", "mla_separate_merge"};
+const char* const kOptionNames[] = {"decode_chunk_pages", "decode_separate_merge", "decode_wgs_per_cu",
+                                               "mla_chunk_tokens", "mla_separate_merge", "prefill_kv_splits"};
+static_assert(sizeof(kOptionNames) / sizeof(kOptionNames[0]) == kNumOptions, "one name per option");
 
 struct Scratch {
   char* ptr = nullptr;

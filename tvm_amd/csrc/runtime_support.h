@@ -16,6 +16,7 @@ enum Option {
   kOptDecodeWgsPerCu,         // > 0: cap the decode grid at this many workgroups per compute unit
   kOptMlaChunkTokens,         // lower bound of the tokens per split-KV chunk of the MLA kernel, 0 = 128
   kOptMlaSeparateMerge,       // unused (the MLA chunks are always merged in a second launch)
+  kOptPrefillKvSplits,        // > 0: split the keys of every row tile of a paged prefill launch this many ways, 0 = derived
   kNumOptions
 };
 int64_t option(Option id);
@@ -30,7 +31,7 @@ struct ScratchLease {
   char* ptr;        // device memory, at least the requested size, 256-byte aligned
   uint32_t epoch;   // never 0
 };
-enum ScratchUser { kScratchDecode = 0, kScratchMla = 1 };
+enum ScratchUser { kScratchDecode = 0, kScratchMla = 1, kScratchPrefill = 2 };
 ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, size_t counter_bytes);
 
 // Chunk-slot arithmetic of the decode split, on the host (the device functions of the same names in
