@@ -49,11 +49,12 @@ def test_every_chunk_has_exactly_one_slot(name, forced_cp, h_kv):
 
 
 def test_chunk_size_follows_the_work():
-    # ~2300 work items: small batches split finely, huge ones stop at 128 pages per chunk
-    assert tvm_amd.decode_split_plan([0, 4], 4, 8)[0] == 8
-    assert tvm_amd.decode_split_plan([0, 18432], 18432, 8)[0] == 64
+    # 768 work items for small launches up to ~2300 for large ones; chunks of 16 to 128 pages
+    assert tvm_amd.decode_split_plan([0, 4], 4, 8)[0] == 16
+    assert tvm_amd.decode_split_plan([0, 18432], 18432, 8)[0] == 64      # configs[1]: 2304 items
     assert tvm_amd.decode_split_plan([0, 1 << 20], 1 << 20, 8)[0] == 128
-    assert tvm_amd.decode_split_plan([0, 18432], 18432, 1)[0] == 8
+    assert tvm_amd.decode_split_plan([0, 18432], 18432, 1)[0] == 32      # one kv head: 768 items
+    assert tvm_amd.decode_split_plan([0, 8192], 8192, 8)[0] == 64        # one sequence of 131072 tokens
 
 
 def test_options_round_trip_and_reject_unknown_names():

@@ -1,6 +1,7 @@
 // Tuning options and the scratch-buffer pool of the split-KV launchers (see runtime_support.h).
 #include "runtime_support.h"
 
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <cstring>
@@ -75,14 +76,20 @@ ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, s
   return ScratchLease{s.ptr, s.epoch};
 }
 
-// ~2300 work items = three rounds of 3 workgroups x 256 CUs; every item pays ~2 us of fixed cost
-// (locating its sequence, q, the cross-wave merge), so chunks should not be smaller than that buys.
-// One step of the matrix-core decode kernel is 2 pages per wave, 8 per workgroup.
+// Work items of a decode launch: every item pays ~2 us of fixed cost (locating its sequence, q, the
+// cross-wave merge) and every chunk of a sequence is one more partial state for the merge, whose loads
+// are round trips to memory.  Large launches (cfg 2: 147 k pages x kv heads) run best with ~2300 items =
+// three rounds of 3 workgroups x 256 CUs; small ones with fewer and longer items (one sequence of 131 072
+// tokens: 0.110 ms with 32-page chunks, 0.085 with 128; 64 sequences with one kv head: 0.140 ms with
+// 8-page chunks, 0.073 with 64).  One step of the matrix-core decode kernel is 2 pages per wave, 8 per
+// workgroup; chunks are powers of two from 16 to 128 pages.
 int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv) {
   const int64_t forced = option(kOptDecodeChunkPages);
   if (forced >= 8 && forced % 8 == 0) return static_cast<int>(forced);
-  const int64_t cp = nnz_pages * h_kv / 2304;
-  int pow2 = 8;
+  const int64_t work = nnz_pages * h_kv;
+  const int64_t items = std::min<int64_t>(std::max<int64_t>(work / 64, 768), 2304);
+  const int64_t cp = work / items;
+  int pow2 = 16;
   while (pow2 < 128 && pow2 * 3 / 2 <= cp) pow2 *= 2;  // nearest power of two
   return pow2;
 }
