@@ -209,6 +209,20 @@ def test_decode_long_sequence_many_chunks():
     assert_close(gl, el, atol=1e-3, rtol=1e-4, what="long decode lse")
 
 
+@pytest.mark.parametrize("batch", [65, 130, 700, 5000])
+def test_decode_many_short_sequences(batch):
+    """Every work item finds its sequence by a 64-ary search over page_indptr: batches that need one,
+    two and three rounds of it, sequences of 0 to 3 pages and a few long ones with several chunks."""
+    rng = np.random.default_rng(80 + batch)
+    hq, hkv, d = 8, 2, 64
+    kv_lens = [int(x) for x in rng.integers(0, 40, size=batch)]
+    for i in rng.integers(0, batch, size=5):
+        kv_lens[int(i)] = int(rng.integers(300, 900))
+    go, gl, eo, el = _decode_both(rng, kv_lens, hq, hkv, d, npages=8 + sum((n + 15) // 16 for n in kv_lens))
+    assert_close(go, eo, what=f"decode out, {batch} sequences")
+    assert_close(gl, el, atol=1e-3, rtol=1e-4, what=f"decode lse, {batch} sequences")
+
+
 def test_decode_ignores_garbage_beyond_last_page_len():
     """Slots of the last page beyond last_page_len may hold NaN/Inf bit patterns."""
     rng = np.random.default_rng(8)

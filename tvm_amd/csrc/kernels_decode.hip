@@ -60,20 +60,24 @@ struct DecodeParams {
   float scale_log2;  // sm_scale * log2(e)
 };
 
-// Same answer as find_sequence, computed by one wavefront with one round trip per 64 sequences:
-// lane i evaluates slot_begin(base + i) <= slot, and because slot_begin is increasing the number
-// of set lanes is the position of the last sequence that qualifies.
+// Same answer as find_sequence, computed by one wavefront as a 64-ary search: the lanes probe
+// slot_begin at 64 evenly spaced sequences of the range that is left, and because slot_begin is
+// increasing the number of lanes that qualify tells which sixty-fourth holds the answer.  One round
+// trip to memory per factor of 64 in the batch size (a linear scan in blocks of 64 sequences cost a
+// launch of 2048 sequences up to 32 dependent round trips per work item).
 __device__ __forceinline__ int find_sequence_wave(const int32_t* page_indptr, int batch, int cp, int slot,
                                                   int lane) {
-  int b = 0;
-  for (int base = 0; base < batch; base += 64) {
-    const int idx = base + lane;
-    const bool le = idx < batch && slot_begin(page_indptr, idx, cp) <= slot;
-    const int count = __popcll(__ballot(le));
-    if (count > 0) b = base + count - 1;
-    if (count < 64) break;
+  int lo = 0, n = batch;  // the answer lies in [lo, lo + n), and slot_begin(lo) <= slot
+  while (n > 64) {
+    const int stride = (n + 63) >> 6;
+    const int idx = lo + lane * stride;
+    const bool le = idx < lo + n && slot_begin(page_indptr, idx, cp) <= slot;
+    const int first = lo + (__popcll(__ballot(le)) - 1) * stride;  // lane 0 always qualifies
+    n = min(stride, lo + n - first);
+    lo = first;
   }
-  return b;
+  const bool le = lane < n && slot_begin(page_indptr, lo + lane, cp) <= slot;
+  return lo + max(__popcll(__ballot(le)), 1) - 1;
 }
 
 // Merge of the per-chunk partial states of one (sequence, query head) row by one wavefront.
