@@ -162,16 +162,20 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : 2) void 
     seq_k0 = __builtin_amdgcn_readlane(lk0, b);
     seq_k1 = __builtin_amdgcn_readlane(lk1, b);
   } else {
-    int lo = 0, hi = p.batch_size - 1;
-    while (lo < hi) {
-      int mid = (lo + hi + 1) >> 1;
-      if (tile_slot_begin(p.q_indptr, mid, group) <= slot) {
-        lo = mid;
-      } else {
-        hi = mid - 1;
-      }
+    // the last sequence whose first slot is at or before this one, by a 64-ary search of the wave: the
+    // lanes probe 64 evenly spaced sequences of the range that is left, one round trip to memory per
+    // factor of 64 in the batch size (tile_slot_begin is increasing and 0 for sequence 0)
+    int lo = 0, n = p.batch_size;
+    while (n > 64) {
+      const int stride = (n + 63) >> 6;
+      const int idx = lo + lane * stride;
+      const bool le = idx < lo + n && tile_slot_begin(p.q_indptr, idx, group) <= slot;
+      const int first = lo + (__popcll(__ballot(le)) - 1) * stride;
+      n = min(stride, lo + n - first);
+      lo = first;
     }
-    b = lo;
+    const bool le = lane < n && tile_slot_begin(p.q_indptr, lo + lane, group) <= slot;
+    b = __builtin_amdgcn_readfirstlane(lo + max(static_cast<int>(__popcll(__ballot(le))), 1) - 1);
     local_slot = slot - tile_slot_begin(p.q_indptr, b, group);
     seq_q0 = p.q_indptr[b];
     seq_q1 = p.q_indptr[b + 1];
