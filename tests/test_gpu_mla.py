@@ -103,6 +103,22 @@ def test_mla_as_many_tokens_as_sequences_but_not_a_decode_step():
     assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla mixed lse")
 
 
+@pytest.mark.parametrize("causal", [1, 0])
+def test_mla_few_tokens_per_sequence_split_kv(causal):
+    """A draft to verify (a few tokens per sequence) and a short chunk late in a long sequence have as few
+    row tiles as a decode step: the launcher plans every token as a one-token sequence of its own (under
+    the causal mask token j of n sees the first L - n + j + 1 keys) and splits the KV."""
+    rng = np.random.default_rng(36 + causal)
+    for kv_lens, q_lens in (([1500, 64, 700, 65, 4, 900, 130, 33], [4, 4, 4, 4, 4, 4, 4, 4]),   # verify
+                            ([3000], [64]),                                                       # one short chunk
+                            ([900, 5, 300, 0, 420, 77], [3, 5, 0, 2, 1, 7])):                    # ragged, empty sequences
+        if causal:
+            kv_lens = [max(k, q) for k, q in zip(kv_lens, q_lens)]
+        go, gl, eo, el = _mla_both(rng, kv_lens, q_lens, 64, npages=8 + sum((n + 63) // 64 for n in kv_lens), causal=causal)
+        assert_close(go, eo, what=f"mla few tokens out, q_lens {q_lens}")
+        assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"mla few tokens lse, q_lens {q_lens}")
+
+
 def test_mla_decode_heads_not_a_multiple_of_the_row_tile():
     rng = np.random.default_rng(34)
     kv_lens = [900, 33, 257]

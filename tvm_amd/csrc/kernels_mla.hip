@@ -61,6 +61,10 @@ struct MlaParams {
   int page_shift;    // log2(page_size) when it is a power of two, else -1
   int causal;
   int split;         // 1: decode-shaped call, the KV of the sequences is cut into chunks (see mla_split_plan)
+  // split launch of a call with several tokens per sequence (a draft to verify, a short chunk): every
+  // token is planned as a sequence of its own with one token, batch_size counts the tokens and tokens_of
+  // is the number of real sequences behind q_indptr / page_indptr / last_page_len; 0 otherwise
+  int tokens_of;
   int min_chunk_tiles;  // split: lower bound of the chunk length
   int row_tiles;     // split: row tiles of a one-token sequence, ceil(h_q / MLA_BM)
   float scale_log2;
@@ -172,7 +176,30 @@ struct MlaSeqInfo {
 };
 __device__ __forceinline__ MlaSeqInfo mla_seq_info(const MlaParams& p, int b) {
   MlaSeqInfo s{0, 0, 0, 0, 0, 0};
-  if (b < p.batch_size) {
+  if (b < p.batch_size && p.tokens_of > 0) {
+    // token b of the call as a one-token sequence: under the causal mask token j of n sees the first
+    // L - n + j + 1 of its sequence's L keys (python/tvm/relax/frontend/nn/llm/_kernel_common.py:130-135),
+    // which is plain attention over that many keys
+    int lo = 0, hi = p.tokens_of - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (p.q_indptr[mid] <= b) {
+        lo = mid;
+      } else {
+        hi = mid - 1;
+      }
+    }
+    const int first = p.q_indptr[lo];
+    const int n = p.q_indptr[lo + 1] - first;
+    const int npages = p.page_indptr[lo + 1] - p.page_indptr[lo];
+    const int len = npages > 0 ? (npages - 1) * p.page_size + p.last_page_len[lo] : 0;
+    s.q_start = b;
+    s.qo_len = 1;
+    s.pbeg = p.page_indptr[lo];
+    s.kv_len = p.causal ? max(0, min(len, len - n + (b - first) + 1)) : len;
+    s.npages = (s.kv_len + p.page_size - 1) / p.page_size;
+    s.cost = (s.kv_len + MLA_BN - 1) / MLA_BN;
+  } else if (b < p.batch_size) {
     s.q_start = p.q_indptr[b];
     s.qo_len = p.q_indptr[b + 1] - s.q_start;
     s.pbeg = p.page_indptr[b];
@@ -255,20 +282,25 @@ __device__ __forceinline__ void mla_merge_heads(const MlaParams& p, int q_row, i
   static_assert(DV == 512, "16 lanes x 32 features");
   const int sub = lane >> 4;   // which of the wave's four heads
   const int part = lane & 15;  // features part*32 .. +31
-  for (int h0 = h_lo; h0 < h_hi; h0 += waves * 4) {
-    const int h = h0 + wave * 4 + sub;
+  // Few heads mean many chunks (a block merges h_q / nchunks heads): then a wave takes one head and its
+  // four lane groups share the head's chunks, 4 CB of them in flight, and fold their states at the end.
+  const bool share = h_hi - h_lo <= waves;
+  const int heads_per_wave = share ? 1 : 4;
+  const int cstep = share ? 4 : 1, cfirst = share ? sub : 0;
+  for (int h0 = h_lo; h0 < h_hi; h0 += waves * heads_per_wave) {
+    const int h = share ? h0 + wave : h0 + wave * 4 + sub;
     const bool valid = h < h_hi;
     const int hh = valid ? h : h_lo;  // lanes without a head repeat a valid one and drop the result
     float acc[32];
 #pragma unroll
     for (int e = 0; e < 32; ++e) acc[e] = 0.f;
     float top = -3.0e38f, wsum = 0.f;
-    for (int c0 = 0; c0 < nchunks; c0 += CB) {
+    for (int c0 = cfirst; c0 < nchunks; c0 += CB * cstep) {
       float lse_c[CB];
       half8_t o_c[CB][4];
 #pragma unroll
       for (int k = 0; k < CB; ++k) {
-        const int c = min(c0 + k, nchunks - 1);  // past the end: the last chunk again, with weight 0
+        const int c = min(c0 + k * cstep, nchunks - 1);  // past the end: the last chunk again, with weight 0
         const int64_t row = static_cast<int64_t>(first + c) * p.h_q + hh;
         lse_c[k] = p.part_lse[row];
 #pragma unroll
@@ -276,7 +308,7 @@ __device__ __forceinline__ void mla_merge_heads(const MlaParams& p, int q_row, i
       }
       float block_top = top;
 #pragma unroll
-      for (int k = 0; k < CB; ++k) block_top = fmaxf(block_top, c0 + k < nchunks ? lse_c[k] : -3.0e38f);
+      for (int k = 0; k < CB; ++k) block_top = fmaxf(block_top, c0 + k * cstep < nchunks ? lse_c[k] : -3.0e38f);
       const float keep = fast_exp2(top - block_top);  // 0 in the first round
       top = block_top;
       wsum *= keep;
@@ -284,7 +316,7 @@ __device__ __forceinline__ void mla_merge_heads(const MlaParams& p, int q_row, i
       for (int e = 0; e < 32; ++e) acc[e] *= keep;
 #pragma unroll
       for (int k = 0; k < CB; ++k) {
-        const float w = c0 + k < nchunks ? fast_exp2(lse_c[k] - top) : 0.f;
+        const float w = c0 + k * cstep < nchunks ? fast_exp2(lse_c[k] - top) : 0.f;
         wsum += w;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -293,7 +325,23 @@ __device__ __forceinline__ void mla_merge_heads(const MlaParams& p, int q_row, i
         }
       }
     }
-    if (valid) {
+    if (share) {  // (wave-uniform) fold the states of the four lane groups; a group without chunks has weight 0
+      float top_all = fmaxf(top, __shfl_xor(top, 16, 64));
+      top_all = fmaxf(top_all, __shfl_xor(top_all, 32, 64));
+      const float keep = fast_exp2(top - top_all);
+      top = top_all;
+      wsum *= keep;
+      wsum += __shfl_xor(wsum, 16, 64);
+      wsum += __shfl_xor(wsum, 32, 64);
+#pragma unroll
+      for (int e = 0; e < 32; ++e) {
+        float a = acc[e] * keep;
+        a += __shfl_xor(a, 16, 64);
+        a += __shfl_xor(a, 32, 64);
+        acc[e] = a;
+      }
+    }
+    if (valid && (!share || sub == 0)) {
       const float inv = 1.0f / wsum;  // the chunk that holds the maximum weighs 1
       const int64_t grow = static_cast<int64_t>(q_row) * p.h_q + h;
       half_t* out = p.output + grow * DV + part * 32;
@@ -826,8 +874,14 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
   const int cus = compute_units();
   const int row_tiles = (h_q + MLA_BM - 1) / MLA_BM;
   int64_t grid = slots;
-  if (total_q == batch_size && static_cast<int64_t>(batch_size) * row_tiles * 2 <= cus && batch_size <= MLA_MAX_SPLIT_BATCH &&
-      nnz_pages > 0 && nnz_pages * page_size < (int64_t{1} << 26)) {
+  // A call with a few tokens per sequence (a draft to verify, a short chunk late in a long prompt) is in the
+  // same position: its tokens are planned as one-token sequences of their own.
+  if (total_q * row_tiles * 2 <= cus && total_q <= MLA_MAX_SPLIT_BATCH && nnz_pages > 0 &&
+      nnz_pages * page_size < (int64_t{1} << 26)) {
+    if (total_q != batch_size) {
+      p.tokens_of = batch_size;
+      p.batch_size = static_cast<int>(total_q);
+    }
     const int64_t cslots = cus / row_tiles;
     p.split = 1;
     p.row_tiles = row_tiles;
