@@ -93,6 +93,18 @@ def test_mla_decode_batch_beyond_one_sequence_per_lane():
     assert not go[3].any() and np.all(gl[3] == np.float32(-5e4))
 
 
+def test_mla_decode_batch_beyond_one_split_launch():
+    """200 long sequences: more than one split launch plans, so the step is cut into two split launches
+    over slices of the index arrays; a few empty and short sequences among them."""
+    rng = np.random.default_rng(38)
+    kv_lens = [int(x) for x in rng.integers(1030, 1300, size=200)]
+    kv_lens[0], kv_lens[99], kv_lens[100], kv_lens[199] = 0, 1, 2600, 7
+    go, gl, eo, el = _mla_both(rng, kv_lens, [1] * 200, 64, npages=8 + sum((n + 63) // 64 for n in kv_lens), heads=16)
+    assert_close(go, eo, what="mla two-launch decode out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla two-launch decode lse")
+    assert not go[0].any() and np.all(gl[0] == np.float32(-5e4))
+
+
 def test_mla_as_many_tokens_as_sequences_but_not_a_decode_step():
     """total_q == batch makes the launcher split the KV; sequences that do not have exactly one
     query token must still come out right (they are done unsplit by the workgroups of chunk 0)."""

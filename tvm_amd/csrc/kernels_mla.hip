@@ -852,6 +852,25 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
       << "batch_prefill_paged_kv_mla: NULL tensor";
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_prefill_paged_kv_mla: NULL page table";
   constexpr int DQK = 576, DV = 512;
+  // A decode step of more sequences than one split launch plans (two per lane of the planning wave) with
+  // long sequences would run one workgroup per sequence, as long as its longest one and in arbitrary
+  // order: it is cut into equal parts of at most that many sequences, each a split launch of its own
+  // (200 sequences of 2048-8192 tokens: 0.57 ms in one unsplit launch).  The index arrays hold absolute
+  // offsets, so a part is the same call on a slice of them.
+  if (total_q == batch_size && batch_size > MLA_MAX_SPLIT_BATCH && batch_size <= 4 * MLA_MAX_SPLIT_BATCH &&
+      static_cast<int64_t>(MLA_MAX_SPLIT_BATCH) * ((h_q + MLA_BM - 1) / MLA_BM) * 2 <= compute_units() &&
+      nnz_pages * page_size / batch_size >= 1024) {
+    const int parts = (batch_size + MLA_MAX_SPLIT_BATCH - 1) / MLA_MAX_SPLIT_BATCH;
+    for (int i = 0; i < parts; ++i) {
+      const int lo = static_cast<int>(static_cast<int64_t>(i) * batch_size / parts);
+      const int hi = static_cast<int>(static_cast<int64_t>(i + 1) * batch_size / parts);
+      const int rc = tvmkv_batch_prefill_paged_kv_mla(q, q_indptr + lo, pages, page_indptr + lo, page_values, length_info + lo,
+                                                      output, lse, causal, sm_scale, hi - lo, hi - lo, nnz_pages, num_pages,
+                                                      h_q, d_latent, d_rope, page_size, stream);
+      if (rc != TVMKV_OK) return rc;
+    }
+    return TVMKV_OK;
+  }
   MlaParams p{};
   p.q = static_cast<const half_t*>(q);
   p.q_indptr = q_indptr;
