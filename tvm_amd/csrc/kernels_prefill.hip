@@ -808,21 +808,33 @@ __global__ __launch_bounds__(256) void prefill_split_merge_kernel(const half_t* 
   if (piece == 0) lse[row] = w_sum > 0.f ? s_max + fast_log2(w_sum) : kNegInit;
 }
 
-// How many ways to split the keys of a launch with `workgroups` row-tile workgroups (an upper bound:
-// spare slots included) whose sequences hold avg_keys keys on average.  Enough workgroups for two
-// rounds of the chip's two per compute unit, no share shorter than 8 tiles, at most 64 shares.  More
-// shares than that cost more in start-up, epilogue and merge traffic than they gain in balance
-// (64 sequences of 1024-8192 keys with a 4-token chain each, 576 workgroups: 0.241 ms unsplit, 0.217 ms
-// with 2 shares, 0.226 with 4, 0.239 with 8; a 63-node tree per sequence, 1520 workgroups, matrix-bound:
-// 0.409 ms unsplit, 0.442 with 2 shares).
-static int pick_kv_splits(int64_t workgroups, int64_t avg_keys) {
+// How many ways to split the keys of a launch of total_q query tokens in `batch` sequences whose
+// sequences hold avg_keys keys on average (shapes only: no read of the index arrays).  The launch has at
+// least max(total_q * group / BM, batch) row tiles, times h_kv workgroups, and the chip holds two
+// workgroups per compute unit.
+//  * Less than half a round of workgroups: as many shares as fill two rounds.
+//  * Up to one round, of row tiles that are at most half full (a draft chain or a small tree per
+//    sequence): the K/V stream decides and two shares balance it (64 sequences of 1024-8192 keys with a
+//    4-token chain each: 0.241 ms unsplit, 0.217 with 2 shares, 0.226 with 4, 0.239 with 8).
+//  * Otherwise none: workgroups that end early leave their compute unit to the one that shares it, and
+//    shares only add start-up, epilogue and merge traffic (16 sequences with 128-token chunks on
+//    2000-6000 keys, 512 workgroups: 0.171 ms unsplit, 0.183 with 2 shares; a 63-node tree per sequence,
+//    1008 workgroups, matrix-bound: 0.409 against 0.442).
+// No share shorter than 8 tiles on average, at most 64 shares.
+static int pick_kv_splits(int64_t total_q, int group, int batch, int h_kv, int64_t avg_keys) {
   const int64_t forced = option(kOptPrefillKvSplits);
   if (forced > 0) return static_cast<int>(std::min<int64_t>(forced, 64));
-  const int64_t target = static_cast<int64_t>(compute_units()) * 2 * 2;
-  if (workgroups >= target) return 1;
-  const int64_t by_work = (target + workgroups - 1) / std::max<int64_t>(workgroups, 1);
+  const int64_t resident = static_cast<int64_t>(compute_units()) * 2;
+  const int64_t tiles = std::max<int64_t>((total_q * group + BM - 1) / BM, batch);
+  const int64_t workgroups = tiles * h_kv;
+  int64_t want = 1;
+  if (workgroups * 2 <= resident) {
+    want = (2 * resident + workgroups - 1) / workgroups;
+  } else if (workgroups <= resident && total_q * group * 2 <= tiles * BM) {
+    want = 2;
+  }
   const int64_t by_length = avg_keys / (8 * BN);
-  return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(std::min(by_work, by_length), 64)));
+  return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(std::min(want, by_length), 64)));
 }
 
 // Redirects the launch described by p to scratch memory when it is to be split; finish() merges.
@@ -834,8 +846,7 @@ struct KvSplit {
   KvSplit(PrefillParams& p, int64_t total_q, int64_t avg_keys, int dv, hipStream_t stream)
       : output(p.output), lse(p.lse), rows(total_q * p.h_q), splits(1) {
     if (p.merge_into) return;  // the epilogue merges into the caller's state: one workgroup per row tile
-    const int64_t slots = total_q * p.group / BM + p.batch_size;
-    splits = pick_kv_splits(slots * p.h_kv, avg_keys);
+    splits = pick_kv_splits(total_q, p.group, p.batch_size, p.h_kv, avg_keys);
     if (splits <= 1) return;
     const size_t o_bytes = static_cast<size_t>(splits) * rows * dv * sizeof(half_t);
     const size_t lse_bytes = static_cast<size_t>(splits) * rows * sizeof(float);
