@@ -433,6 +433,13 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   }
   const int rows = qo_len * h_q;
   // (a sequence of a split call that is not a decode step is one chunk: its workgroup walks all its row tiles)
+  if (!p.split) {
+    // a sequence's row tiles from the last to the first: under the causal mask the last rows see the most
+    // keys, and the workgroups that start last decide when the kernel ends
+    const int tiles = (rows + MLA_BM - 1) / MLA_BM;
+    const int local = r0 / MLA_BM;
+    if (local < tiles) r0 = (tiles - 1 - local) * MLA_BM;
+  }
 
   const int ps = p.page_size;
 
