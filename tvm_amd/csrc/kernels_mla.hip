@@ -481,13 +481,9 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   };
   if (tile_lo < tile_hi) load_page_ids(tile_lo);
   __builtin_amdgcn_sched_barrier(0);
-  // Q^T fragments (B operand): column = query col, contraction slots = features ks*16 + half*8 .. +7
+  // Q^T fragments (B operand): column = query col, contraction slots = features ks*16 + half*8 .. +7;
+  // filled below, through LDS
   half8_t qf[KS];
-  {
-    const half_t* qrow = p.q + (static_cast<int64_t>(q_start + my_pos) * h_q + my_head) * DQK + half * 8;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_valid ? ld16(qrow + ks * 16).h8 : zero16().h8;
-  }
   // O^T accumulators: register 16*db + j is feature db*32 + (j/4)*8 + half*4 + j%4 of query col
   static_assert(DB * 16 == 256, "O fills the accumulation registers");
   static_for<DB * 16>([&](auto r) { acc_zero<decltype(r)::value>(); });
@@ -714,9 +710,68 @@ __global__ __launch_bounds__(MLA_WAVES * 64, 1) void mla_paged_kernel(MlaParams 
   // of the workgroup (a tile beyond a wave's own causal bound is masked like the diagonal one):
   // with 128 heads a workgroup is a single position anyway.
   const int n_tiles = tile_hi - tile_lo;
+  // ---- the query rows ---------------------------------------------------------------------------
+  // A wave's 32 query rows are 32 consecutive rows of q, 36 KiB: the shape of a tile.  Loaded straight
+  // into the fragment layout, every load instruction touches 32 rows x 32 bytes and the texture cache
+  // looks up 32 lines for it (10 k cycles for the four waves of a decode step, the longest part of the
+  // workgroup's start-up); copied to LDS like a tile, an instruction moves 8 rows x 128 bytes, and
+  // the fragments come out of LDS the way the K fragments do.  A wave's rows fill one pipeline stage,
+  // and stages 2 and 3 are free until the tiles 2 and 3 are copied: waves 0 and 1 go first, beside the
+  // load of the page ids, waves 2 and 3 after them, beside the copies of the first two tiles.
+  {
+    // the wave's first row (a wave past the end of the rows copies the last row, and zeroes what it reads)
+    const int q_first = min(first_row_wave, rows - 1);
+    const half_t* q_wave = p.q + (static_cast<int64_t>(q_start) * h_q + q_first) * DQK;
+    const int q_last = rows - 1 - q_first;  // rows past it repeat it
+    const int q_stage = 2 + (wave & 1);
+    const uint32_t q_at = lds_base + q_stage * (STAGE * 2);
+    auto copy_q = [&]() {
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    if (s < n_tiles) issue_tile(tile_lo + s);
+      for (int n = 0; n < NCOPY; ++n) {
+        const int blk = n >> 2;
+        const int rg = n & 3;
+        const int row = rg * 8 + (lane >> 3);
+        const int piece = (lane & 7) ^ mla_swizzle(row);
+        const uint32_t src = min(row, q_last);
+        copy16_to_lds(q_wave, src * (DQK * 2) + (blk * 64 + piece * 8) * 2, q_at + (blk * BLK + rg * 8 * 64) * 2);
+      }
+    };
+    auto read_q = [&]() {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) qf[ks] = read_k_frag(q_at + k_rel, ks);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      if (!row_valid) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = zero16().h8;
+      }
+    };
+    if (wave < 2) {  // (wave is a scalar: uniform branches)
+      copy_q();
+      wait_vmcnt<0>();
+      read_q();
+    }
+    __syncthreads();  // stages 2 and 3 are free again
+    // the page ids have long arrived; said here, so that the wait the compiler puts in front of their first use
+    // (it waits for every load in flight) does not fall behind the copies of the query rows
+    asm volatile("" : "+v"(page_ids));
+    if (wave >= 2) copy_q();
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      if (s < n_tiles) issue_tile(tile_lo + s);
+    }
+    if (wave >= 2) {
+      // copies complete in order: the query rows are in when no more than the tile copies issued after them are outstanding
+      if (n_tiles >= 2) {
+        wait_vmcnt<2 * COPIES>();
+      } else if (n_tiles == 1) {
+        wait_vmcnt<COPIES>();
+      } else {
+        wait_vmcnt<0>();
+      }
+      read_q();
+    }
+    // (the copies of tile 2 into stage 2 are issued after the barrier of tile_ready(0), which every wave reaches
+    //  with its query rows in registers)
   }
   auto tile_ready = [&](int w) {
     // copies complete in order: it is enough that no more than the next tile's copies are outstanding
