@@ -368,6 +368,36 @@ def extras(torch, K, dev):
     del pages
     torch.cuda.empty_cache()
 
+    # ---- decode away from configs[1]: one long sequence, few long ones, many short ones, one kv head ----
+    def decode_shape(batch, lo, hi, hq_, hkv_, seed):
+        rng_ = np.random.default_rng(seed)
+        ctx_ = rng_.integers(lo, hi, size=batch, endpoint=True)
+        npg_ = (ctx_ + 15) // 16
+        ip_ = np.concatenate([[0], np.cumsum(npg_)])
+        pool_ = int(ip_[-1]) + 64
+        perm_ = rng_.permutation(pool_).astype(np.int32)
+        pages_ = torch.empty((pool_, 2, hkv_, 16, 128), dtype=torch.float16, device=dev)
+        for lo_ in range(0, pool_, 8192):
+            pages_[lo_:lo_ + 8192].normal_()
+        q_ = torch.randn((batch, hq_, 128), device=dev).to(torch.float16)
+        o_ = torch.empty_like(q_)
+        l_ = torch.empty((batch, hq_), dtype=torch.float32, device=dev)
+        z_ = torch.zeros(batch, dtype=torch.int32, device=dev)
+        a_ = (q_, pages_, i32(ip_), i32(perm_[:ip_[-1]]), i32((ctx_ - 1) % 16 + 1), z_, z_, o_, l_, 0, 1.0, 1e4, 128 ** -0.5)
+        K.batch_decode_paged_kv(*a_)
+        ms_ = time_region(torch, lambda i: K.batch_decode_paged_kv(*a_), 20, SETTLE_S)
+        nb_ = float(ctx_.sum()) * 2 * hkv_ * 128 * 2 + 2 * batch * hq_ * 128 * 2
+        return {"ms": round(ms_, 4), "MB": round(nb_ / 1e6, 1), "frac_of_hbm_peak": round(nb_ / ms_ / 1e6 / HBM_PEAK_GBPS, 4)}
+
+    out["decode_other_shapes"] = {
+        "workload": "batch x context, query / kv heads, D128, page 16, permuted pool: the split-KV chunk rule, the chunk merge "
+                    "and the search for a work item's sequence away from configs[1]",
+        "1 x 131072, 32/8": decode_shape(1, 131072, 131072, 32, 8, 11),
+        "4 x 32768, 32/8": decode_shape(4, 32768, 32768, 32, 8, 12),
+        "2048 x U[64,512], 32/8": decode_shape(2048, 64, 512, 32, 8, 13),
+        "64 x U[1024,8192], 32/1": decode_shape(64, 1024, 8192, 32, 1, 14)}
+    torch.cuda.empty_cache()
+
     # ---- sliding window + attention sinks, and a token-tree verify step, on configs[1]'s shape ----
     hq, hkv, d, ps, nseq = 32, 8, 128, 16, 64
     rng = np.random.default_rng(7)
@@ -580,6 +610,13 @@ def extras(torch, K, dev):
     out["mla_decode"]["workload"] = "configs[4] decode: batch 32, ctx U[2048,8192] seed 4, 128 heads, 576-wide latent rows, page 64"
     mla_case("mla_prefill", np.full(4, 2048), np.full(4, 1024), 6, 1)
     out["mla_prefill"]["workload"] = "configs[4] prefill: 4 seqs, 1024-token chunk on a 2048-token prefix (chunk already appended), causal"
+    mla_case("mla_verify_4_tokens", ctx - 4, np.full(32, 4, dtype=np.int64), 7, 1)
+    out["mla_verify_4_tokens"]["workload"] = ("configs[4]'s decode batch with 4 tokens per sequence (a draft to verify), causal: every token is "
+                                              "planned as a one-token sequence and the KV is split as in a decode step")
+    ctx200 = np.random.default_rng(8).integers(2048, 8192, size=200, endpoint=True)
+    mla_case("mla_decode_200_sequences", ctx200 - 1, np.ones(200, dtype=np.int64), 9, 0)
+    out["mla_decode_200_sequences"]["workload"] = ("200 sequences, ctx U[2048,8192], one token each: more than one split launch plans, "
+                                                   "cut into two split launches of 100")
     return out
 
 
