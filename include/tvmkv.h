@@ -70,8 +70,8 @@ int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void
  * high_freq_factor, original_max_position_embeddings.  LONGROPE (:164-188): the default divisors times a
  * per-dimension factor tensor, cos and sin scaled by sqrt(1 + ln(max / original_max) / ln(original_max)).
  * YARN (:191-255): interpolated / extrapolated inverse frequencies blended over the dimensions between
- * the correction dims of beta_fast and beta_slow.  Rotation is over the whole head (rotary_dim ==
- * head_dim) with the rotate-half pairing; the gptj / llama4 interleaved pairings are not built. */
+ * the correction dims of beta_fast and beta_slow.  Rotation is over the first rotary_dim features of a head
+ * (the whole head by default) with the rotate-half pairing; the gptj / llama4 interleaved pairings are not built. */
 enum {
   TVMKV_ROPE_FREQ_DEFAULT = 0,
   TVMKV_ROPE_FREQ_LLAMA3 = 1,
@@ -80,7 +80,9 @@ enum {
 };
 typedef struct tvmkv_rope_scaling {
   int32_t rope_type;
-  int32_t reserved;
+  int32_t rotary_dim;     /* features 0 .. rotary_dim-1 of a head are rotated, in pairs (d, d + rotary_dim/2), with
+                             frequencies over rotary_dim; the others pass through (position_embedding.py:507-520).
+                             0 = head_dim.  Even, at most head_dim; any frequency variant. */
   double factor;          /* llama3, yarn */
   double low_freq_factor; /* llama3 */
   double high_freq_factor;

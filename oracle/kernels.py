@@ -59,7 +59,7 @@ def fused_rope(qkv, position_map, q, k, v, apply_rope, *, theta=1e4, scale=1.0, 
 
 class RopeScaling(ctypes.Structure):
     """orc_rope_scaling; `from_dict` takes the reference's rope_scaling dictionary (position_embedding.py:258-299)."""
-    _fields_ = [("rope_type", ctypes.c_int32), ("reserved", ctypes.c_int32), ("factor", ctypes.c_double),
+    _fields_ = [("rope_type", ctypes.c_int32), ("rotary_dim", ctypes.c_int32), ("factor", ctypes.c_double),
                 ("low_freq_factor", ctypes.c_double), ("high_freq_factor", ctypes.c_double),
                 ("beta_fast", ctypes.c_double), ("beta_slow", ctypes.c_double),
                 ("max_position_embeddings", ctypes.c_int64), ("original_max_position_embeddings", ctypes.c_int64)]
@@ -69,7 +69,7 @@ class RopeScaling(ctypes.Structure):
     def from_dict(cls, rope_scaling):
         out = cls()
         out.rope_type = cls.TYPES[rope_scaling.get("rope_type", "default")]
-        for key in ("factor", "low_freq_factor", "high_freq_factor", "beta_fast", "beta_slow",
+        for key in ("rotary_dim", "factor", "low_freq_factor", "high_freq_factor", "beta_fast", "beta_slow",
                     "max_position_embeddings", "original_max_position_embeddings"):
             if key in rope_scaling:
                 setattr(out, key, rope_scaling[key])

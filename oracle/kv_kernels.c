@@ -167,7 +167,7 @@ void orc_fused_rope(const f16* qkv, const int32_t* position_map, f16* q, f16* k,
  * against default; longrope with unit factors and max = orig against default, bit for bit. */
 typedef struct {
   int32_t rope_type; /* 0 default, 1 llama3, 2 longrope, 3 yarn */
-  int32_t reserved;
+  int32_t rotary_dim; /* 0 = head_dim */
   double factor, low_freq_factor, high_freq_factor, beta_fast, beta_slow;
   int64_t max_position_embeddings, original_max_position_embeddings;
 } orc_rope_scaling;
@@ -214,7 +214,7 @@ void orc_fused_rope_scaled(const f16* qkv, const int32_t* position_map, f16* q, 
                            int64_t apply_rope, float theta, float scale, const orc_rope_scaling* sc,
                            const float* ext_factors) {
   int fused_heads = num_q_heads + 2 * num_kv_heads;
-  int R = head_dim;
+  int R = (sc != NULL && sc->rotary_dim > 0) ? sc->rotary_dim : head_dim; /* position_embedding.py:507-520 */
   const float* ext = ext_factors;
   if (ext != NULL && sc != NULL && !(seq_len > sc->original_max_position_embeddings)) ext += R / 2;
   for (int64_t s = 0; s < seq_len; ++s) {
@@ -225,7 +225,7 @@ void orc_fused_rope_scaled(const f16* qkv, const int32_t* position_map, f16* q, 
                      ? k + (s * num_kv_heads + (h - num_q_heads)) * head_dim
                      : v + (s * num_kv_heads + (h - num_q_heads - num_kv_heads)) * head_dim;
       for (int d = 0; d < head_dim; ++d) {
-        if (h >= num_q_heads + num_kv_heads || !(apply_rope > 0)) {
+        if (h >= num_q_heads + num_kv_heads || !(apply_rope > 0) || d >= R) {
           dst[d] = x[d];
           continue;
         }

@@ -41,6 +41,32 @@ def test_fused_rope(d, hq, hkv, apply_rope):
     assert exact > 0.99, f"only {exact:.4f} of the rotated q elements are bit-identical to the oracle"
 
 
+@pytest.mark.parametrize("rope_scaling", [
+    {"rope_type": "default", "rotary_dim": 32}, {"rope_type": "default", "rotary_dim": 40},
+    {"rope_type": "llama3", "rotary_dim": 64, "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+     "original_max_position_embeddings": 8192},
+    {"rope_type": "yarn", "rotary_dim": 64, "factor": 40.0, "beta_fast": 32, "beta_slow": 1,
+     "original_max_position_embeddings": 4096}])
+@pytest.mark.parametrize("d", [128, 64])
+def test_fused_rope_partial_rotation(d, rope_scaling):
+    """rotary_dim < head_dim: only the first features rotate (position_embedding.py:507-520), with any
+    frequency variant; the rest of q and k, and v, pass through bit for bit."""
+    rng = np.random.default_rng(91)
+    hq, hkv = 8, 2
+    r = rope_scaling["rotary_dim"]
+    pos = np.array([0, 1, 2, 3, 100, 511, 2047, 4096, 65535, 7, 9, 33], np.int32)
+    n = len(pos)
+    qkv = rng.standard_normal((n, hq + 2 * hkv, d)).astype(F16)
+    eq, ek, ev = np.zeros((n, hq, d), F16), np.zeros((n, hkv, d), F16), np.zeros((n, hkv, d), F16)
+    ok.fused_rope_scaled(qkv, pos, eq, ek, ev, 1, rope_scaling)
+    q, k, v = (torch.full(a.shape, 7.0, dtype=torch.float16, device=DEV) for a in (eq, ek, ev))
+    K.fused_rope_scaled(dev(qkv), i32(pos), q, k, v, 1, rope_scaling)
+    assert np.array_equal(host(v), ev)
+    assert np.array_equal(host(q)[..., r:], qkv[:, :hq, r:]) and np.array_equal(host(k)[..., r:], qkv[:, hq:hq + hkv, r:])
+    assert_close(host(q), eq, atol=1e-3, rtol=2e-3, what="partial rope q")
+    assert_close(host(k), ek, atol=1e-3, rtol=2e-3, what="partial rope k")
+
+
 def test_fused_rope_append_equals_rope_then_append():
     """One launch for split + RoPE + append: bit-identical q, k, v and pages to the two kernels."""
     rng = np.random.default_rng(42)

@@ -618,6 +618,29 @@ def test_rope_variants_reduce_to_default():
     assert np.array_equal(q, qkv[:, :hq]) and np.array_equal(k, qkv[:, hq:hq + hkv])
 
 
+@pytest.mark.parametrize("d,rotary_dim", [(128, 32), (128, 64), (64, 16), (128, 40), (128, 128)])
+def test_partial_rotation_is_the_closed_form_on_the_first_features(d, rotary_dim):
+    """rotary_dim < head_dim (python/tvm/relax/frontend/nn/llm/position_embedding.py:507-520): the first
+    rotary_dim features rotate as a head of that width would (the reference test's closed form on that slice,
+    pairs (i, i + rotary_dim/2), frequencies over rotary_dim), the others pass through bit for bit."""
+    rng = np.random.default_rng(90 + rotary_dim)
+    hq, hkv = 4, 2
+    pos = np.array([0, 1, 17, 511, 2047, 4096], np.int32)
+    n = len(pos)
+    qkv = rng.standard_normal((n, hq + 2 * hkv, d)).astype(F16)
+    q, k, v = np.zeros((n, hq, d), F16), np.zeros((n, hkv, d), F16), np.zeros((n, hkv, d), F16)
+    ok.fused_rope_scaled(qkv, pos, q, k, v, 1, {"rope_type": "default", "rotary_dim": rotary_dim})
+    assert np.array_equal(v, qkv[:, hq + hkv:])
+    for got, src in ((q, qkv[:, :hq]), (k, qkv[:, hq:hq + hkv])):
+        assert np.array_equal(got[..., rotary_dim:], src[..., rotary_dim:])
+        want = cf.apply_rotary(src[..., :rotary_dim], pos)
+        assert_close(got[..., :rotary_dim], want, atol=2e-3, rtol=2e-3, what=f"partial rotation, {rotary_dim} of {d}")
+    if rotary_dim == d:  # the whole head: the plain kernel, bit for bit
+        q2, k2, v2 = np.zeros_like(q), np.zeros_like(k), np.zeros_like(v)
+        ok.fused_rope(qkv, pos, q2, k2, v2, 1)
+        assert np.array_equal(q, q2) and np.array_equal(k, k2)
+
+
 def test_longrope_factors_and_magnitude():
     """The angle is the default one over the factor of the dimension; cos and sin carry
     sqrt(1 + ln(max/orig)/ln(orig)); the long factors apply only to calls with more rows than orig."""

@@ -43,15 +43,17 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
                                                          const float* __restrict__ ext_factors,
                                                          half_t* __restrict__ pages,
                                                          const int32_t* __restrict__ append_position_map,
-                                                         int page_size) {
+                                                         int page_size, int rotary_dim) {
   constexpr int kThreadsPerHead = D / 16;  // a thread owns d-range [8c, 8c+8) and its partner +D/2
-  __shared__ float cs_lds[D];  // [0, D/2): for the elements of the lower half, [D/2, D): of the upper half
+  // element d < R = rotary_dim: [0, R/2) for the elements of the lower half, [R/2, R) of the upper half
+  __shared__ float cs_lds[D];
   __shared__ float sn_lds[D];
+  const int R = rotary_dim;
   const int64_t s = blockIdx.x;  // token
   const int fused_heads = num_q_heads + 2 * num_kv_heads;
   if (apply_rope > 0) {
     const float pos_scaled = static_cast<float>(position_map[s]) * scale;
-    for (int i = threadIdx.x; i < (halves_differ ? D : D / 2); i += 256) {
+    for (int i = threadIdx.x; i < (halves_differ ? R : R / 2); i += 256) {
       // default / longrope: position over a divisor (times the model's per-dimension factor, if any);
       // llama3 / yarn: position times an inverse frequency (position_embedding.py:130-255)
       float freq;
@@ -64,8 +66,8 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
       cs_lds[i] = cs;
       sn_lds[i] = sn;
       if (!halves_differ) {
-        cs_lds[i + D / 2] = cs;
-        sn_lds[i + D / 2] = sn;
+        cs_lds[i + R / 2] = cs;
+        sn_lds[i + R / 2] = sn;
       }
     }
     __syncthreads();
@@ -86,7 +88,27 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
     } else {
       dst = v + (s * num_kv_heads + (h - num_q_heads - num_kv_heads)) * D;
     }
-    if (apply_rope > 0 && h < num_q_heads + num_kv_heads) {
+    if (apply_rope > 0 && h < num_q_heads + num_kv_heads && R < D) {
+      // only the first R features rotate, in pairs (d, d + R/2) that are no longer this thread's two
+      // vectors (python/tvm/relax/frontend/nn/llm/position_embedding.py:507-520): element by element, the
+      // partner read from the input row
+      const half_t* row = qkv + (s * fused_heads + h) * D;
+      Vec16 out_lo = lo, out_hi = hi;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int dl = c * 8 + e, dh = D / 2 + c * 8 + e;
+        if (dl < R) {
+          const float other = dl < R / 2 ? -static_cast<float>(row[dl + R / 2]) : static_cast<float>(row[dl - R / 2]);
+          out_lo.h[e] = static_cast<half_t>(cs_lds[dl] * static_cast<float>(lo.h[e]) + sn_lds[dl] * other);
+        }
+        if (dh < R) {
+          const float other = dh < R / 2 ? -static_cast<float>(row[dh + R / 2]) : static_cast<float>(row[dh - R / 2]);
+          out_hi.h[e] = static_cast<half_t>(cs_lds[dh] * static_cast<float>(hi.h[e]) + sn_lds[dh] * other);
+        }
+      }
+      lo = out_lo;
+      hi = out_hi;
+    } else if (apply_rope > 0 && h < num_q_heads + num_kv_heads) {
       Vec16 out_lo, out_hi;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -430,11 +452,14 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
     KV_CHECK(append_position_map != nullptr && page_size > 0) << "fused_rope_append: NULL position map or bad page size";
     KV_CHECK(num_pages * page_size <= INT32_MAX) << "fused_rope_append: slot ids do not fit int32";
   }
+  const int rotary_dim = scaling != nullptr && scaling->rotary_dim > 0 ? scaling->rotary_dim : head_dim;
+  KV_CHECK(rotary_dim % 2 == 0 && rotary_dim <= head_dim)
+      << "fused_rope: rotary_dim " << rotary_dim << " must be even and at most head_dim " << head_dim;
   RopeDivisors div;
   float magnitude = 1.0f;
   bool halves_differ = false;
   const bool table_is_inverse =
-      rope_table(scaling, head_dim, rope_theta, seq_len, &ext_factors, &div, &magnitude, &halves_differ);
+      rope_table(scaling, rotary_dim, rope_theta, seq_len, &ext_factors, &div, &magnitude, &halves_differ);
   KV_CHECK(seq_len < (int64_t{1} << 31)) << "fused_rope: too many tokens for one launch";
   const float scale = static_cast<float>(rope_scale);
   auto launch = [&](auto kernel) {
@@ -443,7 +468,7 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
                        seq_len, num_q_heads, num_kv_heads, static_cast<int>(apply_rope > 0), scale, div,
                        static_cast<int>(table_is_inverse), static_cast<int>(halves_differ), magnitude, ext_factors,
                        static_cast<half_t*>(pages),
-                       append_position_map, page_size);
+                       append_position_map, page_size, rotary_dim);
   };
   if (head_dim == 64) {
     if (append) launch(fused_rope_kernel<64, true>); else launch(fused_rope_kernel<64, false>);

@@ -408,10 +408,14 @@ class PagedKVCache {
     compute_stream_ = stream;
   }
   void SetRopeScaling(const tvmkv_rope_scaling* scaling, const float* rope_ext_factors) {
-    has_rope_scaling_ = scaling != nullptr && scaling->rope_type != TVMKV_ROPE_FREQ_DEFAULT;
+    // a description that differs from the default rotation: another frequency rule, or only part of the head rotated
+    has_rope_scaling_ = scaling != nullptr && (scaling->rope_type != TVMKV_ROPE_FREQ_DEFAULT ||
+                                               (scaling->rotary_dim > 0 && scaling->rotary_dim != qk_head_dim_));
     KV_UNSUPPORTED(has_rope_scaling_ && rope_mode_ == TVMKV_ROPE_INLINE)
-        << "RoPE scaling variants are not built for caches that rotate inside the attention kernels (inline RoPE)";
-    KV_CHECK(has_rope_scaling_ || rope_ext_factors == nullptr) << "rope_ext_factors needs a longrope scaling description";
+        << "RoPE scaling variants and partial rotation are not built for caches that rotate inside the attention "
+           "kernels (inline RoPE)";
+    KV_CHECK((scaling != nullptr && scaling->rope_type == TVMKV_ROPE_FREQ_LONGROPE) || rope_ext_factors == nullptr)
+        << "rope_ext_factors needs a longrope scaling description";
     if (has_rope_scaling_) rope_scaling_ = *scaling;
     rope_ext_factors_ = rope_ext_factors;
   }

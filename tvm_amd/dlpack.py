@@ -29,7 +29,7 @@ class DLTensor(ctypes.Structure):
 
 class RopeScaling(ctypes.Structure):
     """struct tvmkv_rope_scaling of include/tvmkv.h."""
-    _fields_ = [("rope_type", ctypes.c_int32), ("reserved", ctypes.c_int32), ("factor", ctypes.c_double),
+    _fields_ = [("rope_type", ctypes.c_int32), ("rotary_dim", ctypes.c_int32), ("factor", ctypes.c_double),
                 ("low_freq_factor", ctypes.c_double), ("high_freq_factor", ctypes.c_double),
                 ("beta_fast", ctypes.c_double), ("beta_slow", ctypes.c_double),
                 ("max_position_embeddings", ctypes.c_int64), ("original_max_position_embeddings", ctypes.c_int64)]
@@ -41,7 +41,7 @@ class RopeScaling(ctypes.Structure):
         """From the reference's ``rope_scaling`` dictionary (position_embedding.py:258-299)."""
         out = cls()
         out.rope_type = cls.TYPES[rope_scaling.get("rope_type", "default")]
-        for key in ("factor", "low_freq_factor", "high_freq_factor", "beta_fast", "beta_slow",
+        for key in ("rotary_dim", "factor", "low_freq_factor", "high_freq_factor", "beta_fast", "beta_slow",
                     "max_position_embeddings", "original_max_position_embeddings"):
             if key in rope_scaling:
                 setattr(out, key, rope_scaling[key])
