@@ -166,7 +166,7 @@ void orc_fused_rope(const f16* qkv, const int32_t* position_map, f16* q, f16* k,
  * between); yarn against the published formula with its rounding removed and, for factor = 1,
  * against default; longrope with unit factors and max = orig against default, bit for bit. */
 typedef struct {
-  int32_t rope_type; /* 0 default, 1 llama3, 2 longrope, 3 yarn */
+  int32_t rope_type; /* 0 default, 1 llama3, 2 longrope, 3 yarn, 4 gptj */
   int32_t rotary_dim; /* 0 = head_dim */
   double factor, low_freq_factor, high_freq_factor, beta_fast, beta_slow;
   int64_t max_position_embeddings, original_max_position_embeddings;
@@ -178,6 +178,7 @@ float orc_rope_angle(const orc_rope_scaling* sc, float s, int d, int R, float th
   float power = powf(theta, (float)((d * 2) % R) / (float)R);
   *magnitude = 1.0f;
   if (sc == NULL || sc->rope_type == 0) return s / power;
+  if (sc->rope_type == 4) return s / powf(theta, (float)((2 * (d / 2)) % R) / (float)R); /* rope_freq_gptj, :70-76 */
   if (sc->rope_type == 1) {
     float orig = 1.0f / power;
     double inv_diff = 1.0 / (sc->high_freq_factor - sc->low_freq_factor);
@@ -233,6 +234,7 @@ void orc_fused_rope_scaled(const f16* qkv, const int32_t* position_map, f16* q, 
         float freq = orc_rope_angle(sc, (float)position_map[s] * scale, d, R, theta, ext, &magnitude);
         float c = (cosf(freq) * magnitude) * h2f(x[d]);
         f16 other = d < R / 2 ? (f16)(x[d + R / 2] ^ 0x8000u) : x[d - R / 2];
+        if (sc != NULL && sc->rope_type == 4) other = d % 2 == 0 ? (f16)(x[d + 1] ^ 0x8000u) : x[d - 1]; /* :509-514 */
         float sn = (sinf(freq) * magnitude) * h2f(other);
         dst[d] = f2h(c + sn);
       }

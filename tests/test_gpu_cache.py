@@ -129,6 +129,7 @@ def test_short_chunk_against_a_long_cached_sequence():
     dict(rope_scaling={"rope_type": "yarn", "factor": 40.0, "beta_fast": 32, "beta_slow": 1,
                        "original_max_position_embeddings": 4096}),
     dict(rope_scaling={"rope_type": "default", "rotary_dim": 32}),
+    dict(rope_scaling={"rope_type": "gptj", "rotary_dim": 64}),
     dict(rope_scaling={"rope_type": "longrope", "max_position_embeddings": 131072, "original_max_position_embeddings": 64},
          rope_ext_factors=np.concatenate([np.linspace(1.0, 8.0, 64), np.linspace(1.0, 1.3, 64)]).astype(np.float32)),
 ])

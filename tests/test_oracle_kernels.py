@@ -635,10 +635,33 @@ def test_partial_rotation_is_the_closed_form_on_the_first_features(d, rotary_dim
         assert np.array_equal(got[..., rotary_dim:], src[..., rotary_dim:])
         want = cf.apply_rotary(src[..., :rotary_dim], pos)
         assert_close(got[..., :rotary_dim], want, atol=2e-3, rtol=2e-3, what=f"partial rotation, {rotary_dim} of {d}")
-    if rotary_dim == d:  # the whole head: the plain kernel, bit for bit
+    if rotary_dim == d:  # the whole head: the plain kernel (to one fp16 ulp: the two loops round in different places)
         q2, k2, v2 = np.zeros_like(q), np.zeros_like(k), np.zeros_like(v)
         ok.fused_rope(qkv, pos, q2, k2, v2, 1)
-        assert np.array_equal(q, q2) and np.array_equal(k, k2)
+        assert_close(q, q2, atol=1e-3, rtol=1e-3, what="whole-head rotary_dim q")
+        assert_close(k, k2, atol=1e-3, rtol=1e-3, what="whole-head rotary_dim k")
+
+
+@pytest.mark.parametrize("d,rotary_dim", [(128, 128), (128, 64), (64, 32)])
+def test_gptj_pairing_is_the_default_rotation_of_the_deinterleaved_head(d, rotary_dim):
+    """rope_type gptj (position_embedding.py:70-76, 509-514) rotates the pairs (2i, 2i + 1) at the frequency the
+    default rule gives pair i: moving the even features to the front and the odd ones behind them turns it into
+    the default rotation, so the reference test's closed form on the permuted slice pins it."""
+    rng = np.random.default_rng(95 + rotary_dim)
+    hq, hkv = 4, 2
+    pos = np.array([0, 1, 17, 511, 2047, 4096], np.int32)
+    n = len(pos)
+    qkv = rng.standard_normal((n, hq + 2 * hkv, d)).astype(F16)
+    q, k, v = np.zeros((n, hq, d), F16), np.zeros((n, hkv, d), F16), np.zeros((n, hkv, d), F16)
+    ok.fused_rope_scaled(qkv, pos, q, k, v, 1, {"rope_type": "gptj", "rotary_dim": rotary_dim})
+    assert np.array_equal(v, qkv[:, hq + hkv:])
+    for got, src in ((q, qkv[:, :hq]), (k, qkv[:, hq:hq + hkv])):
+        assert np.array_equal(got[..., rotary_dim:], src[..., rotary_dim:])
+        part = src[..., :rotary_dim]
+        rotated = cf.apply_rotary(np.concatenate([part[..., 0::2], part[..., 1::2]], axis=-1), pos)
+        want = np.empty_like(rotated)
+        want[..., 0::2], want[..., 1::2] = rotated[..., :rotary_dim // 2], rotated[..., rotary_dim // 2:]
+        assert_close(got[..., :rotary_dim], want, atol=2e-3, rtol=2e-3, what=f"gptj rotation, {rotary_dim} of {d}")
 
 
 def test_longrope_factors_and_magnitude():

@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
                                                          const float* __restrict__ ext_factors,
                                                          half_t* __restrict__ pages,
                                                          const int32_t* __restrict__ append_position_map,
-                                                         int page_size, int rotary_dim) {
+                                                         int page_size, int rotary_dim, int interleaved) {
   constexpr int kThreadsPerHead = D / 16;  // a thread owns d-range [8c, 8c+8) and its partner +D/2
   // element d < R = rotary_dim: [0, R/2) for the elements of the lower half, [R/2, R) of the upper half
   __shared__ float cs_lds[D];
@@ -88,7 +88,24 @@ __global__ __launch_bounds__(256) void fused_rope_kernel(const half_t* __restric
     } else {
       dst = v + (s * num_kv_heads + (h - num_q_heads - num_kv_heads)) * D;
     }
-    if (apply_rope > 0 && h < num_q_heads + num_kv_heads && R < D) {
+    if (apply_rope > 0 && h < num_q_heads + num_kv_heads && interleaved) {
+      // gptj pairing (position_embedding.py:509-514): element 2i rotates with 2i + 1, both in one vector
+      Vec16 out_lo = lo, out_hi = hi;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int dl = c * 8 + e, dh = D / 2 + c * 8 + e;
+        if (dl < R) {
+          const float other = (e & 1) == 0 ? -static_cast<float>(lo.h[e + 1]) : static_cast<float>(lo.h[e - 1]);
+          out_lo.h[e] = static_cast<half_t>(cs_lds[dl] * static_cast<float>(lo.h[e]) + sn_lds[dl] * other);
+        }
+        if (dh < R) {
+          const float other = (e & 1) == 0 ? -static_cast<float>(hi.h[e + 1]) : static_cast<float>(hi.h[e - 1]);
+          out_hi.h[e] = static_cast<half_t>(cs_lds[dh] * static_cast<float>(hi.h[e]) + sn_lds[dh] * other);
+        }
+      }
+      lo = out_lo;
+      hi = out_hi;
+    } else if (apply_rope > 0 && h < num_q_heads + num_kv_heads && R < D) {
       // only the first R features rotate, in pairs (d, d + R/2) that are no longer this thread's two
       // vectors (python/tvm/relax/frontend/nn/llm/position_embedding.py:507-520): element by element, the
       // partner read from the input row
@@ -379,6 +396,12 @@ static bool rope_table(const tvmkv_rope_scaling* scaling, int head_dim, double r
   const float d_range = static_cast<float>(head_dim);
   *magnitude = 1.0f;
   auto power = [&](int i) { return powf(theta, static_cast<float>((i * 2) % head_dim) / d_range); };
+  if (type == TVMKV_ROPE_FREQ_GPTJ) {  // element d rotates at the frequency of its pair d / 2: one entry per element
+    KV_CHECK(*ext_factors == nullptr) << "fused_rope: rope_ext_factors needs a longrope scaling description";
+    *halves_differ = true;
+    for (int d = 0; d < head_dim; ++d) table->v[d] = powf(theta, static_cast<float>((2 * (d / 2)) % head_dim) / d_range);
+    return false;
+  }
   if (type == TVMKV_ROPE_FREQ_DEFAULT || type == TVMKV_ROPE_FREQ_LONGROPE) {
     for (int i = 0; i < head_dim / 2; ++i) table->v[i] = power(i);
     if (type == TVMKV_ROPE_FREQ_LONGROPE) {
@@ -413,7 +436,7 @@ static bool rope_table(const tvmkv_rope_scaling* scaling, int head_dim, double r
     return true;
   }
   KV_UNSUPPORTED(type != TVMKV_ROPE_FREQ_YARN)
-      << "fused_rope: rope type " << type << " is not built (default, llama3, longrope, yarn)";
+      << "fused_rope: rope type " << type << " is not built (default, llama3, longrope, yarn, gptj)";
   KV_CHECK(scaling->factor != 0 && rope_theta > 1.0) << "fused_rope: yarn scaling needs factor != 0 and theta > 1";
   const double inv_theta_log_scale = 1.0 / (2.0 * std::log(rope_theta));  // kv_cache.py:363-365
   auto correction_dim = [&](double rotations) {
@@ -468,7 +491,8 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
                        seq_len, num_q_heads, num_kv_heads, static_cast<int>(apply_rope > 0), scale, div,
                        static_cast<int>(table_is_inverse), static_cast<int>(halves_differ), magnitude, ext_factors,
                        static_cast<half_t*>(pages),
-                       append_position_map, page_size, rotary_dim);
+                       append_position_map, page_size, rotary_dim,
+                       static_cast<int>(scaling != nullptr && scaling->rope_type == TVMKV_ROPE_FREQ_GPTJ));
   };
   if (head_dim == 64) {
     if (append) launch(fused_rope_kernel<64, true>); else launch(fused_rope_kernel<64, false>);
