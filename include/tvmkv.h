@@ -71,13 +71,15 @@ int tvmkv_fused_rope(const void* qkv, const int32_t* position_map, void* q, void
  * per-dimension factor tensor, cos and sin scaled by sqrt(1 + ln(max / original_max) / ln(original_max)).
  * YARN (:191-255): interpolated / extrapolated inverse frequencies blended over the dimensions between
  * the correction dims of beta_fast and beta_slow.  Rotation is over the first rotary_dim features of a head
- * (the whole head by default), with the rotate-half pairing or, for GPTJ, in interleaved pairs; llama4 is not built. */
+ * (the whole head by default), with the rotate-half pairing or, for GPTJ, in interleaved pairs. */
 enum {
   TVMKV_ROPE_FREQ_DEFAULT = 0,
   TVMKV_ROPE_FREQ_LLAMA3 = 1,
   TVMKV_ROPE_FREQ_LONGROPE = 2,
   TVMKV_ROPE_FREQ_YARN = 3,
-  TVMKV_ROPE_FREQ_GPTJ = 4 /* :70-76, :509-514: pairs (2i, 2i+1) instead of (i, i + rotary_dim/2), default frequencies */
+  TVMKV_ROPE_FREQ_GPTJ = 4, /* :70-76, :509-514: pairs (2i, 2i+1) instead of (i, i + rotary_dim/2), default frequencies */
+  TVMKV_ROPE_FREQ_LLAMA4 = 5 /* :79-127: the llama3 smoothing (or, with equal low and high factors, a hard threshold on
+                                the wavelength) on the frequency of pair d / 2, rotate-half pairing; same fields as LLAMA3 */
 };
 typedef struct tvmkv_rope_scaling {
   int32_t rope_type;

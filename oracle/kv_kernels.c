@@ -166,7 +166,7 @@ void orc_fused_rope(const f16* qkv, const int32_t* position_map, f16* q, f16* k,
  * between); yarn against the published formula with its rounding removed and, for factor = 1,
  * against default; longrope with unit factors and max = orig against default, bit for bit. */
 typedef struct {
-  int32_t rope_type; /* 0 default, 1 llama3, 2 longrope, 3 yarn, 4 gptj */
+  int32_t rope_type; /* 0 default, 1 llama3, 2 longrope, 3 yarn, 4 gptj, 5 llama4 */
   int32_t rotary_dim; /* 0 = head_dim */
   double factor, low_freq_factor, high_freq_factor, beta_fast, beta_slow;
   int64_t max_position_embeddings, original_max_position_embeddings;
@@ -179,6 +179,20 @@ float orc_rope_angle(const orc_rope_scaling* sc, float s, int d, int R, float th
   *magnitude = 1.0f;
   if (sc == NULL || sc->rope_type == 0) return s / power;
   if (sc->rope_type == 4) return s / powf(theta, (float)((2 * (d / 2)) % R) / (float)R); /* rope_freq_gptj, :70-76 */
+  if (sc->rope_type == 5) { /* rope_freq_llama4, :79-127 */
+    float orig = 1.0f / powf(theta, (float)(2 * (d / 2)) / (float)R);
+    if (sc->high_freq_factor == sc->low_freq_factor) {
+      float wavelength = (float)(2 * M_PI) / orig;
+      float threshold = (float)((double)sc->original_max_position_embeddings / sc->low_freq_factor);
+      return s * (wavelength > threshold ? orig / (float)sc->factor : orig);
+    }
+    double inv_diff = 1.0 / (sc->high_freq_factor - sc->low_freq_factor);
+    float inv_factor = (float)(1.0 / sc->factor);
+    float alpha = (float)((double)sc->original_max_position_embeddings / (2 * M_PI) * inv_diff);
+    float beta = (float)(sc->low_freq_factor * inv_diff);
+    float smooth = fmaxf(0.0f, fminf(1.0f, alpha * orig - beta));
+    return s * ((1.0f - smooth) * orig * inv_factor + smooth * orig);
+  }
   if (sc->rope_type == 1) {
     float orig = 1.0f / power;
     double inv_diff = 1.0 / (sc->high_freq_factor - sc->low_freq_factor);

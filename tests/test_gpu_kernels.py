@@ -44,6 +44,10 @@ def test_fused_rope(d, hq, hkv, apply_rope):
 @pytest.mark.parametrize("rope_scaling", [
     {"rope_type": "default", "rotary_dim": 32}, {"rope_type": "default", "rotary_dim": 40},
     {"rope_type": "gptj", "rotary_dim": 64}, {"rope_type": "gptj", "rotary_dim": 32},
+    {"rope_type": "llama4", "rotary_dim": 64, "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+     "original_max_position_embeddings": 8192},
+    {"rope_type": "llama4", "rotary_dim": 64, "factor": 16.0, "low_freq_factor": 1.0, "high_freq_factor": 1.0,
+     "original_max_position_embeddings": 8192},
     {"rope_type": "llama3", "rotary_dim": 64, "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
      "original_max_position_embeddings": 8192},
     {"rope_type": "yarn", "rotary_dim": 64, "factor": 40.0, "beta_fast": 32, "beta_slow": 1,

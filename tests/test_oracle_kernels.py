@@ -664,6 +664,28 @@ def test_gptj_pairing_is_the_default_rotation_of_the_deinterleaved_head(d, rotar
         assert_close(got[..., :rotary_dim], want, atol=2e-3, rtol=2e-3, what=f"gptj rotation, {rotary_dim} of {d}")
 
 
+def test_llama4_is_the_llama3_rule_on_the_frequency_of_pair_d_over_2():
+    """rope_freq_llama4 (position_embedding.py:79-127) smooths like llama3 but takes the frequency of pair d // 2
+    (no wrap at the half): element d gets the angle llama3 gives element d // 2.  With equal low and high factors it
+    is a hard threshold on the wavelength: frequencies whose wavelength exceeds original_max / low_freq_factor are
+    divided by the factor, the others kept."""
+    theta, r = 5e5, 128
+    sc = {"rope_type": "llama4", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+          "original_max_position_embeddings": 8192}
+    l3 = dict(sc, rope_type="llama3")
+    for d in range(r):
+        a4, m4 = ok.rope_angle(sc, 1234.0, d, r, theta)
+        a3, _ = ok.rope_angle(l3, 1234.0, d // 2, r, theta)
+        assert m4 == 1.0 and a4 == a3, d
+    hard = dict(sc, high_freq_factor=1.0)
+    for d in range(r):
+        orig = np.float32(1.0) / np.float32(theta) ** (np.float32(2 * (d // 2)) / np.float32(r))
+        wavelength = 2 * np.pi / orig
+        a, _ = ok.rope_angle(hard, 100.0, d, r, theta)
+        want = 100.0 * (orig / 8.0 if wavelength > 8192 else orig)
+        assert abs(a - want) <= 1e-5 * abs(want), d
+
+
 def test_longrope_factors_and_magnitude():
     """The angle is the default one over the factor of the dimension; cos and sin carry
     sqrt(1 + ln(max/orig)/ln(orig)); the long factors apply only to calls with more rows than orig."""

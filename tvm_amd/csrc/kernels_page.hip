@@ -402,6 +402,28 @@ static bool rope_table(const tvmkv_rope_scaling* scaling, int head_dim, double r
     for (int d = 0; d < head_dim; ++d) table->v[d] = powf(theta, static_cast<float>((2 * (d / 2)) % head_dim) / d_range);
     return false;
   }
+  if (type == TVMKV_ROPE_FREQ_LLAMA4) {  // position_embedding.py:79-127: one inverse frequency per element, of pair d / 2
+    KV_CHECK(*ext_factors == nullptr) << "fused_rope: rope_ext_factors needs a longrope scaling description";
+    KV_CHECK(scaling->factor != 0 && scaling->low_freq_factor != 0) << "fused_rope: llama4 scaling needs factor != 0 and low_freq_factor != 0";
+    *halves_differ = true;
+    const bool hard = scaling->high_freq_factor == scaling->low_freq_factor;
+    const double inv_diff = hard ? 0.0 : 1.0 / (scaling->high_freq_factor - scaling->low_freq_factor);
+    const float inv_factor = static_cast<float>(1.0 / scaling->factor);
+    const float alpha = static_cast<float>(static_cast<double>(scaling->original_max_position_embeddings) / (2 * M_PI) * inv_diff);
+    const float beta = static_cast<float>(scaling->low_freq_factor * inv_diff);
+    const float threshold = static_cast<float>(static_cast<double>(scaling->original_max_position_embeddings) / scaling->low_freq_factor);
+    for (int d = 0; d < head_dim; ++d) {
+      const float orig = 1.0f / powf(theta, static_cast<float>(2 * (d / 2)) / d_range);
+      if (hard) {
+        const float wavelength = static_cast<float>(2 * M_PI) / orig;
+        table->v[d] = wavelength > threshold ? orig / static_cast<float>(scaling->factor) : orig;
+      } else {
+        const float smooth = fmaxf(0.0f, fminf(1.0f, alpha * orig - beta));
+        table->v[d] = (1.0f - smooth) * orig * inv_factor + smooth * orig;
+      }
+    }
+    return true;
+  }
   if (type == TVMKV_ROPE_FREQ_DEFAULT || type == TVMKV_ROPE_FREQ_LONGROPE) {
     for (int i = 0; i < head_dim / 2; ++i) table->v[i] = power(i);
     if (type == TVMKV_ROPE_FREQ_LONGROPE) {
@@ -436,7 +458,7 @@ static bool rope_table(const tvmkv_rope_scaling* scaling, int head_dim, double r
     return true;
   }
   KV_UNSUPPORTED(type != TVMKV_ROPE_FREQ_YARN)
-      << "fused_rope: rope type " << type << " is not built (default, llama3, longrope, yarn, gptj)";
+      << "fused_rope: rope type " << type << " is not built (default, llama3, longrope, yarn, gptj, llama4)";
   KV_CHECK(scaling->factor != 0 && rope_theta > 1.0) << "fused_rope: yarn scaling needs factor != 0 and theta > 1";
   const double inv_theta_log_scale = 1.0 / (2.0 * std::log(rope_theta));  // kv_cache.py:363-365
   auto correction_dim = [&](double rotations) {

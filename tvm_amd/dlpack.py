@@ -34,7 +34,7 @@ class RopeScaling(ctypes.Structure):
                 ("beta_fast", ctypes.c_double), ("beta_slow", ctypes.c_double),
                 ("max_position_embeddings", ctypes.c_int64), ("original_max_position_embeddings", ctypes.c_int64)]
 
-    TYPES = {"default": 0, "llama3": 1, "longrope": 2, "yarn": 3, "gptj": 4}
+    TYPES = {"default": 0, "llama3": 1, "longrope": 2, "yarn": 3, "gptj": 4, "llama4": 5}
 
     @classmethod
     def from_dict(cls, rope_scaling):
