@@ -105,6 +105,21 @@ def test_mla_decode_batch_beyond_one_split_launch():
     assert not go[0].any() and np.all(gl[0] == np.float32(-5e4))
 
 
+@pytest.mark.parametrize("causal", [1, 0])
+def test_mla_draft_verification_beyond_one_split_launch(causal):
+    """60 long sequences with 1 to 5 tokens each, about 190 tokens: more one-token sequences than one split
+    launch plans, so the call is cut into parts of consecutive tokens (sequences straddle the parts)."""
+    rng = np.random.default_rng(39 + causal)
+    kv_lens = [int(x) for x in rng.integers(1030, 1300, size=60)]
+    q_lens = [int(x) for x in rng.integers(1, 6, size=60)]
+    kv_lens[7], q_lens[7] = 2600, 5
+    go, gl, eo, el = _mla_both(rng, kv_lens, q_lens, 64, npages=8 + sum((n + 63) // 64 for n in kv_lens), causal=causal,
+                               heads=16)
+    assert 128 < sum(q_lens) <= 512
+    assert_close(go, eo, what="mla verify in parts out")
+    assert_close(gl, el, atol=2e-3, rtol=1e-4, what="mla verify in parts lse")
+
+
 def test_mla_as_many_tokens_as_sequences_but_not_a_decode_step():
     """total_q == batch makes the launcher split the KV; sequences that do not have exactly one
     query token must still come out right (they are done unsplit by the workgroups of chunk 0)."""

@@ -65,6 +65,7 @@ struct MlaParams {
   // token is planned as a sequence of its own with one token, batch_size counts the tokens and tokens_of
   // is the number of real sequences behind q_indptr / page_indptr / last_page_len; 0 otherwise
   int tokens_of;
+  int token_base;    // with tokens_of > 0: the launch plans tokens token_base .. token_base + batch_size - 1 of the call
   int min_chunk_tiles;  // split: lower bound of the chunk length
   int row_tiles;     // split: row tiles of a one-token sequence, ceil(h_q / MLA_BM)
   float scale_log2;
@@ -180,10 +181,11 @@ __device__ __forceinline__ MlaSeqInfo mla_seq_info(const MlaParams& p, int b) {
     // token b of the call as a one-token sequence: under the causal mask token j of n sees the first
     // L - n + j + 1 of its sequence's L keys (python/tvm/relax/frontend/nn/llm/_kernel_common.py:130-135),
     // which is plain attention over that many keys
+    const int token = p.token_base + b;
     int lo = 0, hi = p.tokens_of - 1;
     while (lo < hi) {
       const int mid = (lo + hi + 1) >> 1;
-      if (p.q_indptr[mid] <= b) {
+      if (p.q_indptr[mid] <= token) {
         lo = mid;
       } else {
         hi = mid - 1;
@@ -193,10 +195,10 @@ __device__ __forceinline__ MlaSeqInfo mla_seq_info(const MlaParams& p, int b) {
     const int n = p.q_indptr[lo + 1] - first;
     const int npages = p.page_indptr[lo + 1] - p.page_indptr[lo];
     const int len = npages > 0 ? (npages - 1) * p.page_size + p.last_page_len[lo] : 0;
-    s.q_start = b;
+    s.q_start = token;
     s.qo_len = 1;
     s.pbeg = p.page_indptr[lo];
-    s.kv_len = p.causal ? max(0, min(len, len - n + (b - first) + 1)) : len;
+    s.kv_len = p.causal ? max(0, min(len, len - n + (token - first) + 1)) : len;
     s.npages = (s.kv_len + p.page_size - 1) / p.page_size;
     s.cost = (s.kv_len + MLA_BN - 1) / MLA_BN;
   } else if (b < p.batch_size) {
@@ -896,12 +898,13 @@ __global__ __launch_bounds__(256) void mla_merge_kernel(MlaParams p) {
 
 using namespace tvmkv;
 
-extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_indptr, const void* pages,
-                                                const int32_t* page_indptr, const int32_t* page_values,
-                                                const int32_t* length_info, void* output, float* lse,
-                                                int64_t causal, double sm_scale, int32_t batch_size,
-                                                int64_t total_q, int64_t nnz_pages, int64_t num_pages, int32_t h_q,
-                                                int32_t d_latent, int32_t d_rope, int32_t page_size, void* stream) {
+// token_count >= 0: the launch covers the tokens token_base .. token_base + token_count - 1 of the call only, each
+// planned as a one-token sequence (a part of a call that was cut up, see below); -1: the whole call.
+static int mla_entry(const void* q, const int32_t* q_indptr, const void* pages, const int32_t* page_indptr,
+                     const int32_t* page_values, const int32_t* length_info, void* output, float* lse, int64_t causal,
+                     double sm_scale, int32_t batch_size, int64_t total_q, int64_t nnz_pages, int64_t num_pages,
+                     int32_t h_q, int32_t d_latent, int32_t d_rope, int32_t page_size, void* stream, int64_t token_base,
+                     int64_t token_count) {
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0) << "batch_prefill_paged_kv_mla: bad shape";
   KV_UNSUPPORTED(d_latent != 512 || d_rope != 64)
@@ -919,16 +922,32 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
   // order: it is cut into equal parts of at most that many sequences, each a split launch of its own
   // (200 sequences of 2048-8192 tokens: 0.57 ms in one unsplit launch).  The index arrays hold absolute
   // offsets, so a part is the same call on a slice of them.
-  if (total_q == batch_size && batch_size > MLA_MAX_SPLIT_BATCH && batch_size <= 4 * MLA_MAX_SPLIT_BATCH &&
-      static_cast<int64_t>(MLA_MAX_SPLIT_BATCH) * ((h_q + MLA_BM - 1) / MLA_BM) * 2 <= compute_units() &&
-      nnz_pages * page_size / batch_size >= 1024) {
+  const bool parts_fit = static_cast<int64_t>(MLA_MAX_SPLIT_BATCH) * ((h_q + MLA_BM - 1) / MLA_BM) * 2 <= compute_units() &&
+                         nnz_pages > 0 && nnz_pages * page_size < (int64_t{1} << 26) &&
+                         nnz_pages * page_size / batch_size >= 1024;
+  if (token_count < 0 && total_q == batch_size && batch_size > MLA_MAX_SPLIT_BATCH &&
+      batch_size <= 4 * MLA_MAX_SPLIT_BATCH && parts_fit) {
     const int parts = (batch_size + MLA_MAX_SPLIT_BATCH - 1) / MLA_MAX_SPLIT_BATCH;
     for (int i = 0; i < parts; ++i) {
       const int lo = static_cast<int>(static_cast<int64_t>(i) * batch_size / parts);
       const int hi = static_cast<int>(static_cast<int64_t>(i + 1) * batch_size / parts);
-      const int rc = tvmkv_batch_prefill_paged_kv_mla(q, q_indptr + lo, pages, page_indptr + lo, page_values, length_info + lo,
-                                                      output, lse, causal, sm_scale, hi - lo, hi - lo, nnz_pages, num_pages,
-                                                      h_q, d_latent, d_rope, page_size, stream);
+      const int rc = mla_entry(q, q_indptr + lo, pages, page_indptr + lo, page_values, length_info + lo, output, lse,
+                               causal, sm_scale, hi - lo, hi - lo, nnz_pages, num_pages, h_q, d_latent, d_rope, page_size,
+                               stream, 0, -1);
+      if (rc != TVMKV_OK) return rc;
+    }
+    return TVMKV_OK;
+  }
+  // The same for a call with a few tokens per sequence (a draft to verify) and more tokens than one launch plans:
+  // parts of at most that many consecutive tokens, each planned as one-token sequences over the whole index arrays.
+  if (token_count < 0 && total_q != batch_size && total_q > MLA_MAX_SPLIT_BATCH && total_q <= 4 * MLA_MAX_SPLIT_BATCH &&
+      parts_fit) {
+    const int parts = static_cast<int>((total_q + MLA_MAX_SPLIT_BATCH - 1) / MLA_MAX_SPLIT_BATCH);
+    for (int i = 0; i < parts; ++i) {
+      const int64_t lo = i * total_q / parts, hi = (i + 1) * total_q / parts;
+      const int rc = mla_entry(q, q_indptr, pages, page_indptr, page_values, length_info, output, lse, causal, sm_scale,
+                               batch_size, total_q, nnz_pages, num_pages, h_q, d_latent, d_rope, page_size, stream, lo,
+                               hi - lo);
       if (rc != TVMKV_OK) return rc;
     }
     return TVMKV_OK;
@@ -957,11 +976,15 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
   int64_t grid = slots;
   // A call with a few tokens per sequence (a draft to verify, a short chunk late in a long prompt) is in the
   // same position: its tokens are planned as one-token sequences of their own.
-  if (total_q * row_tiles * 2 <= cus && total_q <= MLA_MAX_SPLIT_BATCH && nnz_pages > 0 &&
+  const int64_t planned = token_count >= 0 ? token_count : total_q;
+  KV_CHECK(token_count < 0 || (planned * row_tiles * 2 <= cus && planned <= MLA_MAX_SPLIT_BATCH))
+      << "batch_prefill_paged_kv_mla: a part of a call must fit one split launch";
+  if (planned * row_tiles * 2 <= cus && planned <= MLA_MAX_SPLIT_BATCH && nnz_pages > 0 &&
       nnz_pages * page_size < (int64_t{1} << 26)) {
-    if (total_q != batch_size) {
+    if (token_count >= 0 || total_q != batch_size) {
       p.tokens_of = batch_size;
-      p.batch_size = static_cast<int>(total_q);
+      p.batch_size = static_cast<int>(planned);
+      p.token_base = static_cast<int>(token_base);
     }
     const int64_t cslots = cus / row_tiles;
     p.split = 1;
@@ -1004,4 +1027,14 @@ extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_
     KV_LAUNCH_CHECK();
   }
   KV_API_END();
+}
+
+extern "C" int tvmkv_batch_prefill_paged_kv_mla(const void* q, const int32_t* q_indptr, const void* pages,
+                                                const int32_t* page_indptr, const int32_t* page_values,
+                                                const int32_t* length_info, void* output, float* lse,
+                                                int64_t causal, double sm_scale, int32_t batch_size,
+                                                int64_t total_q, int64_t nnz_pages, int64_t num_pages, int32_t h_q,
+                                                int32_t d_latent, int32_t d_rope, int32_t page_size, void* stream) {
+  return mla_entry(q, q_indptr, pages, page_indptr, page_values, length_info, output, lse, causal, sm_scale, batch_size,
+                   total_q, nnz_pages, num_pages, h_q, d_latent, d_rope, page_size, stream, 0, -1);
 }
