@@ -36,9 +36,10 @@ inline void Check(int rc) { TVM_FFI_ICHECK_EQ(rc, 0) << "tvmkv: " << tvmkv_last_
 // reference's kernel (position_embedding.py:444-667), so the kernel function is made per model.
 Function MakeFusedRope(double rope_scale, double rope_theta, int64_t rope_type, double factor, double low_freq_factor,
                        double high_freq_factor, double beta_fast, double beta_slow, int64_t max_position_embeddings,
-                       int64_t original_max_position_embeddings) {
+                       int64_t original_max_position_embeddings, int64_t rotary_dim) {
   tvmkv_rope_scaling scaling{};
   scaling.rope_type = static_cast<int32_t>(rope_type);
+  scaling.rotary_dim = static_cast<int32_t>(rotary_dim);  // 0 = the whole head
   scaling.factor = factor;
   scaling.low_freq_factor = low_freq_factor;
   scaling.high_freq_factor = high_freq_factor;
