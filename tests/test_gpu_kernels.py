@@ -623,6 +623,16 @@ def test_prefill_split_over_the_keys(hq, hkv, d, splits):
                                           i32(last), go, gl, d ** -0.5)
         assert_close(host(go), eo, what=f"one-pass chunked prefill out, {splits} splits")
         assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"one-pass chunked prefill lse, {splits} splits")
+        # the same step as the cache composes it for forked sequences: the ragged kernel's state, then the paged
+        # kernel merged into it (split: the merge kernel folds the caller's state in with the shares)
+        go2 = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+        gl2 = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+        K.batch_prefill_ragged_kv(dev(q), i32(ind), dev(k), dev(v), i32(ind), i32(zq), i32(zb), go2, gl2, 1, 0, 1.0, 1e4,
+                                  d ** -0.5)
+        K.batch_prefill_paged_kv(dev(q), i32(ind), dev(pages), i32(pindptr), i32(pvalues), i32(last), i32(zb), i32(zq), go2,
+                                 gl2, 0, 0, 1.0, 1e4, d ** -0.5, merge_into=True)
+        assert_close(host(go2), eo, what=f"paged merged into ragged out, {splits} splits")
+        assert_close(host(gl2), el, atol=2e-3, rtol=1e-4, what=f"paged merged into ragged lse, {splits} splits")
     finally:
         tvm_amd.set_option("prefill_kv_splits", prev)
 

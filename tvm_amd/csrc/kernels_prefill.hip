@@ -782,7 +782,8 @@ static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const Pr
 template <int DV>
 __global__ __launch_bounds__(256) void prefill_split_merge_kernel(const half_t* __restrict__ part_o,
                                                                   const float* __restrict__ part_lse, half_t* __restrict__ output,
-                                                                  float* __restrict__ lse, int64_t rows, int splits) {
+                                                                  float* __restrict__ lse, int64_t rows, int splits,
+                                                                  int merge_into) {
   constexpr int TPR = DV / 8;  // threads per row, 8 features each
   const int64_t row = static_cast<int64_t>(blockIdx.x) * (256 / TPR) + threadIdx.x / TPR;
   const int piece = threadIdx.x % TPR;
@@ -791,7 +792,20 @@ __global__ __launch_bounds__(256) void prefill_split_merge_kernel(const half_t* 
   for (int i = 0; i < splits; ++i) s_max = fmaxf(s_max, part_lse[i * rows + row]);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float w_sum = 0.f;
-  if (s_max > kNegInit) {
+  const bool any_share = s_max > kNegInit;
+  if (merge_into) {
+    // output / lse already hold a state of the same rows (the launch was asked to merge into it): it is one more
+    // state of the sum; shares that are all empty count as the one empty state (out 0, lse -5e4) an unsplit
+    // launch would have merged
+    const float s_prev = lse[row];
+    s_max = fmaxf(s_max, s_prev);
+    const float w = fast_exp2(s_prev - s_max);
+    const Vec16 v = ld16(output + row * DV + piece * 8);
+    w_sum = w + (any_share ? 0.f : fast_exp2(kNegInit - s_max));
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = w * static_cast<float>(v.h8[e]);
+  }
+  if (any_share) {
     for (int i = 0; i < splits; ++i) {
       const float w = fast_exp2(part_lse[i * rows + row] - s_max);
       const Vec16 v = ld16(part_o + (i * rows + row) * DV + piece * 8);
@@ -843,9 +857,9 @@ struct KvSplit {
   float* lse;
   int64_t rows;
   int splits;
+  int merge_into = 0;
   KvSplit(PrefillParams& p, int64_t total_q, int64_t avg_keys, int dv, hipStream_t stream)
       : output(p.output), lse(p.lse), rows(total_q * p.h_q), splits(1) {
-    if (p.merge_into) return;  // the epilogue merges into the caller's state: one workgroup per row tile
     splits = pick_kv_splits(total_q, p.group, p.batch_size, p.h_kv, avg_keys);
     if (splits <= 1) return;
     const size_t o_bytes = static_cast<size_t>(splits) * rows * dv * sizeof(half_t);
@@ -855,6 +869,8 @@ struct KvSplit {
     p.lse = reinterpret_cast<float*>(ws + o_bytes);
     p.kv_splits = splits;
     p.split_rows = rows;
+    merge_into = p.merge_into;  // the shares write plain states; the merge kernel folds the caller's state in
+    p.merge_into = 0;
   }
   void finish(const PrefillParams& p, int dv, hipStream_t stream) const {
     if (splits <= 1) return;
@@ -862,11 +878,11 @@ struct KvSplit {
     const unsigned rows_per_block = 256 / (dv / 8);
     const dim3 grid(static_cast<unsigned>((rows + rows_per_block - 1) / rows_per_block));
     if (dv == 128) {
-      hipLaunchKernelGGL(prefill_split_merge_kernel<128>, grid, dim3(256), 0, stream, p.output, p.lse, output, lse, rows, splits);
+      hipLaunchKernelGGL(prefill_split_merge_kernel<128>, grid, dim3(256), 0, stream, p.output, p.lse, output, lse, rows, splits, merge_into);
     } else if (dv == 64) {
-      hipLaunchKernelGGL(prefill_split_merge_kernel<64>, grid, dim3(256), 0, stream, p.output, p.lse, output, lse, rows, splits);
+      hipLaunchKernelGGL(prefill_split_merge_kernel<64>, grid, dim3(256), 0, stream, p.output, p.lse, output, lse, rows, splits, merge_into);
     } else {
-      hipLaunchKernelGGL(prefill_split_merge_kernel<256>, grid, dim3(256), 0, stream, p.output, p.lse, output, lse, rows, splits);
+      hipLaunchKernelGGL(prefill_split_merge_kernel<256>, grid, dim3(256), 0, stream, p.output, p.lse, output, lse, rows, splits, merge_into);
     }
   }
 };
