@@ -41,10 +41,11 @@ namespace tvmkv {
 __device__ unsigned long long prefill_clock_counters[4];
 static int g_prefill_clock_probe = 0;
 
-// Pipeline depth: as many stages as fit next to a second workgroup (NW = 4) or alone (NW = 8).
+// Pipeline depth: as many stages as fit next to the other workgroups of the CU (NW = 4: one more, two
+// more at head dim 64, whose kernels need a third of the registers) or alone (NW = 8).
 constexpr int prefill_stages(int dqk, int dv) {
   const int stage_bytes = BN * (dqk + dv) * 2;
-  const int budget = (NW == 8 ? 160 : 80) * 1024;
+  const int budget = (NW == 8 ? 160 : (dqk == 64 ? 53 : 80)) * 1024;
   return budget / stage_bytes >= 4 ? 4 : (budget / stage_bytes >= 3 ? 3 : 2);
 }
 
@@ -70,7 +71,7 @@ constexpr size_t prefill_lds_bytes(int dqk, int dv) {
 // causal mask -- a chunked-prefill step in one pass, on one key axis whose paged part is padded to
 // a whole number of tiles (the padding is masked like the end of a sequence).
 template <int DQK, int DV, int SRC, int PS, bool EXT>
-__global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : 2) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
+__global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 64 ? 3 : 2)) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
   constexpr bool PAGED = SRC == kPaged, BOTH = SRC == kBoth;
   static_assert(!(BOTH && EXT), "the combined pass exists for the plain cache only");
   static_assert(DQK % 64 == 0 && DV % 64 == 0, "feature dims must be multiples of 64");
