@@ -258,7 +258,10 @@ int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t*
  * batch_size) * h_q * (head_dim + 2) * 4 bytes, chunk_pages as tvmkv_decode_split_plan reports
  * (configs of 64 x 8k-token and 8 x 128k-token sequences need 6 and 11 MiB).  All calls on a device
  * share the array: calls that overlap on one device (different streams) race, stream-ordered
- * calls do not. */
+ * calls do not.  A call captured into a graph may be replayed: the workgroup that merges the chunks
+ * of a sequence puts the arrival counter back to zero.  (tvmkv_batch_decode_paged_kv under capture
+ * works on a stream it has been called on before with shapes at least as large; when it would have
+ * to allocate it returns TVMKV_EINVAL and leaves the capture intact.) */
 int tvmkv_batch_decode_paged_kv_noalloc(const void* q, const void* pages, const int32_t* page_indptr,
                                         const int32_t* page_values, const int32_t* length_info,
                                         const int32_t* k_rope_pos_offset,

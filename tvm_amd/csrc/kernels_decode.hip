@@ -504,7 +504,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
   // every wave waits until its own have completed, the barrier collects the waves, one thread
   // counts the workgroup in with a device-scope atomic, and the workgroup that completes the count
   // reads the states with device-scope loads.  The counter carries the launch's epoch in its upper
-  // half: the maximum brings a word of an older launch to (epoch, 0) and leaves this launch's alone.
+  // half: the maximum brings a word of an older launch (one that was abandoned half way, too) to
+  // (epoch, 0) and leaves this launch's alone.
   if (p.arrivals != nullptr && !single_chunk) {
     wait_vmcnt<0>();
     __syncthreads();
@@ -515,6 +516,12 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
       const unsigned long long before =
           __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       sm_last = static_cast<uint32_t>(before) == static_cast<uint32_t>(nchunks - 1);
+      // everyone has arrived: nobody of this launch touches the counter again.  Back to (epoch, 0), so
+      // that a launch with the same arguments (a captured graph that is replayed) counts from zero.
+      if (sm_last) {
+        __hip_atomic_store(counter, static_cast<unsigned long long>(p.epoch) << 32, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
     __syncthreads();
     if (sm_last) {

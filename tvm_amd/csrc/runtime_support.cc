@@ -53,6 +53,16 @@ ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, s
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   Scratch& s = g_scratch[std::make_tuple(dev, stream, static_cast<int>(user))];
   if (s.bytes < bytes || s.counter_bytes < counter_bytes) {
+    // growing means hipMalloc, hipFree and a memset: none of them belongs into a graph under capture
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (stream != nullptr && hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+      (void)hipGetLastError();
+      capture = hipStreamCaptureStatusNone;
+    }
+    KV_CHECK(capture == hipStreamCaptureStatusNone)
+        << "the stream is being captured into a graph and this call needs " << bytes << " bytes of scratch memory that "
+        << "are not allocated yet: run the same call once on this stream before the capture starts, or use "
+        << "tvmkv_batch_decode_paged_kv_noalloc";
     if (s.ptr != nullptr) {
       // launches still queued on this stream read the old buffer; nobody else ever does
       HIP_CHECK(hipStreamSynchronize(stream));
