@@ -252,6 +252,11 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
   constexpr int PPR = D / 8;                // 16-byte pieces per row
   constexpr int RPI = 64 / PPR;             // rows one copy instruction covers
   constexpr int DM_VTILE = 2 * PS * D;      // halfs of a wave's V tile: two pages, row-major
+  // K fragments by whole 128-byte lines (see the main loop); the head dim 64 kernel with inline RoPE
+  // keeps the half-line form, where a feature and its rotation partner lie in one lane
+  constexpr bool KLINE = !(EXT && D == 64);
+  constexpr int TI = KS / 2;                // K load instructions per 8-token tile (KLINE)
+  constexpr int NPAIR = KLINE ? KS / 4 : KS / 2;  // fragment pairs (f, f + D/2) of a K token in one lane
   static_assert(D == 64 || D == 128 || D == 256, "head dim");
   static_assert(DM_VTILE * sizeof(half_t) >= 16 * D * sizeof(float), "the merge buffer aliases the V tile");
   __shared__ __attribute__((aligned(16))) half_t Vt_all[4][DM_VTILE];
@@ -297,11 +302,15 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
   // physical token t is attended to iff t < sink or win_lo <= t < kv_len
   const int sink = EXT && p.sink_size != nullptr ? p.sink_size[b] : 0;
   const int win_lo = EXT && p.window_offset != nullptr ? p.window_offset[b] : 0;
-  float divr[4 * KS];  // RoPE divisors of this lane's features ks*32 + g4*8 + i, ks < KS/2
+  // RoPE divisors of the first halves of this lane's K fragment pairs: features i*32 + g4*8 + e, or
+  // with KLINE i*64 + (c16&1)*32 + g4*8 + e
+  float divr[8 * (NPAIR > 0 ? NPAIR : 1)];
   float k_pos0 = 0.f;
   if (EXT && p.rotary) {
 #pragma unroll
-    for (int i = 0; i < 4 * KS; ++i) divr[i] = div.v[(i >> 3) * 32 + g4 * 8 + (i & 7)];
+    for (int i = 0; i < 8 * NPAIR; ++i) {
+      divr[i] = div.v[KLINE ? (i >> 3) * 64 + (c16 & 1) * 32 + g4 * 8 + (i & 7) : (i >> 3) * 32 + g4 * 8 + (i & 7)];
+    }
     k_pos0 = static_cast<float>(p.k_rope_pos_offset[b]);
   }
 
@@ -316,7 +325,12 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
       // feature f < D/2 rotates with f + D/2: k-step ks with ks + KS/2
       const float q_pos = static_cast<float>(p.q_rope_position[b]) * p.rope_scale;
 #pragma unroll
-      for (int ks = 0; ks < KS / 2; ++ks) rope_pair(qv[ks].h8, qv[ks + KS / 2].h8, q_pos, divr + 8 * ks);
+      for (int ks = 0; ks < KS / 2; ++ks) {
+        float qdiv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qdiv[e] = div.v[ks * 32 + g4 * 8 + e];
+        rope_pair(qv[ks].h8, qv[ks + KS / 2].h8, q_pos, qdiv);
+      }
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[ks] = qv[ks].h8;
@@ -329,15 +343,25 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
   // V^T fragment via the transposing read: lane li of a 16-lane group points at 4 features of token
   // (li >> 2) of the group's 4 tokens and receives feature li of the group's 16 for the 4 tokens
   const uint32_t vt_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)Vt));
-  const int v_row = 4 * g4 + (c16 >> 2);             // + PS for the second page: same swizzle
+  // the 8 contraction slots of lane group g4 are 4 tokens of each page: 4*g4 .. 4*g4+3, or with KLINE
+  // 2*g4, 2*g4+1, 8+2*g4, 8+2*g4+1 (the order in which the score product leaves them in a lane)
+  const int v_row = KLINE ? ((c16 >> 3) & 1) * 8 + 2 * g4 + ((c16 >> 2) & 1)
+                          : 4 * g4 + (c16 >> 2);     // + PS for the second page: same swizzle
   const int v_swz = dm_swizzle<D>(v_row);
   const int v_lane_off = v_row * D + (c16 & 1) * 4;
   const int v_piece = (c16 & 3) >> 1;                // + 2 * feature block
 
-  // One step = pages (pi, pi+1).  K: lane reads row c16 of the page, features ks*32 + g4*8, with
-  // ordinary loads: each request is a quarter of a 256-byte row, and partial rows with the streaming
-  // hint measured 10-15 % less bandwidth than without it (whole rows: 8 % more).  K through LDS
-  // with whole-row copies like V measured slower than this (two workgroups per CU instead of three).
+  // One step = pages (pi, pi+1).  K comes straight from global memory in the MFMA A layout, where lane
+  // (c16, g4) holds 16 bytes of A-row c16.  Were A-row c16 simply token c16, one load instruction would
+  // touch a quarter of 16 rows of 256 bytes, half a 128-byte line each, and partial lines with the
+  // streaming hint measured 10-15 % less bandwidth than without it.  KLINE: an instruction covers 8
+  // tokens x one whole line.  A-rows 2t and 2t+1 are token t's features [0,32) and [32,64) of that
+  // line, so one fragment goes through two MFMAs, one against the q features of the even rows and one
+  // against those of the odd rows (the matrix cores idle at 4 %), and token t's score is row 2t of the
+  // first plus row 2t+1 of the second, both in one lane.  Whole lines take the streaming hint: 0.1965
+  // -> 0.1915 ms on 64 sequences of 1024-8192 tokens; 4 tokens x a whole 256-byte row per instruction
+  // (four MFMAs per fragment) measured the same as this.  K through LDS with whole-row copies like V
+  // measured slower (two workgroups per CU instead of three).
   // V: copy instructions of 1 KiB each (4 rows of head dim 128, 8 of head dim 64) fill the wave's LDS tile; rows at or past
   // kv_len repeat the last cached row of their page and a missing second page repeats the first
   // (their P is 0, and 0 times cached data is 0, whereas unwritten memory could hold NaN patterns).
@@ -362,7 +386,13 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
       }
       if (pi + h < page_hi) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
+        for (int ks = 0; ks < KS; ++ks) {
+          if (KLINE) {  // fragment ks: tile ks / TI (8 tokens), line ks % TI of the row
+            r.k[h][ks] = ld16_nt(kbase + ((ks / TI) * 8 + (c16 >> 1)) * D + (ks % TI) * 64 + (c16 & 1) * 32 + g4 * 8);
+          } else {
+            r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
+          }
+        }
       } else {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) r.k[h][ks] = zero16();
@@ -376,32 +406,52 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
                              : (pi + 2) * PS > kv_len;
     auto attended = [&](int t) { return EXT ? (t < sink || (t >= win_lo && t < kv_len)) : t < kv_len; };
     if (EXT && p.rotary) {
-      // the key of this lane in page h is physical token (pi+h)*PS + c16; logical index = position
+      // the key of this lane in page h is physical token (pi+h)*PS + c16 (KLINE: + 8*tile + c16/2);
+      // logical index = position
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const int t = (pi + h) * PS + c16;
-        const int logical = t < sink ? t : t - win_lo + sink;
-        const float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
 #pragma unroll
-        for (int ks = 0; ks < KS / 2; ++ks) rope_pair(r.k[h][ks].h8, r.k[h][ks + KS / 2].h8, pos, divr + 8 * ks);
+        for (int tile = 0; tile < (KLINE ? 2 : 1); ++tile) {
+          const int t = (pi + h) * PS + (KLINE ? tile * 8 + (c16 >> 1) : c16);
+          const int logical = t < sink ? t : t - win_lo + sink;
+          const float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
+          Vec16* frag = r.k[h] + (KLINE ? tile * TI : 0);
+#pragma unroll
+          for (int i = 0; i < NPAIR; ++i) rope_pair(frag[i].h8, frag[i + NPAIR].h8, pos, divr + 8 * i);
+        }
       }
     }
     // ---- S^T = K Q^T for both pages ---------------------------------------------------------
     float4_t s[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      s[h] = float4_t{0.f, 0.f, 0.f, 0.f};
+      if (KLINE) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) s[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][ks].h8, qf[ks], s[h], 0, 0, 0);
+        for (int tile = 0; tile < 2; ++tile) {
+          float4_t even = float4_t{0.f, 0.f, 0.f, 0.f}, odd = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < TI; ++i) {
+            even = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][tile * TI + i].h8, qf[2 * i], even, 0, 0, 0);
+            odd = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][tile * TI + i].h8, qf[2 * i + 1], odd, 0, 0, 0);
+          }
+          s[h][tile * 2 + 0] = even[0] + odd[1];
+          s[h][tile * 2 + 1] = even[2] + odd[3];
+        }
+      } else {
+        s[h] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][ks].h8, qf[ks], s[h], 0, 0, 0);
+      }
     }
-    // s[h][j]: token (pi+h)*PS + 4*g4 + j, head c16
+    // s[h][j]: token (pi+h)*PS + token_of(j), head c16
+    auto token_of = [&](int j) { return KLINE ? 8 * (j >> 1) + 2 * g4 + (j & 1) : 4 * g4 + j; };
     float mx = kNegInit;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float v = s[h][j] * p.scale_log2;
-        if (partial) v = attended((pi + h) * PS + 4 * g4 + j) ? v : kNegInit;
+        if (partial) v = attended((pi + h) * PS + token_of(j)) ? v : kNegInit;
         s[h][j] = v;
         mx = fmaxf(mx, v);
       }
@@ -423,12 +473,12 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float pj = fast_exp2(s[h][j] - m_new);
-        if (partial) pj = attended((pi + h) * PS + 4 * g4 + j) ? pj : 0.f;
+        if (partial) pj = attended((pi + h) * PS + token_of(j)) ? pj : 0.f;
         lsum += pj;
         pf[h * 4 + j] = static_cast<half_t>(pj);
       }
     }
-    // ---- O^T += V^T P^T: contraction slot g4*8 + i <-> page i/4, token 4*g4 + i%4 ------------
+    // ---- O^T += V^T P^T: contraction slot g4*8 + i <-> page i/4, token token_of(i%4) ----------
     // The tile is written (by the copies) and read by this wave only: the copies are done when
     // vmcnt reaches 0, and the reads below are done before the MFMAs that use them are issued,
     // which is before the next step's copies in program order.
