@@ -22,6 +22,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <mutex>
+#include <type_traits>
 
 #include "kernels_common.cuh"
 #include "runtime_support.h"
@@ -243,7 +244,11 @@ struct DecodeRopeDivisors {
 // inline RoPE (q at q_rope_position[b], the key with logical index t at k_rope_pos_offset[b] + t,
 // _decode_kernels.py:141-156).  Attention does not depend on the order of the keys, so the pages are
 // still walked in physical order; evicted tokens are masked and logical indices only feed RoPE.
-template <bool EXT, int D>
+// REREAD: the group has several blocks of 16 heads, whose work items read the same K/V rows one after
+// the other: those rows are loaded without the streaming hint, so that the L2 keeps them for the next
+// head block (64 sequences, 32 query heads on one kv head: 0.077 against 0.083 ms).  Chosen at run
+// time inside one kernel, the load flavour cost the single-block case 4 %.
+template <bool EXT, int D, bool REREAD>
 __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_kernel(DecodeParams p, int group, int num_items,
                                                              DecodeRopeDivisors div) {
   constexpr int PS = DM_PS;
@@ -381,14 +386,16 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
       for (int i = 0; i < PS / RPI; ++i) {
         const int row = i * RPI + lane / PPR;
         const int piece = (lane % PPR) ^ dm_swizzle<D>(h * PS + row);
-        copy16_to_lds_nt(vbase, static_cast<uint32_t>(min(row, last_row) * (D * 2) + piece * 16),
-                      vt_lds + (h * PS + i * RPI) * (D * 2));
+        const uint32_t src_off = static_cast<uint32_t>(min(row, last_row) * (D * 2) + piece * 16);
+        const uint32_t dst = vt_lds + (h * PS + i * RPI) * (D * 2);
+        if (REREAD) copy16_to_lds(vbase, src_off, dst); else copy16_to_lds_nt(vbase, src_off, dst);
       }
       if (pi + h < page_hi) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           if (KLINE) {  // fragment ks: tile ks / TI (8 tokens), line ks % TI of the row
-            r.k[h][ks] = ld16_nt(kbase + ((ks / TI) * 8 + (c16 >> 1)) * D + (ks % TI) * 64 + (c16 & 1) * 32 + g4 * 8);
+            const half_t* src = kbase + ((ks / TI) * 8 + (c16 >> 1)) * D + (ks % TI) * 64 + (c16 & 1) * 32 + g4 * 8;
+            r.k[h][ks] = REREAD ? ld16(src) : ld16_nt(src);
           } else {
             r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
           }
@@ -696,12 +703,20 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group, static_cast<int>(num_items), div);
   };
+  auto launch_d = [&](auto dim) {
+    constexpr int kD = decltype(dim)::value;
+    if (head_blocks > 1) {
+      if (ext) launch(decode_mfma_kernel<true, kD, true>); else launch(decode_mfma_kernel<false, kD, true>);
+    } else {
+      if (ext) launch(decode_mfma_kernel<true, kD, false>); else launch(decode_mfma_kernel<false, kD, false>);
+    }
+  };
   if (d == 128) {
-    if (ext) launch(decode_mfma_kernel<true, 128>); else launch(decode_mfma_kernel<false, 128>);
+    launch_d(std::integral_constant<int, 128>{});
   } else if (d == 256) {
-    if (ext) launch(decode_mfma_kernel<true, 256>); else launch(decode_mfma_kernel<false, 256>);
+    launch_d(std::integral_constant<int, 256>{});
   } else {
-    if (ext) launch(decode_mfma_kernel<true, 64>); else launch(decode_mfma_kernel<false, 64>);
+    launch_d(std::integral_constant<int, 64>{});
   }
   if (!fused) {
     KV_LAUNCH_CHECK();
