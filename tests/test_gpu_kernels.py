@@ -436,10 +436,16 @@ def _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages, page_size=16):
 
 @pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
 @pytest.mark.parametrize("causal", [0, 1])
-def test_paged_prefill_against_oracle(hq, hkv, d, causal):
+@pytest.mark.parametrize("rows", ["one row tile per sequence", "several row tiles per sequence"])
+def test_paged_prefill_against_oracle(hq, hkv, d, causal, rows):
+    """Both forms of the paged kernel: launches with at most one row tile per sequence and kv head on
+    average copy K/V with the streaming hint, the others without."""
     rng = np.random.default_rng(11)
     kv_lens = [40, 16, 0, 75, 200, 64, 1]
     q_lens = [7, 16, 3, 30, 64, 1, 1]
+    if rows.startswith("several"):
+        kv_lens = [300, 0, 75, 130]
+        q_lens = [290, 5, 64, 129]
     if causal:  # causal paged calls see a KV that already holds the queries' own tokens
         kv_lens = [max(k, q) for k, q in zip(kv_lens, q_lens)]
     go, gl, eo, el = _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages=64)
@@ -671,13 +677,16 @@ def test_layer_sliding_window_mask_known_answer_on_the_gpu():
 @pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
 @pytest.mark.parametrize("rotary", [0, 1])
 @pytest.mark.parametrize("causal,window", [(0, 1024), (1, 0), (1, 5), (1, 40)])
-def test_paged_prefill_sliding_cache_layer_window_and_inline_rope(hq, hkv, d, rotary, causal, window):
+@pytest.mark.parametrize("long_q", [False, True])
+def test_paged_prefill_sliding_cache_layer_window_and_inline_rope(hq, hkv, d, rotary, causal, window, long_q):
     """length_info (3, B), the per-layer window mask (window > 0 together with causal; with
-    window = 0 or without causal the reference falls back to the plain masks) and rotary_mode = 1."""
+    window = 0 or without causal the reference falls back to the plain masks) and rotary_mode = 1.
+    long_q: several row tiles per sequence, the form of the kernel that copies K/V without the
+    streaming hint."""
     from tests.test_oracle_kernels import sliding_case
     rng = np.random.default_rng(24)
     spec = [(100, 4, 20), (257, 0, 0), (330, 16, 48), (33, 2, 2), (64, 16, 32), (90, 0, 17)]
-    q_lens = [7, 64, 33, 3, 1, 30]
+    q_lens = [70, 250, 290, 3, 1, 30] if long_q else [7, 64, 33, 3, 1, 30]
     pages, pindptr, pvalues, info, k_log, _ = sliding_case(rng, spec, hkv, d, npages=64)
     n = sum(q_lens)
     qindptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
