@@ -51,7 +51,11 @@ def test_every_chunk_has_exactly_one_slot(name, forced_cp, h_kv):
 def test_chunk_size_follows_the_work():
     # 768 work items for small launches up to ~2300 for large ones; chunks of 16 to 128 pages
     assert tvm_amd.decode_split_plan([0, 4], 4, 8)[0] == 16
-    assert tvm_amd.decode_split_plan([0, 18432], 18432, 8)[0] == 64      # configs[1]: 2304 items
+    cfg2 = [288 * i for i in range(65)]
+    assert tvm_amd.decode_split_plan(cfg2, 18432, 8)[0] == 64            # configs[1]: 2304 items
+    assert tvm_amd.decode_split_plan([0, 18432], 18432, 8)[0] == 128     # as one sequence: fewer states to merge
+    short = [80 * i for i in range(257)]
+    assert tvm_amd.decode_split_plan(short, 80 * 256, 8)[0] == 128       # 256 short sequences: no split at all
     assert tvm_amd.decode_split_plan([0, 1 << 20], 1 << 20, 8)[0] == 128
     assert tvm_amd.decode_split_plan([0, 18432], 18432, 1)[0] == 32      # one kv head: 768 items
     assert tvm_amd.decode_split_plan([0, 8192], 8192, 8)[0] == 64        # one sequence of 131072 tokens

@@ -668,7 +668,7 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   // sized in those and counted in pages of the table
   p.page_shift = 0;
   while ((16 << p.page_shift) < page_size) ++p.page_shift;
-  p.chunk_pages = std::max(1, decode_pick_chunk_pages(nnz_pages << p.page_shift, h_kv) >> p.page_shift);
+  p.chunk_pages = std::max(1, decode_pick_chunk_pages(nnz_pages << p.page_shift, h_kv, batch_size) >> p.page_shift);
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
   const int64_t slots = nnz_pages / p.chunk_pages + batch_size;
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many chunks";
@@ -773,7 +773,7 @@ extern "C" int tvmkv_decode_split_plan(const int32_t* page_indptr_host, int32_t 
   KV_API_BEGIN();
   KV_CHECK(page_indptr_host && chunk_pages && num_slots && batch_size > 0 && h_kv > 0 && nnz_pages >= 0)
       << "decode_split_plan: bad argument";
-  const int cp = decode_pick_chunk_pages(nnz_pages, h_kv);
+  const int cp = decode_pick_chunk_pages(nnz_pages, h_kv, batch_size);
   const int64_t slots = nnz_pages / cp + batch_size;
   *chunk_pages = cp;
   *num_slots = slots;

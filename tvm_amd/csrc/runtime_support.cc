@@ -92,8 +92,13 @@ ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, s
 // three rounds of 3 workgroups x 256 CUs; small ones with fewer and longer items (one sequence of 131 072
 // tokens: 0.110 ms with 32-page chunks, 0.085 with 128; 64 sequences with one kv head: 0.140 ms with
 // 8-page chunks, 0.073 with 64).  One step of the matrix-core decode kernel is 2 pages per wave, 8 per
-// workgroup; chunks are powers of two from 16 to 128 pages.
-int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv) {
+// workgroup; chunks are powers of two from 16 to 128 pages.  Two cases take longer chunks than that:
+//  * more than 16 chunks per sequence while at least 768 items remain: the states of a sequence are
+//    merged by one workgroup, a serial tail (8 sequences of 16-65 k tokens: 0.245 ms with 64 pages,
+//    0.236 with 128);
+//  * sequences that fit one 128-page chunk on average, enough of them to fill the chip without a split:
+//    no partial states at all (256 sequences of 512-2048 tokens: 0.220 ms with 64 pages, 0.210 with 128).
+int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
   const int64_t forced = option(kOptDecodeChunkPages);
   if (forced >= 8 && forced % 8 == 0) return static_cast<int>(forced);
   const int64_t work = nnz_pages * h_kv;
@@ -101,6 +106,9 @@ int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv) {
   const int64_t cp = work / items;
   int pow2 = 16;
   while (pow2 < 128 && pow2 * 3 / 2 <= cp) pow2 *= 2;  // nearest power of two
+  const int64_t per_seq = nnz_pages / std::max(batch, 1);
+  while (pow2 < 128 && per_seq / pow2 > 16 && work / (pow2 * 2) >= 768) pow2 *= 2;
+  if (per_seq <= 96 && static_cast<int64_t>(batch) * h_kv >= 1536) pow2 = 128;
   return pow2;
 }
 

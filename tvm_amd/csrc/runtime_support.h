@@ -36,7 +36,7 @@ ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, s
 
 // Chunk-slot arithmetic of the decode split, on the host (the device functions of the same names in
 // kernels_decode.hip compute the same values; the tests compare both against a direct enumeration).
-int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv);
+int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch);
 
 }  // namespace tvmkv
 
