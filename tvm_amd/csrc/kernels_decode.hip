@@ -362,7 +362,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
   // streaming hint measured 10-15 % less bandwidth than without it.  KLINE: an instruction covers 8
   // tokens x one whole line.  A-rows 2t and 2t+1 are token t's features [0,32) and [32,64) of that
   // line, so one fragment goes through two MFMAs, one against the q features of the even rows and one
-  // against those of the odd rows (the matrix cores idle at 4 %), and token t's score is row 2t of the
+  // against those of the odd rows (the matrix cores are busy 5 % of the time), and token t's score is row 2t of the
   // first plus row 2t+1 of the second, both in one lane.  Whole lines take the streaming hint: 0.1965
   // -> 0.1915 ms on 64 sequences of 1024-8192 tokens; 4 tokens x a whole 256-byte row per instruction
   // (four MFMAs per fragment) measured the same as this.  K through LDS with whole-row copies like V
