@@ -155,7 +155,7 @@ def calibrate(num_bytes=2 << 30, iters=10, quiet=False):
     Prints one JSON line unless `quiet`."""
     import torch
 
-    from tvm_amd import kernels as K
+    from tvm_amd import bench_aids as K  # libtvmkv_bench.so: the measurement aids, not the product library
 
     dev = "cuda:0"
     src = torch.empty(num_bytes // 2, dtype=torch.float16, device=dev).normal_()
@@ -309,26 +309,195 @@ def cache_object_prefill(torch, dev, layers=8):
             "tflops": round(tflops, 1), "frac_of_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
 
 
-# HBM bytes per launch of the decode entry point, from rocprofv3 counter runs of this file
-# (profiles/decode_mfma_kernel_cfg2_batched_decode.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 in KiB per
-# dispatch of decode_mfma_kernel (it merges the chunks itself); the scales come from the plain copy
-# kernel of known size (profiles/stream_copy_kernel_2GiB_calibration.txt).  Measured on the default
-# workload (--steps 16 --warmup 3, 1 182 904 320 algorithmic bytes per launch) and kept as bytes of
-# traffic per algorithmic byte: the kernel reads every K/V row once whatever the context lengths are,
-# and the rest (q, outputs, split-KV partial states) scales with the same page tables, so the ratio
-# carries over to the page tables of any --steps / --warmup of this workload.
-TRAFFIC_MEASURED_ON_BYTES = 1182904320
-TRAFFIC_KIB = {"decode_mfma_kernel": (581458.0 * 2.0, 6281.5)}
-TRAFFIC_PER_ALGORITHMIC_BYTE = sum(r + w for r, w in TRAFFIC_KIB.values()) * 1024 / TRAFFIC_MEASURED_ON_BYTES
+# HBM bytes per launch of the decode entry point, from rocprofv3 counter runs of this file.  The one
+# place the figures live is the rocprofv3 summary profiles/decode_mfma_kernel_cfg2_batched_decode.txt,
+# which carries them on a line `traffic_record: {...}` (FETCH_SIZE and WRITE_SIZE in KiB per dispatch of
+# decode_mfma_kernel, which merges the chunks itself, the scale of each counter from the plain copy
+# kernel of known size, profiles/stream_copy_kernel_2GiB_calibration.txt, and the algorithmic bytes of
+# the launch they were measured on).  They are kept as bytes of traffic per algorithmic byte: the kernel
+# reads every K/V row once whatever the context lengths are, and the rest (q, outputs, split-KV partial
+# states) scales with the same page tables, so the ratio carries over to the page tables of any
+# --steps / --warmup of this workload.  Without the file the traffic is reported as null.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "decode_mfma_kernel_cfg2_batched_decode.txt")
+
+
+def traffic_per_algorithmic_byte():
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                if line.startswith("traffic_record:"):
+                    r = json.loads(line[len("traffic_record:"):])
+                    kib = r["fetch_size_kib"] * r["fetch_scale"] + r["write_size_kib"] * r["write_scale"]
+                    return kib * 1024.0 / r["algorithmic_bytes"]
+    except (OSError, ValueError, KeyError):
+        pass
+    return None
 
 
 def measured_traffic(algorithmic_bytes):
-    return int(round(TRAFFIC_PER_ALGORITHMIC_BYTE * algorithmic_bytes))
+    ratio = traffic_per_algorithmic_byte()
+    return None if ratio is None else int(round(ratio * algorithmic_bytes))
+
+
+def prefill_cpu_baseline(torch, pw, t, budget_s=10.0):
+    """The chunked-prefill step of configs[2] on the CPU oracle (split + RoPE, ragged causal attention of
+    the chunk, attention over the cached prefix, merge: the reference's llvm kernels restated, one
+    thread), on a bounded sample: kv head 0 with its 4 query heads (1/8 of the heads) of the sequences
+    with the least work first, until `budget_s` seconds are spent; its outputs are compared with the
+    rows the GPU step wrote."""
+    from oracle import kernels as ok
+
+    group = HQ // HKV
+    flops_seq = 4.0 * group * D * (pw["chunk"] * (pw["chunk"] + 1) / 2 + pw["chunk"] * pw["prefix"])
+    qkv, pos_all, out_gpu = t["qkv"], t["q_rope_position"].cpu().numpy(), t["out"]
+    spent, flops, seqs, err = 0.0, 0.0, [], 0.0
+    for b in np.argsort(flops_seq):
+        c, pre = int(pw["chunk"][b]), int(pw["prefix"][b])
+        r0, r1 = int(pw["q_indptr"][b]), int(pw["q_indptr"][b + 1])
+        heads = list(range(group)) + [HQ, HQ + HKV]
+        sub = qkv[r0:r1][:, heads].cpu().numpy()
+        ids = pw["page_values"][int(pw["page_indptr"][b]):int(pw["page_indptr"][b + 1])]
+        pool = t["pages"][torch.tensor(ids, dtype=torch.int64, device=qkv.device)][:, :, 0:1].contiguous().cpu().numpy()
+        if len(ids) == 0:
+            pool = np.zeros((1, 2, 1, PS, D), np.float16)
+        q = np.zeros((c, group, D), np.float16)
+        k = np.zeros((c, 1, D), np.float16)
+        v = np.zeros((c, 1, D), np.float16)
+        eo, el = np.zeros((c, group, D), np.float16), np.zeros((c, group), np.float32)
+        to, tl = np.zeros((c, group, D), np.float16), np.zeros((c, group), np.float32)
+        ind = np.array([0, c], np.int32)
+        zq, zb = np.zeros(c, np.int32), np.zeros(1, np.int32)
+        c0 = time.perf_counter()
+        ok.fused_rope(sub, pos_all[r0:r1], q, k, v, 1)
+        ok.prefill_ragged(q, ind, k, v, ind, zq, zb, eo, el, 1, 0, 1.0, 1e4, D ** -0.5)
+        ok.prefill_paged(q, ind, pool, np.array([0, len(ids)], np.int32), np.arange(len(ids), dtype=np.int32),
+                         pw["last_page_len"][b:b + 1], zb, zq, to, tl, 0, 0, 1.0, 1e4, D ** -0.5)
+        ok.merge_state_inplace(eo, el, to, tl)
+        spent += time.perf_counter() - c0
+        flops += float(flops_seq[b])
+        seqs.append(int(b))
+        err = max(err, float(np.max(np.abs(out_gpu[r0:r1, :group].cpu().numpy().astype(np.float32) - eo.astype(np.float32)))))
+        if spent > budget_s:
+            break
+    return {"value": round(flops / spent / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"kv head 0 with its {group} query heads (1/{HKV} of the heads) of sequences {seqs} of the same "
+                      f"workload, least work first ({flops / 1e9:.1f} of {pw['flops'] / 1e9:.1f} GFLOP), split+RoPE, ragged "
+                      f"causal + paged + merge as the reference composes the step, 1 thread, {spent:.1f} s",
+            "gpu_vs_cpu_max_abs_err": err}
+
+
+def cfg1_decode(torch, dev, steps=16):
+    """configs[0] (the reference's CPU-runnable case): 4 sequences with contexts 512/1024/1500/2048 built
+    through the cache verbs in a 1024-page pool (pages in allocation order), then decode steps that
+    append one token per sequence.  Checked against the committed golden fixture (page table and append
+    indices bit for bit, output within atol = rtol = 1e-2), timed on the GPU, and the same decode step
+    (split + RoPE + decode attention) timed on the CPU oracle, one thread."""
+    from oracle import kernels as ok
+    from tests.golden import make_fixtures as mf
+    from tests.gpu_util import GpuCache
+    from tvm_amd import get_global_func as gf
+
+    c = mf.CFG1
+    gold = np.load(os.path.join(ROOT, "tests", "golden", "cfg1_decode.npz"))
+    cache = GpuCache(mf.cfg1_cache_config(), 1, c["hq"], c["hkv"], c["d"], c["d"], rope_mode=1)
+    seen = {}
+
+    def grab():
+        for name in mf.PER_DEPTH:
+            seen[name] = cache.cache.aux(name, 0)
+        for name in mf.GLOBAL:
+            seen[name] = cache.cache.aux(name)
+
+    _, out = mf.cfg1_drive(cache, grab)
+    tables_equal = all(seen[name] == list(gold[name]) for name in mf.PER_DEPTH + mf.GLOBAL)
+    tol = 1e-2 + 1e-2 * np.abs(gold["out"].astype(np.float32))
+    err = np.abs(out.astype(np.float32) - gold["out"].astype(np.float32))
+    B, heads = len(c["ctx"]), c["hq"] + 2 * c["hkv"]
+    ids, ones = list(range(B)), [1] * B
+    sm = c["d"] ** -0.5
+    qkv = torch.randn((B, heads, c["d"]), device=dev).to(torch.float16)
+    o = torch.empty((B, c["hq"], c["d"]), dtype=torch.float16, device=dev)
+    cache.cache.set_stream(torch.cuda.current_stream().cuda_stream)
+    f_begin, f_end = gf("vm.builtin.kv_state_begin_forward"), gf("vm.builtin.kv_state_end_forward")
+    f_attn = gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")
+
+    def step(_):
+        f_begin(cache.cache, ids, ones, None)
+        f_attn(cache.cache, 0, sm, qkv, o)
+        f_end(cache.cache)
+
+    for _ in range(3):
+        step(0)
+    ms = time_region(torch, step, steps)
+    # CPU: the same kind of step on the fixture's page table (contexts + 1), K/V values do not matter for time
+    rng = np.random.default_rng(0)
+    ip = np.asarray(gold["page_indptr"], np.int32)
+    pv = np.asarray(gold["page_indices"], np.int32)
+    pages = rng.standard_normal((c["pool_pages"], 2, c["hkv"], c["page"], c["d"])).astype(np.float16)
+    qh = np.zeros((B, c["hq"], c["d"]), np.float16)
+    kh = np.zeros((B, c["hkv"], c["d"]), np.float16)
+    vh = np.zeros((B, c["hkv"], c["d"]), np.float16)
+    eo, el = np.zeros((B, c["hq"], c["d"]), np.float16), np.zeros((B, c["hq"]), np.float32)
+    z = np.zeros(B, np.int32)
+    c0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        ok.fused_rope(gold["qkv"], gold["q_rope_position_map"], qh, kh, vh, 1)
+        ok.decode(qh, pages, ip, pv, np.asarray(gold["last_page_len"], np.int32), z, z, eo, el, 0, 1.0, 1e4, sm)
+    cpu_s = (time.perf_counter() - c0) / reps
+    kv_tokens = sum(c["ctx"]) + B
+    return {"workload": "configs[0]: 4 seqs, ctx 512/1024/1500/2048, Hq32/Hkv8/D128, page 16, 1024-page pool, pages in "
+                        "allocation order through add_sequence / begin_forward; decode steps through the cache object",
+            "parity": {"page_table_and_append_indices_bit_exact_vs_fixture": bool(tables_equal),
+                       "output_within_atol_rtol_1e-2_of_fixture": bool(np.all(err <= tol)),
+                       "max_abs_err": float(err.max())},
+            "ms_per_step": round(ms, 4), "tokens_per_s": round(B / (ms * 1e-3), 1),
+            "note": "20.8 MB of K/V per step sit in the 256 MB memory-side cache: a parity configuration, not a bandwidth claim",
+            "cpu_baseline": {"value": round(B / cpu_s, 2), "unit": "tokens/s", "cores": 1, "kind": "port",
+                             "GBps": round(kv_tokens * TOKEN_BYTES / cpu_s / 1e9, 3),
+                             "sample": f"{reps} decode steps of this configuration (split+RoPE and decode attention over "
+                                       f"{kv_tokens} cached tokens), 1 thread, {cpu_s * reps:.2f} s"}}
+
+
+def mla_cpu_baseline(heads_sample=4, budget_s=8.0):
+    """The oracle's restatement of the reference's absorbed-MLA paged kernel (a GPU-only TIR kernel: the
+    reference has no CPU kernel for MLA, python/tvm/relax/frontend/nn/llm/kv_cache.py:676-677) on a
+    sample of configs[4]'s decode batch: `heads_sample` of the 128 heads of the first sequences, until
+    `budget_s` seconds are spent."""
+    from oracle import kernels as ok
+
+    rng = np.random.default_rng(4)
+    ctx = rng.integers(2048, 8192, size=32, endpoint=True)
+    dl, dr, ps = 512, 64, 64
+    spent, flops, nbytes, done = 0.0, 0.0, 0.0, 0
+    for b in range(len(ctx)):
+        n = int(ctx[b])
+        npg = (n + ps - 1) // ps
+        pages = (rng.standard_normal((npg, ps, dl + dr)) * 0.5).astype(np.float16)
+        q = (rng.standard_normal((1, heads_sample, dl + dr)) * 0.5).astype(np.float16)
+        eo, el = np.zeros((1, heads_sample, dl), np.float16), np.zeros((1, heads_sample), np.float32)
+        c0 = time.perf_counter()
+        ok.prefill_paged_mla(q, np.array([0, 1], np.int32), pages, np.array([0, npg], np.int32),
+                             np.arange(npg, dtype=np.int32), np.array([(n - 1) % ps + 1], np.int32), eo, el, 0,
+                             (128 + 64) ** -0.5, d_latent=dl)
+        spent += time.perf_counter() - c0
+        flops += 2.0 * heads_sample * (2 * dl + dr) * n
+        nbytes += n * (dl + dr) * 2.0
+        done += 1
+        if spent > budget_s:
+            break
+    return {"value": round(flops / spent / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "note": "no reference CPU kernel exists for MLA; this is the oracle's CPU restatement of the reference's GPU-only TIR kernel",
+            "sample": f"{heads_sample} of 128 heads of the first {done} sequences of configs[4]'s decode batch, one query "
+                      f"token each, 1 thread, {spent:.1f} s",
+            "tokens_per_s_scaled_to_128_heads": round(done / spent * heads_sample / 128.0, 4)}
 
 
 def extras(torch, K, dev):
     """configs[3] and configs[4] of BASELINE.json, and the sliding-window and token-tree variants of the
     attention kernels on configs[1]'s shape; kernels only (inputs resident, HIP events)."""
+    from tvm_amd.bench_aids import ClockSampler
+
     out = {}
 
     def i32(a):
@@ -395,7 +564,8 @@ def extras(torch, K, dev):
         "1 x 131072, 32/8": decode_shape(1, 131072, 131072, 32, 8, 11),
         "4 x 32768, 32/8": decode_shape(4, 32768, 32768, 32, 8, 12),
         "2048 x U[64,512], 32/8": decode_shape(2048, 64, 512, 32, 8, 13),
-        "64 x U[1024,8192], 32/1": decode_shape(64, 1024, 8192, 32, 1, 14)}
+        "64 x U[1024,8192], 32/1": decode_shape(64, 1024, 8192, 32, 1, 14),
+        "64 x U[1024,8192], 64/1": decode_shape(64, 1024, 8192, 64, 1, 15)}
     torch.cuda.empty_cache()
 
     # ---- sliding window + attention sinks, and a token-tree verify step, on configs[1]'s shape ----
@@ -456,6 +626,30 @@ def extras(torch, K, dev):
                                      "tflops_sliding_form": round(flops / ms_slid / 1e9, 1),
                                      "frac_of_mfma_peak": round(flops / ms_slid / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
 
+    # ---- uniform long prefill work: no short sequences, no causal diagonal, no ragged tail ----------
+    uq, uk = 2048, 4096
+    unp = uk // ps
+    uip = np.arange(9) * unp
+    uqi = np.arange(9) * uq
+    uqt = torch.randn((8 * uq, hq, d), device=dev).to(torch.float16)
+    uo = torch.empty_like(uqt)
+    ul = torch.empty((8 * uq, hq), dtype=torch.float32, device=dev)
+    uzq = torch.zeros(8 * uq, dtype=torch.int32, device=dev)
+    uargs = (uqt, i32(uqi), pages, i32(uip), i32(perm[:uip[-1]]), i32(np.full(8, ps)), z8, uzq, uo, ul, 0, 0, 1.0, 1e4,
+             d ** -0.5)
+    K.batch_prefill_paged_kv(*uargs)
+    settle(torch, lambda i: K.batch_prefill_paged_kv(*uargs))
+    with ClockSampler() as clock_u:
+        ms_u = time_region(torch, lambda i: K.batch_prefill_paged_kv(*uargs), 20)
+    uflops = 4.0 * hq * d * 8 * uq * uk
+    out["prefill_uniform"] = {"workload": f"8 seqs x {uq} query tokens against {uk} cached tokens each, every key visible "
+                                          "(paged prefill kernel, Hq32/Hkv8/D128, page 16, permuted pool): the attention "
+                                          "kernel without configs[2]'s short sequences, diagonal and tail",
+                              "ms": round(ms_u, 4), "tflops": round(uflops / ms_u / 1e9, 1),
+                              "frac_of_mfma_peak": round(uflops / ms_u / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                              "shader_clock_MHz": round(clock_u.mhz, 1)}
+    del uqt, uo, ul
+
     def preorder(depth):  # (first, second) labels of a complete binary tree listed in depth-first order
         labels = []
 
@@ -485,12 +679,9 @@ def extras(torch, K, dev):
         args = (q, i32(qi), pages, i32(indptr), i32(perm[:indptr[-1]]), i32((kv - 1) % ps + 1), z, zq, o, lse, 0, 1.0,
                 1e4, d ** -0.5, i32(qi), i32(np.tile(labels, (nseq, 1)).reshape(-1)))
         K.tree_attn_paged_kv(*args)
-        K.prefill_clock_probe(True)
         settle(torch, lambda i: K.tree_attn_paged_kv(*args))
-        K.prefill_clock_probe_read(reset=True)
-        ms = time_region(torch, lambda i: K.tree_attn_paged_kv(*args), 20)
-        cycles, ticks, _ = K.prefill_clock_probe_read(reset=True)
-        K.prefill_clock_probe(False)
+        with ClockSampler() as clock:
+            ms = time_region(torch, lambda i: K.tree_attn_paged_kv(*args), 20)
         depth_sum = float(sum((lv + 1) * 2 ** lv for lv in range(depth)))  # visible tree tokens summed over the nodes
         flops = 4.0 * hq * d * (float(ctx.sum()) * nodes + nseq * depth_sum)
         nbytes = float(kv.sum()) * 2 * hkv * d * 2 + 2 * nseq * nodes * hq * d * 2
@@ -499,7 +690,7 @@ def extras(torch, K, dev):
                 "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
                 "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
                 "GBps": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
-                "shader_clock_MHz": round(cycles / max(ticks, 1) * 100.0, 1)}
+                "shader_clock_MHz": round(clock.mhz, 1)}
 
     out["token_tree_verify"] = tree_verify(6)            # 63 nodes: 252 rows per kv head, two row tiles, compute-bound
     out["token_tree_verify_15_nodes"] = tree_verify(4)   # 60 rows per kv head: one row tile, the K/V stream decides
@@ -528,6 +719,48 @@ def extras(torch, K, dev):
         "speedup": round(ms_whole / ms_split, 2), "GBps": round(nbytes / ms_split / 1e6, 1),
         "frac_of_hbm_peak": round(nbytes / ms_split / 1e6 / HBM_PEAK_GBPS, 4)}
     del pages
+    torch.cuda.empty_cache()
+
+    # ---- the other head dims: decode on configs[1]'s lengths, the one-pass chunked prefill on configs[2]'s ----
+    def head_dim_leg(d_, hq_, hkv_):
+        rng_ = np.random.default_rng(1)
+        ctx_ = rng_.integers(1024, 8192, size=64, endpoint=True)
+        npg_ = (ctx_ + ps - 1) // ps
+        ip_ = np.concatenate([[0], np.cumsum(npg_)])
+        pw_ = prefill_workload()
+        pool_ = max(int(ip_[-1]), pw_["pool_pages"]) + 8
+        perm_ = rng_.permutation(pool_).astype(np.int32)
+        pages_ = torch.empty((pool_, 2, hkv_, ps, d_), dtype=torch.float16, device=dev)
+        for lo_ in range(0, pool_, 8192):
+            pages_[lo_:lo_ + 8192].normal_()
+        q_ = torch.randn((64, hq_, d_), device=dev).to(torch.float16)
+        o_ = torch.empty_like(q_)
+        l_ = torch.empty((64, hq_), dtype=torch.float32, device=dev)
+        z_ = torch.zeros(64, dtype=torch.int32, device=dev)
+        a_ = (q_, pages_, i32(ip_), i32(perm_[:ip_[-1]]), i32((ctx_ - 1) % ps + 1), z_, z_, o_, l_, 0, 1.0, 1e4, d_ ** -0.5)
+        K.batch_decode_paged_kv(*a_)
+        ms_d = time_region(torch, lambda i: K.batch_decode_paged_kv(*a_), 20, SETTLE_S)
+        nb_ = float(ctx_.sum()) * 2 * hkv_ * d_ * 2 + 2 * 64 * hq_ * d_ * 2
+        n_ = int(pw_["q_indptr"][-1])
+        qp_ = torch.randn((n_, hq_, d_), device=dev).to(torch.float16)
+        kp_ = torch.randn((n_, hkv_, d_), device=dev).to(torch.float16)
+        vp_ = torch.randn((n_, hkv_, d_), device=dev).to(torch.float16)
+        op_ = torch.empty_like(qp_)
+        lp_ = torch.empty((n_, hq_), dtype=torch.float32, device=dev)
+        b_ = (qp_, i32(pw_["q_indptr"]), kp_, vp_, pages_, i32(pw_["page_indptr"]), i32(pw_["page_values"]),
+              i32(pw_["last_page_len"]), op_, lp_, d_ ** -0.5)
+        K.batch_prefill_cached_and_new_kv(*b_)
+        ms_p = time_region(torch, lambda i: K.batch_prefill_cached_and_new_kv(*b_), 20, SETTLE_S)
+        fl_ = pw_["flops"] / (HQ * D) * (hq_ * d_)
+        return {"decode_ms": round(ms_d, 4), "decode_frac_of_hbm_peak": round(nb_ / ms_d / 1e6 / HBM_PEAK_GBPS, 4),
+                "prefill_ms": round(ms_p, 4), "prefill_tflops": round(fl_ / ms_p / 1e9, 1),
+                "prefill_frac_of_mfma_peak": round(fl_ / ms_p / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+
+    out["other_head_dims"] = {
+        "workload": "decode of 64 seqs ctx U[1024,8192] (configs[1]'s lengths) and the one-pass chunked-prefill kernel on "
+                    "configs[2]'s 8 sequences, page 16, at the head dims beside 128 (query / kv heads)",
+        "D64, 32/8": head_dim_leg(64, 32, 8),
+        "D256, 16/8": head_dim_leg(256, 16, 8)}
     torch.cuda.empty_cache()
 
     # ---- configs[4]: MLA, 128 heads, latent 512 + rope 64, page 64 ------------------------------
@@ -636,7 +869,8 @@ def hold(which, seconds):
     elif which == "mfma":
         ops = torch.randn((256, 16), device=dev).to(torch.float16)
         sums = torch.empty((512, 256), dtype=torch.float32, device=dev)
-        fn = lambda i: K.mfma_loop(ops, sums, 4096)
+        from tvm_amd import bench_aids
+        fn = lambda i: bench_aids.mfma_loop(ops, sums, 4096)
         unit, work = "TFLOP/s (random operands)", 2.0 * 32 * 32 * 16 * 8 * 4096 * 4 * 512 / 1e12
     elif which in ("mla_prefill", "mla_decode"):
         hq, dl, dr, ps = 128, 512, 64, 64
@@ -712,6 +946,7 @@ def main():
     import torch
 
     from tvm_amd import kernels as K  # raises if libtvmkv.so is missing: there is no fallback
+    from tvm_amd.bench_aids import ClockSampler
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
@@ -795,7 +1030,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(gbps_decode, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps_decode / HBM_PEAK_GBPS, 4),
                      "traffic": measured_traffic(int(decode_bytes)),
-                     "traffic_per_algorithmic_byte": round(TRAFFIC_PER_ALGORITHMIC_BYTE, 4),
+                     "traffic_per_algorithmic_byte": (None if traffic_per_algorithmic_byte() is None
+                                                      else round(traffic_per_algorithmic_byte(), 4)),
                      "kernel": "tvmkv_batch_decode_paged_kv (decode_mfma_kernel, chunk merge fused)",
                      "ms": round(ms_decode, 4), "algorithmic_bytes": int(decode_bytes)},
     }
@@ -803,18 +1039,15 @@ def main():
     # ---- chunked prefill (configs[2]): ragged causal + paged non-causal + merge + append -------
     if not args.no_prefill:
         pw = prefill_workload()
-        prefill_step, _ = make_prefill_step(torch, K, pw, gen, dev)
+        prefill_step, prefill_tensors = make_prefill_step(torch, K, pw, gen, dev)
 
         for _ in range(3):
             prefill_step(0)
         ms_cold = time_region(torch, prefill_step, 10)  # ten launches as they come, clocks still ramping
         settle(torch, prefill_step)
-        K.prefill_clock_probe(True)
-        K.prefill_clock_probe_read(reset=True)
-        ms_prefill = time_region(torch, prefill_step, max(K_steps, 10))
-        cycles, ticks, _ = K.prefill_clock_probe_read(reset=True)
-        K.prefill_clock_probe(False)
-        shader_mhz = cycles / max(ticks, 1) * 100.0
+        with ClockSampler() as clock:
+            ms_prefill = time_region(torch, prefill_step, max(K_steps, 10))
+        shader_mhz = clock.mhz
         tflops = pw["flops"] / (ms_prefill * 1e-3) / 1e12
         result["prefill"] = {"workload": "configs[2]: chunked causal prefill, 8 seqs, prefix U[0,4096], chunk "
                                          "U[128,2048] seed 2 (RoPE of k + append of the new K/V rows in one launch; causal attention over the new chunk and attention over the cached prefix in one pass that rotates q itself)",
@@ -824,8 +1057,8 @@ def main():
                              "ms_first_ten_launches": round(ms_cold, 4),
                              "shader_clock_MHz": round(shader_mhz, 1),
                              "frac_of_mfma_peak_at_that_clock": round(tflops / (MFMA_F16_PEAK_TFLOPS * shader_mhz / 2400.0), 4),
-                             "clock_note": "average shader clock over the workgroups of the timed attention launches "
-                                           "(s_memtime / s_memrealtime inside the kernel); the 2.5 PFLOP/s peak is quoted at 2400 MHz"}
+                             "clock_note": "shader clock over the timed launches (a one-wave sampler kernel on a second stream "
+                                           "reads s_memtime / s_memrealtime beside them); the 2.5 PFLOP/s peak is quoted at 2400 MHz"}
 
     # What the simplest kernels reach on this box, next to the datasheet peaks.  After the timed legs:
     # the MFMA loop heats the chip and the clock of what follows drops.
@@ -910,11 +1143,20 @@ def main():
                                             "sample": f"the same {par_steps} decode steps, one task per sequence on "
                                                       f"{threads} threads, {par_s:.1f} s",
                                             "tokens_per_s": round(B * par_steps / par_s, 2)}
+        if "prefill" in result:
+            result["prefill"]["cpu_baseline"] = prefill_cpu_baseline(torch, pw, prefill_tensors)
+        result["cfg1_decode"] = cfg1_decode(torch, dev)
+
 
     if not args.no_extras:
         del pages, qkv
         torch.cuda.empty_cache()
         result["extras"] = extras(torch, K, dev)
+        if not args.no_cpu_baseline:
+            cpu_mla = mla_cpu_baseline()
+            result["extras"]["mla_decode"]["cpu_baseline"] = cpu_mla
+            result["extras"]["mla_prefill"]["cpu_baseline"] = dict(cpu_mla, sample=cpu_mla["sample"] + " (the same kernel "
+                                                                   "serves prefill-shaped calls: the per-flop rate carries over)")
         torch.cuda.empty_cache()
         result["extras"]["cache_object_decode"] = cache_object_decode(torch, dev)
         torch.cuda.empty_cache()

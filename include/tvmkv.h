@@ -376,30 +376,22 @@ int tvmkv_decode_split_plan(const int32_t* page_indptr_host, int32_t batch_size,
                             int32_t h_kv, int32_t* chunk_pages, int64_t* num_slots, int32_t* slot_seq,
                             int32_t* slot_chunk, int64_t slot_capacity);
 
-/* Measurement utilities (no counterpart in the reference): a plain streaming read (XOR-folded,
- * the result is discarded) and a plain copy of `num_bytes` (a multiple of 16) bytes.  The
- * benchmark uses them to calibrate the achievable HBM bandwidth of the box, and the profiling
- * notes use the copy to scale the FETCH_SIZE / WRITE_SIZE counters. `sink` is 4 writable bytes. */
-int tvmkv_stream_read(const void* src, int64_t num_bytes, void* sink, void* stream);
-/* the same read with non-temporal loads, the kind the decode kernel issues */
-int tvmkv_stream_read_nt(const void* src, int64_t num_bytes, void* sink, void* stream);
-int tvmkv_stream_copy(const void* src, void* dst, int64_t num_bytes, void* stream);
-/* Matrix-core calibration (no counterpart in the reference): `workgroups` workgroups of 4 waves run
- * `iters` rounds of 8 v_mfma_f32_32x32x16_f16 each (4 accumulators, nothing else in the loop) on the
- * A and B fragments read from `operands` (256 lanes x 16 halfs); `out` gets workgroups x 256
- * floats.  2 * 32 * 32 * 16 * 8 * iters * 4 * workgroups flop per launch. */
-int tvmkv_mfma_loop(const void* operands, float* out, int32_t iters, int32_t workgroups, void* stream);
-/* Clock probe of the prefill kernels (no counterpart in the reference; a measurement aid).  The
- * shader clock of this chip follows the power the kernel draws, so a fraction of the datasheet
- * matrix peak (quoted at 2.4 GHz) says little without the clock the kernel really ran at.  After
- * tvmkv_prefill_clock_probe(1) every workgroup of every prefill / tree-attention launch of this
- * process adds three numbers to counters on its device: the shader cycles and the 100 MHz ticks
- * between its start and its end, and 1.  tvmkv_prefill_clock_probe_read synchronizes the current
- * device, copies the three sums to counters[0..2] (cycles, ticks, workgroups) and clears them if
- * reset != 0: cycles / ticks * 100 MHz is the average shader clock.  Not thread-safe against
- * concurrent launches; costs two timestamp reads and three atomics per workgroup while enabled. */
-int tvmkv_prefill_clock_probe(int32_t enable);
-int tvmkv_prefill_clock_probe_read(uint64_t* counters, int32_t reset);
+/* Frees the split-KV scratch buffers that the launchers keep for (current device, stream), after
+ * synchronising the stream (no counterpart in the reference).  The launchers keep one buffer per device,
+ * stream and kernel family, grown on demand and otherwise never freed: a caller that creates and destroys
+ * streams calls this before it destroys one.  A buffer whose address a graph under capture has recorded is
+ * not freed but kept until the process ends (the graph may be replayed at any time); for the same reason a
+ * larger eager call on a stream that was captured from leaves the old buffer in place and allocates the
+ * new one beside it.  Refused while the stream is being captured. */
+int tvmkv_release_scratch(void* stream);
+/* Test aid (no counterpart in the reference): sets the launch count of every pooled scratch buffer and of
+ * the built-in buffers of tvmkv_batch_decode_paged_kv_noalloc.  The arrival counters of a split-KV launch
+ * are tagged with the low 32 bits of that count; the tests set it just below 2^32 and run launches across
+ * the wrap. */
+int tvmkv_debug_set_scratch_launches(uint64_t launches);
+/* The same arithmetic on the host alone: advances *launches and returns the epoch of that launch (never
+ * 0); *wrapped = 1 when the epochs started over, which is when the launchers clear the counters. */
+uint32_t tvmkv_debug_next_scratch_epoch(uint64_t* launches, int32_t* wrapped);
 
 /* ======================================================================================
  * (2) Cache object

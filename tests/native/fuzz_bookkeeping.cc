@@ -186,5 +186,34 @@ int main(int argc, char** argv) {
     if (length.empty() && !book.Empty() && rejected == 0) Fail("cache not empty without sequences");
   }
   std::printf("seed %u: %d operations, %ld steps, %ld rejected\n", seed, operations, steps, rejected);
+
+  // A long-running cache: forks inside pages and removals, over and over, without a Clear().  The page-id
+  // arena must settle (every slice a fork or a removal gives back can serve a later request) and so must
+  // the copy log.
+  book.Clear();
+  book.AddSequence(0);
+  {
+    const int64_t ids[1] = {0}, lens[1] = {200};
+    book.BeginForward(ids, lens, 1, nullptr, 0);
+  }
+  int64_t child = 1, arena_after_warmup = 0;
+  for (int cycle = 0; cycle < 20000; ++cycle) {
+    const int live = pick(1, 4);
+    for (int j = 0; j < live; ++j) book.ForkSequence(0, child + j, pick(1, 200));
+    for (int j = 0; j < live; ++j) {
+      const int64_t ids[1] = {child + j}, lens[1] = {static_cast<int64_t>(pick(1, 40))};
+      book.BeginForward(ids, lens, 1, nullptr, 0);
+    }
+    for (int j = 0; j < live; ++j) book.RemoveSequence(child + j);
+    child += live;
+    if (cycle == 2000) arena_after_warmup = book.PageArenaInUse();
+    if (cycle > 2000 && book.PageArenaInUse() > 2 * arena_after_warmup + 1024) {
+      Fail("page-id arena keeps growing", book.PageArenaInUse(), arena_after_warmup);
+    }
+    book.TrimCopyLog(book.CopyLog().size());
+    if (book.CopyLog().size() > KVBookkeeper::kCopyLogCap) Fail("copy log keeps growing", static_cast<long>(book.CopyLog().size()));
+  }
+  std::printf("churn: arena %ld entries after 2000 cycles, %ld after 20000\n", static_cast<long>(arena_after_warmup),
+              static_cast<long>(book.PageArenaInUse()));
   return 0;
 }

@@ -23,8 +23,35 @@ def test_library_exports_every_declared_symbol():
     assert not missing, f"declared under include/ but not exported: {missing}"
 
 
+def test_bench_library_exports_every_declared_symbol():
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "tvmkv_bench.h")).read(), flags=re.S)
+    names = sorted(set(re.findall(r"\b(tvmkvb_[a-z0-9_]+)\s*\(", text)))
+    assert names == sorted(_lib.BENCH_SIGNATURES)
+    handle = ctypes.CDLL(_lib.BENCH_LIB_PATH)
+    assert not [n for n in names if not hasattr(handle, n)]
+    product = ctypes.CDLL(tvm_amd.LIB_PATH)
+    assert not [n for n in ("tvmkv_mfma_loop", "tvmkv_stream_read", "tvmkv_prefill_clock_probe") if hasattr(product, n)], \
+        "measurement aids belong to libtvmkv_bench.so, not to the product library"
+
+
+def test_scratch_epochs_skip_zero_at_the_wrap():
+    """The epoch that tags a launch's arrival counters is the low half of a 64-bit launch count and never 0."""
+    from tvm_amd._lib import lib
+
+    fn = lib().tvmkv_debug_next_scratch_epoch
+    fn.argtypes = [ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_int32)]
+    fn.restype = ctypes.c_uint32
+    count, wrapped = ctypes.c_uint64((1 << 32) - 3), ctypes.c_int32(0)
+    seen = []
+    for _ in range(5):
+        seen.append((fn(ctypes.byref(count), ctypes.byref(wrapped)), wrapped.value))
+    assert seen == [(0xfffffffe, 0), (0xffffffff, 0), (1, 1), (2, 0), (3, 0)]
+    assert count.value == (1 << 32) + 3
+
+
 def test_python_signatures_cover_the_header():
-    names = set(declared_functions()) - {"tvmkv_last_error", "tvmkv_version", "tvmkv_cache_destroy"}
+    names = set(declared_functions()) - {"tvmkv_last_error", "tvmkv_version", "tvmkv_cache_destroy",
+                                         "tvmkv_debug_next_scratch_epoch"}
     assert names == set(_lib.SIGNATURES), names ^ set(_lib.SIGNATURES)
 
 

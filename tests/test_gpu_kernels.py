@@ -3,10 +3,13 @@
 Integer/byte work (append scatter, gathers, page copies) must be bit-exact; attention outputs
 are fp16 with fp32 accumulation and must agree within atol = rtol = 1e-2 (the tolerance the
 path is specified to); RoPE outputs are compared at one fp16 ulp."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
 
+import tvm_amd
 from oracle import kernels as ok
 from tests.gpu_util import DEV, dev, host, i32
 from tests.util import ATOL, RTOL, assert_close, assert_close_where_keys, build_paged_kv, rows_without_keys
@@ -917,43 +920,78 @@ def test_prefill_one_pass_with_queries_from_the_fused_qkv(hq, hkv, d, apply_rope
 
 
 def test_measurement_utilities():
-    """The calibration kernels of the benchmark: the copy copies, the reads leave their input alone,
-    and the MFMA loop adds up what its instruction count says (integers in fp32, so exactly)."""
+    """The calibration kernels of the benchmark (libtvmkv_bench.so): the copy copies, the reads leave their
+    input alone, and the MFMA loop adds up what its instruction count says (integers in fp32, so exactly)."""
+    from tvm_amd import bench_aids as A
+
     src = torch.arange(1 << 16, dtype=torch.int32, device=DEV)
     dst = torch.zeros_like(src)
     sink = torch.zeros(4, dtype=torch.int32, device=DEV)
-    K.stream_copy(src, dst)
-    K.stream_read(src, sink)
-    K.stream_read_nt(src, sink)
+    A.stream_copy(src, dst)
+    A.stream_read(src, sink)
+    A.stream_read_nt(src, sink)
     torch.cuda.synchronize()
     assert torch.equal(src, dst) and torch.equal(src, torch.arange(1 << 16, dtype=torch.int32, device=DEV))
     ops = torch.full((256, 16), 0.5, dtype=torch.float16, device=DEV)
     out = torch.zeros((3, 256), dtype=torch.float32, device=DEV)
     iters = 5
-    K.mfma_loop(ops, out, iters)
+    A.mfma_loop(ops, out, iters)
     torch.cuda.synchronize()
     # one instruction adds 16 * 0.5 * 0.5 = 4 to each of its 16 results per lane; 8 instructions a round
     assert torch.all(out == 4.0 * 16 * 8 * iters)
 
 
-def test_prefill_clock_probe_counts_workgroups_and_leaves_results_alone():
-    """The clock probe adds (shader cycles, 100 MHz ticks, 1) per workgroup while it is switched on,
-    nothing while it is off, and does not change what the kernel computes."""
-    rng = np.random.default_rng(77)
-    lens = [300, 5, 200]
-    K.prefill_clock_probe(False)
-    K.prefill_clock_probe_read(reset=True)
-    base_out, base_lse, eo, el = _ragged_both(rng, lens, 32, 8, 128, 128, 1)
-    assert K.prefill_clock_probe_read(reset=True) == (0, 0, 0)
-    K.prefill_clock_probe(True)
+def test_clock_sampler_runs_beside_a_kernel_and_ends():
+    """The one-wave clock sampler on its own stream: it ends when the host sets the flag (and by itself
+    after max_seconds), and reports a plausible shader clock for the time a kernel ran beside it."""
+    from tvm_amd import bench_aids as A
+
+    ops = torch.full((256, 16), 0.5, dtype=torch.float16, device=DEV)
+    out = torch.zeros((256, 256), dtype=torch.float32, device=DEV)
+    with A.ClockSampler(max_seconds=2.0) as clock:
+        for _ in range(20):
+            A.mfma_loop(ops, out, 512)
+    assert 200.0 < clock.mhz < 4000.0, clock.mhz
+    # without the flag it ends after max_seconds by itself
+    sampler = A.ClockSampler(max_seconds=0.05)
+    sampler.__enter__()
+    sampler.stream.synchronize()
+    assert int(sampler.out.cpu()[1]) >= int(0.05 * 1e8)
+    sampler.__exit__(None, None, None)
+
+
+def test_scratch_epoch_wrap_and_release():
+    """Split-KV launches across the wrap of the 32-bit epoch that tags their arrival counters (the launch
+    count is set just below 2^32), through the pooled buffer and through the built-in one of the entry
+    point that allocates nothing; then the pooled buffers of the stream are released and the next call
+    allocates afresh.  Every output equals the one before."""
+    from tvm_amd._lib import check, lib
+
+    rng = np.random.default_rng(5)
+    kv = [700, 33, 1500, 260]
+    pages, ip, pv, last, _, _ = build_paged_kv(rng, kv, 170, 8, 16, 128)
+    q = rng.standard_normal((4, 32, 128)).astype(F16)
+    z = np.zeros(4, np.int32)
+    args = (dev(q), dev(pages), i32(ip), i32(pv), i32(last), i32(z), i32(z))
+
+    def run(noalloc):
+        o = torch.zeros((4, 32, 128), dtype=torch.float16, device=DEV)
+        s = torch.zeros((4, 32), dtype=torch.float32, device=DEV)
+        K.batch_decode_paged_kv(*args, o, s, 0, 1.0, 1e4, 128 ** -0.5, noalloc=noalloc)
+        return host(o), host(s)
+
+    prev = tvm_amd.set_option("decode_chunk_pages", 8)  # several chunks per sequence: the fused merge counts arrivals
     try:
-        rng = np.random.default_rng(77)
-        out, lse, _, _ = _ragged_both(rng, lens, 32, 8, 128, 128, 1)
-        cycles, ticks, workgroups = K.prefill_clock_probe_read(reset=True)
+        base = run(False)
+        base_noalloc = run(True)
+        assert np.array_equal(base[0], base_noalloc[0])
+        check(lib().tvmkv_debug_set_scratch_launches((1 << 32) - 3))
+        for _ in range(6):  # epochs 0xfffffffe, 0xffffffff, then 1, 2, ... from cleared counters
+            for noalloc in (False, True):
+                o, s = run(noalloc)
+                assert np.array_equal(o, base[0]) and np.array_equal(s, base[1])
+        check(lib().tvmkv_release_scratch(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        o, s = run(False)
+        assert np.array_equal(o, base[0]) and np.array_equal(s, base[1])
     finally:
-        K.prefill_clock_probe(False)
-    assert np.array_equal(out, base_out) and np.array_equal(lse, base_lse)
-    # row tiles: ceil(len * group / 128) per sequence and kv head, group 4, 8 kv heads
-    assert workgroups == 8 * sum((n * 4 + 127) // 128 for n in lens)
-    assert ticks > 0 and 200.0 < cycles / ticks * 100.0 < 4000.0, (cycles, ticks)
-    assert K.prefill_clock_probe_read(reset=False) == (0, 0, 0)
+        tvm_amd.set_option("decode_chunk_pages", prev)

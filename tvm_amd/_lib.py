@@ -58,13 +58,9 @@ SIGNATURES = {
     "tvmkv_compact_kv_copy": [c_vp, c_vp, c_vp, c_i32, c_i32, c_i64, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_set_option": [ctypes.c_char_p, c_i64],
     "tvmkv_get_option": [ctypes.c_char_p, p_i64],
+    "tvmkv_release_scratch": [c_vp],
+    "tvmkv_debug_set_scratch_launches": [ctypes.c_uint64],
     "tvmkv_decode_split_plan": [p_i32, c_i32, c_i64, c_i32, p_i32, p_i64, p_i32, p_i32, c_i64],
-    "tvmkv_stream_read": [c_vp, c_i64, c_vp, c_vp],
-    "tvmkv_stream_read_nt": [c_vp, c_i64, c_vp, c_vp],
-    "tvmkv_mfma_loop": [c_vp, c_vp, c_i32, c_i32, c_vp],
-    "tvmkv_prefill_clock_probe": [c_i32],
-    "tvmkv_prefill_clock_probe_read": [c_vp, c_i32],
-    "tvmkv_stream_copy": [c_vp, c_vp, c_i64, c_vp],
     "tvmkv_cache_create": [p_i64, c_i32, p_i64, c_i32, c_i64, c_i64, c_i64, c_i64, p_i64, c_i32, c_i32, c_i32,
                            c_f64, c_f64, c_i32, c_i32, ctypes.POINTER(c_vp)],
     "tvmkv_cache_set_stream": [c_vp, c_vp],
@@ -113,7 +109,33 @@ SIGNATURES = {
     "tvmkv_dl_compact_kv_copy": [c_vp] * 3 + [c_i64, c_vp],
 }
 
+# include/tvmkv_bench.h: the measurement aids of bench.py, a library of their own
+BENCH_LIB_PATH = os.path.join(_HERE, "lib", "libtvmkv_bench.so")
+BENCH_SIGNATURES = {
+    "tvmkvb_stream_read": [c_vp, c_i64, c_vp, c_vp],
+    "tvmkvb_stream_read_nt": [c_vp, c_i64, c_vp, c_vp],
+    "tvmkvb_stream_copy": [c_vp, c_vp, c_i64, c_vp],
+    "tvmkvb_mfma_loop": [c_vp, c_vp, c_i32, c_i32, c_vp],
+    "tvmkvb_clock_sampler": [c_vp, ctypes.c_uint64, c_vp, c_vp],
+}
+
 _lib = None
+_bench_lib = None
+
+
+def bench_lib():
+    """libtvmkv_bench.so (measurement aids; not part of the drop-in library) with argtypes set."""
+    global _bench_lib
+    if _bench_lib is None:
+        if not os.path.exists(BENCH_LIB_PATH):
+            raise ImportError(f"{BENCH_LIB_PATH} is missing: build it with `make -C tvm_amd/csrc`.")
+        handle = ctypes.CDLL(BENCH_LIB_PATH)
+        for name, argtypes in BENCH_SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+        _bench_lib = handle
+    return _bench_lib
 
 
 def lib():

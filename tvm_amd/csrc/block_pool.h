@@ -114,15 +114,32 @@ class BlockPool {
     std::memmove(base + i, base + i + 1, static_cast<size_t>(s.count - i - 1) * sizeof(int32_t));
     --s.count;
   }
-  // The first n pages of `from` become the pages of `to` (which has none): the slice is cut in two,
-  // no page id moves.
+  // The first n pages of `from` become the pages of `to` (which has none).  Where both parts keep at least
+  // kMinSlice entries the slice is cut in two and no page id moves; otherwise a cut would leave a slice
+  // that no later request can reuse (requests are for kMinSlice entries or more), so `to` gets a slice of
+  // its own and the rest of `from` moves to the front of the old one.
   void SplitFront(int32_t from, int32_t n, int32_t to) {
+    if (n >= kMinSlice && slice_[from].capacity - n >= kMinSlice) {
+      Slice& f = slice_[from];
+      slice_[to] = Slice{f.offset, n, n};
+      f.offset += n;
+      f.count -= n;
+      f.capacity -= n;
+      return;
+    }
+    int32_t want = kMinSlice;
+    while (want < n) want *= 2;
+    Slice fresh = Allocate(want);  // may move the arena: take addresses afterwards
     Slice& f = slice_[from];
-    slice_[to] = Slice{f.offset, n, n};
-    f.offset += n;
+    int32_t* base = arena_.data() + f.offset;
+    std::memcpy(arena_.data() + fresh.offset, base, static_cast<size_t>(n) * sizeof(int32_t));
+    std::memmove(base, base + n, static_cast<size_t>(f.count - n) * sizeof(int32_t));
     f.count -= n;
-    f.capacity -= n;
+    fresh.count = n;
+    slice_[to] = fresh;
   }
+  // int32 entries of the arena handed out so far (free slices included): what a long-running cache holds
+  int64_t ArenaInUse() const { return bump_; }
 
  private:
   struct Slice {
@@ -158,7 +175,7 @@ class BlockPool {
   }
   void Grow(int32_t b) {
     const Slice old = slice_[b];
-    int32_t want = 4;
+    int32_t want = kMinSlice;
     while (want <= old.capacity) want *= 2;
     Slice fresh = Allocate(want);
     if (old.count > 0) {
@@ -170,6 +187,7 @@ class BlockPool {
   }
 
   static constexpr int kClasses = 32;
+  static constexpr int32_t kMinSlice = 4;  // no slice is smaller: every free slice can serve some request
   std::vector<Slice> slice_;
   std::vector<int32_t> free_blocks_;
   std::vector<int32_t> arena_;

@@ -603,28 +603,40 @@ constexpr size_t kStaticScratchBytes = 24u << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 struct StaticScratch {
-  char* ptr = nullptr;   // device address of `scratch` on this device
-  uint32_t epoch = 0;
+  char* ptr = nullptr;    // device address of `scratch` on this device
+  uint64_t launches = 0;  // the epoch of a launch is the low half
 };
 static StaticScratch g_static_scratch[64];
 static std::mutex g_static_scratch_mutex;
 
-static ScratchLease lease_static_scratch(size_t bytes) {
+static ScratchLease lease_static_scratch(size_t bytes, hipStream_t stream) {
   int dev = 0;
   HIP_CHECK(hipGetDevice(&dev));
   KV_CHECK(dev >= 0 && dev < 64) << "device ordinal " << dev << " out of range";
   KV_CHECK(bytes <= kStaticScratchBytes)
       << "batch_decode_paged_kv_noalloc: the call needs " << bytes << " bytes of scratch memory, the built-in "
       << "buffer has " << kStaticScratchBytes << "; use tvmkv_batch_decode_paged_kv for this shape";
-  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  std::unique_lock<std::mutex> lock(g_static_scratch_mutex);
   StaticScratch& s = g_static_scratch[dev];
   if (s.ptr == nullptr) {
     void* ptr = nullptr;
     HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
     s.ptr = static_cast<char*>(ptr);  // device memory of a loaded code object starts out zeroed
   }
-  KV_CHECK(s.epoch != 0xffffffffu) << "batch_decode_paged_kv_noalloc: 2^32 calls on this device; counters exhausted";
-  return ScratchLease{s.ptr, ++s.epoch};
+  bool wrapped = false;
+  const uint32_t epoch = next_scratch_epoch(&s.launches, &wrapped);
+  // 2^32 calls on this device: the epochs start over at 1 from counters cleared by a kernel in stream
+  // order (no allocation, no memset node)
+  if (wrapped) zero_scratch_counters(s.ptr, kArrivalBytes, stream);
+  return ScratchLease{s.ptr, epoch, std::move(lock)};
+}
+
+extern "C" int tvmkv_debug_set_scratch_launches(uint64_t launches) {
+  KV_API_BEGIN();
+  debug_set_scratch_launches(launches);
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  for (auto& s : g_static_scratch) s.launches = launches;
+  KV_API_END();
 }
 
 // Body of the decode entry point.  lease(bytes) hands out the scratch memory of the call: arrival
@@ -759,7 +771,7 @@ extern "C" int tvmkv_batch_decode_paged_kv_noalloc(const void* q, const void* pa
                                                    int32_t d, int32_t page_size, int32_t sliding_window,
                                                    void* stream) {
   KV_API_BEGIN();
-  decode_entry([&](size_t bytes) { return lease_static_scratch(bytes); }, q, pages, page_indptr, page_values,
+  decode_entry([&](size_t bytes) { return lease_static_scratch(bytes, as_stream(stream)); }, q, pages, page_indptr, page_values,
                length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode, rope_scale, rope_theta,
                sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window, stream);
   KV_API_END();

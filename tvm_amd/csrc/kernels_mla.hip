@@ -953,6 +953,7 @@ static int mla_entry(const void* q, const int32_t* q_indptr, const void* pages, 
     return TVMKV_OK;
   }
   MlaParams p{};
+  ScratchLease lease{};  // held until the launches are enqueued
   p.q = static_cast<const half_t*>(q);
   p.q_indptr = q_indptr;
   p.pages = static_cast<const half_t*>(pages);
@@ -995,7 +996,8 @@ static int mla_entry(const void* q, const int32_t* q_indptr, const void* pages, 
     const size_t part_rows = static_cast<size_t>(cslots) * h_q;
     const size_t part_o_bytes = part_rows * DV * sizeof(half_t);
     const size_t part_lse_bytes = (part_rows * sizeof(float) + 15) / 16 * 16;
-    char* ws = lease_scratch(kScratchMla, as_stream(stream), part_o_bytes + part_lse_bytes + cslots * sizeof(int4), 0).ptr;
+    lease = lease_scratch(kScratchMla, as_stream(stream), part_o_bytes + part_lse_bytes + cslots * sizeof(int4), 0);
+    char* ws = lease.ptr;
     p.part_o = reinterpret_cast<half_t*>(ws);
     p.part_lse = reinterpret_cast<float*>(ws + part_o_bytes);
     p.slot_plan = reinterpret_cast<int4*>(ws + part_o_bytes + part_lse_bytes);

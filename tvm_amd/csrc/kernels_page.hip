@@ -326,56 +326,6 @@ __global__ __launch_bounds__(256) void merge_state_inplace_kernel(half_t* __rest
   if (c == 0) s[row] = log2f(s_val + s_other_val) + s_max;
 }
 
-// ------------------------------------------------------------------------------------------
-// Measurement utilities: a plain streaming read and a plain copy of known size, used to
-// calibrate what the memory system delivers and to scale hardware traffic counters.
-// ------------------------------------------------------------------------------------------
-template <bool NT>  // NT: loads carry the non-temporal hint, as the decode kernel's do
-__global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ src, int64_t n16,
-                                                          uint32_t* __restrict__ sink) {
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  uint32_t acc = 0;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride) {
-    const Vec16 v = NT ? ld16_nt(src + i) : ld16(src + i);
-    acc ^= v.w[0] ^ v.w[1] ^ v.w[2] ^ v.w[3];
-  }
-  if (acc == 0x9e3779b9u) sink[0] = acc;  // keeps the loads alive; practically never taken
-}
-
-__global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
-                                                          int64_t n16) {
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
-}
-
-// Matrix-core calibration: every wave runs `iters` rounds of 8 independent-enough
-// v_mfma_f32_32x32x16_f16 (4 accumulators) on operands it read once from `operands` (8 halfs per lane
-// for A and for B).  Nothing else is in the loop: this is what the matrix pipes of the box deliver,
-// and it depends on the operand values (the clock drops with random data).
-__global__ __launch_bounds__(256) void mfma_loop_kernel(const half_t* __restrict__ operands, float* __restrict__ out,
-                                                        int iters) {
-  const int tid = threadIdx.x;
-  const half8_t a = *reinterpret_cast<const half8_t*>(operands + tid * 16);
-  const half8_t b = *reinterpret_cast<const half8_t*>(operands + tid * 16 + 8);
-  float16_t acc[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
-  }
-  for (int it = 0; it < iters; ++it) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[j & 3], 0, 0, 0);
-  }
-  float sum = 0.f;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) sum += acc[j][i];
-  }
-  out[static_cast<int64_t>(blockIdx.x) * 256 + tid] = sum;
-}
-
 inline dim3 grid_for(int64_t threads, int block = 256) { return dim3(static_cast<unsigned>((threads + block - 1) / block)); }
 
 }  // namespace tvmkv
@@ -676,45 +626,6 @@ int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr, const 
   hipLaunchKernelGGL(compact_kv_copy_kernel, grid_for(threads), dim3(256), 0, as_stream(stream),
                      static_cast<half_t*>(pages), copy_length_indptr, copy_src_dst_pos, batch_size,
                      total_copy_length, num_kv_heads, page_size, head_dim);
-  KV_LAUNCH_CHECK();
-  KV_API_END();
-}
-
-int tvmkv_stream_read_nt(const void* src, int64_t num_bytes, void* sink, void* stream) {
-  KV_API_BEGIN();
-  KV_CHECK(src && sink && num_bytes >= 0 && num_bytes % 16 == 0) << "stream_read_nt: bad arguments";
-  if (num_bytes == 0) return TVMKV_OK;
-  hipLaunchKernelGGL(stream_read_kernel<true>, dim3(256 * 16), dim3(256), 0, as_stream(stream),
-                     static_cast<const uint4*>(src), num_bytes / 16, static_cast<uint32_t*>(sink));
-  KV_LAUNCH_CHECK();
-  KV_API_END();
-}
-
-int tvmkv_stream_read(const void* src, int64_t num_bytes, void* sink, void* stream) {
-  KV_API_BEGIN();
-  KV_CHECK(src && sink && num_bytes >= 0 && num_bytes % 16 == 0) << "stream_read: bad arguments";
-  if (num_bytes == 0) return TVMKV_OK;
-  hipLaunchKernelGGL(stream_read_kernel<false>, dim3(256 * 16), dim3(256), 0, as_stream(stream),
-                     static_cast<const uint4*>(src), num_bytes / 16, static_cast<uint32_t*>(sink));
-  KV_LAUNCH_CHECK();
-  KV_API_END();
-}
-
-int tvmkv_stream_copy(const void* src, void* dst, int64_t num_bytes, void* stream) {
-  KV_API_BEGIN();
-  KV_CHECK(src && dst && num_bytes >= 0 && num_bytes % 16 == 0) << "stream_copy: bad arguments";
-  if (num_bytes == 0) return TVMKV_OK;
-  hipLaunchKernelGGL(stream_copy_kernel, dim3(256 * 16), dim3(256), 0, as_stream(stream),
-                     static_cast<const uint4*>(src), static_cast<uint4*>(dst), num_bytes / 16);
-  KV_LAUNCH_CHECK();
-  KV_API_END();
-}
-
-int tvmkv_mfma_loop(const void* operands, float* out, int32_t iters, int32_t workgroups, void* stream) {
-  KV_API_BEGIN();
-  KV_CHECK(operands && out && iters >= 0 && workgroups > 0) << "mfma_loop: bad arguments";
-  hipLaunchKernelGGL(mfma_loop_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0, as_stream(stream),
-                     static_cast<const half_t*>(operands), out, iters);
   KV_LAUNCH_CHECK();
   KV_API_END();
 }

@@ -34,13 +34,6 @@
 
 namespace tvmkv {
 
-// Clock probe (a measurement aid, off unless tvmkv_prefill_clock_probe(1) was called): thread 0 of
-// every workgroup adds the shader cycles (s_memtime) and the 100 MHz ticks (s_memrealtime) that
-// passed between its start and its end, and 1, to these three counters.  cycles / ticks * 100 MHz
-// is the shader clock the chip actually ran the kernel at.
-__device__ unsigned long long prefill_clock_counters[4];
-static int g_prefill_clock_probe = 0;
-
 // Pipeline depth: as many stages as fit next to the other workgroups of the CU (NW = 4: one more, two
 // more at head dim 64, whose kernels need a third of the registers) or alone (NW = 8).
 constexpr int prefill_stages(int dqk, int dv) {
@@ -99,11 +92,6 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
   // two stages; the workgroup's 4 waves each copy 16 of the 64 token rows of a tile
   extern __shared__ __attribute__((aligned(16))) half_t lds_tiles[];
 
-  unsigned long long probe_cycles = 0, probe_ticks = 0;
-  if (p.clock_probe) {
-    probe_cycles = __builtin_amdgcn_s_memtime();
-    probe_ticks = __builtin_amdgcn_s_memrealtime();
-  }
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
@@ -696,12 +684,6 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
     }
   }
 
-  if (p.clock_probe && tid == 0) {
-    atomicAdd(&prefill_clock_counters[0], __builtin_amdgcn_s_memtime() - probe_cycles);
-    atomicAdd(&prefill_clock_counters[1], __builtin_amdgcn_s_memrealtime() - probe_ticks);
-    atomicAdd(&prefill_clock_counters[2], 1ull);
-  }
-
   // ---- epilogue ------------------------------------------------------------------------------
   lsum = sum_xor32(lsum);
   const float denom = lsum + fast_exp2(kNegInit - m);  // the d = 1 of the initial state
@@ -772,11 +754,9 @@ static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const Pr
                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     attr_set = true;
   }
-  PrefillParams launch = p;
-  launch.clock_probe = g_prefill_clock_probe;
   hipLaunchKernelGGL((prefill_kernel<DQK, DV, SRC, PS, EXT, STREAM>),
                      dim3(p.h_kv, static_cast<unsigned>(slots), static_cast<unsigned>(std::max(1, p.kv_splits))),
-                     dim3(NW * 64), lds_bytes, stream, launch, div);
+                     dim3(NW * 64), lds_bytes, stream, p, div);
 }
 
 // ---- split over the keys ---------------------------------------------------------------------
@@ -870,6 +850,7 @@ struct KvSplit {
   int64_t rows;
   int splits;
   int merge_into = 0;
+  ScratchLease lease{};
   KvSplit(PrefillParams& p, int64_t total_q, int64_t avg_keys, int dv, hipStream_t stream)
       : output(p.output), lse(p.lse), rows(total_q * p.h_q), splits(1) {
     // at most one row tile per (sequence, kv head) on average: the paged kernels stream the K/V rows
@@ -878,7 +859,8 @@ struct KvSplit {
     if (splits <= 1) return;
     const size_t o_bytes = static_cast<size_t>(splits) * rows * dv * sizeof(half_t);
     const size_t lse_bytes = static_cast<size_t>(splits) * rows * sizeof(float);
-    char* ws = lease_scratch(kScratchPrefill, stream, o_bytes + lse_bytes, 0).ptr;
+    lease = lease_scratch(kScratchPrefill, stream, o_bytes + lse_bytes, 0);  // held until the merge is enqueued
+    char* ws = lease.ptr;
     p.output = reinterpret_cast<half_t*>(ws);
     p.lse = reinterpret_cast<float*>(ws + o_bytes);
     p.kv_splits = splits;
@@ -940,26 +922,6 @@ static void launch_prefill(const PrefillParams& p, int64_t total_q, bool ext, do
 using namespace tvmkv;
 
 extern "C" {
-
-int tvmkv_prefill_clock_probe(int32_t enable) {
-  KV_API_BEGIN();
-  g_prefill_clock_probe = enable != 0;
-  KV_API_END();
-}
-
-int tvmkv_prefill_clock_probe_read(uint64_t* counters, int32_t reset) {
-  KV_API_BEGIN();
-  KV_CHECK(counters != nullptr) << "prefill_clock_probe_read: NULL output";
-  unsigned long long host[4] = {0, 0, 0, 0};
-  HIP_CHECK(hipDeviceSynchronize());
-  HIP_CHECK(hipMemcpyFromSymbol(host, HIP_SYMBOL(prefill_clock_counters), sizeof(host)));
-  for (int i = 0; i < 3; ++i) counters[i] = host[i];
-  if (reset) {
-    const unsigned long long zero[4] = {0, 0, 0, 0};
-    HIP_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(prefill_clock_counters), zero, sizeof(zero)));
-  }
-  KV_API_END();
-}
 
 int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const void* k, const void* v,
                                   const int32_t* kv_indptr, const int32_t* q_rope_position,

@@ -686,6 +686,16 @@ void KVBookkeeper::BuildTreeMasks(const int64_t* token_tree_parent_ptr, int64_t 
 
 // :1566-1659
 bool KVBookkeeper::CommitAcceptedTokenTreeNodes(const int64_t* seq_ids, const int64_t* leaf_indices, int num) {
+  // The reference takes the batch of the last step for granted (its only caller is its own VM); here the
+  // call comes through a C ABI: a different batch would index the step's arrays out of range or pop the
+  // wrong sequences, so it is refused before anything changes.
+  KV_CHECK(num >= 0 && static_cast<size_t>(num) == cur_seq_ids_.size())
+      << "commit_accepted_token_tree_nodes: " << num << " sequences, the last step had " << cur_seq_ids_.size();
+  for (int i = 0; i < num; ++i) {
+    KV_CHECK(seq_ids[i] == cur_seq_ids_[i])
+        << "commit_accepted_token_tree_nodes: sequence " << seq_ids[i] << " at position " << i
+        << ", the last step had sequence " << cur_seq_ids_[i] << " there";
+  }
   bool is_chain = true;
   for (int i = 0; i < num; ++i) {
     const SeqRecord& seq = seqs_[RequireSeq(seq_ids[i])];

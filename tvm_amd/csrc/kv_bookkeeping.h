@@ -12,6 +12,8 @@
 #ifndef TVMKV_CSRC_KV_BOOKKEEPING_H_
 #define TVMKV_CSRC_KV_BOOKKEEPING_H_
 
+#include <algorithm>
+#include <cstddef>
 #include <cstdint>
 #include <string>
 #include <unordered_map>
@@ -102,7 +104,17 @@ class KVBookkeeper {
   const std::vector<int32_t>& commit_copy_src_pos() const { return commit_src_; }
   const std::vector<int32_t>& commit_copy_dst_pos() const { return commit_dst_; }
   // (src page, target page, tokens) of every partial-page copy a fork has asked for since Clear
+  int64_t PageArenaInUse() const { return blocks_.ArenaInUse(); }
   const std::vector<int64_t>& CopyLog() const { return copy_log_; }
+  // The log only grows between two Clear() calls; once it holds more than kCopyLogCap numbers, the oldest
+  // of its first `consumed` numbers are dropped down to kCopyLogKeep.  Returns how many were dropped.
+  static constexpr size_t kCopyLogCap = 3 * 8192, kCopyLogKeep = 3 * 1024;
+  size_t TrimCopyLog(size_t consumed) {
+    if (copy_log_.size() <= kCopyLogCap) return 0;
+    const size_t drop = std::min(consumed, copy_log_.size() - kCopyLogKeep) / 3 * 3;
+    copy_log_.erase(copy_log_.begin(), copy_log_.begin() + static_cast<std::ptrdiff_t>(drop));
+    return drop;
+  }
   std::vector<int64_t> DumpState() const;
   AuxSpan FindAux(const std::string& name, int depth) const;
 

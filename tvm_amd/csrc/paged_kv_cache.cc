@@ -140,8 +140,7 @@ class PagedKVCache {
 
   // :1566-1659
   void CommitAcceptedTokenTreeNodes(const int64_t* seq_ids, const int64_t* leaf_indices, int num) {
-    const int64_t batch_size = book_->batch_size();
-    if (book_->CommitAcceptedTokenTreeNodes(seq_ids, leaf_indices, num)) CompactKVCopy(batch_size);
+    if (book_->CommitAcceptedTokenTreeNodes(seq_ids, leaf_indices, num)) CompactKVCopy(num);
     IssuePageCopies();  // a pop into a shared block forks
   }
 
@@ -545,6 +544,12 @@ class PagedKVCache {
   void IssuePageCopies() {
     const std::vector<int64_t>& log = book_->CopyLog();
     if (page_copies_issued_ == log.size()) return;
+    // everything up to here is (about to be) issued: a long log drops its oldest entries on the way out
+    struct Trim {
+      KVBookkeeper* book;
+      size_t* issued;
+      ~Trim() { *issued -= book->TrimCopyLog(*issued); }
+    } trim{book_.get(), &page_copies_issued_};
     if (device_ < 0) {
       page_copies_issued_ = log.size();
       return;

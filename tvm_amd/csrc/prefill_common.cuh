@@ -56,7 +56,6 @@ struct PrefillParams {
   int64_t split_rows;
   int page_shift;   // pages hold 16 << page_shift tokens; the kernel walks them as runs of 16-token pages
   int stream_kv;    // != 0: every K/V row is read by one row tile only: copy it with the streaming hint
-  int clock_probe;  // != 0: add this workgroup's shader cycles and 100 MHz ticks to the probe counters
 };
 
 // theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use

@@ -1,6 +1,8 @@
 // Tuning options and the scratch-buffer pool of the split-KV launchers (see runtime_support.h).
 #include "runtime_support.h"
 
+#include <hip/hip_runtime.h>
+
 #include <algorithm>
 #include <atomic>
 #include <cstdlib>
@@ -8,6 +10,7 @@
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 #include "common.h"
 
@@ -38,35 +41,74 @@ struct Scratch {
   char* ptr = nullptr;
   size_t bytes = 0;
   size_t counter_bytes = 0;
-  uint32_t epoch = 0;
+  uint64_t launches = 0;       // launches served from this buffer; the epoch of a launch is its low half
+  bool seen_in_capture = false;  // a graph under capture has recorded this buffer's address
 };
 std::mutex g_scratch_mutex;
 std::map<std::tuple<int, hipStream_t, int>, Scratch> g_scratch;
+// Buffers that a captured graph may still name after their entry has grown: kept until the process ends.
+std::vector<char*> g_retired;
+
+__global__ void zero_words_kernel(unsigned long long* words, size_t count) {
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < count;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    words[i] = 0ull;
+  }
+}
+
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (stream != nullptr && hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+    (void)hipGetLastError();
+    capture = hipStreamCaptureStatusNone;
+  }
+  return capture != hipStreamCaptureStatusNone;
+}
 
 }  // namespace
 
 int64_t option(Option id) { return g_options.value[id].load(std::memory_order_relaxed); }
 
+uint32_t next_scratch_epoch(uint64_t* launches, bool* wrapped) {
+  ++*launches;
+  *wrapped = false;
+  if (static_cast<uint32_t>(*launches) == 0) {  // 2^32 launches: the epochs start over at 1
+    ++*launches;
+    *wrapped = true;
+  }
+  return static_cast<uint32_t>(*launches);
+}
+
+void zero_scratch_counters(char* ptr, size_t counter_bytes, hipStream_t stream) {
+  if (counter_bytes == 0) return;
+  const size_t words = counter_bytes / sizeof(unsigned long long);
+  hipLaunchKernelGGL(zero_words_kernel, dim3(64), dim3(256), 0, stream, reinterpret_cast<unsigned long long*>(ptr), words);
+  HIP_CHECK(hipGetLastError());
+}
+
 ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, size_t counter_bytes) {
   int dev = 0;
   HIP_CHECK(hipGetDevice(&dev));
-  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  // held by the lease until the caller has enqueued its launch: a thread that grows (and frees) this
+  // entry's buffer first synchronises the stream, and by then the launch is on it
+  std::unique_lock<std::mutex> lock(g_scratch_mutex);
   Scratch& s = g_scratch[std::make_tuple(dev, stream, static_cast<int>(user))];
+  const bool capturing = stream_is_capturing(stream);
   if (s.bytes < bytes || s.counter_bytes < counter_bytes) {
-    // growing means hipMalloc, hipFree and a memset: none of them belongs into a graph under capture
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (stream != nullptr && hipStreamIsCapturing(stream, &capture) != hipSuccess) {
-      (void)hipGetLastError();
-      capture = hipStreamCaptureStatusNone;
-    }
-    KV_CHECK(capture == hipStreamCaptureStatusNone)
+    // growing means hipMalloc and hipFree: neither belongs into a graph under capture
+    KV_CHECK(!capturing)
         << "the stream is being captured into a graph and this call needs " << bytes << " bytes of scratch memory that "
         << "are not allocated yet: run the same call once on this stream before the capture starts, or use "
         << "tvmkv_batch_decode_paged_kv_noalloc";
     if (s.ptr != nullptr) {
-      // launches still queued on this stream read the old buffer; nobody else ever does
-      HIP_CHECK(hipStreamSynchronize(stream));
-      HIP_CHECK(hipFree(s.ptr));
+      if (s.seen_in_capture) {
+        // a captured graph holds this address in its kernel arguments and may be replayed at any time
+        g_retired.push_back(s.ptr);
+      } else {
+        // launches still queued on this stream read the old buffer; nobody else ever does
+        HIP_CHECK(hipStreamSynchronize(stream));
+        HIP_CHECK(hipFree(s.ptr));
+      }
       s = Scratch{};
     }
     const size_t want = bytes + bytes / 2;
@@ -75,15 +117,46 @@ ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, s
     s.ptr = static_cast<char*>(ptr);
     s.bytes = want;
     s.counter_bytes = counter_bytes;
-    s.epoch = 0;
-    HIP_CHECK(hipMemsetAsync(s.ptr, 0, counter_bytes, stream));
+    s.launches = 0;
+    zero_scratch_counters(s.ptr, counter_bytes, stream);  // a kernel, not a memset node
   }
-  if (++s.epoch == 0) {
-    // 2^32 launches on this buffer: start the epochs over from clean counters
-    HIP_CHECK(hipMemsetAsync(s.ptr, 0, s.counter_bytes, stream));
-    s.epoch = 1;
+  s.seen_in_capture = s.seen_in_capture || capturing;
+  bool wrapped = false;
+  const uint32_t epoch = next_scratch_epoch(&s.launches, &wrapped);
+  // Every launch leaves its counters at (epoch, 0), and the kernels bring a word of an older epoch up to
+  // their own with a maximum: after the wrap an abandoned launch's word would compare as newer, so the
+  // counters start over from zero (a kernel in stream order; recorded into a graph it is harmless).
+  if (wrapped) zero_scratch_counters(s.ptr, s.counter_bytes, stream);
+  return ScratchLease{s.ptr, epoch, std::move(lock)};
+}
+
+void release_scratch(hipStream_t stream) {
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  KV_CHECK(!stream_is_capturing(stream)) << "tvmkv_release_scratch: the stream is being captured";
+  bool synced = false;
+  for (auto it = g_scratch.begin(); it != g_scratch.end();) {
+    if (std::get<0>(it->first) != dev || std::get<1>(it->first) != stream) {
+      ++it;
+      continue;
+    }
+    if (it->second.ptr != nullptr) {
+      if (it->second.seen_in_capture) {
+        g_retired.push_back(it->second.ptr);
+      } else {
+        if (!synced) HIP_CHECK(hipStreamSynchronize(stream));
+        synced = true;
+        HIP_CHECK(hipFree(it->second.ptr));
+      }
+    }
+    it = g_scratch.erase(it);
   }
-  return ScratchLease{s.ptr, s.epoch};
+}
+
+void debug_set_scratch_launches(uint64_t launches) {
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  for (auto& entry : g_scratch) entry.second.launches = launches;
 }
 
 // Work items of a decode launch: every item pays ~2 us of fixed cost (locating its sequence, q, the
@@ -126,6 +199,19 @@ int tvmkv_set_option(const char* name, int64_t value) {
     }
   }
   KV_CHECK(false) << "tvmkv_set_option: unknown option \"" << name << "\"";
+  KV_API_END();
+}
+
+uint32_t tvmkv_debug_next_scratch_epoch(uint64_t* launches, int32_t* wrapped) {
+  bool w = false;
+  const uint32_t epoch = tvmkv::next_scratch_epoch(launches, &w);
+  *wrapped = w ? 1 : 0;
+  return epoch;
+}
+
+int tvmkv_release_scratch(void* stream) {
+  KV_API_BEGIN();
+  tvmkv::release_scratch(static_cast<hipStream_t>(stream));
   KV_API_END();
 }
 

@@ -7,6 +7,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <mutex>
 
 namespace tvmkv {
 
@@ -23,16 +24,29 @@ int64_t option(Option id);
 
 // Scratch memory of a split-KV launch.  A buffer belongs to one (device, stream, user): launches on
 // one stream are ordered and may share it, launches on different streams (two caches, two layers in
-// flight) never do.  The first `counter_bytes` bytes hold arrival counters that are never reset:
-// every launch gets a new `epoch`, a counter is a 64-bit word (epoch << 32 | arrivals), and a word
-// left behind by an earlier launch -- also one that failed or was abandoned half way -- carries an
-// older epoch and counts as zero.
+// flight) never do.  The first `counter_bytes` bytes hold arrival counters that are not reset between
+// launches: every launch gets a new `epoch`, a counter is a 64-bit word (epoch << 32 | arrivals), and a
+// word left behind by an earlier launch -- also one that failed or was abandoned half way -- carries an
+// older epoch and counts as zero.  The epoch is the low half of a 64-bit launch count; when it wraps
+// (2^32 launches on one buffer) the counters are cleared by a kernel in stream order and the epochs
+// start over at 1.
+// The lease keeps the pool locked until it is destroyed: hold it until the launch that uses the buffer
+// has been enqueued, so that a second host thread on the same stream cannot free the buffer in between.
 struct ScratchLease {
   char* ptr;        // device memory, at least the requested size, 256-byte aligned
   uint32_t epoch;   // never 0
+  std::unique_lock<std::mutex> lock;
 };
 enum ScratchUser { kScratchDecode = 0, kScratchMla = 1, kScratchPrefill = 2 };
 ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, size_t counter_bytes);
+// Frees the buffers of (current device, stream) after synchronising the stream; a buffer whose address
+// a graph under capture has recorded is kept until the process ends instead.
+void release_scratch(hipStream_t stream);
+// The epoch of the next launch from a 64-bit launch count (host arithmetic only).
+uint32_t next_scratch_epoch(uint64_t* launches, bool* wrapped);
+void zero_scratch_counters(char* ptr, size_t counter_bytes, hipStream_t stream);
+// Test aid: sets the launch count of every pooled buffer (to run a launch across the epoch wrap).
+void debug_set_scratch_launches(uint64_t launches);
 
 // Chunk-slot arithmetic of the decode split, on the host (the device functions of the same names in
 // kernels_decode.hip compute the same values; the tests compare both against a direct enumeration).

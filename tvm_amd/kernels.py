@@ -242,39 +242,3 @@ def compact_kv_copy(pages, copy_length_indptr, copy_src_dst_pos, batch_size):
     num_pages, _, hkv, ps, d = pages.shape
     check(lib().tvmkv_compact_kv_copy(_p(pages), _p(copy_length_indptr), _p(copy_src_dst_pos), batch_size,
                                       copy_src_dst_pos.shape[1], num_pages, hkv, ps, d, _stream()))
-
-
-def mfma_loop(operands, out, iters):
-    """Matrix-core calibration loop: operands (256, 16) fp16, out (workgroups, 256) fp32."""
-    _f16(operands)
-    assert operands.numel() == 256 * 16 and out.dtype == torch.float32 and out.shape[1] == 256
-    check(lib().tvmkv_mfma_loop(_p(operands), _p(out), int(iters), out.shape[0], _stream()))
-
-
-def prefill_clock_probe(enable):
-    """Switches the clock probe of the prefill kernels on or off (a measurement aid)."""
-    check(lib().tvmkv_prefill_clock_probe(int(bool(enable))))
-
-
-def prefill_clock_probe_read(reset=True):
-    """(shader cycles, 100 MHz ticks, workgroups) summed over the prefill launches since the last
-    reset on the current device; cycles / ticks * 100 is the average shader clock in MHz."""
-    import ctypes
-    buf = (ctypes.c_uint64 * 3)()
-    check(lib().tvmkv_prefill_clock_probe_read(ctypes.cast(buf, ctypes.c_void_p), int(bool(reset))))
-    return int(buf[0]), int(buf[1]), int(buf[2])
-
-
-def stream_read_nt(src, sink):
-    """stream_read with non-temporal loads."""
-    check(lib().tvmkv_stream_read_nt(_p(src), src.numel() * src.element_size(), _p(sink), _stream()))
-
-
-def stream_read(src, sink):
-    """Plain streaming read of the whole tensor (bandwidth calibration)."""
-    check(lib().tvmkv_stream_read(_p(src), src.numel() * src.element_size(), _p(sink), _stream()))
-
-
-def stream_copy(src, dst):
-    """Plain copy of the whole tensor (bandwidth calibration, counter scaling)."""
-    check(lib().tvmkv_stream_copy(_p(src), _p(dst), src.numel() * src.element_size(), _stream()))
