@@ -249,6 +249,24 @@ int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t*
                                 int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
                                 int32_t d, int32_t page_size, int32_t sliding_window, void* stream);
 
+/* Slots 24 + 13 + 17 in one launch (no counterpart among the reference's kernels; what
+ * AttentionWithFusedQKV does for a decode step, src/runtime/vm/paged_kv_cache.cc:1360-1373 and
+ * :2236-2260, as three kernels): the decode step of one layer over a plain cache.  qkv is the fused
+ * (batch, h_q + 2 h_kv, d) tensor of the step, one new token per sequence.  The kernel reads q from it
+ * and rotates it at q_rope_position[b] (apply_rope != 0: rotate-half RoPE with the default frequencies
+ * theta^(-2i/d); 0: no rotation); the work items of every sequence's last chunk rotate the new k row the
+ * same way and write it and the v row to slot append_position_map[b] (page * page_size + offset, -1 =
+ * none) of `pages`, wait for those stores and then attend to the slot like to any cached token.  The
+ * page table must already cover the new token, i.e. the step appends before it attends
+ * (paged_kv_cache.cc:990-997).  Results as tvmkv_batch_decode_paged_kv; the same head dims and page
+ * sizes; a group of more than 16 query heads per kv head is served by work items of 32 heads. */
+int tvmkv_fused_decode_step(const void* qkv, void* pages, const int32_t* page_indptr, const int32_t* page_values,
+                            const int32_t* last_page_len, const int32_t* q_rope_position,
+                            const int32_t* append_position_map, void* output, float* lse, int64_t apply_rope,
+                            double rope_scale, double rope_theta, double sm_scale, int32_t batch_size,
+                            int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv, int32_t d,
+                            int32_t page_size, void* stream);
+
 /* tvmkv_batch_decode_paged_kv for callers that cannot allocate.  It has no counterpart in the
  * reference; it is for code under HIP graph capture, tight serving loops and harnesses that
  * forbid hipMalloc.  Arguments and results as tvmkv_batch_decode_paged_kv.  Its scratch memory
@@ -362,7 +380,9 @@ int tvmkv_compact_kv_copy(void* pages, const int32_t* copy_length_indptr,
  *   prefill_kv_splits      > 0: the paged prefill, one-pass chunked prefill and paged tree-attention launches
  *                          split the keys of every row tile over this many workgroups (at most 64) and merge
  *                          the states in a second launch; 0 = derived from the shapes (launches with few row
- *                          tiles and long cached sequences are split, all others are not) */
+ *                          tiles and long cached sequences are split, all others are not)
+ *   no_fused_decode_step   != 0: the cache object runs a plain decode step as two launches (split + RoPE +
+ *                          append, then decode attention) instead of tvmkv_fused_decode_step */
 int tvmkv_set_option(const char* name, int64_t value);
 int tvmkv_get_option(const char* name, int64_t* value);
 

@@ -21,12 +21,6 @@ int tvmkvb_stream_copy(const void* src, void* dst, int64_t num_bytes, void* stre
  * accumulators, nothing else in the loop) on the A and B fragments read from `operands` (256 lanes x 16
  * halfs); `out` gets workgroups x 256 floats.  2 * 32 * 32 * 16 * 8 * iters * 4 * workgroups flop. */
 int tvmkvb_mfma_loop(const void* operands, float* out, int32_t iters, int32_t workgroups, void* stream);
-/* One wave that reads the shader-cycle counter and the 100 MHz counter until *stop_flag (pinned host
- * memory the host sets to non-zero) or until max_ticks 100 MHz ticks (at most 10^9) have passed, then
- * writes {cycles, ticks} to `out` (two device uint64).  Launched on a second stream beside the kernel under
- * test: cycles / ticks * 100 MHz is the shader clock during that time. */
-int tvmkvb_clock_sampler(const int32_t* stop_flag, uint64_t max_ticks, uint64_t* out, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -941,25 +941,6 @@ def test_measurement_utilities():
     assert torch.all(out == 4.0 * 16 * 8 * iters)
 
 
-def test_clock_sampler_runs_beside_a_kernel_and_ends():
-    """The one-wave clock sampler on its own stream: it ends when the host sets the flag (and by itself
-    after max_seconds), and reports a plausible shader clock for the time a kernel ran beside it."""
-    from tvm_amd import bench_aids as A
-
-    ops = torch.full((256, 16), 0.5, dtype=torch.float16, device=DEV)
-    out = torch.zeros((256, 256), dtype=torch.float32, device=DEV)
-    with A.ClockSampler(max_seconds=2.0) as clock:
-        for _ in range(20):
-            A.mfma_loop(ops, out, 512)
-    assert 200.0 < clock.mhz < 4000.0, clock.mhz
-    # without the flag it ends after max_seconds by itself
-    sampler = A.ClockSampler(max_seconds=0.05)
-    sampler.__enter__()
-    sampler.stream.synchronize()
-    assert int(sampler.out.cpu()[1]) >= int(0.05 * 1e8)
-    sampler.__exit__(None, None, None)
-
-
 def test_scratch_epoch_wrap_and_release():
     """Split-KV launches across the wrap of the 32-bit epoch that tags their arrival counters (the launch
     count is set just below 2^32), through the pooled buffer and through the built-in one of the entry
@@ -995,3 +976,62 @@ def test_scratch_epoch_wrap_and_release():
         assert np.array_equal(o, base[0]) and np.array_equal(s, base[1])
     finally:
         tvm_amd.set_option("decode_chunk_pages", prev)
+
+
+# ------------------------------------------------------------------------------ fused decode step
+@pytest.mark.parametrize("hq,hkv,d,ps,apply_rope", [(32, 8, 128, 16, 1), (32, 8, 128, 16, 0), (8, 2, 64, 32, 1),
+                                                    (32, 1, 128, 16, 1), (64, 1, 128, 16, 1), (20, 1, 64, 16, 1),
+                                                    (16, 8, 256, 16, 1), (64, 8, 128, 64, 1)])
+def test_fused_decode_step(hq, hkv, d, ps, apply_rope):
+    """Split + RoPE + append + decode attention of a step in one launch (tvmkv_fused_decode_step) against
+    the oracle's three kernels, and against the library's own two launches: the slot of the new token holds
+    NaN patterns before the call, so a work item that attended before the append landed would show."""
+    rng = np.random.default_rng(90 + hq + d)
+    kv_lens = [1, 16, 17, 33, 700, 2500, 64, ps + 1, 3 * ps]   # the new token included
+    b = len(kv_lens)
+    npages = 4 + sum((n + ps - 1) // ps for n in kv_lens)
+    pages, ip, pv, last, _, _ = build_paged_kv(rng, kv_lens, npages, hkv, ps, d)
+    slots = np.array([pv[ip[i] + (n - 1) // ps] * ps + (n - 1) % ps for i, n in enumerate(kv_lens)], np.int32)
+    q_pos = (rng.integers(0, 3000, size=b) + np.array(kv_lens) - 1).astype(np.int32)
+    qkv = rng.standard_normal((b, hq + 2 * hkv, d)).astype(F16)
+    # oracle: split + RoPE, append, decode
+    eq, ek, ev = np.zeros((b, hq, d), F16), np.zeros((b, hkv, d), F16), np.zeros((b, hkv, d), F16)
+    ok.fused_rope(qkv, q_pos, eq, ek, ev, apply_rope)
+    epages = pages.copy()
+    ok.transpose_append(epages, ek, ev, slots)
+    eo, el = np.zeros((b, hq, d), F16), np.zeros((b, hq), np.float32)
+    z = np.zeros(b, np.int32)
+    ok.decode(eq, epages, ip, pv, last, z, z, eo, el, 0, 1.0, 1e4, d ** -0.5)
+    # the new token's slot is poisoned on the device side
+    poisoned = pages.copy()
+    for s in slots:
+        poisoned[s // ps, :, :, s % ps, :] = np.float16(np.nan)
+    # the library's two launches
+    p2 = dev(poisoned)
+    q2, k2, v2 = (torch.zeros(a.shape, dtype=torch.float16, device=DEV) for a in (eq, ek, ev))
+    o2 = torch.zeros((b, hq, d), dtype=torch.float16, device=DEV)
+    l2 = torch.zeros((b, hq), dtype=torch.float32, device=DEV)
+    K.fused_rope_append(dev(qkv), i32(q_pos), q2, k2, v2, apply_rope, p2, i32(slots), 1.0, 1e4)
+    K.batch_decode_paged_kv(q2, p2, i32(ip), i32(pv), i32(last), i32(z), i32(z), o2, l2, 0, 1.0, 1e4, d ** -0.5)
+    # one launch
+    p1 = dev(poisoned)
+    o1 = torch.full((b, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    l1 = torch.full((b, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.fused_decode_step(dev(qkv), p1, i32(ip), i32(pv), i32(last), i32(q_pos), i32(slots), o1, l1, apply_rope, 1.0, 1e4,
+                        d ** -0.5)
+    assert torch.equal(p1, p2), "the fused step must leave the pool as split + RoPE + append does"
+    gp = host(p1)
+    assert np.array_equal(gp[:, 1], epages[:, 1])                      # V rows: a copy
+    assert_close(gp[:, 0], epages[:, 0], atol=2e-3, rtol=1e-3, what="appended K rows vs oracle")  # one fp16 ulp
+    assert_close(host(o1), eo, what="fused step out vs oracle")
+    assert_close(host(l1), el, atol=1e-3, rtol=1e-4, what="fused step lse vs oracle")
+    assert_close(host(o1), host(o2), atol=2e-3, rtol=2e-3, what="fused step out vs two launches")
+
+
+def test_decode_group_of_64_heads():
+    """One kv head for 64 query heads: two work items of 32 heads per chunk; 16 kv heads x 64: the same at head dim 64."""
+    for hq, hkv, d in ((64, 1, 128), (128, 2, 64)):
+        rng = np.random.default_rng(28)
+        go, gl, eo, el = _decode_both(rng, [5, 130, 3000, 16, 0], hq, hkv, d, 220)
+        assert_close(go, eo, what=f"decode out {hq}/{hkv}/{d}")
+        assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"decode lse {hq}/{hkv}/{d}")

@@ -45,6 +45,8 @@ SIGNATURES = {
                                                  c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_decode_paged_kv_noalloc": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32,
                                                          c_i32, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_fused_decode_step": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32, c_i32, c_i32, c_i32,
+                                             c_vp],
     "tvmkv_batch_tree_attn": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i32, c_i32, c_i32, c_vp],
     "tvmkv_tree_attn_paged_kv": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_vp, c_vp, c_i32, c_i64, c_i64, c_i64,
                                                c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
@@ -116,7 +118,6 @@ BENCH_SIGNATURES = {
     "tvmkvb_stream_read_nt": [c_vp, c_i64, c_vp, c_vp],
     "tvmkvb_stream_copy": [c_vp, c_vp, c_i64, c_vp],
     "tvmkvb_mfma_loop": [c_vp, c_vp, c_i32, c_i32, c_vp],
-    "tvmkvb_clock_sampler": [c_vp, ctypes.c_uint64, c_vp, c_vp],
 }
 
 _lib = None

@@ -1,8 +1,7 @@
 // Measurement aids of the benchmark, built into their own library (libtvmkv_bench.so) so that the
 // product library carries product code only: plain streaming reads and a copy of known size (what the
 // memory system of the box delivers; the scale of the hardware traffic counters), a loop of nothing but
-// fp16 matrix instructions (what the matrix cores deliver), and a clock sampler (the shader clock a
-// kernel on another stream really runs at).  None of it has a counterpart in the reference.
+// fp16 matrix instructions (what the matrix cores deliver).  None of it has a counterpart in the reference.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -61,27 +60,6 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(const _Float16* __restri
   out[static_cast<int64_t>(blockIdx.x) * 256 + tid] = sum;
 }
 
-// One wave that sleeps and reads two clocks: s_memtime counts shader cycles, s_memrealtime 100 MHz
-// ticks.  It ends when the host sets *stop (pinned host memory) or after max_ticks, whichever comes
-// first, so it always ends; out = {cycles, ticks} over its life.  Run on a second stream beside the
-// kernel under test, cycles / ticks * 100 MHz is the shader clock that kernel ran at.
-__global__ __launch_bounds__(64) void clock_sampler_kernel(const int* stop, unsigned long long max_ticks,
-                                                           unsigned long long* out) {
-  if (threadIdx.x != 0) return;
-  const unsigned long long c0 = __builtin_amdgcn_s_memtime();
-  const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
-  unsigned long long c1 = c0, t1 = t0;
-  for (;;) {
-    __builtin_amdgcn_s_sleep(127);
-    c1 = __builtin_amdgcn_s_memtime();
-    t1 = __builtin_amdgcn_s_memrealtime();
-    if (t1 - t0 >= max_ticks) break;
-    if (__hip_atomic_load(stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) break;
-  }
-  out[0] = c1 - c0;
-  out[1] = t1 - t0;
-}
-
 int finish() { return static_cast<int>(hipGetLastError()); }
 
 }  // namespace
@@ -116,14 +94,6 @@ int tvmkvb_mfma_loop(const void* operands, float* out, int32_t iters, int32_t wo
   if (!operands || !out || iters < 0 || workgroups <= 0) return -1;
   hipLaunchKernelGGL(mfma_loop_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<const _Float16*>(operands), out, iters);
-  return finish();
-}
-
-int tvmkvb_clock_sampler(const int32_t* stop_flag, uint64_t max_ticks, uint64_t* out, void* stream) {
-  if (!stop_flag || !out || max_ticks == 0 || max_ticks > 1000000000ull) return -1;  // at most 10 s
-  hipLaunchKernelGGL(clock_sampler_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
-                     reinterpret_cast<const int*>(stop_flag), static_cast<unsigned long long>(max_ticks),
-                     reinterpret_cast<unsigned long long*>(out));
   return finish();
 }
 

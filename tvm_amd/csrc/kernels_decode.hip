@@ -59,6 +59,14 @@ struct DecodeParams {
   int chunk_pages;
   int page_shift;  // pages hold 16 << page_shift tokens; the kernel walks them as runs of 16-token pages
   float scale_log2;  // sm_scale * log2(e)
+  // fused step (decode_mfma_kernel<..., FUSED = true>): the launch does the split + RoPE + append of the
+  // step's new token itself.  q is read from the fused (B, h_q + 2 h_kv, D) tensor and rotated at
+  // q_rope_position[b]; the work items of a sequence's last chunk rotate its new k row, write it and the
+  // v row to slot append_slot[b] of the page pool, and then attend to them like to any cached token.
+  const half_t* qkv;
+  half_t* pages_rw;             // == pages
+  const int32_t* append_slot;   // (B) page * page_size + offset, -1 = none
+  int apply_rope;               // 0: q and k are used as they come
 };
 
 // Same answer as find_sequence, computed by one wavefront as a 64-ary search: the lanes probe
@@ -248,9 +256,16 @@ struct DecodeRopeDivisors {
 // the other: those rows are loaded without the streaming hint, so that the L2 keeps them for the next
 // head block (64 sequences, 32 query heads on one kv head: 0.077 against 0.083 ms).  Chosen at run
 // time inside one kernel, the load flavour cost the single-block case 4 %.
-template <bool EXT, int D, bool REREAD>
-__global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_kernel(DecodeParams p, int group, int num_items,
+// HB: blocks of 16 query heads per work item (1 or 2).  A group of up to 32 heads is one work item whose K
+// fragments and V tile feed the matrix instructions of both blocks, so the K/V rows are fetched once
+// (one kv head with 32 query heads: two items that each streamed the rows before); larger groups take
+// several such items.
+// FUSED (plain cache only): the launch also does the step's split + RoPE + append, see DecodeParams.
+template <bool EXT, int D, bool REREAD, int HB = 1, bool FUSED = false>
+__global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void decode_mfma_kernel(DecodeParams p, int group, int num_items,
                                                              DecodeRopeDivisors div) {
+  static_assert(HB == 1 || HB == 2, "head blocks per work item");
+  static_assert(!(FUSED && EXT), "the fused step exists for the plain cache");
   constexpr int PS = DM_PS;
   constexpr int KS = D / 32;                // k-steps of the score product
   constexpr int DB = D / 16;                // 16-wide output feature blocks
@@ -281,14 +296,15 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
 
   // Persistent workgroups: item = (chunk slot, kv head, block of 16 heads of the group), strided over
   // the grid.  Neighbouring workgroups take the head blocks and kv heads of one slot, i.e. the same pages.
-  const int head_blocks = (group + 15) >> 4;
+  constexpr int HPI = 16 * HB;  // query heads per work item
+  const int head_blocks = (group + HPI - 1) / HPI;
   for (int item = blockIdx.x; item < num_items; item += gridDim.x) {
   const int slot = item / (p.h_kv * head_blocks);
   const int rest = item - slot * (p.h_kv * head_blocks);
   const int kvh = rest / head_blocks;
   const int hb = rest - kvh * head_blocks;
-  const int hq0 = kvh * group + hb * 16;      // first query head of this item
-  const int heads = min(16, group - hb * 16);  // and how many
+  const int hq0 = kvh * group + hb * HPI;      // first query head of this item
+  const int heads = min(HPI, group - hb * HPI);  // and how many
   const int b = find_sequence_wave(p.page_indptr, p.batch_size, cp, slot, lane);
   const int pbeg = p.page_indptr[b];
   const int npages = p.page_indptr[b + 1] - pbeg;
@@ -319,13 +335,83 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
     k_pos0 = static_cast<float>(p.k_rope_pos_offset[b]);
   }
 
-  // Q^T fragments (B operand): column = head c16 of the group, contraction slots = 8 features.
-  half8_t qf[KS];
-  {
-    const half_t* qrow = p.q + (static_cast<int64_t>(b) * p.h_q + hq0 + c16) * D + g4 * 8;
+  // The fused step's append: every work item of the sequence's last chunk writes the new token's k row
+  // (rotated with the precise sinf / cosf, the arithmetic of fused_rope_kernel) and v row of its kv head
+  // to the page slot, waits until the stores have completed and meets the other waves at a barrier.  All
+  // loads of this workgroup come after that, through the same vector cache and L2 as the stores; the
+  // items of other head blocks of the same kv head write the same bytes.
+  if (FUSED && chunk == nchunks - 1) {
+    const int32_t aslot = p.append_slot[b];
+    if (aslot >= 0) {
+      const int page_tokens = PS << psh;
+      const half_t* krow = p.qkv + (static_cast<int64_t>(b) * (p.h_q + 2 * p.h_kv) + p.h_q + kvh) * D;
+      const half_t* vrow = krow + static_cast<int64_t>(p.h_kv) * D;
+      half_t* kdst = p.pages_rw + (static_cast<int64_t>(aslot / page_tokens) * 2 * p.h_kv + kvh) * head_stride +
+                     (aslot % page_tokens) * D;
+      half_t* vdst = kdst + static_cast<int64_t>(p.h_kv) * head_stride;
+      if (tid < D / 2) {
+        const float xl = static_cast<float>(krow[tid]);
+        const float xh = static_cast<float>(krow[tid + D / 2]);
+        if (p.apply_rope) {
+          const float freq = static_cast<float>(p.q_rope_position[b]) * p.rope_scale / div.v[tid];
+          const float cs = cosf(freq), sn = sinf(freq);
+          kdst[tid] = static_cast<half_t>(cs * xl + sn * (-xh));
+          kdst[tid + D / 2] = static_cast<half_t>(cs * xh + sn * xl);
+        } else {
+          kdst[tid] = krow[tid];
+          kdst[tid + D / 2] = krow[tid + D / 2];
+        }
+      } else if (tid >= 128 && tid < 128 + D / 8) {
+        st16(vdst + (tid - 128) * 8, ld16(vrow + (tid - 128) * 8));
+      }
+    }
+    wait_vmcnt<0>();
+    __syncthreads();
+  }
+
+  // The fused step rotates q itself.  A lane needs the angles of its 8 * KS/2 feature pairs, the same
+  // for every head and so for the 16 lanes of its group: each lane computes ONE of them (pair
+  // (i / 8) * 32 + g4 * 8 + i % 8 for i = c16, and i = 16 + c16 at head dim 256; spare lanes repeat one) and
+  // the group shares them through lane shuffles -- a twentieth of the sin / cos work of every lane
+  // computing all of its own.
+  constexpr int NA = 4 * KS;               // angles a lane needs
+  constexpr int PER_LANE = (NA + 15) / 16;  // angles a lane computes (head dim 256: two)
+  float rope_sn[PER_LANE], rope_cs[PER_LANE];
+  if (FUSED && p.apply_rope) {
+    const float q_pos = static_cast<float>(p.q_rope_position[b]) * p.rope_scale;
+#pragma unroll
+    for (int r = 0; r < PER_LANE; ++r) {
+      const int mine = min(r * 16 + c16, NA - 1);
+      sincos_reduced(q_pos / div.v[(mine >> 3) * 32 + g4 * 8 + (mine & 7)], rope_sn[r], rope_cs[r]);
+    }
+  }
+
+  // Q^T fragments (B operand): column = head c16 of block j of the item, contraction slots = 8 features.
+  half8_t qf[HB][KS];
+#pragma unroll
+  for (int j = 0; j < HB; ++j) {
+    const bool head_valid = j * 16 + c16 < heads;
+    const half_t* qrow = FUSED ? p.qkv + (static_cast<int64_t>(b) * (p.h_q + 2 * p.h_kv) + hq0 + j * 16 + c16) * D + g4 * 8
+                               : p.q + (static_cast<int64_t>(b) * p.h_q + hq0 + j * 16 + c16) * D + g4 * 8;
     Vec16 qv[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qv[ks] = c16 < heads ? ld16(qrow + ks * 32) : zero16();
+    for (int ks = 0; ks < KS; ++ks) qv[ks] = head_valid ? ld16(qrow + ks * 32) : zero16();
+    if (FUSED && p.apply_rope) {
+      // the arithmetic of rope_pair with the shared angles: fp32, one rounding to fp16
+#pragma unroll
+      for (int ks = 0; ks < KS / 2; ++ks) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int i = ks * 8 + e;  // angle i sits in lane i % 16 of this lane's group
+          const float cs = __shfl(rope_cs[i / 16], (lane & 48) + (i & 15), 64);
+          const float sn = __shfl(rope_sn[i / 16], (lane & 48) + (i & 15), 64);
+          const float xl = static_cast<float>(qv[ks].h8[e]);
+          const float xh = static_cast<float>(qv[ks + KS / 2].h8[e]);
+          qv[ks].h8[e] = static_cast<half_t>(cs * xl + sn * (-xh));
+          qv[ks + KS / 2].h8[e] = static_cast<half_t>(cs * xh + sn * xl);
+        }
+      }
+    }
     if (EXT && p.rotary) {
       // feature f < D/2 rotates with f + D/2: k-step ks with ks + KS/2
       const float q_pos = static_cast<float>(p.q_rope_position[b]) * p.rope_scale;
@@ -338,12 +424,20 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
       }
     }
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = qv[ks].h8;
+    for (int ks = 0; ks < KS; ++ks) qf[j][ks] = qv[ks].h8;
   }
-  float4_t o[DB];
+  float4_t o[HB][DB];
 #pragma unroll
-  for (int db = 0; db < DB; ++db) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
-  float m = kNegInit, lsum = 0.f;
+  for (int j = 0; j < HB; ++j) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db) o[j][db] = float4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  float m[HB], lsum[HB];
+#pragma unroll
+  for (int j = 0; j < HB; ++j) {
+    m[j] = kNegInit;
+    lsum[j] = 0.f;
+  }
 
   // V^T fragment via the transposing read: lane li of a 16-lane group points at 4 features of token
   // (li >> 2) of the group's 4 tokens and receives feature li of the group's 16 for the 4 tokens
@@ -428,61 +522,67 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
         }
       }
     }
-    // ---- S^T = K Q^T for both pages ---------------------------------------------------------
-    float4_t s[2];
+    // ---- S^T = K Q^T for both pages, every head block against the same K fragments --------------
+    // s[j][h][e]: head block j, token (pi+h)*PS + token_of(e), head j*16 + c16
+    auto token_of = [&](int e) { return KLINE ? 8 * (e >> 1) + 2 * g4 + (e & 1) : 4 * g4 + e; };
+    float4_t s[HB][2];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      if (KLINE) {
+    for (int j = 0; j < HB; ++j) {
 #pragma unroll
-        for (int tile = 0; tile < 2; ++tile) {
-          float4_t even = float4_t{0.f, 0.f, 0.f, 0.f}, odd = float4_t{0.f, 0.f, 0.f, 0.f};
+      for (int h = 0; h < 2; ++h) {
+        if (KLINE) {
 #pragma unroll
-          for (int i = 0; i < TI; ++i) {
-            even = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][tile * TI + i].h8, qf[2 * i], even, 0, 0, 0);
-            odd = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][tile * TI + i].h8, qf[2 * i + 1], odd, 0, 0, 0);
+          for (int tile = 0; tile < 2; ++tile) {
+            float4_t even = float4_t{0.f, 0.f, 0.f, 0.f}, odd = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+              even = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][tile * TI + i].h8, qf[j][2 * i], even, 0, 0, 0);
+              odd = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][tile * TI + i].h8, qf[j][2 * i + 1], odd, 0, 0, 0);
+            }
+            s[j][h][tile * 2 + 0] = even[0] + odd[1];
+            s[j][h][tile * 2 + 1] = even[2] + odd[3];
           }
-          s[h][tile * 2 + 0] = even[0] + odd[1];
-          s[h][tile * 2 + 1] = even[2] + odd[3];
+        } else {
+          s[j][h] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) s[j][h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][ks].h8, qf[j][ks], s[j][h], 0, 0, 0);
         }
-      } else {
-        s[h] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.k[h][ks].h8, qf[ks], s[h], 0, 0, 0);
       }
     }
-    // s[h][j]: token (pi+h)*PS + token_of(j), head c16
-    auto token_of = [&](int j) { return KLINE ? 8 * (j >> 1) + 2 * g4 + (j & 1) : 4 * g4 + j; };
-    float mx = kNegInit;
+    half8_t pf[HB];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int j = 0; j < HB; ++j) {
+      float mx = kNegInit;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float v = s[h][j] * p.scale_log2;
-        if (partial) v = attended((pi + h) * PS + token_of(j)) ? v : kNegInit;
-        s[h][j] = v;
-        mx = fmaxf(mx, v);
+      for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float v = s[j][h][e] * p.scale_log2;
+          if (partial) v = attended((pi + h) * PS + token_of(e)) ? v : kNegInit;
+          s[j][h][e] = v;
+          mx = fmaxf(mx, v);
+        }
       }
-    }
-    mx = max_xor32(max_xor16(mx));
-    // the reference point moves only when the maximum exceeds it by more than 2^8 (p stays <= 256):
-    // after the first steps almost no step rescales O
-    const float m_new = mx > m + 8.0f ? mx : m;
-    const float alpha = fast_exp2(m - m_new);
-    m = m_new;
-    lsum *= alpha;
-    if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {
+      mx = max_xor32(max_xor16(mx));
+      // the reference point moves only when the maximum exceeds it by more than 2^8 (p stays <= 256):
+      // after the first steps almost no step rescales O
+      const float m_new = mx > m[j] + 8.0f ? mx : m[j];
+      const float alpha = fast_exp2(m[j] - m_new);
+      m[j] = m_new;
+      lsum[j] *= alpha;
+      if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.0f))) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db) o[db] *= alpha;
-    }
-    half8_t pf;
+        for (int db = 0; db < DB; ++db) o[j][db] *= alpha;
+      }
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+      for (int h = 0; h < 2; ++h) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float pj = fast_exp2(s[h][j] - m_new);
-        if (partial) pj = attended((pi + h) * PS + token_of(j)) ? pj : 0.f;
-        lsum += pj;
-        pf[h * 4 + j] = static_cast<half_t>(pj);
+        for (int e = 0; e < 4; ++e) {
+          float pj = fast_exp2(s[j][h][e] - m_new);
+          if (partial) pj = attended((pi + h) * PS + token_of(e)) ? pj : 0.f;
+          lsum[j] += pj;
+          pf[j][h * 4 + e] = static_cast<half_t>(pj);
+        }
       }
     }
     // ---- O^T += V^T P^T: contraction slot g4*8 + i <-> page i/4, token token_of(i%4) ----------
@@ -498,7 +598,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
       half8_t a;
       a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
       a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pf, o[db], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < HB; ++j) o[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pf[j], o[j][db], 0, 0, 0);
     }
   };
 
@@ -511,47 +612,50 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (EXT ? 2 : 3)) void decode_mfma_
     consume(pi, ra);
   }
 
-  // ---- the row sums are per lane group: add them up; m is already common -----------------------
-  lsum = sum_xor32(sum_xor16(lsum));
-
-  // ---- merge the 4 waves through LDS: o[db][j] is feature db*16 + 4*g4 + j of head c16 ---------
-  // (the wave's V tile is dead now and becomes its [16][D] fp32 output buffer)
-  float* sm_o_w = reinterpret_cast<float*>(Vt_all[wave]);
-#pragma unroll
-  for (int db = 0; db < DB; ++db) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) sm_o_w[c16 * D + db * 16 + 4 * g4 + j] = o[db][j];
-  }
-  if (g4 == 0) {
-    sm_m[wave][c16] = m;
-    sm_l[wave][c16] = lsum;
-  }
-  __syncthreads();
-
+  // ---- merge the 4 waves through LDS, one head block at a time: o[j][db][e] is feature db*16 + 4*g4 + e
+  // of head j*16 + c16 (the wave's V tile is dead now and becomes its [16][D] fp32 output buffer) -----
   const bool single_chunk = nchunks == 1;
-  for (int idx = tid; idx < heads * D; idx += 256) {
-    const int g = idx / D;
-    const int d = idx % D;
-    float mx = sm_m[0][g];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, sm_m[w][g]);
-    float lt = 0.f, acc = 0.f;
+  for (int j = 0; j < HB; ++j) {
+    if (j > 0) __syncthreads();  // the previous block's sums have been read
+    // the row sums are per lane group: add them up; m is already common
+    const float lrow = sum_xor32(sum_xor16(lsum[j]));
+    float* sm_o_w = reinterpret_cast<float*>(Vt_all[wave]);
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float sc = fast_exp2(sm_m[w][g] - mx);
-      lt += sm_l[w][g] * sc;
-      acc += reinterpret_cast<const float*>(Vt_all[w])[g * D + d] * sc;
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sm_o_w[c16 * D + db * 16 + 4 * g4 + e] = o[j][db][e];
     }
-    const int hq = hq0 + g;
-    if (single_chunk) {
-      const float denom = lt + fast_exp2(kNegInit - mx);
-      p.output[(static_cast<int64_t>(b) * p.h_q + hq) * D + d] = static_cast<half_t>(acc / denom);
-      if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = mx + fast_log2(denom);
-    } else {
-      store_partial(p.part_o + (static_cast<int64_t>(slot) * p.h_q + hq) * D + d, acc);
-      if (d == 0) {
-        store_partial(p.part_ml + (static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 0, mx);
-        store_partial(p.part_ml + (static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 1, lt);
+    if (g4 == 0) {
+      sm_m[wave][c16] = m[j];
+      sm_l[wave][c16] = lrow;
+    }
+    __syncthreads();
+    const int heads_here = min(16, heads - j * 16);
+    for (int idx = tid; idx < heads_here * D; idx += 256) {
+      const int g = idx / D;
+      const int d = idx % D;
+      float mx = sm_m[0][g];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) mx = fmaxf(mx, sm_m[w][g]);
+      float lt = 0.f, acc = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float sc = fast_exp2(sm_m[w][g] - mx);
+        lt += sm_l[w][g] * sc;
+        acc += reinterpret_cast<const float*>(Vt_all[w])[g * D + d] * sc;
+      }
+      const int hq = hq0 + j * 16 + g;
+      if (single_chunk) {
+        const float denom = lt + fast_exp2(kNegInit - mx);
+        p.output[(static_cast<int64_t>(b) * p.h_q + hq) * D + d] = static_cast<half_t>(acc / denom);
+        if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = mx + fast_log2(denom);
+      } else {
+        store_partial(p.part_o + (static_cast<int64_t>(slot) * p.h_q + hq) * D + d, acc);
+        if (d == 0) {
+          store_partial(p.part_ml + (static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 0, mx);
+          store_partial(p.part_ml + (static_cast<int64_t>(slot) * p.h_q + hq) * 2 + 1, lt);
+        }
       }
     }
   }
@@ -639,10 +743,17 @@ extern "C" int tvmkv_debug_set_scratch_launches(uint64_t launches) {
   KV_API_END();
 }
 
+// The fused step's extra arguments (qkv == nullptr: a plain decode call)
+struct FusedStep {
+  const void* qkv = nullptr;
+  const int32_t* append_position_map = nullptr;
+  int apply_rope = 0;
+};
+
 // Body of the decode entry point.  lease(bytes) hands out the scratch memory of the call: arrival
 // counters in the first kArrivalBytes, partial states behind them.
 template <class Lease>
-static void decode_entry(Lease&& lease, const void* q, const void* pages, const int32_t* page_indptr, const int32_t* page_values,
+static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void* q, const void* pages, const int32_t* page_indptr, const int32_t* page_values,
                          const int32_t* length_info, const int32_t* k_rope_pos_offset,
                          const int32_t* q_rope_position, void* output, float* lse, int64_t rotary_mode,
                          double rope_scale, double rope_theta, double sm_scale, int32_t batch_size,
@@ -655,7 +766,10 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
       << "batch_decode_paged_kv: page_size " << page_size << " is not built (16, 32, 64, 128)";
   KV_UNSUPPORTED(d != 64 && d != 128 && d != 256) << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 128, 256)";
   if (batch_size == 0) return;
-  KV_CHECK(q && pages && page_indptr && length_info && output && lse) << "batch_decode_paged_kv: NULL tensor";
+  const bool fused_launch = fused_step.qkv != nullptr;
+  KV_CHECK((q || fused_launch) && pages && page_indptr && length_info && output && lse) << "batch_decode_paged_kv: NULL tensor";
+  KV_CHECK(!fused_launch || (!ext && fused_step.append_position_map && q_rope_position))
+      << "fused decode step: plain cache only, and it needs the append slots and the positions";
   KV_CHECK(nnz_pages == 0 || page_values) << "batch_decode_paged_kv: NULL page table";
   hipStream_t s = as_stream(stream);
 
@@ -682,6 +796,10 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   while ((16 << p.page_shift) < page_size) ++p.page_shift;
   p.chunk_pages = std::max(1, decode_pick_chunk_pages(nnz_pages << p.page_shift, h_kv, batch_size) >> p.page_shift);
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
+  p.qkv = static_cast<const half_t*>(fused_step.qkv);
+  p.pages_rw = const_cast<half_t*>(p.pages);
+  p.append_slot = fused_step.append_position_map;
+  p.apply_rope = fused_step.apply_rope;
   const int64_t slots = nnz_pages / p.chunk_pages + batch_size;
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many chunks";
   const size_t part_o_bytes = static_cast<size_t>(slots) * h_q * d * sizeof(float);
@@ -693,7 +811,10 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   p.epoch = ws.epoch;
 
   const int group = h_q / h_kv;
-  const int head_blocks = (group + 15) / 16;
+  // groups of more than 16 heads: work items of 32 heads (two blocks against the same K/V fragments)
+  // (head dim 256 keeps items of 16: two blocks of its accumulators do not fit the register file)
+  const int heads_per_item = (group > 16 && d <= 128) ? 32 : 16;
+  const int head_blocks = (group + heads_per_item - 1) / heads_per_item;
   const int64_t num_items = slots * h_kv * head_blocks;
   KV_CHECK(num_items < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many work items";
   // One item per workgroup by default (measured a little faster than a resident-size grid
@@ -707,8 +828,9 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
                      option(kOptDecodeSeparateMerge) == 0;
   if (fused) p.arrivals = reinterpret_cast<unsigned long long*>(ws.ptr);
   DecodeRopeDivisors div{};
-  if (p.rotary) {
-    KV_CHECK(k_rope_pos_offset && q_rope_position) << "batch_decode_paged_kv: inline RoPE needs the position arrays";
+  if (p.rotary || (fused_launch && p.apply_rope)) {
+    KV_CHECK(k_rope_pos_offset || fused_launch) << "batch_decode_paged_kv: inline RoPE needs the position arrays";
+    KV_CHECK(q_rope_position) << "batch_decode_paged_kv: inline RoPE needs the position arrays";
     const float theta = static_cast<float>(rope_theta);
     for (int i = 0; i < d / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(d));
   }
@@ -717,8 +839,21 @@ static void decode_entry(Lease&& lease, const void* q, const void* pages, const 
   };
   auto launch_d = [&](auto dim) {
     constexpr int kD = decltype(dim)::value;
-    if (head_blocks > 1) {
-      if (ext) launch(decode_mfma_kernel<true, kD, true>); else launch(decode_mfma_kernel<false, kD, true>);
+    constexpr int kWide = kD <= 128 ? 2 : 1;  // head blocks per item for groups of more than 16 heads
+    const bool wide = heads_per_item == 32;
+    const bool reread = head_blocks > 1;       // several items read the same K/V rows
+    if (fused_launch) {
+      if (reread) {
+        launch(decode_mfma_kernel<false, kD, true, kWide, true>);
+      } else if (wide) {
+        launch(decode_mfma_kernel<false, kD, false, kWide, true>);
+      } else {
+        launch(decode_mfma_kernel<false, kD, false, 1, true>);
+      }
+    } else if (reread) {
+      if (ext) launch(decode_mfma_kernel<true, kD, true, kWide>); else launch(decode_mfma_kernel<false, kD, true, kWide>);
+    } else if (wide) {
+      if (ext) launch(decode_mfma_kernel<true, kD, false, kWide>); else launch(decode_mfma_kernel<false, kD, false, kWide>);
     } else {
       if (ext) launch(decode_mfma_kernel<true, kD, false>); else launch(decode_mfma_kernel<false, kD, false>);
     }
@@ -752,9 +887,33 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
                                            int32_t d, int32_t page_size, int32_t sliding_window, void* stream) {
   KV_API_BEGIN();
   hipStream_t s = as_stream(stream);
-  decode_entry([&](size_t bytes) { return lease_scratch(kScratchDecode, s, bytes, kArrivalBytes); }, q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode,
+  decode_entry([&](size_t bytes) { return lease_scratch(kScratchDecode, s, bytes, kArrivalBytes); }, FusedStep{}, q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode,
                rope_scale, rope_theta, sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d, page_size,
                sliding_window, stream);
+  KV_API_END();
+}
+
+// A decode step of one layer in one launch: split of the fused qkv tensor, RoPE of q and of the new k
+// row (apply_rope != 0, default frequencies), append of the new k / v rows to slot
+// append_position_map[b] and decode attention over the page table, which must already cover the new
+// token (the cache reserves before it attends when it appends before attention).
+extern "C" int tvmkv_fused_decode_step(const void* qkv, void* pages, const int32_t* page_indptr,
+                                       const int32_t* page_values, const int32_t* last_page_len,
+                                       const int32_t* q_rope_position, const int32_t* append_position_map,
+                                       void* output, float* lse, int64_t apply_rope, double rope_scale,
+                                       double rope_theta, double sm_scale, int32_t batch_size, int64_t nnz_pages,
+                                       int64_t num_pages, int32_t h_q, int32_t h_kv, int32_t d, int32_t page_size,
+                                       void* stream) {
+  KV_API_BEGIN();
+  hipStream_t s = as_stream(stream);
+  KV_CHECK(batch_size == 0 || (qkv && append_position_map && q_rope_position)) << "fused_decode_step: NULL tensor";
+  FusedStep step;
+  step.qkv = qkv;
+  step.append_position_map = append_position_map;
+  step.apply_rope = apply_rope != 0;
+  decode_entry([&](size_t bytes) { return lease_scratch(kScratchDecode, s, bytes, kArrivalBytes); }, step, nullptr, pages,
+               page_indptr, page_values, last_page_len, nullptr, q_rope_position, output, lse, 0, rope_scale, rope_theta,
+               sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d, page_size, 0, stream);
   KV_API_END();
 }
 
@@ -771,7 +930,7 @@ extern "C" int tvmkv_batch_decode_paged_kv_noalloc(const void* q, const void* pa
                                                    int32_t d, int32_t page_size, int32_t sliding_window,
                                                    void* stream) {
   KV_API_BEGIN();
-  decode_entry([&](size_t bytes) { return lease_static_scratch(bytes, as_stream(stream)); }, q, pages, page_indptr, page_values,
+  decode_entry([&](size_t bytes) { return lease_static_scratch(bytes, as_stream(stream)); }, FusedStep{}, q, pages, page_indptr, page_values,
                length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode, rope_scale, rope_theta,
                sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window, stream);
   KV_API_END();

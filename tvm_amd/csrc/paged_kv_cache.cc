@@ -11,6 +11,7 @@
 
 #include "common.h"
 #include "kv_bookkeeping.h"
+#include "runtime_support.h"
 
 namespace tvmkv {
 
@@ -187,6 +188,18 @@ class PagedKVCache {
                                                total_seq_length, num_total_pages_, num_kv_heads_, page_size_,
                                                qk_head_dim_, compute_stream_));
       }
+      RecordComputeEvent();
+      return;
+    }
+    // A decode step of a plain cache in one launch: the decode kernel reads q from qkv and rotates it,
+    // and the work items of every sequence's last chunk rotate and append the new k / v rows before they
+    // attend to them (parts 2, 3 and 5).
+    if (FusedDecodeStepApplies(layer_id)) {
+      Launch(tvmkv_fused_decode_step(qkv, pages_[local_layer_id], Dev(s.page_indptr[0]), Dev(s.page_indices[0]),
+                                     Dev(s.length_info[0]), Dev(s.q_rope_position_map), Dev(s.append_position_map), out,
+                                     merged_lse_, rope_normal, rotary_scale_, rotary_theta_, sm_scale,
+                                     book_->batch_size(), s.page_indices[0].size, num_total_pages_, num_qo_heads_,
+                                     num_kv_heads_, qk_head_dim_, page_size_, compute_stream_));
       RecordComputeEvent();
       return;
     }
@@ -609,6 +622,16 @@ class PagedKVCache {
 
   // A chunked-prefill step of a plain cache (one depth, no sliding window, no inline RoPE, no token
   // tree) can run as one pass over the cached and the new tokens.
+  // One sequence per entry, one token each, appended before attention, one level of blocks, a plain cache
+  // whose keys are stored rotated (or not rotated at all) with the default frequencies.
+  bool FusedDecodeStepApplies(int64_t layer_id) const {
+    const StepLayout& s = book_->step();
+    return s.append_before_attn && s.is_decode_request && s.num_depths == 1 && s.is_chain[0] && s.use_decode_kernel[0] &&
+           !support_sliding_window_ && attn_kinds_[layer_id] == TVMKV_ATTN_MHA && rope_mode_ != TVMKV_ROPE_INLINE &&
+           !has_rope_scaling_ && qk_head_dim_ == v_head_dim_ &&
+           (qk_head_dim_ == 64 || qk_head_dim_ == 128 || qk_head_dim_ == 256) && option(kOptNoFusedDecodeStep) == 0;
+  }
+
   bool OnePassPrefillApplies(int64_t layer_id) const {
     const StepLayout& s = book_->step();
     return !s.append_before_attn && s.num_depths == 1 && s.is_chain[0] && !s.use_decode_kernel[0] &&

@@ -23,7 +23,8 @@ struct OptionTable {
   OptionTable() {
     static const char* const env_names[] = {"TVMKV_DECODE_CHUNK_PAGES", "TVMKV_DECODE_SEPARATE_MERGE",
                                                        "TVMKV_DECODE_WGS_PER_CU", "TVMKV_MLA_CHUNK_TOKENS",
-                                                       "TVMKV_MLA_SEPARATE_MERGE", "TVMKV_PREFILL_KV_SPLITS"};
+                                                       "TVMKV_MLA_SEPARATE_MERGE", "TVMKV_PREFILL_KV_SPLITS",
+                                                       "TVMKV_NO_FUSED_DECODE_STEP"};
     static_assert(sizeof(env_names) / sizeof(env_names[0]) == kNumOptions, "one environment variable per option");
     for (int i = 0; i < kNumOptions; ++i) {
       const char* text = std::getenv(env_names[i]);  // once, when the library is loaded
@@ -34,7 +35,8 @@ struct OptionTable {
 OptionTable g_options;
 
 const char* const kOptionNames[] = {"decode_chunk_pages", "decode_separate_merge", "decode_wgs_per_cu",
-                                               "mla_chunk_tokens", "mla_separate_merge", "prefill_kv_splits"};
+                                               "mla_chunk_tokens", "mla_separate_merge", "prefill_kv_splits",
+                                               "no_fused_decode_step"};
 static_assert(sizeof(kOptionNames) / sizeof(kOptionNames[0]) == kNumOptions, "one name per option");
 
 struct Scratch {

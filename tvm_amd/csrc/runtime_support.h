@@ -18,6 +18,7 @@ enum Option {
   kOptMlaChunkTokens,         // lower bound of the tokens per split-KV chunk of the MLA kernel, 0 = 128
   kOptMlaSeparateMerge,       // unused (the MLA chunks are always merged in a second launch)
   kOptPrefillKvSplits,        // > 0: split the keys of every row tile of a paged prefill launch this many ways, 0 = derived
+  kOptNoFusedDecodeStep,      // != 0: the cache object runs a decode step as split+RoPE+append and decode, two launches
   kNumOptions
 };
 int64_t option(Option id);

@@ -149,6 +149,20 @@ def batch_prefill_cached_and_new_kv_fused_q(qkv, q_rope_position, apply_rope, ro
         q_indptr.shape[0] - 1, qkv.shape[0], page_values.shape[0], num_pages, hq, hkv, d, ps, _stream()))
 
 
+def fused_decode_step(qkv, pages, page_indptr, page_values, last_page_len, q_rope_position, append_position_map,
+                      output, lse, apply_rope, rope_scale, rope_theta, sm_scale):
+    """One launch for the decode step of a layer: split of qkv, RoPE, append of the new k / v rows and
+    decode attention (tvmkv_fused_decode_step); the page table covers the new tokens."""
+    _f16(qkv, pages, output)
+    _i32(page_indptr, page_values, last_page_len, q_rope_position, append_position_map)
+    num_pages, _, hkv, ps, d = pages.shape
+    hq = qkv.shape[1] - 2 * hkv
+    check(lib().tvmkv_fused_decode_step(
+        _p(qkv), _p(pages), _p(page_indptr), _p(page_values), _p(last_page_len), _p(q_rope_position),
+        _p(append_position_map), _p(output), _p(lse), int(apply_rope), float(rope_scale), float(rope_theta),
+        float(sm_scale), qkv.shape[0], page_values.shape[0], num_pages, hq, hkv, d, ps, _stream()))
+
+
 def batch_decode_paged_kv(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position,
                           output, lse, rotary_mode, rope_scale, rope_theta, sm_scale, noalloc=False):
     """noalloc=True calls the entry point that takes its scratch memory from the library's built-in
