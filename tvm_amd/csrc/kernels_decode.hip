@@ -338,35 +338,22 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
   // The fused step's append: every work item of the sequence's last chunk writes the new token's k row
   // (rotated with the precise sinf / cosf, the arithmetic of fused_rope_kernel) and v row of its kv head
   // to the page slot, waits until the stores have completed and meets the other waves at a barrier.  All
-  // loads of this workgroup come after that, through the same vector cache and L2 as the stores; the
-  // items of other head blocks of the same kv head write the same bytes.
-  if (FUSED && chunk == nchunks - 1) {
-    const int32_t aslot = p.append_slot[b];
-    if (aslot >= 0) {
-      const int page_tokens = PS << psh;
-      const half_t* krow = p.qkv + (static_cast<int64_t>(b) * (p.h_q + 2 * p.h_kv) + p.h_q + kvh) * D;
-      const half_t* vrow = krow + static_cast<int64_t>(p.h_kv) * D;
-      half_t* kdst = p.pages_rw + (static_cast<int64_t>(aslot / page_tokens) * 2 * p.h_kv + kvh) * head_stride +
-                     (aslot % page_tokens) * D;
-      half_t* vdst = kdst + static_cast<int64_t>(p.h_kv) * head_stride;
-      if (tid < D / 2) {
-        const float xl = static_cast<float>(krow[tid]);
-        const float xh = static_cast<float>(krow[tid + D / 2]);
-        if (p.apply_rope) {
-          const float freq = static_cast<float>(p.q_rope_position[b]) * p.rope_scale / div.v[tid];
-          const float cs = cosf(freq), sn = sinf(freq);
-          kdst[tid] = static_cast<half_t>(cs * xl + sn * (-xh));
-          kdst[tid + D / 2] = static_cast<half_t>(cs * xh + sn * xl);
-        } else {
-          kdst[tid] = krow[tid];
-          kdst[tid + D / 2] = krow[tid + D / 2];
-        }
-      } else if (tid >= 128 && tid < 128 + D / 8) {
-        st16(vdst + (tid - 128) * 8, ld16(vrow + (tid - 128) * 8));
-      }
+  // K/V loads of this workgroup come after that, through the same vector cache and L2 as the stores; the
+  // items of other head blocks of the same kv head write the same bytes.  The loads of the append are
+  // issued here, its arithmetic and stores follow the q fragments below, whose loads are in flight beside them.
+  const bool appends = FUSED && chunk == nchunks - 1;
+  int32_t aslot = -1;
+  float app_xl = 0.f, app_xh = 0.f;
+  Vec16 app_v = zero16();
+  if (appends) {
+    aslot = p.append_slot[b];
+    const half_t* krow = p.qkv + (static_cast<int64_t>(b) * (p.h_q + 2 * p.h_kv) + p.h_q + kvh) * D;
+    if (tid < D / 2) {
+      app_xl = static_cast<float>(krow[tid]);
+      app_xh = static_cast<float>(krow[tid + D / 2]);
+    } else if (tid >= 128 && tid < 128 + D / 8) {
+      app_v = ld16(krow + static_cast<int64_t>(p.h_kv) * D + (tid - 128) * 8);
     }
-    wait_vmcnt<0>();
-    __syncthreads();
   }
 
   // The fused step rotates q itself.  A lane needs the angles of its 8 * KS/2 feature pairs, the same
@@ -425,6 +412,29 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[j][ks] = qv[ks].h8;
+  }
+  if (appends) {
+    if (aslot >= 0) {
+      const int page_tokens = PS << psh;
+      half_t* kdst = p.pages_rw + (static_cast<int64_t>(aslot / page_tokens) * 2 * p.h_kv + kvh) * head_stride +
+                     (aslot % page_tokens) * D;
+      half_t* vdst = kdst + static_cast<int64_t>(p.h_kv) * head_stride;
+      if (tid < D / 2) {
+        if (p.apply_rope) {
+          const float freq = static_cast<float>(p.q_rope_position[b]) * p.rope_scale / div.v[tid];
+          const float cs = cosf(freq), sn = sinf(freq);
+          kdst[tid] = static_cast<half_t>(cs * app_xl + sn * (-app_xh));
+          kdst[tid + D / 2] = static_cast<half_t>(cs * app_xh + sn * app_xl);
+        } else {
+          kdst[tid] = static_cast<half_t>(app_xl);
+          kdst[tid + D / 2] = static_cast<half_t>(app_xh);
+        }
+      } else if (tid >= 128 && tid < 128 + D / 8) {
+        st16(vdst + (tid - 128) * 8, app_v);
+      }
+    }
+    wait_vmcnt<0>();
+    __syncthreads();
   }
   float4_t o[HB][DB];
 #pragma unroll
@@ -794,7 +804,14 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   // sized in those and counted in pages of the table
   p.page_shift = 0;
   while ((16 << p.page_shift) < page_size) ++p.page_shift;
-  p.chunk_pages = std::max(1, decode_pick_chunk_pages(nnz_pages << p.page_shift, h_kv, batch_size) >> p.page_shift);
+  const int group = h_q / h_kv;
+  // groups of more than 16 heads: work items of 32 heads (two blocks against the same K/V fragments;
+  // head dim 256 keeps items of 16: two blocks of its accumulators do not fit the register file)
+  const int heads_per_item = (group > 16 && d <= 128) ? 32 : 16;
+  const int head_blocks = (group + heads_per_item - 1) / heads_per_item;
+  const int chunk16 = heads_per_item == 32 ? decode_pick_chunk_pages_wide(nnz_pages << p.page_shift, h_kv, batch_size, head_blocks)
+                                           : decode_pick_chunk_pages(nnz_pages << p.page_shift, h_kv, batch_size);
+  p.chunk_pages = std::max(1, chunk16 >> p.page_shift);
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
   p.qkv = static_cast<const half_t*>(fused_step.qkv);
   p.pages_rw = const_cast<half_t*>(p.pages);
@@ -810,11 +827,6 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   p.arrivals = nullptr;
   p.epoch = ws.epoch;
 
-  const int group = h_q / h_kv;
-  // groups of more than 16 heads: work items of 32 heads (two blocks against the same K/V fragments)
-  // (head dim 256 keeps items of 16: two blocks of its accumulators do not fit the register file)
-  const int heads_per_item = (group > 16 && d <= 128) ? 32 : 16;
-  const int head_blocks = (group + heads_per_item - 1) / heads_per_item;
   const int64_t num_items = slots * h_kv * head_blocks;
   KV_CHECK(num_items < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many work items";
   // One item per workgroup by default (measured a little faster than a resident-size grid
@@ -824,8 +836,11 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   if (wgs_per_cu > 0) grid_x = std::min<int64_t>(num_items, static_cast<int64_t>(compute_units()) * wgs_per_cu);
   // the chunk merge is done by the last workgroup of each (sequence, kv head, head block) when the
   // arrival counters fit their region; the option decode_separate_merge keeps the second kernel
+  // (items of 32 heads leave the merge to the second kernel: the workgroup that arrives last would merge
+  // 32 rows, eight per wave one after the other, every load a round trip to memory, while the second
+  // kernel gives every row a wave of its own: 32 q / 1 kv heads 0.065 -> 0.053 ms, 64 / 1 0.096 -> 0.074)
   const bool fused = static_cast<size_t>(batch_size) * h_kv * head_blocks * sizeof(unsigned long long) <= kArrivalBytes &&
-                     option(kOptDecodeSeparateMerge) == 0;
+                     option(kOptDecodeSeparateMerge) == 0 && heads_per_item == 16;
   if (fused) p.arrivals = reinterpret_cast<unsigned long long*>(ws.ptr);
   DecodeRopeDivisors div{};
   if (p.rotary || (fused_launch && p.apply_rope)) {

@@ -187,6 +187,23 @@ int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
   return pow2;
 }
 
+// Work items of 32 query heads (GQA groups above 16): an item does twice the matrix and softmax work per
+// K/V byte, two workgroups fit a compute unit, and every chunk of a sequence is a partial state of 32 (or
+// 64, 128 ...) heads to merge.  Such launches run best with few, long items: the longest chunk that still
+// leaves 320 items, 16 pages if none does.  Measured with the chunk merge as a second kernel (ms at chunks
+// of 16 / 32 / 64 / 128 pages; 64 sequences of 1024-8192 tokens unless noted):
+//   32 q / 1 kv heads 0.058 0.054 0.047 0.059      64 / 1   0.089 0.075 0.074 0.063
+//   64 / 2            0.098 0.085 0.084 0.077      128 / 4  0.168 0.143 0.135 0.142
+//   16 sequences, 32 / 1   0.024 0.024 0.034 0.054     256 of 512-2048 tokens, 32 / 1   0.067 0.062 0.060 0.060
+int decode_pick_chunk_pages_wide(int64_t nnz_pages, int h_kv, int batch, int head_blocks) {
+  const int64_t forced = option(kOptDecodeChunkPages);
+  if (forced >= 8 && forced % 8 == 0) return static_cast<int>(forced);
+  for (int cp = 128; cp > 16; cp /= 2) {
+    if ((nnz_pages / cp + batch) * h_kv * head_blocks >= 320) return cp;
+  }
+  return 16;
+}
+
 }  // namespace tvmkv
 
 extern "C" {
