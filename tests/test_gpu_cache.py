@@ -95,9 +95,10 @@ class Mirror:
             assert_close(gk, ek, atol=1e-3, rtol=2e-3, what=f"cached K of seq {sid}")
 
 
-@pytest.mark.parametrize("page_size", [16, 32, 64])
-def test_identical_inputs_through_oracle_and_gpu_caches(page_size):
-    m = Mirror([16, 4096, 1024, page_size, 0], 2, 32, 8, 128)
+@pytest.mark.parametrize("page_size,hq,hkv,d", [(16, 32, 8, 128), (32, 32, 8, 128), (64, 32, 8, 128), (16, 8, 2, 96),
+                                                (32, 12, 4, 80), (16, 4, 4, 112)])
+def test_identical_inputs_through_oracle_and_gpu_caches(page_size, hq, hkv, d):
+    m = Mirror([16, 4096, 1024, page_size, 0], 2, hq, hkv, d)
     m.step([(0, 60), (1, 88), (2, 17), (3, 4)])
     m.step([((4, 3, -1), 35)])
     m.step([((5, 0, 33), 20)])            # fork inside a page -> page copy on the device
@@ -182,11 +183,11 @@ def test_error_paths_on_the_device_cache():
     cache.add_sequence(1)
     with pytest.raises(tvm_amd.KVError, match="The KV cache is full"):
         cache.begin_forward([1], [80])
-    # a kernel's refusal surfaces through the cache call: head_dim 96 is not built
-    c2 = GpuCache([4, 64, 32, 16, 0], 1, 8, 2, 96, 96, rope_mode=0)
+    # a kernel's refusal surfaces through the cache call: head_dim 72 is not built
+    c2 = GpuCache([4, 64, 32, 16, 0], 1, 8, 2, 72, 72, rope_mode=0)
     c2.add_sequence(0)
-    qkv96 = torch.zeros((1, 12, 96), dtype=torch.float16, device=DEV)
-    out96 = torch.zeros((1, 8, 96), dtype=torch.float16, device=DEV)
+    qkv96 = torch.zeros((1, 12, 72), dtype=torch.float16, device=DEV)
+    out96 = torch.zeros((1, 8, 72), dtype=torch.float16, device=DEV)
     c2.begin_forward([0], [1])
     with pytest.raises(tvm_amd.KVError, match="is not built"):
         attn(c2.cache, 0, 1.0, qkv96, out96)

@@ -21,7 +21,7 @@ F16 = np.float16
 
 
 # ------------------------------------------------------------------------------ RoPE / append
-@pytest.mark.parametrize("d,hq,hkv", [(128, 32, 8), (64, 8, 2), (256, 4, 4)])
+@pytest.mark.parametrize("d,hq,hkv", [(128, 32, 8), (64, 8, 2), (256, 4, 4), (80, 8, 2), (96, 32, 8), (112, 4, 4)])
 @pytest.mark.parametrize("apply_rope", [1, 0])
 def test_fused_rope(d, hq, hkv, apply_rope):
     rng = np.random.default_rng(0)
@@ -167,7 +167,7 @@ def test_copy_single_page_and_compact_copy_bit_exact():
 
 
 # ------------------------------------------------------------------------------ merge
-@pytest.mark.parametrize("h,d", [(32, 128), (8, 64), (128, 512)])
+@pytest.mark.parametrize("h,d", [(32, 128), (8, 64), (128, 512), (8, 80), (32, 96), (4, 112), (3, 40)])
 def test_merge_state_inplace(h, d):
     rng = np.random.default_rng(4)
     n = 37
@@ -202,7 +202,7 @@ def _decode_both(rng, kv_lens, hq, hkv, d, npages, scale=1.0, page_size=16):
 
 
 @pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (64, 8, 128), (8, 8, 128), (8, 4, 64), (16, 2, 64), (8, 2, 256),
-                                      (16, 16, 256)])
+                                      (16, 16, 256), (8, 2, 80), (32, 8, 96), (6, 2, 112), (32, 1, 96), (40, 1, 80)])
 def test_decode_ragged_lengths_against_oracle(hq, hkv, d):
     rng = np.random.default_rng(5)
     # empty, single token, page boundaries, several chunks, spare slots
@@ -319,11 +319,11 @@ def test_decode_inline_rope_plain_cache_and_scaled_positions():
 
 
 def test_decode_rejects_what_is_not_built():
-    t = torch.zeros((1, 8, 96), dtype=torch.float16, device=DEV)
-    pages = torch.zeros((2, 2, 2, 16, 96), dtype=torch.float16, device=DEV)
+    t = torch.zeros((1, 8, 72), dtype=torch.float16, device=DEV)
+    pages = torch.zeros((2, 2, 2, 16, 72), dtype=torch.float16, device=DEV)
     lse = torch.zeros((1, 8), dtype=torch.float32, device=DEV)
     one = i32([0, 1])
-    with pytest.raises(KVError, match="head_dim 96 is not built") as info:
+    with pytest.raises(KVError, match="head_dim 72 is not built") as info:
         K.batch_decode_paged_kv(t, pages, one, i32([0]), i32([1]), i32([0]), i32([0]), t, lse, 0, 1.0, 1e4, 1.0)
     assert info.value.code == -2
 
@@ -378,7 +378,7 @@ def _ragged_both(rng, lens, hq, hkv, dqk, dv, causal, scale=1.0):
 
 
 @pytest.mark.parametrize("hq,hkv,dqk,dv", [(32, 8, 128, 128), (8, 8, 128, 128), (8, 2, 64, 64), (16, 16, 192, 128),
-                                           (8, 2, 256, 256)])
+                                           (8, 2, 256, 256), (8, 2, 80, 80), (32, 8, 96, 96), (6, 2, 112, 112)])
 @pytest.mark.parametrize("causal", [1, 0])
 def test_ragged_prefill_against_oracle(hq, hkv, dqk, dv, causal):
     rng = np.random.default_rng(9)
@@ -437,7 +437,7 @@ def _paged_both(rng, kv_lens, q_lens, hq, hkv, d, causal, npages, page_size=16):
     return host(go), host(gl), eo, el
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256), (8, 2, 80), (32, 8, 96), (6, 2, 112)])
 @pytest.mark.parametrize("causal", [0, 1])
 @pytest.mark.parametrize("rows", ["one row tile per sequence", "several row tiles per sequence"])
 def test_paged_prefill_against_oracle(hq, hkv, d, causal, rows):
@@ -1035,3 +1035,20 @@ def test_decode_group_of_64_heads():
         go, gl, eo, el = _decode_both(rng, [5, 130, 3000, 16, 0], hq, hkv, d, 220)
         assert_close(go, eo, what=f"decode out {hq}/{hkv}/{d}")
         assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"decode lse {hq}/{hkv}/{d}")
+
+
+def test_head_dims_between_64_and_128_refuse_what_they_do_not_have():
+    """Head dims 80, 96 and 112 run on the head dim 128 kernels of the plain cache; the sliding-window /
+    inline-RoPE forms and the one-pass chunked prefill are not built for them and say so."""
+    t = torch.zeros((1, 8, 96), dtype=torch.float16, device=DEV)
+    pages = torch.zeros((2, 2, 2, 16, 96), dtype=torch.float16, device=DEV)
+    lse = torch.zeros((1, 8), dtype=torch.float32, device=DEV)
+    one, z = i32([0, 1]), i32([0])
+    with pytest.raises(KVError, match="plain cache only") as info:
+        K.batch_decode_paged_kv(t, pages, one, z, i32([1]), z, z, t, lse, 1, 1.0, 1e4, 1.0)
+    assert info.value.code == -2
+    with pytest.raises(KVError, match="plain cache only"):
+        K.batch_prefill_paged_kv(t, one, pages, one, z, i32([1]), z, z, t, lse, 1, 1, 1.0, 1e4, 1.0)
+    kv = torch.zeros((1, 2, 96), dtype=torch.float16, device=DEV)
+    with pytest.raises(KVError, match="is not built"):
+        K.batch_prefill_cached_and_new_kv(t, one, kv, kv, pages, one, z, i32([1]), t, lse, 1.0)

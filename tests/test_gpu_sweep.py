@@ -61,9 +61,10 @@ def _check(go, gl, eo, el, desc, no_keys=None):
     assert_close(g_l, el, atol=3e-3, rtol=1e-4, what=f"lse {desc}")
 
 
-def _kernel_case(case):
+def _kernel_case(case, padded_d=None):
+    """padded_d: a head dim of 80, 96 or 112 -- built for the plain decode, paged and ragged kernels."""
     rng = np.random.default_rng(77000 + case)
-    kind = KINDS[case % 6]
+    kind = KINDS[case % 6] if padded_d is None else ["decode", "paged", "ragged"][case % 3]
     hq, hkv = HEADS[int(rng.integers(len(HEADS)))]
     d = int(rng.choice([64, 128, 128, 256]))
     ps = int(rng.choice([16, 16, 32, 64, 128]))
@@ -72,6 +73,8 @@ def _kernel_case(case):
         b = min(b, 17)
     sliding = int(rng.integers(2)) if kind in ("decode", "paged") else 0
     rotary = int(rng.integers(2)) if kind in ("decode", "paged", "ragged", "tree_ragged") else 0
+    if padded_d is not None:
+        d, sliding, rotary = padded_d, 0, 0
     desc = json.dumps(dict(case=case, kind=kind, hq=hq, hkv=hkv, d=d, ps=ps, b=b, sliding=sliding, rotary=rotary))
     print("CASE", desc, flush=True)
 
@@ -215,6 +218,12 @@ def test_random_attention_kernel_cases_with_forced_splits(block):
     finally:
         tvm_amd.set_option("prefill_kv_splits", prev_splits)
         tvm_amd.set_option("decode_chunk_pages", prev_chunk)
+
+
+@pytest.mark.parametrize("d", [80, 96, 112])
+def test_random_attention_kernel_cases_head_dims_80_96_112(d):
+    for case in range(2000 + d, 2000 + d + 9):
+        _kernel_case(case, padded_d=d)
 
 
 def _mla_case(case):

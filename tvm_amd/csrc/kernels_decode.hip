@@ -67,6 +67,9 @@ struct DecodeParams {
   half_t* pages_rw;             // == pages
   const int32_t* append_slot;   // (B) page * page_size + offset, -1 = none
   int apply_rope;               // 0: q and k are used as they come
+  // padded head dims (80, 96, 112 on the head dim 128 kernel): elements per row of q, the pages and the
+  // output in memory; 0 = the kernel's head dim
+  int d_mem;
 };
 
 // Same answer as find_sequence, computed by one wavefront as a 64-ary search: the lanes probe
@@ -129,7 +132,8 @@ template <int D, bool COHERENT>
 __device__ __forceinline__ void merge_row(const DecodeParams& p, int b, int hq, int nchunks, int lane) {
   constexpr int EPL = D / 64;  // features per lane
   const int64_t row = static_cast<int64_t>(b) * p.h_q + hq;
-  half_t* out = p.output + row * D + lane * EPL;
+  const int dm = p.d_mem > 0 ? p.d_mem : D;
+  half_t* out = p.output + row * dm + lane * EPL;
   const int s0 = slot_begin(p.page_indptr, b, p.chunk_pages);
   float mx = kNegInit, lsum = 0.f;
   float acc[EPL];
@@ -180,7 +184,9 @@ __device__ __forceinline__ void merge_row(const DecodeParams& p, int b, int hq, 
   const float denom = lsum + fast_exp2(kNegInit - mx);
   const float inv = 1.0f / denom;
 #pragma unroll
-  for (int e = 0; e < EPL; ++e) out[e] = static_cast<half_t>(acc[e] * inv);
+  for (int e = 0; e < EPL; ++e) {
+    if (lane * EPL + e < dm) out[e] = static_cast<half_t>(acc[e] * inv);
+  }
   if (lane == 0) p.lse[row] = mx + fast_log2(denom);
 }
 
@@ -189,8 +195,11 @@ template <int D>
 __device__ __forceinline__ void empty_row(const DecodeParams& p, int b, int hq, int lane) {
   constexpr int EPL = D / 64;
   const int64_t row = static_cast<int64_t>(b) * p.h_q + hq;
+  const int dm = p.d_mem > 0 ? p.d_mem : D;
 #pragma unroll
-  for (int e = 0; e < EPL; ++e) p.output[row * D + lane * EPL + e] = static_cast<half_t>(0.f);
+  for (int e = 0; e < EPL; ++e) {
+    if (lane * EPL + e < dm) p.output[row * dm + lane * EPL + e] = static_cast<half_t>(0.f);
+  }
   if (lane == 0) p.lse[row] = kNegInit;
 }
 
@@ -261,11 +270,16 @@ struct DecodeRopeDivisors {
 // (one kv head with 32 query heads: two items that each streamed the rows before); larger groups take
 // several such items.
 // FUSED (plain cache only): the launch also does the step's split + RoPE + append, see DecodeParams.
-template <bool EXT, int D, bool REREAD, int HB = 1, bool FUSED = false>
+// PAD: rows of q, the pages and the output hold p.d_mem (80, 96, 112) elements, fewer than the kernel's
+// head dim: the missing q features are zero, K fragments and V pieces beyond the row repeat its last 16
+// bytes (finite values that meet zeros, or feed output features that are not stored).
+template <bool EXT, int D, bool REREAD, int HB = 1, bool FUSED = false, bool PAD = false>
 __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void decode_mfma_kernel(DecodeParams p, int group, int num_items,
                                                              DecodeRopeDivisors div) {
   static_assert(HB == 1 || HB == 2, "head blocks per work item");
   static_assert(!(FUSED && EXT), "the fused step exists for the plain cache");
+  static_assert(!PAD || (!EXT && !FUSED), "padded head dims: plain cache, no in-kernel RoPE");
+  const int dm = PAD ? p.d_mem : D;  // elements per row in memory
   constexpr int PS = DM_PS;
   constexpr int KS = D / 32;                // k-steps of the score product
   constexpr int DB = D / 16;                // 16-wide output feature blocks
@@ -292,7 +306,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
   const int cp = p.chunk_pages;
   half_t* Vt = Vt_all[wave];
   const int psh = p.page_shift;  // a page of the table is 1 << psh of the 16-token pages the steps consume
-  const int64_t head_stride = static_cast<int64_t>(PS << psh) * D;
+  const int64_t head_stride = static_cast<int64_t>(PS << psh) * dm;
 
   // Persistent workgroups: item = (chunk slot, kv head, block of 16 heads of the group), strided over
   // the grid.  Neighbouring workgroups take the head blocks and kv heads of one slot, i.e. the same pages.
@@ -379,10 +393,10 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
   for (int j = 0; j < HB; ++j) {
     const bool head_valid = j * 16 + c16 < heads;
     const half_t* qrow = FUSED ? p.qkv + (static_cast<int64_t>(b) * (p.h_q + 2 * p.h_kv) + hq0 + j * 16 + c16) * D + g4 * 8
-                               : p.q + (static_cast<int64_t>(b) * p.h_q + hq0 + j * 16 + c16) * D + g4 * 8;
+                               : p.q + (static_cast<int64_t>(b) * p.h_q + hq0 + j * 16 + c16) * dm + g4 * 8;
     Vec16 qv[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qv[ks] = head_valid ? ld16(qrow + ks * 32) : zero16();
+    for (int ks = 0; ks < KS; ++ks) qv[ks] = (head_valid && (!PAD || ks * 32 + g4 * 8 < dm)) ? ld16(qrow + ks * 32) : zero16();
     if (FUSED && p.apply_rope) {
       // the arithmetic of rope_pair with the shared angles: fp32, one rounding to fp16
 #pragma unroll
@@ -483,14 +497,15 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
       const int pg = min(pi + h, page_hi - 1);
       const int page = __builtin_amdgcn_readfirstlane(p.page_values[pbeg + (pg >> psh)]);
       const half_t* kbase = p.pages + (static_cast<int64_t>(page) * 2 * p.h_kv + kvh) * head_stride +
-                            __builtin_amdgcn_readfirstlane(pg & ((1 << psh) - 1)) * (PS * D);
+                            __builtin_amdgcn_readfirstlane(pg & ((1 << psh) - 1)) * (PS * dm);
       const half_t* vbase = kbase + static_cast<int64_t>(p.h_kv) * head_stride;
       const int last_row = min(PS, kv_len - pg * PS) - 1;  // >= 0: every page of the table holds a token
 #pragma unroll
       for (int i = 0; i < PS / RPI; ++i) {
         const int row = i * RPI + lane / PPR;
-        const int piece = (lane % PPR) ^ dm_swizzle<D>(h * PS + row);
-        const uint32_t src_off = static_cast<uint32_t>(min(row, last_row) * (D * 2) + piece * 16);
+        int piece = (lane % PPR) ^ dm_swizzle<D>(h * PS + row);
+        if (PAD) piece = min(piece, dm / 8 - 1);
+        const uint32_t src_off = static_cast<uint32_t>(min(row, last_row) * (dm * 2) + piece * 16);
         const uint32_t dst = vt_lds + (h * PS + i * RPI) * (D * 2);
         if (REREAD) copy16_to_lds(vbase, src_off, dst); else copy16_to_lds_nt(vbase, src_off, dst);
       }
@@ -498,7 +513,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           if (KLINE) {  // fragment ks: tile ks / TI (8 tokens), line ks % TI of the row
-            const half_t* src = kbase + ((ks / TI) * 8 + (c16 >> 1)) * D + (ks % TI) * 64 + (c16 & 1) * 32 + g4 * 8;
+            const int feature = (ks % TI) * 64 + (c16 & 1) * 32 + g4 * 8;
+            const half_t* src = kbase + ((ks / TI) * 8 + (c16 >> 1)) * dm + (PAD ? min(feature, dm - 8) : feature);
             r.k[h][ks] = REREAD ? ld16(src) : ld16_nt(src);
           } else {
             r.k[h][ks] = ld16(kbase + c16 * D + ks * 32 + g4 * 8);
@@ -658,7 +674,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
       const int hq = hq0 + j * 16 + g;
       if (single_chunk) {
         const float denom = lt + fast_exp2(kNegInit - mx);
-        p.output[(static_cast<int64_t>(b) * p.h_q + hq) * D + d] = static_cast<half_t>(acc / denom);
+        if (!PAD || d < dm) p.output[(static_cast<int64_t>(b) * p.h_q + hq) * dm + d] = static_cast<half_t>(acc / denom);
         if (d == 0) p.lse[static_cast<int64_t>(b) * p.h_q + hq] = mx + fast_log2(denom);
       } else {
         store_partial(p.part_o + (static_cast<int64_t>(slot) * p.h_q + hq) * D + d, acc);
@@ -774,7 +790,12 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   const bool ext = rotary_mode != 0 || sliding_window != 0;
   KV_UNSUPPORTED(page_size < 16 || page_size > 128 || (page_size & (page_size - 1)) != 0)
       << "batch_decode_paged_kv: page_size " << page_size << " is not built (16, 32, 64, 128)";
-  KV_UNSUPPORTED(d != 64 && d != 128 && d != 256) << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 128, 256)";
+  const bool padded = d == 80 || d == 96 || d == 112;  // run on the head dim 128 kernel, rows of d elements
+  KV_UNSUPPORTED(d != 64 && d != 128 && d != 256 && !padded)
+      << "batch_decode_paged_kv: head_dim " << d << " is not built (64, 80, 96, 112, 128, 256)";
+  KV_UNSUPPORTED(padded && (ext || fused_step.qkv != nullptr))
+      << "batch_decode_paged_kv: head_dim " << d << " is built for the plain cache only (no sliding window or inline RoPE)";
+  const int dk = padded ? 128 : d;  // the kernel's head dim
   if (batch_size == 0) return;
   const bool fused_launch = fused_step.qkv != nullptr;
   KV_CHECK((q || fused_launch) && pages && page_indptr && length_info && output && lse) << "batch_decode_paged_kv: NULL tensor";
@@ -807,7 +828,7 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   const int group = h_q / h_kv;
   // groups of more than 16 heads: work items of 32 heads (two blocks against the same K/V fragments;
   // head dim 256 keeps items of 16: two blocks of its accumulators do not fit the register file)
-  const int heads_per_item = (group > 16 && d <= 128) ? 32 : 16;
+  const int heads_per_item = (group > 16 && dk <= 128) ? 32 : 16;
   const int head_blocks = (group + heads_per_item - 1) / heads_per_item;
   const int chunk16 = heads_per_item == 32 ? decode_pick_chunk_pages_wide(nnz_pages << p.page_shift, h_kv, batch_size, head_blocks)
                                            : decode_pick_chunk_pages(nnz_pages << p.page_shift, h_kv, batch_size);
@@ -819,7 +840,8 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   p.apply_rope = fused_step.apply_rope;
   const int64_t slots = nnz_pages / p.chunk_pages + batch_size;
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many chunks";
-  const size_t part_o_bytes = static_cast<size_t>(slots) * h_q * d * sizeof(float);
+  const size_t part_o_bytes = static_cast<size_t>(slots) * h_q * dk * sizeof(float);
+  p.d_mem = padded ? d : 0;
   const size_t part_ml_bytes = static_cast<size_t>(slots) * h_q * 2 * sizeof(float);
   const ScratchLease ws = lease(kArrivalBytes + part_o_bytes + part_ml_bytes);
   p.part_o = reinterpret_cast<float*>(ws.ptr + kArrivalBytes);
@@ -849,6 +871,18 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
     const float theta = static_cast<float>(rope_theta);
     for (int i = 0; i < d / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(d));
   }
+  if (padded) {
+    auto launch_padded = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group, static_cast<int>(num_items), div);
+    };
+    if (head_blocks > 1) {
+      launch_padded(decode_mfma_kernel<false, 128, true, 2, false, true>);
+    } else if (heads_per_item == 32) {
+      launch_padded(decode_mfma_kernel<false, 128, false, 2, false, true>);
+    } else {
+      launch_padded(decode_mfma_kernel<false, 128, false, 1, false, true>);
+    }
+  }
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group, static_cast<int>(num_items), div);
   };
@@ -873,7 +907,9 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
       if (ext) launch(decode_mfma_kernel<true, kD, false>); else launch(decode_mfma_kernel<false, kD, false>);
     }
   };
-  if (d == 128) {
+  if (padded) {
+    // launched above
+  } else if (d == 128) {
     launch_d(std::integral_constant<int, 128>{});
   } else if (d == 256) {
     launch_d(std::integral_constant<int, 256>{});
@@ -882,7 +918,7 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   }
   if (!fused) {
     KV_LAUNCH_CHECK();
-    if (d == 128) {
+    if (dk == 128) {
       hipLaunchKernelGGL(decode_merge_kernel<128>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);
     } else if (d == 256) {
       hipLaunchKernelGGL(decode_merge_kernel<256>, dim3((batch_size * h_q + 3) / 4), dim3(256), 0, s, p, batch_size * h_q);

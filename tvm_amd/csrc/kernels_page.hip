@@ -303,12 +303,13 @@ __global__ __launch_bounds__(256) void compact_kv_copy_kernel(half_t* __restrict
 __global__ __launch_bounds__(256) void merge_state_inplace_kernel(half_t* __restrict__ v, float* __restrict__ s,
                                                                   const half_t* __restrict__ v_other,
                                                                   const float* __restrict__ s_other, int64_t rows,
-                                                                  int d) {
+                                                                  int d, int lanes_per_row) {
+  // lanes_per_row: d / 8 rounded up to a divisor of 64, so that the lanes of a row share a wavefront
   const int chunks = d / 8;
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int c = gid % chunks;
-  const int64_t row = gid / chunks;
-  if (row >= rows) return;
+  const int c = gid % lanes_per_row;
+  const int64_t row = gid / lanes_per_row;
+  if (row >= rows || c >= chunks) return;
   float s_val = s[row];
   float s_other_val = s_other[row];
   const float s_max = fmaxf(s_val, s_other_val);
@@ -438,8 +439,8 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
                            const int32_t* append_position_map, int64_t num_pages, int32_t page_size, void* stream) {
   KV_API_BEGIN();
   KV_CHECK(seq_len >= 0 && num_q_heads > 0 && num_kv_heads > 0) << "fused_rope: bad shape";
-  KV_UNSUPPORTED(head_dim != 64 && head_dim != 128 && head_dim != 256)
-      << "fused_rope: head_dim " << head_dim << " is not built (64, 128, 256)";
+  KV_UNSUPPORTED(head_dim != 64 && head_dim != 128 && head_dim != 256 && head_dim != 80 && head_dim != 96 && head_dim != 112)
+      << "fused_rope: head_dim " << head_dim << " is not built (64, 80, 96, 112, 128, 256)";
   if (seq_len == 0) return TVMKV_OK;
   const bool append = pages != nullptr;
   KV_CHECK(qkv && position_map && (q || append) && k && v) << "fused_rope: NULL tensor";
@@ -470,6 +471,12 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
     if (append) launch(fused_rope_kernel<64, true>); else launch(fused_rope_kernel<64, false>);
   } else if (head_dim == 128) {
     if (append) launch(fused_rope_kernel<128, true>); else launch(fused_rope_kernel<128, false>);
+  } else if (head_dim == 80) {
+    if (append) launch(fused_rope_kernel<80, true>); else launch(fused_rope_kernel<80, false>);
+  } else if (head_dim == 96) {
+    if (append) launch(fused_rope_kernel<96, true>); else launch(fused_rope_kernel<96, false>);
+  } else if (head_dim == 112) {
+    if (append) launch(fused_rope_kernel<112, true>); else launch(fused_rope_kernel<112, false>);
   } else {
     if (append) launch(fused_rope_kernel<256, true>); else launch(fused_rope_kernel<256, false>);
   }
@@ -634,14 +641,16 @@ int tvmkv_merge_state_inplace(void* v, float* s, const void* v_other, const floa
                               int32_t d, void* stream) {
   KV_API_BEGIN();
   KV_CHECK(n >= 0 && h > 0) << "merge_state_inplace: bad shape";
-  // D/8 lanes of one wavefront own a row: D/8 must divide 64.
-  KV_UNSUPPORTED(d <= 0 || d % 8 != 0 || d > 512 || 64 % (d / 8) != 0)
-      << "merge_state_inplace: head dim " << d << " is not built (8..512, D/8 a divisor of 64)";
+  // the lanes of a row share a wavefront: D/8 rounded up to a power of two lanes per row
+  KV_UNSUPPORTED(d <= 0 || d % 8 != 0 || d > 512)
+      << "merge_state_inplace: head dim " << d << " is not built (a multiple of 8 up to 512)";
+  int lanes_per_row = 1;
+  while (lanes_per_row < d / 8) lanes_per_row *= 2;
   if (n == 0) return TVMKV_OK;
   KV_CHECK(v && s && v_other && s_other) << "merge_state_inplace: NULL tensor";
   const int64_t rows = n * h;
-  hipLaunchKernelGGL(merge_state_inplace_kernel, grid_for(rows * (d / 8)), dim3(256), 0, as_stream(stream),
-                     static_cast<half_t*>(v), s, static_cast<const half_t*>(v_other), s_other, rows, d);
+  hipLaunchKernelGGL(merge_state_inplace_kernel, grid_for(rows * lanes_per_row), dim3(256), 0, as_stream(stream),
+                     static_cast<half_t*>(v), s, static_cast<const half_t*>(v_other), s_other, rows, d, lanes_per_row);
   KV_LAUNCH_CHECK();
   KV_API_END();
 }

@@ -67,9 +67,17 @@ constexpr size_t prefill_lds_bytes(int dqk, int dv) {
 // sequence, decode-shaped calls): the tiles are copied with the streaming hint like the decode kernel's
 // (a 15-node tree per sequence 0.252 -> 0.231 ms).  Where row tiles share K/V rows the hint costs 2-4 %,
 // and choosing the copy at run time inside one kernel cost the shared case 1.5 %.
-template <int DQK, int DV, int SRC, int PS, bool EXT, bool STREAM = false>
+// PAD: the head dim in memory, p.d_mem (80, 96, 112: a multiple of 16 below the template's), is smaller
+// than the tile the kernel computes on.  Rows of q, k, v, the pages and the output keep d_mem elements;
+// the q fragments of the missing features are zero, the K/V copies fill the missing 16-byte pieces of a
+// row with a repeat of its last piece (finite values that meet zeros in the score product and only reach
+// output features that are not stored), and the epilogue stores the first d_mem features.
+template <int DQK, int DV, int SRC, int PS, bool EXT, bool STREAM = false, bool PAD = false>
 __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 64 ? 3 : 2)) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
   constexpr bool PAGED = SRC == kPaged, BOTH = SRC == kBoth;
+  static_assert(!PAD || (!EXT && !BOTH && DQK == DV), "padded head dims: plain ragged and paged kernels");
+  const int dqm = PAD ? p.d_mem : DQK;  // elements per q / k row in memory
+  const int dvm = PAD ? p.d_mem : DV;   // elements per v / output row in memory
   auto copy_kv = [](const void* base, uint32_t off, uint32_t dst) {
     if (STREAM) copy16_to_lds_nt(base, off, dst); else copy16_to_lds(base, off, dst);
   };
@@ -267,10 +275,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
 
   half8_t qf[KS];
   {
-    const int64_t q_token_stride = p.q_token_stride != 0 ? p.q_token_stride : static_cast<int64_t>(p.h_q) * DQK;
-    const half_t* qrow = p.q + static_cast<int64_t>(q_start + my_pos) * q_token_stride + my_head * DQK + half * 8;
+    const int64_t q_token_stride = p.q_token_stride != 0 ? p.q_token_stride : static_cast<int64_t>(p.h_q) * dqm;
+    const half_t* qrow = p.q + static_cast<int64_t>(q_start + my_pos) * q_token_stride + my_head * dqm + half * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_valid ? ld16(qrow + ks * 16).h8 : zero16().h8;
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = (row_valid && (!PAD || ks * 16 < dqm)) ? ld16(qrow + ks * 16).h8 : zero16().h8;
     if (q_rope && row_valid) {
       const float q_pos = static_cast<float>(p.q_rope_position[q_start + my_pos]) * p.rope_scale;
 #pragma unroll
@@ -310,10 +318,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
   // Ragged: the base is the sequence's first K/V row of this head, the offset token * row stride,
   // so one sequence's K (or V) must stay below 4 GiB.  Paged: the base is the page, the offset the
   // row inside it.
-  const half_t* k_seq = PAGED ? nullptr : uniform_ptr(p.k + (static_cast<int64_t>(kv_start) * p.h_kv + kvh) * DQK);
-  const half_t* v_seq = PAGED ? nullptr : uniform_ptr(p.v + (static_cast<int64_t>(kv_start) * p.h_kv + kvh) * DV);
-  const uint32_t k_stride_bytes = static_cast<uint32_t>(p.h_kv) * DQK * 2;
-  const uint32_t v_stride_bytes = static_cast<uint32_t>(p.h_kv) * DV * 2;
+  const half_t* k_seq = PAGED ? nullptr : uniform_ptr(p.k + (static_cast<int64_t>(kv_start) * p.h_kv + kvh) * dqm);
+  const half_t* v_seq = PAGED ? nullptr : uniform_ptr(p.v + (static_cast<int64_t>(kv_start) * p.h_kv + kvh) * dvm);
+  const uint32_t k_stride_bytes = static_cast<uint32_t>(p.h_kv) * dqm * 2;
+  const uint32_t v_stride_bytes = static_cast<uint32_t>(p.h_kv) * dvm * 2;
   // Issues copy instructions [FIRST, FIRST + COUNT) of the wave's COPIES for `tile` (K blocks first,
   // then V), so that the caller can spread them over its arithmetic: a burst of all copies of all
   // waves right after the barrier queues up in front of the one address unit of the CU, and the
@@ -329,8 +337,8 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
     const half_t* vbase = v_seq;
     if (from_pages) {
       const int page = __builtin_amdgcn_readlane(page_ids, tile & 63);
-      kbase = p.pages + (((static_cast<int64_t>(page >> 3) * 2 * p.h_kv + kvh) << psh) + (page & 7)) * (PS * DQK);
-      vbase = kbase + (static_cast<int64_t>(p.h_kv) << psh) * (PS * DQK);
+      kbase = p.pages + (((static_cast<int64_t>(page >> 3) * 2 * p.h_kv + kvh) << psh) + (page & 7)) * (PS * dqm);
+      vbase = kbase + (static_cast<int64_t>(p.h_kv) << psh) * (PS * dqm);
     }
 #pragma unroll
     for (int blk = 0; blk < KBLK; ++blk) {
@@ -340,9 +348,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
         const int idx = blk * (RPW / RPI) + i;
         if (idx < FIRST || idx >= FIRST + COUNT) continue;
         const int row = wave_u * RPW + i * RPI + lane / KCH;
-        const int piece = (lane % KCH) ^ k_swizzle<KW>(row);
+        int piece = (lane % KCH) ^ k_swizzle<KW>(row);
+        if (PAD) piece = min(piece, dqm / 8 - 1);
         const uint32_t t = min(kv0 + row, last_row);
-        const uint32_t off = (from_pages ? (t % PS) * (DQK * 2) : __umul24(t, k_stride_bytes)) + (blk * KW + piece * 8) * 2;
+        const uint32_t off = (from_pages ? (t % PS) * (dqm * 2) : __umul24(t, k_stride_bytes)) + (blk * KW + piece * 8) * 2;
         copy_kv(kbase, off, stage + (blk * (BN * KW) + (wave_u * RPW + i * RPI) * KW) * 2);
       }
     }
@@ -354,9 +363,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
         const int idx = DQK / 8 / NW + blk * (RPW / RPI) + i;
         if (idx < FIRST || idx >= FIRST + COUNT) continue;
         const int row = wave_u * RPW + i * RPI + lane / VCH;
-        const int piece = (lane % VCH) ^ v_swizzle<VW>(row);
+        int piece = (lane % VCH) ^ v_swizzle<VW>(row);
+        if (PAD) piece = min(piece, dvm / 8 - 1);
         const uint32_t t = min(kv0 + row, last_row);
-        const uint32_t off = (from_pages ? (t % PS) * (DV * 2) : __umul24(t, v_stride_bytes)) + (blk * VW + piece * 8) * 2;
+        const uint32_t off = (from_pages ? (t % PS) * (dvm * 2) : __umul24(t, v_stride_bytes)) + (blk * VW + piece * 8) * 2;
         copy_kv(vbase, off, stage + (BN * DQK + blk * (BN * VW) + (wave_u * RPW + i * RPI) * VW) * 2);
       }
     }
@@ -398,7 +408,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
   };
   auto issue_tile = [&](int tile) {
     if ((PAGED || (BOTH && tile < prefix_tiles)) && (tile & 63) == 0) load_page_ids(tile);
-    if constexpr (DQK == 128 && DV == 128 && NW == 4 && PS == 16) {
+    if constexpr (DQK == 128 && DV == 128 && NW == 4 && PS == 16 && !PAD) {
       const bool from_pages = BOTH ? tile < prefix_tiles : PAGED;
       const int rows_left = from_pages ? last_tok + 1 - tile * BN : (BOTH ? last_new + 1 - (tile * BN - prefix_pad)
                                                                           : last_tok + 1 - tile * BN);
@@ -690,7 +700,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
   if (row_valid) {
     const float inv = 1.0f / denom;
     const int64_t out_row = (SRC != kRagged && p.kv_splits > 1 ? blockIdx.z * p.split_rows : 0) + static_cast<int64_t>(q_start + my_pos) * p.h_q + my_head;
-    half_t* orow = p.output + out_row * DV + half * 4;
+    half_t* orow = p.output + out_row * dvm + half * 4;
     float* lse_ptr = p.lse + out_row;
     const float my_lse = m + fast_log2(denom);
     if (p.merge_into) {
@@ -707,6 +717,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
       for (int db = 0; db < DB; ++db) {
 #pragma unroll
         for (int j4 = 0; j4 < 4; ++j4) {
+          if (PAD && db * 32 + j4 * 8 >= dvm) continue;
           half4_t* dst = reinterpret_cast<half4_t*>(orow + db * 32 + j4 * 8);
           const half4_t prev = *dst;
           half4_t out4;
@@ -723,6 +734,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
       for (int db = 0; db < DB; ++db) {
 #pragma unroll
         for (int j4 = 0; j4 < 4; ++j4) {
+          if (PAD && db * 32 + j4 * 8 >= dvm) continue;
           half4_t out4;
 #pragma unroll
           for (int e = 0; e < 4; ++e) out4[e] = static_cast<half_t>(o[db][j4 * 4 + e] * inv);
@@ -742,7 +754,7 @@ static int paged_page_shift(int32_t page_size) {
   return shift;
 }
 
-template <int DQK, int DV, int SRC, int PS, bool EXT, bool STREAM = false>
+template <int DQK, int DV, int SRC, int PS, bool EXT, bool STREAM = false, bool PAD = false>
 static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const PrefillRopeDivisors& div,
                                hipStream_t stream) {
   const int64_t slots = total_q * p.group / BM + p.batch_size;
@@ -750,11 +762,11 @@ static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const Pr
   constexpr size_t lds_bytes = prefill_lds_bytes(DQK, DV);
   static bool attr_set = false;  // per instantiation; the attribute is per function, not per device
   if (lds_bytes > 48 * 1024 && !attr_set) {
-    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, SRC, PS, EXT, STREAM>),
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, SRC, PS, EXT, STREAM, PAD>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     attr_set = true;
   }
-  hipLaunchKernelGGL((prefill_kernel<DQK, DV, SRC, PS, EXT, STREAM>),
+  hipLaunchKernelGGL((prefill_kernel<DQK, DV, SRC, PS, EXT, STREAM, PAD>),
                      dim3(p.h_kv, static_cast<unsigned>(slots), static_cast<unsigned>(std::max(1, p.kv_splits))),
                      dim3(NW * 64), lds_bytes, stream, p, div);
 }
@@ -856,6 +868,7 @@ struct KvSplit {
     // at most one row tile per (sequence, kv head) on average: the paged kernels stream the K/V rows
     p.stream_kv = total_q * p.group <= static_cast<int64_t>(p.batch_size) * BM;
     splits = pick_kv_splits(total_q, p.group, p.batch_size, p.h_kv, avg_keys);
+    if (dv % 64 != 0) splits = 1;  // padded head dims (80, 96, 112): the merge kernel is not built for their rows
     if (splits <= 1) return;
     const size_t o_bytes = static_cast<size_t>(splits) * rows * dv * sizeof(half_t);
     const size_t lse_bytes = static_cast<size_t>(splits) * rows * sizeof(float);
@@ -917,6 +930,19 @@ static void launch_prefill(const PrefillParams& p, int64_t total_q, bool ext, do
   }
 }
 
+// Head dims 80, 96 and 112: the head dim 128 kernel on rows of d elements (plain cache, no in-kernel RoPE)
+static bool padded_head_dim(int d) { return d == 80 || d == 96 || d == 112; }
+
+template <int SRC>
+static void launch_prefill_padded(PrefillParams p, int64_t total_q, int d, bool ext, const char* what, hipStream_t stream) {
+  if (ext) {
+    throw Error(TVMKV_EUNSUPPORTED, std::string(what) + ": head_dim " + std::to_string(d) +
+                                        " is built for the plain cache only (no sliding window, inline RoPE or token tree)");
+  }
+  p.d_mem = d;
+  launch_prefill_ext<128, 128, SRC, 16, false, false, true>(p, total_q, PrefillRopeDivisors{}, stream);
+}
+
 }  // namespace tvmkv
 
 using namespace tvmkv;
@@ -964,9 +990,11 @@ int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const 
     launch_prefill<256, 256, kRagged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d_qk == 192 && d_v == 128) {
     launch_prefill<192, 128, kRagged, 16>(p, total_q, ext, rope_theta, s);
+  } else if (d_qk == d_v && padded_head_dim(d_qk)) {
+    launch_prefill_padded<kRagged>(p, total_q, d_qk, ext, "batch_prefill_ragged_kv", s);
   } else {
     KV_UNSUPPORTED(true) << "batch_prefill_ragged_kv: (d_qk, d_v) = (" << d_qk << ", " << d_v
-                         << ") is not built ((64,64), (128,128), (192,128), (256,256))";
+                         << ") is not built ((64,64), (80,80), (96,96), (112,112), (128,128), (192,128), (256,256))";
   }
   KV_LAUNCH_CHECK();
   KV_API_END();
@@ -1026,8 +1054,10 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
     launch_prefill<64, 64, kPaged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d == 256) {
     launch_prefill<256, 256, kPaged, 16>(p, total_q, ext, rope_theta, s);
+  } else if (padded_head_dim(d)) {
+    launch_prefill_padded<kPaged>(p, total_q, d, ext, "batch_prefill_paged_kv", s);
   } else {
-    KV_UNSUPPORTED(true) << "batch_prefill_paged_kv: head_dim " << d << " is not built (64, 128, 256)";
+    KV_UNSUPPORTED(true) << "batch_prefill_paged_kv: head_dim " << d << " is not built (64, 80, 96, 112, 128, 256)";
   }
   split.finish(p, d, s);
   KV_LAUNCH_CHECK();

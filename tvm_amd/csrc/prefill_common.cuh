@@ -56,6 +56,7 @@ struct PrefillParams {
   int64_t split_rows;
   int page_shift;   // pages hold 16 << page_shift tokens; the kernel walks them as runs of 16-token pages
   int stream_kv;    // != 0: every K/V row is read by one row tile only: copy it with the streaming hint
+  int d_mem;        // padded head dims (prefill_kernel<..., PAD = true>): elements per row in memory
 };
 
 // theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
