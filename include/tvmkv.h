@@ -249,6 +249,47 @@ int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t*
                                 int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
                                 int32_t d, int32_t page_size, int32_t sliding_window, void* stream);
 
+/* The attention launchers with a frequency variant for their in-kernel RoPE (rotary_mode != 0).  The
+ * reference bakes the model's rope_scaling dictionary into every attention kernel when it builds them
+ * (python/tvm/relax/frontend/nn/llm/_decode_kernels.py:138,150,301,321; _prefill_kernels.py:159,171,336,357,
+ * 752,758,877,894; kv_cache.py:494-497); here the description travels with the call.  rope_scaling NULL =
+ * the default frequencies, i.e. the launchers without the suffix.  As in the reference's `_rope`
+ * (_kernel_common.py:115-127) the attention kernels rotate the whole head with the rotate-half pairing,
+ * whatever rotary_dim or pairing the split-rotary kernel of the variant uses, and take no factor tensor
+ * (LONGROPE inside the attention kernels is the default frequencies times its magnitude).  The other
+ * arguments are those of the launcher without the suffix; tvmkv_batch_prefill_paged_kv_scaled takes
+ * merge_into != 0 for tvmkv_batch_prefill_paged_kv_merge. */
+int tvmkv_batch_decode_paged_kv_scaled(const void* q, const void* pages, const int32_t* page_indptr,
+                                       const int32_t* page_values, const int32_t* length_info,
+                                       const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,
+                                       void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                                       double rope_theta, double sm_scale, int32_t batch_size,
+                                       int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                                       int32_t d, int32_t page_size, int32_t sliding_window,
+                                       const tvmkv_rope_scaling* rope_scaling, void* stream);
+int tvmkv_batch_prefill_ragged_kv_scaled(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                                         const int32_t* kv_indptr, const int32_t* q_rope_position,
+                                         const int32_t* k_rope_pos_offset, void* output, float* lse,
+                                         int64_t causal, int64_t rotary_mode, double rope_scale,
+                                         double rope_theta, double sm_scale, int32_t batch_size, int64_t total_q,
+                                         int32_t h_q, int32_t h_kv, int32_t d_qk, int32_t d_v,
+                                         const tvmkv_rope_scaling* rope_scaling, void* stream);
+int tvmkv_batch_prefill_paged_kv_scaled(const void* q, const int32_t* q_indptr, const void* pages,
+                                        const int32_t* page_indptr, const int32_t* page_values,
+                                        const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                                        const int32_t* q_rope_position, void* output, float* lse, int64_t causal,
+                                        int64_t rotary_mode, double rope_scale, double rope_theta,
+                                        double sm_scale, int32_t batch_size, int64_t total_q, int64_t nnz_pages,
+                                        int64_t num_pages, int32_t h_q, int32_t h_kv, int32_t d,
+                                        int32_t page_size, int32_t sliding_window, int32_t sliding_window_size,
+                                        int32_t merge_into, const tvmkv_rope_scaling* rope_scaling, void* stream);
+int tvmkv_batch_tree_attn_scaled(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                                 const int32_t* kv_indptr, const int32_t* q_rope_position,
+                                 const int32_t* mn_indptr, const int32_t* mask, void* output, float* lse,
+                                 int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                                 int32_t batch_size, int64_t total_q, int32_t h_q, int32_t h_kv, int32_t d,
+                                 const tvmkv_rope_scaling* rope_scaling, void* stream);
+
 /* Slots 24 + 13 + 17 in one launch (no counterpart among the reference's kernels; what
  * AttentionWithFusedQKV does for a decode step, src/runtime/vm/paged_kv_cache.cc:1360-1373 and
  * :2236-2260, as three kernels): the decode step of one layer over a plain cache.  qkv is the fused

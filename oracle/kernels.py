@@ -87,6 +87,23 @@ def rope_angle(rope_scaling, pos_scaled, d, rotary_dim, theta, ext=None):
     return float(angle), float(mag.value)
 
 
+class inline_rope_scaling:
+    """`with inline_rope_scaling(rope_scaling):` -- inside the block the attention kernels' own RoPE (rotary_mode 1)
+    uses this frequency variant, the way the reference bakes the model's rope_scaling dictionary into the kernels it
+    builds (_decode_kernels.py:49,138,150; _prefill_kernels.py:54-60,159,171,677,752,758).  A library setting."""
+
+    def __init__(self, rope_scaling):
+        self.sc = None if not rope_scaling else RopeScaling.from_dict(rope_scaling)
+
+    def __enter__(self):
+        lib().orc_set_inline_rope_scaling(None if self.sc is None else ctypes.byref(self.sc))
+        return self
+
+    def __exit__(self, *exc):
+        lib().orc_set_inline_rope_scaling(None)
+        return False
+
+
 def fused_rope_scaled(qkv, position_map, q, k, v, apply_rope, rope_scaling, *, theta=1e4, scale=1.0, ext_factors=None):
     n, fused, d = qkv.shape
     hq, hkv = q.shape[1], k.shape[1]

@@ -221,6 +221,31 @@ float orc_rope_angle(const orc_rope_scaling* sc, float s, int d, int R, float th
   return s * (inter * (1.0f - mask) + extra * mask);
 }
 
+/* The RoPE of the attention kernels (_kernel_common.py:115-127): the whole head, rotate-half pairing,
+ * the model's frequency variant baked in when the reference builds the kernel (rope_scaling argument of
+ * the kernel factories, _decode_kernels.py:49,181; _prefill_kernels.py:54-60,217-223,677,795).  Here the
+ * variant is a setting of the oracle library: NULL = default frequencies.  The attention kernels pass no
+ * factor tensor, so longrope is the default frequencies times its magnitude (position_embedding.py:164-188). */
+static const orc_rope_scaling* g_inline_scaling = NULL;
+static orc_rope_scaling g_inline_scaling_copy;
+void orc_set_inline_rope_scaling(const orc_rope_scaling* sc) {
+  if (sc == NULL) {
+    g_inline_scaling = NULL;
+  } else {
+    g_inline_scaling_copy = *sc;
+    g_inline_scaling = &g_inline_scaling_copy;
+  }
+}
+static inline f16 rope_elem_inline(const f16* x, int d, int D, float pos_times_scale, float theta) {
+  if (g_inline_scaling == NULL) return rope_elem(x, d, D, pos_times_scale, theta);
+  float magnitude;
+  float freq = orc_rope_angle(g_inline_scaling, pos_times_scale, d, D, theta, NULL, &magnitude);
+  float c = cosf(freq) * magnitude * h2f(x[d]);
+  f16 other = d < D / 2 ? (f16)(x[d + D / 2] ^ 0x8000u) : x[d - D / 2];
+  float sn = sinf(freq) * magnitude * h2f(other);
+  return f2h(c + sn);
+}
+
 /* fused_rope / fused_rope_longrope_scaling (position_embedding.py:525-667) with a frequency variant.
  * ext_factors: NULL or R floats, long factors then short ones; the long ones apply when
  * seq_len > original_max_position_embeddings (:601). */
@@ -367,7 +392,7 @@ void orc_decode(const f16* Q, const f16* pages, const int32_t* page_table_indptr
       for (int d = 0; d < D; ++d) O_local[d] = 0.0f;
       for (int d = 0; d < D; ++d)
         Q_local[d] = rotary_mode == 1
-                         ? h2f(rope_elem(qrow, d, D, (float)q_rope_position[b] * rope_scale, rope_theta))
+                         ? h2f(rope_elem_inline(qrow, d, D, (float)q_rope_position[b] * rope_scale, rope_theta))
                          : h2f(qrow[d]);
       for (int row_idx = 0; row_idx < kv_len; ++row_idx) {
         int so = seq_offset(row_idx, b, length_info, B, sliding_window);
@@ -377,7 +402,7 @@ void orc_decode(const f16* Q, const f16* pages, const int32_t* page_table_indptr
         const f16* vrow = PAGE_AT(pages, H_kv, page_size, D, page_no, 1, h_qo / group_size, page_offset);
         for (int d = 0; d < D; ++d)
           K_local[d] = rotary_mode == 1
-                           ? h2f(rope_elem(krow, d, D, (float)(k_rope_pos_offset[b] + row_idx) * rope_scale, rope_theta))
+                           ? h2f(rope_elem_inline(krow, d, D, (float)(k_rope_pos_offset[b] + row_idx) * rope_scale, rope_theta))
                            : h2f(krow[d]);
         float S_val = 0.0f;
         for (int d = 0; d < D; ++d) S_val += Q_local[d] * K_local[d];
@@ -452,7 +477,7 @@ static void prefill_paged_impl(const f16* q, const int32_t* q_indptr, const f16*
         const f16* qrow = q + ((int64_t)curl_q * h_q + h_qo) * d;
         for (int i = 0; i < d; ++i)
           Q_local[i] = rotary_mode == 1
-                           ? h2f(rope_elem(qrow, i, d, (float)q_rope_position[curl_q] * rope_scale, rope_theta))
+                           ? h2f(rope_elem_inline(qrow, i, d, (float)q_rope_position[curl_q] * rope_scale, rope_theta))
                            : h2f(qrow[i]);
         for (int row_idx = 0; row_idx < kv_len; ++row_idx) {
           int so = seq_offset(row_idx, b_idx, length_info, batch_size, sliding_window);
@@ -462,7 +487,7 @@ static void prefill_paged_impl(const f16* q, const int32_t* q_indptr, const f16*
           const f16* vrow = PAGE_AT(pages, h_kv, page_size, d, page_no, 1, h_qo / group_size, page_offset);
           for (int i = 0; i < d; ++i) {
             K_local[i] = rotary_mode == 1
-                             ? h2f(rope_elem(krow, i, d, (float)(k_rope_pos_offset[b_idx] + row_idx) * rope_scale, rope_theta))
+                             ? h2f(rope_elem_inline(krow, i, d, (float)(k_rope_pos_offset[b_idx] + row_idx) * rope_scale, rope_theta))
                              : h2f(krow[i]);
             V_local[i] = h2f(vrow[i]);
           }
@@ -557,7 +582,7 @@ static void prefill_ragged_impl(const f16* q, const int32_t* q_indptr, const f16
         const f16* qrow = q + ((int64_t)(q_indptr[b] + q_idx) * h_q + h) * d_qk;
         for (int i = 0; i < d_qk; ++i)
           qbuf[i] = rotary_mode == 1
-                        ? h2f(rope_elem(qrow, i, d_qk, (float)q_rope_position[q_indptr[b] + q_idx] * rope_scale, rope_theta))
+                        ? h2f(rope_elem_inline(qrow, i, d_qk, (float)q_rope_position[q_indptr[b] + q_idx] * rope_scale, rope_theta))
                         : h2f(qrow[i]);
         for (int k_idx = 0; k_idx < kv_len; ++k_idx) {
           float attention_score;
@@ -570,7 +595,7 @@ static void prefill_ragged_impl(const f16* q, const int32_t* q_indptr, const f16
                         : (mn_indptr ? q_rope_position[kv_indptr[b] + k_idx] : k_rope_pos_offset[b] + k_idx);
             for (int i = 0; i < d_qk; ++i) {
               float key_val = rotary_mode == 1
-                                  ? h2f(rope_elem(krow, i, d_qk, (float)k_pos * rope_scale, rope_theta))
+                                  ? h2f(rope_elem_inline(krow, i, d_qk, (float)k_pos * rope_scale, rope_theta))
                                   : h2f(krow[i]);
               result += qbuf[i] * key_val;
             }

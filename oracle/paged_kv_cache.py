@@ -216,7 +216,8 @@ class OraclePagedKVCache:
         if host.append_before_attn:
             ok.transpose_append(self.pages[layer_id], k, v, aux["append_position_map"])
         o_view = np.zeros((total, self.hq, self.dqk), self.dtype)
-        self._attention_internal(layer_id, q, k, v, o_view, sm_scale)
+        with self._inline_rope():
+            self._attention_internal(layer_id, q, k, v, o_view, sm_scale)
         out[:total] = o_view
         if not host.append_before_attn:
             ok.transpose_append(self.pages[layer_id], k, v, aux["append_position_map"])
@@ -227,18 +228,26 @@ class OraclePagedKVCache:
         total = sum(self.host.cur_append_lengths)
         if not (q.shape[0] == current_k.shape[0] == current_v.shape[0] == out.shape[0] == total):
             raise hc.CacheError("attention_with_shared_kv: row counts do not match the batch")
-        self._attention_internal(source_layer_id, q, current_k, current_v, out, sm_scale)
+        with self._inline_rope():
+            self._attention_internal(source_layer_id, q, current_k, current_v, out, sm_scale)
+
+    def _inline_rope(self):
+        """The frequency variant the reference bakes into its attention kernels (kv_cache.py:494-497, :680-682):
+        in force while a cache that rotates inside the attention kernels runs them."""
+        return ok.inline_rope_scaling(self.rope_scaling if self.rope_mode == hc.ROPE_INLINE else None)
 
     def self_attention(self, layer_id, sm_scale, q, k, v, out, lse):
-        if self.attn_kinds[layer_id] == hc.ATTN_MHA:
-            self._self_attn(q, k, v, out, lse, sm_scale, self.rope_mode)
-        else:
-            self._self_attn(q, k, v, out, lse, sm_scale, hc.ROPE_NONE)
+        with self._inline_rope():
+            if self.attn_kinds[layer_id] == hc.ATTN_MHA:
+                self._self_attn(q, k, v, out, lse, sm_scale, self.rope_mode)
+            else:
+                self._self_attn(q, k, v, out, lse, sm_scale, hc.ROPE_NONE)
 
     def cross_attention(self, layer_id, sm_scale, q, out, lse):
         host, aux = self.host, self.host.aux
         if self.attn_kinds[layer_id] == hc.ATTN_MHA:
-            self._mha_cross_attn(layer_id, q, out, lse, sm_scale, True, False)
+            with self._inline_rope():
+                self._mha_cross_attn(layer_id, q, out, lse, sm_scale, True, False)
             return
         total = q.shape[0]
         temp_out = np.zeros((total, self.hq, self.dv), self.dtype)

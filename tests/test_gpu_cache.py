@@ -144,11 +144,25 @@ def test_rope_frequency_variants_through_the_cache(rope):
     m.step([((3, 1, 40), 25), (0, 2)])
 
 
-def test_rope_variants_need_a_cache_that_rotates_up_front():
-    with pytest.raises(tvm_amd.KVError, match="inline RoPE") as info:
-        GpuCache([8, 2048, 512, 16, 1], 1, 32, 8, 128, 128, rope_scaling={"rope_type": "llama3", "factor": 8.0,
-                 "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 8192})
-    assert info.value.code == -2
+@pytest.mark.parametrize("rope", [
+    dict(rope_theta=5e5, rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                                       "original_max_position_embeddings": 8192}),
+    dict(rope_scaling={"rope_type": "yarn", "factor": 40.0, "beta_fast": 32, "beta_slow": 1,
+                       "original_max_position_embeddings": 4096}),
+    dict(rope_scaling={"rope_type": "longrope", "max_position_embeddings": 131072, "original_max_position_embeddings": 4096}),
+    dict(rope_scaling={"rope_type": "llama4", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                       "original_max_position_embeddings": 8192}),
+], ids=lambda r: r["rope_scaling"]["rope_type"])
+@pytest.mark.parametrize("sliding", [0, 1])
+def test_rope_frequency_variants_in_a_cache_that_rotates_inside_the_attention_kernels(rope, sliding):
+    """Inline-RoPE caches (rope mode 2; a sliding-window cache is always one): K is stored unrotated, and every
+    attention kernel rotates q and k itself with the model's frequency variant -- prefill (ragged + paged +
+    merge), decode and a fork with two block depths, against the oracle cache with the same variant in force."""
+    m = Mirror([8, 2048, 512, 16, sliding], 1, 8, 2, 128, rope_mode=2, **rope)
+    m.step([(0, 60), (1, 88), (2, 17)])
+    m.step([(0, 1), (1, 1), (2, 1)])
+    m.step([((3, 1, 40), 25), (0, 2)])
+    m.step([(3, 1), (1, 1)])
 
 
 def test_cfg1_decode_through_the_cache_verbs():

@@ -1052,3 +1052,101 @@ def test_head_dims_between_64_and_128_refuse_what_they_do_not_have():
     kv = torch.zeros((1, 2, 96), dtype=torch.float16, device=DEV)
     with pytest.raises(KVError, match="is not built"):
         K.batch_prefill_cached_and_new_kv(t, one, kv, kv, pages, one, z, i32([1]), t, lse, 1.0)
+
+
+# ------------------------------------------------------------------------------ frequency variants in the kernels
+ROPE_VARIANTS = [
+    {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+     "original_max_position_embeddings": 8192},
+    {"rope_type": "yarn", "factor": 40.0, "beta_fast": 32, "beta_slow": 1, "original_max_position_embeddings": 4096},
+    {"rope_type": "longrope", "max_position_embeddings": 131072, "original_max_position_embeddings": 4096},
+    {"rope_type": "gptj"},
+    {"rope_type": "llama4", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+     "original_max_position_embeddings": 8192},
+]
+
+
+@pytest.mark.parametrize("rope_scaling", ROPE_VARIANTS, ids=lambda sc: sc["rope_type"])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (4, 2, 64), (20, 1, 128)])
+def test_inline_rope_frequency_variants(rope_scaling, hq, hkv, d):
+    """rotary_mode = 1 with the model's frequency variant (the *_scaled launchers) in the decode, paged prefill,
+    ragged prefill and ragged tree-attention kernels, against the oracle with the same variant in force."""
+    from tests.util import random_forest, tree_order
+    rng = np.random.default_rng(300 + d + hq)
+    sm = d ** -0.5
+    # (the oracle recomputes the rotation for every score element: the shapes are small)
+    # decode over a sliding-window cache (sinks, an evicted gap) and a plain one
+    kv = [5, 130, 600, 64]
+    pages, ip, pv, last, _, _ = build_paged_kv(rng, kv, 60, hkv, 16, d)
+    info = np.array([last, [2, 40, 300, 0], [1, 4, 0, 0]], np.int32)  # window offsets, sink sizes
+    q = rng.standard_normal((4, hq, d)).astype(F16)
+    k_off = np.array([0, 7, 3000, 11], np.int32)
+    logical = np.array([kv[i] - info[1][i] + info[2][i] for i in range(4)])
+    q_pos = (k_off + logical - 1).astype(np.int32)
+    for length_info in (last, info):
+        eo, el = np.zeros((4, hq, d), F16), np.zeros((4, hq), np.float32)
+        with ok.inline_rope_scaling(rope_scaling):
+            ok.decode(q, pages, ip, pv, length_info, k_off, q_pos, eo, el, 1, 1.0, 1e4, sm)
+        go = torch.zeros((4, hq, d), dtype=torch.float16, device=DEV)
+        gl = torch.zeros((4, hq), dtype=torch.float32, device=DEV)
+        K.batch_decode_paged_kv(dev(q), dev(pages), i32(ip), i32(pv), i32(length_info), i32(k_off), i32(q_pos), go, gl, 1,
+                                1.0, 1e4, sm, rope_scaling=rope_scaling)
+        assert_close(host(go), eo, what="decode out, frequency variant")
+        assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="decode lse, frequency variant")
+    # paged prefill, causal
+    ql = [7, 33, 70, 1]
+    kvp = [5, 130, 200, 64]
+    kvp = [max(a, b) for a, b in zip(kvp, ql)]
+    pages, ip, pv, last, _, _ = build_paged_kv(rng, kvp, 40, hkv, 16, d)
+    n = sum(ql)
+    ind = np.concatenate([[0], np.cumsum(ql)]).astype(np.int32)
+    qp = rng.standard_normal((n, hq, d)).astype(F16)
+    pos = np.concatenate([k_off[i] + kvp[i] - ql[i] + np.arange(ql[i]) for i in range(4)]).astype(np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    with ok.inline_rope_scaling(rope_scaling):
+        ok.prefill_paged(qp, ind, pages, ip, pv, last, k_off, pos, eo, el, 1, 1, 1.0, 1e4, sm)
+    go = torch.zeros((n, hq, d), dtype=torch.float16, device=DEV)
+    gl = torch.zeros((n, hq), dtype=torch.float32, device=DEV)
+    K.batch_prefill_paged_kv(dev(qp), i32(ind), dev(pages), i32(ip), i32(pv), i32(last), i32(k_off), i32(pos), go, gl, 1, 1,
+                             1.0, 1e4, sm, rope_scaling=rope_scaling)
+    assert_close(host(go), eo, what="paged out, frequency variant")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="paged lse, frequency variant")
+    # ragged prefill
+    kr = rng.standard_normal((n, hkv, d)).astype(F16)
+    vr = rng.standard_normal((n, hkv, d)).astype(F16)
+    off = np.array([0, 50, 900, 3], np.int32)
+    rpos = np.concatenate([off[i] + np.arange(ql[i]) for i in range(4)]).astype(np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    with ok.inline_rope_scaling(rope_scaling):
+        ok.prefill_ragged(qp, ind, kr, vr, ind, rpos, off, eo, el, 1, 1, 1.0, 1e4, sm)
+    go.zero_()
+    gl.zero_()
+    K.batch_prefill_ragged_kv(dev(qp), i32(ind), dev(kr), dev(vr), i32(ind), i32(rpos), i32(off), go, gl, 1, 1, 1.0, 1e4,
+                              sm, rope_scaling=rope_scaling)
+    assert_close(host(go), eo, what="ragged out, frequency variant")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="ragged lse, frequency variant")
+    # ragged tree attention: positions are depths
+    trees = [random_forest(rng, s_) for s_ in (7, 15, 33)]
+    sizes = [len(t) for t in trees]
+    nt = sum(sizes)
+    tind = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    qt = rng.standard_normal((nt, hq, d)).astype(F16)
+    kt = rng.standard_normal((nt, hkv, d)).astype(F16)
+    vt = rng.standard_normal((nt, hkv, d)).astype(F16)
+    mask = np.concatenate([tree_order(t) for t in trees])
+    depth = []
+    for i, t in enumerate(trees):
+        dep = []
+        for parent in t:
+            dep.append(0 if parent == -1 else dep[parent] + 1)
+        depth += [200 * i + x for x in dep]
+    tpos = np.array(depth, np.int32)
+    eo, el = np.zeros((nt, hq, d), F16), np.zeros((nt, hq), np.float32)
+    with ok.inline_rope_scaling(rope_scaling):
+        ok.tree_attn_ragged(qt, tind, kt, vt, tind, tpos, tind, mask, eo, el, 1, 1.0, 1e4, sm)
+    go = torch.zeros((nt, hq, d), dtype=torch.float16, device=DEV)
+    gl = torch.zeros((nt, hq), dtype=torch.float32, device=DEV)
+    K.batch_tree_attn(dev(qt), i32(tind), dev(kt), dev(vt), i32(tind), i32(tpos), i32(tind), i32(mask), go, gl, 1, 1.0,
+                      1e4, sm, rope_scaling=rope_scaling)
+    assert_close(host(go), eo, what="tree out, frequency variant")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="tree lse, frequency variant")

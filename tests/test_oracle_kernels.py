@@ -712,3 +712,77 @@ def test_longrope_factors_and_magnitude():
         lo = m * (np.cos(ang) * x[:, :D // 2] - np.sin(ang) * x[:, D // 2:])
         hi = m * (np.cos(ang) * x[:, D // 2:] + np.sin(ang) * x[:, :D // 2])
         assert_close(q[:, 0], np.concatenate([lo, hi], axis=1).astype(np.float16), atol=2e-3, rtol=2e-3, what="longrope q")
+
+
+# ------------------------------------------------- frequency variants inside the attention kernels
+LONGROPE = {"rope_type": "longrope", "max_position_embeddings": 131072, "original_max_position_embeddings": 4096}
+GPTJ = {"rope_type": "gptj"}
+LLAMA4 = {"rope_type": "llama4", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+          "original_max_position_embeddings": 8192}
+
+
+def rotate_whole_head(x, positions, rope_scaling, theta=1e4, scale=1.0):
+    """What the reference's attention kernels do to a row before they use it (_kernel_common.py:115-127):
+    element d of the WHOLE head gets cos * x[d] + sin * (-x[d + D/2] or x[d - D/2]) at the angle the variant
+    gives element d (ok.rope_angle, pinned above), rounded to fp16.  x: (rows, heads, D)."""
+    rows, heads, D = x.shape
+    out = np.zeros_like(x)
+    xf = x.astype(np.float32)
+    for r in range(rows):
+        for d in range(D):
+            angle, mag = ok.rope_angle(rope_scaling, np.float32(positions[r]) * np.float32(scale), d, D, theta)
+            c = np.float32(np.cos(np.float32(angle))) * np.float32(mag)
+            s_ = np.float32(np.sin(np.float32(angle))) * np.float32(mag)
+            other = -xf[r, :, d + D // 2] if d < D // 2 else xf[r, :, d - D // 2]
+            out[r, :, d] = (c * xf[r, :, d] + s_ * other).astype(np.float16)
+    return out
+
+
+@pytest.mark.parametrize("rope_scaling", [LLAMA3, YARN, LONGROPE, GPTJ, LLAMA4], ids=lambda sc: sc["rope_type"])
+def test_inline_rope_variants_equal_attention_over_rotated_rows(rope_scaling):
+    """The oracle's attention kernels with rotary_mode = 1 and a frequency variant in force equal the same kernels
+    with rotary_mode = 0 on rows rotated beforehand: decode (keys at k_rope_pos_offset + t, the query at its
+    position) and the ragged kernel (queries and keys of a chunk)."""
+    rng = np.random.default_rng(123)
+    hq, hkv, d, ps = 4, 2, 64, 16
+    kv_lens = [37, 5]
+    pages, ip, pv, last, ks, vs = build_paged_kv(rng, kv_lens, 6, hkv, ps, d)
+    k_off = np.array([100, 3], np.int32)
+    q_pos = np.array([100 + 36, 3 + 4], np.int32)
+    q = rng.standard_normal((2, hq, d)).astype(F16)
+    z = np.zeros(2, np.int32)
+    inline_o, inline_l = np.zeros((2, hq, d), F16), np.zeros((2, hq), np.float32)
+    with ok.inline_rope_scaling(rope_scaling):
+        ok.decode(q, pages, ip, pv, last, k_off, q_pos, inline_o, inline_l, 1, 1.0, 1e4, d ** -0.5)
+    rotated_pages = pages.copy()
+    for b, n in enumerate(kv_lens):
+        rk = rotate_whole_head(ks[b], k_off[b] + np.arange(n), rope_scaling)
+        for t in range(n):
+            rotated_pages[pv[ip[b] + t // ps], 0, :, t % ps] = rk[t]
+    rq = rotate_whole_head(q, q_pos, rope_scaling)
+    plain_o, plain_l = np.zeros_like(inline_o), np.zeros_like(inline_l)
+    ok.decode(rq, rotated_pages, ip, pv, last, z, z, plain_o, plain_l, 0, 1.0, 1e4, d ** -0.5)
+    assert_close(inline_o, plain_o, atol=2e-3, rtol=2e-3, what="decode, inline variant vs rotated rows")
+    assert_close(inline_l, plain_l, atol=2e-3, rtol=1e-4, what="decode lse")
+    # the variant really changes something (or, for magnitude-only longrope, scales the scores)
+    default_o = np.zeros_like(inline_o)
+    default_l = np.zeros_like(inline_l)
+    ok.decode(q, pages, ip, pv, last, k_off, q_pos, default_o, default_l, 1, 1.0, 1e4, d ** -0.5)
+    assert np.abs(default_l - inline_l).max() > 1e-3
+    # ragged
+    lens = [9, 20]
+    n = sum(lens)
+    ind = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    qr = rng.standard_normal((n, hq, d)).astype(F16)
+    kr = rng.standard_normal((n, hkv, d)).astype(F16)
+    vr = rng.standard_normal((n, hkv, d)).astype(F16)
+    off = np.array([50, 7], np.int32)
+    pos = np.concatenate([off[i] + np.arange(lens[i]) for i in range(2)]).astype(np.int32)
+    io, il = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+    with ok.inline_rope_scaling(rope_scaling):
+        ok.prefill_ragged(qr, ind, kr, vr, ind, pos, off, io, il, 1, 1, 1.0, 1e4, d ** -0.5)
+    po, pl = np.zeros_like(io), np.zeros_like(il)
+    ok.prefill_ragged(rotate_whole_head(qr, pos, rope_scaling), ind, rotate_whole_head(kr, pos, rope_scaling), vr, ind,
+                      np.zeros(n, np.int32), z, po, pl, 1, 0, 1.0, 1e4, d ** -0.5)
+    assert_close(io, po, atol=2e-3, rtol=2e-3, what="ragged, inline variant vs rotated rows")
+    assert_close(il, pl, atol=2e-3, rtol=1e-4, what="ragged lse")

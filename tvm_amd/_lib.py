@@ -45,6 +45,15 @@ SIGNATURES = {
                                                  c_i32, c_i32, c_i32, c_vp],
     "tvmkv_batch_decode_paged_kv_noalloc": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32,
                                                          c_i32, c_i32, c_i32, c_i32, c_vp],
+    "tvmkv_batch_decode_paged_kv_scaled": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32, c_i32,
+                                                        c_i32, c_i32, c_i32, c_vp, c_vp],
+    "tvmkv_batch_prefill_ragged_kv_scaled": [c_vp] * 9 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i32,
+                                                          c_i32, c_i32, c_i32, c_vp, c_vp],
+    "tvmkv_batch_prefill_paged_kv_scaled": [c_vp] * 10 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64,
+                                                          c_i64, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
+                                                          c_vp, c_vp],
+    "tvmkv_batch_tree_attn_scaled": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i32, c_i32, c_i32,
+                                                   c_vp, c_vp],
     "tvmkv_fused_decode_step": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i64, c_i32, c_i32, c_i32, c_i32,
                                              c_vp],
     "tvmkv_batch_tree_attn": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_i32, c_i64, c_i32, c_i32, c_i32, c_vp],

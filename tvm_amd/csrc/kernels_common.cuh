@@ -192,6 +192,41 @@ __device__ __forceinline__ void rope_pair(half8_t& lo, half8_t& hi, float pos_sc
   }
 }
 
+// The table an attention kernel rotates q and k with (in-kernel RoPE, rotate-half pairing over the whole
+// head, python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-127).  v[d], d < D: the divisor of element
+// d's angle (angle = position / v[d]) or, with `inverse`, its inverse frequency (angle = position * v[d]);
+// element d and its partner d + D/2 share an angle unless `halves_differ`; cos and sin are multiplied by
+// `magnitude`.  Built on the host in float32 in the reference's order of operations (inline_rope_table).
+constexpr int kMaxHeadDim = 256;
+struct InlineRopeTable {
+  float v[kMaxHeadDim];
+  int inverse;
+  int halves_differ;
+  float magnitude;
+};
+
+// rope_pair for any frequency variant: table entries of the 8 elements of `lo` and of `hi`.
+__device__ __forceinline__ void rope_pair_ex(half8_t& lo, half8_t& hi, float pos_scaled, const float* tbl_lo8,
+                                             const float* tbl_hi8, int inverse, int halves_differ, float magnitude) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float sn, cs;
+    sincos_reduced(inverse ? pos_scaled * tbl_lo8[i] : pos_scaled / tbl_lo8[i], sn, cs);
+    sn *= magnitude;
+    cs *= magnitude;
+    float sn_hi = sn, cs_hi = cs;
+    if (halves_differ) {
+      sincos_reduced(inverse ? pos_scaled * tbl_hi8[i] : pos_scaled / tbl_hi8[i], sn_hi, cs_hi);
+      sn_hi *= magnitude;
+      cs_hi *= magnitude;
+    }
+    const float xl = static_cast<float>(lo[i]);
+    const float xh = static_cast<float>(hi[i]);
+    lo[i] = static_cast<half_t>(cs * xl + sn * (-xh));
+    hi[i] = static_cast<half_t>(cs_hi * xh + sn_hi * xl);
+  }
+}
+
 // Compute units of the current device (cached per device).
 inline int compute_units() {
   static int cached[64] = {0};

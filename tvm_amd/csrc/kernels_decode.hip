@@ -70,6 +70,11 @@ struct DecodeParams {
   // padded head dims (80, 96, 112 on the head dim 128 kernel): elements per row of q, the pages and the
   // output in memory; 0 = the kernel's head dim
   int d_mem;
+  // how the entries of the RoPE table are used (InlineRopeTable): position * entry instead of position /
+  // entry; separate entries for the two halves of a head; a factor on cos and sin
+  int rope_inverse;
+  int rope_halves_differ;
+  float rope_magnitude;
 };
 
 // Same answer as find_sequence, computed by one wavefront as a 64-ary search: the lanes probe
@@ -250,9 +255,10 @@ __device__ __forceinline__ int dm_swizzle(int row) {
   return D >= 128 ? (row & 7) << 1 : ((row >> 1) & 3) << 1;
 }
 
-// theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
+// One entry per element of the head for in-kernel RoPE (the default: theta^(2i/D) for elements i and
+// i + D/2), computed on the host with the libm call the CPU kernels use; DecodeParams says how they are used
 struct DecodeRopeDivisors {
-  float v[128];
+  float v[256];
 };
 
 // EXT = false: plain cache, q and k already rotated (or no RoPE).  EXT = true adds the sliding-window
@@ -339,12 +345,15 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
   const int win_lo = EXT && p.window_offset != nullptr ? p.window_offset[b] : 0;
   // RoPE divisors of the first halves of this lane's K fragment pairs: features i*32 + g4*8 + e, or
   // with KLINE i*64 + (c16&1)*32 + g4*8 + e
-  float divr[8 * (NPAIR > 0 ? NPAIR : 1)];
+  // (and of the second halves, features + D/2, which differ from the first in some frequency variants)
+  float divr[8 * (NPAIR > 0 ? NPAIR : 1)], divh[8 * (NPAIR > 0 ? NPAIR : 1)];
   float k_pos0 = 0.f;
   if (EXT && p.rotary) {
 #pragma unroll
     for (int i = 0; i < 8 * NPAIR; ++i) {
-      divr[i] = div.v[KLINE ? (i >> 3) * 64 + (c16 & 1) * 32 + g4 * 8 + (i & 7) : (i >> 3) * 32 + g4 * 8 + (i & 7)];
+      const int f = KLINE ? (i >> 3) * 64 + (c16 & 1) * 32 + g4 * 8 + (i & 7) : (i >> 3) * 32 + g4 * 8 + (i & 7);
+      divr[i] = div.v[f];
+      divh[i] = div.v[f + D / 2];
     }
     k_pos0 = static_cast<float>(p.k_rope_pos_offset[b]);
   }
@@ -418,10 +427,13 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
       const float q_pos = static_cast<float>(p.q_rope_position[b]) * p.rope_scale;
 #pragma unroll
       for (int ks = 0; ks < KS / 2; ++ks) {
-        float qdiv[8];
+        float qdiv[8], qdivh[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qdiv[e] = div.v[ks * 32 + g4 * 8 + e];
-        rope_pair(qv[ks].h8, qv[ks + KS / 2].h8, q_pos, qdiv);
+        for (int e = 0; e < 8; ++e) {
+          qdiv[e] = div.v[ks * 32 + g4 * 8 + e];
+          qdivh[e] = div.v[D / 2 + ks * 32 + g4 * 8 + e];
+        }
+        rope_pair_ex(qv[ks].h8, qv[ks + KS / 2].h8, q_pos, qdiv, qdivh, p.rope_inverse, p.rope_halves_differ, p.rope_magnitude);
       }
     }
 #pragma unroll
@@ -544,7 +556,10 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
           const float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
           Vec16* frag = r.k[h] + (KLINE ? tile * TI : 0);
 #pragma unroll
-          for (int i = 0; i < NPAIR; ++i) rope_pair(frag[i].h8, frag[i + NPAIR].h8, pos, divr + 8 * i);
+          for (int i = 0; i < NPAIR; ++i) {
+            rope_pair_ex(frag[i].h8, frag[i + NPAIR].h8, pos, divr + 8 * i, divh + 8 * i, p.rope_inverse, p.rope_halves_differ,
+                         p.rope_magnitude);
+          }
         }
       }
     }
@@ -774,6 +789,7 @@ struct FusedStep {
   const void* qkv = nullptr;
   const int32_t* append_position_map = nullptr;
   int apply_rope = 0;
+  const tvmkv_rope_scaling* rope_scaling = nullptr;  // frequency variant of the in-kernel RoPE of a plain call
 };
 
 // Body of the decode entry point.  lease(bytes) hands out the scratch memory of the call: arrival
@@ -842,6 +858,8 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   KV_CHECK(slots < (int64_t{1} << 31)) << "batch_decode_paged_kv: too many chunks";
   const size_t part_o_bytes = static_cast<size_t>(slots) * h_q * dk * sizeof(float);
   p.d_mem = padded ? d : 0;
+  p.rope_inverse = p.rope_halves_differ = 0;
+  p.rope_magnitude = 1.0f;
   const size_t part_ml_bytes = static_cast<size_t>(slots) * h_q * 2 * sizeof(float);
   const ScratchLease ws = lease(kArrivalBytes + part_o_bytes + part_ml_bytes);
   p.part_o = reinterpret_cast<float*>(ws.ptr + kArrivalBytes);
@@ -868,8 +886,11 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   if (p.rotary || (fused_launch && p.apply_rope)) {
     KV_CHECK(k_rope_pos_offset || fused_launch) << "batch_decode_paged_kv: inline RoPE needs the position arrays";
     KV_CHECK(q_rope_position) << "batch_decode_paged_kv: inline RoPE needs the position arrays";
-    const float theta = static_cast<float>(rope_theta);
-    for (int i = 0; i < d / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(d));
+    const InlineRopeHost table = inline_rope_table(fused_launch ? nullptr : fused_step.rope_scaling, d, rope_theta);
+    for (int i = 0; i < d; ++i) div.v[i] = table.v[i];
+    p.rope_inverse = table.inverse;
+    p.rope_halves_differ = table.halves_differ;
+    p.rope_magnitude = table.magnitude;
   }
   if (padded) {
     auto launch_padded = [&](auto kernel) {
@@ -939,6 +960,26 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
   KV_API_BEGIN();
   hipStream_t s = as_stream(stream);
   decode_entry([&](size_t bytes) { return lease_scratch(kScratchDecode, s, bytes, kArrivalBytes); }, FusedStep{}, q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode,
+               rope_scale, rope_theta, sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d, page_size,
+               sliding_window, stream);
+  KV_API_END();
+}
+
+// tvmkv_batch_decode_paged_kv with a frequency variant for the in-kernel RoPE (rotary_mode != 0)
+extern "C" int tvmkv_batch_decode_paged_kv_scaled(const void* q, const void* pages, const int32_t* page_indptr,
+                                                  const int32_t* page_values, const int32_t* length_info,
+                                                  const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,
+                                                  void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                                                  double rope_theta, double sm_scale, int32_t batch_size,
+                                                  int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
+                                                  int32_t d, int32_t page_size, int32_t sliding_window,
+                                                  const tvmkv_rope_scaling* rope_scaling, void* stream) {
+  KV_API_BEGIN();
+  hipStream_t s = as_stream(stream);
+  FusedStep plain;
+  plain.rope_scaling = rope_scaling;
+  decode_entry([&](size_t bytes) { return lease_scratch(kScratchDecode, s, bytes, kArrivalBytes); }, plain, q, pages,
+               page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode,
                rope_scale, rope_theta, sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d, page_size,
                sliding_window, stream);
   KV_API_END();

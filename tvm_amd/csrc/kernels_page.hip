@@ -8,6 +8,7 @@
 #include <cmath>
 
 #include "kernels_common.cuh"
+#include "runtime_support.h"
 
 namespace tvmkv {
 
@@ -22,7 +23,6 @@ namespace tvmkv {
 // One entry per element of the head: element d and its rotation partner d + D/2 share an angle in
 // every variant but yarn, whose blend between interpolated and extrapolated frequencies is indexed
 // by the element (position_embedding.py:244-247).
-constexpr int kMaxHeadDim = 256;
 struct RopeDivisors {
   float v[kMaxHeadDim];
 };
@@ -656,3 +656,27 @@ int tvmkv_merge_state_inplace(void* v, float* s, const void* v_other, const floa
 }
 
 }  // extern "C"
+
+namespace tvmkv {
+
+InlineRopeHost inline_rope_table(const ::tvmkv_rope_scaling* scaling, int head_dim, double rope_theta) {
+  KV_CHECK(head_dim > 0 && head_dim <= kMaxHeadDim && head_dim % 2 == 0) << "in-kernel RoPE: head_dim " << head_dim;
+  InlineRopeHost out{};
+  RopeDivisors table{};
+  const float* no_factors = nullptr;  // the attention kernels take no factor tensor (_kernel_common.py:115-127)
+  bool differ = false;
+  tvmkv_rope_scaling whole_head{};
+  if (scaling != nullptr) {
+    whole_head = *scaling;
+    whole_head.rotary_dim = 0;  // the attention kernels rotate the whole head, whatever the split-rotary kernel does
+  }
+  out.inverse = rope_table(scaling != nullptr ? &whole_head : nullptr, head_dim, rope_theta, /*seq_len=*/0, &no_factors, &table,
+                           &out.magnitude, &differ)
+                    ? 1
+                    : 0;
+  out.halves_differ = differ ? 1 : 0;
+  for (int d = 0; d < head_dim; ++d) out.v[d] = differ ? table.v[d] : table.v[d % (head_dim / 2)];
+  return out;
+}
+
+}  // namespace tvmkv

@@ -225,10 +225,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
   const int kv_len = phys_len - win_lo + sink;
   // number of logical keys -> physical end of the tokens that hold them
   auto to_phys = [&](int n) { return (!EXT || n <= sink) ? n : n - sink + win_lo; };
-  __shared__ float div_lds[DQK > 128 ? 128 : 64];
+  __shared__ float div_lds[DQK > 256 ? 256 : DQK];
   const bool q_rope = (EXT && p.rotary) || (BOTH && p.q_inline_rope != 0);  // uniform over the launch
   if (q_rope) {
-    if (tid < DQK / 2) div_lds[tid] = div.v[tid];
+    if (tid < DQK && tid < 256) div_lds[tid] = div.v[tid];
     __syncthreads();
   }
 
@@ -282,7 +282,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
     if (q_rope && row_valid) {
       const float q_pos = static_cast<float>(p.q_rope_position[q_start + my_pos]) * p.rope_scale;
 #pragma unroll
-      for (int ks = 0; ks < KS / 2; ++ks) rope_pair(qf[ks], qf[ks + KS / 2], q_pos, div_lds + ks * 16 + half * 8);
+      for (int ks = 0; ks < KS / 2; ++ks) {
+        rope_pair_ex(qf[ks], qf[ks + KS / 2], q_pos, div_lds + ks * 16 + half * 8, div_lds + DQK / 2 + ks * 16 + half * 8,
+                     p.rope_inverse, p.rope_halves_differ, p.rope_magnitude);
+      }
     }
   }
   const float k_pos0 = (EXT && p.rotary) ? static_cast<float>(p.k_rope_pos_offset[b]) : 0.f;
@@ -659,7 +662,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
         float pos = (k_pos0 + static_cast<float>(logical)) * p.rope_scale;
         if (!PAGED && p.k_pos_from_q) pos = static_cast<float>(p.q_rope_position[kv_start + t]) * p.rope_scale;
 #pragma unroll
-        for (int ks = 0; ks < KS / 2; ++ks) rope_pair(kf[ks], kf[ks + KS / 2], pos, div_lds + ks * 16 + half * 8);
+        for (int ks = 0; ks < KS / 2; ++ks) {
+          rope_pair_ex(kf[ks], kf[ks + KS / 2], pos, div_lds + ks * 16 + half * 8, div_lds + DQK / 2 + ks * 16 + half * 8,
+                       p.rope_inverse, p.rope_halves_differ, p.rope_magnitude);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
       float16_t acc = qk(kf);
@@ -898,14 +904,24 @@ struct KvSplit {
 
 // The extended kernels (sliding-window cache, per-layer window, inline RoPE) exist for the head
 // dims that RoPE models use here; d_qk 192 / d_v 128 is the MLA self-attention, which has neither.
+// scaling: the frequency variant of the in-kernel RoPE (NULL: default); used when the launch rotates at all
 template <int DQK, int DV, int SRC, int PS>
-static void launch_prefill(const PrefillParams& p, int64_t total_q, bool ext, double rope_theta, hipStream_t stream) {
+static void launch_prefill(const PrefillParams& params, int64_t total_q, bool ext, double rope_theta, hipStream_t stream,
+                           const tvmkv_rope_scaling* scaling = nullptr) {
   PrefillRopeDivisors div{};
-  if (!ext) {
-    if (p.q_inline_rope) {
-      const float theta = static_cast<float>(rope_theta);
-      for (int i = 0; i < DQK / 2 && i < 128; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DQK));
+  PrefillParams p = params;
+  p.rope_magnitude = 1.0f;
+  auto fill_table = [&]() {
+    if constexpr (DQK <= 256) {
+      const InlineRopeHost table = inline_rope_table(scaling, DQK, rope_theta);
+      for (int i = 0; i < DQK; ++i) div.v[i] = table.v[i];
+      p.rope_inverse = table.inverse;
+      p.rope_halves_differ = table.halves_differ;
+      p.rope_magnitude = table.magnitude;
     }
+  };
+  if (!ext) {
+    if (p.q_inline_rope) fill_table();
     if constexpr (SRC == kPaged) {
       if (p.stream_kv) {
         launch_prefill_ext<DQK, DV, SRC, PS, false, true>(p, total_q, div, stream);
@@ -916,8 +932,7 @@ static void launch_prefill(const PrefillParams& p, int64_t total_q, bool ext, do
     return;
   }
   if constexpr (DQK == DV && SRC != kBoth) {
-    const float theta = static_cast<float>(rope_theta);
-    for (int i = 0; i < DQK / 2; ++i) div.v[i] = powf(theta, static_cast<float>(i * 2) / static_cast<float>(DQK));
+    if (p.rotary) fill_table();
     if constexpr (SRC == kPaged) {
       if (p.stream_kv) {
         launch_prefill_ext<DQK, DV, SRC, PS, true, true>(p, total_q, div, stream);
@@ -949,12 +964,12 @@ using namespace tvmkv;
 
 extern "C" {
 
-int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const void* k, const void* v,
-                                  const int32_t* kv_indptr, const int32_t* q_rope_position,
-                                  const int32_t* k_rope_pos_offset, void* output, float* lse, int64_t causal,
-                                  int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
-                                  int32_t batch_size, int64_t total_q, int32_t h_q, int32_t h_kv, int32_t d_qk,
-                                  int32_t d_v, void* stream) {
+static int ragged_prefill(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                          const int32_t* kv_indptr, const int32_t* q_rope_position,
+                          const int32_t* k_rope_pos_offset, void* output, float* lse, int64_t causal,
+                          int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                          int32_t batch_size, int64_t total_q, int32_t h_q, int32_t h_kv, int32_t d_qk,
+                          int32_t d_v, const tvmkv_rope_scaling* scaling, void* stream) {
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_ragged_kv: bad shape";
@@ -983,11 +998,11 @@ int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const 
   const bool ext = p.rotary != 0;
   hipStream_t s = as_stream(stream);
   if (d_qk == 128 && d_v == 128) {
-    launch_prefill<128, 128, kRagged, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<128, 128, kRagged, 16>(p, total_q, ext, rope_theta, s, scaling);
   } else if (d_qk == 64 && d_v == 64) {
-    launch_prefill<64, 64, kRagged, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<64, 64, kRagged, 16>(p, total_q, ext, rope_theta, s, scaling);
   } else if (d_qk == 256 && d_v == 256) {
-    launch_prefill<256, 256, kRagged, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<256, 256, kRagged, 16>(p, total_q, ext, rope_theta, s, scaling);
   } else if (d_qk == 192 && d_v == 128) {
     launch_prefill<192, 128, kRagged, 16>(p, total_q, ext, rope_theta, s);
   } else if (d_qk == d_v && padded_head_dim(d_qk)) {
@@ -1000,13 +1015,34 @@ int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const 
   KV_API_END();
 }
 
+int tvmkv_batch_prefill_ragged_kv(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                                  const int32_t* kv_indptr, const int32_t* q_rope_position,
+                                  const int32_t* k_rope_pos_offset, void* output, float* lse, int64_t causal,
+                                  int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                                  int32_t batch_size, int64_t total_q, int32_t h_q, int32_t h_kv, int32_t d_qk,
+                                  int32_t d_v, void* stream) {
+  return ragged_prefill(q, q_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_offset, output, lse, causal, rotary_mode,
+                        rope_scale, rope_theta, sm_scale, batch_size, total_q, h_q, h_kv, d_qk, d_v, nullptr, stream);
+}
+
+int tvmkv_batch_prefill_ragged_kv_scaled(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                                         const int32_t* kv_indptr, const int32_t* q_rope_position,
+                                         const int32_t* k_rope_pos_offset, void* output, float* lse, int64_t causal,
+                                         int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                                         int32_t batch_size, int64_t total_q, int32_t h_q, int32_t h_kv, int32_t d_qk,
+                                         int32_t d_v, const tvmkv_rope_scaling* rope_scaling, void* stream) {
+  return ragged_prefill(q, q_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_offset, output, lse, causal, rotary_mode,
+                        rope_scale, rope_theta, sm_scale, batch_size, total_q, h_q, h_kv, d_qk, d_v, rope_scaling, stream);
+}
+
 static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pages, const int32_t* page_indptr,
                          const int32_t* page_values, const int32_t* length_info, const int32_t* k_rope_pos_offset,
                          const int32_t* q_rope_position, void* output, float* lse, int64_t causal,
                          int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
                          int32_t batch_size, int64_t total_q, int64_t nnz_pages, int64_t num_pages, int32_t h_q,
                          int32_t h_kv, int32_t d, int32_t page_size, int32_t sliding_window,
-                         int32_t sliding_window_size, bool merge_into, void* stream) {
+                         int32_t sliding_window_size, bool merge_into, void* stream,
+                         const tvmkv_rope_scaling* scaling = nullptr) {
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_paged_kv: bad shape";
@@ -1049,11 +1085,11 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
   hipStream_t s = as_stream(stream);
   const KvSplit split(p, total_q, nnz_pages * page_size / batch_size, d, s);
   if (d == 128) {
-    launch_prefill<128, 128, kPaged, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<128, 128, kPaged, 16>(p, total_q, ext, rope_theta, s, scaling);
   } else if (d == 64) {
-    launch_prefill<64, 64, kPaged, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<64, 64, kPaged, 16>(p, total_q, ext, rope_theta, s, scaling);
   } else if (d == 256) {
-    launch_prefill<256, 256, kPaged, 16>(p, total_q, ext, rope_theta, s);
+    launch_prefill<256, 256, kPaged, 16>(p, total_q, ext, rope_theta, s, scaling);
   } else if (padded_head_dim(d)) {
     launch_prefill_padded<kPaged>(p, total_q, d, ext, "batch_prefill_paged_kv", s);
   } else {
@@ -1090,6 +1126,21 @@ int tvmkv_batch_prefill_paged_kv_merge(const void* q, const int32_t* q_indptr, c
                        output, lse, causal, rotary_mode, rope_scale, rope_theta, sm_scale, batch_size, total_q,
                        nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window, sliding_window_size,
                        /*merge_into=*/true, stream);
+}
+
+int tvmkv_batch_prefill_paged_kv_scaled(const void* q, const int32_t* q_indptr, const void* pages,
+                                        const int32_t* page_indptr, const int32_t* page_values,
+                                        const int32_t* length_info, const int32_t* k_rope_pos_offset,
+                                        const int32_t* q_rope_position, void* output, float* lse, int64_t causal,
+                                        int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                                        int32_t batch_size, int64_t total_q, int64_t nnz_pages, int64_t num_pages,
+                                        int32_t h_q, int32_t h_kv, int32_t d, int32_t page_size, int32_t sliding_window,
+                                        int32_t sliding_window_size, int32_t merge_into,
+                                        const tvmkv_rope_scaling* rope_scaling, void* stream) {
+  return paged_prefill(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position,
+                       output, lse, causal, rotary_mode, rope_scale, rope_theta, sm_scale, batch_size, total_q,
+                       nnz_pages, num_pages, h_q, h_kv, d, page_size, sliding_window, sliding_window_size,
+                       merge_into != 0, stream, rope_scaling);
 }
 
 static int cached_and_new(const void* q, int64_t q_token_stride, const int32_t* q_rope_position, int64_t apply_rope,
@@ -1172,11 +1223,11 @@ int tvmkv_batch_prefill_cached_and_new_kv_fused_q(const void* qkv, const int32_t
                         batch_size, total_q, nnz_pages, num_pages, h_q, h_kv, d, page_size, stream);
 }
 
-int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k, const void* v,
-                          const int32_t* kv_indptr, const int32_t* q_rope_position, const int32_t* mn_indptr,
-                          const int32_t* mask, void* output, float* lse, int64_t rotary_mode, double rope_scale,
-                          double rope_theta, double sm_scale, int32_t batch_size, int64_t total_q, int32_t h_q,
-                          int32_t h_kv, int32_t d, void* stream) {
+static int tree_attn_ragged(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                            const int32_t* kv_indptr, const int32_t* q_rope_position, const int32_t* mn_indptr,
+                            const int32_t* mask, void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                            double rope_theta, double sm_scale, int32_t batch_size, int64_t total_q, int32_t h_q,
+                            int32_t h_kv, int32_t d, const tvmkv_rope_scaling* scaling, void* stream) {
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0) << "batch_tree_attn: bad shape";
   if (batch_size == 0 || total_q == 0) return TVMKV_OK;
@@ -1205,16 +1256,34 @@ int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k,
   p.tree_order = mask;
   hipStream_t s = as_stream(stream);
   if (d == 128) {
-    launch_prefill<128, 128, kRagged, 16>(p, total_q, true, rope_theta, s);
+    launch_prefill<128, 128, kRagged, 16>(p, total_q, true, rope_theta, s, scaling);
   } else if (d == 64) {
-    launch_prefill<64, 64, kRagged, 16>(p, total_q, true, rope_theta, s);
+    launch_prefill<64, 64, kRagged, 16>(p, total_q, true, rope_theta, s, scaling);
   } else if (d == 256) {
-    launch_prefill<256, 256, kRagged, 16>(p, total_q, true, rope_theta, s);
+    launch_prefill<256, 256, kRagged, 16>(p, total_q, true, rope_theta, s, scaling);
   } else {
     KV_UNSUPPORTED(true) << "batch_tree_attn: head_dim " << d << " is not built (64, 128, 256)";
   }
   KV_LAUNCH_CHECK();
   KV_API_END();
+}
+
+int tvmkv_batch_tree_attn(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                          const int32_t* kv_indptr, const int32_t* q_rope_position, const int32_t* mn_indptr,
+                          const int32_t* mask, void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                          double rope_theta, double sm_scale, int32_t batch_size, int64_t total_q, int32_t h_q,
+                          int32_t h_kv, int32_t d, void* stream) {
+  return tree_attn_ragged(q, q_indptr, k, v, kv_indptr, q_rope_position, mn_indptr, mask, output, lse, rotary_mode, rope_scale,
+                          rope_theta, sm_scale, batch_size, total_q, h_q, h_kv, d, nullptr, stream);
+}
+
+int tvmkv_batch_tree_attn_scaled(const void* q, const int32_t* q_indptr, const void* k, const void* v,
+                                 const int32_t* kv_indptr, const int32_t* q_rope_position, const int32_t* mn_indptr,
+                                 const int32_t* mask, void* output, float* lse, int64_t rotary_mode, double rope_scale,
+                                 double rope_theta, double sm_scale, int32_t batch_size, int64_t total_q, int32_t h_q,
+                                 int32_t h_kv, int32_t d, const tvmkv_rope_scaling* rope_scaling, void* stream) {
+  return tree_attn_ragged(q, q_indptr, k, v, kv_indptr, q_rope_position, mn_indptr, mask, output, lse, rotary_mode, rope_scale,
+                          rope_theta, sm_scale, batch_size, total_q, h_q, h_kv, d, rope_scaling, stream);
 }
 
 int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void* pages, const int32_t* page_indptr,

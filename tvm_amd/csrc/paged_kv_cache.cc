@@ -280,11 +280,11 @@ class PagedKVCache {
       return;
     }
     const int rotary = attn_kinds_[layer_id] == TVMKV_ATTN_MHA ? (rope_mode_ == TVMKV_ROPE_INLINE) : 0;
-    Launch(tvmkv_batch_prefill_ragged_kv(q, Dev(s.cur_append_lengths_indptr), k, v, Dev(s.cur_append_lengths_indptr),
-                                         Dev(s.q_rope_position_map), Dev(s.k_ragged_rope_pos_offset), o, lse,
-                                         /*causal=*/1, rotary, rotary_scale_, rotary_theta_, sm_scale,
-                                         book_->batch_size(), total_seq_length, num_qo_heads_, k_heads, qk_dim, v_dim,
-                                         compute_stream_));
+    Launch(tvmkv_batch_prefill_ragged_kv_scaled(q, Dev(s.cur_append_lengths_indptr), k, v, Dev(s.cur_append_lengths_indptr),
+                                                Dev(s.q_rope_position_map), Dev(s.k_ragged_rope_pos_offset), o, lse,
+                                                /*causal=*/1, rotary, rotary_scale_, rotary_theta_, sm_scale,
+                                                book_->batch_size(), total_seq_length, num_qo_heads_, k_heads, qk_dim, v_dim,
+                                                InlineScaling(), compute_stream_));
     RecordComputeEvent();
   }
 
@@ -423,9 +423,8 @@ class PagedKVCache {
     // a description that differs from the default rotation: another frequency rule, or only part of the head rotated
     has_rope_scaling_ = scaling != nullptr && (scaling->rope_type != TVMKV_ROPE_FREQ_DEFAULT ||
                                                (scaling->rotary_dim > 0 && scaling->rotary_dim != qk_head_dim_));
-    KV_UNSUPPORTED(has_rope_scaling_ && rope_mode_ == TVMKV_ROPE_INLINE)
-        << "RoPE scaling variants and partial rotation are not built for caches that rotate inside the attention "
-           "kernels (inline RoPE)";
+    // (a cache that rotates inside the attention kernels hands the description to them: they rotate the whole
+    // head with the variant's frequencies, python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-127)
     KV_CHECK((scaling != nullptr && scaling->rope_type == TVMKV_ROPE_FREQ_LONGROPE) || rope_ext_factors == nullptr)
         << "rope_ext_factors needs a longrope scaling description";
     if (has_rope_scaling_) rope_scaling_ = *scaling;
@@ -672,19 +671,20 @@ class PagedKVCache {
     const StepLayout& s = book_->step();
     const int rope_inline = rope_mode_ == TVMKV_ROPE_INLINE;
     if (s.is_chain[0]) {
-      Launch(tvmkv_batch_prefill_ragged_kv(q, Dev(s.cur_append_lengths_indptr), k, v, Dev(s.cur_append_lengths_indptr),
-                                           Dev(s.q_rope_position_map), Dev(s.k_ragged_rope_pos_offset), o, lse,
-                                           /*causal=*/1, rope_inline, rotary_scale_, rotary_theta_, sm_scale,
-                                           book_->batch_size(), total_seq_length, num_qo_heads_, num_kv_heads_,
-                                           qk_head_dim_, v_head_dim_, compute_stream_));
+      Launch(tvmkv_batch_prefill_ragged_kv_scaled(q, Dev(s.cur_append_lengths_indptr), k, v, Dev(s.cur_append_lengths_indptr),
+                                                  Dev(s.q_rope_position_map), Dev(s.k_ragged_rope_pos_offset), o, lse,
+                                                  /*causal=*/1, rope_inline, rotary_scale_, rotary_theta_, sm_scale,
+                                                  book_->batch_size(), total_seq_length, num_qo_heads_, num_kv_heads_,
+                                                  qk_head_dim_, v_head_dim_, InlineScaling(), compute_stream_));
     } else {
       // the batch forms token trees
       KV_CHECK(s.tree_attn_mask[0].present() && s.tree_attn_mn_indptr[0].present()) << "token-tree mask is not on the device";
       KV_CHECK(qk_head_dim_ == v_head_dim_) << "tree attention needs equal qk and v head dims";
-      Launch(tvmkv_batch_tree_attn(q, Dev(s.cur_append_lengths_indptr), k, v, Dev(s.cur_append_lengths_indptr),
-                                   Dev(s.q_rope_position_map), Dev(s.tree_attn_mn_indptr[0]), Dev(s.tree_attn_mask[0]), o,
-                                   lse, rope_inline, rotary_scale_, rotary_theta_, sm_scale, book_->batch_size(),
-                                   total_seq_length, num_qo_heads_, num_kv_heads_, qk_head_dim_, compute_stream_));
+      Launch(tvmkv_batch_tree_attn_scaled(q, Dev(s.cur_append_lengths_indptr), k, v, Dev(s.cur_append_lengths_indptr),
+                                          Dev(s.q_rope_position_map), Dev(s.tree_attn_mn_indptr[0]), Dev(s.tree_attn_mask[0]), o,
+                                          lse, rope_inline, rotary_scale_, rotary_theta_, sm_scale, book_->batch_size(),
+                                          total_seq_length, num_qo_heads_, num_kv_heads_, qk_head_dim_, InlineScaling(),
+                                          compute_stream_));
     }
   }
 
@@ -721,26 +721,29 @@ class PagedKVCache {
                                         total_seq_length, nnz_pages, num_total_pages_, num_qo_heads_, num_kv_heads_,
                                         qk_head_dim_, page_size_, sliding_window, compute_stream_));
       } else if (s.use_decode_kernel[d]) {
-        Launch(tvmkv_batch_decode_paged_kv(q, pages_[local_layer_id], page_indptr, page_indices, length_info, k_rope_pos,
-                                           q_pos, attn_output, attn_lse, rotary_mode, rotary_scale, rotary_theta, sm_scale,
-                                           entries, nnz_pages, num_total_pages_, num_qo_heads_, num_kv_heads_,
-                                           qk_head_dim_, page_size_, sliding_window, compute_stream_));
+        Launch(tvmkv_batch_decode_paged_kv_scaled(q, pages_[local_layer_id], page_indptr, page_indices, length_info,
+                                                  k_rope_pos, q_pos, attn_output, attn_lse, rotary_mode, rotary_scale,
+                                                  rotary_theta, sm_scale, entries, nnz_pages, num_total_pages_,
+                                                  num_qo_heads_, num_kv_heads_, qk_head_dim_, page_size_, sliding_window,
+                                                  InlineScaling(), compute_stream_));
       } else if (!is_first_kernel) {
         // The prefill kernel merges its state into (o, lse) in its epilogue: one launch for the
         // kernel and the merge of :2285-2292, and no temporary output.
-        Launch(tvmkv_batch_prefill_paged_kv_merge(q, qo_indptr, pages_[local_layer_id], page_indptr, page_indices,
-                                                  length_info, k_rope_pos, q_pos, o, lse, causal, rotary_mode, rotary_scale,
-                                                  rotary_theta, sm_scale, entries, total_seq_length, nnz_pages,
-                                                  num_total_pages_, num_qo_heads_, num_kv_heads_, qk_head_dim_, page_size_,
-                                                  sliding_window, layer_sliding_window_size_, compute_stream_));
+        Launch(tvmkv_batch_prefill_paged_kv_scaled(q, qo_indptr, pages_[local_layer_id], page_indptr, page_indices,
+                                                   length_info, k_rope_pos, q_pos, o, lse, causal, rotary_mode, rotary_scale,
+                                                   rotary_theta, sm_scale, entries, total_seq_length, nnz_pages,
+                                                   num_total_pages_, num_qo_heads_, num_kv_heads_, qk_head_dim_, page_size_,
+                                                   sliding_window, layer_sliding_window_size_, /*merge_into=*/1,
+                                                   InlineScaling(), compute_stream_));
         cross_attn_computed = true;
         continue;
       } else {
-        Launch(tvmkv_batch_prefill_paged_kv(q, qo_indptr, pages_[local_layer_id], page_indptr, page_indices, length_info,
-                                            k_rope_pos, q_pos, attn_output, attn_lse, causal, rotary_mode, rotary_scale,
-                                            rotary_theta, sm_scale, entries, total_seq_length, nnz_pages, num_total_pages_,
-                                            num_qo_heads_, num_kv_heads_, qk_head_dim_, page_size_, sliding_window,
-                                            layer_sliding_window_size_, compute_stream_));
+        Launch(tvmkv_batch_prefill_paged_kv_scaled(q, qo_indptr, pages_[local_layer_id], page_indptr, page_indices,
+                                                   length_info, k_rope_pos, q_pos, attn_output, attn_lse, causal, rotary_mode,
+                                                   rotary_scale, rotary_theta, sm_scale, entries, total_seq_length, nnz_pages,
+                                                   num_total_pages_, num_qo_heads_, num_kv_heads_, qk_head_dim_, page_size_,
+                                                   sliding_window, layer_sliding_window_size_, /*merge_into=*/0,
+                                                   InlineScaling(), compute_stream_));
       }
       if (!is_first_kernel) {
         Launch(tvmkv_merge_state_inplace(o, lse, temp_out_, temp_lse_, total_seq_length, num_qo_heads_, v_head_dim_,
@@ -813,6 +816,10 @@ class PagedKVCache {
   int rope_mode_ = TVMKV_ROPE_NORMAL;
   double rotary_scale_, rotary_theta_;
 
+  // the frequency variant of the in-kernel RoPE: the attention kernels of a cache in inline-RoPE mode
+  const tvmkv_rope_scaling* InlineScaling() const {
+    return (has_rope_scaling_ && rope_mode_ == TVMKV_ROPE_INLINE) ? &rope_scaling_ : nullptr;
+  }
   bool has_rope_scaling_ = false;
   tvmkv_rope_scaling rope_scaling_{};
   const float* rope_ext_factors_ = nullptr;

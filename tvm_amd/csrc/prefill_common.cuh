@@ -57,11 +57,17 @@ struct PrefillParams {
   int page_shift;   // pages hold 16 << page_shift tokens; the kernel walks them as runs of 16-token pages
   int stream_kv;    // != 0: every K/V row is read by one row tile only: copy it with the streaming hint
   int d_mem;        // padded head dims (prefill_kernel<..., PAD = true>): elements per row in memory
+  // how the entries of the RoPE table are used (InlineRopeTable): position * entry instead of position /
+  // entry; separate entries for the two halves of a head; a factor on cos and sin
+  int rope_inverse;
+  int rope_halves_differ;
+  float rope_magnitude;
 };
 
-// theta^(2i/D), i < D/2, computed on the host with the libm call the CPU kernels use
+// One entry per element of the head for in-kernel RoPE (the default: theta^(2i/D) for elements i and
+// i + D/2), computed on the host with the libm call the CPU kernels use
 struct PrefillRopeDivisors {
-  float v[128];
+  float v[256];
 };
 
 __device__ __forceinline__ int tile_slot_begin(const int32_t* q_indptr, int b, int group) {

@@ -9,6 +9,8 @@
 #include <cstdint>
 #include <mutex>
 
+struct tvmkv_rope_scaling;  // include/tvmkv.h
+
 namespace tvmkv {
 
 enum Option {
@@ -48,6 +50,17 @@ uint32_t next_scratch_epoch(uint64_t* launches, bool* wrapped);
 void zero_scratch_counters(char* ptr, size_t counter_bytes, hipStream_t stream);
 // Test aid: sets the launch count of every pooled buffer (to run a launch across the epoch wrap).
 void debug_set_scratch_launches(uint64_t launches);
+
+// The table of an attention kernel's in-kernel RoPE for a frequency variant (NULL: the default
+// frequencies): entries for all head_dim elements, see InlineRopeTable in kernels_common.cuh.  Host
+// arithmetic only (defined next to the split-rotary kernel's tables in kernels_page.hip).
+struct InlineRopeHost {
+  float v[256];
+  int inverse;
+  int halves_differ;
+  float magnitude;
+};
+InlineRopeHost inline_rope_table(const ::tvmkv_rope_scaling* scaling, int head_dim, double rope_theta);
 
 // Chunk-slot arithmetic of the decode split, on the host (the device functions of the same names in
 // kernels_decode.hip compute the same values; the tests compare both against a direct enumeration).

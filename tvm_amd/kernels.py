@@ -96,30 +96,48 @@ def tir_kv_cache_transpose_append_mla(pages, kv_data, position_map):
                                                     position_map.shape[0], num_pages, ps, d, _stream()))
 
 
+def _scaling_arg(rope_scaling):
+    """The reference's rope_scaling dictionary (position_embedding.py:258-299) as the C description, kept
+    alive by the caller for the duration of the call; None = the default frequencies."""
+    from .dlpack import RopeScaling
+    scaling = RopeScaling.from_dict(rope_scaling)
+    return scaling, ctypes.c_void_p(ctypes.addressof(scaling))
+
+
 def batch_prefill_ragged_kv(q, q_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_offset, output, lse,
-                            causal, rotary_mode, rope_scale, rope_theta, sm_scale):
+                            causal, rotary_mode, rope_scale, rope_theta, sm_scale, rope_scaling=None):
+    """rope_scaling: the frequency variant of the in-kernel RoPE (rotary_mode = 1), the reference's dictionary."""
     _f16(q, k, v, output)
     _i32(q_indptr, kv_indptr, q_rope_position, k_rope_pos_offset)
-    check(lib().tvmkv_batch_prefill_ragged_kv(
-        _p(q), _p(q_indptr), _p(k), _p(v), _p(kv_indptr), _p(q_rope_position), _p(k_rope_pos_offset), _p(output),
-        _p(lse), int(causal), int(rotary_mode), float(rope_scale), float(rope_theta), float(sm_scale),
-        q_indptr.shape[0] - 1, q.shape[0], q.shape[1], k.shape[1], q.shape[2], v.shape[2], _stream()))
+    args = (_p(q), _p(q_indptr), _p(k), _p(v), _p(kv_indptr), _p(q_rope_position), _p(k_rope_pos_offset), _p(output),
+            _p(lse), int(causal), int(rotary_mode), float(rope_scale), float(rope_theta), float(sm_scale),
+            q_indptr.shape[0] - 1, q.shape[0], q.shape[1], k.shape[1], q.shape[2], v.shape[2])
+    if rope_scaling:
+        keep, ptr = _scaling_arg(rope_scaling)
+        check(lib().tvmkv_batch_prefill_ragged_kv_scaled(*args, ptr, _stream()))
+    else:
+        check(lib().tvmkv_batch_prefill_ragged_kv(*args, _stream()))
 
 
 def batch_prefill_paged_kv(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset,
                            q_rope_position, output, lse, causal, rotary_mode, rope_scale, rope_theta, sm_scale,
-                           sliding_window_size=1024, merge_into=False):
+                           sliding_window_size=1024, merge_into=False, rope_scaling=None):
     """merge_into: output / lse hold an attention state of the same rows; merge into it instead of
-    overwriting (one launch for the paged kernel and merge_state_inplace)."""
+    overwriting (one launch for the paged kernel and merge_state_inplace).  rope_scaling: the frequency
+    variant of the in-kernel RoPE (rotary_mode = 1), the reference's dictionary."""
     _f16(q, pages, output)
     _i32(q_indptr, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position)
     num_pages, _, hkv, ps, d = pages.shape
-    fn = lib().tvmkv_batch_prefill_paged_kv_merge if merge_into else lib().tvmkv_batch_prefill_paged_kv
-    check(fn(
-        _p(q), _p(q_indptr), _p(pages), _p(page_indptr), _p(page_values), _p(length_info), _p(k_rope_pos_offset),
-        _p(q_rope_position), _p(output), _p(lse), int(causal), int(rotary_mode), float(rope_scale),
-        float(rope_theta), float(sm_scale), q_indptr.shape[0] - 1, q.shape[0], page_values.shape[0], num_pages,
-        q.shape[1], hkv, d, ps, int(length_info.dim() == 2), int(sliding_window_size), _stream()))
+    args = (_p(q), _p(q_indptr), _p(pages), _p(page_indptr), _p(page_values), _p(length_info), _p(k_rope_pos_offset),
+            _p(q_rope_position), _p(output), _p(lse), int(causal), int(rotary_mode), float(rope_scale),
+            float(rope_theta), float(sm_scale), q_indptr.shape[0] - 1, q.shape[0], page_values.shape[0], num_pages,
+            q.shape[1], hkv, d, ps, int(length_info.dim() == 2), int(sliding_window_size))
+    if rope_scaling:
+        keep, ptr = _scaling_arg(rope_scaling)
+        check(lib().tvmkv_batch_prefill_paged_kv_scaled(*args, int(bool(merge_into)), ptr, _stream()))
+    else:
+        fn = lib().tvmkv_batch_prefill_paged_kv_merge if merge_into else lib().tvmkv_batch_prefill_paged_kv
+        check(fn(*args, _stream()))
 
 
 def batch_prefill_cached_and_new_kv(q, q_indptr, k, v, pages, page_indptr, page_values, last_page_len, output, lse,
@@ -164,28 +182,37 @@ def fused_decode_step(qkv, pages, page_indptr, page_values, last_page_len, q_rop
 
 
 def batch_decode_paged_kv(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position,
-                          output, lse, rotary_mode, rope_scale, rope_theta, sm_scale, noalloc=False):
+                          output, lse, rotary_mode, rope_scale, rope_theta, sm_scale, noalloc=False, rope_scaling=None):
     """noalloc=True calls the entry point that takes its scratch memory from the library's built-in
-    per-device array instead of allocating (tvmkv_batch_decode_paged_kv_noalloc)."""
+    per-device array instead of allocating (tvmkv_batch_decode_paged_kv_noalloc).  rope_scaling: the
+    frequency variant of the in-kernel RoPE (rotary_mode = 1), the reference's dictionary."""
     _f16(q, pages, output)
     _i32(page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position)
     num_pages, _, hkv, ps, d = pages.shape
+    args = (_p(q), _p(pages), _p(page_indptr), _p(page_values), _p(length_info), _p(k_rope_pos_offset),
+            _p(q_rope_position), _p(output), _p(lse), int(rotary_mode), float(rope_scale), float(rope_theta),
+            float(sm_scale), q.shape[0], page_values.shape[0], num_pages, q.shape[1], hkv, d, ps,
+            int(length_info.dim() == 2))
+    if rope_scaling:
+        keep, ptr = _scaling_arg(rope_scaling)
+        check(lib().tvmkv_batch_decode_paged_kv_scaled(*args, ptr, _stream()))
+        return
     entry = lib().tvmkv_batch_decode_paged_kv_noalloc if noalloc else lib().tvmkv_batch_decode_paged_kv
-    check(entry(
-        _p(q), _p(pages), _p(page_indptr), _p(page_values), _p(length_info), _p(k_rope_pos_offset),
-        _p(q_rope_position), _p(output), _p(lse), int(rotary_mode), float(rope_scale), float(rope_theta),
-        float(sm_scale), q.shape[0], page_values.shape[0], num_pages, q.shape[1], hkv, d, ps,
-        int(length_info.dim() == 2), _stream()))
+    check(entry(*args, _stream()))
 
 
 def batch_tree_attn(q, q_indptr, k, v, kv_indptr, q_rope_position, mn_indptr, mask, output, lse, rotary_mode,
-                    rope_scale, rope_theta, sm_scale):
+                    rope_scale, rope_theta, sm_scale, rope_scaling=None):
     _f16(q, k, v, output)
     _i32(q_indptr, kv_indptr, q_rope_position, mn_indptr, mask)
-    check(lib().tvmkv_batch_tree_attn(
-        _p(q), _p(q_indptr), _p(k), _p(v), _p(kv_indptr), _p(q_rope_position), _p(mn_indptr), _p(mask), _p(output),
-        _p(lse), int(rotary_mode), float(rope_scale), float(rope_theta), float(sm_scale), q_indptr.shape[0] - 1,
-        q.shape[0], q.shape[1], k.shape[1], q.shape[2], _stream()))
+    args = (_p(q), _p(q_indptr), _p(k), _p(v), _p(kv_indptr), _p(q_rope_position), _p(mn_indptr), _p(mask), _p(output),
+            _p(lse), int(rotary_mode), float(rope_scale), float(rope_theta), float(sm_scale), q_indptr.shape[0] - 1,
+            q.shape[0], q.shape[1], k.shape[1], q.shape[2])
+    if rope_scaling:
+        keep, ptr = _scaling_arg(rope_scaling)
+        check(lib().tvmkv_batch_tree_attn_scaled(*args, ptr, _stream()))
+    else:
+        check(lib().tvmkv_batch_tree_attn(*args, _stream()))
 
 
 def tree_attn_paged_kv(q, q_indptr, pages, page_indptr, page_values, length_info, k_rope_pos_offset,
