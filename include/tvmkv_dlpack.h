@@ -124,6 +124,37 @@ int tvmkv_dl_batch_tree_attn(const DLTensor* q, const DLTensor* qo_indptr, const
                              int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
                              void* stream);
 
+/* The four launchers above that rotate inside the kernel (rotary_mode = 1), for a model whose RoPE has a
+ * frequency variant: the reference compiles rope_scaling into these kernels (_decode_kernels.py:138,150,
+ * _prefill_kernels.py:291-305, tree_attn.py:272-286), so a kernel function is made per model and passes
+ * the model's rope_scaling here (NULL = the default frequencies, the entry points above). */
+int tvmkv_dl_batch_prefill_ragged_kv_scaled(const DLTensor* q, const DLTensor* qo_indptr, const DLTensor* k,
+                                            const DLTensor* v, const DLTensor* kv_indptr,
+                                            const DLTensor* q_rope_position, const DLTensor* k_rope_pos_offset,
+                                            const DLTensor* out, const DLTensor* lse, int64_t causal,
+                                            int64_t rotary_mode, double rope_scale, double rope_theta,
+                                            double sm_scale, const tvmkv_rope_scaling* rope_scaling, void* stream);
+int tvmkv_dl_batch_prefill_paged_kv_scaled(const DLTensor* q, const DLTensor* qo_indptr, const DLTensor* pages,
+                                           const DLTensor* page_indptr, const DLTensor* page_indices,
+                                           const DLTensor* length_info, const DLTensor* k_rope_pos_offset,
+                                           const DLTensor* q_rope_position, const DLTensor* out,
+                                           const DLTensor* lse, int64_t causal, int64_t rotary_mode,
+                                           double rope_scale, double rope_theta, double sm_scale,
+                                           int64_t layer_sliding_window_size,
+                                           const tvmkv_rope_scaling* rope_scaling, void* stream);
+int tvmkv_dl_batch_decode_paged_kv_scaled(const DLTensor* q, const DLTensor* pages, const DLTensor* page_indptr,
+                                          const DLTensor* page_indices, const DLTensor* length_info,
+                                          const DLTensor* k_rope_pos_offset, const DLTensor* q_rope_position,
+                                          const DLTensor* out, const DLTensor* lse, int64_t rotary_mode,
+                                          double rope_scale, double rope_theta, double sm_scale,
+                                          const tvmkv_rope_scaling* rope_scaling, void* stream);
+int tvmkv_dl_batch_tree_attn_scaled(const DLTensor* q, const DLTensor* qo_indptr, const DLTensor* k,
+                                    const DLTensor* v, const DLTensor* kv_indptr,
+                                    const DLTensor* q_rope_position, const DLTensor* tree_attn_mn_indptr,
+                                    const DLTensor* tree_attn_mask, const DLTensor* out, const DLTensor* lse,
+                                    int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                                    const tvmkv_rope_scaling* rope_scaling, void* stream);
+
 /* Slot 22 MLA paged prefill (and decode), attn_backend.h:248-249. */
 int tvmkv_dl_batch_prefill_paged_kv_mla(const DLTensor* q, const DLTensor* qo_indptr,
                                         const DLTensor* pages, const DLTensor* page_indptr,

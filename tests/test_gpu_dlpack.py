@@ -300,3 +300,81 @@ def test_fused_rope_slot_with_frequency_variants(scaling, theta, d):
         assert_close(gq, eq, atol=2e-3, rtol=2e-3, what="rope q")
         assert_close(gk, ek, atol=2e-3, rtol=2e-3, what="rope k")
         assert np.mean(gq == eq) > 0.98, np.mean(gq == eq)
+
+
+@pytest.mark.parametrize("scaling,theta", [(LLAMA3, 5e5), (YARN, 1e4)])
+def test_attention_slots_with_a_frequency_variant_inside_the_kernel(scaling, theta):
+    """Slots 17, 16, 15 and 21 as a model with inline RoPE and a frequency variant gets them: the variant is a
+    property of the kernel function (the reference compiles it in), here an argument of the *_scaled entry
+    points.  The oracle's kernels rotate with the same variant."""
+    rng = np.random.default_rng(107)
+    hq, hkv, d = 8, 2, 128
+    rs = dl.RopeScaling.from_dict(scaling)
+    kv_lens = [1, 17, 300, 64]
+    b = len(kv_lens)
+    pages, indptr, values, last, _, _ = build_paged_kv(rng, kv_lens, 40, hkv, 16, d)
+    pages_dl = offset_f16(pages, pad=64)[0]
+    k_off = rng.integers(0, 3000, size=b).astype(np.int32)
+    with ok.inline_rope_scaling(scaling):
+        # slot 17
+        q = rng.standard_normal((b, hq, d)).astype(F16)
+        q_pos = (k_off + np.array(kv_lens) - 1).astype(np.int32)
+        eo, el = np.zeros((b, hq, d), F16), np.zeros((b, hq), np.float32)
+        ok.decode(q, pages, indptr, values, last, k_off, q_pos, eo, el, 1, 0.5, theta, d ** -0.5)
+        aux = Merged(page_indptr=indptr, page_indices=values, length_info=last, k_rope_pos_offset=k_off, q_rope_position=q_pos)
+        out, lse, get_out = outputs(b, hq, d)
+        dl.call("batch_decode_paged_kv_scaled", offset_f16(q)[0], pages_dl, aux["page_indptr"], aux["page_indices"],
+                aux["length_info"], aux["k_rope_pos_offset"], aux["q_rope_position"], out, dl.tensor(lse), 1, 0.5, theta,
+                d ** -0.5, rs)
+        assert_close(get_out(), eo, what="dl scaled decode out")
+        assert_close(host(lse), el, atol=2e-3, rtol=1e-4, what="dl scaled decode lse")
+        # slot 16, causal
+        q_lens = [1, 5, 40, 64]
+        n = sum(q_lens)
+        qo_indptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+        q = rng.standard_normal((n, hq, d)).astype(F16)
+        q_pos = np.concatenate([k_off[i] + kv_lens[i] - q_lens[i] + np.arange(q_lens[i]) for i in range(b)]).astype(np.int32)
+        eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+        ok.prefill_paged(q, qo_indptr, pages, indptr, values, last, k_off, q_pos, eo, el, 1, 1, 0.5, theta, d ** -0.5)
+        aux = Merged(q_rope_position=q_pos, qo_indptr=qo_indptr, page_indptr=indptr, page_indices=values, length_info=last,
+                     k_rope_pos_offset=k_off)
+        out, lse, get_out = outputs(n, hq, d)
+        dl.call("batch_prefill_paged_kv_scaled", offset_f16(q)[0], aux["qo_indptr"], pages_dl, aux["page_indptr"],
+                aux["page_indices"], aux["length_info"], aux["k_rope_pos_offset"], aux["q_rope_position"], out, dl.tensor(lse),
+                1, 1, 0.5, theta, d ** -0.5, 0, rs)
+        assert_close(get_out(), eo, what="dl scaled paged prefill out")
+        assert_close(host(lse), el, atol=2e-3, rtol=1e-4, what="dl scaled paged prefill lse")
+        # slot 15, causal
+        lens = [33, 1, 70]
+        n = sum(lens)
+        ind = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        q = rng.standard_normal((n, hq, d)).astype(F16)
+        k, v = (rng.standard_normal((n, hkv, d)).astype(F16) for _ in range(2))
+        off = rng.integers(0, 3000, size=len(lens)).astype(np.int32)
+        q_pos = np.concatenate([off[i] + np.arange(lens[i]) for i in range(len(lens))]).astype(np.int32)
+        eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+        ok.prefill_ragged(q, ind, k, v, ind, q_pos, off, eo, el, 1, 1, 0.5, theta, d ** -0.5)
+        aux = Merged(qo_indptr=ind, kv_indptr=ind, q_rope_position=q_pos, k_rope_pos_offset=off)
+        out, lse, get_out = outputs(n, hq, d)
+        dl.call("batch_prefill_ragged_kv_scaled", offset_f16(q)[0], aux["qo_indptr"], offset_f16(k)[0], offset_f16(v)[0],
+                aux["kv_indptr"], aux["q_rope_position"], aux["k_rope_pos_offset"], out, dl.tensor(lse), 1, 1, 0.5, theta,
+                d ** -0.5, rs)
+        assert_close(get_out(), eo, what="dl scaled ragged out")
+        assert_close(host(lse), el, atol=2e-3, rtol=1e-4, what="dl scaled ragged lse")
+        # slot 21
+        trees = [REFERENCE_TREES[0], random_forest(rng, 20)]
+        lens = [len(t) for t in trees]
+        n = sum(lens)
+        ind = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        q, k, v = (rng.standard_normal((n, h, d)).astype(F16) for h in (hq, hkv, hkv))
+        mask = np.concatenate([tree_order(t) for t in trees])
+        q_pos = rng.integers(0, 3000, size=n).astype(np.int32)
+        eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), np.float32)
+        ok.tree_attn_ragged(q, ind, k, v, ind, q_pos, ind, mask, eo, el, 1, 0.5, theta, d ** -0.5)
+        aux = Merged(qo_indptr=ind, kv_indptr=ind, q_rope_position=q_pos, mn_indptr=ind, mask=np.asarray(mask).reshape(-1))
+        out, lse, get_out = outputs(n, hq, d)
+        dl.call("batch_tree_attn_scaled", offset_f16(q)[0], aux["qo_indptr"], offset_f16(k)[0], offset_f16(v)[0],
+                aux["kv_indptr"], aux["q_rope_position"], aux["mn_indptr"], aux["mask"], out, dl.tensor(lse), 1, 0.5, theta,
+                d ** -0.5, rs)
+        assert_close(get_out(), eo, what="dl scaled tree out")
+        assert_close(host(lse), el, atol=2e-3, rtol=1e-4, what="dl scaled tree lse")

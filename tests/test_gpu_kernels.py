@@ -457,7 +457,7 @@ def test_paged_prefill_against_oracle(hq, hkv, d, causal, rows):
 
 
 @pytest.mark.parametrize("page_size", [32, 64, 128])
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(16, 4, 128), (8, 2, 64)])
 def test_paged_kernels_with_other_page_sizes(page_size, hq, hkv, d):
     """Pages of 32, 64 and 128 tokens through every kernel that reads the page pool with 16-token steps:
     plain and causal paged prefill, the sliding-window / inline-RoPE forms of prefill and decode, the
@@ -550,7 +550,7 @@ def test_paged_kernels_with_other_page_sizes(page_size, hq, hkv, d):
     assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"one-pass chunked prefill lse, page size {ps}")
 
 
-@pytest.mark.parametrize("hq,hkv,d,splits", [(32, 8, 128, 0), (32, 8, 128, 3), (8, 2, 64, 5), (8, 2, 64, 64), (8, 2, 256, 2)])
+@pytest.mark.parametrize("hq,hkv,d,splits", [(16, 4, 128, 0), (16, 4, 128, 3), (8, 2, 64, 5), (8, 2, 64, 64), (8, 2, 256, 2)])
 def test_prefill_split_over_the_keys(hq, hkv, d, splits):
     """Launches with few row tiles split every row tile's keys over several workgroups and merge the
     states: the derived split (few queries against long cached sequences) and forced ones (more shares
@@ -677,7 +677,7 @@ def test_layer_sliding_window_mask_known_answer_on_the_gpu():
     assert_close(host(go)[:, 0, 0], np.array([4, 5], F16), atol=1e-3, rtol=1e-3, what="sliding window known answer")
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (8, 2, 256)])
+@pytest.mark.parametrize("hq,hkv,d", [(16, 4, 128), (8, 2, 64), (8, 2, 256)])
 @pytest.mark.parametrize("rotary", [0, 1])
 @pytest.mark.parametrize("causal,window", [(0, 1024), (1, 0), (1, 5), (1, 40)])
 @pytest.mark.parametrize("long_q", [False, True])

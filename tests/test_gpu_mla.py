@@ -141,7 +141,9 @@ def test_mla_few_tokens_per_sequence_split_kv(causal):
                             ([900, 5, 300, 0, 420, 77], [3, 5, 0, 2, 1, 7])):                    # ragged, empty sequences
         if causal:
             kv_lens = [max(k, q) for k, q in zip(kv_lens, q_lens)]
-        go, gl, eo, el = _mla_both(rng, kv_lens, q_lens, 64, npages=8 + sum((n + 63) // 64 for n in kv_lens), causal=causal)
+        heads = 64 if len(kv_lens) == 1 else 128   # the long single chunk is most of the oracle's time
+        go, gl, eo, el = _mla_both(rng, kv_lens, q_lens, 64, npages=8 + sum((n + 63) // 64 for n in kv_lens), causal=causal,
+                                   heads=heads)
         assert_close(go, eo, what=f"mla few tokens out, q_lens {q_lens}")
         assert_close(gl, el, atol=2e-3, rtol=1e-4, what=f"mla few tokens lse, q_lens {q_lens}")
 

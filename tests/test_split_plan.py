@@ -58,7 +58,9 @@ def test_chunk_size_follows_the_work():
     assert tvm_amd.decode_split_plan(short, 80 * 256, 8)[0] == 128       # 256 short sequences: no split at all
     assert tvm_amd.decode_split_plan([0, 1 << 20], 1 << 20, 8)[0] == 128
     assert tvm_amd.decode_split_plan([0, 18432], 18432, 1)[0] == 32      # one kv head: 768 items
-    assert tvm_amd.decode_split_plan([0, 8192], 8192, 8)[0] == 64        # one sequence of 131072 tokens
+    assert tvm_amd.decode_split_plan([0, 8192], 8192, 8)[0] == 128       # one sequence of 131072 tokens: 64 states, not 128
+    assert tvm_amd.decode_split_plan([0, 4096, 8192], 8192, 8)[0] == 128  # two of 65536
+    assert tvm_amd.decode_split_plan([0, 2048, 4096, 6144, 8192], 8192, 8)[0] == 64   # four of 32768: 32 states each
 
 
 def test_options_round_trip_and_reject_unknown_names():

@@ -112,6 +112,10 @@ SIGNATURES = {
     "tvmkv_dl_batch_decode_paged_kv": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_vp],
     "tvmkv_dl_tree_attn_paged_kv": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_vp, c_vp, c_vp],
     "tvmkv_dl_batch_tree_attn": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_vp],
+    "tvmkv_dl_batch_prefill_ragged_kv_scaled": [c_vp] * 9 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_vp, c_vp],
+    "tvmkv_dl_batch_prefill_paged_kv_scaled": [c_vp] * 10 + [c_i64, c_i64, c_f64, c_f64, c_f64, c_i64, c_vp, c_vp],
+    "tvmkv_dl_batch_decode_paged_kv_scaled": [c_vp] * 9 + [c_i64, c_f64, c_f64, c_f64, c_vp, c_vp],
+    "tvmkv_dl_batch_tree_attn_scaled": [c_vp] * 10 + [c_i64, c_f64, c_f64, c_f64, c_vp, c_vp],
     "tvmkv_dl_batch_prefill_paged_kv_mla": [c_vp] * 8 + [c_i64, c_f64, c_vp],
     "tvmkv_dl_merge_state_inplace": [c_vp] * 5,
     "tvmkv_dl_copy_single_page": [c_vp, c_i64, c_i64, c_i64, c_vp],

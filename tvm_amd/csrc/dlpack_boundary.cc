@@ -197,11 +197,11 @@ int tvmkv_dl_transpose_append_mla(const DLTensor* pages_, const DLTensor* kv_, c
   KV_API_END();
 }
 
-int tvmkv_dl_batch_prefill_ragged_kv(const DLTensor* q_, const DLTensor* qo_indptr_, const DLTensor* k_,
+int tvmkv_dl_batch_prefill_ragged_kv_scaled(const DLTensor* q_, const DLTensor* qo_indptr_, const DLTensor* k_,
                                      const DLTensor* v_, const DLTensor* kv_indptr_, const DLTensor* q_rope_position_,
                                      const DLTensor* k_rope_pos_offset_, const DLTensor* out_, const DLTensor* lse_,
                                      int64_t causal, int64_t rotary_mode, double rope_scale, double rope_theta,
-                                     double sm_scale, void* stream) {
+                                     double sm_scale, const tvmkv_rope_scaling* rope_scaling, void* stream) {
   KV_API_BEGIN();
   Arg q = Take(q_, "q", kF16, {3}), qo_indptr = Take(qo_indptr_, "qo_indptr", kI32, {1});
   Arg k = Take(k_, "k", kF16, {3}), v = Take(v_, "v", kF16, {3}), kv_indptr = Take(kv_indptr_, "kv_indptr", kI32, {1});
@@ -219,20 +219,20 @@ int tvmkv_dl_batch_prefill_ragged_kv(const DLTensor* q_, const DLTensor* qo_indp
   Expect(q_pos.dim(0) >= rows, q_pos, "(at least the rows of q,)");
   Expect(out.dim(0) == rows && out.dim(1) == q.dim(1) && out.dim(2) == v.dim(2), out, "(rows of q, h_q, d_v)");
   Expect(lse.dim(0) == rows && lse.dim(1) == q.dim(1), lse, "(rows of q, h_q)");
-  Launch(device, [&] { return tvmkv_batch_prefill_ragged_kv(q.ptr(), qo_indptr.i32(), k.ptr(), v.ptr(), kv_indptr.i32(), q_pos.i32(),
+  Launch(device, [&] { return tvmkv_batch_prefill_ragged_kv_scaled(q.ptr(), qo_indptr.i32(), k.ptr(), v.ptr(), kv_indptr.i32(), q_pos.i32(),
                                        k_off.i32(), out.ptr(), lse.f32(), causal, rotary_mode, rope_scale, rope_theta,
                                        sm_scale, static_cast<int32_t>(batch), rows, static_cast<int32_t>(q.dim(1)),
                                        static_cast<int32_t>(k.dim(1)), static_cast<int32_t>(q.dim(2)),
-                                       static_cast<int32_t>(v.dim(2)), stream); });
+                                       static_cast<int32_t>(v.dim(2)), rope_scaling, stream); });
   KV_API_END();
 }
 
-int tvmkv_dl_batch_prefill_paged_kv(const DLTensor* q_, const DLTensor* qo_indptr_, const DLTensor* pages_,
+int tvmkv_dl_batch_prefill_paged_kv_scaled(const DLTensor* q_, const DLTensor* qo_indptr_, const DLTensor* pages_,
                                     const DLTensor* page_indptr_, const DLTensor* page_indices_,
                                     const DLTensor* length_info_, const DLTensor* k_rope_pos_offset_,
                                     const DLTensor* q_rope_position_, const DLTensor* out_, const DLTensor* lse_,
                                     int64_t causal, int64_t rotary_mode, double rope_scale, double rope_theta,
-                                    double sm_scale, int64_t layer_sliding_window_size, void* stream) {
+                                    double sm_scale, int64_t layer_sliding_window_size, const tvmkv_rope_scaling* rope_scaling, void* stream) {
   KV_API_BEGIN();
   Arg q = Take(q_, "q", kF16, {3}), qo_indptr = Take(qo_indptr_, "qo_indptr", kI32, {1});
   Arg pages = Take(pages_, "pages", kF16, {5}), page_indptr = Take(page_indptr_, "page_indptr", kI32, {1});
@@ -244,19 +244,19 @@ int tvmkv_dl_batch_prefill_paged_kv(const DLTensor* q_, const DLTensor* qo_indpt
   const int device = SameDevice({q, qo_indptr, pages, page_indptr, page_indices, length_info, k_off, q_pos, out, lse});
   const PagedShapes s = CheckPaged(q, pages, page_indptr, page_indices, length_info, k_off, q_pos, out, lse);
   Expect(qo_indptr.dim(0) == s.batch + 1, qo_indptr, "(batch + 1,)");
-  Launch(device, [&] { return tvmkv_batch_prefill_paged_kv(q.ptr(), qo_indptr.i32(), pages.ptr(), page_indptr.i32(), page_indices.i32(),
+  Launch(device, [&] { return tvmkv_batch_prefill_paged_kv_scaled(q.ptr(), qo_indptr.i32(), pages.ptr(), page_indptr.i32(), page_indices.i32(),
                                       length_info.i32(), k_off.i32(), q_pos.i32(), out.ptr(), lse.f32(), causal,
                                       rotary_mode, rope_scale, rope_theta, sm_scale, static_cast<int32_t>(s.batch), s.rows,
                                       s.nnz_pages, s.num_pages, s.h_q, s.h_kv, s.d, s.page_size, s.sliding,
-                                      static_cast<int32_t>(layer_sliding_window_size), stream); });
+                                      static_cast<int32_t>(layer_sliding_window_size), /*merge_into=*/0, rope_scaling, stream); });
   KV_API_END();
 }
 
-int tvmkv_dl_batch_decode_paged_kv(const DLTensor* q_, const DLTensor* pages_, const DLTensor* page_indptr_,
+int tvmkv_dl_batch_decode_paged_kv_scaled(const DLTensor* q_, const DLTensor* pages_, const DLTensor* page_indptr_,
                                    const DLTensor* page_indices_, const DLTensor* length_info_,
                                    const DLTensor* k_rope_pos_offset_, const DLTensor* q_rope_position_,
                                    const DLTensor* out_, const DLTensor* lse_, int64_t rotary_mode, double rope_scale,
-                                   double rope_theta, double sm_scale, void* stream) {
+                                   double rope_theta, double sm_scale, const tvmkv_rope_scaling* rope_scaling, void* stream) {
   KV_API_BEGIN();
   Arg q = Take(q_, "q", kF16, {3}), pages = Take(pages_, "pages", kF16, {5});
   Arg page_indptr = Take(page_indptr_, "page_indptr", kI32, {1});
@@ -268,10 +268,10 @@ int tvmkv_dl_batch_decode_paged_kv(const DLTensor* q_, const DLTensor* pages_, c
   const int device = SameDevice({q, pages, page_indptr, page_indices, length_info, k_off, q_pos, out, lse});
   const PagedShapes s = CheckPaged(q, pages, page_indptr, page_indices, length_info, k_off, q_pos, out, lse);
   Expect(s.rows == s.batch, q, "(batch, h_q, head_dim): one query per page-table entry");
-  Launch(device, [&] { return tvmkv_batch_decode_paged_kv(q.ptr(), pages.ptr(), page_indptr.i32(), page_indices.i32(), length_info.i32(),
+  Launch(device, [&] { return tvmkv_batch_decode_paged_kv_scaled(q.ptr(), pages.ptr(), page_indptr.i32(), page_indices.i32(), length_info.i32(),
                                      k_off.i32(), q_pos.i32(), out.ptr(), lse.f32(), rotary_mode, rope_scale, rope_theta,
                                      sm_scale, static_cast<int32_t>(s.batch), s.nnz_pages, s.num_pages, s.h_q, s.h_kv, s.d,
-                                     s.page_size, s.sliding, stream); });
+                                     s.page_size, s.sliding, rope_scaling, stream); });
   KV_API_END();
 }
 
@@ -304,11 +304,11 @@ int tvmkv_dl_tree_attn_paged_kv(const DLTensor* q_, const DLTensor* qo_indptr_, 
   KV_API_END();
 }
 
-int tvmkv_dl_batch_tree_attn(const DLTensor* q_, const DLTensor* qo_indptr_, const DLTensor* k_, const DLTensor* v_,
+int tvmkv_dl_batch_tree_attn_scaled(const DLTensor* q_, const DLTensor* qo_indptr_, const DLTensor* k_, const DLTensor* v_,
                              const DLTensor* kv_indptr_, const DLTensor* q_rope_position_,
                              const DLTensor* tree_attn_mn_indptr_, const DLTensor* tree_attn_mask_, const DLTensor* out_,
                              const DLTensor* lse_, int64_t rotary_mode, double rope_scale, double rope_theta,
-                             double sm_scale, void* stream) {
+                             double sm_scale, const tvmkv_rope_scaling* rope_scaling, void* stream) {
   KV_API_BEGIN();
   Arg q = Take(q_, "q", kF16, {3}), qo_indptr = Take(qo_indptr_, "qo_indptr", kI32, {1});
   Arg k = Take(k_, "k", kF16, {3}), v = Take(v_, "v", kF16, {3}), kv_indptr = Take(kv_indptr_, "kv_indptr", kI32, {1});
@@ -328,10 +328,10 @@ int tvmkv_dl_batch_tree_attn(const DLTensor* q_, const DLTensor* qo_indptr_, con
   Expect(q_pos.dim(0) >= rows, q_pos, "(at least the rows of q,)");
   Expect(out.dim(0) == rows && out.dim(1) == q.dim(1) && out.dim(2) == q.dim(2), out, "the shape of q");
   Expect(lse.dim(0) == rows && lse.dim(1) == q.dim(1), lse, "(rows of q, h_q)");
-  Launch(device, [&] { return tvmkv_batch_tree_attn(q.ptr(), qo_indptr.i32(), k.ptr(), v.ptr(), kv_indptr.i32(), q_pos.i32(), mn_indptr.i32(),
+  Launch(device, [&] { return tvmkv_batch_tree_attn_scaled(q.ptr(), qo_indptr.i32(), k.ptr(), v.ptr(), kv_indptr.i32(), q_pos.i32(), mn_indptr.i32(),
                                mask.i32(), out.ptr(), lse.f32(), rotary_mode, rope_scale, rope_theta, sm_scale,
                                static_cast<int32_t>(batch), rows, static_cast<int32_t>(q.dim(1)),
-                               static_cast<int32_t>(k.dim(1)), static_cast<int32_t>(q.dim(2)), stream); });
+                               static_cast<int32_t>(k.dim(1)), static_cast<int32_t>(q.dim(2)), rope_scaling, stream); });
   KV_API_END();
 }
 
@@ -440,6 +440,45 @@ int tvmkv_dl_compact_kv_copy(const DLTensor* pages_, const DLTensor* copy_length
                                static_cast<int32_t>(pos.dim(1)), pages.dim(0), static_cast<int32_t>(pages.dim(2)),
                                static_cast<int32_t>(pages.dim(3)), static_cast<int32_t>(pages.dim(4)), stream); });
   KV_API_END();
+}
+
+// The entry points without a frequency variant: the default frequencies theta^(-2i/d).
+int tvmkv_dl_batch_prefill_ragged_kv(const DLTensor* q, const DLTensor* qo_indptr, const DLTensor* k, const DLTensor* v,
+                                     const DLTensor* kv_indptr, const DLTensor* q_rope_position,
+                                     const DLTensor* k_rope_pos_offset, const DLTensor* out, const DLTensor* lse,
+                                     int64_t causal, int64_t rotary_mode, double rope_scale, double rope_theta,
+                                     double sm_scale, void* stream) {
+  return tvmkv_dl_batch_prefill_ragged_kv_scaled(q, qo_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_offset, out, lse,
+                                                 causal, rotary_mode, rope_scale, rope_theta, sm_scale, nullptr, stream);
+}
+
+int tvmkv_dl_batch_prefill_paged_kv(const DLTensor* q, const DLTensor* qo_indptr, const DLTensor* pages,
+                                    const DLTensor* page_indptr, const DLTensor* page_indices, const DLTensor* length_info,
+                                    const DLTensor* k_rope_pos_offset, const DLTensor* q_rope_position, const DLTensor* out,
+                                    const DLTensor* lse, int64_t causal, int64_t rotary_mode, double rope_scale,
+                                    double rope_theta, double sm_scale, int64_t layer_sliding_window_size, void* stream) {
+  return tvmkv_dl_batch_prefill_paged_kv_scaled(q, qo_indptr, pages, page_indptr, page_indices, length_info, k_rope_pos_offset,
+                                                q_rope_position, out, lse, causal, rotary_mode, rope_scale, rope_theta,
+                                                sm_scale, layer_sliding_window_size, nullptr, stream);
+}
+
+int tvmkv_dl_batch_decode_paged_kv(const DLTensor* q, const DLTensor* pages, const DLTensor* page_indptr,
+                                   const DLTensor* page_indices, const DLTensor* length_info,
+                                   const DLTensor* k_rope_pos_offset, const DLTensor* q_rope_position, const DLTensor* out,
+                                   const DLTensor* lse, int64_t rotary_mode, double rope_scale, double rope_theta,
+                                   double sm_scale, void* stream) {
+  return tvmkv_dl_batch_decode_paged_kv_scaled(q, pages, page_indptr, page_indices, length_info, k_rope_pos_offset,
+                                               q_rope_position, out, lse, rotary_mode, rope_scale, rope_theta, sm_scale,
+                                               nullptr, stream);
+}
+
+int tvmkv_dl_batch_tree_attn(const DLTensor* q, const DLTensor* qo_indptr, const DLTensor* k, const DLTensor* v,
+                             const DLTensor* kv_indptr, const DLTensor* q_rope_position,
+                             const DLTensor* tree_attn_mn_indptr, const DLTensor* tree_attn_mask, const DLTensor* out,
+                             const DLTensor* lse, int64_t rotary_mode, double rope_scale, double rope_theta,
+                             double sm_scale, void* stream) {
+  return tvmkv_dl_batch_tree_attn_scaled(q, qo_indptr, k, v, kv_indptr, q_rope_position, tree_attn_mn_indptr, tree_attn_mask,
+                                         out, lse, rotary_mode, rope_scale, rope_theta, sm_scale, nullptr, stream);
 }
 
 }  // extern "C"

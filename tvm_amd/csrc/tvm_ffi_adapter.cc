@@ -32,11 +32,9 @@ inline const DLTensor* T(const Tensor& t) { return t.operator->(); }
 inline void* StreamOf(const Tensor& t) { return TVMFFIEnvGetStream(t->device.device_type, t->device.device_id); }
 inline void Check(int rc) { TVM_FFI_ICHECK_EQ(rc, 0) << "tvmkv: " << tvmkv_last_error(); }
 
-// Slot 24 for a model: RoPE scale / theta and the frequency variant are compile-time constants of the
-// reference's kernel (position_embedding.py:444-667), so the kernel function is made per model.
-Function MakeFusedRope(double rope_scale, double rope_theta, int64_t rope_type, double factor, double low_freq_factor,
-                       double high_freq_factor, double beta_fast, double beta_slow, int64_t max_position_embeddings,
-                       int64_t original_max_position_embeddings, int64_t rotary_dim) {
+tvmkv_rope_scaling Scaling(int64_t rope_type, double factor, double low_freq_factor, double high_freq_factor, double beta_fast,
+                           double beta_slow, int64_t max_position_embeddings, int64_t original_max_position_embeddings,
+                           int64_t rotary_dim) {
   tvmkv_rope_scaling scaling{};
   scaling.rope_type = static_cast<int32_t>(rope_type);
   scaling.rotary_dim = static_cast<int32_t>(rotary_dim);  // 0 = the whole head
@@ -47,6 +45,16 @@ Function MakeFusedRope(double rope_scale, double rope_theta, int64_t rope_type, 
   scaling.beta_slow = beta_slow;
   scaling.max_position_embeddings = max_position_embeddings;
   scaling.original_max_position_embeddings = original_max_position_embeddings;
+  return scaling;
+}
+
+// Slot 24 for a model: RoPE scale / theta and the frequency variant are compile-time constants of the
+// reference's kernel (position_embedding.py:444-667), so the kernel function is made per model.
+Function MakeFusedRope(double rope_scale, double rope_theta, int64_t rope_type, double factor, double low_freq_factor,
+                       double high_freq_factor, double beta_fast, double beta_slow, int64_t max_position_embeddings,
+                       int64_t original_max_position_embeddings, int64_t rotary_dim) {
+  const tvmkv_rope_scaling scaling = Scaling(rope_type, factor, low_freq_factor, high_freq_factor, beta_fast, beta_slow,
+                                             max_position_embeddings, original_max_position_embeddings, rotary_dim);
   return Function::FromPacked([=](tvm::ffi::PackedArgs args, tvm::ffi::Any* rv) {
     // (qkv, q_rope_position_map, q, k, v, apply_rope) or (..., v, rope_ext_factors): paged_kv_cache.cc:1360-1366
     TVM_FFI_ICHECK_EQ(args.size(), 6) << "tvmkv fused_rope takes 6 arguments";
@@ -81,6 +89,56 @@ Function MakePagedPrefillSlidingWindow(int64_t layer_sliding_window_size) {
     PagedPrefill(layer_sliding_window_size, q, qo_indptr, pages, page_indptr, page_indices, length_info, k_rope_pos_offset,
                  q_rope_position, out, lse, causal, rotary_mode, rope_scale, rope_theta, sm_scale);
   });
+}
+
+// Slots 15, 16 / 18, 17 / 19 and 21 for a model whose cache rotates inside the attention kernels (rope_mode
+// inline) and whose RoPE has a frequency variant: the reference compiles rope_scaling into those kernels too
+// (_decode_kernels.py:138,150; _prefill_kernels.py:291-305; tree_attn.py:272-286).  slot: 15, 16, 17 or 21;
+// layer_sliding_window_size as for slot 18 (0 otherwise).
+Function MakeAttentionWithRopeScaling(int64_t slot, int64_t layer_sliding_window_size, int64_t rope_type, double factor,
+                                      double low_freq_factor, double high_freq_factor, double beta_fast, double beta_slow,
+                                      int64_t max_position_embeddings, int64_t original_max_position_embeddings) {
+  const tvmkv_rope_scaling scaling = Scaling(rope_type, factor, low_freq_factor, high_freq_factor, beta_fast, beta_slow,
+                                             max_position_embeddings, original_max_position_embeddings, 0);
+  switch (slot) {
+    case 15:
+      return Function::FromTyped([=](Tensor q, Tensor qo_indptr, Tensor k, Tensor v, Tensor kv_indptr, Tensor q_rope_position,
+                                     Tensor k_rope_pos_offset, Tensor out, Tensor lse, int64_t causal, int64_t rotary_mode,
+                                     double rope_scale, double rope_theta, double sm_scale) {
+        Check(tvmkv_dl_batch_prefill_ragged_kv_scaled(T(q), T(qo_indptr), T(k), T(v), T(kv_indptr), T(q_rope_position),
+                                                      T(k_rope_pos_offset), T(out), T(lse), causal, rotary_mode, rope_scale,
+                                                      rope_theta, sm_scale, &scaling, StreamOf(q)));
+      });
+    case 16:
+      return Function::FromTyped([=](Tensor q, Tensor qo_indptr, Tensor pages, Tensor page_indptr, Tensor page_indices,
+                                     Tensor length_info, Tensor k_rope_pos_offset, Tensor q_rope_position, Tensor out,
+                                     Tensor lse, int64_t causal, int64_t rotary_mode, double rope_scale, double rope_theta,
+                                     double sm_scale) {
+        Check(tvmkv_dl_batch_prefill_paged_kv_scaled(T(q), T(qo_indptr), T(pages), T(page_indptr), T(page_indices),
+                                                     T(length_info), T(k_rope_pos_offset), T(q_rope_position), T(out), T(lse),
+                                                     causal, rotary_mode, rope_scale, rope_theta, sm_scale,
+                                                     layer_sliding_window_size, &scaling, StreamOf(q)));
+      });
+    case 17:
+      return Function::FromTyped([=](Tensor q, Tensor pages, Tensor page_indptr, Tensor page_indices, Tensor length_info,
+                                     Tensor k_rope_pos_offset, Tensor q_rope_position, Tensor out, Tensor lse,
+                                     int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale) {
+        Check(tvmkv_dl_batch_decode_paged_kv_scaled(T(q), T(pages), T(page_indptr), T(page_indices), T(length_info),
+                                                    T(k_rope_pos_offset), T(q_rope_position), T(out), T(lse), rotary_mode,
+                                                    rope_scale, rope_theta, sm_scale, &scaling, StreamOf(q)));
+      });
+    case 21:
+      return Function::FromTyped([=](Tensor q, Tensor qo_indptr, Tensor k, Tensor v, Tensor kv_indptr, Tensor q_rope_position,
+                                     Tensor tree_attn_mn_indptr, Tensor tree_attn_mask, Tensor out, Tensor lse,
+                                     int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale) {
+        Check(tvmkv_dl_batch_tree_attn_scaled(T(q), T(qo_indptr), T(k), T(v), T(kv_indptr), T(q_rope_position),
+                                              T(tree_attn_mn_indptr), T(tree_attn_mask), T(out), T(lse), rotary_mode,
+                                              rope_scale, rope_theta, sm_scale, &scaling, StreamOf(q)));
+      });
+    default:
+      TVM_FFI_THROW(ValueError) << "tvmkv.make_attention_with_rope_scaling: slot must be 15, 16, 17 or 21";
+  }
+  return Function();
 }
 
 }  // namespace
@@ -159,6 +217,8 @@ TVM_FFI_STATIC_INIT_BLOCK() {
            })
       // slot 24 f_split_rotary: tvmkv.make_fused_rope(scale, theta, rope_type, ...) -> kernel
       .def("tvmkv.make_fused_rope", MakeFusedRope)
+      // slots 15 / 16 / 17 / 21 of a model with inline RoPE and a frequency variant -> kernel
+      .def("tvmkv.make_attention_with_rope_scaling", MakeAttentionWithRopeScaling)
       // slot 25 f_copy_single_page (MHA and MLA layers: the rank of `pages` tells)
       .def("tvmkv.copy_single_page",
            [](Tensor pages, int64_t src_page_id, int64_t tgt_page_id, int64_t copy_length) {
