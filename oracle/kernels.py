@@ -3,7 +3,8 @@
 TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()`` and the
 ``cpu_baseline`` leg of ``bench.py``; the shipped package never imports it.
 
-Every wrapper takes numpy arrays (fp16 as ``np.float16``, indices as ``np.int32``) in the
+Every wrapper takes numpy arrays (K/V/q storage as ``np.float16`` or, for the MHA kernels, ``np.float32``:
+the dtype of the first array picks the build of the C file; indices as ``np.int32``) in the
 argument order of the reference kernel it restates and writes its outputs in place, like
 the destination-passing kernels of the reference.
 """
@@ -15,18 +16,29 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liborc_kernels.so")
+_LIB_PATH_F32 = os.path.join(_HERE, "liborc_kernels_f32.so")   # the same file compiled for float32 storage
 _lib = None
+_lib_f32 = None
 
 
 def build(force=False):
-    """Compile the C oracle with the committed Makefile."""
-    if force and os.path.exists(_LIB_PATH):
-        os.remove(_LIB_PATH)
-    subprocess.check_call(["make", "-C", _HERE, "liborc_kernels.so"], stdout=subprocess.DEVNULL)
+    """Compile the C oracle with the committed Makefile (both storage types)."""
+    for path in (_LIB_PATH, _LIB_PATH_F32):
+        if force and os.path.exists(path):
+            os.remove(path)
+    subprocess.check_call(["make", "-C", _HERE, "all"], stdout=subprocess.DEVNULL)
 
 
-def lib():
-    global _lib
+def lib(like=None):
+    """The oracle library; `like`: an array whose dtype selects the storage type (float32 or, by default, float16)."""
+    global _lib, _lib_f32
+    if like is not None and like.dtype == np.float32:
+        if _lib_f32 is None:
+            if not os.path.exists(_LIB_PATH_F32):
+                build()
+            _lib_f32 = ctypes.CDLL(_LIB_PATH_F32)
+        return _lib_f32
+    assert like is None or like.dtype == np.float16, like.dtype
     if _lib is None:
         if not os.path.exists(_LIB_PATH):
             build()
@@ -52,7 +64,7 @@ def fused_rope(qkv, position_map, q, k, v, apply_rope, *, theta=1e4, scale=1.0, 
     hq, hkv = q.shape[1], k.shape[1]
     assert fused == hq + 2 * hkv
     pm = _i32(position_map)
-    lib().orc_fused_rope(_p(qkv), _p(pm), _p(q), _p(k), _p(v), _c_i64(n), _c_int(hq), _c_int(hkv),
+    lib(qkv).orc_fused_rope(_p(qkv), _p(pm), _p(q), _p(k), _p(v), _c_i64(n), _c_int(hq), _c_int(hkv),
                          _c_int(d), _c_int(rotary_dim or d), _c_i64(int(apply_rope)), _c_f(theta),
                          _c_f(scale))
 
@@ -111,7 +123,7 @@ def fused_rope_scaled(qkv, position_map, q, k, v, apply_rope, rope_scaling, *, t
     pm = _i32(position_map)
     sc = RopeScaling.from_dict(rope_scaling)
     ext = None if ext_factors is None else np.ascontiguousarray(ext_factors, dtype=np.float32)
-    lib().orc_fused_rope_scaled(_p(qkv), _p(pm), _p(q), _p(k), _p(v), _c_i64(n), _c_int(hq), _c_int(hkv), _c_int(d),
+    lib(qkv).orc_fused_rope_scaled(_p(qkv), _p(pm), _p(q), _p(k), _p(v), _c_i64(n), _c_int(hq), _c_int(hkv), _c_int(d),
                                 _c_i64(int(apply_rope)), _c_f(theta), _c_f(scale), ctypes.byref(sc),
                                 None if ext is None else _p(ext))
 
@@ -120,7 +132,7 @@ def transpose_append(pages, k_data, v_data, position_map):
     _, two, hkv, ps, d = pages.shape
     assert two == 2
     pm = _i32(position_map)
-    lib().orc_transpose_append(_p(pages), _p(k_data), _p(v_data), _p(pm), _c_i64(len(pm)),
+    lib(pages).orc_transpose_append(_p(pages), _p(k_data), _p(v_data), _p(pm), _c_i64(len(pm)),
                                _c_int(hkv), _c_int(ps), _c_int(d))
 
 
@@ -134,7 +146,7 @@ def transpose_append_mla(pages, kv_data, position_map):
 def debug_get_kv(pages, position_map, k_data, v_data, layer_id):
     _, _, hkv, ps, d = pages.shape
     pm = _i32(position_map)
-    lib().orc_debug_get_kv(_p(pages), _p(pm), _p(k_data), _p(v_data), _c_i64(layer_id),
+    lib(pages).orc_debug_get_kv(_p(pages), _p(pm), _p(k_data), _p(v_data), _c_i64(layer_id),
                            _c_i64(len(pm)), _c_int(hkv), _c_int(ps), _c_int(d))
 
 
@@ -147,7 +159,7 @@ def debug_get_kv_mla(pages, position_map, kv_data, layer_id):
 
 def copy_single_page(pages, src_page_id, tgt_page_id, copy_length):
     _, _, hkv, ps, d = pages.shape
-    lib().orc_copy_single_page(_p(pages), _c_i64(src_page_id), _c_i64(tgt_page_id),
+    lib(pages).orc_copy_single_page(_p(pages), _c_i64(src_page_id), _c_i64(tgt_page_id),
                                _c_i64(copy_length), _c_int(hkv), _c_int(ps), _c_int(d))
 
 
@@ -161,7 +173,7 @@ def compact_kv_copy(pages, copy_length_indptr, copy_src_dst_pos, batch_size):
     _, _, hkv, ps, d = pages.shape
     ip = _i32(copy_length_indptr)
     sd = _i32(copy_src_dst_pos)
-    lib().orc_compact_kv_copy(_p(pages), _p(ip), _p(sd), _c_int(batch_size), _c_int(sd.shape[1]),
+    lib(pages).orc_compact_kv_copy(_p(pages), _p(ip), _p(sd), _c_int(batch_size), _c_int(sd.shape[1]),
                               _c_int(hkv), _c_int(ps), _c_int(d))
 
 
@@ -171,7 +183,7 @@ def decode(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q
     _, _, hkv, ps, _ = pages.shape
     li = _i32(length_info)
     args = [_i32(page_indptr), _i32(page_values), li, _i32(k_rope_pos_offset), _i32(q_rope_position)]
-    lib().orc_decode(_p(q), _p(pages), *[_p(a) for a in args], _p(output), _p(lse), _c_int(b),
+    lib(q).orc_decode(_p(q), _p(pages), *[_p(a) for a in args], _p(output), _p(lse), _c_int(b),
                      _c_int(hq), _c_int(hkv), _c_int(d), _c_int(ps), _c_int(int(li.ndim == 2)),
                      _c_int(rotary_mode), _c_f(rope_scale), _c_f(rope_theta), _c_f(sm_scale))
 
@@ -182,14 +194,14 @@ def decode_range(q, pages, page_indptr, page_values, length_info, k_rope_pos_off
     _, _, hkv, ps, _ = pages.shape
     args = [_i32(page_indptr), _i32(page_values), _i32(length_info), _i32(k_rope_pos_offset),
             _i32(q_rope_position)]
-    lib().orc_decode_range(_p(q), _p(pages), *[_p(a) for a in args], _p(output), _p(lse),
+    lib(q).orc_decode_range(_p(q), _p(pages), *[_p(a) for a in args], _p(output), _p(lse),
                            _c_int(b_begin), _c_int(b_end), _c_int(b), _c_int(hq), _c_int(hkv),
                            _c_int(d), _c_int(ps), _c_f(sm_scale))
 
 
 def merge_state_inplace(v, s, v_other, s_other):
     n, h, d = v.shape
-    lib().orc_merge_state_inplace(_p(v), _p(s), _p(v_other), _p(s_other), _c_i64(n), _c_int(h),
+    lib(v).orc_merge_state_inplace(_p(v), _p(s), _p(v_other), _p(s_other), _c_i64(n), _c_int(h),
                                   _c_int(d))
 
 
@@ -201,7 +213,7 @@ def prefill_paged(q, q_indptr, pages, page_indptr, page_values, length_info, k_r
     qi = _i32(q_indptr)
     li = _i32(length_info)
     args = [_i32(page_indptr), _i32(page_values), li, _i32(k_rope_pos_offset), _i32(q_rope_position)]
-    lib().orc_prefill_paged(_p(q), _p(qi), _p(pages), *[_p(a) for a in args], _p(output), _p(lse),
+    lib(q).orc_prefill_paged(_p(q), _p(qi), _p(pages), *[_p(a) for a in args], _p(output), _p(lse),
                             _c_int(len(qi) - 1), _c_int(hq), _c_int(hkv), _c_int(d), _c_int(ps),
                             _c_int(int(li.ndim == 2)), _c_int(sliding_window_size),
                             _c_int(int(causal)), _c_int(rotary_mode), _c_f(rope_scale),
@@ -214,7 +226,7 @@ def prefill_ragged(q, q_indptr, k, v, kv_indptr, q_rope_position, k_rope_pos_off
     _, hkv, dv = v.shape
     qi, ki = _i32(q_indptr), _i32(kv_indptr)
     qp, ko = _i32(q_rope_position), _i32(k_rope_pos_offset)
-    lib().orc_prefill_ragged(_p(q), _p(qi), _p(k), _p(v), _p(ki), _p(qp), _p(ko), _p(output),
+    lib(q).orc_prefill_ragged(_p(q), _p(qi), _p(k), _p(v), _p(ki), _p(qp), _p(ko), _p(output),
                              _p(lse), _c_int(len(qi) - 1), _c_int(hq), _c_int(hkv), _c_int(dqk),
                              _c_int(dv), _c_int(int(causal)), _c_int(rotary_mode),
                              _c_f(rope_scale), _c_f(rope_theta), _c_f(sm_scale))
@@ -227,7 +239,7 @@ def tree_attn_ragged(q, q_indptr, k, v, kv_indptr, q_rope_position, mn_indptr, m
     _, hkv, _ = v.shape
     qi, ki, qp = _i32(q_indptr), _i32(kv_indptr), _i32(q_rope_position)
     mi, mk = _i32(mn_indptr), _i32(mask)
-    lib().orc_tree_attn_ragged(_p(q), _p(qi), _p(k), _p(v), _p(ki), _p(qp), _p(mi), _p(mk), _p(output),
+    lib(q).orc_tree_attn_ragged(_p(q), _p(qi), _p(k), _p(v), _p(ki), _p(qp), _p(mi), _p(mk), _p(output),
                                _p(lse), _c_int(len(qi) - 1), _c_int(hq), _c_int(hkv), _c_int(d),
                                _c_int(rotary_mode), _c_f(rope_scale), _c_f(rope_theta), _c_f(sm_scale))
 
@@ -242,7 +254,7 @@ def tree_attn_paged(q, q_indptr, pages, page_indptr, page_values, length_info, k
     li = _i32(length_info)
     args = [_i32(page_indptr), _i32(page_values), li, _i32(k_rope_pos_offset), _i32(q_rope_position)]
     ti, to = _i32(tree_order_indptr), _i32(tree_order)
-    lib().orc_tree_attn_paged(_p(q), _p(qi), _p(pages), *[_p(a) for a in args], _p(output), _p(lse),
+    lib(q).orc_tree_attn_paged(_p(q), _p(qi), _p(pages), *[_p(a) for a in args], _p(output), _p(lse),
                               _c_int(len(qi) - 1), _c_int(hq), _c_int(hkv), _c_int(d), _c_int(ps),
                               _c_int(int(li.ndim == 2)), _c_int(rotary_mode), _c_f(rope_scale),
                               _c_f(rope_theta), _c_f(sm_scale), _p(ti), _p(to))

@@ -55,10 +55,23 @@
 #include <stdlib.h>
 #include <string.h>
 
+/* The reference builds every kernel for a storage dtype (its tests run "float16" and "float32",
+ * tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_cpu.py:269-276); arithmetic is float32
+ * either way and results are cast to the storage type where the TIR kernels cast.  This file is compiled
+ * twice: as it is for fp16 storage (liborc_kernels.so), and with -DORC_F32 for float32 storage
+ * (liborc_kernels_f32.so), where `f16` names a float and the conversions are the identity. */
+#ifdef ORC_F32
+typedef float f16;
+static inline float h2f(f16 h) { return h; }
+static inline f16 f2h(float f) { return f; }
+static inline f16 negated(f16 x) { return -x; }
+#else
 typedef uint16_t f16;
 
 static inline float h2f(f16 h) { return _cvtsh_ss(h); }
 static inline f16 f2h(float f) { return _cvtss_sh(f, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC); }
+static inline f16 negated(f16 x) { return (f16)(x ^ 0x8000u); }
+#endif
 
 #define LOG2E_F ((float)1.4426950408889634) /* math.log2(math.exp(1)) */
 
@@ -117,7 +130,7 @@ static inline int check_tree_order(const int32_t* tree_order_indptr, const int32
 static inline f16 rope_elem(const f16* x, int d, int rotary_dim, float pos_times_scale, float theta) {
   float freq = pos_times_scale / powf(theta, (float)((d * 2) % rotary_dim) / (float)rotary_dim);
   float c = cosf(freq) * h2f(x[d]);
-  f16 other = d < rotary_dim / 2 ? (f16)(x[d + rotary_dim / 2] ^ 0x8000u) : x[d - rotary_dim / 2];
+  f16 other = d < rotary_dim / 2 ? negated(x[d + rotary_dim / 2]) : x[d - rotary_dim / 2];
   float s = sinf(freq) * h2f(other);
   return f2h(c + s);
 }
@@ -241,7 +254,7 @@ static inline f16 rope_elem_inline(const f16* x, int d, int D, float pos_times_s
   float magnitude;
   float freq = orc_rope_angle(g_inline_scaling, pos_times_scale, d, D, theta, NULL, &magnitude);
   float c = cosf(freq) * magnitude * h2f(x[d]);
-  f16 other = d < D / 2 ? (f16)(x[d + D / 2] ^ 0x8000u) : x[d - D / 2];
+  f16 other = d < D / 2 ? negated(x[d + D / 2]) : x[d - D / 2];
   float sn = sinf(freq) * magnitude * h2f(other);
   return f2h(c + sn);
 }
@@ -272,8 +285,8 @@ void orc_fused_rope_scaled(const f16* qkv, const int32_t* position_map, f16* q, 
         float magnitude;
         float freq = orc_rope_angle(sc, (float)position_map[s] * scale, d, R, theta, ext, &magnitude);
         float c = (cosf(freq) * magnitude) * h2f(x[d]);
-        f16 other = d < R / 2 ? (f16)(x[d + R / 2] ^ 0x8000u) : x[d - R / 2];
-        if (sc != NULL && sc->rope_type == 4) other = d % 2 == 0 ? (f16)(x[d + 1] ^ 0x8000u) : x[d - 1]; /* :509-514 */
+        f16 other = d < R / 2 ? negated(x[d + R / 2]) : x[d - R / 2];
+        if (sc != NULL && sc->rope_type == 4) other = d % 2 == 0 ? negated(x[d + 1]) : x[d - 1]; /* :509-514 */
         float sn = (sinf(freq) * magnitude) * h2f(other);
         dst[d] = f2h(c + sn);
       }

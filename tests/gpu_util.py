@@ -28,13 +28,18 @@ class GpuCache:
     """The library's cache behind the interface of oracle.paged_kv_cache.OraclePagedKVCache."""
 
     def __init__(self, cache_config, num_layers, hq, hkv, dqk, dv, attn_kinds=None, rope_mode=1, rope_scale=1.0,
-                 rope_theta=1e4, rope_scaling=None, rope_ext_factors=None):
+                 rope_theta=1e4, rope_scaling=None, rope_ext_factors=None, dtype=np.float16):
         attn_kinds = list(attn_kinds) if attn_kinds is not None else [0] * num_layers
         ext = None if rope_ext_factors is None else dev(np.asarray(rope_ext_factors, dtype=np.float32))
         self.cache = gf("vm.builtin.paged_attention_kv_cache_create")(
             list(cache_config), [0, num_layers], hq, hkv, dqk, dv, attn_kinds, False, rope_mode, rope_scale,
-            rope_theta, ext, torch.empty((), dtype=torch.float16, device=DEV), rope_scaling=rope_scaling)
+            rope_theta, ext, torch.empty((), dtype=self._torch(dtype), device=DEV), rope_scaling=rope_scaling)
         self.num_layers, self.hq, self.hkv, self.dqk, self.dv = num_layers, hq, hkv, dqk, dv
+        self.dtype = self._torch(dtype)
+
+    @staticmethod
+    def _torch(dtype):
+        return torch.float32 if np.dtype(dtype) == np.float32 else torch.float16
 
     def clear(self):
         gf("vm.builtin.kv_state_clear")(self.cache)
@@ -67,25 +72,25 @@ class GpuCache:
         return gf("vm.builtin.attention_kv_cache_empty")(self.cache)
 
     def attention_with_fused_qkv(self, layer, sm_scale, qkv, out):
-        o = torch.zeros(out.shape, dtype=torch.float16, device=DEV)
+        o = torch.zeros(out.shape, dtype=self.dtype, device=DEV)
         gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")(self.cache, layer, sm_scale, dev(qkv), o)
         out[...] = host(o)
 
     def attention_with_shared_kv(self, source_layer, sm_scale, q, current_k, current_v, out):
-        o = torch.zeros(out.shape, dtype=torch.float16, device=DEV)
+        o = torch.zeros(out.shape, dtype=self.dtype, device=DEV)
         gf("vm.builtin.attention_kv_cache_attention_with_shared_kv")(self.cache, source_layer, sm_scale, dev(q),
                                                                      dev(current_k), dev(current_v), o)
         out[...] = host(o)
 
     def self_attention(self, layer, sm_scale, q, k, v, out, lse):
-        o = torch.zeros(out.shape, dtype=torch.float16, device=DEV)
+        o = torch.zeros(out.shape, dtype=self.dtype, device=DEV)
         s = torch.zeros(lse.shape, dtype=torch.float32, device=DEV)
         gf("vm.builtin.attention_kv_cache_self_attention")(self.cache, layer, sm_scale, dev(q), dev(k), dev(v), o, s)
         out[...] = host(o)
         lse[...] = host(s)
 
     def cross_attention(self, layer, sm_scale, q, out, lse):
-        o = torch.zeros(out.shape, dtype=torch.float16, device=DEV)
+        o = torch.zeros(out.shape, dtype=self.dtype, device=DEV)
         s = torch.zeros(lse.shape, dtype=torch.float32, device=DEV)
         gf("vm.builtin.attention_kv_cache_cross_attention")(self.cache, layer, sm_scale, dev(q), o, s)
         out[...] = host(o)
@@ -102,13 +107,13 @@ class GpuCache:
         return o_self, lse_self
 
     def debug_get_kv(self, sid, start, end, k, v):
-        kd = torch.zeros(k.shape, dtype=torch.float16, device=DEV)
-        vd = torch.zeros(v.shape, dtype=torch.float16, device=DEV)
+        kd = torch.zeros(k.shape, dtype=self.dtype, device=DEV)
+        vd = torch.zeros(v.shape, dtype=self.dtype, device=DEV)
         gf("vm.builtin.attention_kv_cache_debug_get_kv")(self.cache, sid, start, end, kd, vd)
         k[...] = host(kd)
         v[...] = host(vd)
 
     def debug_get_kv_mla(self, sid, start, end, kv):
-        kd = torch.zeros(kv.shape, dtype=torch.float16, device=DEV)
+        kd = torch.zeros(kv.shape, dtype=self.dtype, device=DEV)
         gf("vm.builtin.attention_kv_cache_debug_get_kv_mla")(self.cache, sid, start, end, kd)
         kv[...] = host(kd)

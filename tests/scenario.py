@@ -20,8 +20,9 @@ ROPE_NONE, ROPE_NORMAL, ROPE_INLINE = 0, 1, 2
 
 class Scenario:
     def __init__(self, cache, num_layers, hq, hkv, d, rope_mode=ROPE_NORMAL, rope_scale=1.0,
-                 rope_theta=1e4, seed=0, tol=2e-3, normal=False, on_step=None):
+                 rope_theta=1e4, seed=0, tol=2e-3, normal=False, on_step=None, dtype=np.float16):
         self.cache = cache
+        self.dtype = dtype  # storage type of the cache under test (float16 or float32)
         self.num_layers, self.hq, self.hkv, self.d = num_layers, hq, hkv, d
         self.rope_mode, self.rope_scale, self.rope_theta = rope_mode, rope_scale, rope_theta
         self.rng = np.random.default_rng(seed)
@@ -35,8 +36,8 @@ class Scenario:
 
     def _rand(self, *shape):
         if self.normal:
-            return self.rng.standard_normal(shape).astype(np.float16)
-        return self.rng.random(shape).astype(np.float16)  # the reference test draws uniform [0,1)
+            return self.rng.standard_normal(shape).astype(self.dtype)
+        return self.rng.random(shape).astype(self.dtype)  # the reference test draws uniform [0,1)
 
     def verify_cached_kv(self, seq_ids):
         for sid in seq_ids:
@@ -44,7 +45,7 @@ class Scenario:
             n = ek.shape[1]
             if n == 0:
                 continue
-            k = np.zeros((self.num_layers, n, self.hkv, self.d), np.float16)
+            k = np.zeros((self.num_layers, n, self.hkv, self.d), self.dtype)
             v = np.zeros_like(k)
             self.cache.debug_get_kv(sid, 0, n, k, v)
             assert_close(k, ek, atol=2e-3, rtol=2e-3, what=f"cached k of seq {sid}")
@@ -73,8 +74,8 @@ class Scenario:
                 sid = item
                 if sid not in self.cached_k:
                     cache.add_sequence(sid)
-                    self.cached_k[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), np.float16)
-                    self.cached_v[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), np.float16)
+                    self.cached_k[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), self.dtype)
+                    self.cached_v[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), self.dtype)
             seq_ids.append(sid)
             append_lengths.append(n)
 
@@ -107,7 +108,7 @@ class Scenario:
             positions.append(pos)
             if self.rope_mode == ROPE_NORMAL:
                 k_store = np.stack([cf.apply_rotary(k[l], pos, self.rope_scale, self.rope_theta)
-                                    for l in range(self.num_layers)]).astype(np.float16)
+                                    for l in range(self.num_layers)]).astype(self.dtype)
             else:
                 k_store = k
             self.cached_k[sid] = np.concatenate([self.cached_k[sid], k_store], axis=1)
@@ -121,7 +122,7 @@ class Scenario:
             qkv = np.concatenate([np.concatenate([q[layer] for q in new_q]),
                                   np.concatenate([k[layer] for k in new_k]),
                                   np.concatenate([v[layer] for v in new_v])], axis=1)
-            out = np.zeros((total, self.hq, self.d), np.float16)
+            out = np.zeros((total, self.hq, self.d), self.dtype)
             cache.attention_with_fused_qkv(layer, self.sm_scale, np.ascontiguousarray(qkv), out)
             cursor = 0
             for i, (sid, n) in enumerate(zip(seq_ids, append_lengths)):
@@ -170,8 +171,8 @@ class Scenario:
     def add_with_window(self, sid, window, sink):
         self.cache.add_sequence(sid)
         self.cache.enable_sliding_window_for_seq(sid, window, sink)
-        self.cached_k[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), np.float16)
-        self.cached_v[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), np.float16)
+        self.cached_k[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), self.dtype)
+        self.cached_v[sid] = np.zeros((self.num_layers, 0, self.hkv, self.d), self.dtype)
         self.window[sid] = (window, sink)
 
     def fork_with_window(self, parent, sid, pos, window, sink):

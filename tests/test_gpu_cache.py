@@ -32,10 +32,13 @@ def test_reference_scenarios_on_the_gpu(runner, d, rope_mode):
 class Mirror:
     """Feeds the oracle cache and the GPU cache the same calls and the same tensors."""
 
-    def __init__(self, cache_config, layers, hq, hkv, d, rope_mode=1, **rope):
-        self.o = OraclePagedKVCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode, **rope)
-        self.g = GpuCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode, **rope)
+    def __init__(self, cache_config, layers, hq, hkv, d, rope_mode=1, dtype=np.float16, **rope):
+        self.o = OraclePagedKVCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode, dtype=dtype, **rope)
+        self.g = GpuCache(cache_config, layers, hq, hkv, d, d, rope_mode=rope_mode, dtype=dtype, **rope)
         self.layers, self.hq, self.hkv, self.d = layers, hq, hkv, d
+        self.dtype = dtype
+        # float32 storage: what is left is the order of the float32 sums and the device's exp2 / sin / cos
+        self.tol = dict(atol=2e-4, rtol=2e-4) if dtype == np.float32 else {}
         self.rng = np.random.default_rng(21)
         self.lengths = {}
 
@@ -76,18 +79,18 @@ class Mirror:
         self.compare_bookkeeping()
         total = sum(lens)
         for layer in range(self.layers):
-            qkv = self.rng.standard_normal((total, self.hq + 2 * self.hkv, self.d)).astype(np.float16)
-            eo = np.zeros((total, self.hq, self.d), np.float16)
+            qkv = self.rng.standard_normal((total, self.hq + 2 * self.hkv, self.d)).astype(self.dtype)
+            eo = np.zeros((total, self.hq, self.d), self.dtype)
             go = np.zeros_like(eo)
             self.o.attention_with_fused_qkv(layer, self.d ** -0.5, qkv, eo)
             self.g.attention_with_fused_qkv(layer, self.d ** -0.5, qkv, go)
-            assert_close(go, eo, what=f"layer {layer} output vs oracle cache")
+            assert_close(go, eo, what=f"layer {layer} output vs oracle cache", **self.tol)
         self.o.end_forward()
         self.g.end_forward()
         for sid, n in zip(ids, lens):
             self.lengths[sid] += n
             L = self.lengths[sid]
-            ek = np.zeros((self.layers, L, self.hkv, self.d), np.float16)
+            ek = np.zeros((self.layers, L, self.hkv, self.d), self.dtype)
             ev, gk, gv = np.zeros_like(ek), np.zeros_like(ek), np.zeros_like(ek)
             self.o.debug_get_kv(sid, 0, L, ek, ev)
             self.g.debug_get_kv(sid, 0, L, gk, gv)
@@ -110,6 +113,55 @@ def test_identical_inputs_through_oracle_and_gpu_caches(page_size, hq, hkv, d):
     m.lengths[6] -= 30
     m.step([(6, 1), (1, 200)])
     m.step([(i, 1) for i in (0, 1, 2, 4, 5, 6)])
+
+
+@pytest.mark.parametrize("dtype,page_size,hq,hkv,d", [(np.float32, 16, 8, 2, 128), (np.float32, 16, 32, 4, 64),
+                                                      (np.float16, 24, 8, 2, 128), (np.float16, 5, 8, 2, 64),
+                                                      (np.float32, 12, 6, 2, 72), (np.float16, 16, 8, 2, 72),
+                                                      (np.float16, 48, 20, 1, 128)])
+def test_float32_storage_other_page_sizes_and_head_dims_through_both_caches(dtype, page_size, hq, hkv, d):
+    """What the reference's kernel factories accept beside the tuned shapes (its tests run float32 storage,
+    test_runtime_builtin_paged_attention_kv_cache_cpu.py:269-276; page size and head dim are free parameters of
+    every factory): the cache runs these on the generic matrix-core kernels.  Same calls and tensors through the
+    oracle cache (the oracle's float32 build for float32 storage), page tables and pool state bit for bit."""
+    m = Mirror([16, 2048, 512, page_size, 0], 2, hq, hkv, d, dtype=dtype)
+    m.step([(0, 60), (1, 88), (2, 17), (3, 4)])
+    m.step([((4, 3, -1), 35)])
+    m.step([((5, 0, 33), 20)])            # fork inside a page -> page copy on the device
+    m.step([(0, 1), (1, 1), (2, 1), (4, 1), (5, 1)])
+    m.step([((6, 5, -1), 40), (2, 3)])
+    m.step([(6, 1), (5, 1), (0, 1)])      # two block depths + merge_state
+    m.o.popn(6, 30)
+    m.g.popn(6, 30)
+    m.lengths[6] -= 30
+    m.step([(6, 1), (1, 200)])
+    m.step([(i, 1) for i in (0, 1, 2, 4, 5, 6)])
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("runner", [S.run_prefill_and_decode, S.run_remove_sequence, S.run_fork_sequence,
+                                    S.run_unlimited_depth, S.run_popn])
+def test_reference_scenarios_float32_storage(runner, d):
+    """The float32 rows of the reference's fixture (head dims 64 and 128, RopeMode.NORMAL,
+    test_runtime_builtin_paged_attention_kv_cache_cpu.py:269-276) with its geometry, against the numpy closed form."""
+    layers, hq, hkv = 2, 32, 4
+    cache = GpuCache([32, 2048, 512, 16, 0], layers, hq, hkv, d, d, rope_mode=S.ROPE_NORMAL, dtype=np.float32)
+    sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=S.ROPE_NORMAL, seed=5, tol=1e-3, dtype=np.float32)
+    runner(sc)
+
+
+def test_storage_type_of_the_tensors_is_checked():
+    cache = GpuCache([4, 64, 32, 16, 0], 1, 8, 2, 128, 128, dtype=np.float32)
+    cache.add_sequence(0)
+    cache.begin_forward([0], [2])
+    qkv = torch.zeros((2, 12, 128), dtype=torch.float16, device=DEV)
+    out = torch.zeros((2, 8, 128), dtype=torch.float16, device=DEV)
+    with pytest.raises(tvm_amd.KVError, match="stores float32"):
+        gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")(cache.cache, 0, 1.0, qkv, out)
+    with pytest.raises(tvm_amd.KVError, match="plain cache"):
+        GpuCache([4, 64, 32, 16, 1], 1, 8, 2, 128, 128, dtype=np.float32)   # float32 storage with a sliding window
+    with pytest.raises(tvm_amd.KVError, match="plain cache"):
+        GpuCache([4, 64, 32, 24, 0], 1, 8, 2, 128, 128, rope_mode=2)         # pages of 24 tokens with inline RoPE
 
 
 def test_short_chunk_against_a_long_cached_sequence():
@@ -197,11 +249,12 @@ def test_error_paths_on_the_device_cache():
     cache.add_sequence(1)
     with pytest.raises(tvm_amd.KVError, match="The KV cache is full"):
         cache.begin_forward([1], [80])
-    # a kernel's refusal surfaces through the cache call: head_dim 72 is not built
-    c2 = GpuCache([4, 64, 32, 16, 0], 1, 8, 2, 72, 72, rope_mode=0)
+    # a kernel's refusal surfaces through the cache call: head_dim 68 is not built (the generic kernels take
+    # multiples of 8)
+    c2 = GpuCache([4, 64, 32, 16, 0], 1, 8, 2, 68, 68, rope_mode=0)
     c2.add_sequence(0)
-    qkv96 = torch.zeros((1, 12, 72), dtype=torch.float16, device=DEV)
-    out96 = torch.zeros((1, 8, 72), dtype=torch.float16, device=DEV)
+    qkv96 = torch.zeros((1, 12, 68), dtype=torch.float16, device=DEV)
+    out96 = torch.zeros((1, 8, 68), dtype=torch.float16, device=DEV)
     c2.begin_forward([0], [1])
     with pytest.raises(tvm_amd.KVError, match="is not built"):
         attn(c2.cache, 0, 1.0, qkv96, out96)

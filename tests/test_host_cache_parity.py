@@ -285,3 +285,27 @@ class _Fake:
 
     def is_contiguous(self):
         return True
+
+
+def test_storage_types_and_shapes_a_cache_accepts():
+    """float16 and float32 storage (the reference's tests run both); float32, pages other than 16 / 32 / 64 / 128
+    tokens and other head dims are the plain cache (no sliding window, no RoPE inside the attention kernels)."""
+    import torch
+    create = tvm_amd.get_global_func("vm.builtin.paged_attention_kv_cache_create")
+
+    def make(config, d, rope_mode, dtype):
+        return create(config, [0, 1], 8, 2, d, d, [0], False, rope_mode, 1.0, 1e4, None, torch.empty((), dtype=dtype))
+
+    for dtype in (torch.float16, torch.float32):
+        cache = make([4, 64, 32, 16, 0], 128, 1, dtype)
+        assert cache.dtype_bits == (16 if dtype == torch.float16 else 32)
+        tvm_amd.get_global_func("vm.builtin.kv_state_add_sequence")(cache, 0)
+    make([4, 64, 32, 24, 0], 72, 1, torch.float16)           # pages of 24 tokens, head dim 72: the generic kernels
+    with pytest.raises(tvm_amd.KVError, match="plain cache"):
+        make([4, 64, 32, 24, 1], 128, 0, torch.float16)      # pages of 24 tokens with a sliding window
+    with pytest.raises(tvm_amd.KVError, match="plain cache"):
+        make([4, 64, 32, 16, 1], 128, 1, torch.float32)      # float32 with a sliding window
+    with pytest.raises(tvm_amd.KVError, match="plain cache"):
+        make([4, 64, 32, 24, 0], 128, 2, torch.float16)      # pages of 24 tokens with RoPE inside the kernels
+    with pytest.raises(tvm_amd.KVError, match="float16 and float32"):
+        make([4, 64, 32, 16, 0], 128, 1, torch.bfloat16)

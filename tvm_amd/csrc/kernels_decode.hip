@@ -26,6 +26,7 @@
 
 #include "kernels_common.cuh"
 #include "runtime_support.h"
+#include "typed_kernels.h"
 #include "split_plan.h"
 
 namespace tvmkv {
@@ -279,7 +280,10 @@ struct DecodeRopeDivisors {
 // PAD: rows of q, the pages and the output hold p.d_mem (80, 96, 112) elements, fewer than the kernel's
 // head dim: the missing q features are zero, K fragments and V pieces beyond the row repeat its last 16
 // bytes (finite values that meet zeros, or feed output features that are not stored).
-template <bool EXT, int D, bool REREAD, int HB = 1, bool FUSED = false, bool PAD = false>
+// VARIANT (with EXT): the in-kernel RoPE takes a frequency variant (rope_pair_ex: a table entry per element,
+// inverse frequencies, a magnitude).  A kernel of its own: the second set of table entries and the general
+// rotation made every extended launch spill (46-143 registers) while they sat in the same kernel.
+template <bool EXT, int D, bool REREAD, int HB = 1, bool FUSED = false, bool PAD = false, bool VARIANT = false>
 __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void decode_mfma_kernel(DecodeParams p, int group, int num_items,
                                                              DecodeRopeDivisors div) {
   static_assert(HB == 1 || HB == 2, "head blocks per work item");
@@ -346,14 +350,14 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
   // RoPE divisors of the first halves of this lane's K fragment pairs: features i*32 + g4*8 + e, or
   // with KLINE i*64 + (c16&1)*32 + g4*8 + e
   // (and of the second halves, features + D/2, which differ from the first in some frequency variants)
-  float divr[8 * (NPAIR > 0 ? NPAIR : 1)], divh[8 * (NPAIR > 0 ? NPAIR : 1)];
+  float divr[8 * (NPAIR > 0 ? NPAIR : 1)], divh[VARIANT ? 8 * (NPAIR > 0 ? NPAIR : 1) : 1];
   float k_pos0 = 0.f;
   if (EXT && p.rotary) {
 #pragma unroll
     for (int i = 0; i < 8 * NPAIR; ++i) {
       const int f = KLINE ? (i >> 3) * 64 + (c16 & 1) * 32 + g4 * 8 + (i & 7) : (i >> 3) * 32 + g4 * 8 + (i & 7);
       divr[i] = div.v[f];
-      divh[i] = div.v[f + D / 2];
+      if constexpr (VARIANT) divh[i] = div.v[f + D / 2];
     }
     k_pos0 = static_cast<float>(p.k_rope_pos_offset[b]);
   }
@@ -427,13 +431,17 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
       const float q_pos = static_cast<float>(p.q_rope_position[b]) * p.rope_scale;
 #pragma unroll
       for (int ks = 0; ks < KS / 2; ++ks) {
-        float qdiv[8], qdivh[8];
+        float qdiv[8], qdivh[VARIANT ? 8 : 1];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           qdiv[e] = div.v[ks * 32 + g4 * 8 + e];
-          qdivh[e] = div.v[D / 2 + ks * 32 + g4 * 8 + e];
+          if constexpr (VARIANT) qdivh[e] = div.v[D / 2 + ks * 32 + g4 * 8 + e];
         }
-        rope_pair_ex(qv[ks].h8, qv[ks + KS / 2].h8, q_pos, qdiv, qdivh, p.rope_inverse, p.rope_halves_differ, p.rope_magnitude);
+        if constexpr (VARIANT) {
+          rope_pair_ex(qv[ks].h8, qv[ks + KS / 2].h8, q_pos, qdiv, qdivh, p.rope_inverse, p.rope_halves_differ, p.rope_magnitude);
+        } else {
+          rope_pair(qv[ks].h8, qv[ks + KS / 2].h8, q_pos, qdiv);
+        }
       }
     }
 #pragma unroll
@@ -557,8 +565,12 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : ((EXT || HB > 1) ? 2 : 3)) void 
           Vec16* frag = r.k[h] + (KLINE ? tile * TI : 0);
 #pragma unroll
           for (int i = 0; i < NPAIR; ++i) {
-            rope_pair_ex(frag[i].h8, frag[i + NPAIR].h8, pos, divr + 8 * i, divh + 8 * i, p.rope_inverse, p.rope_halves_differ,
-                         p.rope_magnitude);
+            if constexpr (VARIANT) {
+              rope_pair_ex(frag[i].h8, frag[i + NPAIR].h8, pos, divr + 8 * i, divh + 8 * i, p.rope_inverse, p.rope_halves_differ,
+                           p.rope_magnitude);
+            } else {
+              rope_pair(frag[i].h8, frag[i + NPAIR].h8, pos, divr + 8 * i);
+            }
           }
         }
       }
@@ -907,6 +919,8 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid_x)), dim3(256), 0, s, p, group, static_cast<int>(num_items), div);
   };
+  // the default frequencies (one divisor per pair, position / divisor) have the kernel without the general rotation
+  const bool variant = p.rotary && (p.rope_inverse != 0 || p.rope_halves_differ != 0 || p.rope_magnitude != 1.0f);
   auto launch_d = [&](auto dim) {
     constexpr int kD = decltype(dim)::value;
     constexpr int kWide = kD <= 128 ? 2 : 1;  // head blocks per item for groups of more than 16 heads
@@ -919,6 +933,14 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
         launch(decode_mfma_kernel<false, kD, false, kWide, true>);
       } else {
         launch(decode_mfma_kernel<false, kD, false, 1, true>);
+      }
+    } else if (ext && variant) {
+      if (reread) {
+        launch(decode_mfma_kernel<true, kD, true, kWide, false, false, true>);
+      } else if (wide) {
+        launch(decode_mfma_kernel<true, kD, false, kWide, false, false, true>);
+      } else {
+        launch(decode_mfma_kernel<true, kD, false, 1, false, false, true>);
       }
     } else if (reread) {
       if (ext) launch(decode_mfma_kernel<true, kD, true, kWide>); else launch(decode_mfma_kernel<false, kD, true, kWide>);
@@ -950,6 +972,36 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   KV_LAUNCH_CHECK();
 }
 
+// Shapes the tuned kernel is not built for (pages other than 16 / 32 / 64 / 128 tokens, other head dims) run on
+// the generic matrix-core kernel when the call is one it serves: a plain cache, no rotation inside the kernel.
+static bool decode_goes_generic(int64_t rotary_mode, int32_t sliding_window, int32_t d, int32_t page_size) {
+  return rotary_mode == 0 && sliding_window == 0 && (!tuned_page_size(page_size) || !tuned_head_dim(d));
+}
+static int decode_generic(const void* q, const void* pages, const int32_t* page_indptr, const int32_t* page_values,
+                          const int32_t* length_info, void* output, float* lse, double sm_scale, int32_t batch_size,
+                          int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv, int32_t d, int32_t page_size,
+                          void* stream) {
+  GenericAttention a;
+  a.what = "batch_decode_paged_kv";
+  a.q = q;
+  a.pages = pages;
+  a.page_indptr = page_indptr;
+  a.page_values = page_values;
+  a.last_page_len = length_info;
+  a.out = output;
+  a.lse = lse;
+  a.total_q = batch_size;
+  a.nnz_pages = nnz_pages;
+  a.num_pages = num_pages;
+  a.batch = batch_size;
+  a.h_q = h_q;
+  a.h_kv = h_kv;
+  a.d = d;
+  a.page_size = page_size;
+  a.sm_scale = sm_scale;
+  return generic_attention(a, stream);
+}
+
 extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, const int32_t* page_indptr,
                                            const int32_t* page_values, const int32_t* length_info,
                                            const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,
@@ -957,6 +1009,10 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
                                            double rope_theta, double sm_scale, int32_t batch_size,
                                            int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
                                            int32_t d, int32_t page_size, int32_t sliding_window, void* stream) {
+  if (decode_goes_generic(rotary_mode, sliding_window, d, page_size)) {
+    return decode_generic(q, pages, page_indptr, page_values, length_info, output, lse, sm_scale, batch_size, nnz_pages, num_pages,
+                          h_q, h_kv, d, page_size, stream);
+  }
   KV_API_BEGIN();
   hipStream_t s = as_stream(stream);
   decode_entry([&](size_t bytes) { return lease_scratch(kScratchDecode, s, bytes, kArrivalBytes); }, FusedStep{}, q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, output, lse, rotary_mode,
@@ -974,6 +1030,10 @@ extern "C" int tvmkv_batch_decode_paged_kv_scaled(const void* q, const void* pag
                                                   int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
                                                   int32_t d, int32_t page_size, int32_t sliding_window,
                                                   const tvmkv_rope_scaling* rope_scaling, void* stream) {
+  if (decode_goes_generic(rotary_mode, sliding_window, d, page_size)) {
+    return decode_generic(q, pages, page_indptr, page_values, length_info, output, lse, sm_scale, batch_size, nnz_pages, num_pages,
+                          h_q, h_kv, d, page_size, stream);
+  }
   KV_API_BEGIN();
   hipStream_t s = as_stream(stream);
   FusedStep plain;

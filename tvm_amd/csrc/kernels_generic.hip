@@ -1,0 +1,447 @@
+// Generic MHA attention for gfx950: what the reference's kernel factories accept for a plain cache and the
+// tuned fp16 kernels are not built for -- float32 storage, pages of any size, head dims that are a multiple
+// of 4 (fp32) or 8 (fp16) up to 256.  One kernel serves ragged prefill (_prefill_kernels.py:677-923), paged
+// prefill (:54-391), paged decode (_decode_kernels.py:49-411) and both token-tree forms (tree_attn.py:93-259,
+// :634-797): float32 arithmetic on v_mfma_f32_16x16x4_f32, base-2 online softmax (m = -5e4 to start with),
+// K and V rows read straight from memory into matrix operands with one page-table lookup per row.
+//
+// Tile: ROWS = 16 * NB query rows of one (sequence, kv head) -- a row is a (token, head of the GQA group)
+// pair -- against 16 keys per step and wave.  The four waves of a workgroup take every fourth 16-key block
+// and fold their states at the end through LDS; launches with few row tiles also split the keys over
+// workgroups (partial states in scratch memory, merged by a second kernel).
+//
+// Matrix operand layout (v_mfma_f32_16x16x4_f32): lane = 16 * k + i holds A[i][k] and B[k][i]; the result
+// register r of lane 16 * g + j is C[4 g + r][j].  The contraction index is a free choice as long as A and
+// B agree, so for S^T = K Q^T lane (i, g) loads features 16 s + 4 g .. + 3 of key i as one 16-byte piece and
+// feeds one component to each of four instructions; for O^T += V^T P the four keys 4 g + m of lane group g
+// are the contraction slots, which is the order in which lane (j, g) holds the probabilities of row j.
+#include <algorithm>
+
+#include "kernels_common.cuh"
+#include "runtime_support.h"
+#include "typed_kernels.h"
+
+namespace tvmkv {
+namespace {
+
+struct GAttn {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* pages;
+  const int32_t* q_indptr;
+  const int32_t* kv_indptr;
+  const int32_t* page_indptr;
+  const int32_t* page_values;
+  const int32_t* last_page_len;
+  const int32_t* tree_indptr;
+  const int32_t* tree_labels;
+  void* out;
+  float* lse;
+  float* part_o;  // (splits, total_q, h_q, d) normalised partial outputs
+  float* part_s;  // (splits, total_q, h_q) their base-2 log-sum-exp, kNoKeys for an empty share
+  int64_t total_q;
+  int batch, h_q, h_kv, d, page_size, causal, splits;
+  float scale_log2;
+};
+
+constexpr float kMasked = -1.0e30f;  // a masked score; exp2 of it is 0 against any running maximum
+constexpr float kNoKeys = -1.0e30f;  // the log-sum-exp of a share that saw no key
+
+template <typename T>
+__device__ __forceinline__ float4_t load4(const T* p);
+template <>
+__device__ __forceinline__ float4_t load4<float>(const float* p) {
+  return *reinterpret_cast<const float4_t*>(p);
+}
+template <>
+__device__ __forceinline__ float4_t load4<half_t>(const half_t* p) {
+  const half4_t h = *reinterpret_cast<const half4_t*>(p);
+  float4_t f;
+  f[0] = static_cast<float>(h[0]);
+  f[1] = static_cast<float>(h[1]);
+  f[2] = static_cast<float>(h[2]);
+  f[3] = static_cast<float>(h[3]);
+  return f;
+}
+__device__ __forceinline__ void store4(float* p, float4_t v) { *reinterpret_cast<float4_t*>(p) = v; }
+__device__ __forceinline__ void store4(half_t* p, float4_t v) {
+  half4_t h;
+  h[0] = static_cast<half_t>(v[0]);
+  h[1] = static_cast<half_t>(v[1]);
+  h[2] = static_cast<half_t>(v[2]);
+  h[3] = static_cast<half_t>(v[3]);
+  *reinterpret_cast<half4_t*>(p) = h;
+}
+
+template <typename T, int DMAX, int NB>
+__global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(GAttn p) {
+  constexpr int ROWS = 16 * NB;
+  constexpr int KS = DMAX / 16;  // 16-feature steps of the score product = 16-feature blocks of the output
+  __shared__ __attribute__((aligned(16))) float o_lds[2 * ROWS * DMAX];
+  __shared__ float ml_lds[2 * ROWS * 2];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int j = lane & 15;  // query row of a 16-row block (matrix column) / key of a block / feature of a block
+  const int g = lane >> 4;
+  const int group = p.h_q / p.h_kv;
+  const int kvh = blockIdx.y;
+  const int split = blockIdx.z;
+  const int d = p.d;
+
+  // the sequence of this row-tile slot: sequence b owns the slots from (q_start(b) * group) / ROWS + b on
+  auto q_begin = [&](int b) { return p.q_indptr != nullptr ? p.q_indptr[b] : b; };
+  auto slot_begin = [&](int b) { return static_cast<int>(static_cast<int64_t>(q_begin(b)) * group / ROWS) + b; };
+  const int slot = blockIdx.x;
+  int lo = 0, hi = p.batch - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (slot_begin(mid) <= slot) {
+      lo = mid;
+    } else {
+      hi = mid - 1;
+    }
+  }
+  const int b = lo;
+  const int q_start = q_begin(b);
+  const int qo_len = q_begin(b + 1) - q_start;
+  const int rows = qo_len * group;
+  const int r0 = (slot - slot_begin(b)) * ROWS;
+  if (r0 >= rows) return;  // the whole workgroup: a slot beyond the sequence's last row tile
+
+  const bool paged = p.pages != nullptr;
+  int kv_len, kv_start = 0, pbeg = 0;
+  if (paged) {
+    pbeg = p.page_indptr[b];
+    const int npages = p.page_indptr[b + 1] - pbeg;
+    kv_len = npages > 0 ? (npages - 1) * p.page_size + p.last_page_len[b] : 0;  // _kernel_common.py:155-159
+  } else {
+    kv_start = p.kv_indptr[b];
+    kv_len = p.kv_indptr[b + 1] - kv_start;
+  }
+  const bool tree = p.tree_labels != nullptr;
+  int tree_len = 0, tree_start = 0, tree_base = 0;
+  if (tree) {
+    tree_base = p.tree_indptr[b];
+    tree_len = p.tree_indptr[b + 1] - tree_base;
+    tree_start = kv_len - tree_len;
+  }
+  const bool causal = p.causal != 0 && !tree;
+
+  // this lane's query rows (one per 16-row block): key limit, tree label, q fragments
+  int limit[NB];
+  int child_first[NB];
+  float4_t qf[NB][KS];
+  const T* qbase = static_cast<const T*>(p.q);
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int row = r0 + nb * 16 + j;
+    const bool valid = row < rows;
+    const int qi = valid ? row / group : 0;
+    const int head = kvh * group + (valid ? row % group : 0);
+    limit[nb] = !valid ? 0 : (causal ? max(0, min(kv_len, kv_len - qo_len + qi + 1)) : kv_len);
+    child_first[nb] = 0;
+    if (tree && valid && tree_len > 0) {  // the queries are the last qo_len nodes of the tree
+      const int node = min(max(qi + tree_len - qo_len, 0), tree_len - 1);
+      child_first[nb] = p.tree_labels[2 * static_cast<int64_t>(tree_base + node)];
+    }
+    const T* qrow = qbase + (static_cast<int64_t>(q_start + qi) * p.h_q + head) * d;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int f = 16 * s + 4 * g;
+      float4_t z = {0.f, 0.f, 0.f, 0.f};
+      qf[nb][s] = (valid && f < d) ? load4<T>(qrow + f) : z;
+    }
+  }
+  // keys of this row tile, and this workgroup's share of their 16-key blocks
+  const int last_row = min(rows, r0 + ROWS) - 1;
+  const int tile_limit = causal ? max(0, min(kv_len, kv_len - qo_len + last_row / group + 1)) : kv_len;
+  const int nkb = (tile_limit + 15) / 16;
+  const int kb_lo = static_cast<int>(static_cast<int64_t>(split) * nkb / p.splits);
+  const int kb_hi = static_cast<int>(static_cast<int64_t>(split + 1) * nkb / p.splits);
+
+  float m[NB], lsum[NB];
+  float4_t o[NB][KS];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    m[nb] = kNegInit;
+    lsum[nb] = 0.f;
+#pragma unroll
+    for (int fb = 0; fb < KS; ++fb) {
+      float4_t z = {0.f, 0.f, 0.f, 0.f};
+      o[nb][fb] = z;
+    }
+  }
+
+  const T* kbase = paged ? static_cast<const T*>(p.pages) : static_cast<const T*>(p.k);
+  const T* vbase = paged ? static_cast<const T*>(p.pages) : static_cast<const T*>(p.v);
+  const int ps = p.page_size;
+  for (int kb = kb_lo + wave; kb < kb_hi; kb += 4) {
+    // row of key kb * 16 + j in its tensor (rows of d elements); keys past the end repeat the last one (masked)
+    const int t = min(kb * 16 + j, kv_len - 1);
+    int krow, vrow;
+    if (paged) {
+      const int pg = t / ps;
+      const int page = p.page_values[pbeg + pg];
+      krow = ((page * 2) * p.h_kv + kvh) * ps + (t - pg * ps);  // pages (num_pages, 2, h_kv, page_size, d)
+      vrow = krow + p.h_kv * ps;
+    } else {
+      krow = vrow = (kv_start + t) * p.h_kv + kvh;
+    }
+    float4_t kf[KS];
+    const T* krow_ptr = kbase + static_cast<int64_t>(krow) * d;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int f = 16 * s + 4 * g;
+      float4_t z = {0.f, 0.f, 0.f, 0.f};
+      kf[s] = f < d ? load4<T>(krow_ptr + f) : z;
+    }
+    // V^T operands: feature fb * 16 + j of the four keys 4 g + m
+    float vf[KS][4];
+#pragma unroll
+    for (int mm = 0; mm < 4; ++mm) {
+      const int vr = __shfl(vrow, 4 * g + mm);
+      const T* vrow_ptr = vbase + static_cast<int64_t>(vr) * d;
+#pragma unroll
+      for (int fb = 0; fb < KS; ++fb) {
+        const int f = fb * 16 + j;
+        vf[fb][mm] = f < d ? static_cast<float>(vrow_ptr[f]) : 0.f;
+      }
+    }
+    const bool in_tree = tree && kb * 16 + 15 >= tree_start;  // wave-uniform
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s][c], qf[nb][s][c], acc, 0, 0, 0);
+      }
+      // acc[r]: key kb * 16 + 4 g + r, query row nb * 16 + j
+      float sc[4];
+      float mx = kMasked;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = kb * 16 + 4 * g + r;
+        bool visible = key < limit[nb];
+        if (in_tree && key >= tree_start && key < kv_len) {  // tree_attn.py:48-65
+          const int32_t* parent = p.tree_labels + 2 * static_cast<int64_t>(tree_base + key - tree_start);
+          visible = visible && child_first[nb] >= parent[0] && child_first[nb] < parent[1];
+        }
+        sc[r] = visible ? acc[r] * p.scale_log2 : kMasked;
+        mx = fmaxf(mx, sc[r]);
+      }
+      mx = max_xor32(max_xor16(mx));  // over the four lane groups that hold the row's other keys
+      const float m_new = fmaxf(m[nb], mx);
+      const float alpha = fast_exp2(m[nb] - m_new);
+      m[nb] = m_new;
+      float pr[4];
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pr[r] = fast_exp2(sc[r] - m_new);
+        sum += pr[r];
+      }
+      lsum[nb] = lsum[nb] * alpha + sum;
+#pragma unroll
+      for (int fb = 0; fb < KS; ++fb) {
+        o[nb][fb] *= alpha;
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) o[nb][fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[fb][mm], pr[mm], o[nb][fb], 0, 0, 0);
+      }
+    }
+  }
+  // the row sums of the four lane groups
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) lsum[nb] = sum_xor32(sum_xor16(lsum[nb]));
+
+  // ---- the four waves' states into wave 0: waves 2, 3 -> 0, 1, then 1 -> 0 --------------------------------
+  // o[nb][fb][r] of lane (j, g) is feature fb * 16 + 4 g + r of row nb * 16 + j
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+      for (int fb = 0; fb < KS; ++fb) store4(o_lds + (buf * ROWS + nb * 16 + j) * DMAX + fb * 16 + 4 * g, o[nb][fb]);
+      if (g == 0) {
+        ml_lds[(buf * ROWS + nb * 16 + j) * 2 + 0] = m[nb];
+        ml_lds[(buf * ROWS + nb * 16 + j) * 2 + 1] = lsum[nb];
+      }
+    }
+  };
+  auto take = [&](int buf) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const float m_other = ml_lds[(buf * ROWS + nb * 16 + j) * 2 + 0];
+      const float l_other = ml_lds[(buf * ROWS + nb * 16 + j) * 2 + 1];
+      const float m_new = fmaxf(m[nb], m_other);
+      const float mine = fast_exp2(m[nb] - m_new), theirs = fast_exp2(m_other - m_new);
+      m[nb] = m_new;
+      lsum[nb] = lsum[nb] * mine + l_other * theirs;
+#pragma unroll
+      for (int fb = 0; fb < KS; ++fb) {
+        const float4_t other = *reinterpret_cast<const float4_t*>(o_lds + (buf * ROWS + nb * 16 + j) * DMAX + fb * 16 + 4 * g);
+        o[nb][fb] = o[nb][fb] * mine + other * theirs;
+      }
+    }
+  };
+  if (wave >= 2) put(wave - 2);
+  __syncthreads();
+  if (wave < 2) take(wave);
+  __syncthreads();
+  if (wave == 1) put(0);
+  __syncthreads();
+  if (wave != 0) return;
+  take(0);
+
+  // ---- wave 0 writes the rows: the result, or this share's partial state -----------------------------------
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int row = r0 + nb * 16 + j;
+    if (row >= rows) continue;
+    const int64_t out_row = static_cast<int64_t>(q_start + row / group) * p.h_q + kvh * group + row % group;
+    const bool any = lsum[nb] > 0.f;
+    const float inv = any ? 1.0f / lsum[nb] : 0.f;
+    const float s_row = any ? m[nb] + fast_log2(lsum[nb]) : kNoKeys;
+    if (p.splits == 1) {
+      T* dst = static_cast<T*>(p.out) + out_row * d;
+#pragma unroll
+      for (int fb = 0; fb < KS; ++fb) {
+        const int f = fb * 16 + 4 * g;
+        if (f < d) store4(dst + f, o[nb][fb] * inv);
+      }
+      // a row without keys: out = 0 and the state the reference's kernels start from, m = -5e4, d = 1
+      if (g == 0) p.lse[out_row] = any ? s_row : kNegInit;
+    } else {
+      float* dst = p.part_o + (static_cast<int64_t>(split) * p.total_q * p.h_q + out_row) * d;
+#pragma unroll
+      for (int fb = 0; fb < KS; ++fb) {
+        const int f = fb * 16 + 4 * g;
+        if (f < d) store4(dst + f, o[nb][fb] * inv);
+      }
+      if (g == 0) p.part_s[static_cast<int64_t>(split) * p.total_q * p.h_q + out_row] = s_row;
+    }
+  }
+}
+
+// The shares of a split launch: one workgroup of 64 lanes per (query, head) row.
+template <typename T>
+__global__ __launch_bounds__(64) void generic_merge_kernel(const float* part_o, const float* part_s, T* out, float* lse,
+                                                          int64_t rows, int d, int splits) {
+  const int64_t row = blockIdx.x;
+  float s_max = kNoKeys;
+  for (int z = 0; z < splits; ++z) s_max = fmaxf(s_max, part_s[z * rows + row]);
+  const bool any = s_max > 0.5f * kNoKeys;
+  float total = 0.f;
+  for (int z = 0; z < splits; ++z) total += any ? fast_exp2(part_s[z * rows + row] - s_max) : 0.f;
+  for (int f = threadIdx.x; f < d; f += 64) {
+    float acc = 0.f;
+    for (int z = 0; z < splits; ++z) {
+      const float w = any ? fast_exp2(part_s[z * rows + row] - s_max) : 0.f;
+      acc += w * part_o[(z * rows + row) * d + f];
+    }
+    out[row * d + f] = static_cast<T>(any ? acc / total : 0.f);
+  }
+  if (threadIdx.x == 0) lse[row] = any ? s_max + fast_log2(total) : kNegInit;
+}
+
+template <typename T>
+void launch_attention(const GAttn& p, int rows_hint, hipStream_t stream) {
+  const int group = p.h_q / p.h_kv;
+  auto run = [&](auto kernel, int rows_per_tile) {
+    const int64_t slots = p.total_q * group / rows_per_tile + p.batch;
+    KV_CHECK(slots < (int64_t{1} << 31)) << "too many row tiles for one launch";
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(slots), p.h_kv, p.splits), dim3(256), 0, stream, p);
+  };
+  const bool wide = rows_hint > 16;  // more than one 16-row block per (sequence, kv head) on average
+  if (p.d <= 64) {
+    if (wide) run(generic_attn_kernel<T, 64, 2>, 32); else run(generic_attn_kernel<T, 64, 1>, 16);
+  } else if (p.d <= 128) {
+    if (wide) run(generic_attn_kernel<T, 128, 2>, 32); else run(generic_attn_kernel<T, 128, 1>, 16);
+  } else {
+    run(generic_attn_kernel<T, 256, 1>, 16);
+  }
+  KV_LAUNCH_CHECK();
+}
+
+}  // namespace
+
+int generic_attention(const GenericAttention& a, void* stream_) {
+  KV_API_BEGIN();
+  hipStream_t stream = as_stream(stream_);
+  const bool f32 = a.elem_bits == 32;
+  KV_CHECK(a.elem_bits == 16 || a.elem_bits == 32) << a.what << ": elem_bits must be 16 or 32";
+  KV_CHECK(a.batch >= 0 && a.total_q >= 0 && a.h_q > 0 && a.h_kv > 0 && a.h_q % a.h_kv == 0) << a.what << ": bad shape";
+  KV_UNSUPPORTED(a.d <= 0 || a.d > 256 || a.d % (f32 ? 4 : 8) != 0)
+      << a.what << ": head_dim " << a.d << " is not built (the generic kernels take multiples of " << (f32 ? 4 : 8)
+      << " up to 256)";
+  if (a.batch == 0 || a.total_q == 0) return TVMKV_OK;
+  const bool paged = a.pages != nullptr;
+  KV_CHECK(a.q && a.out && a.lse) << a.what << ": NULL tensor";
+  if (paged) {
+    KV_CHECK(a.page_indptr && a.page_values && a.last_page_len && a.page_size > 0) << a.what << ": NULL page table or bad page size";
+    KV_CHECK(a.num_pages * 2 * a.h_kv * a.page_size < (int64_t{1} << 31)) << a.what << ": the page pool has too many rows for 32-bit row ids";
+  } else {
+    KV_CHECK(a.k && a.v && a.kv_indptr) << a.what << ": NULL tensor";
+  }
+  KV_CHECK((a.tree_indptr == nullptr) == (a.tree_labels == nullptr)) << a.what << ": tree_indptr and the labels come together";
+  KV_CHECK(a.total_q * a.h_q < (int64_t{1} << 31)) << a.what << ": too many rows for one launch";
+
+  GAttn p{};
+  p.q = a.q;
+  p.k = a.k;
+  p.v = a.v;
+  p.pages = a.pages;
+  p.q_indptr = a.q_indptr;
+  p.kv_indptr = a.kv_indptr;
+  p.page_indptr = a.page_indptr;
+  p.page_values = a.page_values;
+  p.last_page_len = a.last_page_len;
+  p.tree_indptr = a.tree_indptr;
+  p.tree_labels = a.tree_labels;
+  p.out = a.out;
+  p.lse = a.lse;
+  p.total_q = a.total_q;
+  p.batch = a.batch;
+  p.h_q = a.h_q;
+  p.h_kv = a.h_kv;
+  p.d = a.d;
+  p.page_size = a.page_size;
+  p.causal = a.causal;
+  p.scale_log2 = static_cast<float>(a.sm_scale) * kLog2e;
+  const int group = a.h_q / a.h_kv;
+  const int rows_hint = static_cast<int>(std::min<int64_t>(a.total_q * group / a.batch, 1 << 20));
+  // Few row tiles against long page lists: split the keys over workgroups until the chip has ~8 workgroups
+  // per compute unit, at least 128 keys (8 blocks) per share on average.  Shapes only: no device read.
+  p.splits = 1;
+  ScratchLease lease{};
+  if (paged) {
+    const int rows_per_tile = (rows_hint > 16 && a.d <= 128) ? 32 : 16;
+    const int64_t tiles = (a.total_q * group / rows_per_tile + a.batch) * a.h_kv;
+    const int64_t keys_per_seq = a.nnz_pages * a.page_size / a.batch;
+    const int64_t want = 8 * static_cast<int64_t>(compute_units()) / std::max<int64_t>(tiles, 1);
+    p.splits = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>({want, keys_per_seq / 128, 64})));
+  }
+  if (p.splits > 1) {
+    const size_t o_bytes = static_cast<size_t>(p.splits) * a.total_q * a.h_q * a.d * sizeof(float);
+    const size_t s_bytes = static_cast<size_t>(p.splits) * a.total_q * a.h_q * sizeof(float);
+    lease = lease_scratch(kScratchGeneric, stream, o_bytes + s_bytes, 0);  // held until the merge is enqueued
+    p.part_o = reinterpret_cast<float*>(lease.ptr);
+    p.part_s = reinterpret_cast<float*>(lease.ptr + o_bytes);
+  }
+  if (f32) launch_attention<float>(p, rows_hint, stream); else launch_attention<half_t>(p, rows_hint, stream);
+  if (p.splits > 1) {
+    const int64_t rows = a.total_q * a.h_q;
+    if (f32) {
+      hipLaunchKernelGGL(generic_merge_kernel<float>, dim3(static_cast<unsigned>(rows)), dim3(64), 0, stream, p.part_o, p.part_s,
+                         static_cast<float*>(a.out), a.lse, rows, a.d, p.splits);
+    } else {
+      hipLaunchKernelGGL(generic_merge_kernel<half_t>, dim3(static_cast<unsigned>(rows)), dim3(64), 0, stream, p.part_o, p.part_s,
+                         static_cast<half_t*>(a.out), a.lse, rows, a.d, p.splits);
+    }
+    KV_LAUNCH_CHECK();
+  }
+  KV_API_END();
+}
+
+}  // namespace tvmkv

@@ -7,7 +7,10 @@
 // run of full 128-byte lines.
 #include <cmath>
 
+#include <type_traits>
+
 #include "kernels_common.cuh"
+#include "typed_kernels.h"
 #include "runtime_support.h"
 
 namespace tvmkv {
@@ -327,6 +330,103 @@ __global__ __launch_bounds__(256) void merge_state_inplace_kernel(half_t* __rest
   if (c == 0) s[row] = log2f(s_val + s_other_val) + s_max;
 }
 
+// The split-rotary kernel for what the vectorised one above is not built for: float32 storage and head dims
+// outside its list (any even head dim up to kMaxHeadDim).  The same tables and the same arithmetic, one
+// element per thread and step: element e of a rotating head becomes cos * x[e] + sin * partner(e), the partner
+// being -x[e + R/2] / x[e - R/2], or -x[e + 1] / x[e - 1] for the gptj pairing.
+template <typename T, bool APPEND>
+__global__ __launch_bounds__(256) void fused_rope_any_kernel(const T* __restrict__ qkv, const int32_t* __restrict__ position_map,
+                                                             T* __restrict__ q, T* __restrict__ k, T* __restrict__ v,
+                                                             int num_q_heads, int num_kv_heads, int D, int apply_rope,
+                                                             float scale, RopeDivisors div, int table_is_inverse,
+                                                             int halves_differ, float magnitude,
+                                                             const float* __restrict__ ext_factors, T* __restrict__ pages,
+                                                             const int32_t* __restrict__ append_position_map, int page_size,
+                                                             int rotary_dim, int interleaved) {
+  __shared__ float cs_lds[kMaxHeadDim];
+  __shared__ float sn_lds[kMaxHeadDim];
+  const int R = rotary_dim;
+  const int64_t s = blockIdx.x;  // token
+  const int fused_heads = num_q_heads + 2 * num_kv_heads;
+  if (apply_rope > 0) {
+    const float pos_scaled = static_cast<float>(position_map[s]) * scale;
+    for (int i = threadIdx.x; i < (halves_differ ? R : R / 2); i += 256) {
+      float freq;
+      if (table_is_inverse) {
+        freq = pos_scaled * div.v[i];
+      } else {
+        freq = pos_scaled / (ext_factors != nullptr ? ext_factors[i] * div.v[i] : div.v[i]);
+      }
+      const float cs = cosf(freq) * magnitude, sn = sinf(freq) * magnitude;
+      cs_lds[i] = cs;
+      sn_lds[i] = sn;
+      if (!halves_differ) {
+        cs_lds[i + R / 2] = cs;
+        sn_lds[i + R / 2] = sn;
+      }
+    }
+    __syncthreads();
+  }
+  const int32_t slot = APPEND ? append_position_map[s] : -1;
+  const int first = q == nullptr ? num_q_heads * D : 0;  // q == NULL: the q rows are left alone
+  for (int idx = first + threadIdx.x; idx < fused_heads * D; idx += 256) {
+    const int h = idx / D, e = idx - h * D;
+    const T* row = qkv + (s * fused_heads + h) * D;
+    float x = static_cast<float>(row[e]);
+    T result = row[e];
+    if (apply_rope > 0 && h < num_q_heads + num_kv_heads && e < R) {
+      float other;
+      if (interleaved) {
+        other = (e & 1) == 0 ? -static_cast<float>(row[e + 1]) : static_cast<float>(row[e - 1]);
+      } else {
+        other = e < R / 2 ? -static_cast<float>(row[e + R / 2]) : static_cast<float>(row[e - R / 2]);
+      }
+      result = static_cast<T>(cs_lds[e] * x + sn_lds[e] * other);
+    }
+    if (h < num_q_heads) {
+      q[(s * num_q_heads + h) * D + e] = result;
+      continue;
+    }
+    const int kv = h >= num_q_heads + num_kv_heads;
+    const int head = h - num_q_heads - kv * num_kv_heads;
+    (kv ? v : k)[(s * num_kv_heads + head) * D + e] = result;
+    if (APPEND && slot != -1) {
+      pages[((static_cast<int64_t>(slot / page_size) * 2 + kv) * num_kv_heads + head) * (static_cast<int64_t>(page_size) * D) +
+            static_cast<int64_t>(slot % page_size) * D + e] = result;
+    }
+  }
+}
+
+// merge_state_inplace for float32 storage: one thread per 4 features; the threads of a row read S before the
+// one that owns piece 0 rewrites it only if they share a wavefront, so S goes through registers first and the
+// new value is written after every lane of the row has used the old one (rows never straddle wavefronts: the
+// lanes per row are a power of two up to 64).
+__global__ __launch_bounds__(256) void merge_state_inplace_f32_kernel(float* __restrict__ v, float* __restrict__ s,
+                                                                      const float* __restrict__ v_other,
+                                                                      const float* __restrict__ s_other, int64_t rows, int d,
+                                                                      int lanes_per_row) {
+  const int chunks = d / 4;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int lane_in_row = gid % lanes_per_row;
+  const int64_t row = gid / lanes_per_row;
+  if (row >= rows) return;
+  float s_val = s[row];
+  float s_other_val = s_other[row];
+  const float s_max = fmaxf(s_val, s_other_val);
+  s_val = exp2f(s_val - s_max);
+  s_other_val = exp2f(s_other_val - s_max);
+  const float scale = s_val / (s_val + s_other_val);
+  const float other_scale = s_other_val / (s_val + s_other_val);
+  for (int c = lane_in_row; c < chunks; c += lanes_per_row) {
+    float4_t a = *reinterpret_cast<const float4_t*>(v + row * d + c * 4);
+    const float4_t b = *reinterpret_cast<const float4_t*>(v_other + row * d + c * 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) a[e] = a[e] * scale + b[e] * other_scale;
+    *reinterpret_cast<float4_t*>(v + row * d + c * 4) = a;
+  }
+  if (lane_in_row == 0) s[row] = log2f(s_val + s_other_val) + s_max;
+}
+
 inline dim3 grid_for(int64_t threads, int block = 256) { return dim3(static_cast<unsigned>((threads + block - 1) / block)); }
 
 }  // namespace tvmkv
@@ -436,11 +536,15 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
                            int64_t apply_rope, const float* ext_factors, const tvmkv_rope_scaling* scaling,
                            int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
                            int32_t head_dim, double rope_scale, double rope_theta, void* pages,
-                           const int32_t* append_position_map, int64_t num_pages, int32_t page_size, void* stream) {
+                           const int32_t* append_position_map, int64_t num_pages, int32_t page_size, void* stream,
+                           int elem_bits = 16) {
   KV_API_BEGIN();
   KV_CHECK(seq_len >= 0 && num_q_heads > 0 && num_kv_heads > 0) << "fused_rope: bad shape";
-  KV_UNSUPPORTED(head_dim != 64 && head_dim != 128 && head_dim != 256 && head_dim != 80 && head_dim != 96 && head_dim != 112)
-      << "fused_rope: head_dim " << head_dim << " is not built (64, 80, 96, 112, 128, 256)";
+  KV_CHECK(elem_bits == 16 || elem_bits == 32) << "fused_rope: elem_bits must be 16 or 32";
+  KV_UNSUPPORTED(head_dim <= 0 || head_dim > kMaxHeadDim || head_dim % 2 != 0)
+      << "fused_rope: head_dim " << head_dim << " is not built (even head dims up to " << kMaxHeadDim << ")";
+  const bool vectorised = elem_bits == 16 && (head_dim == 64 || head_dim == 128 || head_dim == 256 || head_dim == 80 ||
+                                              head_dim == 96 || head_dim == 112);
   if (seq_len == 0) return TVMKV_OK;
   const bool append = pages != nullptr;
   KV_CHECK(qkv && position_map && (q || append) && k && v) << "fused_rope: NULL tensor";
@@ -467,7 +571,23 @@ static int fused_rope_impl(const void* qkv, const int32_t* position_map, void* q
                        append_position_map, page_size, rotary_dim,
                        static_cast<int>(scaling != nullptr && scaling->rope_type == TVMKV_ROPE_FREQ_GPTJ));
   };
-  if (head_dim == 64) {
+  auto launch_any = [&](auto kernel, auto* typed_null) {
+    using T = std::remove_pointer_t<decltype(typed_null)>;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(seq_len)), dim3(256), 0, as_stream(stream), static_cast<const T*>(qkv),
+                       position_map, static_cast<T*>(q), static_cast<T*>(k), static_cast<T*>(v), num_q_heads, num_kv_heads,
+                       head_dim, static_cast<int>(apply_rope > 0), scale, div, static_cast<int>(table_is_inverse),
+                       static_cast<int>(halves_differ), magnitude, ext_factors, static_cast<T*>(pages), append_position_map,
+                       page_size, rotary_dim, static_cast<int>(scaling != nullptr && scaling->rope_type == TVMKV_ROPE_FREQ_GPTJ));
+  };
+  if (!vectorised) {
+    if (elem_bits == 32) {
+      if (append) launch_any(fused_rope_any_kernel<float, true>, static_cast<float*>(nullptr));
+      else launch_any(fused_rope_any_kernel<float, false>, static_cast<float*>(nullptr));
+    } else {
+      if (append) launch_any(fused_rope_any_kernel<half_t, true>, static_cast<half_t*>(nullptr));
+      else launch_any(fused_rope_any_kernel<half_t, false>, static_cast<half_t*>(nullptr));
+    }
+  } else if (head_dim == 64) {
     if (append) launch(fused_rope_kernel<64, true>); else launch(fused_rope_kernel<64, false>);
   } else if (head_dim == 128) {
     if (append) launch(fused_rope_kernel<128, true>); else launch(fused_rope_kernel<128, false>);
@@ -658,6 +778,34 @@ int tvmkv_merge_state_inplace(void* v, float* s, const void* v_other, const floa
 }  // extern "C"
 
 namespace tvmkv {
+
+int typed_fused_rope(int elem_bits, const void* qkv, const int32_t* position_map, void* q, void* k, void* v,
+                     int64_t apply_rope, const float* rope_ext_factors, const tvmkv_rope_scaling* scaling, void* pages,
+                     const int32_t* append_position_map, int64_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
+                     int32_t head_dim, int64_t num_pages, int32_t page_size, double rope_scale, double rope_theta,
+                     void* stream) {
+  return fused_rope_impl(qkv, position_map, q, k, v, apply_rope, rope_ext_factors, scaling, seq_len, num_q_heads, num_kv_heads,
+                         head_dim, rope_scale, rope_theta, pages, append_position_map, num_pages, page_size, stream, elem_bits);
+}
+
+int typed_merge_state_inplace(int elem_bits, void* v, float* s, const void* v_other, const float* s_other, int64_t n,
+                              int32_t h, int32_t d, void* stream) {
+  if (elem_bits == 16) return tvmkv_merge_state_inplace(v, s, v_other, s_other, n, h, d, stream);
+  KV_API_BEGIN();
+  KV_CHECK(elem_bits == 32) << "merge_state_inplace: elem_bits must be 16 or 32";
+  KV_CHECK(n >= 0 && h > 0) << "merge_state_inplace: bad shape";
+  KV_UNSUPPORTED(d <= 0 || d % 4 != 0 || d > 512)
+      << "merge_state_inplace: head dim " << d << " is not built (float32: a multiple of 4 up to 512)";
+  if (n == 0) return TVMKV_OK;
+  KV_CHECK(v && s && v_other && s_other) << "merge_state_inplace: NULL tensor";
+  int lanes_per_row = 1;
+  while (lanes_per_row < d / 4 && lanes_per_row < 64) lanes_per_row *= 2;
+  const int64_t rows = n * h;
+  hipLaunchKernelGGL(merge_state_inplace_f32_kernel, grid_for(rows * lanes_per_row), dim3(256), 0, as_stream(stream),
+                     static_cast<float*>(v), s, static_cast<const float*>(v_other), s_other, rows, d, lanes_per_row);
+  KV_LAUNCH_CHECK();
+  KV_API_END();
+}
 
 InlineRopeHost inline_rope_table(const ::tvmkv_rope_scaling* scaling, int head_dim, double rope_theta) {
   KV_CHECK(head_dim > 0 && head_dim <= kMaxHeadDim && head_dim % 2 == 0) << "in-kernel RoPE: head_dim " << head_dim;

@@ -31,6 +31,7 @@
 
 #include "prefill_common.cuh"
 #include "runtime_support.h"
+#include "typed_kernels.h"
 
 namespace tvmkv {
 
@@ -72,7 +73,10 @@ constexpr size_t prefill_lds_bytes(int dqk, int dv) {
 // the q fragments of the missing features are zero, the K/V copies fill the missing 16-byte pieces of a
 // row with a repeat of its last piece (finite values that meet zeros in the score product and only reach
 // output features that are not stored), and the epilogue stores the first d_mem features.
-template <int DQK, int DV, int SRC, int PS, bool EXT, bool STREAM = false, bool PAD = false>
+// VARIANT: the in-kernel RoPE takes a frequency variant (a table entry per element, inverse frequencies, a
+// magnitude: rope_pair_ex).  A kernel of its own: the general rotation holds more values than the default one,
+// and inside one kernel it made every extended launch spill (67-87 registers at head dim 128).
+template <int DQK, int DV, int SRC, int PS, bool EXT, bool STREAM = false, bool PAD = false, bool VARIANT = false>
 __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 64 ? 3 : 2)) void prefill_kernel(PrefillParams p, PrefillRopeDivisors div) {
   constexpr bool PAGED = SRC == kPaged, BOTH = SRC == kBoth;
   static_assert(!PAD || (!EXT && !BOTH && DQK == DV), "padded head dims: plain ragged and paged kernels");
@@ -283,8 +287,12 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
       const float q_pos = static_cast<float>(p.q_rope_position[q_start + my_pos]) * p.rope_scale;
 #pragma unroll
       for (int ks = 0; ks < KS / 2; ++ks) {
-        rope_pair_ex(qf[ks], qf[ks + KS / 2], q_pos, div_lds + ks * 16 + half * 8, div_lds + DQK / 2 + ks * 16 + half * 8,
-                     p.rope_inverse, p.rope_halves_differ, p.rope_magnitude);
+        if constexpr (VARIANT) {
+          rope_pair_ex(qf[ks], qf[ks + KS / 2], q_pos, div_lds + ks * 16 + half * 8, div_lds + DQK / 2 + ks * 16 + half * 8,
+                       p.rope_inverse, p.rope_halves_differ, p.rope_magnitude);
+        } else {
+          rope_pair(qf[ks], qf[ks + KS / 2], q_pos, div_lds + ks * 16 + half * 8);
+        }
       }
     }
   }
@@ -663,8 +671,12 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 || DQK + DV > 320) ? 1 : (DQK == 
         if (!PAGED && p.k_pos_from_q) pos = static_cast<float>(p.q_rope_position[kv_start + t]) * p.rope_scale;
 #pragma unroll
         for (int ks = 0; ks < KS / 2; ++ks) {
-          rope_pair_ex(kf[ks], kf[ks + KS / 2], pos, div_lds + ks * 16 + half * 8, div_lds + DQK / 2 + ks * 16 + half * 8,
-                       p.rope_inverse, p.rope_halves_differ, p.rope_magnitude);
+          if constexpr (VARIANT) {
+            rope_pair_ex(kf[ks], kf[ks + KS / 2], pos, div_lds + ks * 16 + half * 8, div_lds + DQK / 2 + ks * 16 + half * 8,
+                         p.rope_inverse, p.rope_halves_differ, p.rope_magnitude);
+          } else {
+            rope_pair(kf[ks], kf[ks + KS / 2], pos, div_lds + ks * 16 + half * 8);
+          }
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -760,7 +772,7 @@ static int paged_page_shift(int32_t page_size) {
   return shift;
 }
 
-template <int DQK, int DV, int SRC, int PS, bool EXT, bool STREAM = false, bool PAD = false>
+template <int DQK, int DV, int SRC, int PS, bool EXT, bool STREAM = false, bool PAD = false, bool VARIANT = false>
 static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const PrefillRopeDivisors& div,
                                hipStream_t stream) {
   const int64_t slots = total_q * p.group / BM + p.batch_size;
@@ -768,11 +780,11 @@ static void launch_prefill_ext(const PrefillParams& p, int64_t total_q, const Pr
   constexpr size_t lds_bytes = prefill_lds_bytes(DQK, DV);
   static bool attr_set = false;  // per instantiation; the attribute is per function, not per device
   if (lds_bytes > 48 * 1024 && !attr_set) {
-    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, SRC, PS, EXT, STREAM, PAD>),
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<DQK, DV, SRC, PS, EXT, STREAM, PAD, VARIANT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     attr_set = true;
   }
-  hipLaunchKernelGGL((prefill_kernel<DQK, DV, SRC, PS, EXT, STREAM, PAD>),
+  hipLaunchKernelGGL((prefill_kernel<DQK, DV, SRC, PS, EXT, STREAM, PAD, VARIANT>),
                      dim3(p.h_kv, static_cast<unsigned>(slots), static_cast<unsigned>(std::max(1, p.kv_splits))),
                      dim3(NW * 64), lds_bytes, stream, p, div);
 }
@@ -933,13 +945,23 @@ static void launch_prefill(const PrefillParams& params, int64_t total_q, bool ex
   }
   if constexpr (DQK == DV && SRC != kBoth) {
     if (p.rotary) fill_table();
+    // the default frequencies (one divisor per pair, position / divisor) have the kernel without the general rotation
+    const bool variant = p.rotary && (p.rope_inverse != 0 || p.rope_halves_differ != 0 || p.rope_magnitude != 1.0f);
     if constexpr (SRC == kPaged) {
       if (p.stream_kv) {
-        launch_prefill_ext<DQK, DV, SRC, PS, true, true>(p, total_q, div, stream);
+        if (variant) {
+          launch_prefill_ext<DQK, DV, SRC, PS, true, true, false, true>(p, total_q, div, stream);
+        } else {
+          launch_prefill_ext<DQK, DV, SRC, PS, true, true>(p, total_q, div, stream);
+        }
         return;
       }
     }
-    launch_prefill_ext<DQK, DV, SRC, PS, true>(p, total_q, div, stream);
+    if (variant) {
+      launch_prefill_ext<DQK, DV, SRC, PS, true, false, false, true>(p, total_q, div, stream);
+    } else {
+      launch_prefill_ext<DQK, DV, SRC, PS, true>(p, total_q, div, stream);
+    }
   } else {
     throw Error(TVMKV_EUNSUPPORTED, "prefill: inline RoPE / sliding window are not built for this head shape");
   }
@@ -970,6 +992,26 @@ static int ragged_prefill(const void* q, const int32_t* q_indptr, const void* k,
                           int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
                           int32_t batch_size, int64_t total_q, int32_t h_q, int32_t h_kv, int32_t d_qk,
                           int32_t d_v, const tvmkv_rope_scaling* scaling, void* stream) {
+  // head dims the tuned kernel is not built for: the generic matrix-core kernel (no rotation inside it)
+  if (rotary_mode == 0 && d_qk == d_v && !tuned_head_dim(d_qk)) {
+    GenericAttention a;
+    a.what = "batch_prefill_ragged_kv";
+    a.q = q;
+    a.q_indptr = q_indptr;
+    a.k = k;
+    a.v = v;
+    a.kv_indptr = kv_indptr;
+    a.out = output;
+    a.lse = lse;
+    a.total_q = total_q;
+    a.batch = batch_size;
+    a.h_q = h_q;
+    a.h_kv = h_kv;
+    a.d = d_qk;
+    a.causal = causal > 0;
+    a.sm_scale = sm_scale;
+    return generic_attention(a, stream);
+  }
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_ragged_kv: bad shape";
@@ -1043,6 +1085,31 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
                          int32_t h_kv, int32_t d, int32_t page_size, int32_t sliding_window,
                          int32_t sliding_window_size, bool merge_into, void* stream,
                          const tvmkv_rope_scaling* scaling = nullptr) {
+  // pages other than 16 / 32 / 64 / 128 tokens, other head dims: the generic matrix-core kernel, for a plain
+  // cache without rotation inside the kernel (its caller merges states with merge_state_inplace)
+  if (rotary_mode == 0 && sliding_window == 0 && !merge_into && (!tuned_page_size(page_size) || !tuned_head_dim(d))) {
+    GenericAttention a;
+    a.what = "batch_prefill_paged_kv";
+    a.q = q;
+    a.q_indptr = q_indptr;
+    a.pages = pages;
+    a.page_indptr = page_indptr;
+    a.page_values = page_values;
+    a.last_page_len = length_info;
+    a.out = output;
+    a.lse = lse;
+    a.total_q = total_q;
+    a.nnz_pages = nnz_pages;
+    a.num_pages = num_pages;
+    a.batch = batch_size;
+    a.h_q = h_q;
+    a.h_kv = h_kv;
+    a.d = d;
+    a.page_size = page_size;
+    a.causal = causal > 0;
+    a.sm_scale = sm_scale;
+    return generic_attention(a, stream);
+  }
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "batch_prefill_paged_kv: bad shape";
@@ -1228,6 +1295,26 @@ static int tree_attn_ragged(const void* q, const int32_t* q_indptr, const void* 
                             const int32_t* mask, void* output, float* lse, int64_t rotary_mode, double rope_scale,
                             double rope_theta, double sm_scale, int32_t batch_size, int64_t total_q, int32_t h_q,
                             int32_t h_kv, int32_t d, const tvmkv_rope_scaling* scaling, void* stream) {
+  if (rotary_mode == 0 && d != 64 && d != 128 && d != 256) {  // the generic matrix-core kernel
+    GenericAttention a;
+    a.what = "batch_tree_attn";
+    a.q = q;
+    a.q_indptr = q_indptr;
+    a.k = k;
+    a.v = v;
+    a.kv_indptr = kv_indptr;
+    a.tree_indptr = mn_indptr;
+    a.tree_labels = mask;
+    a.out = output;
+    a.lse = lse;
+    a.total_q = total_q;
+    a.batch = batch_size;
+    a.h_q = h_q;
+    a.h_kv = h_kv;
+    a.d = d;
+    a.sm_scale = sm_scale;
+    return generic_attention(a, stream);
+  }
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0) << "batch_tree_attn: bad shape";
   if (batch_size == 0 || total_q == 0) return TVMKV_OK;
@@ -1293,6 +1380,30 @@ int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void*
                              const int32_t* tree_order_indptr, const int32_t* tree_order, int32_t batch_size,
                              int64_t total_q, int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
                              int32_t d, int32_t page_size, int32_t sliding_window, void* stream) {
+  if (rotary_mode == 0 && sliding_window == 0 && (!tuned_page_size(page_size) || (d != 64 && d != 128 && d != 256))) {
+    GenericAttention a;  // the generic matrix-core kernel
+    a.what = "tree_attn_paged_kv";
+    a.q = q;
+    a.q_indptr = q_indptr;
+    a.pages = pages;
+    a.page_indptr = page_indptr;
+    a.page_values = page_values;
+    a.last_page_len = length_info;
+    a.tree_indptr = tree_order_indptr;
+    a.tree_labels = tree_order;
+    a.out = output;
+    a.lse = lse;
+    a.total_q = total_q;
+    a.nnz_pages = nnz_pages;
+    a.num_pages = num_pages;
+    a.batch = batch_size;
+    a.h_q = h_q;
+    a.h_kv = h_kv;
+    a.d = d;
+    a.page_size = page_size;
+    a.sm_scale = sm_scale;
+    return generic_attention(a, stream);
+  }
   KV_API_BEGIN();
   KV_CHECK(batch_size >= 0 && total_q >= 0 && h_q > 0 && h_kv > 0 && h_q % h_kv == 0)
       << "tree_attn_paged_kv: bad shape";

@@ -12,6 +12,7 @@
 #include "common.h"
 #include "kv_bookkeeping.h"
 #include "runtime_support.h"
+#include "typed_kernels.h"
 
 namespace tvmkv {
 
@@ -65,7 +66,23 @@ class PagedKVCache {
     }
     KV_UNSUPPORTED(enable_kv_transfer)
         << "KV transfer (disaggregation) needs a second device and is not built in this library";
-    KV_UNSUPPORTED(dtype_bits != 16) << "only fp16 KV storage is built (got " << dtype_bits << " bits)";
+    KV_UNSUPPORTED(dtype_bits != 16 && dtype_bits != 32)
+        << "KV storage is built for float16 and float32 (got " << dtype_bits << " bits)";
+    elem_bits_ = dtype_bits;
+    // What the tuned fp16 kernels are not built for runs on the generic ones: float32 storage, pages other than
+    // 16 / 32 / 64 / 128 tokens, other head dims.  Those serve the plain cache.
+    bool has_mha_layer = false;
+    for (int64_t kind : attn_kinds_) has_mha_layer |= (kind != TVMKV_ATTN_MLA);
+    generic_ = has_mha_layer && (elem_bits_ == 32 || !tuned_page_size(static_cast<int>(page_size_)) ||
+                                 (!has_mla && !tuned_head_dim(static_cast<int>(qk_head_dim_))));
+    if (generic_) {
+      KV_UNSUPPORTED(has_mla) << "float32 storage, pages other than 16 / 32 / 64 / 128 tokens and other head dims are "
+                              << "not built for caches with MLA layers";
+      KV_UNSUPPORTED(support_sliding_window_ || has_layer_sliding || rope_mode_ == TVMKV_ROPE_INLINE)
+          << "float32 storage, pages other than 16 / 32 / 64 / 128 tokens and head dims other than 64 / 80 / 96 / 112 / "
+          << "128 / 256 are built for the plain cache: no sliding window, no RoPE inside the attention kernels";
+      KV_UNSUPPORTED(qk_head_dim_ != v_head_dim_) << "the generic kernels need equal qk and v head dims";
+    }
     KV_CHECK(static_cast<int64_t>(attn_kinds_.size()) >= layer_end)
         << "attn_kinds must cover every layer id up to " << layer_end;
     for (int64_t kind : attn_kinds_) {
@@ -166,6 +183,24 @@ class PagedKVCache {
     // A chunked-prefill step of a plain cache in two launches: k is rotated and the new k / v rows go
     // into their page slots (part 2 without q, part 3), then one pass over the cached and the new
     // tokens that reads the queries from qkv and rotates them itself (parts 2 and 5).
+    if (generic_) {
+      // split + RoPE (+ append when the rows may go in before attention), the attention kernels of the step, the
+      // append afterwards otherwise: the reference's flow (:1360-1401) on the typed and generic kernels
+      const bool early = s.append_before_attn || !support_sliding_window_;
+      const bool rotate = rope_normal || rope_ext_factors_ != nullptr;
+      Launch(typed_fused_rope(elem_bits_, qkv, Dev(s.q_rope_position_map), temp_q_, temp_k_, temp_v_, rotate, rope_ext_factors_,
+                              has_rope_scaling_ ? &rope_scaling_ : nullptr, early ? pages_[local_layer_id] : nullptr,
+                              early ? Dev(s.append_position_map) : nullptr, total_seq_length, num_qo_heads_, num_kv_heads_,
+                              qk_head_dim_, num_total_pages_, page_size_, rotary_scale_, rotary_theta_, compute_stream_));
+      AttentionInternal(layer_id, temp_q_, temp_k_, temp_v_, out, total_seq_length, sm_scale);
+      if (!early) {
+        Launch(tvmkv_kv_cache_transpose_append(pages_[local_layer_id], temp_k_, temp_v_, Dev(s.append_position_map),
+                                               total_seq_length, num_total_pages_, num_kv_heads_, page_size_,
+                                               CopyDim(), compute_stream_));
+      }
+      RecordComputeEvent();
+      return;
+    }
     if (has_rope_scaling_) {
       // the model's frequency variant lives in the split-rotary kernel only: q, k and v take the round trip
       const bool early = s.append_before_attn || !support_sliding_window_;
@@ -280,6 +315,13 @@ class PagedKVCache {
       return;
     }
     const int rotary = attn_kinds_[layer_id] == TVMKV_ATTN_MHA ? (rope_mode_ == TVMKV_ROPE_INLINE) : 0;
+    if (generic_ && attn_kinds_[layer_id] == TVMKV_ATTN_MHA) {
+      KV_CHECK(k_heads == num_kv_heads_ && qk_dim == qk_head_dim_ && v_dim == v_head_dim_)
+          << "self_attention: k/v shapes do not match the cache";
+      GenericRagged(q, k, v, o, lse, total_seq_length, sm_scale, /*tree=*/false);
+      RecordComputeEvent();
+      return;
+    }
     Launch(tvmkv_batch_prefill_ragged_kv_scaled(q, Dev(s.cur_append_lengths_indptr), k, v, Dev(s.cur_append_lengths_indptr),
                                                 Dev(s.q_rope_position_map), Dev(s.k_ragged_rope_pos_offset), o, lse,
                                                 /*causal=*/1, rotary, rotary_scale_, rotary_theta_, sm_scale,
@@ -321,7 +363,7 @@ class PagedKVCache {
   void MergeAttnOutputInplace(void* o_self, float* lse_self, const void* o_cross, const float* lse_cross, int64_t rows,
                               int heads, int dim) {
     RequireDevice();
-    Launch(tvmkv_merge_state_inplace(o_self, lse_self, o_cross, lse_cross, rows, heads, dim, compute_stream_));
+    Launch(typed_merge_state_inplace(elem_bits_, o_self, lse_self, o_cross, lse_cross, rows, heads, dim, compute_stream_));
   }
 
   // :1661-1667
@@ -351,7 +393,7 @@ class PagedKVCache {
         } else {
           KV_CHECK(kind == TVMKV_ATTN_MHA) << "Only MHA is supported for DebugGetKV";
           Launch(tvmkv_kv_cache_debug_get_kv(pages_[layer], map_dev, k_data, v_data, layer, map.size(), num_total_pages_,
-                                             num_kv_heads_, page_size_, qk_head_dim_, compute_stream_));
+                                             num_kv_heads_, page_size_, CopyDim(), compute_stream_));
         }
       }
       HIP_CHECK(hipStreamSynchronize(compute_stream_));
@@ -452,7 +494,7 @@ class PagedKVCache {
     const int64_t kind = attn_kinds_[local_layer + layer_id_begin_offset_];
     // GetKVCacheShape, attn_utils.h:74-87
     if (kind == TVMKV_ATTN_MLA) return num_total_pages_ * page_size_ * qk_head_dim_ * 2;
-    return num_total_pages_ * 2 * num_kv_heads_ * page_size_ * qk_head_dim_ * 2;
+    return num_total_pages_ * 2 * num_kv_heads_ * page_size_ * qk_head_dim_ * (elem_bits_ / 8);
   }
   // Device address of an array of the current step (nullptr when the step does not have it).
   const int32_t* Dev(const AuxSpan& span) const {
@@ -470,11 +512,11 @@ class PagedKVCache {
       bool has_mha = false;
       for (int64_t kind : attn_kinds_) has_mha |= (kind != TVMKV_ATTN_MLA);
       if (has_mha) {
-        HIP_CHECK(hipMalloc(&temp_q_, prefill_chunk_size_ * num_qo_heads_ * qk_head_dim_ * 2));
-        HIP_CHECK(hipMalloc(&temp_k_, prefill_chunk_size_ * num_kv_heads_ * qk_head_dim_ * 2));
-        HIP_CHECK(hipMalloc(&temp_v_, prefill_chunk_size_ * num_kv_heads_ * v_head_dim_ * 2));
+        HIP_CHECK(hipMalloc(&temp_q_, prefill_chunk_size_ * num_qo_heads_ * qk_head_dim_ * (elem_bits_ / 8)));
+        HIP_CHECK(hipMalloc(&temp_k_, prefill_chunk_size_ * num_kv_heads_ * qk_head_dim_ * (elem_bits_ / 8)));
+        HIP_CHECK(hipMalloc(&temp_v_, prefill_chunk_size_ * num_kv_heads_ * v_head_dim_ * (elem_bits_ / 8)));
       }
-      HIP_CHECK(hipMalloc(&temp_out_, prefill_chunk_size_ * num_qo_heads_ * v_head_dim_ * 2));
+      HIP_CHECK(hipMalloc(&temp_out_, prefill_chunk_size_ * num_qo_heads_ * v_head_dim_ * (elem_bits_ / 8)));
       HIP_CHECK(hipMalloc(&temp_lse_, prefill_chunk_size_ * num_qo_heads_ * sizeof(float)));
       HIP_CHECK(hipMalloc(&merged_lse_, prefill_chunk_size_ * num_qo_heads_ * sizeof(float)));
       aux_capacity_ = book_->RequiredCapacity();
@@ -578,7 +620,7 @@ class PagedKVCache {
                                             qk_head_dim_, copy_stream_));
         } else {
           Launch(tvmkv_copy_single_page(pages_[layer], src, tgt, copy_length, num_total_pages_, num_kv_heads_,
-                                        page_size_, qk_head_dim_, copy_stream_));
+                                        page_size_, CopyDim(), copy_stream_));
         }
       }
     }
@@ -613,7 +655,7 @@ class PagedKVCache {
     commit_staging_used_ = true;
     for (int64_t layer = 0; layer < num_layers_; ++layer) {
       Launch(tvmkv_compact_kv_copy(pages_[layer], device, device + pos_begin, batch_size, total_copy_length,
-                                   num_total_pages_, num_kv_heads_, page_size_, qk_head_dim_, copy_stream_));
+                                   num_total_pages_, num_kv_heads_, page_size_, CopyDim(), copy_stream_));
     }
     // The next step's first kernel waits for the copy stream (paged_kv_cache.cc:767-769).
     copy_stream_has_work_ = true;
@@ -625,15 +667,15 @@ class PagedKVCache {
   // whose keys are stored rotated (or not rotated at all) with the default frequencies.
   bool FusedDecodeStepApplies(int64_t layer_id) const {
     const StepLayout& s = book_->step();
-    return s.append_before_attn && s.is_decode_request && s.num_depths == 1 && s.is_chain[0] && s.use_decode_kernel[0] &&
-           !support_sliding_window_ && attn_kinds_[layer_id] == TVMKV_ATTN_MHA && rope_mode_ != TVMKV_ROPE_INLINE &&
+    return !generic_ && s.append_before_attn && s.is_decode_request && s.num_depths == 1 && s.is_chain[0] &&
+           s.use_decode_kernel[0] && !support_sliding_window_ && attn_kinds_[layer_id] == TVMKV_ATTN_MHA && rope_mode_ != TVMKV_ROPE_INLINE &&
            !has_rope_scaling_ && qk_head_dim_ == v_head_dim_ &&
            (qk_head_dim_ == 64 || qk_head_dim_ == 128 || qk_head_dim_ == 256) && option(kOptNoFusedDecodeStep) == 0;
   }
 
   bool OnePassPrefillApplies(int64_t layer_id) const {
     const StepLayout& s = book_->step();
-    return !s.append_before_attn && s.num_depths == 1 && s.is_chain[0] && !s.use_decode_kernel[0] &&
+    return !generic_ && !s.append_before_attn && s.num_depths == 1 && s.is_chain[0] && !s.use_decode_kernel[0] &&
            s.page_indices[0].size > 0 && !support_sliding_window_ && attn_kinds_[layer_id] == TVMKV_ATTN_MHA &&
            rope_mode_ != TVMKV_ROPE_INLINE && qk_head_dim_ == v_head_dim_ && (qk_head_dim_ == 64 || qk_head_dim_ == 128);
   }
@@ -670,6 +712,13 @@ class PagedKVCache {
                            double sm_scale) {
     const StepLayout& s = book_->step();
     const int rope_inline = rope_mode_ == TVMKV_ROPE_INLINE;
+    if (generic_) {
+      if (!s.is_chain[0]) {
+        KV_CHECK(s.tree_attn_mask[0].present() && s.tree_attn_mn_indptr[0].present()) << "token-tree mask is not on the device";
+      }
+      GenericRagged(q, k, v, o, lse, total_seq_length, sm_scale, /*tree=*/!s.is_chain[0]);
+      return;
+    }
     if (s.is_chain[0]) {
       Launch(tvmkv_batch_prefill_ragged_kv_scaled(q, Dev(s.cur_append_lengths_indptr), k, v, Dev(s.cur_append_lengths_indptr),
                                                   Dev(s.q_rope_position_map), Dev(s.k_ragged_rope_pos_offset), o, lse,
@@ -686,6 +735,37 @@ class PagedKVCache {
                                           total_seq_length, num_qo_heads_, num_kv_heads_, qk_head_dim_, InlineScaling(),
                                           compute_stream_));
     }
+  }
+
+  // feature extent of a K/V row for the copy kernels, which move rows as fp16 elements whatever they hold
+  int32_t CopyDim() const { return copy_dim(elem_bits_, static_cast<int32_t>(qk_head_dim_)); }
+
+  // causal self-attention over the step's new tokens (or the token-tree mask) on the generic kernel
+  void GenericRagged(const void* q, const void* k, const void* v, void* o, float* lse, int64_t total_seq_length,
+                     double sm_scale, bool tree) {
+    const StepLayout& s = book_->step();
+    GenericAttention a;
+    a.what = "self attention";
+    a.elem_bits = elem_bits_;
+    a.q = q;
+    a.q_indptr = Dev(s.cur_append_lengths_indptr);
+    a.k = k;
+    a.v = v;
+    a.kv_indptr = Dev(s.cur_append_lengths_indptr);
+    if (tree) {
+      a.tree_indptr = Dev(s.tree_attn_mn_indptr[0]);
+      a.tree_labels = Dev(s.tree_attn_mask[0]);
+    }
+    a.out = o;
+    a.lse = lse;
+    a.total_q = total_seq_length;
+    a.batch = book_->batch_size();
+    a.h_q = static_cast<int32_t>(num_qo_heads_);
+    a.h_kv = static_cast<int32_t>(num_kv_heads_);
+    a.d = static_cast<int32_t>(qk_head_dim_);
+    a.causal = 1;
+    a.sm_scale = sm_scale;
+    Launch(generic_attention(a, compute_stream_));
   }
 
   // :2216-2299
@@ -712,7 +792,36 @@ class PagedKVCache {
       const int32_t* q_pos = Dev(s.q_rope_position_map);
       const int64_t entries = s.qo_indptr[d].size - 1;
       const int64_t nnz_pages = page_indices_span.size;
-      if (s.append_before_attn && !s.is_chain[d]) {
+      if (generic_) {
+        GenericAttention a;
+        a.what = "cross attention";
+        a.elem_bits = elem_bits_;
+        a.q = q;
+        a.q_indptr = qo_indptr;
+        a.pages = pages_[local_layer_id];
+        a.page_indptr = page_indptr;
+        a.page_values = page_indices;
+        a.last_page_len = length_info;
+        if (s.append_before_attn && !s.is_chain[d]) {
+          KV_CHECK(s.tree_attn_mask[d].present() && s.tree_attn_mn_indptr[d].present())
+              << "token-tree mask is not on the device";
+          a.tree_indptr = Dev(s.tree_attn_mn_indptr[d]);
+          a.tree_labels = Dev(s.tree_attn_mask[d]);
+        }
+        a.out = attn_output;
+        a.lse = attn_lse;
+        a.total_q = total_seq_length;
+        a.nnz_pages = nnz_pages;
+        a.num_pages = num_total_pages_;
+        a.batch = static_cast<int32_t>(entries);
+        a.h_q = static_cast<int32_t>(num_qo_heads_);
+        a.h_kv = static_cast<int32_t>(num_kv_heads_);
+        a.d = static_cast<int32_t>(qk_head_dim_);
+        a.page_size = static_cast<int32_t>(page_size_);
+        a.causal = causal;
+        a.sm_scale = sm_scale;
+        Launch(generic_attention(a, compute_stream_));
+      } else if (s.append_before_attn && !s.is_chain[d]) {
         KV_CHECK(s.tree_attn_mask[d].present() && s.tree_attn_mn_indptr[d].present())
             << "token-tree mask is not on the device";
         Launch(tvmkv_tree_attn_paged_kv(q, qo_indptr, pages_[local_layer_id], page_indptr, page_indices, length_info,
@@ -746,8 +855,8 @@ class PagedKVCache {
                                                    InlineScaling(), compute_stream_));
       }
       if (!is_first_kernel) {
-        Launch(tvmkv_merge_state_inplace(o, lse, temp_out_, temp_lse_, total_seq_length, num_qo_heads_, v_head_dim_,
-                                         compute_stream_));
+        Launch(typed_merge_state_inplace(elem_bits_, o, lse, temp_out_, temp_lse_, total_seq_length, num_qo_heads_,
+                                         v_head_dim_, compute_stream_));
       } else {
         is_first_kernel = false;
       }
@@ -811,6 +920,8 @@ class PagedKVCache {
   int64_t num_qo_heads_, num_kv_heads_, qk_head_dim_, v_head_dim_;
   int64_t num_total_pages_ = 0, prefill_chunk_size_, reserved_num_seqs_ = 0;
   bool support_sliding_window_ = false;
+  int elem_bits_ = 16;    // storage type of the MHA layers: 16 (fp16) or 32 (float32)
+  bool generic_ = false;  // the MHA layers run on the typed / generic kernels (typed_kernels.h)
   int64_t layer_sliding_window_size_ = 1024;
   std::vector<int64_t> attn_kinds_;
   int rope_mode_ = TVMKV_ROPE_NORMAL;

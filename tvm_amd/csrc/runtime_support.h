@@ -40,7 +40,7 @@ struct ScratchLease {
   uint32_t epoch;   // never 0
   std::unique_lock<std::mutex> lock;
 };
-enum ScratchUser { kScratchDecode = 0, kScratchMla = 1, kScratchPrefill = 2 };
+enum ScratchUser { kScratchDecode = 0, kScratchMla = 1, kScratchPrefill = 2, kScratchGeneric = 3 };
 ScratchLease lease_scratch(ScratchUser user, hipStream_t stream, size_t bytes, size_t counter_bytes);
 // Frees the buffers of (current device, stream) after synchronising the stream; a buffer whose address
 // a graph under capture has recorded is kept until the process ends instead.

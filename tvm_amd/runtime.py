@@ -48,11 +48,23 @@ def _require_contiguous(*tensors):
             raise KVError(-1, "tensors handed to the KV cache must be contiguous")
 
 
+def _require_storage(cache, *tensors):
+    """q / k / v / output tensors have the cache's storage type (the reference checks the same,
+    src/runtime/vm/paged_kv_cache.cc:1318-1320): the library sees pointers only."""
+    for t in tensors:
+        element_size = getattr(t, "element_size", None)
+        if t is None or element_size is None:
+            continue  # not a torch tensor: the caller vouches for what the pointer holds
+        if not t.is_floating_point() or element_size() * 8 != cache.dtype_bits:
+            raise KVError(-1, f"the KV cache stores float{cache.dtype_bits}; got a tensor of {t.dtype}")
+
+
 class PagedAttentionKVCache:
     """Handle of a cache object created by ``vm.builtin.paged_attention_kv_cache_create``."""
 
-    def __init__(self, handle, num_layers, num_kv_heads, qk_head_dim, v_head_dim):
+    def __init__(self, handle, num_layers, num_kv_heads, qk_head_dim, v_head_dim, dtype_bits=16):
         self._handle = handle
+        self.dtype_bits = dtype_bits  # storage type of the K/V pages and of every q / k / v / output tensor
         self.num_layers = num_layers
         self.num_kv_heads = num_kv_heads
         self.qk_head_dim = qk_head_dim
@@ -154,10 +166,10 @@ def _dtype_bits(init):
     if dtype is None:
         return 16
     name = str(dtype)
-    if "float16" in name or "half" in name:
-        return 16
     if "bfloat16" in name:
         return -16  # rejected by the library with a clear message
+    if "float16" in name or "half" in name:
+        return 16
     if "float32" in name:
         return 32
     return 0
@@ -183,7 +195,7 @@ def _create(cache_config, layer_indptr, num_qo_heads, num_kv_heads, qk_head_dim,
                                    int(rope_mode), float(rope_scale), float(rope_theta), _dtype_bits(init),
                                    _device_index(init), ctypes.byref(out)))
     cache = PagedAttentionKVCache(out.value, layer_indptr[-1] - layer_indptr[0], num_kv_heads, qk_head_dim,
-                                  v_head_dim)
+                                  v_head_dim, _dtype_bits(init))
     if rope_scaling:
         from .dlpack import RopeScaling
         scaling = RopeScaling.from_dict(rope_scaling)
@@ -214,12 +226,14 @@ def _int_query(fn_name):
 
 def _attention_with_fused_qkv(cache, layer_id, sm_scale, qkv, out):
     _require_contiguous(qkv, out)
+    _require_storage(cache, qkv, out)
     check(lib().tvmkv_attention_kv_cache_attention_with_fused_qkv(
         cache.handle, layer_id, float(sm_scale), _ptr(qkv), qkv.shape[0], _ptr(out), out.shape[0]))
 
 
 def _self_attention(cache, layer_id, sm_scale, q, k, v, o, lse):
     _require_contiguous(q, k, v, o, lse)
+    _require_storage(cache, q, k, v, o)
     if not (q.shape[0] == k.shape[0] == v.shape[0] == o.shape[0]):
         raise KVError(-1, "self_attention: q, k, v, o must have the same number of rows")
     check(lib().tvmkv_attention_kv_cache_self_attention(
@@ -229,6 +243,7 @@ def _self_attention(cache, layer_id, sm_scale, q, k, v, o, lse):
 
 def _cross_attention(cache, layer_id, sm_scale, q, o, lse):
     _require_contiguous(q, o, lse)
+    _require_storage(cache, q, o)
     if q.shape[0] != o.shape[0]:
         raise KVError(-1, "cross_attention: q and o must have the same number of rows")
     check(lib().tvmkv_attention_kv_cache_cross_attention(
@@ -237,6 +252,7 @@ def _cross_attention(cache, layer_id, sm_scale, q, o, lse):
 
 def _attention_with_shared_kv(cache, source_layer_id, sm_scale, q, current_k, current_v, o):
     _require_contiguous(q, current_k, current_v, o)
+    _require_storage(cache, q, current_k, current_v, o)
     if not (q.shape[0] == current_k.shape[0] == current_v.shape[0] == o.shape[0]):
         raise KVError(-1, "attention_with_shared_kv: q, current_k, current_v, o must have the same number of rows")
     if current_k.shape[1] != cache.num_kv_heads or current_k.shape[2] != cache.qk_head_dim or \
@@ -249,12 +265,14 @@ def _attention_with_shared_kv(cache, source_layer_id, sm_scale, q, current_k, cu
 
 def _append_mla_kv(cache, layer_id, kv):
     _require_contiguous(kv)
+    _require_storage(cache, kv)
     check(lib().tvmkv_attention_kv_cache_append_mla_kv(cache.handle, layer_id, _ptr(kv), kv.shape[0]))
     return cache
 
 
 def _merge_attn_output_inplace(cache, o_self, lse_self, o_cross, lse_cross):
     _require_contiguous(o_self, lse_self, o_cross, lse_cross)
+    _require_storage(cache, o_self, o_cross)
     check(lib().tvmkv_attention_kv_cache_merge_attn_output_inplace(
         cache.handle, _ptr(o_self), _ptr(lse_self), _ptr(o_cross), _ptr(lse_cross), o_self.shape[0],
         o_self.shape[1], o_self.shape[2]))
@@ -263,6 +281,7 @@ def _merge_attn_output_inplace(cache, o_self, lse_self, o_cross, lse_cross):
 
 def _debug_get_kv(cache, seq_id, start_pos, end_pos, k_data, v_data):
     _require_contiguous(k_data, v_data)
+    _require_storage(cache, k_data, v_data)
     expect = (cache.num_layers, end_pos - start_pos, cache.num_kv_heads, cache.qk_head_dim)
     for t in (k_data, v_data):
         if tuple(t.shape) != expect:
@@ -274,6 +293,7 @@ def _debug_get_kv(cache, seq_id, start_pos, end_pos, k_data, v_data):
 
 def _debug_get_kv_mla(cache, seq_id, start_pos, end_pos, kv_data):
     _require_contiguous(kv_data)
+    _require_storage(cache, kv_data)
     expect = (cache.num_layers, end_pos - start_pos, cache.qk_head_dim)
     if tuple(kv_data.shape) != expect:
         raise KVError(-1, f"DebugGetKV expects the kv_data in layout (num_layers, seq_length, qk_head_dim) = {expect}")
