@@ -750,6 +750,54 @@ def extras(torch, K, dev):
                 "prefill_ms": round(ms_p, 4), "prefill_tflops": round(fl_ / ms_p / 1e9, 1),
                 "prefill_frac_of_mfma_peak": round(fl_ / ms_p / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
 
+    # ---- the generic kernels: float32 storage, pages that are not a power of two ---------------------------
+    def generic_leg():
+        from tvm_amd import dlpack as dl
+        rng_ = np.random.default_rng(1)
+        ctx_ = rng_.integers(1024, 8192, size=64, endpoint=True)
+        res = {"workload": "what the tuned fp16 kernels are not built for, on the generic matrix-core kernels (float32 "
+                           "arithmetic, v_mfma_f32_16x16x4_f32, K/V rows straight from their pages): decode of 64 seqs ctx "
+                           "U[1024,8192] Hq32/Hkv8/D128 with float32 storage (page 16) and with fp16 pages of 24 tokens; "
+                           "causal self-attention of 4 x 2048 tokens with float32 storage"}
+        for name, tdt, ps_ in (("decode_float32_storage", torch.float32, 16), ("decode_fp16_pages_of_24_tokens", torch.float16, 24)):
+            npg_ = (ctx_ + ps_ - 1) // ps_
+            ip_ = np.concatenate([[0], np.cumsum(npg_)])
+            pool_ = int(ip_[-1]) + 8
+            perm_ = rng_.permutation(pool_).astype(np.int32)
+            pages_ = torch.empty((pool_, 2, HKV, ps_, D), dtype=tdt, device=dev)
+            for lo_ in range(0, pool_, 4096):
+                pages_[lo_:lo_ + 4096].normal_()
+            q_ = torch.randn((64, HQ, D), device=dev).to(tdt)
+            o_ = torch.empty_like(q_)
+            l_ = torch.empty((64, HQ), dtype=torch.float32, device=dev)
+            z_ = torch.zeros(64, dtype=torch.int32, device=dev)
+            ints = [i32(ip_), i32(perm_[:ip_[-1]]), i32((ctx_ - 1) % ps_ + 1)]
+            a_ = (dl.tensor(q_), dl.tensor(pages_), dl.tensor(ints[0]), dl.tensor(ints[1]), dl.tensor(ints[2]), dl.tensor(z_),
+                  dl.tensor(z_), dl.tensor(o_), dl.tensor(l_), 0, 1.0, 1e4, D ** -0.5)
+            dl.call("batch_decode_paged_kv", *a_)
+            ms_ = time_region(torch, lambda i: dl.call("batch_decode_paged_kv", *a_), 20, SETTLE_S)
+            nb_ = float(ctx_.sum()) * 2 * HKV * D * q_.element_size() + 2 * 64 * HQ * D * q_.element_size()
+            res[name] = {"ms": round(ms_, 4), "GBps": round(nb_ / ms_ / 1e6, 1),
+                         "frac_of_hbm_peak": round(nb_ / ms_ / 1e6 / HBM_PEAK_GBPS, 4)}
+            del pages_
+        n_, c_ = 4, 2048
+        q_, k_, v_ = (torch.randn((n_ * c_, h_, D), device=dev) for h_ in (HQ, HKV, HKV))
+        o_ = torch.empty_like(q_)
+        l_ = torch.empty((n_ * c_, HQ), dtype=torch.float32, device=dev)
+        ind_ = i32(np.arange(n_ + 1) * c_)
+        zq_, zb_ = torch.zeros(n_ * c_, dtype=torch.int32, device=dev), torch.zeros(n_, dtype=torch.int32, device=dev)
+        a_ = (dl.tensor(q_), dl.tensor(ind_), dl.tensor(k_), dl.tensor(v_), dl.tensor(ind_), dl.tensor(zq_), dl.tensor(zb_),
+              dl.tensor(o_), dl.tensor(l_), 1, 0, 1.0, 1e4, D ** -0.5)
+        dl.call("batch_prefill_ragged_kv", *a_)
+        ms_ = time_region(torch, lambda i: dl.call("batch_prefill_ragged_kv", *a_), 5, SETTLE_S)
+        fl_ = 4.0 * HQ * D * n_ * c_ * (c_ + 1) / 2
+        res["causal_prefill_float32_storage"] = {"ms": round(ms_, 4), "tflops": round(fl_ / ms_ / 1e9, 1),
+                                                 "frac_of_fp32_mfma_peak": round(fl_ / ms_ / 1e9 / 157.3, 4)}
+        return res
+
+    out["generic_kernels"] = generic_leg()
+    torch.cuda.empty_cache()
+
     out["other_head_dims"] = {
         "workload": "decode of 64 seqs ctx U[1024,8192] (configs[1]'s lengths) and the one-pass chunked-prefill kernel on "
                     "configs[2]'s 8 sequences, page 16, at the head dims beside 128 (query / kv heads)",

@@ -15,6 +15,19 @@
  *      1027-1035) must already have that offset added.  `stream` is a hipStream_t (NULL = the
  *      null stream).  Launchers are asynchronous and never synchronise the device.
  *
+ *      Shapes.  The tuned kernels are fp16 with pages of 16 / 32 / 64 / 128 tokens and head dims
+ *      64 / 80 / 96 / 112 / 128 / 256 (the comment of each launcher says what it has of them).
+ *      A plain call (rotary_mode 0, one-row length_info) with another page size or head dim is
+ *      handed to generic matrix-core kernels (float32 arithmetic, v_mfma_f32_16x16x4_f32; any
+ *      page size, head dims that are a multiple of 8 up to 256): the reference's kernel
+ *      factories take both as free parameters (_decode_kernels.py:49,181;
+ *      _prefill_kernels.py:54-60,217-225).  The same kernels serve float32 K/V storage, which the
+ *      reference's tests also run (tests/python/relax/
+ *      test_runtime_builtin_paged_attention_kv_cache_cpu.py:269-276): float32 tensors are taken
+ *      by the tensor-level entry points of tvmkv_dlpack.h, where the dtype travels in the
+ *      tensor, and by a cache object created with dtype_bits 32; the pointer-level launchers of
+ *      this file are fp16.
+ *
  *  (2) CACHE OBJECT.  `tvmkv_cache_*` / `tvmkv_kv_state_*` / `tvmkv_attention_kv_cache_*`:
  *      the host-side page pool, block tree and per-step auxiliary arrays, with the verbs and
  *      error behaviour of the reference's global functions `vm.builtin.kv_state_*` and
@@ -474,7 +487,11 @@ typedef struct tvmkv_cache tvmkv_cache;
  *                  support_sliding_window(, layer_sliding_window_size)]   (n_config 5 or 6)
  *   layer_indptr  [begin, end] layer range owned by this cache (one group: {0, num_layers})
  *   attn_kinds    one TVMKV_ATTN_* per global layer id
- *   dtype_bits    16 (fp16 storage; the only one built)
+ *   dtype_bits    16 (fp16 storage) or 32 (float32 storage: every q / k / v / output tensor handed to the
+ *                 verbs is float32 then).  float32 storage, page sizes other than 16 / 32 / 64 / 128 and
+ *                 head dims other than 64 / 80 / 96 / 112 / 128 / 256 (multiples of 8, of 4 for float32, up
+ *                 to 256) run on the generic kernels and are built for the plain cache: no sliding
+ *                 window, no RoPE inside the attention kernels, no MLA layers (TVMKV_EUNSUPPORTED)
  *   device_id     HIP device ordinal, or -1 for a HOST-ONLY cache: page-pool bookkeeping and
  *                 auxiliary arrays work, anything that touches device memory returns
  *                 TVMKV_ENODEVICE. */
@@ -489,8 +506,8 @@ void tvmkv_cache_destroy(tvmkv_cache* cache);
  * created with, paged_kv_cache.cc:2583) and, for longrope, the factor tensor the reference's create call
  * takes as `rope_ext_factors` (device memory, head_dim float32, kept by reference: it must outlive the
  * cache).  scaling NULL or rope_type DEFAULT: back to plain frequencies.  Caches that rotate inside the
- * attention kernels (RoPE mode inline, i.e. sliding-window caches) only have the plain frequencies:
- * TVMKV_EUNSUPPORTED. */
+ * attention kernels (RoPE mode inline, i.e. sliding-window caches) hand the variant to those kernels (the
+ * *_scaled launchers); they take no factor tensor. */
 int tvmkv_cache_set_rope_scaling(tvmkv_cache* cache, const tvmkv_rope_scaling* scaling,
                                  const float* rope_ext_factors);
 /* Stream on which the cache enqueues kernels (the reference uses the device's current stream,

@@ -16,6 +16,12 @@
  * type and id (all tensors on one ROCm device), dtype, ndim, compact strides, consistent shapes and
  * alignment of `data + byte_offset`; a mismatch returns TVMKV_EINVAL and tvmkv_last_error() names the
  * argument.  Return codes as in tvmkv.h.
+ *
+ * Storage type.  q / k / v / pages / out of the MHA slots (13, 15-21, 23-27) are float16 or float32, the
+ * same in every tensor of a call (the reference builds each kernel for one storage dtype); lse and the
+ * RoPE factor tensor are float32, index arrays int32.  float32 storage runs on the generic kernels
+ * (tvmkv.h, "Shapes"): plain calls only -- rotary_mode 1 and the (3, batch) length_info return
+ * TVMKV_EUNSUPPORTED.  The MLA slots (14, 22) are float16.
  */
 #ifndef TVMKV_DLPACK_H_
 #define TVMKV_DLPACK_H_

@@ -291,3 +291,111 @@ def test_fp16_pages_and_head_dims_outside_the_tuned_set(hq, hkv, d, ps):
     assert np.array_equal(host(gv), ev)
     assert_close(host(gq), eq, atol=2e-3, rtol=2e-3, what="rope q")
     assert_close(host(gk), ek, atol=2e-3, rtol=2e-3, what="rope k")
+
+
+def _random_generic_case(case):
+    """One random launch of the generic kernel: storage type, head shape, head dim, page size, sequence lengths
+    and the form of the call (decode, paged prefill with either mask, ragged prefill, both token-tree forms) all
+    drawn from the seed; float32 storage goes through the tensor-level boundary, fp16 through the launchers."""
+    rng = np.random.default_rng(88000 + case)
+    dtype = F32 if rng.random() < 0.5 else F16
+    hq, hkv = [(8, 2), (4, 4), (32, 8), (12, 1), (20, 2), (48, 2)][rng.integers(6)]
+    step = 4 if dtype == F32 else 8
+    d = int(rng.integers(2, 256 // step + 1)) * step
+    if dtype == F16 and d in (64, 80, 96, 112, 128, 256):
+        ps = int(rng.choice([1, 3, 5, 7, 8, 12, 24, 40, 48, 100]))   # a page size the tuned kernels do not have
+    else:
+        ps = int(rng.choice([1, 3, 5, 8, 12, 16, 24, 32, 48, 64, 100]))
+    kind = ["decode", "paged", "paged_causal", "ragged", "tree_ragged", "tree_paged"][rng.integers(6)]
+    b = int(rng.integers(1, 9))
+    edge = [0, 1, 15, 16, 17, 31, 32, 33, ps, ps + 1, 2 * ps - 1, 255, 256, 257]
+    length = lambda hi: int(rng.choice(edge)) if rng.random() < 0.4 else int(rng.integers(0, hi))
+    torch_dtype = torch.float32 if dtype == F32 else torch.float16
+    what = f"case {case}: {kind} {np.dtype(dtype).name} heads {hq}/{hkv} d {d} page {ps}"
+
+    def outputs(n):
+        return (torch.full((n, hq, d), 7.0, dtype=torch_dtype, device=DEV), torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV))
+
+    sm = d ** -0.5
+    if kind in ("decode", "paged", "paged_causal", "tree_paged"):
+        causal = int(kind == "paged_causal")
+        if kind == "tree_paged":
+            trees = [random_forest(rng, int(rng.integers(1, 40))) for _ in range(b)]
+            new_lens = [int(rng.integers(1, len(t) + 1)) for t in trees]
+            kv_lens = [length(400) + len(t) for t in trees]
+            q_lens = new_lens
+        else:
+            kv_lens = [length(1500) for _ in range(b)]
+            q_lens = [1] * b if kind == "decode" else [max(1, length(150)) for _ in range(b)]
+            if causal:
+                kv_lens = [max(k, ql) for k, ql in zip(kv_lens, q_lens)]
+        pages, indptr, values, last, qindptr, q = paged_case(rng, kv_lens, q_lens, hq, hkv, d, ps, dtype)
+        n = len(q)
+        zb, zq = np.zeros(b, np.int32), np.zeros(n, np.int32)
+        eo, el = np.zeros((n, hq, d), dtype), np.zeros((n, hq), F32)
+        go, gl = outputs(n)
+        if kind == "tree_paged":
+            tindptr = np.concatenate([[0], np.cumsum([len(t) for t in trees])]).astype(np.int32)
+            labels = np.concatenate([tree_order(t) for t in trees]).astype(np.int32)
+            ok.tree_attn_paged(q, qindptr, pages, indptr, values, last, zb, zq, eo, el, 0, 1.0, 1e4, sm, tindptr, labels)
+            if dtype == F32:
+                dl.call("tree_attn_paged_kv", T(q)[1], TI(qindptr), T(pages)[1], TI(indptr), TI(values), TI(last), TI(zb), TI(zq),
+                        dl.tensor(go), dl.tensor(gl), 0, 1.0, 1e4, sm, TI(tindptr), TI(labels.reshape(-1)))
+            else:
+                K.tree_attn_paged_kv(dev(q), i32(qindptr), dev(pages), i32(indptr), i32(values), i32(last), i32(zb), i32(zq), go, gl,
+                                     0, 1.0, 1e4, sm, i32(tindptr), i32(labels))
+        elif kind == "decode":
+            ok.decode(q, pages, indptr, values, last, zb, zb, eo, el, 0, 1.0, 1e4, sm)
+            if dtype == F32:
+                dl.call("batch_decode_paged_kv", T(q)[1], T(pages)[1], TI(indptr), TI(values), TI(last), TI(zb), TI(zb),
+                        dl.tensor(go), dl.tensor(gl), 0, 1.0, 1e4, sm)
+            else:
+                K.batch_decode_paged_kv(dev(q), dev(pages), i32(indptr), i32(values), i32(last), i32(zb), i32(zb), go, gl, 0, 1.0,
+                                        1e4, sm)
+        else:
+            ok.prefill_paged(q, qindptr, pages, indptr, values, last, zb, zq, eo, el, causal, 0, 1.0, 1e4, sm)
+            if dtype == F32:
+                dl.call("batch_prefill_paged_kv", T(q)[1], TI(qindptr), T(pages)[1], TI(indptr), TI(values), TI(last), TI(zb),
+                        TI(zq), dl.tensor(go), dl.tensor(gl), causal, 0, 1.0, 1e4, sm, 0)
+            else:
+                K.batch_prefill_paged_kv(dev(q), i32(qindptr), dev(pages), i32(indptr), i32(values), i32(last), i32(zb), i32(zq),
+                                         go, gl, causal, 0, 1.0, 1e4, sm)
+    else:
+        if kind == "tree_ragged":
+            trees = [random_forest(rng, int(rng.integers(1, 70))) for _ in range(b)]
+            lens = [len(t) for t in trees]
+        else:
+            lens = [max(1, length(300)) for _ in range(b)]
+        n = sum(lens)
+        ind = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        q, k, v = (rng.standard_normal((n, h, d)).astype(dtype) for h in (hq, hkv, hkv))
+        zq, zb = np.zeros(n, np.int32), np.zeros(b, np.int32)
+        eo, el = np.zeros((n, hq, d), dtype), np.zeros((n, hq), F32)
+        go, gl = outputs(n)
+        if dtype == F16 and d in (64, 128, 256) or (dtype == F16 and kind == "ragged" and d in (80, 96, 112)):
+            return  # the tuned kernels' shapes: covered by their own sweep
+        if kind == "tree_ragged":
+            mask = np.concatenate([tree_order(t) for t in trees]).astype(np.int32)
+            ok.tree_attn_ragged(q, ind, k, v, ind, zq, ind, mask, eo, el, 0, 1.0, 1e4, sm)
+            if dtype == F32:
+                dl.call("batch_tree_attn", T(q)[1], TI(ind), T(k)[1], T(v)[1], TI(ind), TI(zq), TI(ind), TI(mask.reshape(-1)),
+                        dl.tensor(go), dl.tensor(gl), 0, 1.0, 1e4, sm)
+            else:
+                K.batch_tree_attn(dev(q), i32(ind), dev(k), dev(v), i32(ind), i32(zq), i32(ind), i32(mask), go, gl, 0, 1.0, 1e4, sm)
+        else:
+            causal = int(rng.integers(2))
+            ok.prefill_ragged(q, ind, k, v, ind, zq, zb, eo, el, causal, 0, 1.0, 1e4, sm)
+            if dtype == F32:
+                dl.call("batch_prefill_ragged_kv", T(q)[1], TI(ind), T(k)[1], T(v)[1], TI(ind), TI(zq), TI(zb), dl.tensor(go),
+                        dl.tensor(gl), causal, 0, 1.0, 1e4, sm)
+            else:
+                K.batch_prefill_ragged_kv(dev(q), i32(ind), dev(k), dev(v), i32(ind), i32(zq), i32(zb), go, gl, causal, 0, 1.0,
+                                          1e4, sm)
+    assert_close(host(go), eo, what=what + " out", **tol(dtype))
+    assert_close(host(gl), el, atol=2e-3 if dtype == F16 else 3e-4, rtol=1e-4, what=what + " lse")
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_generic_kernel_cases(block):
+    for case in range(block * 20, block * 20 + 20):
+        _random_generic_case(case)

@@ -11,10 +11,15 @@
 // workgroups (partial states in scratch memory, merged by a second kernel).
 //
 // Matrix operand layout (v_mfma_f32_16x16x4_f32): lane = 16 * k + i holds A[i][k] and B[k][i]; the result
-// register r of lane 16 * g + j is C[4 g + r][j].  The contraction index is a free choice as long as A and
-// B agree, so for S^T = K Q^T lane (i, g) loads features 16 s + 4 g .. + 3 of key i as one 16-byte piece and
-// feeds one component to each of four instructions; for O^T += V^T P the four keys 4 g + m of lane group g
-// are the contraction slots, which is the order in which lane (j, g) holds the probabilities of row j.
+// register r of lane 16 * g + j is C[4 g + r][j].  Every load of a K / V / q row is one 16-byte piece (4 floats,
+// 8 halfs), which the freedom in numbering the contraction index and the output features allows:
+//  * S^T = K Q^T: the contraction runs over the features in the order that suits the loads -- lane (i, g) loads
+//    piece 4 s + g of key i (of query row i for the B operand) and feeds its elements to consecutive
+//    instructions, so A and B agree by construction;
+//  * O^T += V^T P: the four keys 4 g + m of lane group g are the contraction slots, which is the order in which
+//    lane (j, g) already holds the probabilities of row j; output "block" fb, row i of the product is feature
+//    i * KS + fb, so lane (i, g) reads KS consecutive features of a key (the 16 lanes of a group read a whole
+//    row) and lane (j, g) ends up with runs of KS consecutive output features.
 #include <algorithm>
 
 #include "kernels_common.cuh"
@@ -48,36 +53,60 @@ struct GAttn {
 constexpr float kMasked = -1.0e30f;  // a masked score; exp2 of it is 0 against any running maximum
 constexpr float kNoKeys = -1.0e30f;  // the log-sum-exp of a share that saw no key
 
-template <typename T>
-__device__ __forceinline__ float4_t load4(const T* p);
+// N consecutive elements (N * sizeof(T) = 8 or 16 bytes, aligned) as floats
+template <typename T, int N>
+__device__ __forceinline__ void load_run(const T* p, float* out);
 template <>
-__device__ __forceinline__ float4_t load4<float>(const float* p) {
-  return *reinterpret_cast<const float4_t*>(p);
+__device__ __forceinline__ void load_run<float, 4>(const float* p, float* out) {
+  const float4_t v = *reinterpret_cast<const float4_t*>(p);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) out[e] = v[e];
 }
 template <>
-__device__ __forceinline__ float4_t load4<half_t>(const half_t* p) {
-  const half4_t h = *reinterpret_cast<const half4_t*>(p);
-  float4_t f;
-  f[0] = static_cast<float>(h[0]);
-  f[1] = static_cast<float>(h[1]);
-  f[2] = static_cast<float>(h[2]);
-  f[3] = static_cast<float>(h[3]);
-  return f;
+__device__ __forceinline__ void load_run<half_t, 4>(const half_t* p, float* out) {
+  const half4_t v = *reinterpret_cast<const half4_t*>(p);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) out[e] = static_cast<float>(v[e]);
+}
+template <>
+__device__ __forceinline__ void load_run<half_t, 8>(const half_t* p, float* out) {
+  const half8_t v = *reinterpret_cast<const half8_t*>(p);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = static_cast<float>(v[e]);
+}
+template <typename T, int N>
+__device__ __forceinline__ void store_run(T* p, const float* in);
+template <>
+__device__ __forceinline__ void store_run<float, 4>(float* p, const float* in) {
+  float4_t v;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = in[e];
+  *reinterpret_cast<float4_t*>(p) = v;
+}
+template <>
+__device__ __forceinline__ void store_run<half_t, 4>(half_t* p, const float* in) {
+  half4_t v;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = static_cast<half_t>(in[e]);
+  *reinterpret_cast<half4_t*>(p) = v;
+}
+template <>
+__device__ __forceinline__ void store_run<half_t, 8>(half_t* p, const float* in) {
+  half8_t v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = static_cast<half_t>(in[e]);
+  *reinterpret_cast<half8_t*>(p) = v;
 }
 __device__ __forceinline__ void store4(float* p, float4_t v) { *reinterpret_cast<float4_t*>(p) = v; }
-__device__ __forceinline__ void store4(half_t* p, float4_t v) {
-  half4_t h;
-  h[0] = static_cast<half_t>(v[0]);
-  h[1] = static_cast<half_t>(v[1]);
-  h[2] = static_cast<half_t>(v[2]);
-  h[3] = static_cast<half_t>(v[3]);
-  *reinterpret_cast<half4_t*>(p) = h;
-}
 
 template <typename T, int DMAX, int NB>
 __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(GAttn p) {
   constexpr int ROWS = 16 * NB;
-  constexpr int KS = DMAX / 16;  // 16-feature steps of the score product = 16-feature blocks of the output
+  constexpr int KS = DMAX / 16;  // output feature "blocks": lane (i, g) of the V^T operand owns features i * KS .. + KS - 1
+  constexpr int PIECE = 16 / static_cast<int>(sizeof(T));  // elements of a 16-byte load
+  constexpr int QS = DMAX / (4 * PIECE);                   // load steps of the score product (4 pieces each)
+  constexpr int VP = KS < PIECE ? KS : PIECE;              // elements per load of the V^T operand (8 or 16 bytes)
+  static_assert(KS % VP == 0 && DMAX % (4 * PIECE) == 0, "head dim vs load width");
   __shared__ __attribute__((aligned(16))) float o_lds[2 * ROWS * DMAX];
   __shared__ float ml_lds[2 * ROWS * 2];
 
@@ -132,7 +161,7 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
   // this lane's query rows (one per 16-row block): key limit, tree label, q fragments
   int limit[NB];
   int child_first[NB];
-  float4_t qf[NB][KS];
+  float qf[NB][QS][PIECE];
   const T* qbase = static_cast<const T*>(p.q);
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
@@ -148,10 +177,14 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
     }
     const T* qrow = qbase + (static_cast<int64_t>(q_start + qi) * p.h_q + head) * d;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int f = 16 * s + 4 * g;
-      float4_t z = {0.f, 0.f, 0.f, 0.f};
-      qf[nb][s] = (valid && f < d) ? load4<T>(qrow + f) : z;
+    for (int s = 0; s < QS; ++s) {
+      const int f = (4 * s + g) * PIECE;
+      if (valid && f < d) {
+        load_run<T, PIECE>(qrow + f, qf[nb][s]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < PIECE; ++e) qf[nb][s][e] = 0.f;
+      }
     }
   }
   // keys of this row tile, and this workgroup's share of their 16-key blocks
@@ -189,24 +222,32 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
     } else {
       krow = vrow = (kv_start + t) * p.h_kv + kvh;
     }
-    float4_t kf[KS];
+    float kf[QS][PIECE];
     const T* krow_ptr = kbase + static_cast<int64_t>(krow) * d;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int f = 16 * s + 4 * g;
-      float4_t z = {0.f, 0.f, 0.f, 0.f};
-      kf[s] = f < d ? load4<T>(krow_ptr + f) : z;
+    for (int s = 0; s < QS; ++s) {
+      const int f = (4 * s + g) * PIECE;
+      if (f < d) {
+        load_run<T, PIECE>(krow_ptr + f, kf[s]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < PIECE; ++e) kf[s][e] = 0.f;
+      }
     }
-    // V^T operands: feature fb * 16 + j of the four keys 4 g + m
-    float vf[KS][4];
+    // V^T operands: features j * KS .. + KS - 1 of the four keys 4 g + m
+    float vf[4][KS];
 #pragma unroll
     for (int mm = 0; mm < 4; ++mm) {
       const int vr = __shfl(vrow, 4 * g + mm);
-      const T* vrow_ptr = vbase + static_cast<int64_t>(vr) * d;
+      const T* vrow_ptr = vbase + static_cast<int64_t>(vr) * d + j * KS;
 #pragma unroll
-      for (int fb = 0; fb < KS; ++fb) {
-        const int f = fb * 16 + j;
-        vf[fb][mm] = f < d ? static_cast<float>(vrow_ptr[f]) : 0.f;
+      for (int c = 0; c < KS / VP; ++c) {
+        if (j * KS + c * VP < d) {
+          load_run<T, VP>(vrow_ptr + c * VP, vf[mm] + c * VP);
+        } else {
+#pragma unroll
+          for (int e = 0; e < VP; ++e) vf[mm][c * VP + e] = 0.f;
+        }
       }
     }
     const bool in_tree = tree && kb * 16 + 15 >= tree_start;  // wave-uniform
@@ -214,9 +255,9 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
     for (int nb = 0; nb < NB; ++nb) {
       float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
+      for (int s = 0; s < QS; ++s) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s][c], qf[nb][s][c], acc, 0, 0, 0);
+        for (int c = 0; c < PIECE; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s][c], qf[nb][s][c], acc, 0, 0, 0);
       }
       // acc[r]: key kb * 16 + 4 g + r, query row nb * 16 + j
       float sc[4];
@@ -248,7 +289,7 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
       for (int fb = 0; fb < KS; ++fb) {
         o[nb][fb] *= alpha;
 #pragma unroll
-        for (int mm = 0; mm < 4; ++mm) o[nb][fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[fb][mm], pr[mm], o[nb][fb], 0, 0, 0);
+        for (int mm = 0; mm < 4; ++mm) o[nb][fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[mm][fb], pr[mm], o[nb][fb], 0, 0, 0);
       }
     }
   }
@@ -257,7 +298,7 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
   for (int nb = 0; nb < NB; ++nb) lsum[nb] = sum_xor32(sum_xor16(lsum[nb]));
 
   // ---- the four waves' states into wave 0: waves 2, 3 -> 0, 1, then 1 -> 0 --------------------------------
-  // o[nb][fb][r] of lane (j, g) is feature fb * 16 + 4 g + r of row nb * 16 + j
+  // o[nb][fb][r] of lane (j, g) is feature (4 g + r) * KS + fb of row nb * 16 + j; the slots in LDS are the lane's own
   auto put = [&](int buf) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
@@ -303,21 +344,34 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
     const bool any = lsum[nb] > 0.f;
     const float inv = any ? 1.0f / lsum[nb] : 0.f;
     const float s_row = any ? m[nb] + fast_log2(lsum[nb]) : kNoKeys;
+    // runs of KS consecutive features: (4 g + r) * KS + fb, fb = 0 .. KS - 1
     if (p.splits == 1) {
       T* dst = static_cast<T*>(p.out) + out_row * d;
 #pragma unroll
-      for (int fb = 0; fb < KS; ++fb) {
-        const int f = fb * 16 + 4 * g;
-        if (f < d) store4(dst + f, o[nb][fb] * inv);
+      for (int r = 0; r < 4; ++r) {
+#pragma unroll
+        for (int c = 0; c < KS / VP; ++c) {
+          const int f = (4 * g + r) * KS + c * VP;
+          float run[VP];
+#pragma unroll
+          for (int e = 0; e < VP; ++e) run[e] = o[nb][c * VP + e][r] * inv;
+          if (f < d) store_run<T, VP>(dst + f, run);
+        }
       }
       // a row without keys: out = 0 and the state the reference's kernels start from, m = -5e4, d = 1
       if (g == 0) p.lse[out_row] = any ? s_row : kNegInit;
     } else {
       float* dst = p.part_o + (static_cast<int64_t>(split) * p.total_q * p.h_q + out_row) * d;
 #pragma unroll
-      for (int fb = 0; fb < KS; ++fb) {
-        const int f = fb * 16 + 4 * g;
-        if (f < d) store4(dst + f, o[nb][fb] * inv);
+      for (int r = 0; r < 4; ++r) {
+#pragma unroll
+        for (int c = 0; c < KS / 4; ++c) {
+          const int f = (4 * g + r) * KS + c * 4;
+          float run[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) run[e] = o[nb][c * 4 + e][r] * inv;
+          if (f < d) store_run<float, 4>(dst + f, run);
+        }
       }
       if (g == 0) p.part_s[static_cast<int64_t>(split) * p.total_q * p.h_q + out_row] = s_row;
     }
