@@ -193,19 +193,30 @@ int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
 
 // Work items of 32 query heads (GQA groups above 16): an item does twice the matrix and softmax work per
 // K/V byte, two workgroups fit a compute unit, and every chunk of a sequence is a partial state of 32 (or
-// 64, 128 ...) heads to merge.  Such launches run best with few, long items: the longest chunk that still
-// leaves 320 items, 16 pages if none does.  Measured with the chunk merge as a second kernel (ms at chunks
-// of 16 / 32 / 64 / 128 pages; 64 sequences of 1024-8192 tokens unless noted):
-//   32 q / 1 kv heads 0.058 0.054 0.047 0.059      64 / 1   0.089 0.075 0.074 0.063
-//   64 / 2            0.098 0.085 0.084 0.077      128 / 4  0.168 0.143 0.135 0.142
-//   16 sequences, 32 / 1   0.024 0.024 0.034 0.054     256 of 512-2048 tokens, 32 / 1   0.067 0.062 0.060 0.060
-int decode_pick_chunk_pages_wide(int64_t nnz_pages, int h_kv, int batch, int head_blocks) {
+// 64, 128 ...) heads to merge (in a second kernel).  What decides such a launch is how its workgroups fill
+// the chip: the shortest chunk (a multiple of 8 pages from 16 to 128) whose grid -- chunk slots x kv heads x
+// head blocks -- still fits the workgroups the chip holds at once (resident_items = 2 per compute unit), or
+// twice, three times that when no chunk size fits.  A grid just above a whole number of rounds runs its last
+// workgroups alone; one well below leaves compute units with one workgroup where two would run.  Measured
+// (us; 64 sequences of 1024-8192 tokens, 18 018 pages, unless noted; chunk pages -> time, * = this rule):
+//   32 q / 1 kv   40: 54.2   48*: 42.4   56: 44.9   64: 47.9   96: 51.9   128: 60.7
+//   64 / 1        48: 66.0   64: 72.5    80: 73.6   96*: 58.4  112: 60.4  128: 63.1
+//   64 / 2        48: 79.8   64: 86.1    80: 86.3   96*: 70.3  112: 74.3  128: 80.3
+//   128 / 4       40: 138.0  56: 136.1   64: 137.8  96*: 135.8 128: 148.2
+//   8 sequences of 32k-128k tokens, 64 / 2     64: 180.5   96: 182.7   112*: 160.8   128: 166.9
+//   16 sequences, 32 / 1                       16*: 23.1   24: 22.7    32: 24.2      64: 35.0
+//   256 sequences of 512-2048 tokens, 32 / 1   64: 56.6    80: 58.8    88*           96: 63.3   (32, the rule before: 63.0)
+int decode_pick_chunk_pages_wide(int64_t nnz_pages, int h_kv, int batch, int head_blocks, int resident_items) {
   const int64_t forced = option(kOptDecodeChunkPages);
   if (forced >= 8 && forced % 8 == 0) return static_cast<int>(forced);
-  for (int cp = 128; cp > 16; cp /= 2) {
-    if ((nnz_pages / cp + batch) * h_kv * head_blocks >= 320) return cp;
+  const int64_t per_slot = static_cast<int64_t>(h_kv) * head_blocks;
+  const int64_t capacity = std::max(resident_items, 1);
+  for (int rounds = 1; rounds <= 4; ++rounds) {
+    for (int cp = 16; cp <= 128; cp += 8) {
+      if ((nnz_pages / cp + batch) * per_slot <= capacity * rounds) return cp;
+    }
   }
-  return 16;
+  return 128;
 }
 
 }  // namespace tvmkv
