@@ -521,7 +521,10 @@ int tvmkv_kv_state_remove_sequence(tvmkv_cache* cache, int64_t seq_id);
 int tvmkv_kv_state_fork_sequence(tvmkv_cache* cache, int64_t parent_seq_id, int64_t child_seq_id,
                                  int64_t fork_pos);
 int tvmkv_kv_state_popn(tvmkv_cache* cache, int64_t seq_id, int32_t n);
-/* token_tree_parent_ptr may be NULL (n_tree ignored). */
+/* token_tree_parent_ptr may be NULL (n_tree ignored).  Unknown ids and lengths of 0 are found before anything
+ * changes.  A step that fails later (the pool runs out, a sliding window meets a shared prefix) has already
+ * bumped sequence lengths, as in the reference (paged_kv_cache.cc:919), where such a failure aborts the
+ * program: here the cache then refuses every verb except tvmkv_kv_state_clear with a message that says so. */
 int tvmkv_kv_state_begin_forward(tvmkv_cache* cache, const int64_t* seq_ids,
                                  const int64_t* append_lengths, int32_t batch_size,
                                  const int64_t* token_tree_parent_ptr, int32_t n_tree);

@@ -268,8 +268,20 @@ def test_error_messages_match_the_reference_text():
     add(c, 1)
     with pytest.raises(tvm_amd.KVError, match="The KV cache is full. No page can be allocated."):
         gf("vm.builtin.kv_state_begin_forward")(c, [1], [64])
+    # the failed step had already bumped the sequence's length (as the reference does before it reserves pages,
+    # src/runtime/vm/paged_kv_cache.cc:919): the object refuses everything but clear until it has been cleared
+    with pytest.raises(tvm_amd.KVError, match="call clear before using the cache again"):
+        gf("vm.builtin.kv_state_begin_forward")(c, [0], [1])
+    with pytest.raises(tvm_amd.KVError, match="call clear"):
+        add(c, 2)
+    gf("vm.builtin.kv_state_clear")(c)
+    add(c, 0)
     with pytest.raises(tvm_amd.KVError, match="Append with length 0 is not allowed."):
         gf("vm.builtin.kv_state_begin_forward")(c, [0], [0])
+    # ... while a step that fails before it has changed anything leaves the cache usable
+    with pytest.raises(tvm_amd.KVError, match="cannot be found in KV cache"):
+        gf("vm.builtin.kv_state_begin_forward")(c, [7], [1])
+    gf("vm.builtin.kv_state_begin_forward")(c, [0], [3])
     with pytest.raises(tvm_amd.KVError) as info:
         gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")(c, 0, 1.0, _Fake(), _Fake())
     assert info.value.code == -4  # host-only cache: no device work, no CPU fallback

@@ -65,7 +65,13 @@ void KVBookkeeper::DropSeq(int32_t index) {
 
 // ------------------------------------------------------------------------------------ verbs
 // paged_kv_cache.cc:561-570
+void KVBookkeeper::RequireUsable() const {
+  KV_CHECK(!poisoned_) << "an earlier begin_forward failed after it had started to change the cache; the state of the "
+                       << "page pool is undefined: call clear before using the cache again";
+}
+
 void KVBookkeeper::Clear() {
+  poisoned_ = false;
   seqs_.clear();
   free_seq_slots_.clear();
   seq_index_.clear();
@@ -78,12 +84,14 @@ void KVBookkeeper::Clear() {
 
 // :574-580
 void KVBookkeeper::AddSequence(int64_t seq_id) {
+  RequireUsable();
   KV_CHECK(FindSeq(seq_id) < 0) << "The sequence \"" << seq_id << "\" is already in the KV cache.";
   NewSeq(seq_id, blocks_.Acquire());
 }
 
 // :582-604: blocks that only this sequence holds give their pages back, leaf first
 void KVBookkeeper::RemoveSequence(int64_t seq_id) {
+  RequireUsable();
   const int32_t index = RequireSeq(seq_id);
   int32_t b = seqs_[index].last_block;
   KV_CHECK(blocks_.refcount[b] >= 1) << "block reference count underflow";
@@ -103,6 +111,7 @@ void KVBookkeeper::RemoveSequence(int64_t seq_id) {
 // that block at the page boundary below it (the front part becomes a block both share); a fork
 // point inside a page gives the child a page of its own whose first tokens are copied over.
 void KVBookkeeper::ForkSequence(int64_t parent_seq_id, int64_t child_seq_id, int64_t fork_pos) {
+  RequireUsable();
   const int32_t pi = FindSeq(parent_seq_id);
   KV_CHECK(pi >= 0) << "The parent sequence \"" << parent_seq_id << "\" cannot be found in KV cache.";
   KV_CHECK(FindSeq(child_seq_id) < 0) << "The child sequence \"" << child_seq_id << "\" is already in the KV cache.";
@@ -181,6 +190,7 @@ void KVBookkeeper::ForkSequence(int64_t parent_seq_id, int64_t child_seq_id, int
 
 // :772-801
 void KVBookkeeper::EnableSlidingWindowForSeq(int64_t seq_id, int32_t sliding_window_size, int32_t attn_sink_size) {
+  RequireUsable();
   KV_CHECK(cfg_.support_sliding_window || cfg_.support_layer_sliding_window)
       << "The KV cache does not support sliding window.";
   const int32_t index = RequireSeq(seq_id);
@@ -197,6 +207,7 @@ void KVBookkeeper::EnableSlidingWindowForSeq(int64_t seq_id, int32_t sliding_win
 
 // :803-862
 void KVBookkeeper::PopN(int64_t seq_id, int32_t n) {
+  RequireUsable();
   const int32_t index = RequireSeq(seq_id);
   KV_CHECK(n >= 0) << "The length of popping " << n << " cannot be negative.";
   KV_CHECK(n <= seqs_[index].length) << "The sequence only has length " << seqs_[index].length
@@ -340,7 +351,16 @@ void KVBookkeeper::BeginForward(const int64_t* seq_ids, const int64_t* append_le
   if (cfg_.first_layer_is_mla) {
     KV_CHECK(token_tree_parent_ptr == nullptr) << "Tree attention is not supported yet for MLA";
   }
+  RequireUsable();
   began_forward_ = false;  // until the step is complete
+  // armed at the first change to a sequence, disarmed when the step is complete
+  struct PoisonOnFailure {
+    KVBookkeeper* book;
+    bool armed = false;
+    ~PoisonOnFailure() {
+      if (armed) book->poisoned_ = true;
+    }
+  } guard{this};
   if (buffer_ == nullptr) {
     own_buffer_.resize(RequiredCapacity());
     buffer_ = own_buffer_.data();
@@ -355,12 +375,19 @@ void KVBookkeeper::BeginForward(const int64_t* seq_ids, const int64_t* append_le
   int32_t* k_ragged = last_block_len_before_.data() + B;
   step_ = StepLayout{};
   step_.is_decode_request = true;
+  // what can be checked before anything changes is checked first: every id known, every length positive (the
+  // reference finds these while it already bumps lengths, paged_kv_cache.cc:905-925; the messages are its own)
+  for (int64_t i = 0; i < B; ++i) {
+    RequireSeq(seq_ids[i]);
+    KV_CHECK(append_lengths[i] > 0) << "Append with length 0 is not allowed.";
+  }
   for (int64_t i = 0; i < B; ++i) {
     const int32_t index = RequireSeq(seq_ids[i]);
     SeqRecord& seq = seqs_[index];
     cur_seq_index_[i] = index;
     last_block_len_before_[i] = blocks_.seq_length[seq.last_block];
     k_ragged[i] = seq.length - (seq.committed ? 0 : static_cast<int32_t>(seq.tree_parent.size()));
+    guard.armed = true;
     seq.length += static_cast<int32_t>(append_lengths[i]);
     if (append_lengths[i] != 1) step_.is_decode_request = false;
     step_.total_append_length += append_lengths[i];
@@ -603,6 +630,7 @@ void KVBookkeeper::BeginForward(const int64_t* seq_ids, const int64_t* append_le
   }
   step_.used = uploaded;  // what follows is host-side description only
   began_forward_ = true;
+  guard.armed = false;
 }
 
 // :1800-1928: labels (pre-order number, end of the subtree's range) of every node of every tree
@@ -686,6 +714,7 @@ void KVBookkeeper::BuildTreeMasks(const int64_t* token_tree_parent_ptr, int64_t 
 
 // :1566-1659
 bool KVBookkeeper::CommitAcceptedTokenTreeNodes(const int64_t* seq_ids, const int64_t* leaf_indices, int num) {
+  RequireUsable();
   // The reference takes the batch of the last step for granted (its only caller is its own VM); here the
   // call comes through a C ABI: a different batch would index the step's arrays out of range or pop the
   // wrong sequences, so it is refused before anything changes.

@@ -151,6 +151,13 @@ class KVBookkeeper {
 
   // ---- current step -----------------------------------------------------------------------------
   bool began_forward_ = false;
+  // A begin_forward that fails after it has started to change sequences (the pool runs out, a sliding window
+  // meets a shared prefix, the step buffer overflows) leaves lengths bumped and pages half reserved, as in the
+  // reference (paged_kv_cache.cc:919 bumps seq_length before it reserves).  There the failure aborts the
+  // program; here it comes back as an error code, so the object refuses every verb but Clear() afterwards
+  // instead of handing out slots of a state nobody defined.
+  bool poisoned_ = false;
+  void RequireUsable() const;
   StepLayout step_;
   int32_t* buffer_ = nullptr;
   int64_t capacity_ = 0;

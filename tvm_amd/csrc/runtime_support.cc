@@ -177,6 +177,30 @@ int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
   const int64_t forced = option(kOptDecodeChunkPages);
   if (forced >= 8 && forced % 8 == 0) return static_cast<int>(forced);
   const int64_t work = nnz_pages * h_kv;
+  const int64_t per_sequence = nnz_pages / std::max(batch, 1);
+  if (work <= 65536) {
+    // Small launches (up to 1 M cached tokens x kv heads): the shortest chunk, a multiple of 8 pages from 24 on,
+    // whose grid fits the 3 workgroups x 256 compute units the chip holds at once -- every workgroup starts
+    // at once and none runs alone at the end; one or two very long sequences take 128-page chunks instead when
+    // that still leaves 384 items (more than 32 states per sequence cost more than the items lost).  Measured
+    // (us, chunk pages -> time, * = this rule; the rule before in brackets):
+    //   16 x U[100,4000] tokens, 8 kv heads   16: 29.8  24*: 26.1  32: 28.3  64: 32.1            [16]
+    //   8 x U[2000,6000]                      16: 32.7  24*: 27.4  32: 30.3  64: 32.8            [16]
+    //   4 x 32768                             64: 92.4  88: 87.5   96*: 88.7  128: 99.9          [64]
+    //   64 x U[1024,8192], 16 q / 1 kv head   16: 49.7  24: 44.9   32*: 41.4  40: 37.6  64: 41.6 [16]
+    //   64 x U[64,512]                        16: 23.4  32: 20.0   40*: 20.9  128: 19.4          [16]
+    //   32 x U[100,2000]                      16: 34.6  32: 32.5   40*: 34.2  64: 36.2           [32]
+    //   1 x 131072                            64: 102.3 120: 100.8 128*: 88.1                    [128]
+    int cp = 128;
+    for (int c = 24; c <= 128; c += 8) {
+      if ((nnz_pages / c + batch) * h_kv <= 768) {
+        cp = c;
+        break;
+      }
+    }
+    if (per_sequence / cp > 32 && (nnz_pages / 128 + batch) * h_kv >= 384) cp = 128;
+    return cp;
+  }
   const int64_t items = std::min<int64_t>(std::max<int64_t>(work / 64, 768), 2304);
   const int64_t cp = work / items;
   int pow2 = 16;
