@@ -563,7 +563,10 @@ def extras(torch, K, dev):
         "4 x 32768, 32/8": decode_shape(4, 32768, 32768, 32, 8, 12),
         "2048 x U[64,512], 32/8": decode_shape(2048, 64, 512, 32, 8, 13),
         "64 x U[1024,8192], 32/1": decode_shape(64, 1024, 8192, 32, 1, 14),
-        "64 x U[1024,8192], 64/1": decode_shape(64, 1024, 8192, 64, 1, 15)}
+        "64 x U[1024,8192], 64/1": decode_shape(64, 1024, 8192, 64, 1, 15),
+        "64 x U[1024,8192], 64/2": decode_shape(64, 1024, 8192, 64, 2, 16),
+        "16 x U[100,4000], 32/8": decode_shape(16, 100, 4000, 32, 8, 5),
+        "8 x U[2000,6000], 32/8": decode_shape(8, 2000, 6000, 32, 8, 17)}
     torch.cuda.empty_cache()
 
     # ---- sliding window + attention sinks, and a token-tree verify step, on configs[1]'s shape ----
