@@ -186,6 +186,36 @@ def calibrate(num_bytes=2 << 30, iters=10, quiet=False):
     return out
 
 
+def bare_step_over_layer_pools(torch, dev, layers, seed):
+    """The decode step of configs[1] as bare launches (tvmkv_fused_decode_step), one page pool per layer
+    as a model has them: what the memory system makes of `layers` x 1.2 GB that are read once per step
+    (nothing of a layer's pages is left in the memory-side cache or the TLBs when its turn comes again),
+    without the cache object around the launches.  Returns ms per layer."""
+    from tvm_amd import kernels as K
+
+    wl = decode_workload(pool_pages=20480, steps=1, seed=seed)
+    B = wl["batch"]
+    t = {key: torch.tensor(wl["tables"][0][key], dtype=torch.int32, device=dev)
+         for key in ("page_indptr", "page_values", "last_page_len", "q_rope_position", "append_position_map")}
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    first = torch.empty((wl["pool_pages"], 2, HKV, PS, D), dtype=torch.float16, device=dev)
+    for lo in range(0, wl["pool_pages"], 4096):
+        first[lo:lo + 4096].copy_(torch.randn(first[lo:lo + 4096].shape, generator=gen, device=dev))
+    pools = [first] + [first.clone() for _ in range(layers - 1)]
+    qkv = torch.randn((B, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16)
+    out = torch.empty((B, HQ, D), dtype=torch.float16, device=dev)
+    lse = torch.empty((B, HQ), dtype=torch.float32, device=dev)
+
+    def step(_):
+        for pool in pools:
+            K.fused_decode_step(qkv, pool, t["page_indptr"], t["page_values"], t["last_page_len"], t["q_rope_position"],
+                                t["append_position_map"], out, lse, 1, 1.0, 1e4, D ** -0.5)
+
+    settle(torch, step)
+    return time_region(torch, step, 8) / layers
+
+
 def cache_object_decode(torch, dev, layers=32, seed=1):
     """configs[1] through the cache OBJECT, the way a model drives it (the reference's call order,
     src/runtime/vm/kv_state.cc:33-116): per decode step one begin_forward for all layers, then
@@ -245,13 +275,22 @@ def cache_object_decode(torch, dev, layers=32, seed=1):
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / (steps - 4)
     gpu_ms = start.elapsed_time(stop) / (steps - 4)
+    t0 = time.perf_counter()  # the host's share: how long it takes to enqueue a step on an idle device
+    step()
+    enqueue_ms = (time.perf_counter() - t0) * 1e3
+    torch.cuda.synchronize()
     kv_tokens = float(ctx.sum()) + B * (4 + (steps - 4) / 2.0)  # cached tokens an average timed step attends to
     step_bytes = layers * (kv_tokens * TOKEN_BYTES + B * HQ * D * 2 * 2 + B * (HQ + 2 * HKV) * D * 2 + B * TOKEN_BYTES)
-    return {"workload": f"configs[1] through the cache object: {layers} layers, B=64, ctx U[1024,8192], one begin_forward + "
+    del cache
+    torch.cuda.empty_cache()
+    bare_ms = bare_step_over_layer_pools(torch, dev, layers, seed)
+    return {"ms_per_layer_bare_launches_over_one_pool_per_layer": round(bare_ms, 4),
+            "workload": f"configs[1] through the cache object: {layers} layers, B=64, ctx U[1024,8192], one begin_forward + "
                         f"{layers} x attention_with_fused_qkv + end_forward per decode step, cache filled by chunked prefill "
                         "steps through the same interface",
             "layers": layers, "ms_per_step": round(gpu_ms, 4), "ms_per_layer": round(gpu_ms / layers, 4),
-            "host_wall_ms_per_step": round(wall_ms, 4), "GBps": round(step_bytes / gpu_ms / 1e6, 1),
+            "host_wall_ms_per_step": round(wall_ms, 4), "host_enqueue_ms_per_step": round(enqueue_ms, 4),
+            "GBps": round(step_bytes / gpu_ms / 1e6, 1),
             "frac_of_hbm_peak": round(step_bytes / gpu_ms / 1e6 / HBM_PEAK_GBPS, 4),
             "tokens_per_s": round(B / (gpu_ms * 1e-3), 1)}
 
@@ -758,10 +797,11 @@ def extras(torch, K, dev):
         from tvm_amd import dlpack as dl
         rng_ = np.random.default_rng(1)
         ctx_ = rng_.integers(1024, 8192, size=64, endpoint=True)
-        res = {"workload": "what the tuned fp16 kernels are not built for, on the generic matrix-core kernels (float32 "
-                           "arithmetic, v_mfma_f32_16x16x4_f32, K/V rows straight from their pages): decode of 64 seqs ctx "
-                           "U[1024,8192] Hq32/Hkv8/D128 with float32 storage (page 16) and with fp16 pages of 24 tokens; "
-                           "causal self-attention of 4 x 2048 tokens with float32 storage"}
+        res = {"workload": "what the tuned fp16 kernels are not built for, on the generic matrix-core kernels (K/V rows "
+                           "straight from their pages into the operands of v_mfma_f32_16x16x4_f32, or of the fp16 "
+                           "instructions of that shape for fp16 storage): decode of 64 seqs ctx U[1024,8192] Hq32/Hkv8/D128 "
+                           "with float32 storage (page 16) and with fp16 pages of 24 tokens; causal self-attention of "
+                           "4 x 2048 tokens with float32 storage (D128) and with fp16 storage at head dim 160"}
         for name, tdt, ps_ in (("decode_float32_storage", torch.float32, 16), ("decode_fp16_pages_of_24_tokens", torch.float16, 24)):
             npg_ = (ctx_ + ps_ - 1) // ps_
             ip_ = np.concatenate([[0], np.cumsum(npg_)])
@@ -796,6 +836,16 @@ def extras(torch, K, dev):
         fl_ = 4.0 * HQ * D * n_ * c_ * (c_ + 1) / 2
         res["causal_prefill_float32_storage"] = {"ms": round(ms_, 4), "tflops": round(fl_ / ms_ / 1e9, 1),
                                                  "frac_of_fp32_mfma_peak": round(fl_ / ms_ / 1e9 / 157.3, 4)}
+        d_ = 160
+        q_, k_, v_ = (torch.randn((n_ * c_, h_, d_), device=dev).to(torch.float16) for h_ in (HQ, HKV, HKV))
+        o_ = torch.empty_like(q_)
+        a_ = (dl.tensor(q_), dl.tensor(ind_), dl.tensor(k_), dl.tensor(v_), dl.tensor(ind_), dl.tensor(zq_), dl.tensor(zb_),
+              dl.tensor(o_), dl.tensor(l_), 1, 0, 1.0, 1e4, d_ ** -0.5)
+        dl.call("batch_prefill_ragged_kv", *a_)
+        ms_ = time_region(torch, lambda i: dl.call("batch_prefill_ragged_kv", *a_), 5, SETTLE_S)
+        fl_ = 4.0 * HQ * d_ * n_ * c_ * (c_ + 1) / 2
+        res["causal_prefill_fp16_head_dim_160"] = {"ms": round(ms_, 4), "tflops": round(fl_ / ms_ / 1e9, 1),
+                                                   "frac_of_mfma_peak": round(fl_ / ms_ / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
         return res
 
     out["generic_kernels"] = generic_leg()

@@ -52,7 +52,8 @@ def test_chunk_size_follows_the_work():
     # 768 work items for small launches up to ~2300 for large ones; chunks of 16 to 128 pages
     assert tvm_amd.decode_split_plan([0, 4], 4, 8)[0] == 24             # small launches: 24 pages at least
     cfg2 = [288 * i for i in range(65)]
-    assert tvm_amd.decode_split_plan(cfg2, 18432, 8)[0] == 64            # configs[1]: 2304 items
+    assert tvm_amd.decode_split_plan(cfg2, 18432, 8)[0] == 48            # configs[1]: 64 pages by the item count, its neighbour that does not camp
+    assert tvm_amd.decode_split_plan(cfg2, 18432, 4)[0] == 64            # four kv heads: no camping seen
     assert tvm_amd.decode_split_plan([0, 18432], 18432, 8)[0] == 128     # as one sequence: fewer states to merge
     short = [80 * i for i in range(257)]
     assert tvm_amd.decode_split_plan(short, 80 * 256, 8)[0] == 128       # 256 short sequences: no split at all
@@ -60,7 +61,9 @@ def test_chunk_size_follows_the_work():
     assert tvm_amd.decode_split_plan([0, 18432], 18432, 1)[0] == 32      # one kv head: 768 items
     assert tvm_amd.decode_split_plan([0, 8192], 8192, 8)[0] == 128       # one sequence of 131072 tokens: 64 states, not 128
     assert tvm_amd.decode_split_plan([0, 4096, 8192], 8192, 8)[0] == 128  # two of 65536
-    assert tvm_amd.decode_split_plan([0, 2048, 4096, 6144, 8192], 8192, 8)[0] == 96   # four of 32768: the grid fits 768 workgroups
+    assert tvm_amd.decode_split_plan([0, 2048, 4096, 6144, 8192], 8192, 8)[0] == 104  # four of 32768: the grid fits 768 workgroups (96 would camp)
+    long8 = [5000 * i for i in range(9)]
+    assert tvm_amd.decode_split_plan(long8, 40000, 8)[0] == 112          # eight long sequences: 128 by the states, its neighbour
     assert tvm_amd.decode_split_plan([0, 100, 250, 400, 457], 457, 8)[0] == 24          # (457 / 24 + 4) * 8 = 184 items
 
 

@@ -2,8 +2,10 @@
 // tuned fp16 kernels are not built for -- float32 storage, pages of any size, head dims that are a multiple
 // of 4 (fp32) or 8 (fp16) up to 256.  One kernel serves ragged prefill (_prefill_kernels.py:677-923), paged
 // prefill (:54-391), paged decode (_decode_kernels.py:49-411) and both token-tree forms (tree_attn.py:93-259,
-// :634-797): float32 arithmetic on v_mfma_f32_16x16x4_f32, base-2 online softmax (m = -5e4 to start with),
-// K and V rows read straight from memory into matrix operands with one page-table lookup per row.
+// :634-797): base-2 online softmax (m = -5e4 to start with), K and V rows read straight from memory into matrix
+// operands with one page-table lookup per row.  float32 storage multiplies on v_mfma_f32_16x16x4_f32; fp16 storage
+// on the fp16 instructions of the same shape (v_mfma_f32_16x16x32_f16 for the scores, v_mfma_f32_16x16x16_f16 for
+// the output, the probabilities rounded to fp16 as in the tuned kernels), float32 sums in both.
 //
 // Tile: ROWS = 16 * NB query rows of one (sequence, kv head) -- a row is a (token, head of the GQA group)
 // pair -- against 16 keys per step and wave.  The four waves of a workgroup take every fourth 16-key block
@@ -20,6 +22,10 @@
 //    lane (j, g) already holds the probabilities of row j; output "block" fb, row i of the product is feature
 //    i * KS + fb, so lane (i, g) reads KS consecutive features of a key (the 16 lanes of a group read a whole
 //    row) and lane (j, g) ends up with runs of KS consecutive output features.
+// The fp16 instructions keep both choices: a lane's 8 halfs of a piece are 8 consecutive contraction slots of
+// v_mfma_f32_16x16x32_f16 (lane (i, g) holds A[i][8 g .. 8 g + 7] and B[8 g .. 8 g + 7][i]), and the four keys 4 g + m
+// are the four slots A[i][4 g + m] / B[4 g + m][i] that lane group g holds for v_mfma_f32_16x16x16_f16, so the
+// V^T operand of feature block fb is one half of each of the lane's four key rows.
 #include <algorithm>
 
 #include "kernels_common.cuh"
@@ -62,18 +68,6 @@ __device__ __forceinline__ void load_run<float, 4>(const float* p, float* out) {
 #pragma unroll
   for (int e = 0; e < 4; ++e) out[e] = v[e];
 }
-template <>
-__device__ __forceinline__ void load_run<half_t, 4>(const half_t* p, float* out) {
-  const half4_t v = *reinterpret_cast<const half4_t*>(p);
-#pragma unroll
-  for (int e = 0; e < 4; ++e) out[e] = static_cast<float>(v[e]);
-}
-template <>
-__device__ __forceinline__ void load_run<half_t, 8>(const half_t* p, float* out) {
-  const half8_t v = *reinterpret_cast<const half8_t*>(p);
-#pragma unroll
-  for (int e = 0; e < 8; ++e) out[e] = static_cast<float>(v[e]);
-}
 template <typename T, int N>
 __device__ __forceinline__ void store_run(T* p, const float* in);
 template <>
@@ -99,8 +93,14 @@ __device__ __forceinline__ void store_run<half_t, 8>(half_t* p, const float* in)
 }
 __device__ __forceinline__ void store4(float* p, float4_t v) { *reinterpret_cast<float4_t*>(p) = v; }
 
+// workgroups per CU: the fp16 form holds its operands in half the registers
+constexpr int generic_workgroups(int elem_bytes, int dmax, int nb) {
+  return elem_bytes == 2 ? (dmax > 128 ? 2 : (nb == 1 ? 4 : 3)) : (dmax > 128 ? 1 : (nb == 1 ? 3 : 2));
+}
+
 template <typename T, int DMAX, int NB>
-__global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(GAttn p) {
+__global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void generic_attn_kernel(GAttn p) {
+  constexpr bool HALF = sizeof(T) == 2;
   constexpr int ROWS = 16 * NB;
   constexpr int KS = DMAX / 16;  // output feature "blocks": lane (i, g) of the V^T operand owns features i * KS .. + KS - 1
   constexpr int PIECE = 16 / static_cast<int>(sizeof(T));  // elements of a 16-byte load
@@ -161,7 +161,8 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
   // this lane's query rows (one per 16-row block): key limit, tree label, q fragments
   int limit[NB];
   int child_first[NB];
-  float qf[NB][QS][PIECE];
+  float qf[NB][QS][PIECE];  // float32 storage
+  half8_t qh[NB][QS];       // fp16 storage: the pieces as they are in memory
   const T* qbase = static_cast<const T*>(p.q);
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
@@ -179,7 +180,10 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
 #pragma unroll
     for (int s = 0; s < QS; ++s) {
       const int f = (4 * s + g) * PIECE;
-      if (valid && f < d) {
+      if constexpr (HALF) {
+        half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        qh[nb][s] = valid && f < d ? *reinterpret_cast<const half8_t*>(qrow + f) : z;
+      } else if (valid && f < d) {
         load_run<T, PIECE>(qrow + f, qf[nb][s]);
       } else {
 #pragma unroll
@@ -223,11 +227,15 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
       krow = vrow = (kv_start + t) * p.h_kv + kvh;
     }
     float kf[QS][PIECE];
+    half8_t kh[QS];
     const T* krow_ptr = kbase + static_cast<int64_t>(krow) * d;
 #pragma unroll
     for (int s = 0; s < QS; ++s) {
       const int f = (4 * s + g) * PIECE;
-      if (f < d) {
+      if constexpr (HALF) {
+        half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        kh[s] = f < d ? *reinterpret_cast<const half8_t*>(krow_ptr + f) : z;
+      } else if (f < d) {
         load_run<T, PIECE>(krow_ptr + f, kf[s]);
       } else {
 #pragma unroll
@@ -236,18 +244,36 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
     }
     // V^T operands: features j * KS .. + KS - 1 of the four keys 4 g + m
     float vf[4][KS];
+    half_t vh[4][KS];
 #pragma unroll
     for (int mm = 0; mm < 4; ++mm) {
       const int vr = __shfl(vrow, 4 * g + mm);
       const T* vrow_ptr = vbase + static_cast<int64_t>(vr) * d + j * KS;
 #pragma unroll
       for (int c = 0; c < KS / VP; ++c) {
-        if (j * KS + c * VP < d) {
+        const bool inside = j * KS + c * VP < d;
+        if constexpr (HALF) {
+          typedef half_t run_t __attribute__((ext_vector_type(VP)));
+          run_t run;
+#pragma unroll
+          for (int e = 0; e < VP; ++e) run[e] = 0;
+          if (inside) run = *reinterpret_cast<const run_t*>(vrow_ptr + c * VP);
+#pragma unroll
+          for (int e = 0; e < VP; ++e) vh[mm][c * VP + e] = run[e];
+        } else if (inside) {
           load_run<T, VP>(vrow_ptr + c * VP, vf[mm] + c * VP);
         } else {
 #pragma unroll
           for (int e = 0; e < VP; ++e) vf[mm][c * VP + e] = 0.f;
         }
+      }
+    }
+    half4_t va[KS];  // fp16 storage: feature block fb of the four keys
+    if constexpr (HALF) {
+#pragma unroll
+      for (int fb = 0; fb < KS; ++fb) {
+        half4_t a = {vh[0][fb], vh[1][fb], vh[2][fb], vh[3][fb]};
+        va[fb] = a;
       }
     }
     const bool in_tree = tree && kb * 16 + 15 >= tree_start;  // wave-uniform
@@ -256,8 +282,12 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
       float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < QS; ++s) {
+        if constexpr (HALF) {
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh[s], qh[nb][s], acc, 0, 0, 0);
+        } else {
 #pragma unroll
-        for (int c = 0; c < PIECE; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s][c], qf[nb][s][c], acc, 0, 0, 0);
+          for (int c = 0; c < PIECE; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s][c], qf[nb][s][c], acc, 0, 0, 0);
+        }
       }
       // acc[r]: key kb * 16 + 4 g + r, query row nb * 16 + j
       float sc[4];
@@ -288,8 +318,14 @@ __global__ __launch_bounds__(256, DMAX > 128 ? 1 : 2) void generic_attn_kernel(G
 #pragma unroll
       for (int fb = 0; fb < KS; ++fb) {
         o[nb][fb] *= alpha;
+        if constexpr (HALF) {
+          const half4_t ph = {static_cast<half_t>(pr[0]), static_cast<half_t>(pr[1]), static_cast<half_t>(pr[2]),
+                              static_cast<half_t>(pr[3])};
+          o[nb][fb] = __builtin_amdgcn_mfma_f32_16x16x16f16(va[fb], ph, o[nb][fb], 0, 0, 0);
+        } else {
 #pragma unroll
-        for (int mm = 0; mm < 4; ++mm) o[nb][fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[mm][fb], pr[mm], o[nb][fb], 0, 0, 0);
+          for (int mm = 0; mm < 4; ++mm) o[nb][fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[mm][fb], pr[mm], o[nb][fb], 0, 0, 0);
+        }
       }
     }
   }
@@ -473,7 +509,7 @@ int generic_attention(const GenericAttention& a, void* stream_) {
     const int rows_per_tile = (rows_hint > 16 && a.d <= 128) ? 32 : 16;
     const int64_t tiles = (a.total_q * group / rows_per_tile + a.batch) * a.h_kv;
     const int64_t keys_per_seq = a.nnz_pages * a.page_size / a.batch;
-    const int64_t want = 8 * static_cast<int64_t>(compute_units()) / std::max<int64_t>(tiles, 1);
+    const int64_t want = (f32 ? 8 : 16) * static_cast<int64_t>(compute_units()) / std::max<int64_t>(tiles, 1);
     p.splits = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>({want, keys_per_seq / 128, 64})));
   }
   if (p.splits > 1) {

@@ -167,12 +167,25 @@ void debug_set_scratch_launches(uint64_t launches) {
 // three rounds of 3 workgroups x 256 CUs; small ones with fewer and longer items (one sequence of 131 072
 // tokens: 0.110 ms with 32-page chunks, 0.085 with 128; 64 sequences with one kv head: 0.140 ms with
 // 8-page chunks, 0.073 with 64).  One step of the matrix-core decode kernel is 2 pages per wave, 8 per
-// workgroup; chunks are powers of two from 16 to 128 pages.  Two cases take longer chunks than that:
+// workgroup; chunks are multiples of 8 pages up to 128.  Two cases take longer chunks than that:
 //  * more than 16 chunks per sequence while at least 768 items remain: the states of a sequence are
 //    merged by one workgroup, a serial tail (8 sequences of 16-65 k tokens: 0.245 ms with 64 pages,
 //    0.236 with 128);
 //  * sequences that fit one 128-page chunk on average, enough of them to fill the chip without a split:
 //    no partial states at all (256 sequences of 512-2048 tokens: 0.220 ms with 64 pages, 0.210 with 128).
+// Chunks of 32, 64, 96 or 128 pages put the chunks of a sequence whose pages have consecutive ids -- a cache that
+// was filled sequence by sequence hands them out that way -- at a distance in memory at which the workgroups of
+// the sequence, which walk their chunks in step, keep meeting in the same memory channels.  Seen with 8 and 16 kv
+// heads (pages of 64 and 128 KiB), not with 4 or fewer.  Measured, 8 kv heads, us with permuted / consecutive
+// page ids (chunk pages -> time):
+//   64 x U[1024,8192] (cfg 2)      48: 195.8 / 196.3   56: 194.5 / 196.5   64: 197.8 / 205.1   80: 195.0 / 197.3
+//   8 x U[32768,131072], 64 q      112: 435.1 / 438.8  120: 439.5 / 440.5  128: 436.8 / 478.9  64: 453.3 / 527.3
+//   16 x U[8192,32768]             112: 200.9 / 202.6  64: 206.6 / 231.4   128: 206.6 / 221.6
+//   4 x 32768                      88: 90.2 / 92.1     96: 92.5 / 101.3    104: 91.9 / 93.4
+//   64 x U[1024,8192], 16 kv heads 56: 389.9 / 387.3   32: 390.7 / 425.5   64: 390.2 / 406.0
+//   64 x U[1024,8192], 4 kv heads  56: 126.0 / 123.2   64: 120.5 / 118.2
+static bool camps(int chunk_pages, int h_kv) { return h_kv >= 8 && chunk_pages % 32 == 0; }
+
 int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
   const int64_t forced = option(kOptDecodeChunkPages);
   if (forced >= 8 && forced % 8 == 0) return static_cast<int>(forced);
@@ -193,6 +206,7 @@ int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
     //   1 x 131072                            64: 102.3 120: 100.8 128*: 88.1                    [128]
     int cp = 128;
     for (int c = 24; c <= 128; c += 8) {
+      if (camps(c, h_kv)) continue;
       if ((nnz_pages / c + batch) * h_kv <= 768) {
         cp = c;
         break;
@@ -211,7 +225,11 @@ int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
   // longer chunk takes away (one sequence of 131 072 tokens, 8 kv heads: 0.103 ms with 64 pages, 0.089 with
   // 128; two of 65 536: 0.096 / 0.086; four of 32 768, 32 states each at 64 pages: 0.092 / 0.101)
   while (pow2 < 128 && per_seq / pow2 > 32 && work / (pow2 * 2) >= 384) pow2 *= 2;
-  if (per_seq <= 96 && static_cast<int64_t>(batch) * h_kv >= 1536) pow2 = 128;
+  if (per_seq <= 96 && static_cast<int64_t>(batch) * h_kv >= 1536) return 128;
+  // the neighbours of the powers of two that do not camp (see camps()); one or two sequences keep 128 pages
+  // (64 states of a 131 072-token sequence merge in two rounds of 32)
+  if (camps(pow2, h_kv) && pow2 == 64) return 48;
+  if (camps(pow2, h_kv) && pow2 == 128 && batch > 2) return 112;
   return pow2;
 }
 
