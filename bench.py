@@ -295,6 +295,71 @@ def cache_object_decode(torch, dev, layers=32, seed=1):
             "tokens_per_s": round(B / (gpu_ms * 1e-3), 1)}
 
 
+def cache_object_shared_prefix_decode(torch, dev, layers=8, seed=5):
+    """Decode with a shared prompt through the cache object: 64 sequences forked from one parent that holds a
+    4096-token prefix (kv_state_fork_sequence: the children share the parent's pages, src/runtime/vm/
+    paged_kv_cache.cc:653-770), each with U[256,2048] tokens of its own.  A decode step then has two depths
+    (BeginForward, :884-1212): the shared prefix once for all 64 queries (the paged prefill kernel, 64 x group rows
+    per kv head), every sequence's own tokens (the decode kernel), and the merge of the two states -- the
+    reference's flow for prefix sharing (:2161-2335).  Algorithmic bytes count the prefix once."""
+    from tvm_amd import get_global_func as gf
+
+    rng = np.random.default_rng(seed)
+    B, prefix = 64, 4096
+    own = rng.integers(256, 2048, size=B, endpoint=True)
+    steps = 8
+    capacity = prefix + int(own.sum()) + B * (steps + 8) + (B + 2) * PS
+    cache = gf("vm.builtin.paged_attention_kv_cache_create")(
+        [B + 1, capacity, 4096, PS, 0], [0, layers], HQ, HKV, D, D, [0] * layers, False, 1, 1.0, 1e4, None,
+        torch.empty((), dtype=torch.float16, device=dev))
+    cache.set_stream(torch.cuda.current_stream().cuda_stream)
+    f_add, f_fork = gf("vm.builtin.kv_state_add_sequence"), gf("vm.builtin.kv_state_fork_sequence")
+    f_begin, f_end = gf("vm.builtin.kv_state_begin_forward"), gf("vm.builtin.kv_state_end_forward")
+    f_popn = gf("vm.builtin.kv_state_popn")
+    f_attn = gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")
+    sm_scale = D ** -0.5
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    chunk_qkv = torch.randn((4096, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16)
+    chunk_out = torch.empty((4096, HQ, D), dtype=torch.float16, device=dev)
+
+    def forward(ids, lens, qkv_, out_):
+        f_begin(cache, ids, lens, None)
+        for layer in range(layers):
+            f_attn(cache, layer, sm_scale, qkv_, out_)
+        f_end(cache)
+
+    parent = B
+    f_add(cache, parent)
+    forward([parent], [prefix], chunk_qkv[:prefix], chunk_out[:prefix])
+    for b in range(B):
+        f_fork(cache, parent, b)
+        n = int(own[b])
+        forward([b], [n], chunk_qkv[:n], chunk_out[:n])
+    qkv = torch.randn((B, HQ + 2 * HKV, D), generator=gen, device=dev).to(torch.float16)
+    out = torch.empty((B, HQ, D), dtype=torch.float16, device=dev)
+    ids, ones = list(range(B)), [1] * B
+
+    def step(_):
+        forward(ids, ones, qkv, out)
+        for b in ids:
+            f_popn(cache, b, 1)
+
+    for _ in range(3):
+        step(0)
+    flags = cache.flags()
+    ms = time_region(torch, step, steps, SETTLE_S)
+    nbytes = layers * ((prefix + float(own.sum()) + B) * TOKEN_BYTES + B * HQ * D * 2 * 2 + B * (HQ + 2 * HKV) * D * 2)
+    unshared = layers * ((B * prefix + float(own.sum()) + B) * TOKEN_BYTES + B * HQ * D * 2 * 2)
+    return {"workload": f"64 sequences forked from one 4096-token prompt, U[256,2048] tokens of their own, one token each per "
+                        f"step, {layers} layers through the cache object: per layer split + RoPE + append, the shared prefix "
+                        "for all queries in one paged-prefill launch, the sequences' own tokens in the decode kernel, merge",
+            "layers": layers, "depths": flags["num_depths"], "ms_per_step": round(ms, 4), "ms_per_layer": round(ms / layers, 4),
+            "MB_per_layer": round(nbytes / layers / 1e6, 1), "GBps": round(nbytes / ms / 1e6, 1),
+            "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
+            "MB_per_layer_without_sharing": round(unshared / layers / 1e6, 1)}
+
+
 def cache_object_prefill(torch, dev, layers=8):
     """configs[2] through the cache object: the prefixes are cached by chunked-prefill steps, then every
     timed step appends the 8 chunks in one begin_forward, runs attention_with_fused_qkv on every layer
@@ -1264,6 +1329,8 @@ def main():
         result["extras"]["cache_object_decode"] = cache_object_decode(torch, dev)
         torch.cuda.empty_cache()
         result["extras"]["cache_object_prefill"] = cache_object_prefill(torch, dev)
+        torch.cuda.empty_cache()
+        result["extras"]["cache_object_shared_prefix_decode"] = cache_object_shared_prefix_decode(torch, dev)
     print(json.dumps(result))
 
 
