@@ -779,7 +779,21 @@ class PagedKVCache {
     const double rotary_scale = sliding_layer ? 1 : rotary_scale_;
     const int rotary_mode = rope_mode_ == TVMKV_ROPE_INLINE;
     bool cross_attn_computed = false;
-    for (int d = 0; d < s.num_depths; ++d) {
+    // The reference walks the depths in order and merges each state into the first (:2216-2299).  The merge
+    // is symmetric, and the paged-prefill kernel can merge into an existing state in its own epilogue while the
+    // decode and tree kernels need a temporary output and a merge launch: the depths that run those go first,
+    // so that one of them writes (o, lse) directly and the prefill depths need no launch of their own to merge
+    // (a decode step over a shared prompt: four launches per layer instead of five).
+    int order[kMaxBlockDepth];
+    int n_order = 0;
+    for (int pass = 0; pass < 2; ++pass) {
+      for (int d = 0; d < s.num_depths; ++d) {
+        const bool merges_itself = !generic_ && !(s.append_before_attn && !s.is_chain[d]) && !s.use_decode_kernel[d];
+        if (merges_itself == (pass == 1)) order[n_order++] = d;
+      }
+    }
+    for (int at = 0; at < n_order; ++at) {
+      const int d = order[at];
       if (s.page_indices[d].size == 0) continue;
       void* attn_output = is_first_kernel ? o : temp_out_;
       float* attn_lse = is_first_kernel ? lse : temp_lse_;
