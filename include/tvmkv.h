@@ -328,7 +328,7 @@ int tvmkv_fused_decode_step(const void* qkv, void* pages, const int32_t* page_in
  * per device, held until the process ends; the call makes no hipMalloc / hipFree and returns
  * TVMKV_EINVAL with a message when the shapes need more: 256 KiB + (nnz_pages / chunk_pages +
  * batch_size) * h_q * (head_dim + 2) * 4 bytes, chunk_pages as tvmkv_decode_split_plan reports
- * (configs of 64 x 8k-token and 8 x 128k-token sequences need 6 and 11 MiB).  All calls on a device
+ * (configs of 64 x 8k-token and 8 x 128k-token sequences need 8 and 12 MiB).  All calls on a device
  * share the array: calls that overlap on one device (different streams) race, stream-ordered
  * calls do not.  A call captured into a graph may be replayed: the workgroup that merges the chunks
  * of a sequence puts the arrival counter back to zero.  (tvmkv_batch_decode_paged_kv under capture

@@ -4,7 +4,7 @@ few sequences cut out of the batch:
 
 * a value tensor that is constant per feature must come back as that constant (softmax weights
   sum to one; the reference's phantom denominator term 2^(-5e4 - m) is 0 in fp32 here),
-* split-KV results must not depend on the chunk size,
+* split-KV results must not depend on the chunk size, nor on where the pages of a sequence lie in the pool,
 * lse of a sequence = log2 sum 2^(score), checked with a float64 torch computation per sequence,
 * single sequences of the batch against the oracle.
 """
@@ -82,6 +82,14 @@ def test_decode_full_size_properties(name, batch, lo, hi, hq, pool):
     assert_close(host(out8), host(out128), atol=2e-3, rtol=2e-3, what=f"{name} chunk 8 vs 128")
     assert_close(host(lse8), host(lse128), atol=1e-3, rtol=1e-5, what=f"{name} lse chunk 8 vs 128")
     assert_close(host(out), host(out128), atol=2e-3, rtol=2e-3, what=f"{name} default chunk vs 128")
+    # the same rows at consecutive page ids, the order in which a freshly filled cache hands pages out:
+    # bit-identical (the page table is the only thing that knows where a page lies)
+    ids = torch.tensor(np.asarray(t["page_values"]), dtype=torch.int64, device=DEV)
+    packed = pages.index_select(0, ids)
+    t_packed = dict(t, page_values=np.arange(ids.numel(), dtype=np.int32))
+    out_p, lse_p = _decode(q, packed, t_packed)
+    assert torch.equal(out_p, out) and torch.equal(lse_p, lse), f"{name}: result depends on where the pages lie"
+    del packed
     # the chunk merge done by the last workgroup of each (sequence, kv head) against the same
     # arithmetic in a second kernel: bit-identical, every time (a stale read of another
     # workgroup's partial state would show here)
