@@ -190,13 +190,69 @@ def test_float32_tree_attention_over_pages_and_refusals():
             0, 1.0, 1e4, d ** -0.5, TI(tindptr), TI(labels.reshape(-1)))
     assert_close(host(out), eo, what="f32 tree paged out", **tol(F32))
     assert_close(host(lse), el, atol=2e-4, rtol=1e-5, what="f32 tree paged lse")
-    # float32 storage is the plain cache: rotation inside the kernel and the sliding-window form are refused
-    with pytest.raises(KVError, match="plain cache only"):
-        dl.call("batch_prefill_paged_kv", T(q)[1], TI(qindptr), pages_dl, TI(pindptr), TI(pvalues), TI(last), TI(zb), TI(zq), out_dl,
-                lse_dl, 0, 1, 1.0, 1e4, d ** -0.5, 0)
+    # RoPE inside the kernel over a token tree in the page pool is not built (the reference's kernel asserts the same)
+    with pytest.raises(KVError, match="token trees over the page pool"):
+        dl.call("tree_attn_paged_kv", T(q)[1], TI(qindptr), pages_dl, TI(pindptr), TI(pvalues), TI(last), TI(zb), TI(zq), out_dl,
+                lse_dl, 1, 1.0, 1e4, d ** -0.5, TI(tindptr), TI(labels.reshape(-1)))
     with pytest.raises(KVError, match="float16"):   # mixed storage types in one call
         dl.call("batch_prefill_paged_kv", T(q.astype(F16))[1], TI(qindptr), pages_dl, TI(pindptr), TI(pvalues), TI(last), TI(zb),
                 TI(zq), out_dl, lse_dl, 0, 0, 1.0, 1e4, d ** -0.5, 0)
+
+
+@pytest.mark.parametrize("hq,hkv,d,ps", [(8, 2, 128, 16), (8, 4, 72, 12)])
+def test_float32_sliding_window_cache_window_mask_and_inline_rope(hq, hkv, d, ps):
+    """float32 storage with the (3, batch) length_info of a sliding-window cache, the per-layer window mask and RoPE
+    inside the kernel, through the tensor-level boundary: decode and paged prefill, ragged prefill with rotation."""
+    from tests.util import assert_close_where_keys, rows_without_keys
+    rng = np.random.default_rng(305 + d)
+    spec = [(100, 4, 20), (257, 0, 0), (330, 16, 48), (33, 2, 2), (ps, 0, 0), (90, 0, 17)]   # physical length, sink, window offset
+    need = 4 + sum((x[0] + ps - 1) // ps for x in spec)
+    pages, pindptr, pvalues, last, _, _ = build_paged_kv(rng, [x[0] for x in spec], need, hkv, ps, d, dtype=F32)
+    info = np.array([last, [x[2] for x in spec], [x[1] for x in spec]], np.int32)
+    logical = np.array([n - off + sink for n, sink, off in spec])
+    b = len(spec)
+    k_off = rng.integers(0, 200, size=b).astype(np.int32)
+    _, pages_dl = T(pages)
+    q = rng.standard_normal((b, hq, d)).astype(F32)
+    q_pos = (k_off + logical - 1).astype(np.int32)
+    for rotary in (0, 1):
+        eo, el = np.zeros((b, hq, d), F32), np.zeros((b, hq), F32)
+        ok.decode(q, pages, pindptr, pvalues, info, k_off, q_pos, eo, el, rotary, 1.0, 1e4, d ** -0.5)
+        out, out_dl = T(np.full((b, hq, d), 7.0, F32))
+        lse, lse_dl = T(np.full((b, hq), 7.0, F32))
+        dl.call("batch_decode_paged_kv", T(q)[1], pages_dl, TI(pindptr), TI(pvalues), TI(info), TI(k_off), TI(q_pos), out_dl, lse_dl,
+                rotary, 1.0, 1e4, d ** -0.5)
+        assert_close(host(out), eo, what=f"f32 sliding decode out, rotary {rotary}", atol=1e-3, rtol=1e-3)
+        assert_close(host(lse), el, atol=1e-3, rtol=1e-4, what=f"f32 sliding decode lse, rotary {rotary}")
+    sq_lens = [7, 64, 33, 3, 1, 30]
+    n = sum(sq_lens)
+    qindptr = np.concatenate([[0], np.cumsum(sq_lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F32)
+    q_pos = np.concatenate([k_off[i] + logical[i] - sq_lens[i] + np.arange(sq_lens[i]) for i in range(b)]).astype(np.int32)
+    for causal, window, rotary in ((0, 0, 1), (1, 40, 1), (1, 12, 0)):
+        eo, el = np.zeros((n, hq, d), F32), np.zeros((n, hq), F32)
+        ok.prefill_paged(q, qindptr, pages, pindptr, pvalues, info, k_off, q_pos, eo, el, causal, rotary, 1.0, 1e4, d ** -0.5,
+                         sliding_window_size=window)
+        out, out_dl = T(np.full((n, hq, d), 7.0, F32))
+        lse, lse_dl = T(np.full((n, hq), 7.0, F32))
+        dl.call("batch_prefill_paged_kv", T(q)[1], TI(qindptr), pages_dl, TI(pindptr), TI(pvalues), TI(info), TI(k_off), TI(q_pos),
+                out_dl, lse_dl, causal, rotary, 1.0, 1e4, d ** -0.5, window)
+        assert_close_where_keys(host(out), host(lse), eo, el, rows_without_keys(sq_lens, causal, window), 1e-3,
+                                f"f32 sliding paged, causal {causal}, window {window}, rotary {rotary}")
+    lens = [130, 5, 1, 70]
+    n = sum(lens)
+    ind = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    q, k, v = (rng.standard_normal((n, h, d)).astype(F32) for h in (hq, hkv, hkv))
+    off = rng.integers(0, 100, size=len(lens)).astype(np.int32)
+    pos = np.concatenate([off[i] + np.arange(lens[i]) for i in range(len(lens))]).astype(np.int32)
+    eo, el = np.zeros((n, hq, d), F32), np.zeros((n, hq), F32)
+    ok.prefill_ragged(q, ind, k, v, ind, pos, off, eo, el, 1, 1, 1.0, 1e4, d ** -0.5)
+    out, out_dl = T(np.full((n, hq, d), 7.0, F32))
+    lse, lse_dl = T(np.full((n, hq), 7.0, F32))
+    dl.call("batch_prefill_ragged_kv", T(q)[1], TI(ind), T(k)[1], T(v)[1], TI(ind), TI(pos), TI(off), out_dl, lse_dl, 1, 1, 1.0, 1e4,
+            d ** -0.5)
+    assert_close(host(out), eo, what="f32 ragged out, rotary", atol=1e-3, rtol=1e-3)
+    assert_close(host(lse), el, atol=1e-3, rtol=1e-4, what="f32 ragged lse, rotary")
 
 
 @pytest.mark.parametrize("hq,hkv,d,ps", [(32, 8, 128, 24), (8, 2, 64, 5), (8, 2, 128, 1), (8, 2, 72, 16), (16, 4, 40, 48),
@@ -291,6 +347,81 @@ def test_fp16_pages_and_head_dims_outside_the_tuned_set(hq, hkv, d, ps):
     assert np.array_equal(host(gv), ev)
     assert_close(host(gq), eq, atol=2e-3, rtol=2e-3, what="rope q")
     assert_close(host(gk), ek, atol=2e-3, rtol=2e-3, what="rope k")
+
+
+@pytest.mark.parametrize("hq,hkv,d,ps", [(16, 4, 96, 16), (8, 2, 80, 24), (8, 2, 128, 24), (8, 2, 48, 5), (4, 4, 160, 16),
+                                         (8, 1, 112, 32)])
+def test_fp16_extended_forms_outside_the_tuned_set(hq, hkv, d, ps):
+    """The sliding-window cache (attention sinks, an evicted gap), the per-layer window mask and RoPE inside the
+    kernel at head dims and page sizes the tuned extended kernels are not built for: paged prefill, decode, ragged
+    prefill, the ragged token-tree form, and a frequency variant."""
+    from tests.test_oracle_kernels import sliding_case
+    from tests.util import assert_close_where_keys, rows_without_keys
+    rng = np.random.default_rng(500 + d + ps)
+    spec = [(100, 4, 20), (257, 0, 0), (330, 16, 48), (33, 2, 2), (ps, 0, 0), (90, 0, 17), (900, 8, 40)]
+    spec = [(n, min(sink, n), min(max(off, min(sink, n)), n)) for n, sink, off in spec]
+    sq_lens = [7, 64, 33, 3, 1, 30, 40]
+    need = 4 + sum((x[0] + ps - 1) // ps for x in spec)
+    pages, pindptr, pvalues, info, k_log, _ = sliding_case(rng, spec, hkv, d, ps=ps, npages=need)
+    n = sum(sq_lens)
+    qindptr = np.concatenate([[0], np.cumsum(sq_lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(F16)
+    k_off = rng.integers(0, 200, size=len(spec)).astype(np.int32)
+    q_pos = np.concatenate([k_off[i] + len(k_log[i]) - sq_lens[i] + np.arange(sq_lens[i]) for i in range(len(spec))])
+    q_pos = q_pos.astype(np.int32)
+    for causal, window, rotary in ((0, 0, 1), (1, 40, 1), (1, 12, 0)):
+        eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), F32)
+        ok.prefill_paged(q, qindptr, pages, pindptr, pvalues, info, k_off, q_pos, eo, el, causal, rotary, 1.0, 1e4, d ** -0.5,
+                         sliding_window_size=window)
+        go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+        gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+        K.batch_prefill_paged_kv(dev(q), i32(qindptr), dev(pages), i32(pindptr), i32(pvalues), i32(info), i32(k_off), i32(q_pos),
+                                 go, gl, causal, rotary, 1.0, 1e4, d ** -0.5, sliding_window_size=window)
+        assert_close_where_keys(host(go), host(gl), eo, el, rows_without_keys(sq_lens, causal, window), 2e-3,
+                                f"sliding paged, causal {causal}, window {window}, rotary {rotary}")
+    b = len(spec)
+    qd = rng.standard_normal((b, hq, d)).astype(F16)
+    qd_pos = (k_off + np.array([len(k) for k in k_log]) - 1).astype(np.int32)
+    for rotary, scaling in ((0, None), (1, None), (1, {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                                       "high_freq_factor": 4.0, "original_max_position_embeddings": 64})):
+        eo, el = np.zeros((b, hq, d), F16), np.zeros((b, hq), F32)
+        with ok.inline_rope_scaling(scaling):
+            ok.decode(qd, pages, pindptr, pvalues, info, k_off, qd_pos, eo, el, rotary, 1.0, 1e4, d ** -0.5)
+        go = torch.full((b, hq, d), 7.0, dtype=torch.float16, device=DEV)
+        gl = torch.full((b, hq), 7.0, dtype=torch.float32, device=DEV)
+        K.batch_decode_paged_kv(dev(qd), dev(pages), i32(pindptr), i32(pvalues), i32(info), i32(k_off), i32(qd_pos), go, gl,
+                                rotary, 1.0, 1e4, d ** -0.5, rope_scaling=scaling)
+        assert_close(host(go), eo, what=f"sliding decode out, rotary {rotary}, {scaling and scaling['rope_type']}")
+        assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what=f"sliding decode lse, rotary {rotary}")
+    if d in (64, 128):
+        return  # the ragged forms of these head dims are the tuned kernels'
+    lens = [300, 5, 1, 200]
+    n = sum(lens)
+    ind = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    q, k, v = (rng.standard_normal((n, h, d)).astype(F16) for h in (hq, hkv, hkv))
+    k_off = rng.integers(0, 100, size=len(lens)).astype(np.int32)
+    q_pos = np.concatenate([k_off[i] + np.arange(lens[i]) for i in range(len(lens))]).astype(np.int32)
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), F32)
+    ok.prefill_ragged(q, ind, k, v, ind, q_pos, k_off, eo, el, 1, 1, 1.0, 1e4, d ** -0.5)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_prefill_ragged_kv(dev(q), i32(ind), dev(k), dev(v), i32(ind), i32(q_pos), i32(k_off), go, gl, 1, 1, 1.0, 1e4, d ** -0.5)
+    assert_close(host(go), eo, what="ragged out, rotary")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="ragged lse, rotary")
+    trees = REFERENCE_TREES + [random_forest(rng, 40)]
+    tl = [len(t) for t in trees]
+    n = sum(tl)
+    ind = np.concatenate([[0], np.cumsum(tl)]).astype(np.int32)
+    q, k, v = (rng.standard_normal((n, h, d)).astype(F16) for h in (hq, hkv, hkv))
+    mask = np.concatenate([tree_order(t) for t in trees]).astype(np.int32)
+    q_pos = rng.integers(0, 300, size=n).astype(np.int32)  # a node's depth in a real tree; any values pin the lookup
+    eo, el = np.zeros((n, hq, d), F16), np.zeros((n, hq), F32)
+    ok.tree_attn_ragged(q, ind, k, v, ind, q_pos, ind, mask, eo, el, 1, 1.0, 1e4, d ** -0.5)
+    go = torch.full((n, hq, d), 7.0, dtype=torch.float16, device=DEV)
+    gl = torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV)
+    K.batch_tree_attn(dev(q), i32(ind), dev(k), dev(v), i32(ind), i32(q_pos), i32(ind), i32(mask), go, gl, 1, 1.0, 1e4, d ** -0.5)
+    assert_close(host(go), eo, what="tree ragged out, rotary")
+    assert_close(host(gl), el, atol=2e-3, rtol=1e-4, what="tree ragged lse, rotary")
 
 
 def _random_generic_case(case):

@@ -320,7 +320,7 @@ def test_decode_inline_rope_plain_cache_and_scaled_positions():
 
 def test_decode_rejects_what_is_not_built():
     # head dims outside the tuned set run on the generic kernel, which takes multiples of 8 (fp16) up to 256, and
-    # only for a plain call: with rotation inside the kernel the tuned kernel is asked, and it has no head dim 72
+    # multiples of 16 with rotation inside the kernel
     t = torch.zeros((1, 8, 68), dtype=torch.float16, device=DEV)
     pages = torch.zeros((2, 2, 2, 16, 68), dtype=torch.float16, device=DEV)
     lse = torch.zeros((1, 8), dtype=torch.float32, device=DEV)
@@ -330,7 +330,7 @@ def test_decode_rejects_what_is_not_built():
     assert info.value.code == -2
     t = torch.zeros((1, 8, 72), dtype=torch.float16, device=DEV)
     pages = torch.zeros((2, 2, 2, 16, 72), dtype=torch.float16, device=DEV)
-    with pytest.raises(KVError, match="head_dim 72 is not built") as info:
+    with pytest.raises(KVError, match="multiple of 16, got 72") as info:
         K.batch_decode_paged_kv(t, pages, one, i32([0]), i32([1]), i32([0]), i32([0]), t, lse, 1, 1.0, 1e4, 1.0)
     assert info.value.code == -2
 
@@ -1045,20 +1045,22 @@ def test_decode_group_of_64_heads():
 
 
 def test_head_dims_between_64_and_128_refuse_what_they_do_not_have():
-    """Head dims 80, 96 and 112 run on the head dim 128 kernels of the plain cache; the sliding-window /
-    inline-RoPE forms and the one-pass chunked prefill are not built for them and say so."""
+    """Head dims 80, 96 and 112 run on the head dim 128 kernels of the plain cache and on the generic kernels in
+    the sliding-window / inline-RoPE forms (tests/test_gpu_generic.py); the one-pass chunked prefill and RoPE inside
+    the kernel at a head dim that is not a multiple of 16 are not built and say so."""
     t = torch.zeros((1, 8, 96), dtype=torch.float16, device=DEV)
     pages = torch.zeros((2, 2, 2, 16, 96), dtype=torch.float16, device=DEV)
     lse = torch.zeros((1, 8), dtype=torch.float32, device=DEV)
     one, z = i32([0, 1]), i32([0])
-    with pytest.raises(KVError, match="plain cache only") as info:
+    kv = torch.zeros((1, 2, 96), dtype=torch.float16, device=DEV)
+    with pytest.raises(KVError, match="is not built") as info:
+        K.batch_prefill_cached_and_new_kv(t, one, kv, kv, pages, one, z, i32([1]), t, lse, 1.0)
+    assert info.value.code == -2
+    t = torch.zeros((1, 8, 72), dtype=torch.float16, device=DEV)
+    pages = torch.zeros((2, 2, 2, 16, 72), dtype=torch.float16, device=DEV)
+    with pytest.raises(KVError, match="multiple of 16") as info:
         K.batch_decode_paged_kv(t, pages, one, z, i32([1]), z, z, t, lse, 1, 1.0, 1e4, 1.0)
     assert info.value.code == -2
-    with pytest.raises(KVError, match="plain cache only"):
-        K.batch_prefill_paged_kv(t, one, pages, one, z, i32([1]), z, z, t, lse, 1, 1, 1.0, 1e4, 1.0)
-    kv = torch.zeros((1, 2, 96), dtype=torch.float16, device=DEV)
-    with pytest.raises(KVError, match="is not built"):
-        K.batch_prefill_cached_and_new_kv(t, one, kv, kv, pages, one, z, i32([1]), t, lse, 1.0)
 
 
 # ------------------------------------------------------------------------------ frequency variants in the kernels

@@ -77,12 +77,12 @@ int StorageBits(std::initializer_list<Arg> args) {
   }
   return first.t->dtype.bits;
 }
-// float32 storage runs on the generic kernels: a plain cache, no rotation inside the attention kernels
-void PlainOnly(int bits, int64_t rotary_mode, int sliding, const char* what) {
-  if (bits == 16) return;
-  if (rotary_mode != 0 || sliding != 0) {
+// float32 storage runs on the generic kernels, which have no in-kernel RoPE over a token tree in the page pool
+// (the reference's kernel asserts the same, tree_attn.py:700-702)
+void NoRotaryTreeOverPages(int bits, int64_t rotary_mode, const char* what) {
+  if (bits == 32 && rotary_mode != 0) {
     Thrower t(TVMKV_EUNSUPPORTED, "");
-    t << what << ": float32 storage is built for the plain cache only (no sliding window, no RoPE inside the kernel)";
+    t << what << ": RoPE inside the kernel is not built for token trees over the page pool";
     t.Throw();
   }
 }
@@ -156,10 +156,20 @@ PagedShapes CheckPaged(const Arg& q, const Arg& pages, const Arg& page_indptr, c
 
 // The paged MHA slots on float32 storage: the generic kernel.
 GenericAttention PagedGeneric(const char* what, const PagedShapes& s, const Arg& q, const Arg* qo_indptr, const Arg& pages,
-                              const Arg& page_indptr, const Arg& page_indices, const Arg& length_info, const Arg& out,
-                              const Arg& lse, int64_t causal, double sm_scale) {
+                              const Arg& page_indptr, const Arg& page_indices, const Arg& length_info, const Arg& k_off,
+                              const Arg& q_pos, const Arg& out, const Arg& lse, int64_t causal, int64_t rotary_mode,
+                              double rope_scale, double rope_theta, const tvmkv_rope_scaling* rope_scaling,
+                              int64_t layer_window, double sm_scale) {
   GenericAttention a;
   a.what = what;
+  a.sliding_window = s.sliding;
+  a.layer_window = static_cast<int32_t>(layer_window);
+  a.rotary_mode = rotary_mode;
+  a.q_rope_position = q_pos.i32();
+  a.k_rope_pos_offset = k_off.i32();
+  a.rope_scale = rope_scale;
+  a.rope_theta = rope_theta;
+  a.rope_scaling = rope_scaling;
   a.elem_bits = 32;
   a.q = q.ptr();
   a.q_indptr = qo_indptr != nullptr ? qo_indptr->i32() : nullptr;
@@ -265,7 +275,6 @@ int tvmkv_dl_batch_prefill_ragged_kv_scaled(const DLTensor* q_, const DLTensor* 
   Arg out = Take(out_, "out", kStorage, {3}), lse = Take(lse_, "lse", kF32, {2});
   const int device = SameDevice({q, qo_indptr, k, v, kv_indptr, q_pos, k_off, out, lse});
   const int bits = StorageBits({q, k, v, out});
-  PlainOnly(bits, rotary_mode, 0, "batch_prefill_ragged_kv");
   const int64_t rows = q.dim(0);
   Expect(qo_indptr.dim(0) >= 1, qo_indptr, "(batch + 1,)");
   const int64_t batch = qo_indptr.dim(0) - 1;
@@ -295,6 +304,12 @@ int tvmkv_dl_batch_prefill_ragged_kv_scaled(const DLTensor* q_, const DLTensor* 
     a.d = static_cast<int32_t>(q.dim(2));
     a.causal = causal > 0;
     a.sm_scale = sm_scale;
+    a.rotary_mode = rotary_mode;
+    a.q_rope_position = q_pos.i32();
+    a.k_rope_pos_offset = k_off.i32();
+    a.rope_scale = rope_scale;
+    a.rope_theta = rope_theta;
+    a.rope_scaling = rope_scaling;
     Launch(device, [&] { return generic_attention(a, stream); });
     return TVMKV_OK;
   }
@@ -324,10 +339,10 @@ int tvmkv_dl_batch_prefill_paged_kv_scaled(const DLTensor* q_, const DLTensor* q
   const int bits = StorageBits({q, pages, out});
   const PagedShapes s = CheckPaged(q, pages, page_indptr, page_indices, length_info, k_off, q_pos, out, lse);
   Expect(qo_indptr.dim(0) == s.batch + 1, qo_indptr, "(batch + 1,)");
-  PlainOnly(bits, rotary_mode, s.sliding, "batch_prefill_paged_kv");
   if (bits == 32) {
     const GenericAttention a = PagedGeneric("batch_prefill_paged_kv", s, q, &qo_indptr, pages, page_indptr, page_indices,
-                                            length_info, out, lse, causal, sm_scale);
+                                            length_info, k_off, q_pos, out, lse, causal, rotary_mode, rope_scale, rope_theta,
+                                            rope_scaling, layer_sliding_window_size, sm_scale);
     Launch(device, [&] { return generic_attention(a, stream); });
     return TVMKV_OK;
   }
@@ -356,10 +371,10 @@ int tvmkv_dl_batch_decode_paged_kv_scaled(const DLTensor* q_, const DLTensor* pa
   const int bits = StorageBits({q, pages, out});
   const PagedShapes s = CheckPaged(q, pages, page_indptr, page_indices, length_info, k_off, q_pos, out, lse);
   Expect(s.rows == s.batch, q, "(batch, h_q, head_dim): one query per page-table entry");
-  PlainOnly(bits, rotary_mode, s.sliding, "batch_decode_paged_kv");
   if (bits == 32) {
     const GenericAttention a = PagedGeneric("batch_decode_paged_kv", s, q, nullptr, pages, page_indptr, page_indices, length_info,
-                                            out, lse, 0, sm_scale);
+                                            k_off, q_pos, out, lse, 0, rotary_mode, rope_scale, rope_theta, rope_scaling, 0,
+                                            sm_scale);
     Launch(device, [&] { return generic_attention(a, stream); });
     return TVMKV_OK;
   }
@@ -393,10 +408,10 @@ int tvmkv_dl_tree_attn_paged_kv(const DLTensor* q_, const DLTensor* qo_indptr_, 
   Expect(mn_indptr.dim(0) == s.batch + 1, mn_indptr, "(batch + 1,)");
   // two labels per tree node, flat (the reference uploads it so) or as (nodes, 2)
   Expect(mask.ndim() == 2 ? mask.dim(1) == 2 : mask.dim(0) % 2 == 0, mask, "(2 * nodes,) or (nodes, 2)");
-  PlainOnly(bits, rotary_mode, s.sliding, "tree_attn_paged_kv");
+  NoRotaryTreeOverPages(bits, rotary_mode, "tree_attn_paged_kv");
   if (bits == 32) {
-    GenericAttention a = PagedGeneric("tree_attn_paged_kv", s, q, &qo_indptr, pages, page_indptr, page_indices, length_info, out,
-                                      lse, 0, sm_scale);
+    GenericAttention a = PagedGeneric("tree_attn_paged_kv", s, q, &qo_indptr, pages, page_indptr, page_indices, length_info,
+                                      k_off, q_pos, out, lse, 0, 0, 1.0, 1e4, nullptr, 0, sm_scale);
     a.tree_indptr = mn_indptr.i32();
     a.tree_labels = mask.i32();
     Launch(device, [&] { return generic_attention(a, stream); });
@@ -423,7 +438,6 @@ int tvmkv_dl_batch_tree_attn_scaled(const DLTensor* q_, const DLTensor* qo_indpt
   Arg out = Take(out_, "out", kStorage, {3}), lse = Take(lse_, "lse", kF32, {2});
   const int device = SameDevice({q, qo_indptr, k, v, kv_indptr, q_pos, mn_indptr, mask, out, lse});
   const int bits = StorageBits({q, k, v, out});
-  PlainOnly(bits, rotary_mode, 0, "batch_tree_attn");
   const int64_t rows = q.dim(0);
   Expect(qo_indptr.dim(0) >= 1, qo_indptr, "(batch + 1,)");
   const int64_t batch = qo_indptr.dim(0) - 1;
@@ -454,6 +468,11 @@ int tvmkv_dl_batch_tree_attn_scaled(const DLTensor* q_, const DLTensor* qo_indpt
     a.h_kv = static_cast<int32_t>(k.dim(1));
     a.d = static_cast<int32_t>(q.dim(2));
     a.sm_scale = sm_scale;
+    a.rotary_mode = rotary_mode;  // key t of sequence b sits at q_rope_position[kv_indptr[b] + t]
+    a.q_rope_position = q_pos.i32();
+    a.rope_scale = rope_scale;
+    a.rope_theta = rope_theta;
+    a.rope_scaling = rope_scaling;
     Launch(device, [&] { return generic_attention(a, stream); });
     return TVMKV_OK;
   }

@@ -973,16 +973,27 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
 }
 
 // Shapes the tuned kernel is not built for (pages other than 16 / 32 / 64 / 128 tokens, other head dims) run on
-// the generic matrix-core kernel when the call is one it serves: a plain cache, no rotation inside the kernel.
+// the generic matrix-core kernel (sliding-window caches and RoPE inside the kernel included).  Head dims 80 / 96 /
+// 112 run on the tuned kernel in its plain form only.
 static bool decode_goes_generic(int64_t rotary_mode, int32_t sliding_window, int32_t d, int32_t page_size) {
-  return rotary_mode == 0 && sliding_window == 0 && (!tuned_page_size(page_size) || !tuned_head_dim(d));
+  const bool plain = rotary_mode == 0 && sliding_window == 0;
+  const bool tuned_dim = plain ? tuned_head_dim(d) : (d == 64 || d == 128 || d == 256);
+  return !tuned_page_size(page_size) || !tuned_dim;
 }
 static int decode_generic(const void* q, const void* pages, const int32_t* page_indptr, const int32_t* page_values,
-                          const int32_t* length_info, void* output, float* lse, double sm_scale, int32_t batch_size,
-                          int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv, int32_t d, int32_t page_size,
-                          void* stream) {
+                          const int32_t* length_info, const int32_t* k_rope_pos_offset, const int32_t* q_rope_position,
+                          void* output, float* lse, int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
+                          int32_t batch_size, int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv, int32_t d,
+                          int32_t page_size, int32_t sliding_window, const tvmkv_rope_scaling* rope_scaling, void* stream) {
   GenericAttention a;
   a.what = "batch_decode_paged_kv";
+  a.sliding_window = sliding_window;
+  a.rotary_mode = rotary_mode;
+  a.q_rope_position = q_rope_position;
+  a.k_rope_pos_offset = k_rope_pos_offset;
+  a.rope_scale = rope_scale;
+  a.rope_theta = rope_theta;
+  a.rope_scaling = rope_scaling;
   a.q = q;
   a.pages = pages;
   a.page_indptr = page_indptr;
@@ -1010,8 +1021,9 @@ extern "C" int tvmkv_batch_decode_paged_kv(const void* q, const void* pages, con
                                            int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
                                            int32_t d, int32_t page_size, int32_t sliding_window, void* stream) {
   if (decode_goes_generic(rotary_mode, sliding_window, d, page_size)) {
-    return decode_generic(q, pages, page_indptr, page_values, length_info, output, lse, sm_scale, batch_size, nnz_pages, num_pages,
-                          h_q, h_kv, d, page_size, stream);
+    return decode_generic(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, output, lse,
+                          rotary_mode, rope_scale, rope_theta, sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d,
+                          page_size, sliding_window, nullptr, stream);
   }
   KV_API_BEGIN();
   hipStream_t s = as_stream(stream);
@@ -1031,8 +1043,9 @@ extern "C" int tvmkv_batch_decode_paged_kv_scaled(const void* q, const void* pag
                                                   int32_t d, int32_t page_size, int32_t sliding_window,
                                                   const tvmkv_rope_scaling* rope_scaling, void* stream) {
   if (decode_goes_generic(rotary_mode, sliding_window, d, page_size)) {
-    return decode_generic(q, pages, page_indptr, page_values, length_info, output, lse, sm_scale, batch_size, nnz_pages, num_pages,
-                          h_q, h_kv, d, page_size, stream);
+    return decode_generic(q, pages, page_indptr, page_values, length_info, k_rope_pos_offset, q_rope_position, output, lse,
+                          rotary_mode, rope_scale, rope_theta, sm_scale, batch_size, nnz_pages, num_pages, h_q, h_kv, d,
+                          page_size, sliding_window, rope_scaling, stream);
   }
   KV_API_BEGIN();
   hipStream_t s = as_stream(stream);

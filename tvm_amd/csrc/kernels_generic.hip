@@ -54,6 +54,15 @@ struct GAttn {
   int64_t total_q;
   int batch, h_q, h_kv, d, page_size, causal, splits;
   float scale_log2;
+  // extended form (generic_attn_kernel<..., EXT = true>)
+  const int32_t* window_offset;      // paged, (batch): physical index of the first token of the window, or NULL
+  const int32_t* sink_size;          // paged, (batch): attention-sink tokens kept at the front, or NULL
+  int layer_window;                  // > 0 with causal and a sliding-window cache: the per-layer window mask
+  int rotary;                        // q and k are rotated inside the kernel
+  const int32_t* q_rope_position;    // (total_q) position of each query token
+  const int32_t* k_rope_pos_offset;  // (batch) position of logical key 0; NULL (ragged): key t of sequence b sits at
+                                     // q_rope_position[kv_indptr[b] + t]
+  float rope_scale;
 };
 
 constexpr float kMasked = -1.0e30f;  // a masked score; exp2 of it is 0 against any running maximum
@@ -93,13 +102,56 @@ __device__ __forceinline__ void store_run<half_t, 8>(half_t* p, const float* in)
 }
 __device__ __forceinline__ void store4(float* p, float4_t v) { *reinterpret_cast<float4_t*>(p) = v; }
 
+// In-kernel RoPE of one 16-byte piece of a q / k row (rotate-half over the whole head,
+// python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-127): x[f + e] of the piece at feature f, its partner piece
+// at f +- d/2 from the same row (d/2 is a whole number of pieces), float32 arithmetic, one rounding to the storage
+// type.  tbl: the table of InlineRopeTable in LDS.
+template <int N>
+__device__ __forceinline__ void rotate_run(float* x, const float* partner, bool upper_half, int f, float pos_scaled,
+                                           const float* tbl, int inverse, float magnitude) {
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    float sn, cs;
+    sincos_reduced(inverse ? pos_scaled * tbl[f + e] : pos_scaled / tbl[f + e], sn, cs);
+    x[e] = magnitude * (cs * x[e] + sn * (upper_half ? partner[e] : -partner[e]));
+  }
+}
+__device__ __forceinline__ half8_t rotate_piece(half8_t own, const half_t* row, int f, int d, float pos_scaled, const float* tbl,
+                                                int inverse, float magnitude) {
+  const bool upper = f >= d / 2;
+  const half8_t other = *reinterpret_cast<const half8_t*>(row + (upper ? f - d / 2 : f + d / 2));
+  float x[8], y[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    x[e] = static_cast<float>(own[e]);
+    y[e] = static_cast<float>(other[e]);
+  }
+  rotate_run<8>(x, y, upper, f, pos_scaled, tbl, inverse, magnitude);
+  half8_t out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = static_cast<half_t>(x[e]);
+  return out;
+}
+__device__ __forceinline__ void rotate_piece(float* own, const float* row, int f, int d, float pos_scaled, const float* tbl,
+                                             int inverse, float magnitude) {
+  const bool upper = f >= d / 2;
+  float y[4];
+  load_run<float, 4>(row + (upper ? f - d / 2 : f + d / 2), y);
+  rotate_run<4>(own, y, upper, f, pos_scaled, tbl, inverse, magnitude);
+}
+
 // workgroups per CU: the fp16 form holds its operands in half the registers
 constexpr int generic_workgroups(int elem_bytes, int dmax, int nb) {
   return elem_bytes == 2 ? (dmax > 128 ? 2 : (nb == 1 ? 4 : 3)) : (dmax > 128 ? 1 : (nb == 1 ? 3 : 2));
 }
 
-template <typename T, int DMAX, int NB>
-__global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void generic_attn_kernel(GAttn p) {
+// EXT adds what the extended tuned kernels add: the sliding-window cache (the page table covers `sink` tokens at the
+// front, evicted tokens up to `window_offset`, then the window; keys have logical indices, sink tokens first, that
+// the masks and RoPE use, _kernel_common.py:155-170), the per-layer sliding-window mask (:138-144) and RoPE inside
+// the kernel with any frequency variant (the table, one entry per element; the halves of a variant whose halves
+// differ are rotated by their own entries).
+template <typename T, int DMAX, int NB, bool EXT>
+__global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void generic_attn_kernel(GAttn p, InlineRopeTable rope) {
   constexpr bool HALF = sizeof(T) == 2;
   constexpr int ROWS = 16 * NB;
   constexpr int KS = DMAX / 16;  // output feature "blocks": lane (i, g) of the V^T operand owns features i * KS .. + KS - 1
@@ -109,6 +161,7 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
   static_assert(KS % VP == 0 && DMAX % (4 * PIECE) == 0, "head dim vs load width");
   __shared__ __attribute__((aligned(16))) float o_lds[2 * ROWS * DMAX];
   __shared__ float ml_lds[2 * ROWS * 2];
+  __shared__ float rope_lds[EXT ? kMaxHeadDim : 1];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -138,13 +191,24 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
   const int rows = qo_len * group;
   const int r0 = (slot - slot_begin(b)) * ROWS;
   if (r0 >= rows) return;  // the whole workgroup: a slot beyond the sequence's last row tile
+  const bool rotary = EXT && p.rotary != 0;
+  if (EXT && rotary) {
+    if (tid < d) rope_lds[tid] = rope.v[tid];
+    __syncthreads();
+  }
 
   const bool paged = p.pages != nullptr;
   int kv_len, kv_start = 0, pbeg = 0;
+  int sink = 0, window_first = 0;  // logical key t lies at physical index t (t < sink) or t - sink + window_first
   if (paged) {
     pbeg = p.page_indptr[b];
     const int npages = p.page_indptr[b + 1] - pbeg;
     kv_len = npages > 0 ? (npages - 1) * p.page_size + p.last_page_len[b] : 0;  // _kernel_common.py:155-159
+    if (EXT && p.window_offset != nullptr && npages > 0) {
+      sink = p.sink_size[b];
+      window_first = p.window_offset[b];
+      kv_len = kv_len - window_first + sink;
+    }
   } else {
     kv_start = p.kv_indptr[b];
     kv_len = p.kv_indptr[b + 1] - kv_start;
@@ -157,9 +221,13 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
     tree_start = kv_len - tree_len;
   }
   const bool causal = p.causal != 0 && !tree;
+  // the per-layer window mask replaces the causal one: query i of the chunk sees the last max(window - i - 1, 0)
+  // cached keys (_kernel_common.py:138-144; sliding-window caches only, as the reference passes it)
+  const bool windowed = EXT && causal && p.layer_window > 0 && p.window_offset != nullptr;
 
-  // this lane's query rows (one per 16-row block): key limit, tree label, q fragments
+  // this lane's query rows (one per 16-row block): key limits, tree label, q fragments
   int limit[NB];
+  int lower[NB];
   int child_first[NB];
   float qf[NB][QS][PIECE];  // float32 storage
   half8_t qh[NB][QS];       // fp16 storage: the pieces as they are in memory
@@ -170,7 +238,8 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
     const bool valid = row < rows;
     const int qi = valid ? row / group : 0;
     const int head = kvh * group + (valid ? row % group : 0);
-    limit[nb] = !valid ? 0 : (causal ? max(0, min(kv_len, kv_len - qo_len + qi + 1)) : kv_len);
+    limit[nb] = !valid ? 0 : (causal && !windowed ? max(0, min(kv_len, kv_len - qo_len + qi + 1)) : kv_len);
+    lower[nb] = windowed ? max(kv_len - max(p.layer_window - qi - 1, 0), 0) : 0;
     child_first[nb] = 0;
     if (tree && valid && tree_len > 0) {  // the queries are the last qo_len nodes of the tree
       const int node = min(max(qi + tree_len - qo_len, 0), tree_len - 1);
@@ -189,14 +258,25 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
 #pragma unroll
         for (int e = 0; e < PIECE; ++e) qf[nb][s][e] = 0.f;
       }
+      if (EXT && rotary && valid && f < d) {
+        const float pos = static_cast<float>(p.q_rope_position[q_start + qi]) * p.rope_scale;
+        if constexpr (HALF) {
+          qh[nb][s] = rotate_piece(qh[nb][s], qrow, f, d, pos, rope_lds, rope.inverse, rope.magnitude);
+        } else {
+          rotate_piece(qf[nb][s], qrow, f, d, pos, rope_lds, rope.inverse, rope.magnitude);
+        }
+      }
     }
   }
   // keys of this row tile, and this workgroup's share of their 16-key blocks
   const int last_row = min(rows, r0 + ROWS) - 1;
-  const int tile_limit = causal ? max(0, min(kv_len, kv_len - qo_len + last_row / group + 1)) : kv_len;
-  const int nkb = (tile_limit + 15) / 16;
-  const int kb_lo = static_cast<int>(static_cast<int64_t>(split) * nkb / p.splits);
-  const int kb_hi = static_cast<int>(static_cast<int64_t>(split + 1) * nkb / p.splits);
+  const int tile_limit = causal && !windowed ? max(0, min(kv_len, kv_len - qo_len + last_row / group + 1)) : kv_len;
+  // the first row of the tile sees the most keys of the window
+  const int tile_lower = windowed ? max(kv_len - max(p.layer_window - r0 / group - 1, 0), 0) : 0;
+  const int kb_first = tile_lower / 16;
+  const int nkb = max((tile_limit + 15) / 16 - kb_first, 0);
+  const int kb_lo = kb_first + static_cast<int>(static_cast<int64_t>(split) * nkb / p.splits);
+  const int kb_hi = kb_first + static_cast<int>(static_cast<int64_t>(split + 1) * nkb / p.splits);
 
   float m[NB], lsum[NB];
   float4_t o[NB][KS];
@@ -219,9 +299,10 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
     const int t = min(kb * 16 + j, kv_len - 1);
     int krow, vrow;
     if (paged) {
-      const int pg = t / ps;
+      const int at = EXT && t >= sink ? t - sink + window_first : t;  // _kernel_common.py:162-170
+      const int pg = at / ps;
       const int page = p.page_values[pbeg + pg];
-      krow = ((page * 2) * p.h_kv + kvh) * ps + (t - pg * ps);  // pages (num_pages, 2, h_kv, page_size, d)
+      krow = ((page * 2) * p.h_kv + kvh) * ps + (at - pg * ps);  // pages (num_pages, 2, h_kv, page_size, d)
       vrow = krow + p.h_kv * ps;
     } else {
       krow = vrow = (kv_start + t) * p.h_kv + kvh;
@@ -240,6 +321,21 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
       } else {
 #pragma unroll
         for (int e = 0; e < PIECE; ++e) kf[s][e] = 0.f;
+      }
+    }
+    if (EXT && rotary) {
+      const int key_pos = p.k_rope_pos_offset != nullptr ? p.k_rope_pos_offset[b] + t : p.q_rope_position[kv_start + t];
+      const float pos = static_cast<float>(key_pos) * p.rope_scale;
+#pragma unroll
+      for (int s = 0; s < QS; ++s) {
+        const int f = (4 * s + g) * PIECE;
+        if (f < d) {
+          if constexpr (HALF) {
+            kh[s] = rotate_piece(kh[s], krow_ptr, f, d, pos, rope_lds, rope.inverse, rope.magnitude);
+          } else {
+            rotate_piece(kf[s], krow_ptr, f, d, pos, rope_lds, rope.inverse, rope.magnitude);
+          }
+        }
       }
     }
     // V^T operands: features j * KS .. + KS - 1 of the four keys 4 g + m
@@ -295,7 +391,7 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int key = kb * 16 + 4 * g + r;
-        bool visible = key < limit[nb];
+        bool visible = key < limit[nb] && key >= lower[nb];
         if (in_tree && key >= tree_start && key < kv_len) {  // tree_attn.py:48-65
           const int32_t* parent = p.tree_labels + 2 * static_cast<int64_t>(tree_base + key - tree_start);
           visible = visible && child_first[nb] >= parent[0] && child_first[nb] < parent[1];
@@ -435,21 +531,21 @@ __global__ __launch_bounds__(64) void generic_merge_kernel(const float* part_o, 
   if (threadIdx.x == 0) lse[row] = any ? s_max + fast_log2(total) : kNegInit;
 }
 
-template <typename T>
-void launch_attention(const GAttn& p, int rows_hint, hipStream_t stream) {
+template <typename T, bool EXT>
+void launch_attention(const GAttn& p, const InlineRopeTable& rope, int rows_hint, hipStream_t stream) {
   const int group = p.h_q / p.h_kv;
   auto run = [&](auto kernel, int rows_per_tile) {
     const int64_t slots = p.total_q * group / rows_per_tile + p.batch;
     KV_CHECK(slots < (int64_t{1} << 31)) << "too many row tiles for one launch";
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(slots), p.h_kv, p.splits), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(slots), p.h_kv, p.splits), dim3(256), 0, stream, p, rope);
   };
   const bool wide = rows_hint > 16;  // more than one 16-row block per (sequence, kv head) on average
   if (p.d <= 64) {
-    if (wide) run(generic_attn_kernel<T, 64, 2>, 32); else run(generic_attn_kernel<T, 64, 1>, 16);
+    if (wide) run(generic_attn_kernel<T, 64, 2, EXT>, 32); else run(generic_attn_kernel<T, 64, 1, EXT>, 16);
   } else if (p.d <= 128) {
-    if (wide) run(generic_attn_kernel<T, 128, 2>, 32); else run(generic_attn_kernel<T, 128, 1>, 16);
+    if (wide) run(generic_attn_kernel<T, 128, 2, EXT>, 32); else run(generic_attn_kernel<T, 128, 1, EXT>, 16);
   } else {
-    run(generic_attn_kernel<T, 256, 1>, 16);
+    run(generic_attn_kernel<T, 256, 1, EXT>, 16);
   }
   KV_LAUNCH_CHECK();
 }
@@ -468,6 +564,16 @@ int generic_attention(const GenericAttention& a, void* stream_) {
   if (a.batch == 0 || a.total_q == 0) return TVMKV_OK;
   const bool paged = a.pages != nullptr;
   KV_CHECK(a.q && a.out && a.lse) << a.what << ": NULL tensor";
+  const bool sliding = paged && a.sliding_window != 0;
+  const bool rotary = a.rotary_mode != 0;
+  KV_CHECK(a.sliding_window == 0 || paged) << a.what << ": a sliding-window cache is a paged one";
+  if (rotary) {
+    KV_CHECK(a.q_rope_position != nullptr) << a.what << ": NULL q_rope_position";
+    KV_CHECK(!paged || a.k_rope_pos_offset != nullptr) << a.what << ": NULL k_rope_pos_offset";
+    KV_UNSUPPORTED(a.d % (f32 ? 8 : 16) != 0)
+        << a.what << ": RoPE inside the generic kernels needs a head dim that is a multiple of " << (f32 ? 8 : 16) << ", got "
+        << a.d << " (an element and its partner half a head away are loaded as whole 16-byte pieces)";
+  }
   if (paged) {
     KV_CHECK(a.page_indptr && a.page_values && a.last_page_len && a.page_size > 0) << a.what << ": NULL page table or bad page size";
     KV_CHECK(a.num_pages * 2 * a.h_kv * a.page_size < (int64_t{1} << 31)) << a.what << ": the page pool has too many rows for 32-bit row ids";
@@ -499,6 +605,23 @@ int generic_attention(const GenericAttention& a, void* stream_) {
   p.page_size = a.page_size;
   p.causal = a.causal;
   p.scale_log2 = static_cast<float>(a.sm_scale) * kLog2e;
+  // length_info of a sliding-window cache: (3, batch) = last page length, window offset, sink size (attn_utils.h:483-495)
+  p.window_offset = sliding ? a.last_page_len + a.batch : nullptr;
+  p.sink_size = sliding ? a.last_page_len + 2 * static_cast<int64_t>(a.batch) : nullptr;
+  p.layer_window = sliding ? a.layer_window : 0;
+  p.rotary = rotary ? 1 : 0;
+  p.q_rope_position = a.q_rope_position;
+  p.k_rope_pos_offset = a.k_rope_pos_offset;
+  p.rope_scale = static_cast<float>(a.rope_scale);
+  InlineRopeTable rope{};
+  if (rotary) {
+    const InlineRopeHost table = inline_rope_table(a.rope_scaling, a.d, a.rope_theta);
+    for (int i = 0; i < a.d; ++i) rope.v[i] = table.v[i];
+    rope.inverse = table.inverse;
+    rope.halves_differ = table.halves_differ;
+    rope.magnitude = table.magnitude;
+  }
+  const bool ext = sliding || rotary;
   const int group = a.h_q / a.h_kv;
   const int rows_hint = static_cast<int>(std::min<int64_t>(a.total_q * group / a.batch, 1 << 20));
   // Few row tiles against long page lists: split the keys over workgroups until the chip has ~8 workgroups
@@ -519,7 +642,11 @@ int generic_attention(const GenericAttention& a, void* stream_) {
     p.part_o = reinterpret_cast<float*>(lease.ptr);
     p.part_s = reinterpret_cast<float*>(lease.ptr + o_bytes);
   }
-  if (f32) launch_attention<float>(p, rows_hint, stream); else launch_attention<half_t>(p, rows_hint, stream);
+  if (f32) {
+    if (ext) launch_attention<float, true>(p, rope, rows_hint, stream); else launch_attention<float, false>(p, rope, rows_hint, stream);
+  } else {
+    if (ext) launch_attention<half_t, true>(p, rope, rows_hint, stream); else launch_attention<half_t, false>(p, rope, rows_hint, stream);
+  }
   if (p.splits > 1) {
     const int64_t rows = a.total_q * a.h_q;
     if (f32) {

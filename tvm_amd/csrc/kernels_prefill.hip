@@ -992,10 +992,17 @@ static int ragged_prefill(const void* q, const int32_t* q_indptr, const void* k,
                           int64_t rotary_mode, double rope_scale, double rope_theta, double sm_scale,
                           int32_t batch_size, int64_t total_q, int32_t h_q, int32_t h_kv, int32_t d_qk,
                           int32_t d_v, const tvmkv_rope_scaling* scaling, void* stream) {
-  // head dims the tuned kernel is not built for: the generic matrix-core kernel (no rotation inside it)
-  if (rotary_mode == 0 && d_qk == d_v && !tuned_head_dim(d_qk)) {
+  // head dims the tuned kernel is not built for (80 / 96 / 112 with RoPE inside the kernel among them): the generic
+  // matrix-core kernel
+  if (d_qk == d_v && !(rotary_mode == 0 ? tuned_head_dim(d_qk) : (d_qk == 64 || d_qk == 128 || d_qk == 256))) {
     GenericAttention a;
     a.what = "batch_prefill_ragged_kv";
+    a.rotary_mode = rotary_mode;
+    a.q_rope_position = q_rope_position;
+    a.k_rope_pos_offset = k_rope_pos_offset;
+    a.rope_scale = rope_scale;
+    a.rope_theta = rope_theta;
+    a.rope_scaling = scaling;
     a.q = q;
     a.q_indptr = q_indptr;
     a.k = k;
@@ -1085,11 +1092,20 @@ static int paged_prefill(const void* q, const int32_t* q_indptr, const void* pag
                          int32_t h_kv, int32_t d, int32_t page_size, int32_t sliding_window,
                          int32_t sliding_window_size, bool merge_into, void* stream,
                          const tvmkv_rope_scaling* scaling = nullptr) {
-  // pages other than 16 / 32 / 64 / 128 tokens, other head dims: the generic matrix-core kernel, for a plain
-  // cache without rotation inside the kernel (its caller merges states with merge_state_inplace)
-  if (rotary_mode == 0 && sliding_window == 0 && !merge_into && (!tuned_page_size(page_size) || !tuned_head_dim(d))) {
+  // pages other than 16 / 32 / 64 / 128 tokens, other head dims (80 / 96 / 112 with a sliding-window cache or RoPE
+  // inside the kernel among them): the generic matrix-core kernel (its caller merges states with merge_state_inplace)
+  const bool plain = rotary_mode == 0 && sliding_window == 0;
+  if (!merge_into && (!tuned_page_size(page_size) || !(plain ? tuned_head_dim(d) : (d == 64 || d == 128 || d == 256)))) {
     GenericAttention a;
     a.what = "batch_prefill_paged_kv";
+    a.sliding_window = sliding_window;
+    a.layer_window = sliding_window_size;
+    a.rotary_mode = rotary_mode;
+    a.q_rope_position = q_rope_position;
+    a.k_rope_pos_offset = k_rope_pos_offset;
+    a.rope_scale = rope_scale;
+    a.rope_theta = rope_theta;
+    a.rope_scaling = scaling;
     a.q = q;
     a.q_indptr = q_indptr;
     a.pages = pages;
@@ -1295,9 +1311,14 @@ static int tree_attn_ragged(const void* q, const int32_t* q_indptr, const void* 
                             const int32_t* mask, void* output, float* lse, int64_t rotary_mode, double rope_scale,
                             double rope_theta, double sm_scale, int32_t batch_size, int64_t total_q, int32_t h_q,
                             int32_t h_kv, int32_t d, const tvmkv_rope_scaling* scaling, void* stream) {
-  if (rotary_mode == 0 && d != 64 && d != 128 && d != 256) {  // the generic matrix-core kernel
+  if (d != 64 && d != 128 && d != 256) {  // the generic matrix-core kernel
     GenericAttention a;
     a.what = "batch_tree_attn";
+    a.rotary_mode = rotary_mode;  // key t of sequence b sits at q_rope_position[kv_indptr[b] + t]
+    a.q_rope_position = q_rope_position;
+    a.rope_scale = rope_scale;
+    a.rope_theta = rope_theta;
+    a.rope_scaling = scaling;
     a.q = q;
     a.q_indptr = q_indptr;
     a.k = k;
@@ -1380,9 +1401,10 @@ int tvmkv_tree_attn_paged_kv(const void* q, const int32_t* q_indptr, const void*
                              const int32_t* tree_order_indptr, const int32_t* tree_order, int32_t batch_size,
                              int64_t total_q, int64_t nnz_pages, int64_t num_pages, int32_t h_q, int32_t h_kv,
                              int32_t d, int32_t page_size, int32_t sliding_window, void* stream) {
-  if (rotary_mode == 0 && sliding_window == 0 && (!tuned_page_size(page_size) || (d != 64 && d != 128 && d != 256))) {
+  if (rotary_mode == 0 && (!tuned_page_size(page_size) || (d != 64 && d != 128 && d != 256))) {
     GenericAttention a;  // the generic matrix-core kernel
     a.what = "tree_attn_paged_kv";
+    a.sliding_window = sliding_window;
     a.q = q;
     a.q_indptr = q_indptr;
     a.pages = pages;

@@ -7,8 +7,8 @@
 // everything else those factories accept for a plain cache -- float32 storage, any page size, any head dim
 // that is a multiple of 4 (fp32) or 8 (fp16) up to 256 -- runs on the generic matrix-core kernels of
 // kernels_generic.hip: float32 arithmetic throughout (v_mfma_f32_16x16x4_f32), K and V rows read straight
-// from their pages with one page-table lookup per row.  Not built there: the sliding-window cache
-// (length_info (3, batch)), RoPE inside the attention kernels (rotary_mode 1), MLA.
+// from their pages with one page-table lookup per row, the sliding-window cache (length_info (3, batch)), the
+// per-layer window mask and RoPE inside the kernel included.  Not built there: MLA.
 //
 // elem_bits is 16 or 32.  The functions return the library's error codes and leave the message in the
 // thread's last-error slot, like the extern "C" launchers they stand beside; they are internal: the
@@ -54,6 +54,20 @@ struct GenericAttention {
   int32_t causal = 0;
   double sm_scale = 1.0;
   const char* what = "attention";
+  // The extended form, as the tuned kernels have it.  sliding_window: last_page_len is the (3, batch) length_info of
+  // a sliding-window cache (last page length, window offset, sink size; attn_utils.h:483-495), keys have logical
+  // indices, the sink tokens first (_kernel_common.py:155-170); layer_window > 0 with causal on such a cache: the
+  // per-layer window mask (:138-144).  rotary_mode 1: q and k are rotated inside the kernel, query token i at
+  // q_rope_position[i], logical key t of sequence b at k_rope_pos_offset[b] + t (ragged with k_rope_pos_offset NULL:
+  // at q_rope_position[kv_indptr[b] + t], the token-tree form, tree_attn.py:93-259), frequencies of rope_scaling
+  // (NULL: the default ones).  Needs a head dim that is a multiple of 16 (fp16) or 8 (float32).
+  int32_t sliding_window = 0;
+  int32_t layer_window = 0;
+  int64_t rotary_mode = 0;
+  const int32_t* q_rope_position = nullptr;
+  const int32_t* k_rope_pos_offset = nullptr;
+  double rope_scale = 1.0, rope_theta = 1e4;
+  const tvmkv_rope_scaling* rope_scaling = nullptr;
 };
 int generic_attention(const GenericAttention& args, void* stream);
 
