@@ -108,11 +108,13 @@ class inline_rope_scaling:
         self.sc = None if not rope_scaling else RopeScaling.from_dict(rope_scaling)
 
     def __enter__(self):
-        lib().orc_set_inline_rope_scaling(None if self.sc is None else ctypes.byref(self.sc))
+        for each in (lib(), lib(np.empty(0, np.float32))):  # both builds: the storage type of the call decides later
+            each.orc_set_inline_rope_scaling(None if self.sc is None else ctypes.byref(self.sc))
         return self
 
     def __exit__(self, *exc):
-        lib().orc_set_inline_rope_scaling(None)
+        for each in (lib(), lib(np.empty(0, np.float32))):
+            each.orc_set_inline_rope_scaling(None)
         return False
 
 

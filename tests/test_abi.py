@@ -61,7 +61,7 @@ def test_version_and_error_channel():
     # argument validation happens before any device work, so it can be exercised without a GPU
     rc = lib.tvmkv_batch_decode_paged_kv(None, None, None, None, None, None, None, None, None, 1, 1.0, 1e4, 1.0,
                                          1, 1, 1, 8, 2, 72, 16, 0, None)
-    assert rc == -2 and b"head_dim 72 is not built" in lib.tvmkv_last_error()
+    assert rc == -2 and b"multiple of 16, got 72" in lib.tvmkv_last_error()
     rc = lib.tvmkv_batch_decode_paged_kv(None, None, None, None, None, None, None, None, None, 0, 1.0, 1e4, 1.0,
                                          1, 1, 1, 8, 2, 128, 16, 0, None)
     assert rc == -1 and b"NULL tensor" in lib.tvmkv_last_error()

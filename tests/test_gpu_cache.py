@@ -158,10 +158,35 @@ def test_storage_type_of_the_tensors_is_checked():
     out = torch.zeros((2, 8, 128), dtype=torch.float16, device=DEV)
     with pytest.raises(tvm_amd.KVError, match="stores float32"):
         gf("vm.builtin.attention_kv_cache_attention_with_fused_qkv")(cache.cache, 0, 1.0, qkv, out)
-    with pytest.raises(tvm_amd.KVError, match="plain cache"):
-        GpuCache([4, 64, 32, 16, 1], 1, 8, 2, 128, 128, dtype=np.float32)   # float32 storage with a sliding window
-    with pytest.raises(tvm_amd.KVError, match="plain cache"):
-        GpuCache([4, 64, 32, 24, 0], 1, 8, 2, 128, 128, rope_mode=2)         # pages of 24 tokens with inline RoPE
+
+
+@pytest.mark.parametrize("dtype,page_size,d,tol", [(np.float16, 16, 96, 4e-3), (np.float32, 16, 128, 1e-3),
+                                                   (np.float16, 24, 128, 4e-3), (np.float32, 12, 72, 1e-3)])
+@pytest.mark.parametrize("runner", [S.run_sliding_window, S.run_sliding_window_fork, S.run_sliding_window_page_reuse])
+def test_sliding_window_scenarios_on_the_generic_kernels(runner, dtype, page_size, d, tol):
+    """The reference's sliding-window scenarios (attention sinks, window trimming, forks inside the sink, page reuse;
+    test_runtime_builtin_paged_attention_kv_cache_cpu.py:912-1022) on caches that the tuned extended kernels do not
+    serve: head dim 96, float32 storage, pages of 24 and 12 tokens.  Such a cache rotates inside the attention
+    kernels and hands them the (3, batch) length_info."""
+    layers, hq, hkv = 2, 8, 2
+    cache = GpuCache([32, 2048, 512, page_size, 1], layers, hq, hkv, d, d, rope_mode=S.ROPE_INLINE, dtype=dtype)
+    sc = S.Scenario(cache, layers, hq, hkv, d, rope_mode=S.ROPE_INLINE, seed=4, tol=tol, dtype=dtype)
+    runner(sc)
+
+
+@pytest.mark.parametrize("dtype,page_size,d", [(np.float16, 16, 80), (np.float32, 16, 64), (np.float16, 40, 128)])
+@pytest.mark.parametrize("sliding", [0, 1])
+def test_inline_rope_and_forks_on_the_generic_kernels(dtype, page_size, d, sliding):
+    """Caches that rotate inside the attention kernels (rope mode 2, with and without sliding-window support) at a
+    head dim, a storage type and a page size of the generic kernels, with a frequency variant: prefill (ragged +
+    paged + merge), decode, a fork with two block depths, against the oracle cache."""
+    rope = dict(rope_theta=5e5, rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                              "high_freq_factor": 4.0, "original_max_position_embeddings": 64})
+    m = Mirror([8, 2048, 512, page_size, sliding], 2, 8, 2, d, rope_mode=2, dtype=dtype, **rope)
+    m.step([(0, 60), (1, 88), (2, 17)])
+    m.step([(0, 1), (1, 1), (2, 1)])
+    m.step([((3, 1, 40), 25), (0, 2)])
+    m.step([(3, 1), (1, 1)])
 
 
 def test_short_chunk_against_a_long_cached_sequence():

@@ -301,7 +301,8 @@ class _Fake:
 
 def test_storage_types_and_shapes_a_cache_accepts():
     """float16 and float32 storage (the reference's tests run both); float32, pages other than 16 / 32 / 64 / 128
-    tokens and other head dims are the plain cache (no sliding window, no RoPE inside the attention kernels)."""
+    tokens and other head dims run on the generic kernels, sliding windows and RoPE inside the attention kernels
+    included (that rotation needs a head dim that is a multiple of 16, of 8 with float32)."""
     import torch
     create = tvm_amd.get_global_func("vm.builtin.paged_attention_kv_cache_create")
 
@@ -313,11 +314,13 @@ def test_storage_types_and_shapes_a_cache_accepts():
         assert cache.dtype_bits == (16 if dtype == torch.float16 else 32)
         tvm_amd.get_global_func("vm.builtin.kv_state_add_sequence")(cache, 0)
     make([4, 64, 32, 24, 0], 72, 1, torch.float16)           # pages of 24 tokens, head dim 72: the generic kernels
-    with pytest.raises(tvm_amd.KVError, match="plain cache"):
-        make([4, 64, 32, 24, 1], 128, 0, torch.float16)      # pages of 24 tokens with a sliding window
-    with pytest.raises(tvm_amd.KVError, match="plain cache"):
-        make([4, 64, 32, 16, 1], 128, 1, torch.float32)      # float32 with a sliding window
-    with pytest.raises(tvm_amd.KVError, match="plain cache"):
-        make([4, 64, 32, 24, 0], 128, 2, torch.float16)      # pages of 24 tokens with RoPE inside the kernels
+    make([4, 64, 32, 24, 1], 128, 0, torch.float16)          # pages of 24 tokens with a sliding window
+    make([4, 64, 32, 16, 1], 128, 1, torch.float32)          # float32 with a sliding window (which rotates in the kernels)
+    make([4, 64, 32, 24, 0], 128, 2, torch.float16)          # pages of 24 tokens with RoPE inside the kernels
+    make([4, 64, 32, 16, 1], 96, 1, torch.float16)           # head dim 96 with a sliding window
+    with pytest.raises(tvm_amd.KVError, match="multiple of 16"):
+        make([4, 64, 32, 16, 0], 72, 2, torch.float16)       # RoPE inside the kernels at head dim 72
+    with pytest.raises(tvm_amd.KVError, match="multiple of 8"):
+        make([4, 64, 32, 16, 1], 68, 1, torch.float32)
     with pytest.raises(tvm_amd.KVError, match="float16 and float32"):
         make([4, 64, 32, 16, 0], 128, 1, torch.bfloat16)

@@ -161,3 +161,34 @@ def test_tree_attn_paged_f32_and_odd_page_size():
             eo, el = cf.attention(q[s:e], ks[i], vs[i], d ** -0.5, mask=m)
             assert_close(out[s:e], eo, atol=tol, rtol=tol, what=f"tree paged out seq {i} {dtype.__name__}")
             assert_close(lse[s:e], el, atol=max(tol, 1e-4), rtol=1e-5, what=f"tree paged lse seq {i}")
+
+
+def test_inline_rope_variant_and_sliding_cache_in_the_f32_build():
+    """rotary_mode 1 with a frequency variant and the (3, batch) length_info of a sliding-window cache in the float32
+    build: the variant is a library setting that both builds must receive (without it the float32 build rotates
+    with the default frequencies), and the float32 build must agree with the fp16 build on the same values up to
+    the fp16 roundings of that build."""
+    rng = np.random.default_rng(210)
+    hq, hkv, d, ps = 8, 2, 64, 16
+    spec = [(100, 4, 20), (57, 0, 0), (33, 2, 2)]  # physical length, sink, window offset
+    pages, indptr, values, last, _, _ = build_paged_kv(rng, [x[0] for x in spec], 16, hkv, ps, d, dtype=F32)
+    info = np.array([last, [x[2] for x in spec], [x[1] for x in spec]], np.int32)
+    b = len(spec)
+    q = rng.standard_normal((b, hq, d)).astype(F32)
+    k_off = np.array([0, 300, 4000], np.int32)
+    q_pos = (k_off + np.array([n - off + sink for n, sink, off in spec]) - 1).astype(np.int32)
+    scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": 64}
+    outs = {}
+    for name, sc in (("default", None), ("llama3", scaling)):
+        with ok.inline_rope_scaling(sc):
+            o32, l32 = np.zeros((b, hq, d), F32), np.zeros((b, hq), F32)
+            ok.decode(q, pages, indptr, values, info, k_off, q_pos, o32, l32, 1, 1.0, 1e4, d ** -0.5)
+            o16, l16 = np.zeros((b, hq, d), np.float16), np.zeros((b, hq), F32)
+            ok.decode(q.astype(np.float16), pages.astype(np.float16), indptr, values, info, k_off, q_pos, o16, l16, 1, 1.0, 1e4,
+                      d ** -0.5)
+        assert_close(o32, o16, atol=1e-2, rtol=1e-2, what=f"f32 build vs fp16 build, {name}")
+        assert_close(l32, l16, atol=5e-2, rtol=1e-3, what=f"f32 build vs fp16 build lse, {name}")
+        outs[name] = o32
+    # the variant changes the result: long positions rotate differently
+    assert np.abs(outs["default"] - outs["llama3"]).max() > 1e-2

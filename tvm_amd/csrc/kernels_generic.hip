@@ -561,18 +561,21 @@ int generic_attention(const GenericAttention& a, void* stream_) {
   KV_UNSUPPORTED(a.d <= 0 || a.d > 256 || a.d % (f32 ? 4 : 8) != 0)
       << a.what << ": head_dim " << a.d << " is not built (the generic kernels take multiples of " << (f32 ? 4 : 8)
       << " up to 256)";
+  const bool rotary = a.rotary_mode != 0;
+  KV_UNSUPPORTED(rotary && a.d % (f32 ? 8 : 16) != 0)
+      << a.what << ": RoPE inside the generic kernels needs a head dim that is a multiple of " << (f32 ? 8 : 16) << ", got "
+      << a.d << " (an element and its partner half a head away are loaded as whole 16-byte pieces)";
   if (a.batch == 0 || a.total_q == 0) return TVMKV_OK;
   const bool paged = a.pages != nullptr;
   KV_CHECK(a.q && a.out && a.lse) << a.what << ": NULL tensor";
   const bool sliding = paged && a.sliding_window != 0;
-  const bool rotary = a.rotary_mode != 0;
   KV_CHECK(a.sliding_window == 0 || paged) << a.what << ": a sliding-window cache is a paged one";
   if (rotary) {
+    KV_UNSUPPORTED(paged && a.tree_labels != nullptr)
+        << a.what << ": RoPE inside the kernel is not built for token trees over the page pool (the reference's kernel "
+        << "asserts the same, tree_attn.py:700-702)";
     KV_CHECK(a.q_rope_position != nullptr) << a.what << ": NULL q_rope_position";
     KV_CHECK(!paged || a.k_rope_pos_offset != nullptr) << a.what << ": NULL k_rope_pos_offset";
-    KV_UNSUPPORTED(a.d % (f32 ? 8 : 16) != 0)
-        << a.what << ": RoPE inside the generic kernels needs a head dim that is a multiple of " << (f32 ? 8 : 16) << ", got "
-        << a.d << " (an element and its partner half a head away are loaded as whole 16-byte pieces)";
   }
   if (paged) {
     KV_CHECK(a.page_indptr && a.page_values && a.last_page_len && a.page_size > 0) << a.what << ": NULL page table or bad page size";

@@ -70,17 +70,20 @@ class PagedKVCache {
         << "KV storage is built for float16 and float32 (got " << dtype_bits << " bits)";
     elem_bits_ = dtype_bits;
     // What the tuned fp16 kernels are not built for runs on the generic ones: float32 storage, pages other than
-    // 16 / 32 / 64 / 128 tokens, other head dims.  Those serve the plain cache.
+    // 16 / 32 / 64 / 128 tokens, other head dims -- and head dims 80 / 96 / 112 as soon as the cache has sliding
+    // windows or rotates inside the attention kernels (the tuned kernels have those head dims in their plain form).
     bool has_mha_layer = false;
     for (int64_t kind : attn_kinds_) has_mha_layer |= (kind != TVMKV_ATTN_MLA);
-    generic_ = has_mha_layer && (elem_bits_ == 32 || !tuned_page_size(static_cast<int>(page_size_)) ||
-                                 (!has_mla && !tuned_head_dim(static_cast<int>(qk_head_dim_))));
+    const bool extended = support_sliding_window_ || has_layer_sliding || rope_mode_ == TVMKV_ROPE_INLINE;
+    const int head_dim = static_cast<int>(qk_head_dim_);
+    const bool tuned_dim = extended ? (head_dim == 64 || head_dim == 128 || head_dim == 256) : tuned_head_dim(head_dim);
+    generic_ = has_mha_layer && (elem_bits_ == 32 || !tuned_page_size(static_cast<int>(page_size_)) || (!has_mla && !tuned_dim));
     if (generic_) {
       KV_UNSUPPORTED(has_mla) << "float32 storage, pages other than 16 / 32 / 64 / 128 tokens and other head dims are "
                               << "not built for caches with MLA layers";
-      KV_UNSUPPORTED(support_sliding_window_ || has_layer_sliding || rope_mode_ == TVMKV_ROPE_INLINE)
-          << "float32 storage, pages other than 16 / 32 / 64 / 128 tokens and head dims other than 64 / 80 / 96 / 112 / "
-          << "128 / 256 are built for the plain cache: no sliding window, no RoPE inside the attention kernels";
+      KV_UNSUPPORTED(rope_mode_ == TVMKV_ROPE_INLINE && head_dim % (elem_bits_ == 32 ? 8 : 16) != 0)
+          << "RoPE inside the generic attention kernels (a sliding-window cache rotates there) needs a head dim that is a "
+          << "multiple of " << (elem_bits_ == 32 ? 8 : 16) << ", got " << head_dim;
       KV_UNSUPPORTED(qk_head_dim_ != v_head_dim_) << "the generic kernels need equal qk and v head dims";
     }
     KV_CHECK(static_cast<int64_t>(attn_kinds_.size()) >= layer_end)
@@ -756,6 +759,14 @@ class PagedKVCache {
       a.tree_indptr = Dev(s.tree_attn_mn_indptr[0]);
       a.tree_labels = Dev(s.tree_attn_mask[0]);
     }
+    // RoPE inside the kernel: a chain's key t sits at k_ragged_rope_pos_offset[b] + t, a tree's keys at the
+    // positions of its query tokens (their depths), as in the tuned calls
+    a.rotary_mode = rope_mode_ == TVMKV_ROPE_INLINE;
+    a.q_rope_position = Dev(s.q_rope_position_map);
+    a.k_rope_pos_offset = tree ? nullptr : Dev(s.k_ragged_rope_pos_offset);
+    a.rope_scale = rotary_scale_;
+    a.rope_theta = rotary_theta_;
+    a.rope_scaling = InlineScaling();
     a.out = o;
     a.lse = lse;
     a.total_q = total_seq_length;
@@ -834,6 +845,14 @@ class PagedKVCache {
         a.page_size = static_cast<int32_t>(page_size_);
         a.causal = causal;
         a.sm_scale = sm_scale;
+        a.sliding_window = sliding_window;
+        a.layer_window = static_cast<int32_t>(layer_sliding_window_size_);
+        a.rotary_mode = rotary_mode;
+        a.q_rope_position = q_pos;
+        a.k_rope_pos_offset = k_rope_pos;
+        a.rope_scale = rotary_scale;
+        a.rope_theta = rotary_theta;
+        a.rope_scaling = InlineScaling();
         Launch(generic_attention(a, compute_stream_));
       } else if (s.append_before_attn && !s.is_chain[d]) {
         KV_CHECK(s.tree_attn_mask[d].present() && s.tree_attn_mn_indptr[d].present())
