@@ -17,9 +17,9 @@
  *
  *      Shapes.  The tuned kernels are fp16 with pages of 16 / 32 / 64 / 128 tokens and head dims
  *      64 / 80 / 96 / 112 / 128 / 256 (the comment of each launcher says what it has of them).
- *      A plain call (rotary_mode 0, one-row length_info) with another page size or head dim is
- *      handed to generic matrix-core kernels (float32 arithmetic, v_mfma_f32_16x16x4_f32; any
- *      page size, head dims that are a multiple of 8 up to 256): the reference's kernel
+ *      A call with another page size or head dim (80 / 96 / 112 as soon as it has rotary_mode 1
+ *      or a three-row length_info) is handed to generic matrix-core kernels (float32 sums; any page
+ *      size, head dims that are a multiple of 8 up to 256, of 16 with rotary_mode 1): the reference's kernel
  *      factories take both as free parameters (_decode_kernels.py:49,181;
  *      _prefill_kernels.py:54-60,217-225).  The same kernels serve float32 K/V storage, which the
  *      reference's tests also run (tests/python/relax/
@@ -490,8 +490,10 @@ typedef struct tvmkv_cache tvmkv_cache;
  *   dtype_bits    16 (fp16 storage) or 32 (float32 storage: every q / k / v / output tensor handed to the
  *                 verbs is float32 then).  float32 storage, page sizes other than 16 / 32 / 64 / 128 and
  *                 head dims other than 64 / 80 / 96 / 112 / 128 / 256 (multiples of 8, of 4 for float32, up
- *                 to 256) run on the generic kernels and are built for the plain cache: no sliding
- *                 window, no RoPE inside the attention kernels, no MLA layers (TVMKV_EUNSUPPORTED)
+ *                 to 256) run on the generic kernels, as do head dims 80 / 96 / 112 in a cache with sliding
+ *                 windows or RoPE inside the attention kernels; that rotation needs a head dim that is a
+ *                 multiple of 16 (of 8 for float32), and none of this is built for caches with MLA layers
+ *                 (TVMKV_EUNSUPPORTED)
  *   device_id     HIP device ordinal, or -1 for a HOST-ONLY cache: page-pool bookkeeping and
  *                 auxiliary arrays work, anything that touches device memory returns
  *                 TVMKV_ENODEVICE. */

@@ -20,8 +20,8 @@
  * Storage type.  q / k / v / pages / out of the MHA slots (13, 15-21, 23-27) are float16 or float32, the
  * same in every tensor of a call (the reference builds each kernel for one storage dtype); lse and the
  * RoPE factor tensor are float32, index arrays int32.  float32 storage runs on the generic kernels
- * (tvmkv.h, "Shapes"): plain calls only -- rotary_mode 1 and the (3, batch) length_info return
- * TVMKV_EUNSUPPORTED.  The MLA slots (14, 22) are float16.
+ * (tvmkv.h, "Shapes"), rotary_mode 1 (head dims that are a multiple of 8) and the (3, batch)
+ * length_info included.  The MLA slots (14, 22) are float16.
  */
 #ifndef TVMKV_DLPACK_H_
 #define TVMKV_DLPACK_H_

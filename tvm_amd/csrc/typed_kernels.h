@@ -3,12 +3,12 @@
 // The reference builds every kernel for a storage dtype, a page size and a head dim
 // (python/tvm/relax/frontend/nn/llm/kv_cache.py:559-736; its tests run float16 and float32 storage,
 // tests/python/relax/test_runtime_builtin_paged_attention_kv_cache_cpu.py:269-276).  This library's tuned
-// kernels are fp16 with pages of 16 / 32 / 64 / 128 tokens and head dims 64 / 80 / 96 / 112 / 128 / 256;
-// everything else those factories accept for a plain cache -- float32 storage, any page size, any head dim
-// that is a multiple of 4 (fp32) or 8 (fp16) up to 256 -- runs on the generic matrix-core kernels of
-// kernels_generic.hip: float32 arithmetic throughout (v_mfma_f32_16x16x4_f32), K and V rows read straight
-// from their pages with one page-table lookup per row, the sliding-window cache (length_info (3, batch)), the
-// per-layer window mask and RoPE inside the kernel included.  Not built there: MLA.
+// kernels are fp16 with pages of 16 / 32 / 64 / 128 tokens and head dims 64 / 80 / 96 / 112 / 128 / 256 (80 / 96 /
+// 112 in their plain form only); everything else those factories accept -- float32 storage, any page size, any
+// head dim that is a multiple of 4 (fp32) or 8 (fp16) up to 256 -- runs on the generic matrix-core kernels of
+// kernels_generic.hip: float32 sums, K and V rows read straight from their pages with one page-table lookup per
+// row, the sliding-window cache (length_info (3, batch)), the per-layer window mask and RoPE inside the kernel
+// included.  Not built there: MLA.
 //
 // elem_bits is 16 or 32.  The functions return the library's error codes and leave the message in the
 // thread's last-error slot, like the extern "C" launchers they stand beside; they are internal: the
