@@ -530,3 +530,100 @@ def _random_generic_case(case):
 def test_random_generic_kernel_cases(block):
     for case in range(block * 20, block * 20 + 20):
         _random_generic_case(case)
+
+
+def _random_generic_extended_case(case):
+    """One random launch of the generic kernel's extended form: a sliding-window cache with random sinks and evicted
+    gaps (or a plain one), RoPE inside the kernel or not, the per-layer window mask; decode, paged prefill or ragged
+    prefill; storage type, head shape, head dim and page size drawn from the seed."""
+    from tests.util import assert_close_where_keys, rows_without_keys
+    rng = np.random.default_rng(99000 + case)
+    dtype = F32 if rng.random() < 0.5 else F16
+    hq, hkv = [(8, 2), (4, 4), (32, 8), (12, 1), (20, 2)][rng.integers(5)]
+    step = 8 if dtype == F32 else 16
+    d = int(rng.integers(1, 256 // step + 1)) * step
+    if dtype == F16 and d in (64, 128, 256):
+        ps = int(rng.choice([1, 3, 5, 8, 12, 24, 40, 100]))   # a page size the tuned kernels do not have
+    else:
+        ps = int(rng.choice([1, 3, 5, 8, 12, 16, 24, 32, 64, 100]))
+    kind = ["decode", "paged", "ragged"][rng.integers(3)]
+    rotary = int(rng.integers(2)) if kind != "ragged" else 1
+    sliding = int(rng.integers(2)) if kind != "ragged" else 0
+    if not rotary and not sliding:
+        rotary = 1
+    b = int(rng.integers(1, 7))
+    sm = d ** -0.5
+    torch_dtype = torch.float32 if dtype == F32 else torch.float16
+    what = f"extended case {case}: {kind} {np.dtype(dtype).name} heads {hq}/{hkv} d {d} page {ps} rotary {rotary} sliding {sliding}"
+
+    def outputs(n):
+        return (torch.full((n, hq, d), 7.0, dtype=torch_dtype, device=DEV), torch.full((n, hq), 7.0, dtype=torch.float32, device=DEV))
+
+    if kind == "ragged":
+        lens = [int(rng.integers(1, 200)) for _ in range(b)]
+        n = sum(lens)
+        ind = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        q, k, v = (rng.standard_normal((n, h, d)).astype(dtype) for h in (hq, hkv, hkv))
+        off = rng.integers(0, 3000, size=b).astype(np.int32)
+        pos = np.concatenate([off[i] + np.arange(lens[i]) for i in range(b)]).astype(np.int32)
+        causal = int(rng.integers(2))
+        eo, el = np.zeros((n, hq, d), dtype), np.zeros((n, hq), F32)
+        ok.prefill_ragged(q, ind, k, v, ind, pos, off, eo, el, causal, 1, 1.0, 1e4, sm)
+        go, gl = outputs(n)
+        if dtype == F32:
+            dl.call("batch_prefill_ragged_kv", T(q)[1], TI(ind), T(k)[1], T(v)[1], TI(ind), TI(pos), TI(off), dl.tensor(go),
+                    dl.tensor(gl), causal, 1, 1.0, 1e4, sm)
+        else:
+            K.batch_prefill_ragged_kv(dev(q), i32(ind), dev(k), dev(v), i32(ind), i32(pos), i32(off), go, gl, causal, 1, 1.0, 1e4, sm)
+        assert_close(host(go), eo, what=what + " out", atol=4e-3 if dtype == F16 else 1e-3, rtol=1e-2 if dtype == F16 else 1e-3)
+        assert_close(host(gl), el, atol=2e-3 if dtype == F16 else 1e-3, rtol=1e-4, what=what + " lse")
+        return
+    phys = [int(rng.integers(1, 700)) for _ in range(b)]
+    sinks = [int(rng.integers(0, min(n, 20) + 1)) if sliding else 0 for n in phys]
+    offs = [int(rng.integers(s, n + 1)) if sliding else 0 for s, n in zip(sinks, phys)]
+    offs = [min(o, n - 1) if o > s else s for o, s, n in zip(offs, sinks, phys)]   # at least one visible key
+    logical = np.array([n - o + s for n, o, s in zip(phys, offs, sinks)])
+    need = 4 + sum((n + ps - 1) // ps for n in phys)
+    pages, indptr, values, last, _, _ = build_paged_kv(rng, phys, need, hkv, ps, d, dtype=dtype)
+    info = np.array([last, offs, sinks], np.int32) if sliding else np.asarray(last, np.int32)
+    k_off = rng.integers(0, 3000, size=b).astype(np.int32)
+    if kind == "decode":
+        q = rng.standard_normal((b, hq, d)).astype(dtype)
+        q_pos = (k_off + logical - 1).astype(np.int32)
+        eo, el = np.zeros((b, hq, d), dtype), np.zeros((b, hq), F32)
+        ok.decode(q, pages, indptr, values, info, k_off, q_pos, eo, el, rotary, 1.0, 1e4, sm)
+        go, gl = outputs(b)
+        if dtype == F32:
+            dl.call("batch_decode_paged_kv", T(q)[1], T(pages)[1], TI(indptr), TI(values), TI(info), TI(k_off), TI(q_pos),
+                    dl.tensor(go), dl.tensor(gl), rotary, 1.0, 1e4, sm)
+        else:
+            K.batch_decode_paged_kv(dev(q), dev(pages), i32(indptr), i32(values), i32(info), i32(k_off), i32(q_pos), go, gl, rotary,
+                                    1.0, 1e4, sm)
+        assert_close(host(go), eo, what=what + " out", atol=4e-3 if dtype == F16 else 1e-3, rtol=1e-2 if dtype == F16 else 1e-3)
+        assert_close(host(gl), el, atol=2e-3 if dtype == F16 else 1e-3, rtol=1e-4, what=what + " lse")
+        return
+    q_lens = [int(rng.integers(1, min(int(n), 90) + 1)) for n in logical]
+    n = sum(q_lens)
+    qindptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    q = rng.standard_normal((n, hq, d)).astype(dtype)
+    q_pos = np.concatenate([k_off[i] + logical[i] - q_lens[i] + np.arange(q_lens[i]) for i in range(b)]).astype(np.int32)
+    causal = int(rng.integers(2))
+    window = int(rng.choice([0, 5, 40, 1024])) if (causal and sliding) else 0
+    eo, el = np.zeros((n, hq, d), dtype), np.zeros((n, hq), F32)
+    ok.prefill_paged(q, qindptr, pages, indptr, values, info, k_off, q_pos, eo, el, causal, rotary, 1.0, 1e4, sm,
+                     sliding_window_size=window)
+    go, gl = outputs(n)
+    if dtype == F32:
+        dl.call("batch_prefill_paged_kv", T(q)[1], TI(qindptr), T(pages)[1], TI(indptr), TI(values), TI(info), TI(k_off), TI(q_pos),
+                dl.tensor(go), dl.tensor(gl), causal, rotary, 1.0, 1e4, sm, window)
+    else:
+        K.batch_prefill_paged_kv(dev(q), i32(qindptr), dev(pages), i32(indptr), i32(values), i32(info), i32(k_off), i32(q_pos), go,
+                                 gl, causal, rotary, 1.0, 1e4, sm, sliding_window_size=window)
+    no_keys = rows_without_keys(q_lens, causal, window if sliding else 0)
+    assert_close_where_keys(host(go), host(gl), eo, el, no_keys, 2e-3 if dtype == F16 else 1e-3, what)
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_random_generic_extended_cases(block):
+    for case in range(block * 20, block * 20 + 20):
+        _random_generic_extended_case(case)
