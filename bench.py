@@ -866,7 +866,7 @@ def extras(torch, K, dev):
                            "straight from their pages into the operands of v_mfma_f32_16x16x4_f32, or of the fp16 "
                            "instructions of that shape for fp16 storage): decode of 64 seqs ctx U[1024,8192] Hq32/Hkv8/D128 "
                            "with float32 storage (page 16) and with fp16 pages of 24 tokens; causal self-attention of "
-                           "4 x 2048 tokens with float32 storage (D128) and with fp16 storage at head dim 160"}
+                           "4 x 2048 tokens with float32 storage (D128) and with fp16 storage at head dims 160 and 96 (the latter with RoPE inside the kernel)"}
         for name, tdt, ps_ in (("decode_float32_storage", torch.float32, 16), ("decode_fp16_pages_of_24_tokens", torch.float16, 24)):
             npg_ = (ctx_ + ps_ - 1) // ps_
             ip_ = np.concatenate([[0], np.cumsum(npg_)])
@@ -901,16 +901,18 @@ def extras(torch, K, dev):
         fl_ = 4.0 * HQ * D * n_ * c_ * (c_ + 1) / 2
         res["causal_prefill_float32_storage"] = {"ms": round(ms_, 4), "tflops": round(fl_ / ms_ / 1e9, 1),
                                                  "frac_of_fp32_mfma_peak": round(fl_ / ms_ / 1e9 / 157.3, 4)}
-        d_ = 160
-        q_, k_, v_ = (torch.randn((n_ * c_, h_, d_), device=dev).to(torch.float16) for h_ in (HQ, HKV, HKV))
-        o_ = torch.empty_like(q_)
-        a_ = (dl.tensor(q_), dl.tensor(ind_), dl.tensor(k_), dl.tensor(v_), dl.tensor(ind_), dl.tensor(zq_), dl.tensor(zb_),
-              dl.tensor(o_), dl.tensor(l_), 1, 0, 1.0, 1e4, d_ ** -0.5)
-        dl.call("batch_prefill_ragged_kv", *a_)
-        ms_ = time_region(torch, lambda i: dl.call("batch_prefill_ragged_kv", *a_), 5, SETTLE_S)
-        fl_ = 4.0 * HQ * d_ * n_ * c_ * (c_ + 1) / 2
-        res["causal_prefill_fp16_head_dim_160"] = {"ms": round(ms_, 4), "tflops": round(fl_ / ms_ / 1e9, 1),
-                                                   "frac_of_mfma_peak": round(fl_ / ms_ / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+        for d_, rotary_ in ((160, 0), (96, 1)):  # head dim 96 with RoPE inside the kernel: a sliding-window cache's prefill
+            q_, k_, v_ = (torch.randn((n_ * c_, h_, d_), device=dev).to(torch.float16) for h_ in (HQ, HKV, HKV))
+            o_ = torch.empty_like(q_)
+            pos_ = i32(np.tile(np.arange(c_), n_))
+            a_ = (dl.tensor(q_), dl.tensor(ind_), dl.tensor(k_), dl.tensor(v_), dl.tensor(ind_), dl.tensor(pos_), dl.tensor(zb_),
+                  dl.tensor(o_), dl.tensor(l_), 1, rotary_, 1.0, 1e4, d_ ** -0.5)
+            dl.call("batch_prefill_ragged_kv", *a_)
+            ms_ = time_region(torch, lambda i: dl.call("batch_prefill_ragged_kv", *a_), 5, SETTLE_S)
+            fl_ = 4.0 * HQ * d_ * n_ * c_ * (c_ + 1) / 2
+            name_ = f"causal_prefill_fp16_head_dim_{d_}" + ("_rope_in_kernel" if rotary_ else "")
+            res[name_] = {"ms": round(ms_, 4), "tflops": round(fl_ / ms_ / 1e9, 1),
+                          "frac_of_mfma_peak": round(fl_ / ms_ / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
         return res
 
     out["generic_kernels"] = generic_leg()

@@ -144,6 +144,11 @@ __device__ __forceinline__ void rotate_piece(float* own, const float* row, int f
 constexpr int generic_workgroups(int elem_bytes, int dmax, int nb) {
   return elem_bytes == 2 ? (dmax > 128 ? 2 : (nb == 1 ? 4 : 3)) : (dmax > 128 ? 1 : (nb == 1 ? 3 : 2));
 }
+// 16-row blocks per row tile: one for decode-shaped calls and for head dims above 128 (registers), two when a
+// (sequence, kv head) has more than 16 rows on average.  Three and four blocks (fp16 storage, one workgroup fewer
+// per CU) measured slower: causal self-attention of 4 x 2048 tokens at head dim 72 173 against 195 TFLOP/s, at
+// head dim 48 144 against 197; only calls that rotate inside the kernel gained (head dim 96: 99 against 90).
+inline int generic_row_blocks(int d, int rows_hint) { return d > 128 || rows_hint <= 16 ? 1 : 2; }
 
 // EXT adds what the extended tuned kernels add: the sliding-window cache (the page table covers `sink` tokens at the
 // front, evicted tokens up to `window_offset`, then the window; keys have logical indices, sink tokens first, that
@@ -539,11 +544,11 @@ void launch_attention(const GAttn& p, const InlineRopeTable& rope, int rows_hint
     KV_CHECK(slots < (int64_t{1} << 31)) << "too many row tiles for one launch";
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(slots), p.h_kv, p.splits), dim3(256), 0, stream, p, rope);
   };
-  const bool wide = rows_hint > 16;  // more than one 16-row block per (sequence, kv head) on average
+  const int nb = generic_row_blocks(p.d, rows_hint);
   if (p.d <= 64) {
-    if (wide) run(generic_attn_kernel<T, 64, 2, EXT>, 32); else run(generic_attn_kernel<T, 64, 1, EXT>, 16);
+    if (nb == 2) run(generic_attn_kernel<T, 64, 2, EXT>, 32); else run(generic_attn_kernel<T, 64, 1, EXT>, 16);
   } else if (p.d <= 128) {
-    if (wide) run(generic_attn_kernel<T, 128, 2, EXT>, 32); else run(generic_attn_kernel<T, 128, 1, EXT>, 16);
+    if (nb == 2) run(generic_attn_kernel<T, 128, 2, EXT>, 32); else run(generic_attn_kernel<T, 128, 1, EXT>, 16);
   } else {
     run(generic_attn_kernel<T, 256, 1, EXT>, 16);
   }
@@ -632,7 +637,7 @@ int generic_attention(const GenericAttention& a, void* stream_) {
   p.splits = 1;
   ScratchLease lease{};
   if (paged) {
-    const int rows_per_tile = (rows_hint > 16 && a.d <= 128) ? 32 : 16;
+    const int rows_per_tile = 16 * generic_row_blocks(a.d, rows_hint);
     const int64_t tiles = (a.total_q * group / rows_per_tile + a.batch) * a.h_kv;
     const int64_t keys_per_seq = a.nnz_pages * a.page_size / a.batch;
     const int64_t want = (f32 ? 8 : 16) * static_cast<int64_t>(compute_units()) / std::max<int64_t>(tiles, 1);
