@@ -102,42 +102,38 @@ __device__ __forceinline__ void store_run<half_t, 8>(half_t* p, const float* in)
 }
 __device__ __forceinline__ void store4(float* p, float4_t v) { *reinterpret_cast<float4_t*>(p) = v; }
 
-// In-kernel RoPE of one 16-byte piece of a q / k row (rotate-half over the whole head,
-// python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-127): x[f + e] of the piece at feature f, its partner piece
-// at f +- d/2 from the same row (d/2 is a whole number of pieces), float32 arithmetic, one rounding to the storage
-// type.  tbl: the table of InlineRopeTable in LDS.
+// In-kernel RoPE (rotate-half over the whole head, python/tvm/relax/frontend/nn/llm/_kernel_common.py:115-127) of
+// two 16-byte pieces of a q / k row that lie half a head apart: lo[e] is feature f + e, hi[e] its partner
+// f + d/2 + e.  float32 arithmetic, one rounding to the storage type; tbl: the table of InlineRopeTable in LDS (an
+// element and its partner share the angle unless the variant's halves differ).
 template <int N>
-__device__ __forceinline__ void rotate_run(float* x, const float* partner, bool upper_half, int f, float pos_scaled,
-                                           const float* tbl, int inverse, float magnitude) {
+__device__ __forceinline__ void rotate_pair(float* lo, float* hi, int f, int d, float pos_scaled, const float* tbl, int inverse,
+                                            int halves_differ, float magnitude) {
 #pragma unroll
   for (int e = 0; e < N; ++e) {
     float sn, cs;
     sincos_reduced(inverse ? pos_scaled * tbl[f + e] : pos_scaled / tbl[f + e], sn, cs);
-    x[e] = magnitude * (cs * x[e] + sn * (upper_half ? partner[e] : -partner[e]));
+    float sn_hi = sn, cs_hi = cs;
+    if (halves_differ) sincos_reduced(inverse ? pos_scaled * tbl[f + d / 2 + e] : pos_scaled / tbl[f + d / 2 + e], sn_hi, cs_hi);
+    const float xl = lo[e], xh = hi[e];
+    lo[e] = magnitude * (cs * xl - sn * xh);
+    hi[e] = magnitude * (cs_hi * xh + sn_hi * xl);
   }
 }
-__device__ __forceinline__ half8_t rotate_piece(half8_t own, const half_t* row, int f, int d, float pos_scaled, const float* tbl,
-                                                int inverse, float magnitude) {
-  const bool upper = f >= d / 2;
-  const half8_t other = *reinterpret_cast<const half8_t*>(row + (upper ? f - d / 2 : f + d / 2));
+__device__ __forceinline__ void rotate_pair(half8_t& lo, half8_t& hi, int f, int d, float pos_scaled, const float* tbl, int inverse,
+                                            int halves_differ, float magnitude) {
   float x[8], y[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    x[e] = static_cast<float>(own[e]);
-    y[e] = static_cast<float>(other[e]);
+    x[e] = static_cast<float>(lo[e]);
+    y[e] = static_cast<float>(hi[e]);
   }
-  rotate_run<8>(x, y, upper, f, pos_scaled, tbl, inverse, magnitude);
-  half8_t out;
+  rotate_pair<8>(x, y, f, d, pos_scaled, tbl, inverse, halves_differ, magnitude);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) out[e] = static_cast<half_t>(x[e]);
-  return out;
-}
-__device__ __forceinline__ void rotate_piece(float* own, const float* row, int f, int d, float pos_scaled, const float* tbl,
-                                             int inverse, float magnitude) {
-  const bool upper = f >= d / 2;
-  float y[4];
-  load_run<float, 4>(row + (upper ? f - d / 2 : f + d / 2), y);
-  rotate_run<4>(own, y, upper, f, pos_scaled, tbl, inverse, magnitude);
+  for (int e = 0; e < 8; ++e) {
+    lo[e] = static_cast<half_t>(x[e]);
+    hi[e] = static_cast<half_t>(y[e]);
+  }
 }
 
 // workgroups per CU: the fp16 form holds its operands in half the registers
@@ -237,6 +233,20 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
   float qf[NB][QS][PIECE];  // float32 storage
   half8_t qh[NB][QS];       // fp16 storage: the pieces as they are in memory
   const T* qbase = static_cast<const T*>(p.q);
+  // Which 16-byte piece of a q / k row lane group g feeds to load step s of the score product: any assignment
+  // serves, as long as q and k agree.  Plain: piece 4 s + g.  With rotation inside the kernel: the first half of
+  // the steps takes the pieces of the lower half of the head, the second half their partners half a head away,
+  // so that a lane holds both elements of every rotated pair.
+  static_assert(QS % 2 == 0, "load steps come in pairs");
+  auto piece_feature = [&](int s) {
+    if (!(EXT && rotary)) return (4 * s + g) * PIECE;
+    const int lower = (4 * (s % (QS / 2)) + g) * PIECE;
+    return s < QS / 2 ? lower : lower + d / 2;
+  };
+  auto piece_inside = [&](int s) {
+    if (!(EXT && rotary)) return (4 * s + g) * PIECE < d;
+    return (4 * (s % (QS / 2)) + g) * PIECE < d / 2;
+  };
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     const int row = r0 + nb * 16 + j;
@@ -253,22 +263,28 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
     const T* qrow = qbase + (static_cast<int64_t>(q_start + qi) * p.h_q + head) * d;
 #pragma unroll
     for (int s = 0; s < QS; ++s) {
-      const int f = (4 * s + g) * PIECE;
+      const int f = piece_feature(s);
+      const bool inside = valid && piece_inside(s);
       if constexpr (HALF) {
         half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-        qh[nb][s] = valid && f < d ? *reinterpret_cast<const half8_t*>(qrow + f) : z;
-      } else if (valid && f < d) {
+        qh[nb][s] = inside ? *reinterpret_cast<const half8_t*>(qrow + f) : z;
+      } else if (inside) {
         load_run<T, PIECE>(qrow + f, qf[nb][s]);
       } else {
 #pragma unroll
         for (int e = 0; e < PIECE; ++e) qf[nb][s][e] = 0.f;
       }
-      if (EXT && rotary && valid && f < d) {
-        const float pos = static_cast<float>(p.q_rope_position[q_start + qi]) * p.rope_scale;
+    }
+    if (EXT && rotary && valid) {
+      const float pos = static_cast<float>(p.q_rope_position[q_start + qi]) * p.rope_scale;
+#pragma unroll
+      for (int s = 0; s < QS / 2; ++s) {
+        if (!piece_inside(s)) continue;
         if constexpr (HALF) {
-          qh[nb][s] = rotate_piece(qh[nb][s], qrow, f, d, pos, rope_lds, rope.inverse, rope.magnitude);
+          rotate_pair(qh[nb][s], qh[nb][s + QS / 2], piece_feature(s), d, pos, rope_lds, rope.inverse, rope.halves_differ, rope.magnitude);
         } else {
-          rotate_piece(qf[nb][s], qrow, f, d, pos, rope_lds, rope.inverse, rope.magnitude);
+          rotate_pair<PIECE>(qf[nb][s], qf[nb][s + QS / 2], piece_feature(s), d, pos, rope_lds, rope.inverse, rope.halves_differ,
+                             rope.magnitude);
         }
       }
     }
@@ -317,11 +333,11 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
     const T* krow_ptr = kbase + static_cast<int64_t>(krow) * d;
 #pragma unroll
     for (int s = 0; s < QS; ++s) {
-      const int f = (4 * s + g) * PIECE;
+      const int f = piece_feature(s);
       if constexpr (HALF) {
         half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-        kh[s] = f < d ? *reinterpret_cast<const half8_t*>(krow_ptr + f) : z;
-      } else if (f < d) {
+        kh[s] = piece_inside(s) ? *reinterpret_cast<const half8_t*>(krow_ptr + f) : z;
+      } else if (piece_inside(s)) {
         load_run<T, PIECE>(krow_ptr + f, kf[s]);
       } else {
 #pragma unroll
@@ -332,14 +348,13 @@ __global__ __launch_bounds__(256, generic_workgroups(sizeof(T), DMAX, NB)) void 
       const int key_pos = p.k_rope_pos_offset != nullptr ? p.k_rope_pos_offset[b] + t : p.q_rope_position[kv_start + t];
       const float pos = static_cast<float>(key_pos) * p.rope_scale;
 #pragma unroll
-      for (int s = 0; s < QS; ++s) {
-        const int f = (4 * s + g) * PIECE;
-        if (f < d) {
-          if constexpr (HALF) {
-            kh[s] = rotate_piece(kh[s], krow_ptr, f, d, pos, rope_lds, rope.inverse, rope.magnitude);
-          } else {
-            rotate_piece(kf[s], krow_ptr, f, d, pos, rope_lds, rope.inverse, rope.magnitude);
-          }
+      for (int s = 0; s < QS / 2; ++s) {
+        if (!piece_inside(s)) continue;
+        if constexpr (HALF) {
+          rotate_pair(kh[s], kh[s + QS / 2], piece_feature(s), d, pos, rope_lds, rope.inverse, rope.halves_differ, rope.magnitude);
+        } else {
+          rotate_pair<PIECE>(kf[s], kf[s + QS / 2], piece_feature(s), d, pos, rope_lds, rope.inverse, rope.halves_differ,
+                             rope.magnitude);
         }
       }
     }
