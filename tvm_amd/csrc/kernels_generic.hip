@@ -145,6 +145,11 @@ constexpr int generic_workgroups(int elem_bytes, int dmax, int nb) {
 // per CU) measured slower: causal self-attention of 4 x 2048 tokens at head dim 72 173 against 195 TFLOP/s, at
 // head dim 48 144 against 197; only calls that rotate inside the kernel gained (head dim 96: 99 against 90).
 inline int generic_row_blocks(int d, int rows_hint) { return d > 128 || rows_hint <= 16 ? 1 : 2; }
+// Also measured and not kept: a form for prefill-shaped calls whose four waves take rows of their own and share
+// stages of 32 keys through LDS (a K / V row fetched and rotated once per 128 query rows).  Plain calls ran slower
+// (head dim 72: 156 against 196 TFLOP/s, with the next stage's loads held in registers during the matrix work 109:
+// twelve independent waves per CU hide the loads better than three workgroups in step); calls that rotate inside
+// the kernel gained (head dim 96: 135 against 103).
 
 // EXT adds what the extended tuned kernels add: the sliding-window cache (the page table covers `sink` tokens at the
 // front, evicted tokens up to `window_offset`, then the window; keys have logical indices, sink tokens first, that
