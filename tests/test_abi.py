@@ -69,3 +69,20 @@ def test_version_and_error_channel():
     assert rc == -2 and b"head dim 100" in lib.tvmkv_last_error()
     rc = lib.tvmkv_fused_rope(None, None, None, None, None, 1, 0, 8, 2, 128, 1.0, 1e4, None)
     assert rc == 0  # empty input is a no-op
+
+
+def test_public_headers_are_plain_c(tmp_path):
+    """The boundary is a C ABI: the three public headers compile as C99 and as C++11 on their own, warnings as
+    errors (a binding generator -- cgo, JNI, ctypes codegen -- reads them as C)."""
+    import shutil
+    import subprocess
+
+    src = tmp_path / "headers.c"
+    src.write_text('#include "tvmkv.h"\n#include "tvmkv_dlpack.h"\n#include "tvmkv_bench.h"\n'
+                   "int main(void) { return tvmkv_version() == 0; }\n")
+    include = os.path.join(ROOT, "include")
+    flags = ["-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", include]
+    if shutil.which("gcc"):
+        subprocess.check_call(["gcc", "-std=c99"] + flags + [str(src)])
+    if shutil.which("g++"):
+        subprocess.check_call(["g++", "-std=c++11", "-x", "c++"] + flags + [str(src)])
