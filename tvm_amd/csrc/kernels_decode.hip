@@ -859,7 +859,7 @@ static void decode_entry(Lease&& lease, const FusedStep& fused_step, const void*
   const int heads_per_item = (group > 16 && dk <= 128) ? 32 : 16;
   const int head_blocks = (group + heads_per_item - 1) / heads_per_item;
   const int chunk16 = heads_per_item == 32 ? decode_pick_chunk_pages_wide(nnz_pages << p.page_shift, h_kv, batch_size, head_blocks, 2 * compute_units())
-                                           : decode_pick_chunk_pages(nnz_pages << p.page_shift, h_kv, batch_size);
+                                           : decode_pick_chunk_pages(nnz_pages << p.page_shift, h_kv, batch_size, d);
   p.chunk_pages = std::max(1, chunk16 >> p.page_shift);
   p.scale_log2 = static_cast<float>(sm_scale) * kLog2e;
   p.qkv = static_cast<const half_t*>(fused_step.qkv);

@@ -175,8 +175,8 @@ void debug_set_scratch_launches(uint64_t launches) {
 //    no partial states at all (256 sequences of 512-2048 tokens: 0.220 ms with 64 pages, 0.210 with 128).
 // Chunks of 32, 64, 96 or 128 pages put the chunks of a sequence whose pages have consecutive ids -- a cache that
 // was filled sequence by sequence hands them out that way -- at a distance in memory at which the workgroups of
-// the sequence, which walk their chunks in step, keep meeting in the same memory channels.  Seen with 8 and 16 kv
-// heads (pages of 64 and 128 KiB), not with 4 or fewer.  Measured, 8 kv heads, us with permuted / consecutive
+// the sequence, which walk their chunks in step, keep meeting in the same memory channels.  Seen at head dim 128
+// with 8 and 16 kv heads (pages of 64 and 128 KiB), not with 4 or fewer, and not at head dims 64 and 256.  Measured, 8 kv heads, us with permuted / consecutive
 // page ids (chunk pages -> time):
 //   64 x U[1024,8192] (cfg 2)      48: 195.8 / 196.3   56: 194.5 / 196.5   64: 197.8 / 205.1   80: 195.0 / 197.3
 //   8 x U[32768,131072], 64 q      112: 435.1 / 438.8  120: 439.5 / 440.5  128: 436.8 / 478.9  64: 453.3 / 527.3
@@ -184,9 +184,11 @@ void debug_set_scratch_launches(uint64_t launches) {
 //   4 x 32768                      88: 90.2 / 92.1     96: 92.5 / 101.3    104: 91.9 / 93.4
 //   64 x U[1024,8192], 16 kv heads 56: 389.9 / 387.3   32: 390.7 / 425.5   64: 390.2 / 406.0
 //   64 x U[1024,8192], 4 kv heads  56: 126.0 / 123.2   64: 120.5 / 118.2
-static bool camps(int chunk_pages, int h_kv) { return h_kv >= 8 && chunk_pages % 32 == 0; }
+//   head dim 256, 8 kv heads        48: 437 / 429       64: 421 / 417       80: 417 / 411       (no camping: the rule is left alone)
+//   head dim 64, 8 kv heads         48: 115 / 111       64: 116 / 112       96: 112 / 110       (flat)
+static bool camps(int chunk_pages, int h_kv, int head_dim) { return h_kv >= 8 && head_dim == 128 && chunk_pages % 32 == 0; }
 
-int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
+int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch, int head_dim) {
   const int64_t forced = option(kOptDecodeChunkPages);
   if (forced >= 8 && forced % 8 == 0) return static_cast<int>(forced);
   const int64_t work = nnz_pages * h_kv;
@@ -206,7 +208,7 @@ int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
     //   1 x 131072                            64: 102.3 120: 100.8 128*: 88.1                    [128]
     int cp = 128;
     for (int c = 24; c <= 128; c += 8) {
-      if (camps(c, h_kv)) continue;
+      if (camps(c, h_kv, head_dim)) continue;
       if ((nnz_pages / c + batch) * h_kv <= 768) {
         cp = c;
         break;
@@ -228,8 +230,8 @@ int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch) {
   if (per_seq <= 96 && static_cast<int64_t>(batch) * h_kv >= 1536) return 128;
   // the neighbours of the powers of two that do not camp (see camps()); one or two sequences keep 128 pages
   // (64 states of a 131 072-token sequence merge in two rounds of 32)
-  if (camps(pow2, h_kv) && pow2 == 64) return 48;
-  if (camps(pow2, h_kv) && pow2 == 128 && batch > 2) return 112;
+  if (camps(pow2, h_kv, head_dim) && pow2 == 64) return 48;
+  if (camps(pow2, h_kv, head_dim) && pow2 == 128 && batch > 2) return 112;
   return pow2;
 }
 

@@ -64,7 +64,7 @@ InlineRopeHost inline_rope_table(const ::tvmkv_rope_scaling* scaling, int head_d
 
 // Chunk-slot arithmetic of the decode split, on the host (the device functions of the same names in
 // kernels_decode.hip compute the same values; the tests compare both against a direct enumeration).
-int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch);
+int decode_pick_chunk_pages(int64_t nnz_pages, int h_kv, int batch, int head_dim = 128);
 // the same for launches whose work items carry 32 query heads (GQA groups above 16)
 int decode_pick_chunk_pages_wide(int64_t nnz_pages, int h_kv, int batch, int head_blocks, int resident_items);
 
